@@ -1,0 +1,539 @@
+// Device codecs: quantize_tensor / dequantize_tensor on the GPU, bit-exact with
+// the CPU algorithm of crates/axonml-quant/src/quantize.rs and dequantize.rs,
+// plus the permutation between the packed (`to_bytes`) image and the planar
+// device layout.
+//
+// This file must be compiled with -ffp-contract=off: the reference rounds each
+// multiply, divide, add and subtract separately (f32), and so do these kernels.
+#include <hip/hip_fp16.h>
+
+#include "axq_internal.h"
+
+namespace {
+
+__device__ inline uint16_t f32_to_f16_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
+__device__ inline float f16_bits_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+
+// Rust: v.round().clamp(lo, hi) as iN -- roundf is half away from zero, NaN -> 0.
+__device__ inline int round_clamp(float v, float lo, float hi) {
+    float r = roundf(v);
+    if (isnan(r)) return 0;
+    r = r < lo ? lo : r;
+    r = r > hi ? hi : r;
+    return (int)r;
+}
+
+// Loads the (up to) 32 floats of block `b`; elements past numel are +0.0 and
+// `len` says how many are real.
+__device__ inline void load_block32(const float *src, size_t numel, size_t b, float (&x)[32], int &len) {
+    size_t start = b * 32;
+    size_t rem = numel - start;
+    len = rem < 32 ? (int)rem : 32;
+    if (len == 32) {
+        const float4 *p = reinterpret_cast<const float4 *>(src + start);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float4 v = p[i];
+            x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; i++) x[i] = i < len ? src[start + i] : 0.0f;
+    }
+}
+
+__device__ inline void store_u16(uint8_t *p, uint16_t v) { *reinterpret_cast<uint16_t *>(p) = v; }
+__device__ inline uint16_t load_u16(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
+
+// ---- Q8_0: quantize.rs:82-114, image types.rs:142-147 ---------------------
+__global__ void quant_q8_0_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblk) return;
+    float x[32];
+    int len;
+    load_block32(src, numel, b, x, len);
+    float max_abs = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++)
+        if (i < len) max_abs = fmaxf(max_abs, fabsf(x[i]));
+    float scale = max_abs > 0.0f ? max_abs / 127.0f : 1.0f;
+    uint8_t *o = out + b * 34;
+    store_u16(o, f32_to_f16_bits(scale));
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        int q0 = (2 * i) < len ? round_clamp(x[2 * i] / scale, -127.0f, 127.0f) : 0;
+        int q1 = (2 * i + 1) < len ? round_clamp(x[2 * i + 1] / scale, -127.0f, 127.0f) : 0;
+        store_u16(o + 2 + 2 * i, (uint16_t)((q0 & 0xFF) | ((q1 & 0xFF) << 8)));
+    }
+}
+
+// ---- Q4_0: quantize.rs:121-156, pack types.rs:190-198 ---------------------
+__global__ void quant_q4_0_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblk) return;
+    float x[32];
+    int len;
+    load_block32(src, numel, b, x, len);
+    float max_abs = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++)
+        if (i < len) max_abs = fmaxf(max_abs, fabsf(x[i]));
+    float scale = max_abs > 0.0f ? max_abs / 7.0f : 1.0f;
+    uint8_t *o = out + b * 18;
+    store_u16(o, f32_to_f16_bits(scale));
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int e = 4 * i + j;
+            int q = e < len ? round_clamp(x[e] / scale, -8.0f, 7.0f) : 0;
+            w |= (uint32_t)((q + 8) & 0x0F) << (4 * j);
+        }
+        store_u16(o + 2 + 2 * i, (uint16_t)w);
+    }
+}
+
+// ---- Q4_1: quantize.rs:163-205, image types.rs:249-255 --------------------
+__global__ void quant_q4_1_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblk) return;
+    float x[32];
+    int len;
+    load_block32(src, numel, b, x, len);
+    float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 32; i++)
+        if (i < len) {
+            mn = fminf(mn, x[i]);
+            mx = fmaxf(mx, x[i]);
+        }
+    float scale = mx > mn ? (mx - mn) / 15.0f : 1.0f;
+    uint8_t *o = out + b * 20;
+    store_u16(o, f32_to_f16_bits(scale));
+    store_u16(o + 2, f32_to_f16_bits(mn));
+    int nbytes = len / 2 < 16 ? len / 2 : 16; // the reference's pack loop bound
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int e = 4 * i + j;
+            int q = e < len ? round_clamp((x[e] - mn) / scale, 0.0f, 15.0f) : 0;
+            if ((e >> 1) >= nbytes) q = 0;
+            w |= (uint32_t)(q & 0x0F) << (4 * j);
+        }
+        store_u16(o + 4 + 2 * i, (uint16_t)w);
+    }
+}
+
+// ---- Q5_0 / Q5_1: GGUF layouts; scale rules max_abs/15 and (max-min)/31 ---
+template <bool WITH_MIN>
+__global__ void quant_q5_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblk) return;
+    float x[32];
+    int len;
+    load_block32(src, numel, b, x, len);
+    float scale, mn = 0.0f;
+    if (WITH_MIN) {
+        float lo = INFINITY, hi = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 32; i++)
+            if (i < len) {
+                lo = fminf(lo, x[i]);
+                hi = fmaxf(hi, x[i]);
+            }
+        scale = hi > lo ? (hi - lo) / 31.0f : 1.0f;
+        mn = lo;
+    } else {
+        float max_abs = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 32; i++)
+            if (i < len) max_abs = fmaxf(max_abs, fabsf(x[i]));
+        scale = max_abs > 0.0f ? max_abs / 15.0f : 1.0f;
+    }
+    uint32_t u[32];
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+        if (WITH_MIN)
+            u[i] = i < len ? (uint32_t)round_clamp((x[i] - mn) / scale, 0.0f, 31.0f) : 0u;
+        else
+            u[i] = i < len ? (uint32_t)(round_clamp(x[i] / scale, -16.0f, 15.0f) + 16) : 16u;
+    }
+    uint8_t *o = out + b * (WITH_MIN ? 24 : 22);
+    store_u16(o, f32_to_f16_bits(scale));
+    int off = 2;
+    if (WITH_MIN) {
+        store_u16(o + 2, f32_to_f16_bits(mn));
+        off = 4;
+    }
+    uint32_t qh = 0;
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        qh |= ((u[j] >> 4) & 1u) << j;
+        qh |= ((u[j + 16] >> 4) & 1u) << (j + 16);
+    }
+    store_u16(o + off, (uint16_t)qh);
+    store_u16(o + off + 2, (uint16_t)(qh >> 16));
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        uint32_t b0 = (u[2 * j] & 0x0F) | ((u[2 * j + 16] & 0x0F) << 4);
+        uint32_t b1 = (u[2 * j + 1] & 0x0F) | ((u[2 * j + 17] & 0x0F) << 4);
+        store_u16(o + off + 4 + 2 * j, (uint16_t)(b0 | (b1 << 8)));
+    }
+}
+
+// ---- Q4_K: one lane per 32-element sub-block, 8 lanes per superblock -------
+// Rule: per sub-block mn = min(0, min x), mx = max x, scale = (mx-mn)/15,
+// min = -mn; the superblock's d = max scale / 63, dmin = max min / 63 (stored
+// as f16); 6-bit ls = round(63/max_scale * scale), lm likewise; codes
+// q = clamp(round((x + dmin*lm) / (d*ls)), 0, 15) with the f16-rounded d, dmin.
+__global__ void quant_q4_k_kernel(const float *src, size_t numel, size_t nsb, uint8_t *out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t sb = t >> 3;
+    int s = (int)(t & 7);
+    bool live = sb < nsb;
+    float x[32];
+#pragma unroll
+    for (int i = 0; i < 32; i++) x[i] = 0.0f;
+    if (live) {
+        size_t start = sb * 256 + (size_t)s * 32;
+        if (start + 32 <= numel) {
+            const float4 *p = reinterpret_cast<const float4 *>(src + start);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float4 v = p[i];
+                x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 32; i++)
+                if (start + i < numel) x[i] = src[start + i];
+        }
+    }
+    float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+        mn = fminf(mn, x[i]);
+        mx = fmaxf(mx, x[i]);
+    }
+    if (mn > 0.0f) mn = 0.0f;
+    float scale, smin;
+    if (!(mx > mn)) {
+        scale = 0.0f;
+        smin = isfinite(mn) ? -mn : 0.0f;
+    } else {
+        scale = (mx - mn) / 15.0f;
+        smin = -mn;
+    }
+    float max_scale = scale, max_min = smin;
+#pragma unroll
+    for (int m = 1; m < 8; m <<= 1) {
+        max_scale = fmaxf(max_scale, __shfl_xor(max_scale, m));
+        max_min = fmaxf(max_min, __shfl_xor(max_min, m));
+    }
+    float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+    float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+    int ls = round_clamp(inv_scale * scale, 0.0f, 63.0f);
+    int lm = round_clamp(inv_min * smin, 0.0f, 63.0f);
+    uint16_t dh = f32_to_f16_bits(max_scale / 63.0f);
+    uint16_t dminh = f32_to_f16_bits(max_min / 63.0f);
+    float d = f16_bits_to_f32(dh), dmin = f16_bits_to_f32(dminh);
+    float sd = d * (float)ls;
+    float sm = dmin * (float)lm;
+    // codes as 8 dwords of one code per byte
+    uint32_t cb[8];
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int q = sd == 0.0f ? 0 : round_clamp((x[4 * w + j] + sm) / sd, 0.0f, 15.0f);
+            v |= (uint32_t)q << (8 * j);
+        }
+        cb[w] = v;
+    }
+    // pair partner exchange: even lane (sub-block 2p) holds the low nibbles
+    uint32_t other[8];
+#pragma unroll
+    for (int w = 0; w < 8; w++) other[w] = (uint32_t)__shfl_xor((int)cb[w], 1);
+    // header values of all 8 sub-blocks
+    int base_lane = (int)(threadIdx.x & 63) & ~7;
+    uint32_t lsv[8], lmv[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        lsv[j] = (uint32_t)__shfl(ls, base_lane + j);
+        lmv[j] = (uint32_t)__shfl(lm, base_lane + j);
+    }
+    if (!live) return;
+    uint8_t *o = out + sb * 144;
+    if (s == 0) {
+        uint32_t h[4];
+        h[0] = (uint32_t)dh | ((uint32_t)dminh << 16);
+        uint8_t sc[12];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            sc[j] = (uint8_t)(lsv[j] | ((lsv[j + 4] >> 4) << 6));
+            sc[j + 4] = (uint8_t)(lmv[j] | ((lmv[j + 4] >> 4) << 6));
+            sc[j + 8] = (uint8_t)((lsv[j + 4] & 0x0F) | ((lmv[j + 4] & 0x0F) << 4));
+        }
+#pragma unroll
+        for (int w = 0; w < 3; w++)
+            h[1 + w] = (uint32_t)sc[4 * w] | ((uint32_t)sc[4 * w + 1] << 8) | ((uint32_t)sc[4 * w + 2] << 16) |
+                       ((uint32_t)sc[4 * w + 3] << 24);
+        *reinterpret_cast<uint4 *>(o) = make_uint4(h[0], h[1], h[2], h[3]);
+    }
+    if ((s & 1) == 0) {
+        int p = s >> 1;
+        uint32_t pk[8];
+#pragma unroll
+        for (int w = 0; w < 8; w++) pk[w] = cb[w] | (other[w] << 4);
+        uint4 *q = reinterpret_cast<uint4 *>(o + 16 + 32 * p);
+        q[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        q[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+    }
+}
+
+// ---- F16: quantize.rs:212-218 --------------------------------------------
+__global__ void quant_f16_kernel(const float *src, size_t numel, uint16_t *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < numel) out[i] = f32_to_f16_bits(src[i]);
+}
+__global__ void dequant_f16_kernel(const uint16_t *src, size_t numel, float *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < numel) out[i] = f16_bits_to_f32(src[i]);
+}
+
+// ---- dequantisers: dequantize.rs:89-92, 116-121, 145-151 -------------------
+// One thread per 32 elements; for Q4_K a thread handles one sub-block.
+__global__ void dequant_kernel(int type, const uint8_t *packed, size_t numel, size_t n32, float *out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n32) return;
+    float y[32];
+    switch (type) {
+    case AXQ_Q8_0: {
+        const uint8_t *b = packed + t * 34;
+        float scale = f16_bits_to_f32(load_u16(b));
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            uint16_t w = load_u16(b + 2 + 2 * i);
+            y[2 * i] = (float)(int8_t)(w & 0xFF) * scale;
+            y[2 * i + 1] = (float)(int8_t)(w >> 8) * scale;
+        }
+        break;
+    }
+    case AXQ_Q4_0: {
+        const uint8_t *b = packed + t * 18;
+        float scale = f16_bits_to_f32(load_u16(b));
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t w = load_u16(b + 2 + 2 * i);
+#pragma unroll
+            for (int j = 0; j < 4; j++) y[4 * i + j] = (float)((int)((w >> (4 * j)) & 0x0F) - 8) * scale;
+        }
+        break;
+    }
+    case AXQ_Q4_1: {
+        const uint8_t *b = packed + t * 20;
+        float scale = f16_bits_to_f32(load_u16(b));
+        float mn = f16_bits_to_f32(load_u16(b + 2));
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t w = load_u16(b + 4 + 2 * i);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float a = (float)((w >> (4 * j)) & 0x0F) * scale;
+                y[4 * i + j] = a + mn;
+            }
+        }
+        break;
+    }
+    case AXQ_Q5_0:
+    case AXQ_Q5_1: {
+        bool with_min = type == AXQ_Q5_1;
+        const uint8_t *b = packed + t * (with_min ? 24 : 22);
+        float d = f16_bits_to_f32(load_u16(b));
+        float m = with_min ? f16_bits_to_f32(load_u16(b + 2)) : 0.0f;
+        int off = with_min ? 4 : 2;
+        uint32_t qh = (uint32_t)load_u16(b + off) | ((uint32_t)load_u16(b + off + 2) << 16);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            uint32_t w = load_u16(b + off + 4 + 2 * j);
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                int e = 2 * j + h;
+                uint32_t byte = (w >> (8 * h)) & 0xFF;
+                int u0 = (int)((byte & 0x0F) | (((qh >> e) & 1u) << 4));
+                int u1 = (int)((byte >> 4) | (((qh >> (e + 16)) & 1u) << 4));
+                if (with_min) {
+                    float a = (float)u0 * d;
+                    float c = (float)u1 * d;
+                    y[e] = a + m;
+                    y[e + 16] = c + m;
+                } else {
+                    y[e] = (float)(u0 - 16) * d;
+                    y[e + 16] = (float)(u1 - 16) * d;
+                }
+            }
+        }
+        break;
+    }
+    case AXQ_Q4_K: {
+        size_t sb = t >> 3;
+        int s = (int)(t & 7);
+        const uint8_t *b = packed + sb * 144;
+        float d = f16_bits_to_f32(load_u16(b));
+        float dmin = f16_bits_to_f32(load_u16(b + 2));
+        const uint8_t *sc = b + 4;
+        uint32_t l, m;
+        if (s < 4) {
+            l = sc[s] & 63;
+            m = sc[s + 4] & 63;
+        } else {
+            l = (uint32_t)((sc[s + 4] & 0x0F) | ((sc[s - 4] >> 6) << 4));
+            m = (uint32_t)((sc[s + 4] >> 4) | ((sc[s] >> 6) << 4));
+        }
+        float sd = d * (float)l;
+        float sm = dmin * (float)m;
+        const uint32_t *qs = reinterpret_cast<const uint32_t *>(b + 16 + 32 * (s >> 1));
+        int shift = (s & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t w = qs[i] >> shift;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float a = sd * (float)((w >> (8 * j)) & 0x0F);
+                y[4 * i + j] = a - sm;
+            }
+        }
+        break;
+    }
+    default:
+        return;
+    }
+    size_t start = t * 32;
+    if (start + 32 <= numel) {
+        float4 *o = reinterpret_cast<float4 *>(out + start);
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = make_float4(y[4 * i], y[4 * i + 1], y[4 * i + 2], y[4 * i + 3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; i++)
+            if (start + i < numel) out[start + i] = y[i];
+    }
+}
+
+// ---- packed image <-> planar device layout ---------------------------------
+// One thread per block (per superblock for Q4_K).  to_planar selects the copy
+// direction; the two directions are exact inverses.
+struct PlanarDesc {
+    uint8_t *codes, *meta, *qh;
+    size_t codes_pitch, meta_pitch, qh_pitch;
+    int64_t n_rows, blocks_per_row;
+    int type;
+};
+
+__device__ inline void copy_u16s(uint8_t *dst, const uint8_t *src, int nbytes) {
+    for (int i = 0; i < nbytes; i += 2) store_u16(dst + i, load_u16(src + i));
+}
+
+__global__ void repack_kernel(PlanarDesc d, uint8_t *packed, bool to_planar) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t total = d.n_rows * d.blocks_per_row;
+    if (t >= total) return;
+    int64_t row = t / d.blocks_per_row, blk = t % d.blocks_per_row;
+    int code_bytes, meta_bytes, qh_bytes = 0;
+    switch (d.type) {
+    case AXQ_Q8_0: code_bytes = 32; meta_bytes = 2; break;
+    case AXQ_Q4_0: code_bytes = 16; meta_bytes = 2; break;
+    case AXQ_Q4_1: code_bytes = 16; meta_bytes = 4; break;
+    case AXQ_Q5_0: code_bytes = 16; meta_bytes = 2; qh_bytes = 4; break;
+    case AXQ_Q5_1: code_bytes = 16; meta_bytes = 4; qh_bytes = 4; break;
+    case AXQ_Q4_K: code_bytes = 128; meta_bytes = 16; break;
+    default: return;
+    }
+    uint8_t *img = packed + (size_t)t * (size_t)(code_bytes + meta_bytes + qh_bytes);
+    uint8_t *meta = d.meta + (size_t)row * d.meta_pitch + (size_t)blk * meta_bytes;
+    if (to_planar) copy_u16s(meta, img, meta_bytes); else copy_u16s(img, meta, meta_bytes);
+    if (qh_bytes) {
+        uint8_t *qh = d.qh + (size_t)row * d.qh_pitch + (size_t)blk * 4;
+        if (to_planar) copy_u16s(qh, img + meta_bytes, 4); else copy_u16s(img + meta_bytes, qh, 4);
+    }
+    uint8_t *img_codes = img + meta_bytes + qh_bytes;
+    uint8_t *row_codes = d.codes + (size_t)row * d.codes_pitch;
+    if (d.type == AXQ_Q4_K) {
+        for (int c = 0; c < 8; c++) { // 16-byte runs keep their order inside the run
+            uint8_t *pl = row_codes + q4k_code_offset(d.blocks_per_row, blk, 16 * c);
+            if (to_planar) copy_u16s(pl, img_codes + 16 * c, 16); else copy_u16s(img_codes + 16 * c, pl, 16);
+        }
+    } else {
+        uint8_t *pl = row_codes + (size_t)blk * code_bytes;
+        if (to_planar) copy_u16s(pl, img_codes, code_bytes); else copy_u16s(img_codes, pl, code_bytes);
+    }
+}
+
+inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
+
+} // namespace
+
+int axq_dev_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, uint8_t *packed) {
+    if (numel == 0) return AXQ_OK;
+    size_t nblk = axq_num_blocks(type, numel);
+    const unsigned B = 128;
+    switch (type) {
+    case AXQ_Q8_0: quant_q8_0_kernel<<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_Q4_0: quant_q4_0_kernel<<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_Q4_1: quant_q4_1_kernel<<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_Q5_0: quant_q5_kernel<false><<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_Q5_1: quant_q5_kernel<true><<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_Q4_K: quant_q4_k_kernel<<<grid_for(nblk * 8, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_F16: quant_f16_kernel<<<grid_for(numel, 256), 256, 0, ctx->stream>>>(src, numel, (uint16_t *)packed); break;
+    case AXQ_F32:
+        AXQ_HIP(ctx, hipMemcpyAsync(packed, src, numel * 4, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+        return AXQ_OK;
+    default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", type);
+    }
+    AXQ_LAUNCH_CHECK(ctx, "quantize kernel");
+    return AXQ_OK;
+}
+
+int axq_dev_dequantize(axq_ctx *ctx, int type, const uint8_t *packed, size_t numel, float *dst) {
+    if (numel == 0) return AXQ_OK;
+    switch (type) {
+    case AXQ_Q8_0: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q4_K: {
+        size_t n32 = (numel + 31) / 32;
+        dequant_kernel<<<grid_for(n32, 128), 128, 0, ctx->stream>>>(type, packed, numel, n32, dst);
+        break;
+    }
+    case AXQ_F16:
+        dequant_f16_kernel<<<grid_for(numel, 256), 256, 0, ctx->stream>>>((const uint16_t *)packed, numel, dst);
+        break;
+    case AXQ_F32:
+        AXQ_HIP(ctx, hipMemcpyAsync(dst, packed, numel * 4, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+        return AXQ_OK;
+    default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", type);
+    }
+    AXQ_LAUNCH_CHECK(ctx, "dequantize kernel");
+    return AXQ_OK;
+}
+
+int axq_dev_repack(axq_ctx *ctx, const axq_weight *w, uint8_t *packed, bool to_planar) {
+    if (w->type == AXQ_F16 || w->type == AXQ_F32) {
+        void *dst = to_planar ? (void *)w->codes : (void *)packed;
+        const void *src = to_planar ? (const void *)packed : (const void *)w->codes;
+        AXQ_HIP(ctx, hipMemcpyAsync(dst, src, w->packed_bytes, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+        return AXQ_OK;
+    }
+    PlanarDesc d;
+    d.codes = w->codes; d.meta = w->meta; d.qh = w->qh;
+    d.codes_pitch = w->codes_pitch; d.meta_pitch = w->meta_pitch; d.qh_pitch = w->qh_pitch;
+    d.n_rows = w->n_rows;
+    d.blocks_per_row = w->k / (int64_t)axq_type_block_size(w->type);
+    d.type = w->type;
+    size_t total = (size_t)(d.n_rows * d.blocks_per_row);
+    if (total == 0) return AXQ_OK;
+    repack_kernel<<<grid_for(total, 128), 128, 0, ctx->stream>>>(d, packed, to_planar);
+    AXQ_LAUNCH_CHECK(ctx, "repack kernel");
+    return AXQ_OK;
+}

@@ -1,0 +1,426 @@
+// Decode-path quantized matmul: y[b, n] = sum_k x[b, k] * W[n, k] (+ bias[n]).
+//
+// This fuses the reference composition dequantize_tensor -> transpose ->
+// sgemm (crates/axonml-quant/src/dequantize.rs:34-54,
+// crates/axonml-tensor/src/tensor.rs:1020-1045,
+// crates/axonml-core/src/backends/cpu.rs:566-598) into one pass over the packed
+// weight bytes.  The kernel is HBM-bound: every weight byte is read once.
+//
+// Work decomposition (wave64):
+//   - A lane owns a fixed K-range ("chunk": one 16-byte vector of codes, two for
+//     Q4_K) for the whole kernel, so its slice of x is loaded once into VGPRs
+//     and reused for every row the wave visits.
+//   - 64 consecutive chunks form a wave "slice"; S = ceil(chunks_per_row / 64)
+//     waves of a workgroup cover one row together (split-K), G groups of S
+//     waves share a workgroup, each group walks R rows.
+//   - Per row a lane issues 128-bit loads of codes (fully coalesced: lane
+//     stride 16 B) plus its block's scale data, unpacks in registers and
+//     accumulates; the 64 partial sums are folded with DPP row shifts and row
+//     broadcasts; the S slice totals are added in a fixed order through LDS
+//     (no atomics: results are run-to-run identical).
+//   - U rows are in flight per lane at a time to keep enough HBM requests
+//     outstanding.
+#include <hip/hip_fp16.h>
+
+#include "axq_internal.h"
+
+namespace {
+
+struct GemvArgs {
+    const uint8_t *codes, *meta, *qh;
+    size_t codes_pitch, meta_pitch, qh_pitch;
+    const float *x, *bias;
+    float *y;
+    int n_rows;
+    int cpr;     // chunks per row
+    int S, G, R; // slices per row, row groups per workgroup, rows per group
+    int npass;   // > 1 when a lane must visit several chunks per row
+    float fp8_unit_inv;
+};
+
+typedef float float2v __attribute__((ext_vector_type(2)));
+
+__device__ inline float f16_bits_to_f32(uint32_t h) { return __half2float(__ushort_as_half((unsigned short)h)); }
+
+__device__ inline float ubyte0(uint32_t v) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(v)); return r; }
+__device__ inline float ubyte1(uint32_t v) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(v)); return r; }
+__device__ inline float ubyte2(uint32_t v) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(v)); return r; }
+__device__ inline float ubyte3(uint32_t v) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(v)); return r; }
+
+// Sum over the 64 lanes of a wave; the total is valid in lane 63.
+template <int CTRL, int ROW_MASK, bool BOUND>
+__device__ inline float dpp_add(float v) {
+    int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, BOUND);
+    return v + __builtin_bit_cast(float, t);
+}
+__device__ inline float wave_sum_lane63(float v) {
+    v = dpp_add<0x111, 0xf, true>(v); // row_shr:1
+    v = dpp_add<0x112, 0xf, true>(v); // row_shr:2
+    v = dpp_add<0x114, 0xf, true>(v); // row_shr:4
+    v = dpp_add<0x118, 0xf, true>(v); // row_shr:8  -> lane 15 of each row holds the row total
+    v = dpp_add<0x142, 0xa, false>(v); // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xc, false>(v); // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+// The four bytes of `v` must each hold a value 0..15.  v_cvt_pk_f32_fp8 turns
+// such a byte n into n * unit (the 8-bit float with a 3-bit mantissa is linear
+// over 0..15), two bytes per instruction; x has been pre-multiplied by 1/unit.
+__device__ inline void fma_nibbles4(uint32_t v, const float *xs, float &acc) {
+    float2v a = __builtin_amdgcn_cvt_pk_f32_fp8((int)v, false);
+    float2v b = __builtin_amdgcn_cvt_pk_f32_fp8((int)v, true);
+    acc = fmaf(a[0], xs[0], acc);
+    acc = fmaf(a[1], xs[1], acc);
+    acc = fmaf(b[0], xs[2], acc);
+    acc = fmaf(b[1], xs[3], acc);
+}
+
+// ---------------------------------------------------------------------------
+// Per-type traits.  W = weights per chunk; X holds what a lane keeps of x;
+// Raw what it loads per row; load() issues the loads; dot() folds them.
+// ---------------------------------------------------------------------------
+struct Q4K {
+    static constexpr int W = 64;
+    struct X { float xs[64]; float sum_lo, sum_hi; };
+    struct Raw { uint4 q0, q1, h; };
+    __device__ static void load_x(const GemvArgs &a, const float *x, int chunk, bool active, X &o) {
+        float lo = 0.f, hi = 0.f;
+        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 64);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            float s = (v.x + v.y) + (v.z + v.w);
+            if (i < 8) lo += s; else hi += s;
+            o.xs[4 * i] = v.x * a.fp8_unit_inv; o.xs[4 * i + 1] = v.y * a.fp8_unit_inv;
+            o.xs[4 * i + 2] = v.z * a.fp8_unit_inv; o.xs[4 * i + 3] = v.w * a.fp8_unit_inv;
+        }
+        o.sum_lo = lo; o.sum_hi = hi;
+    }
+    __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
+        // chunk = pair index in the row; slice = chunk / 64; P = pairs in this slice
+        int slice = chunk >> 6, lane_pair = chunk & 63;
+        int P = a.cpr - (slice << 6);
+        P = P < 64 ? P : 64;
+        const uint8_t *base = a.codes + (size_t)row * a.codes_pitch + (size_t)slice * 2048 + (size_t)lane_pair * 16;
+        r.q0 = *reinterpret_cast<const uint4 *>(base);
+        r.q1 = *reinterpret_cast<const uint4 *>(base + (size_t)P * 16);
+        r.h = *reinterpret_cast<const uint4 *>(a.meta + (size_t)row * a.meta_pitch + (size_t)(chunk >> 2) * 16);
+    }
+    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int chunk) {
+        int p = chunk & 3;
+        // 6-bit scale/min of sub-blocks 2p and 2p+1 (ggml get_scale_min_k4 order)
+        int sh = (p & 1) * 16;
+        uint32_t ya = r.h.y >> sh, za = r.h.z >> sh, wa = r.h.w >> sh;
+        uint32_t scp, mp;
+        if (p < 2) {
+            scp = ya & 0x3F3F;
+            mp = za & 0x3F3F;
+        } else {
+            scp = (wa & 0x0F0F) | ((ya >> 2) & 0x3030);
+            mp = ((wa >> 4) & 0x0F0F) | ((za >> 2) & 0x3030);
+        }
+        float d = f16_bits_to_f32(r.h.x & 0xFFFF), dmin = f16_bits_to_f32(r.h.x >> 16);
+        float alo0 = 0.f, alo1 = 0.f, ahi0 = 0.f, ahi1 = 0.f;
+        const uint32_t q0[4] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w};
+        const uint32_t q1[4] = {r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            // first half of the pair: bytes 4w..4w+3 -> elements 4w.. (low), 32+4w.. (high)
+            fma_nibbles4(q0[w] & 0x0F0F0F0Fu, &x.xs[4 * w], alo0);
+            fma_nibbles4((q0[w] >> 4) & 0x0F0F0F0Fu, &x.xs[32 + 4 * w], ahi0);
+            // second half: bytes 16+4w.. -> elements 16+4w.. (low), 48+4w.. (high)
+            fma_nibbles4(q1[w] & 0x0F0F0F0Fu, &x.xs[16 + 4 * w], alo1);
+            fma_nibbles4((q1[w] >> 4) & 0x0F0F0F0Fu, &x.xs[48 + 4 * w], ahi1);
+        }
+        float sc0 = ubyte0(scp), sc1 = ubyte1(scp), m0 = ubyte0(mp), m1 = ubyte1(mp);
+        float pos = fmaf(sc0, alo0 + alo1, sc1 * (ahi0 + ahi1));
+        float neg = fmaf(m0, x.sum_lo, m1 * x.sum_hi);
+        return fmaf(d, pos, -(dmin * neg));
+    }
+};
+
+template <bool WITH_MIN>
+struct Q4x { // Q4_0 / Q4_1: adjacent-pair nibble order (types.rs:179-198)
+    static constexpr int W = 32;
+    struct X { float xs[32]; float sum; };
+    struct Raw { uint4 q; uint32_t m; };
+    __device__ static void load_x(const GemvArgs &a, const float *x, int chunk, bool active, X &o) {
+        float s = 0.f;
+        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 32);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            s += (v.x + v.y) + (v.z + v.w);
+            o.xs[4 * i] = v.x * a.fp8_unit_inv; o.xs[4 * i + 1] = v.y * a.fp8_unit_inv;
+            o.xs[4 * i + 2] = v.z * a.fp8_unit_inv; o.xs[4 * i + 3] = v.w * a.fp8_unit_inv;
+        }
+        o.sum = s;
+    }
+    __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
+        r.q = *reinterpret_cast<const uint4 *>(a.codes + (size_t)row * a.codes_pitch + (size_t)chunk * 16);
+        const uint8_t *m = a.meta + (size_t)row * a.meta_pitch;
+        if (WITH_MIN) r.m = *reinterpret_cast<const uint32_t *>(m + (size_t)chunk * 4);
+        else r.m = *reinterpret_cast<const uint16_t *>(m + (size_t)chunk * 2);
+    }
+    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int) {
+        const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            // dword w: nibble j = element 8w + j; even elements sit in the low nibbles
+            uint32_t lo = q[w] & 0x0F0F0F0Fu, hi = (q[w] >> 4) & 0x0F0F0F0Fu;
+            float2v la = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, false), lb = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, true);
+            float2v ha = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, false), hb = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, true);
+            const float *xs = &x.xs[8 * w];
+            a0 = fmaf(la[0], xs[0], a0); a1 = fmaf(ha[0], xs[1], a1);
+            a0 = fmaf(la[1], xs[2], a0); a1 = fmaf(ha[1], xs[3], a1);
+            a0 = fmaf(lb[0], xs[4], a0); a1 = fmaf(hb[0], xs[5], a1);
+            a0 = fmaf(lb[1], xs[6], a0); a1 = fmaf(hb[1], xs[7], a1);
+        }
+        float scale = f16_bits_to_f32(r.m & 0xFFFF);
+        float acc = a0 + a1;
+        if (WITH_MIN) return fmaf(scale, acc, f16_bits_to_f32(r.m >> 16) * x.sum);
+        return scale * fmaf(-8.0f, x.sum, acc);
+    }
+};
+
+template <bool WITH_MIN>
+struct Q5x { // Q5_0 / Q5_1: byte j = elements j (low nibble) and j+16 (high); qh bit e = bit 4 of element e
+    static constexpr int W = 32;
+    struct X { float xs[32]; float sum; };
+    struct Raw { uint4 q; uint32_t qh; uint32_t m; };
+    __device__ static void load_x(const GemvArgs &, const float *x, int chunk, bool active, X &o) {
+        float s = 0.f;
+        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 32);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            s += (v.x + v.y) + (v.z + v.w);
+            o.xs[4 * i] = v.x; o.xs[4 * i + 1] = v.y; o.xs[4 * i + 2] = v.z; o.xs[4 * i + 3] = v.w;
+        }
+        o.sum = s;
+    }
+    __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
+        r.q = *reinterpret_cast<const uint4 *>(a.codes + (size_t)row * a.codes_pitch + (size_t)chunk * 16);
+        r.qh = *reinterpret_cast<const uint32_t *>(a.qh + (size_t)row * a.qh_pitch + (size_t)chunk * 4);
+        const uint8_t *m = a.meta + (size_t)row * a.meta_pitch;
+        if (WITH_MIN) r.m = *reinterpret_cast<const uint32_t *>(m + (size_t)chunk * 4);
+        else r.m = *reinterpret_cast<const uint16_t *>(m + (size_t)chunk * 2);
+    }
+    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int) {
+        const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            // spread 4 bits of qh to bit 4 of each byte: t * 0x00204081 puts bit i at bit 8i
+            uint32_t bl = (((r.qh >> (4 * w)) & 0xFu) * 0x00204081u) & 0x01010101u;
+            uint32_t bh = (((r.qh >> (16 + 4 * w)) & 0xFu) * 0x00204081u) & 0x01010101u;
+            uint32_t lo = (q[w] & 0x0F0F0F0Fu) | (bl << 4);
+            uint32_t hi = ((q[w] >> 4) & 0x0F0F0F0Fu) | (bh << 4);
+            const float *xl = &x.xs[4 * w], *xh = &x.xs[16 + 4 * w];
+            a0 = fmaf(ubyte0(lo), xl[0], a0); a1 = fmaf(ubyte0(hi), xh[0], a1);
+            a0 = fmaf(ubyte1(lo), xl[1], a0); a1 = fmaf(ubyte1(hi), xh[1], a1);
+            a0 = fmaf(ubyte2(lo), xl[2], a0); a1 = fmaf(ubyte2(hi), xh[2], a1);
+            a0 = fmaf(ubyte3(lo), xl[3], a0); a1 = fmaf(ubyte3(hi), xh[3], a1);
+        }
+        float d = f16_bits_to_f32(r.m & 0xFFFF);
+        float acc = a0 + a1;
+        if (WITH_MIN) return fmaf(d, acc, f16_bits_to_f32(r.m >> 16) * x.sum);
+        return d * fmaf(-16.0f, x.sum, acc);
+    }
+};
+
+struct Q80 { // chunk = 16 int8 = half a block
+    static constexpr int W = 16;
+    struct X { float xs[16]; };
+    struct Raw { uint4 q; uint32_t m; };
+    __device__ static void load_x(const GemvArgs &, const float *x, int chunk, bool active, X &o) {
+        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            o.xs[4 * i] = v.x; o.xs[4 * i + 1] = v.y; o.xs[4 * i + 2] = v.z; o.xs[4 * i + 3] = v.w;
+        }
+    }
+    __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
+        r.q = *reinterpret_cast<const uint4 *>(a.codes + (size_t)row * a.codes_pitch + (size_t)chunk * 16);
+        r.m = *reinterpret_cast<const uint16_t *>(a.meta + (size_t)row * a.meta_pitch + (size_t)(chunk >> 1) * 2);
+    }
+    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int) {
+        const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            int v = (int)q[w];
+            a0 = fmaf((float)(signed char)(v), x.xs[4 * w], a0);
+            a1 = fmaf((float)(signed char)(v >> 8), x.xs[4 * w + 1], a1);
+            a0 = fmaf((float)(signed char)(v >> 16), x.xs[4 * w + 2], a0);
+            a1 = fmaf((float)(v >> 24), x.xs[4 * w + 3], a1);
+        }
+        return f16_bits_to_f32(r.m) * (a0 + a1);
+    }
+};
+
+struct F16W { // chunk = 8 halfs
+    static constexpr int W = 8;
+    struct X { float xs[8]; };
+    struct Raw { uint4 q; };
+    __device__ static void load_x(const GemvArgs &, const float *x, int chunk, bool active, X &o) {
+        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 8);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            o.xs[4 * i] = v.x; o.xs[4 * i + 1] = v.y; o.xs[4 * i + 2] = v.z; o.xs[4 * i + 3] = v.w;
+        }
+    }
+    __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
+        r.q = *reinterpret_cast<const uint4 *>(a.codes + (size_t)row * a.codes_pitch + (size_t)chunk * 16);
+    }
+    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int) {
+        const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            a0 = fmaf(f16_bits_to_f32(q[w] & 0xFFFF), x.xs[2 * w], a0);
+            a1 = fmaf(f16_bits_to_f32(q[w] >> 16), x.xs[2 * w + 1], a1);
+        }
+        return a0 + a1;
+    }
+};
+
+struct F32W { // chunk = 4 floats
+    static constexpr int W = 4;
+    struct X { float xs[4]; };
+    struct Raw { float4 q; };
+    __device__ static void load_x(const GemvArgs &, const float *x, int chunk, bool active, X &o) {
+        float4 v = active ? *reinterpret_cast<const float4 *>(x + (size_t)chunk * 4) : make_float4(0, 0, 0, 0);
+        o.xs[0] = v.x; o.xs[1] = v.y; o.xs[2] = v.z; o.xs[3] = v.w;
+    }
+    __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
+        r.q = *reinterpret_cast<const float4 *>(a.codes + (size_t)row * a.codes_pitch + (size_t)chunk * 16);
+    }
+    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int) {
+        return fmaf(r.q.x, x.xs[0], r.q.y * x.xs[1]) + fmaf(r.q.z, x.xs[2], r.q.w * x.xs[3]);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// The kernel.  U rows in flight per lane.
+// ---------------------------------------------------------------------------
+template <class T, int U>
+__global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
+    extern __shared__ float red[]; // [G][R][S] slice totals
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int grp = wave / a.S, slice = wave - grp * a.S;
+    const int row0 = (blockIdx.x * a.G + grp) * a.R;
+    int row_end = row0 + a.R;
+    row_end = row_end < a.n_rows ? row_end : a.n_rows;
+
+    typename T::X xr;
+    int chunk = slice * 64 + lane;
+    bool active = chunk < a.cpr;
+    int cchunk = active ? chunk : a.cpr - 1; // inactive lanes re-read a valid chunk against x = 0
+    if (a.npass == 1) T::load_x(a, a.x, cchunk, active, xr);
+
+    for (int r = row0; r < row_end; r += U) {
+        float part[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) part[u] = 0.f;
+        for (int pass = 0; pass < a.npass; pass++) {
+            if (a.npass > 1) {
+                chunk = (pass * a.S + slice) * 64 + lane;
+                active = chunk < a.cpr;
+                cchunk = active ? chunk : a.cpr - 1;
+                T::load_x(a, a.x, cchunk, active, xr);
+            }
+            typename T::Raw raw[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                int row = r + u;
+                row = row < a.n_rows ? row : a.n_rows - 1; // rows past the end are loaded and dropped
+                T::load(a, row, cchunk, raw[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) part[u] += T::dot(a, raw[u], xr, cchunk);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float tot = wave_sum_lane63(part[u]);
+            int row = r + u;
+            if (lane == 63 && row < row_end) {
+                if (a.S == 1) a.y[row] = a.bias ? tot + a.bias[row] : tot;
+                else red[(grp * a.R + (row - row0)) * a.S + slice] = tot;
+            }
+        }
+    }
+    if (a.S > 1) {
+        __syncthreads();
+        int t = threadIdx.x;
+        if (t < a.G * a.R) {
+            int g = t / a.R, rr = t - g * a.R;
+            int row = (blockIdx.x * a.G + g) * a.R + rr;
+            if (row < a.n_rows) {
+                float tot = 0.f;
+                for (int s = 0; s < a.S; s++) tot += red[(g * a.R + rr) * a.S + s];
+                a.y[row] = a.bias ? tot + a.bias[row] : tot;
+            }
+        }
+    }
+}
+
+template <class T>
+int launch(axq_ctx *ctx, const axq_weight *w, const float *x, const float *bias, float *y) {
+    GemvArgs a;
+    a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
+    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
+    a.x = x; a.bias = bias; a.y = y;
+    a.n_rows = (int)w->n_rows;
+    a.cpr = (int)(w->k / T::W);
+    a.fp8_unit_inv = ctx->fp8_unit_inv;
+    const int SMAX = 8;
+    int s_need = (a.cpr + 63) / 64;
+    a.S = s_need < SMAX ? s_need : SMAX;
+    a.npass = (s_need + a.S - 1) / a.S;
+    a.G = a.S >= 4 ? 1 : 4 / a.S;
+    constexpr int U = 4;
+    // rows per group: aim for about 8 workgroups per CU-pair while keeping x reuse
+    int cus = ctx->prop.multiProcessorCount;
+    int target_wgs = cus * 2;
+    int R = (a.n_rows + a.G * target_wgs - 1) / (a.G * target_wgs);
+    R = (R + U - 1) / U * U;
+    if (R < U) R = U;
+    if (R > 64) R = 64;
+    a.R = R;
+    int rows_per_wg = a.G * a.R;
+    unsigned grid = (unsigned)((a.n_rows + rows_per_wg - 1) / rows_per_wg);
+    unsigned block = (unsigned)(64 * a.S * a.G);
+    size_t lds = a.S > 1 ? (size_t)a.G * a.R * a.S * sizeof(float) : 0;
+    gemv_kernel<T, U><<<grid, block, lds, ctx->stream>>>(a);
+    AXQ_LAUNCH_CHECK(ctx, "gemv_kernel");
+    return AXQ_OK;
+}
+
+} // namespace
+
+int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y) {
+    if (w->n_rows > INT32_MAX || w->k > INT32_MAX)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
+    for (int b = 0; b < batch; b++) {
+        const float *xb = x + (size_t)b * (size_t)w->k;
+        float *yb = y + (size_t)b * (size_t)w->n_rows;
+        int rc;
+        switch (w->type) {
+        case AXQ_Q4_K: rc = launch<Q4K>(ctx, w, xb, bias, yb); break;
+        case AXQ_Q4_0: rc = launch<Q4x<false>>(ctx, w, xb, bias, yb); break;
+        case AXQ_Q4_1: rc = launch<Q4x<true>>(ctx, w, xb, bias, yb); break;
+        case AXQ_Q5_0: rc = launch<Q5x<false>>(ctx, w, xb, bias, yb); break;
+        case AXQ_Q5_1: rc = launch<Q5x<true>>(ctx, w, xb, bias, yb); break;
+        case AXQ_Q8_0: rc = launch<Q80>(ctx, w, xb, bias, yb); break;
+        case AXQ_F16: rc = launch<F16W>(ctx, w, xb, bias, yb); break;
+        case AXQ_F32: rc = launch<F32W>(ctx, w, xb, bias, yb); break;
+        default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
+        }
+        if (rc) return rc;
+    }
+    return AXQ_OK;
+}

@@ -1,0 +1,92 @@
+// Internal declarations shared by the axq translation units (not installed).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/axq.h"
+
+// ---------------------------------------------------------------------------
+// Context: one device, one stream, an error string, a timer pair.
+// ---------------------------------------------------------------------------
+struct axq_ctx {
+    int device;
+    hipStream_t own_stream;
+    hipStream_t stream; // own_stream or an adopted one
+    hipEvent_t ev_start, ev_stop;
+    hipDeviceProp_t prop;
+    float fp8_unit_inv; // 1 / value(fp8 byte 0x01) as converted by v_cvt_pk_f32_fp8
+    char err[512];
+};
+
+// ---------------------------------------------------------------------------
+// Device-resident weight: "planar" layout, one allocation.
+//
+//   plane 0 (codes)   : the 4/5/8-bit code bytes of every block, row-major,
+//                       row pitch = codes_pitch bytes (16-byte aligned rows)
+//   plane 1 (meta)    : per-block scale data, row-major, meta_pitch bytes/row
+//                         Q8_0, Q4_0, Q5_0 : f16 scale             (2 B/block)
+//                         Q4_1, Q5_1       : f16 scale | f16 min   (4 B/block)
+//                         Q4_K             : d, dmin, scales[12]   (16 B/superblock)
+//   plane 2 (qh)      : Q5_0/Q5_1 only, the 32 high bits of each block (4 B/block)
+//
+// The bytes are exactly those of the packed (`to_bytes`) image, permuted, so
+// upload -> download is the identity and HBM traffic per matmul equals the
+// packed size.  For Q4_K the 128 code bytes of a superblock are further
+// interleaved inside 16-superblock "slices" so that one wavefront reads two
+// fully contiguous 1 KiB runs per row (see q4k_code_offset).
+// ---------------------------------------------------------------------------
+struct axq_weight {
+    int type;
+    int64_t n_rows, k;
+    size_t packed_bytes; // size of the to_bytes image
+    uint8_t *base;       // device allocation
+    size_t alloc_bytes;
+    uint8_t *codes, *meta, *qh;
+    size_t codes_pitch, meta_pitch, qh_pitch;
+    bool owns;
+};
+
+static inline size_t axq_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Byte offset, inside one row of the Q4_K code plane, of byte `b` (0..127) of
+// superblock `sb`.  A slice is 16 superblocks = 64 "pairs" of 32 bytes (pair p
+// of a superblock = bytes 32p..32p+31 = sub-blocks 2p (low nibbles) and 2p+1
+// (high nibbles)).  Inside a slice holding P pairs, the first 16 bytes of every
+// pair come first (16 B x P, pair-major), then the second 16 bytes of every pair.
+__host__ __device__ static inline size_t q4k_code_offset(int64_t nsb_row, int64_t sb, int b) {
+    int64_t slice = sb >> 4;
+    int64_t sb_in = sb & 15;
+    int64_t nsb_slice = (nsb_row - (slice << 4)) < 16 ? (nsb_row - (slice << 4)) : 16;
+    int64_t P = nsb_slice * 4;
+    int64_t pair = sb_in * 4 + (b >> 5);
+    int half = (b >> 4) & 1;
+    return (size_t)(slice * 2048 + (int64_t)half * 16 * P + pair * 16 + (b & 15));
+}
+
+// Error helpers -------------------------------------------------------------
+int axq_fail(axq_ctx *ctx, int code, const char *fmt, ...);
+#define AXQ_HIP(ctx, call, code)                                                              \
+    do {                                                                                      \
+        hipError_t e_ = (call);                                                               \
+        if (e_ != hipSuccess) return axq_fail((ctx), (code), "%s: %s", #call, hipGetErrorString(e_)); \
+    } while (0)
+#define AXQ_LAUNCH_CHECK(ctx, what)                                                           \
+    do {                                                                                      \
+        hipError_t e_ = hipGetLastError();                                                    \
+        if (e_ != hipSuccess)                                                                 \
+            return axq_fail((ctx), AXQ_ERR_KERNEL_LAUNCH_FAILED, "%s: %s", (what), hipGetErrorString(e_)); \
+    } while (0)
+
+// Cross-TU entry points -----------------------------------------------------
+// codec.hip
+int axq_dev_quantize(axq_ctx *ctx, int type, const float *src_dev, size_t numel, uint8_t *packed_dev);
+int axq_dev_dequantize(axq_ctx *ctx, int type, const uint8_t *packed_dev, size_t numel, float *dst_dev);
+int axq_dev_repack(axq_ctx *ctx, const axq_weight *w, uint8_t *packed_dev, bool to_planar);
+// weight.hip
+int axq_weight_alloc(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, axq_weight **out);
+// gemv.hip
+int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x_dev, int batch, const float *bias_dev, float *y_dev);
+// gemm.hip
+int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_dev, int m, float *y_dev);

@@ -1,0 +1,279 @@
+// Codec and weight entry points of the C ABI (host-side staging around the
+// device kernels of axq_codec.hip).
+#include <stdlib.h>
+
+#include "axq_internal.h"
+
+namespace {
+
+// RAII for a temporary device buffer on the context's stream.
+struct DevTemp {
+    axq_ctx *ctx;
+    void *p = nullptr;
+    explicit DevTemp(axq_ctx *c) : ctx(c) {}
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 1); }
+    ~DevTemp() {
+        if (p) {
+            (void)hipStreamSynchronize(ctx->stream);
+            (void)hipFree(p);
+        }
+    }
+};
+
+int check_type(axq_ctx *ctx, int type) {
+    if (axq_type_block_size(type) == 0)
+        return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", type);
+    return AXQ_OK;
+}
+
+int check_mem(axq_ctx *ctx, int mem) {
+    if (mem != AXQ_MEM_HOST && mem != AXQ_MEM_DEVICE)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "mem must be AXQ_MEM_HOST or AXQ_MEM_DEVICE, got %d", mem);
+    return AXQ_OK;
+}
+
+} // namespace
+
+int axq_weight_alloc(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, axq_weight **out) {
+    size_t bs = axq_type_block_size(type);
+    if (n_rows <= 0 || k <= 0)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight must be [n_rows>0, k>0], got [%lld, %lld]",
+                        (long long)n_rows, (long long)k);
+    if ((size_t)k % bs != 0)
+        return axq_fail(ctx, AXQ_ERR_INVALID_BLOCK_SIZE,
+                        "Invalid block size: k=%lld is not a multiple of the %zu-element block of %s", (long long)k, bs,
+                        axq_type_name(type));
+    axq_weight *w = (axq_weight *)calloc(1, sizeof(axq_weight));
+    if (!w) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "out of host memory");
+    w->type = type;
+    w->n_rows = n_rows;
+    w->k = k;
+    w->packed_bytes = axq_packed_bytes(type, (size_t)n_rows * (size_t)k);
+    size_t nblk = (size_t)k / bs;
+    size_t meta_per_block = 0, qh_per_block = 0;
+    switch (type) {
+    case AXQ_Q8_0: w->codes_pitch = (size_t)k; meta_per_block = 2; break;
+    case AXQ_Q4_0: w->codes_pitch = (size_t)k / 2; meta_per_block = 2; break;
+    case AXQ_Q4_1: w->codes_pitch = (size_t)k / 2; meta_per_block = 4; break;
+    case AXQ_Q5_0: w->codes_pitch = (size_t)k / 2; meta_per_block = 2; qh_per_block = 4; break;
+    case AXQ_Q5_1: w->codes_pitch = (size_t)k / 2; meta_per_block = 4; qh_per_block = 4; break;
+    case AXQ_Q4_K: w->codes_pitch = (size_t)k / 2; meta_per_block = 16; break;
+    case AXQ_F16: w->codes_pitch = (size_t)k * 2; break;
+    case AXQ_F32: w->codes_pitch = (size_t)k * 4; break;
+    }
+    w->meta_pitch = nblk * meta_per_block;
+    w->qh_pitch = nblk * qh_per_block;
+    size_t codes_bytes = axq_align_up(w->codes_pitch * (size_t)n_rows, 256);
+    size_t meta_bytes = axq_align_up(w->meta_pitch * (size_t)n_rows, 256);
+    size_t qh_bytes = axq_align_up(w->qh_pitch * (size_t)n_rows, 256);
+    // 64 bytes of slack: the GEMV kernels may read (and discard) up to one
+    // 16-byte vector past the last real byte of a plane.
+    w->alloc_bytes = codes_bytes + meta_bytes + qh_bytes + 256;
+    hipError_t e = hipMalloc((void **)&w->base, w->alloc_bytes);
+    if (e != hipSuccess) {
+        free(w);
+        return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "hipMalloc(%zu): %s", w->alloc_bytes, hipGetErrorString(e));
+    }
+    w->codes = w->base;
+    w->meta = w->base + codes_bytes;
+    w->qh = w->meta + meta_bytes;
+    w->owns = true;
+    // zero the padding so that stray vector reads are deterministic
+    e = hipMemsetAsync(w->base, 0, w->alloc_bytes, ctx->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(w->base);
+        free(w);
+        return axq_fail(ctx, AXQ_ERR_DRIVER, "hipMemsetAsync: %s", hipGetErrorString(e));
+    }
+    *out = w;
+    return AXQ_OK;
+}
+
+extern "C" {
+
+int axq_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, void *packed, int mem) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_quantize: NULL context");
+    int rc;
+    if ((rc = check_type(ctx, type)) || (rc = check_mem(ctx, mem))) return rc;
+    if (numel == 0) return AXQ_OK;
+    if (!src || !packed) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_quantize: NULL pointer");
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    size_t bytes = axq_packed_bytes(type, numel);
+    if (mem == AXQ_MEM_DEVICE) return axq_dev_quantize(ctx, type, src, numel, (uint8_t *)packed);
+    DevTemp dsrc(ctx), dout(ctx);
+    AXQ_HIP(ctx, dsrc.alloc(numel * 4), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, dout.alloc(bytes), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, hipMemcpyAsync(dsrc.p, src, numel * 4, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    if ((rc = axq_dev_quantize(ctx, type, (const float *)dsrc.p, numel, (uint8_t *)dout.p))) return rc;
+    AXQ_HIP(ctx, hipMemcpyAsync(packed, dout.p, bytes, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_dequantize(axq_ctx *ctx, int type, const void *packed, size_t numel, float *dst, int mem) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_dequantize: NULL context");
+    int rc;
+    if ((rc = check_type(ctx, type)) || (rc = check_mem(ctx, mem))) return rc;
+    if (numel == 0) return AXQ_OK;
+    if (!dst || !packed) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_dequantize: NULL pointer");
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    size_t bytes = axq_packed_bytes(type, numel);
+    if (mem == AXQ_MEM_DEVICE) return axq_dev_dequantize(ctx, type, (const uint8_t *)packed, numel, dst);
+    DevTemp dsrc(ctx), dout(ctx);
+    AXQ_HIP(ctx, dsrc.alloc(bytes), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, dout.alloc(numel * 4), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, hipMemcpyAsync(dsrc.p, packed, bytes, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    if ((rc = axq_dev_dequantize(ctx, type, (const uint8_t *)dsrc.p, numel, (float *)dout.p))) return rc;
+    AXQ_HIP(ctx, hipMemcpyAsync(dst, dout.p, numel * 4, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_weight_upload(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, const void *packed, size_t bytes, int mem,
+                      axq_weight **out) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_weight_upload: NULL context");
+    if (!out || !packed) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_weight_upload: NULL pointer");
+    *out = NULL;
+    int rc;
+    if ((rc = check_type(ctx, type)) || (rc = check_mem(ctx, mem))) return rc;
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    axq_weight *w = NULL;
+    if ((rc = axq_weight_alloc(ctx, type, n_rows, k, &w))) return rc;
+    if (bytes != w->packed_bytes) {
+        rc = axq_fail(ctx, AXQ_ERR_DATA_LENGTH_MISMATCH, "Data length mismatch: expected %zu, got %zu", w->packed_bytes,
+                      bytes);
+        axq_weight_free(ctx, w);
+        return rc;
+    }
+    if (mem == AXQ_MEM_DEVICE) {
+        rc = axq_dev_repack(ctx, w, (uint8_t *)packed, true);
+    } else {
+        DevTemp tmp(ctx);
+        hipError_t e = tmp.alloc(bytes);
+        if (e == hipSuccess) e = hipMemcpyAsync(tmp.p, packed, bytes, hipMemcpyHostToDevice, ctx->stream);
+        if (e != hipSuccess)
+            rc = axq_fail(ctx, AXQ_ERR_COPY_FAILED, "staging upload: %s", hipGetErrorString(e));
+        else
+            rc = axq_dev_repack(ctx, w, (uint8_t *)tmp.p, true);
+    }
+    if (rc) {
+        axq_weight_free(ctx, w);
+        return rc;
+    }
+    *out = w;
+    return AXQ_OK;
+}
+
+int axq_weight_quantize(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, const float *wsrc, int mem, axq_weight **out) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_weight_quantize: NULL context");
+    if (!out || !wsrc) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_weight_quantize: NULL pointer");
+    *out = NULL;
+    int rc;
+    if ((rc = check_type(ctx, type)) || (rc = check_mem(ctx, mem))) return rc;
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    axq_weight *w = NULL;
+    if ((rc = axq_weight_alloc(ctx, type, n_rows, k, &w))) return rc;
+    size_t numel = (size_t)n_rows * (size_t)k;
+    {
+        DevTemp fsrc(ctx), img(ctx);
+        const float *src_dev = wsrc;
+        hipError_t e = hipSuccess;
+        if (mem == AXQ_MEM_HOST) {
+            e = fsrc.alloc(numel * 4);
+            if (e == hipSuccess) e = hipMemcpyAsync(fsrc.p, wsrc, numel * 4, hipMemcpyHostToDevice, ctx->stream);
+            src_dev = (const float *)fsrc.p;
+        }
+        if (e == hipSuccess) e = img.alloc(w->packed_bytes);
+        if (e != hipSuccess)
+            rc = axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "staging quantize: %s", hipGetErrorString(e));
+        if (!rc) rc = axq_dev_quantize(ctx, type, src_dev, numel, (uint8_t *)img.p);
+        if (!rc) rc = axq_dev_repack(ctx, w, (uint8_t *)img.p, true);
+    }
+    if (rc) {
+        axq_weight_free(ctx, w);
+        return rc;
+    }
+    *out = w;
+    return AXQ_OK;
+}
+
+int axq_weight_download(axq_ctx *ctx, const axq_weight *w, void *packed, size_t bytes, int mem) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_weight_download: NULL context");
+    if (!w || !packed) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_weight_download: NULL pointer");
+    int rc;
+    if ((rc = check_mem(ctx, mem))) return rc;
+    if (bytes != w->packed_bytes)
+        return axq_fail(ctx, AXQ_ERR_DATA_LENGTH_MISMATCH, "Data length mismatch: expected %zu, got %zu", w->packed_bytes,
+                        bytes);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    if (mem == AXQ_MEM_DEVICE) return axq_dev_repack(ctx, w, (uint8_t *)packed, false);
+    DevTemp tmp(ctx);
+    AXQ_HIP(ctx, tmp.alloc(bytes), AXQ_ERR_ALLOCATION_FAILED);
+    if ((rc = axq_dev_repack(ctx, w, (uint8_t *)tmp.p, false))) return rc;
+    AXQ_HIP(ctx, hipMemcpyAsync(packed, tmp.p, bytes, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_weight_info(const axq_weight *w, int *type, int64_t *n_rows, int64_t *k, size_t *bytes) {
+    if (!w) return AXQ_ERR_INVALID_ARGUMENT;
+    if (type) *type = w->type;
+    if (n_rows) *n_rows = w->n_rows;
+    if (k) *k = w->k;
+    if (bytes) *bytes = w->packed_bytes;
+    return AXQ_OK;
+}
+
+void axq_weight_free(axq_ctx *ctx, axq_weight *w) {
+    if (!w) return;
+    if (w->owns && w->base) {
+        if (ctx) (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(w->base);
+    }
+    free(w);
+}
+
+int axq_gemv_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y, int mem) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_gemv_f32: NULL context");
+    if (!w || !x || !y) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_gemv_f32: NULL pointer");
+    int rc;
+    if ((rc = check_mem(ctx, mem))) return rc;
+    if (batch <= 0) return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: batch must be positive, got %d", batch);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    if (mem == AXQ_MEM_DEVICE) return axq_dev_gemv(ctx, w, x, batch, bias, y);
+    size_t xb = (size_t)batch * (size_t)w->k * 4, yb = (size_t)batch * (size_t)w->n_rows * 4;
+    DevTemp dx(ctx), dy(ctx), db(ctx);
+    AXQ_HIP(ctx, dx.alloc(xb), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, dy.alloc(yb), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, hipMemcpyAsync(dx.p, x, xb, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    if (bias) {
+        AXQ_HIP(ctx, db.alloc((size_t)w->n_rows * 4), AXQ_ERR_ALLOCATION_FAILED);
+        AXQ_HIP(ctx, hipMemcpyAsync(db.p, bias, (size_t)w->n_rows * 4, hipMemcpyHostToDevice, ctx->stream),
+                AXQ_ERR_COPY_FAILED);
+    }
+    if ((rc = axq_dev_gemv(ctx, w, (const float *)dx.p, batch, (const float *)db.p, (float *)dy.p))) return rc;
+    AXQ_HIP(ctx, hipMemcpyAsync(y, dy.p, yb, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y, int mem) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_gemm_bf16: NULL context");
+    if (!w || !x || !y) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_gemm_bf16: NULL pointer");
+    int rc;
+    if ((rc = check_mem(ctx, mem))) return rc;
+    if (m <= 0) return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: m must be positive, got %d", m);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    if (mem == AXQ_MEM_DEVICE) return axq_dev_gemm_bf16(ctx, w, x, m, y);
+    size_t xb = (size_t)m * (size_t)w->k * 2, yb = (size_t)m * (size_t)w->n_rows * 4;
+    DevTemp dx(ctx), dy(ctx);
+    AXQ_HIP(ctx, dx.alloc(xb), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, dy.alloc(yb), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, hipMemcpyAsync(dx.p, x, xb, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    if ((rc = axq_dev_gemm_bf16(ctx, w, (const uint16_t *)dx.p, m, (float *)dy.p))) return rc;
+    AXQ_HIP(ctx, hipMemcpyAsync(y, dy.p, yb, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+} // extern "C"

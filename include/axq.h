@@ -1,0 +1,200 @@
+/*
+ * axq -- MI355X (gfx950) block-quantized matmul path, C ABI.
+ *
+ * This is the drop-in boundary for the `axonml-quant` crate's path
+ * (quantize -> QuantizedTensor -> dequantize / quantized matmul) as an
+ * `axonml-llm` decode or prefill loop would use it.  Every entry point is
+ * plain C: opaque handles, pointers and sizes.  All compute runs in HIP
+ * kernels on the device; there is no CPU fallback -- without a usable GPU
+ * axq_init() fails with AXQ_ERR_DEVICE_NOT_FOUND and nothing else can be
+ * called.
+ *
+ * Conventions
+ *   - Every function returns AXQ_OK (0) or a negative axq_status; none aborts
+ *     and no C++ exception crosses the boundary.  axq_last_error() gives the
+ *     text of the last failure on a context (or of the last failed axq_init
+ *     when called with NULL).
+ *   - "packed" buffers are the concatenation, in block order, of the
+ *     reference's per-block byte images (`to_bytes`,
+ *     crates/axonml-quant/src/types.rs:142-147, 201-206, 249-255); Q5_0, Q5_1
+ *     and Q4_K use the GGUF block layouts.  Blocks run along the flat
+ *     row-major buffer (crates/axonml-quant/src/quantize.rs:84-91).
+ *   - `mem` says where the caller's data pointers live: AXQ_MEM_HOST (the
+ *     library stages them through the device) or AXQ_MEM_DEVICE (used in
+ *     place, on the context's stream, no synchronisation).
+ *   - A context owns one HIP stream (or adopts the caller's through
+ *     axq_set_stream).  Calls on one context must not overlap; distinct
+ *     contexts are independent.  This mirrors the reference CUDA backend's
+ *     "one device, default stream, Send but not re-entrant" convention
+ *     (crates/axonml-core/src/backends/cuda.rs:34-35, 52-55, 224-226).
+ */
+#ifndef AXQ_H
+#define AXQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AXQ_API __attribute__((visibility("default")))
+
+typedef struct axq_ctx axq_ctx;
+typedef struct axq_weight axq_weight;
+typedef struct axq_model axq_model;
+
+/* QuantType, crates/axonml-quant/src/types.rs:17-41, in the same order, with
+ * Q4_K (256-element GGUF superblock) appended. */
+typedef enum {
+    AXQ_Q8_0 = 0,
+    AXQ_Q4_0 = 1,
+    AXQ_Q4_1 = 2,
+    AXQ_Q5_0 = 3,
+    AXQ_Q5_1 = 4,
+    AXQ_F16 = 5,
+    AXQ_F32 = 6,
+    AXQ_Q4_K = 7,
+    AXQ_TYPE_COUNT = 8
+} axq_type;
+
+typedef enum {
+    AXQ_OK = 0,
+    /* QuantError, crates/axonml-quant/src/error.rs:14-57 */
+    AXQ_ERR_INVALID_BLOCK_SIZE = -1,
+    AXQ_ERR_INVALID_QUANT_TYPE = -2,
+    AXQ_ERR_SHAPE_MISMATCH = -3,
+    AXQ_ERR_DATA_LENGTH_MISMATCH = -4,
+    AXQ_ERR_CALIBRATION = -5,
+    AXQ_ERR_OVERFLOW = -6,
+    AXQ_ERR_INVALID_DATA = -7,
+    AXQ_ERR_TENSOR_CONVERSION = -8,
+    /* CudaError, crates/axonml-core/src/backends/cuda.rs:272-289 */
+    AXQ_ERR_DEVICE_NOT_FOUND = -20,
+    AXQ_ERR_ALLOCATION_FAILED = -21,
+    AXQ_ERR_COPY_FAILED = -22,
+    AXQ_ERR_KERNEL_LAUNCH_FAILED = -23,
+    AXQ_ERR_DRIVER = -24,
+    /* boundary misuse (NULL handle or pointer, bad flag) */
+    AXQ_ERR_INVALID_ARGUMENT = -30
+} axq_status;
+
+typedef enum { AXQ_MEM_HOST = 0, AXQ_MEM_DEVICE = 1 } axq_mem;
+
+/* ---- type registry: QuantType methods, types.rs:45-120 ------------------- */
+AXQ_API size_t axq_type_block_size(int type);      /* block_size(), :45-54; 0 if unknown */
+AXQ_API size_t axq_type_bytes_per_block(int type); /* bytes_per_block(), :57-67 */
+AXQ_API size_t axq_type_bits_per_value(int type);  /* bits_per_value(), :70-78 */
+AXQ_API int axq_type_is_block_quantized(int type); /* is_block_quantized(), :86-91 */
+AXQ_API const char *axq_type_name(int type);       /* Display, :108-120; NULL if unknown */
+AXQ_API int axq_type_from_str(const char *s);      /* from_str() with its aliases, :94-105; -1 if unknown */
+AXQ_API size_t axq_num_blocks(int type, size_t numel);   /* ceil(numel / block), quantize.rs:84 */
+AXQ_API size_t axq_packed_bytes(int type, size_t numel); /* QuantizedTensor::size_bytes, types.rs:320-322 */
+AXQ_API const char *axq_status_str(int status);
+
+/* ---- device context: Backend trait, backends/mod.rs:73-100, and
+ *      CudaBackend::new -> Option, backends/cuda.rs:69-81 ------------------ */
+typedef struct {
+    char name[128];
+    char arch[32];
+    int32_t compute_units;
+    int32_t wavefront_size;
+    int32_t lds_bytes_per_cu;
+    int32_t clock_mhz;
+    uint64_t hbm_bytes;
+} axq_device_info_t;
+
+AXQ_API int axq_init(int device, axq_ctx **out);
+AXQ_API void axq_destroy(axq_ctx *ctx);
+AXQ_API const char *axq_last_error(axq_ctx *ctx);
+AXQ_API int axq_device_info(axq_ctx *ctx, axq_device_info_t *out);   /* capabilities() */
+AXQ_API int axq_malloc(axq_ctx *ctx, size_t bytes, void **dptr);     /* allocate() */
+AXQ_API int axq_free(axq_ctx *ctx, void *dptr);                      /* deallocate() */
+AXQ_API int axq_copy_to_device(axq_ctx *ctx, void *dst, const void *src, size_t bytes);
+AXQ_API int axq_copy_to_host(axq_ctx *ctx, void *dst, const void *src, size_t bytes);
+AXQ_API int axq_copy_device_to_device(axq_ctx *ctx, void *dst, const void *src, size_t bytes);
+AXQ_API int axq_synchronize(axq_ctx *ctx);                           /* synchronize() */
+/* Adopt a caller-owned hipStream_t (NULL = back to the context's own). */
+AXQ_API int axq_set_stream(axq_ctx *ctx, void *hip_stream);
+/* HIP-event stopwatch on the context's stream (for the benchmark). */
+AXQ_API int axq_timer_start(axq_ctx *ctx);
+AXQ_API int axq_timer_stop(axq_ctx *ctx, float *elapsed_ms); /* synchronises on the stop event */
+
+/* ---- codecs: quantize_tensor (quantize.rs:36-54) and dequantize_tensor
+ *      (dequantize.rs:34-54), run on the device ---------------------------- */
+/* src: numel f32; packed: axq_packed_bytes(type, numel) bytes. */
+AXQ_API int axq_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, void *packed, int mem);
+/* dst: numel f32 (the tail block is truncated, dequantize.rs:44-50). */
+AXQ_API int axq_dequantize(axq_ctx *ctx, int type, const void *packed, size_t numel, float *dst, int mem);
+
+/* ---- device-resident weights: QuantizedTensor (types.rs:296-334) of shape
+ *      [n_rows, k] as a Linear weight (nn/src/layers/linear.rs:41-42) -------- */
+/* Copies `packed` (bytes must equal axq_packed_bytes(type, n_rows*k)); the
+ * caller keeps ownership of its buffer.  k must be a multiple of the block. */
+AXQ_API int axq_weight_upload(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, const void *packed, size_t bytes,
+                              int mem, axq_weight **out);
+/* quantize_tensor straight into a device-resident weight. */
+AXQ_API int axq_weight_quantize(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, const float *w, int mem,
+                                axq_weight **out);
+/* Returns the exact bytes that were uploaded / produced by the quantiser. */
+AXQ_API int axq_weight_download(axq_ctx *ctx, const axq_weight *w, void *packed, size_t bytes, int mem);
+AXQ_API int axq_weight_info(const axq_weight *w, int *type, int64_t *n_rows, int64_t *k, size_t *bytes);
+AXQ_API void axq_weight_free(axq_ctx *ctx, axq_weight *w);
+
+/* ---- quantized matmul: the composition dequantize_tensor -> Tensor::matmul
+ *      (tensor/src/tensor.rs:1020-1045) behind Linear::forward
+ *      (nn/src/layers/linear.rs:104-140), fused ------------------------------ */
+/* y[batch, n_rows] = x[batch, k] * W^T (+ bias[n_rows] if non-NULL), f32.
+ * Decode path (batch small); bias lives where x and y live. */
+AXQ_API int axq_gemv_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y,
+                         int mem);
+/* y[m, n_rows] = x[m, k] * W^T, x in bf16 (raw uint16), y f32.  Prefill path. */
+AXQ_API int axq_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_bf16, int m, float *y, int mem);
+
+/* ---- decode: LLaMA/Mistral-shape model, llm/src/llama.rs:731-762, 900-977 - */
+/* Field names follow LLaMAConfig / MistralConfig (llama.rs:56-121, mistral.rs:56-70). */
+typedef struct {
+    int32_t vocab_size, hidden_size, intermediate_size, num_hidden_layers;
+    int32_t num_attention_heads, num_key_value_heads, head_dim, max_position_embeddings;
+    float rms_norm_eps, rope_theta;
+} axq_model_config;
+
+typedef enum {
+    AXQ_LIN_Q = 0, AXQ_LIN_K, AXQ_LIN_V, AXQ_LIN_O, AXQ_LIN_GATE, AXQ_LIN_UP, AXQ_LIN_DOWN, AXQ_LIN_COUNT
+} axq_linear_id;
+
+AXQ_API int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out);
+AXQ_API void axq_model_free(axq_model *m);
+/* f16 table [vocab, hidden] (Embedding::lookup, nn/src/layers/embedding.rs:103-146). */
+AXQ_API int axq_model_set_embedding_f16(axq_model *m, const uint16_t *table, int mem);
+/* layer -1 = final norm; which 0 = attention norm, 1 = ffn norm.  f32[hidden]. */
+AXQ_API int axq_model_set_norm(axq_model *m, int layer, int which, const float *w, int mem);
+/* layer -1 = lm_head.  The model copies the weight's blocks; the caller may free `w`. */
+AXQ_API int axq_model_set_linear(axq_model *m, int layer, int which, const axq_weight *w);
+/* Fill every linear (Q4_K by default), the embedding and unit norms from a
+ * seeded device generator: N(0, std) weights.  For benchmarks of random-init
+ * models too large to stage through the host. */
+AXQ_API int axq_model_random_init(axq_model *m, int type, float std, uint64_t seed);
+/* KVCache::clear (attention.rs:80-83). */
+AXQ_API int axq_model_reset(axq_model *m);
+/* forward_with_cache for one token at the cache's current length; appends to
+ * the cache.  logits (f32[vocab], host) may be NULL.  next_token (host) may be NULL. */
+AXQ_API int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_t *next_token);
+/* generate (llama.rs:900-977), greedy: feeds the prompt, then max_new_tokens
+ * steps, each consuming the previous argmax on the device.  out_tokens gets
+ * max_new_tokens ids (host).  Timings (ms, may be NULL) cover prompt and
+ * generation separately. */
+AXQ_API int axq_model_generate(axq_model *m, const int32_t *prompt, int n_prompt, int max_new_tokens,
+                               int32_t *out_tokens, float *prefill_ms, float *decode_ms);
+AXQ_API int axq_model_seq_len(const axq_model *m);
+
+/* ---- benchmark utilities ------------------------------------------------- */
+/* dst[i] ~ N(mean, std) from a counter-based generator (seed, i); with
+ * outlier_p > 0 each element is instead +/-outlier_mag with that probability. */
+AXQ_API int axq_fill_normal_f32(axq_ctx *ctx, float *dst_dev, size_t n, float mean, float std, float outlier_p,
+                                float outlier_mag, uint64_t seed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AXQ_H */

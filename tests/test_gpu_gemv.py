@@ -1,0 +1,112 @@
+"""GPU parity: the decode-path quantized matmul against the CPU oracle.
+
+Bar (north star): max relative error <= 1e-3 against the reference f32 result (accumulation order
+differs), relative error taken against max(|ref_i|, 1e-3 * max|ref|); plus the reference GPU harness's
+own |a-b| <= atol + rtol|b| form (backends/gpu_tests.rs:221-249) with rtol = 1e-3."""
+import numpy as np
+import pytest
+
+import oracle as o
+from axonml_amd import quant as q
+from tests.util import MATMUL_RTOL, assert_close_ref_style, gen_weight, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.F16, o.F32]
+
+
+def _check(ctx, qtype, n, k, batch, seed, outlier_p=0.0, bias=False):
+    rng = np.random.default_rng(seed)
+    w = gen_weight(rng, n, k, outlier_p=outlier_p)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32) if bias else None
+    wq = o.quantize(qtype, w)
+    want = o.matmul_ref(qtype, wq, x, n, k, b)
+    got = q.quantized_matmul(x, q.QuantizedTensor([n, k], qtype, wq), b, ctx)
+    assert got.shape == (batch, n)
+    err = max_rel_err(got, want)
+    assert err <= MATMUL_RTOL, f"{o.TYPE_NAMES[qtype]} [{n},{k}] b={batch}: max rel err {err:.3e}"
+    assert_close_ref_style(got, want, atol=1e-5 * float(np.abs(want).max()), rtol=MATMUL_RTOL)
+    return got, want
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("n,k", [(1, 256), (5, 256), (64, 512), (33, 2048), (17, 4096), (130, 4096 + 512),
+                                  (9, 11008), (12, 14336), (4, 32768 + 2048)])
+def test_gemv_small_shapes(ctx, qtype, n, k):
+    if qtype == o.Q4_K and k % 256:
+        pytest.skip("k must be a multiple of 256 for Q4_K")
+    _check(ctx, qtype, n, k, 1, seed=n * 7 + k)
+
+
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q5_1, o.Q8_0, o.Q4_K])
+@pytest.mark.parametrize("batch", [2, 8])
+def test_gemv_batched_with_bias(ctx, qtype, batch):
+    _check(ctx, qtype, 96, 4096, batch, seed=batch, bias=True)
+
+
+def test_config_q8_0_4096x4096(ctx):
+    _check(ctx, o.Q8_0, 4096, 4096, 1, seed=1)
+
+
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1])
+@pytest.mark.parametrize("n,k", [(11008, 4096), (4096, 11008)])
+@pytest.mark.parametrize("batch", [1, 8])
+def test_config_q4_0_q4_1(ctx, qtype, n, k, batch):
+    _check(ctx, qtype, n, k, batch, seed=2)
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+def test_config_q4_k_headline(ctx, n, k):
+    _check(ctx, o.Q4_K, n, k, 1, seed=3, outlier_p=0.01)
+
+
+@pytest.mark.parametrize("qtype", ALL)
+def test_one_hot_activation_selects_dequantised_column(ctx, qtype):
+    # exactness of the in-register unpack: y = W[:, col] up to the scale factorisation's rounding
+    rng = np.random.default_rng(21)
+    n, k = 40, 1024
+    w = gen_weight(rng, n, k)
+    wq = o.quantize(qtype, w)
+    wd = o.dequantize(qtype, wq, n * k).reshape(n, k)
+    qt = q.QuantizedTensor([n, k], qtype, wq)
+    dw = q.DeviceWeight.upload(qt, ctx)
+    for col in (0, 1, 15, 16, 31, 32, 63, 64, 255, 256, 511, 1023):
+        x = np.zeros((1, k), np.float32)
+        x[0, col] = 1.0
+        y = q.quantized_matmul(x, dw, None, ctx)[0]
+        assert np.allclose(y, wd[:, col], rtol=1e-5, atol=1e-6 * float(np.abs(wd).max())), (o.TYPE_NAMES[qtype], col)
+    dw.free()
+
+
+def test_linearity_and_determinism_at_full_size(ctx):
+    rng = np.random.default_rng(8)
+    n, k = 4096, 14336
+    dw = q.DeviceWeight.quantize(gen_weight(rng, n, k, outlier_p=0.01), q.QuantType.Q4_K, ctx)
+    x1 = rng.standard_normal((1, k)).astype(np.float32)
+    x2 = rng.standard_normal((1, k)).astype(np.float32)
+    y1 = q.quantized_matmul(x1, dw, None, ctx)
+    y2 = q.quantized_matmul(x2, dw, None, ctx)
+    y12 = q.quantized_matmul(x1 + 2 * x2, dw, None, ctx)
+    assert max_rel_err(y12, y1.astype(np.float64) + 2 * y2.astype(np.float64)) < 1e-4
+    assert np.array_equal(q.quantized_matmul(x1, dw, None, ctx), y1)  # no atomics: run-to-run identical
+    dw.free()
+
+
+def test_quantized_linear_keeps_leading_dims(ctx):
+    rng = np.random.default_rng(4)
+    w = gen_weight(rng, 48, 512)
+    lin = q.QuantizedLinear(q.quantize_tensor(w, q.QuantType.Q4_1, ctx), rng.standard_normal(48).astype(np.float32), ctx)
+    x = rng.standard_normal((2, 3, 512)).astype(np.float32)
+    y = lin(x)
+    assert y.shape == (2, 3, 48)
+    want = o.matmul_ref(o.Q4_1, o.quantize(o.Q4_1, w), x.reshape(6, 512), 48, 512, lin.bias).reshape(2, 3, 48)
+    assert max_rel_err(y, want) <= MATMUL_RTOL
+
+
+def test_gemv_shape_errors(ctx):
+    w = q.quantize_tensor(np.zeros((4, 256), np.float32), q.QuantType.Q8_0, ctx)
+    with pytest.raises(q.ShapeMismatch):
+        q.quantized_matmul(np.zeros((1, 128), np.float32), w, None, ctx)
+    with pytest.raises(q.ShapeMismatch):
+        q.quantized_matmul(np.zeros((1, 256), np.float32), w, np.zeros(3, np.float32), ctx)

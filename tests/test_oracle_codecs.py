@@ -1,0 +1,350 @@
+"""Pins the CPU oracle's codecs (oracle/axq_oracle.c) without a GPU.
+
+Sources of truth used here, none of which is the oracle's own formula retyped:
+  * hand-computed known-answer blocks derived from the reference source
+    (crates/axonml-quant/src/quantize.rs, dequantize.rs, types.rs) with scales
+    chosen as powers of two so that every expected code is an obvious integer;
+  * the inputs and tolerances of the reference's own unit tests
+    (types.rs:344-389, quantize.rs:294-345, dequantize.rs:204-272);
+  * numpy's float16 (an independent IEEE binary16 implementation) for the f16
+    conversions the `half` crate performs;
+  * the GGUF block spec, transcribed independently in numpy, for Q5_0/Q5_1/Q4_K.
+"""
+import numpy as np
+import pytest
+
+import oracle as o
+
+
+def u16(p, i):
+    return int(p[i]) | (int(p[i + 1]) << 8)
+
+
+def f16_bits(v):
+    return int(np.array([v], dtype=np.float32).astype(np.float16).view(np.uint16)[0])
+
+
+# --------------------------------------------------------------------------- f16 conversion
+def test_f32_to_f16_matches_numpy_at_every_boundary():
+    # Every finite binary16 value, the midpoint to its successor, and one f32 ulp either side.
+    h = np.arange(0, 0x7C00, dtype=np.uint16)
+    v = h.view(np.float16).astype(np.float64)
+    nxt = (h + 1).view(np.float16).astype(np.float64)
+    nxt[-1] = 65536.0  # the rounding boundary to infinity is 65520
+    mid = ((v + nxt) / 2).astype(np.float32)
+    cand = np.concatenate([v.astype(np.float32), mid, np.nextafter(mid, np.float32(np.inf)),
+                           np.nextafter(mid, np.float32(-np.inf))])
+    cand = np.concatenate([cand, -cand, np.array([np.inf, -np.inf, 1e-10, -1e-10, 7e4, 6.0e-8, 2.9e-8, 3.0e-8],
+                                                 dtype=np.float32)])
+    want = cand.astype(np.float16).view(np.uint16)
+    got = o.f32_to_f16_bits(cand)
+    bad = np.nonzero(want != got)[0]
+    assert bad.size == 0, f"{bad.size} mismatches, first: x={cand[bad[0]]!r} want={want[bad[0]]:#x} got={got[bad[0]]:#x}"
+
+
+def test_f16_to_f32_matches_numpy_for_all_bit_patterns():
+    h = np.arange(0, 0x10000, dtype=np.uint32).astype(np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = o.f16_bits_to_f32(h)
+    finite = np.isfinite(want)
+    assert np.array_equal(want[finite].view(np.uint32), got[finite].view(np.uint32))
+    assert np.array_equal(np.isnan(want), np.isnan(got))
+    assert np.array_equal(want[np.isinf(want)], got[np.isinf(want)])
+
+
+def test_nan_keeps_being_nan():
+    assert (o.f32_to_f16_bits(np.array([np.nan], dtype=np.float32))[0] & 0x7FFF) > 0x7C00
+
+
+# --------------------------------------------------------------------------- registry (types.rs:45-78)
+def test_registry_sizes():
+    L = o.lib()
+    expect = {o.Q8_0: (32, 34), o.Q4_0: (32, 18), o.Q4_1: (32, 20), o.Q5_0: (32, 22), o.Q5_1: (32, 24),
+              o.F16: (1, 2), o.F32: (1, 4), o.Q4_K: (256, 144)}
+    for t, (bs, bb) in expect.items():
+        assert L.axo_block_size(t) == bs and L.axo_bytes_per_block(t) == bb
+    # quantize.rs:294-313: 8 elements -> 1 block, 64 -> 2 blocks
+    assert L.axo_num_blocks(o.Q8_0, 8) == 1 and L.axo_num_blocks(o.Q4_0, 64) == 2
+    assert L.axo_block_size(99) == 0
+
+
+# --------------------------------------------------------------------------- Q8_0 (quantize.rs:82-114)
+def test_q8_0_zero_block_has_scale_one():
+    p = o.quantize(o.Q8_0, np.zeros(32, np.float32))
+    assert p[0] == 0x00 and p[1] == 0x3C  # f16 1.0, little endian (types.rs:144)
+    assert not p[2:].any()
+
+
+def test_q8_0_rounds_half_away_from_zero():
+    # max_abs = 127 -> scale = 1.0 exactly, so q = round(x): Rust's f32::round, not round-half-even.
+    x = np.zeros(32, np.float32)
+    x[:10] = [127, -127, 0.5, -0.5, 1.5, 2.5, -2.5, 3.49, -3.51, 126.5]
+    p = o.quantize(o.Q8_0, x)
+    assert (p[0], p[1]) == (0x00, 0x3C)
+    assert p[2:12].view(np.int8).tolist() == [127, -127, 1, -1, 2, 3, -3, 3, -4, 127]
+    assert not p[12:].any()
+
+
+def test_q8_0_power_of_two_scale_and_f16_rounding_of_scale():
+    x = np.zeros(32, np.float32)
+    x[:4] = [254, 1, 3, 5]  # scale = 2.0 -> 0x4000; 0.5 -> 1, 1.5 -> 2, 2.5 -> 3
+    p = o.quantize(o.Q8_0, x)
+    assert u16(p, 0) == 0x4000
+    assert p[2:6].view(np.int8).tolist() == [127, 1, 2, 3]
+    # the quantiser divides by the f32 scale but stores its f16 rounding (quantize.rs:100-109)
+    x[:4] = [1.0, 0, 0, 0]
+    p = o.quantize(o.Q8_0, x)
+    assert u16(p, 0) == f16_bits(np.float32(1.0) / np.float32(127.0))
+    assert p[2:3].view(np.int8)[0] == 127
+
+
+def test_q8_0_tail_block_is_zero_padded_and_truncated():
+    x = (np.arange(40, dtype=np.float32) - 20.0)
+    p = o.quantize(o.Q8_0, x)
+    assert p.size == 2 * 34
+    assert not p[34 + 2 + 8:].any()  # codes 8..31 of the tail block (quantize.rs:103)
+    y = o.dequantize(o.Q8_0, p, 40)
+    assert y.shape == (40,)  # dequantize.rs:44-50
+    assert np.abs(y - x).max() <= 20 / 127 / 2 + 20 * 2 ** -11
+
+
+# --------------------------------------------------------------------------- Q4_0 (quantize.rs:121-156, types.rs:179-206)
+def test_q4_0_zero_block():
+    p = o.quantize(o.Q4_0, np.zeros(32, np.float32))
+    assert (p[0], p[1]) == (0x00, 0x3C)
+    assert (p[2:] == 0x88).all()  # code 0 + bias 8 in both nibbles
+
+
+def test_q4_0_known_block_scale_one():
+    # max_abs = 7 -> scale 1.0; pairs (2i, 2i+1) -> (low, high) nibble, bias 8 (types.rs:190-198)
+    x = np.zeros(32, np.float32)
+    x[:8] = [7, -7, 6.5, -6.5, 0.5, -0.5, 2.5, -1.4]
+    p = o.quantize(o.Q4_0, x)
+    assert (p[0], p[1]) == (0x00, 0x3C)
+    # codes 7,-7,7,-7,1,-1,3,-1 -> nibbles 15,1,15,1,9,7,11,7
+    assert p[2:6].tolist() == [0x1F, 0x1F, 0x79, 0x7B]
+    assert (p[6:] == 0x88).all()
+
+
+def test_q4_0_reference_pack_unpack_ramp():
+    # types.rs:366-378: the ramp -8..7 twice, scale 1.0.  Bytes typed from Q4Block::pack by hand.
+    img = bytes([0x00, 0x3C] + [0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE] * 2)
+    y = o.dequantize(o.Q4_0, np.frombuffer(img, np.uint8), 32)
+    assert y.tolist() == [float(v) for v in list(range(-8, 8)) * 2]
+
+
+def test_q4_0_scale_is_max_abs_over_seven():
+    x = np.zeros(32, np.float32)
+    x[0], x[1] = -16.0, 16.0
+    p = o.quantize(o.Q4_0, x)
+    assert u16(p, 0) == f16_bits(np.float32(16.0) / np.float32(7.0)) == 0x4092
+    assert p[2] == 0xF1  # -7 -> 1, +7 -> 15
+
+
+# --------------------------------------------------------------------------- Q4_1 (quantize.rs:163-205, types.rs:238-255)
+def test_q4_1_known_block():
+    x = np.zeros(32, np.float32)
+    x[:8] = [0, 15, 0.5, 1.5, 2.5, 14.5, 7, 8]
+    p = o.quantize(o.Q4_1, x)
+    assert u16(p, 0) == 0x3C00 and u16(p, 2) == 0x0000  # scale 1.0, min 0.0
+    assert p[4:8].tolist() == [0xF0, 0x21, 0xF3, 0x87]
+    assert not p[8:].any()
+
+
+def test_q4_1_negative_min_and_constant_block():
+    x = np.full(32, -3.0, np.float32)
+    x[1] = 12.0  # range 15 -> scale 1.0, min -3.0
+    p = o.quantize(o.Q4_1, x)
+    assert u16(p, 0) == 0x3C00 and u16(p, 2) == 0xC200
+    assert p[4] == 0xF0 and not p[5:].any()
+    y = o.dequantize(o.Q4_1, p, 32)
+    assert y[0] == -3.0 and y[1] == 12.0
+    # max == min -> scale 1.0 (quantize.rs:179), min = the constant, all codes 0
+    p = o.quantize(o.Q4_1, np.full(32, 2.5, np.float32))
+    assert u16(p, 0) == 0x3C00 and u16(p, 2) == 0x4100
+    assert not p[4:].any()
+
+
+def test_q4_1_odd_tail_drops_last_code():
+    # quantize.rs:190-194: the pack loop covers min(16, len/2) bytes; len = 3 -> one byte.
+    x = np.zeros(35, np.float32)
+    x[32:] = [1.0, 2.0, 4.0]
+    p = o.quantize(o.Q4_1, x)
+    tail = p[20:]
+    assert u16(tail, 0) == f16_bits(np.float32(3.0) / np.float32(15.0))
+    assert u16(tail, 2) == 0x3C00  # min 1.0
+    assert tail[4] == 0x50 and not tail[5:].any()  # codes 0 and 5; the third element (code 15) is dropped
+    y = o.dequantize(o.Q4_1, p, 35)
+    assert y[34] == 1.0  # decodes as code 0 -> min
+
+
+def test_q4_1_dequant_is_multiply_then_add():
+    # scale = 0.1 (f16 0x2E66 = 0.0999755859375), min = 1/3 (f16 0x3555): q*scale + min in two f32 roundings.
+    img = np.zeros(20, np.uint8)
+    img[0:2] = [0x66, 0x2E]
+    img[2:4] = [0x55, 0x35]
+    img[4] = 0xF7
+    y = o.dequantize(o.Q4_1, img, 32)
+    s, m = np.float32(np.float16(0.1)), np.float32(np.float16(1 / 3))
+    assert y[0] == np.float32(np.float32(7) * s) + m and y[1] == np.float32(np.float32(15) * s) + m
+
+
+# --------------------------------------------------------------------------- the reference's own round-trip tests
+def test_reference_roundtrip_tolerances():
+    x = np.arange(64, dtype=np.float32) / np.float32(10.0)  # dequantize.rs:204-246
+    y8 = o.dequantize(o.Q8_0, o.quantize(o.Q8_0, x), 64)
+    assert np.abs(y8 - x).max() < 0.1
+    y4 = o.dequantize(o.Q4_0, o.quantize(o.Q4_0, x), 64)
+    assert np.abs(y4 - x).max() < 2.0
+    v = np.array([1.0, 2.5, -3.0, 4.25], np.float32)  # dequantize.rs:248-272
+    assert np.abs(o.dequantize(o.F16, o.quantize(o.F16, v), 4) - v).max() < 0.01
+    assert np.array_equal(o.dequantize(o.F32, o.quantize(o.F32, v), 4), v)
+
+
+def test_reference_q8_block_bytes_roundtrip():
+    # types.rs:380-389: scale 0.5, zero codes
+    img = np.zeros(34, np.uint8)
+    img[0:2] = [0x00, 0x38]
+    assert not o.dequantize(o.Q8_0, img, 32).any()
+    img[2] = 0xFE  # -2 * 0.5
+    assert o.dequantize(o.Q8_0, img, 32)[0] == -1.0
+
+
+def test_compression_ordering():
+    # quantize.rs:324-335
+    n = 256
+    assert n * 4 / o.packed_bytes(o.Q8_0, n) > 2.0
+    assert o.packed_bytes(o.Q4_0, n) < o.packed_bytes(o.Q8_0, n)
+
+
+# --------------------------------------------------------------------------- GGUF layouts, by hand-built blocks
+def test_q5_0_layout_hand_block():
+    img = np.zeros(22, np.uint8)
+    img[0:2] = [0x00, 0x3C]  # d = 1.0
+    img[2:6] = [0xFF, 0xFF, 0x00, 0x00]  # qh: elements 0..15 carry bit 4, 16..31 do not
+    img[6:] = [j | ((15 - j) << 4) for j in range(16)]
+    y = o.dequantize(o.Q5_0, img, 32)
+    assert y[:16].tolist() == [float(j) for j in range(16)]  # (j | 16) - 16
+    assert y[16:].tolist() == [float(15 - j - 16) for j in range(16)]
+
+
+def test_q5_1_layout_hand_block():
+    img = np.zeros(24, np.uint8)
+    img[0:2] = [0x00, 0x38]  # d = 0.5
+    img[2:4] = [0x00, 0xC0]  # m = -2.0
+    img[4:8] = [0x01, 0x00, 0x00, 0x80]  # qh bit 0 (element 0) and bit 31 (element 31)
+    img[8:] = [j | ((15 - j) << 4) for j in range(16)]
+    y = o.dequantize(o.Q5_1, img, 32)
+    want = [j * 0.5 - 2.0 for j in range(16)] + [(15 - j) * 0.5 - 2.0 for j in range(16)]
+    want[0] = 16 * 0.5 - 2.0
+    want[31] = (0 + 16) * 0.5 - 2.0
+    assert y.tolist() == want
+
+
+def test_q4_k_layout_hand_block():
+    # 6-bit scales ls and mins lm chosen so that sub-blocks 4..7 use the split high bits.
+    ls = [1, 2, 3, 4, 33, 34, 35, 36]
+    lm = [5, 6, 7, 8, 37, 38, 39, 40]
+    img = np.zeros(144, np.uint8)
+    img[0:2] = [0x00, 0x3C]  # d = 1.0
+    img[2:4] = [0x00, 0x38]  # dmin = 0.5
+    # bytes typed by hand from ggml's get_scale_min_k4 packing
+    img[4:16] = [129, 130, 131, 132, 133, 134, 135, 136, 0x51, 0x62, 0x73, 0x84]
+    for p in range(4):
+        for l in range(32):
+            img[16 + 32 * p + l] = (l & 15) | (((l + 1) & 15) << 4)
+    y = o.dequantize(o.Q4_K, img, 256)
+    for s in range(8):
+        for l in range(32):
+            q = (l & 15) if s % 2 == 0 else ((l + 1) & 15)
+            assert y[32 * s + l] == 1.0 * ls[s] * q - 0.5 * lm[s], (s, l)
+
+
+def _gguf_dequant_numpy(qtype, packed, numel):
+    """Independent numpy transcription of the GGUF block spec (not of the oracle)."""
+    out = []
+    if qtype == o.Q4_K:
+        for b in packed.reshape(-1, 144):
+            d, dmin = b[0:4].view(np.float16).astype(np.float32)
+            sc, qs = b[4:16].astype(np.int32), b[16:]
+            for j in range(8):
+                if j < 4:
+                    l, m = sc[j] & 63, sc[j + 4] & 63
+                else:
+                    l = (sc[j + 4] & 0xF) | ((sc[j - 4] >> 6) << 4)
+                    m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4)
+                q = qs[32 * (j // 2):32 * (j // 2) + 32]
+                q = (q >> 4) if j & 1 else (q & 0xF)
+                out.append(np.float32(d * np.float32(l)) * q.astype(np.float32) - np.float32(dmin * np.float32(m)))
+    else:
+        hdr = 2 if qtype == o.Q5_0 else 4
+        for b in packed.reshape(-1, hdr + 20):
+            d = b[0:2].view(np.float16).astype(np.float32)[0]
+            m = b[2:4].view(np.float16).astype(np.float32)[0] if qtype == o.Q5_1 else np.float32(0)
+            qh = int(b[hdr:hdr + 4].view(np.uint32)[0])
+            qs = b[hdr + 4:].astype(np.int32)
+            hb = np.array([(qh >> e) & 1 for e in range(32)], dtype=np.int32)
+            u = np.concatenate([(qs & 0xF) | (hb[:16] << 4), (qs >> 4) | (hb[16:] << 4)])
+            if qtype == o.Q5_0:
+                out.append((u - 16).astype(np.float32) * d)
+            else:
+                out.append(u.astype(np.float32) * d + m)
+    return np.concatenate(out)[:numel]
+
+
+@pytest.mark.parametrize("qtype", [o.Q5_0, o.Q5_1, o.Q4_K])
+def test_gguf_types_dequant_matches_spec_on_random_quantised_data(qtype):
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal(2048) * 0.02).astype(np.float32)
+    x[rng.random(2048) < 0.01] = 0.5
+    p = o.quantize(qtype, x)
+    assert np.array_equal(o.dequantize(qtype, p, 2048), _gguf_dequant_numpy(qtype, p, 2048))
+
+
+def test_q4_k_six_bit_fields_roundtrip_all_values():
+    # Drive every 6-bit scale value through every sub-block position: a superblock whose sub-block s
+    # spans [0, 15*t] has scale t, so ls_s = round(63 * t_s / max t).
+    for base in range(0, 64, 8):
+        t = np.arange(base, base + 8, dtype=np.float32)
+        t[t == 0] = 0.0
+        x = np.zeros(256, np.float32)
+        for s in range(8):
+            x[32 * s + 1] = 15.0 * t[s]
+        p = o.quantize(o.Q4_K, np.concatenate([x, np.full(256, 0, np.float32)]))[:144]
+        sc = p[4:16].astype(np.int32)
+        got = [(sc[j] & 63) if j < 4 else ((sc[j + 4] & 0xF) | ((sc[j - 4] >> 6) << 4)) for j in range(8)]
+        tmax = t.max()
+        want = [int(np.floor(63.0 * v / tmax + 0.5)) if tmax > 0 else 0 for v in t]
+        assert got == want, (base, got, want)
+
+
+# --------------------------------------------------------------------------- invariants, all types
+@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K])
+def test_roundtrip_error_bound(qtype):
+    rng = np.random.default_rng(11)
+    n = 4096
+    x = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    y = o.dequantize(qtype, o.quantize(qtype, x), n)
+    bs = {o.Q4_K: 32}.get(qtype, 32)
+    xb, yb = x.reshape(-1, bs), y.reshape(-1, bs)
+    levels = {o.Q8_0: 127 * 2, o.Q4_0: 14, o.Q4_1: 15, o.Q5_0: 30, o.Q5_1: 31, o.Q4_K: 15}[qtype]
+    span = xb.max(1) - np.minimum(xb.min(1), 0) if qtype == o.Q4_K else (
+        2 * np.abs(xb).max(1) if qtype in (o.Q8_0, o.Q4_0, o.Q5_0) else xb.max(1) - xb.min(1))
+    step = span / levels
+    slack = 1.6 if qtype == o.Q4_K else 0.51  # Q4_K re-quantises its scale and min to 6 bits
+    assert (np.abs(xb - yb).max(1) <= step * slack + np.abs(xb).max(1) * 2 ** -9).all()
+
+
+def test_q8_0_requantising_dequantised_values_is_idempotent():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(1024).astype(np.float32)
+    p1 = o.quantize(o.Q8_0, x)
+    p2 = o.quantize(o.Q8_0, o.dequantize(o.Q8_0, p1, 1024))
+    # codes survive; scales may move by the f16 rounding of 127*f16(scale)/127
+    assert np.array_equal(p1.reshape(-1, 34)[:, 2:], p2.reshape(-1, 34)[:, 2:])
+
+
+def test_empty_input():
+    for t in range(8):
+        assert o.quantize(t, np.zeros(0, np.float32)).size == 0
+        assert o.dequantize(t, np.zeros(0, np.uint8), 0).size == 0

@@ -1,0 +1,60 @@
+"""Pins the oracle's matmul (the reference composition dequantize -> transpose -> sgemm) on the CPU.
+
+Checks against things the mathematics fixes: the reference's own 2x2 sgemm known answer
+(crates/axonml-core/src/backends/cpu.rs:790-800), numpy float64 matmul of the dequantised weights,
+one-hot activations (select a weight column exactly), all-ones activations (row sums).
+"""
+import numpy as np
+import pytest
+
+import oracle as o
+from tests.util import max_rel_err
+
+ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.F16, o.F32]
+
+
+def test_reference_2x2_known_answer():
+    # cpu.rs:790-800: A = [[1,2],[3,4]], B = [[5,6],[7,8]] -> [19,22,43,50]; here W = B^T (y = x W^T).
+    w = np.array([[5, 7], [6, 8]], np.float32)
+    x = np.array([[1, 2], [3, 4]], np.float32)
+    y = o.matmul_ref(o.F32, w.view(np.uint8).reshape(-1), x, 2, 2)
+    assert y.reshape(-1).tolist() == [19.0, 22.0, 43.0, 50.0]
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("m", [1, 3])
+def test_matches_float64_matmul_of_dequantised_weights(qtype, m):
+    rng = np.random.default_rng(5 + qtype)
+    n, k = 24, 512
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    wq = o.quantize(qtype, w)
+    wd = o.dequantize(qtype, wq, n * k).reshape(n, k)
+    want = x.astype(np.float64) @ wd.astype(np.float64).T + bias
+    got = o.matmul_ref(qtype, wq, x, n, k, bias)
+    assert max_rel_err(got, want) < 1e-4  # f32 accumulation vs f64
+    assert np.abs(o.matmul_f64(wd, x, bias) - want).max() < 1e-12
+
+
+@pytest.mark.parametrize("qtype", ALL)
+def test_one_hot_selects_dequantised_column_exactly(qtype):
+    rng = np.random.default_rng(9)
+    n, k = 8, 256
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    wq = o.quantize(qtype, w)
+    wd = o.dequantize(qtype, wq, n * k).reshape(n, k)
+    for col in (0, 1, 31, 32, 100, 255):
+        x = np.zeros((1, k), np.float32)
+        x[0, col] = 1.0
+        assert np.array_equal(o.matmul_ref(qtype, wq, x, n, k)[0], wd[:, col])
+
+
+def test_all_ones_gives_row_sums():
+    rng = np.random.default_rng(2)
+    n, k = 16, 256
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    wq = o.quantize(o.Q4_K, w)
+    wd = o.dequantize(o.Q4_K, wq, n * k).reshape(n, k)
+    y = o.matmul_ref(o.Q4_K, wq, np.ones((1, k), np.float32), n, k)[0]
+    assert np.allclose(y, wd.astype(np.float64).sum(1), rtol=1e-5, atol=1e-6)

@@ -1,0 +1,33 @@
+"""Shared helpers for the parity tests."""
+import numpy as np
+
+# The path's matmul tolerance: max relative error 1e-3 against the reference f32 result, where the
+# relative error of an output is taken against max(|ref_i|, FLOOR * max_j |ref_j|) so that outputs
+# that happen to be near zero do not divide by nothing.
+MATMUL_RTOL = 1e-3
+REL_FLOOR = 1e-3
+
+
+def max_rel_err(got, want, floor=REL_FLOOR):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    denom = np.maximum(np.abs(want), floor * np.abs(want).max())
+    denom = np.where(denom == 0, 1.0, denom)
+    return float((np.abs(got - want) / denom).max())
+
+
+def assert_close_ref_style(got, want, atol=1e-5, rtol=1e-3):
+    """The reference GPU harness's check: |a - b| <= atol + rtol * |b| (backends/gpu_tests.rs:221-249)."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    bad = np.abs(got - want) > atol + rtol * np.abs(want)
+    assert not bad.any(), f"{int(bad.sum())} of {bad.size} outside atol={atol} rtol={rtol}"
+
+
+def gen_weight(rng, n, k, std=0.02, outlier_p=0.0, outlier_mag=0.5):
+    w = (rng.standard_normal((n, k)) * std).astype(np.float32)
+    if outlier_p > 0:
+        mask = rng.random((n, k)) < outlier_p
+        sign = np.where(rng.random((n, k)) < 0.5, -1.0, 1.0).astype(np.float32)
+        w = np.where(mask, sign * np.float32(outlier_mag), w).astype(np.float32)
+    return w
