@@ -83,12 +83,12 @@ struct Q4K {
     static constexpr int W = 64;
     struct X { float xs[64]; float sum_lo, sum_hi; };
     struct Raw { uint4 q0, q1, h; };
-    __device__ static void load_x(const GemvArgs &a, const float *x, int chunk, bool active, X &o) {
+    template <class F>
+    __device__ static void set_x(const GemvArgs &a, F fetch, X &o) {
         float lo = 0.f, hi = 0.f;
-        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 64);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            float4 v = fetch(i);
             float s = (v.x + v.y) + (v.z + v.w);
             if (i < 8) lo += s; else hi += s;
             o.xs[4 * i] = v.x * a.fp8_unit_inv; o.xs[4 * i + 1] = v.y * a.fp8_unit_inv;
@@ -144,12 +144,12 @@ struct Q4x { // Q4_0 / Q4_1: adjacent-pair nibble order (types.rs:179-198)
     static constexpr int W = 32;
     struct X { float xs[32]; float sum; };
     struct Raw { uint4 q; uint32_t m; };
-    __device__ static void load_x(const GemvArgs &a, const float *x, int chunk, bool active, X &o) {
+    template <class F>
+    __device__ static void set_x(const GemvArgs &a, F fetch, X &o) {
         float s = 0.f;
-        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 32);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            float4 v = fetch(i);
             s += (v.x + v.y) + (v.z + v.w);
             o.xs[4 * i] = v.x * a.fp8_unit_inv; o.xs[4 * i + 1] = v.y * a.fp8_unit_inv;
             o.xs[4 * i + 2] = v.z * a.fp8_unit_inv; o.xs[4 * i + 3] = v.w * a.fp8_unit_inv;
@@ -189,12 +189,12 @@ struct Q5x { // Q5_0 / Q5_1: byte j = elements j (low nibble) and j+16 (high); q
     static constexpr int W = 32;
     struct X { float xs[32]; float sum; };
     struct Raw { uint4 q; uint32_t qh; uint32_t m; };
-    __device__ static void load_x(const GemvArgs &, const float *x, int chunk, bool active, X &o) {
+    template <class F>
+    __device__ static void set_x(const GemvArgs &, F fetch, X &o) {
         float s = 0.f;
-        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 32);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            float4 v = fetch(i);
             s += (v.x + v.y) + (v.z + v.w);
             o.xs[4 * i] = v.x; o.xs[4 * i + 1] = v.y; o.xs[4 * i + 2] = v.z; o.xs[4 * i + 3] = v.w;
         }
@@ -234,11 +234,11 @@ struct Q80 { // chunk = 16 int8 = half a block
     static constexpr int W = 16;
     struct X { float xs[16]; };
     struct Raw { uint4 q; uint32_t m; };
-    __device__ static void load_x(const GemvArgs &, const float *x, int chunk, bool active, X &o) {
-        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 16);
+    template <class F>
+    __device__ static void set_x(const GemvArgs &, F fetch, X &o) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            float4 v = fetch(i);
             o.xs[4 * i] = v.x; o.xs[4 * i + 1] = v.y; o.xs[4 * i + 2] = v.z; o.xs[4 * i + 3] = v.w;
         }
     }
@@ -265,11 +265,11 @@ struct F16W { // chunk = 8 halfs
     static constexpr int W = 8;
     struct X { float xs[8]; };
     struct Raw { uint4 q; };
-    __device__ static void load_x(const GemvArgs &, const float *x, int chunk, bool active, X &o) {
-        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)chunk * 8);
+    template <class F>
+    __device__ static void set_x(const GemvArgs &, F fetch, X &o) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            float4 v = active ? p[i] : make_float4(0, 0, 0, 0);
+            float4 v = fetch(i);
             o.xs[4 * i] = v.x; o.xs[4 * i + 1] = v.y; o.xs[4 * i + 2] = v.z; o.xs[4 * i + 3] = v.w;
         }
     }
@@ -292,8 +292,9 @@ struct F32W { // chunk = 4 floats
     static constexpr int W = 4;
     struct X { float xs[4]; };
     struct Raw { float4 q; };
-    __device__ static void load_x(const GemvArgs &, const float *x, int chunk, bool active, X &o) {
-        float4 v = active ? *reinterpret_cast<const float4 *>(x + (size_t)chunk * 4) : make_float4(0, 0, 0, 0);
+    template <class F>
+    __device__ static void set_x(const GemvArgs &, F fetch, X &o) {
+        float4 v = fetch(0);
         o.xs[0] = v.x; o.xs[1] = v.y; o.xs[2] = v.z; o.xs[3] = v.w;
     }
     __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
@@ -304,8 +305,16 @@ struct F32W { // chunk = 4 floats
     }
 };
 
+// x straight from global memory (fallback kernel)
+template <class T>
+__device__ inline void load_x_global(const GemvArgs &a, int chunk, bool active, typename T::X &o) {
+    const float4 *p = reinterpret_cast<const float4 *>(a.x + (size_t)chunk * T::W);
+    T::set_x(a, [&](int i) { return active ? p[i] : make_float4(0, 0, 0, 0); }, o);
+}
+
 // ---------------------------------------------------------------------------
-// The kernel.  U rows in flight per lane.
+// Fallback kernel (any K): x is read from global memory per wave, U rows in
+// flight per lane, several passes over K when one lane cannot cover its share.
 // ---------------------------------------------------------------------------
 template <class T, int U>
 __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
@@ -320,7 +329,7 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
     int chunk = slice * 64 + lane;
     bool active = chunk < a.cpr;
     int cchunk = active ? chunk : a.cpr - 1; // inactive lanes re-read a valid chunk against x = 0
-    if (a.npass == 1) T::load_x(a, a.x, cchunk, active, xr);
+    if (a.npass == 1) load_x_global<T>(a, cchunk, active, xr);
 
     for (int r = row0; r < row_end; r += U) {
         float part[U];
@@ -331,7 +340,7 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
                 chunk = (pass * a.S + slice) * 64 + lane;
                 active = chunk < a.cpr;
                 cchunk = active ? chunk : a.cpr - 1;
-                T::load_x(a, a.x, cchunk, active, xr);
+                load_x_global<T>(a, cchunk, active, xr);
             }
             typename T::Raw raw[U];
 #pragma unroll
@@ -368,6 +377,125 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Staged kernel (K*4 bytes of x fit in LDS): the main path.
+//   - one workgroup per compute unit's share of the rows, up to 8 waves;
+//   - x is fetched once per workgroup (coalesced), parked in LDS in a
+//     [slice][vector][lane] order so that every lane then pulls its own
+//     K-range into registers without bank conflicts (a short last slice is
+//     packed with its own lane count as the stride);
+//   - the weight loads of the first 2*U rows of every wave are issued before
+//     the x staging, so the whole working set of the workgroup is in flight
+//     at once and HBM latency is paid once;
+//   - later row batches are double-buffered (load batch i+2 after consuming i).
+// ---------------------------------------------------------------------------
+constexpr int XT = 8; // x vectors staged per thread, at most
+
+template <class T, int U>
+__device__ inline void load_batch(const GemvArgs &a, int r, int row_end, int cchunk, typename T::Raw (&raw)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        int row = r + u;
+        row = row < row_end ? row : row_end - 1; // short batches re-read their last row (cache hit, result dropped)
+        T::load(a, row, cchunk, raw[u]);
+    }
+}
+
+template <class T, int U>
+__device__ inline void fold_batch(const GemvArgs &a, const typename T::Raw (&raw)[U], const typename T::X &xr, int cchunk,
+                                  int r, int row0, int row_end, int grp, int slice, int lane, float *red) {
+    float part[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) part[u] = T::dot(a, raw[u], xr, cchunk);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        float tot = wave_sum_lane63(part[u]);
+        int row = r + u;
+        if (lane == 63 && row < row_end) {
+            if (a.S == 1) a.y[row] = a.bias ? tot + a.bias[row] : tot;
+            else red[(grp * a.R + (row - row0)) * a.S + slice] = tot;
+        }
+    }
+}
+
+template <class T, int U>
+__global__ void __launch_bounds__(512) gemv_staged_kernel(GemvArgs a) {
+    extern __shared__ float4 lds4[];
+    constexpr int F4 = T::W / 4; // float4 per chunk
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int grp = wave / a.S, slice = wave - grp * a.S;
+    const int nf4 = a.cpr * F4;
+    float *red = reinterpret_cast<float *>(lds4 + nf4);
+
+    // 1. x: global -> registers, issued first so that it comes back first
+    float4 xt[XT];
+    const float4 *xg = reinterpret_cast<const float4 *>(a.x);
+#pragma unroll
+    for (int j = 0; j < XT; j++) {
+        int f = tid + (int)blockDim.x * j;
+        xt[j] = f < nf4 ? xg[f] : make_float4(0, 0, 0, 0);
+    }
+
+    // 2. weights of the first two row batches
+    const int chunk = slice * 64 + lane;
+    const bool active = chunk < a.cpr;
+    const int cchunk = active ? chunk : a.cpr - 1;
+    const int row0 = (blockIdx.x * a.G + grp) * a.R;
+    int row_end = row0 + a.R;
+    row_end = row_end < a.n_rows ? row_end : a.n_rows;
+    const bool has_rows = row0 < row_end;
+    typename T::Raw A[U], B[U];
+    if (has_rows) {
+        load_batch<T, U>(a, row0, row_end, cchunk, A);
+        if (row0 + U < row_end) load_batch<T, U>(a, row0 + U, row_end, cchunk, B);
+    }
+
+    // 3. x: registers -> LDS (swizzled) -> this lane's K-range
+#pragma unroll
+    for (int j = 0; j < XT; j++) {
+        int f = tid + (int)blockDim.x * j;
+        if (f < nf4) {
+            int c = f / F4, i = f - c * F4;
+            int sl = c >> 6;
+            int P = a.cpr - (sl << 6); // chunks in this slice (the last one may be short)
+            P = P < 64 ? P : 64;
+            lds4[sl * (64 * F4) + i * P + (c & 63)] = xt[j];
+        }
+    }
+    __syncthreads();
+    typename T::X xr;
+    {
+        const float4 *mine = lds4 + slice * (64 * F4) + lane;
+        int P = a.cpr - (slice << 6);
+        P = P < 64 ? P : 64;
+        T::set_x(a, [&](int i) { return active ? mine[i * P] : make_float4(0, 0, 0, 0); }, xr);
+    }
+
+    // 4. fold the batches
+    if (has_rows) {
+        for (int r = row0; r < row_end; r += 2 * U) {
+            fold_batch<T, U>(a, A, xr, cchunk, r, row0, row_end, grp, slice, lane, red);
+            if (r + 2 * U < row_end) load_batch<T, U>(a, r + 2 * U, row_end, cchunk, A);
+            if (r + U < row_end) {
+                fold_batch<T, U>(a, B, xr, cchunk, r + U, row0, row_end, grp, slice, lane, red);
+                if (r + 3 * U < row_end) load_batch<T, U>(a, r + 3 * U, row_end, cchunk, B);
+            }
+        }
+    }
+    if (a.S > 1) {
+        __syncthreads();
+        for (int t = tid; t < a.G * a.R; t += (int)blockDim.x) {
+            int g = t / a.R, rr = t - g * a.R;
+            int row = (blockIdx.x * a.G + g) * a.R + rr;
+            if (row < a.n_rows) {
+                float tot = 0.f;
+                for (int s = 0; s < a.S; s++) tot += red[(g * a.R + rr) * a.S + s];
+                a.y[row] = a.bias ? tot + a.bias[row] : tot;
+            }
+        }
+    }
+}
+
 template <class T>
 int launch(axq_ctx *ctx, const axq_weight *w, const float *x, const float *bias, float *y) {
     GemvArgs a;
@@ -377,14 +505,34 @@ int launch(axq_ctx *ctx, const axq_weight *w, const float *x, const float *bias,
     a.n_rows = (int)w->n_rows;
     a.cpr = (int)(w->k / T::W);
     a.fp8_unit_inv = ctx->fp8_unit_inv;
-    const int SMAX = 8;
+    int cus = ctx->prop.multiProcessorCount;
+    constexpr int U = 4;
     int s_need = (a.cpr + 63) / 64;
+    constexpr int F4 = T::W / 4;
+    if (s_need <= 8) {
+        // staged path: up to 8 waves per workgroup, one workgroup per CU
+        a.S = s_need;
+        a.G = 8 / a.S;
+        a.npass = 1;
+        if ((F4 + a.G - 1) / a.G <= XT) {
+            int groups = cus * a.G;
+            a.R = (a.n_rows + groups - 1) / groups;
+            if (a.R < 1) a.R = 1;
+            int rows_per_wg = a.G * a.R;
+            unsigned grid = (unsigned)((a.n_rows + rows_per_wg - 1) / rows_per_wg);
+            unsigned block = (unsigned)(64 * a.S * a.G);
+            size_t lds = (size_t)a.cpr * F4 * 16 + (size_t)a.G * a.R * a.S * sizeof(float);
+            if (lds <= 64 * 1024 && a.R <= 1024) {
+                gemv_staged_kernel<T, U><<<grid, block, lds, ctx->stream>>>(a);
+                AXQ_LAUNCH_CHECK(ctx, "gemv_staged_kernel");
+                return AXQ_OK;
+            }
+        }
+    }
+    const int SMAX = 8;
     a.S = s_need < SMAX ? s_need : SMAX;
     a.npass = (s_need + a.S - 1) / a.S;
     a.G = a.S >= 4 ? 1 : 4 / a.S;
-    constexpr int U = 4;
-    // rows per group: aim for about 8 workgroups per CU-pair while keeping x reuse
-    int cus = ctx->prop.multiProcessorCount;
     int target_wgs = cus * 2;
     int R = (a.n_rows + a.G * target_wgs - 1) / (a.G * target_wgs);
     R = (R + U - 1) / U * U;

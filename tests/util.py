@@ -1,11 +1,16 @@
 """Shared helpers for the parity tests."""
 import numpy as np
 
-# The path's matmul tolerance: max relative error 1e-3 against the reference f32 result, where the
-# relative error of an output is taken against max(|ref_i|, FLOOR * max_j |ref_j|) so that outputs
-# that happen to be near zero do not divide by nothing.
+# The path's matmul tolerance: max relative error 1e-3 against the reference f32 result.  The relative
+# error of output i is |y_i - ref_i| / max(|ref_i|, FLOOR * max_j |ref_j|), so that outputs that happen
+# to be near zero do not divide by nothing.  Two floors are used:
+#   REL_FLOOR = 1e-2 against the f32 oracle (the reference's own result).  A tighter floor would measure
+#     the reference's accumulation noise, not the kernel: the oracle's f32 sgemm already sits 9e-4 away
+#     from the exact product at a 1e-3 floor for K = 11008 (tests/test_oracle_matmul.py pins that).
+#   STRICT_FLOOR = 1e-3 against the float64 product of the same dequantised weights (the exact answer).
 MATMUL_RTOL = 1e-3
-REL_FLOOR = 1e-3
+REL_FLOOR = 1e-2
+STRICT_FLOOR = 1e-3
 
 
 def max_rel_err(got, want, floor=REL_FLOOR):
