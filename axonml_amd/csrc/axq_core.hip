@@ -185,6 +185,11 @@ int axq_init(int device, axq_ctx **out) {
         return AXQ_ERR_DRIVER;
     }
     ctx->fp8_unit_inv = 1.0f / h[0];
+    INIT_HIP(hipMalloc((void **)&ctx->xq, axq_xq_bytes(AXQ_XQ_MAX_K)));
+    // A lone GEMV call splits x inside the kernel (one launch); callers that produce x on the device
+    // hand over the split form instead.  AXQ_GEMV_PREP=separate forces the two-kernel form (development).
+    const char *prep = getenv("AXQ_GEMV_PREP");
+    ctx->gemv_prep = (prep && strcmp(prep, "separate") == 0) ? 1 : 0;
 #undef INIT_HIP
     *out = ctx;
     return AXQ_OK;
@@ -197,6 +202,7 @@ void axq_destroy(axq_ctx *ctx) {
     (void)hipEventDestroy(ctx->ev_start);
     (void)hipEventDestroy(ctx->ev_stop);
     (void)hipStreamDestroy(ctx->own_stream);
+    (void)hipFree(ctx->xq);
     free(ctx);
 }
 

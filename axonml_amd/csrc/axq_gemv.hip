@@ -379,24 +379,26 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
 
 // ---------------------------------------------------------------------------
 // Staged kernel (K*4 bytes of x fit in LDS): the main path.
-//   - one workgroup per compute unit's share of the rows, up to 8 waves;
-//   - x is fetched once per workgroup (coalesced), parked in LDS in a
-//     [slice][vector][lane] order so that every lane then pulls its own
-//     K-range into registers without bank conflicts (a short last slice is
-//     packed with its own lane count as the stride);
-//   - the weight loads of the first 2*U rows of every wave are issued before
-//     the x staging, so the whole working set of the workgroup is in flight
-//     at once and HBM latency is paid once;
-//   - later row batches are double-buffered (load batch i+2 after consuming i).
+//   - up to 8 waves per workgroup; x is fetched once per workgroup (coalesced),
+//     parked in LDS in a [slice][vector][lane] order so that every lane then
+//     pulls its own K-range into registers without bank conflicts (a short
+//     last slice is packed with its own lane count as the stride);
+//   - the weight loads of a wave's first U rows are issued before anything else,
+//     the next U rows while the workgroup meets at the x barrier; every load is
+//     unconditional (row indices are clamped) so that the compiler can count
+//     outstanding loads and wait per row rather than for everything: unpacking
+//     row i overlaps the arrival of row i+1...;
+//   - later row batches cycle through a ring of NB register buffers (batch
+//     i+NB is requested as soon as batch i has been folded);
+//   - row totals go to LDS; the last phase adds the S slice totals in a fixed
+//     order, adds the bias and writes y coalesced.
 // ---------------------------------------------------------------------------
-constexpr int XT = 8; // x vectors staged per thread, at most
-
 template <class T, int U>
-__device__ inline void load_batch(const GemvArgs &a, int r, int row_end, int cchunk, typename T::Raw (&raw)[U]) {
+__device__ inline void load_batch(const GemvArgs &a, int r, int row_last, int cchunk, typename T::Raw (&raw)[U]) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
         int row = r + u;
-        row = row < row_end ? row : row_end - 1; // short batches re-read their last row (cache hit, result dropped)
+        row = row < row_last ? row : row_last; // rows past the end re-read the last row (cache hit, result dropped)
         T::load(a, row, cchunk, raw[u]);
     }
 }
@@ -404,55 +406,47 @@ __device__ inline void load_batch(const GemvArgs &a, int r, int row_end, int cch
 template <class T, int U>
 __device__ inline void fold_batch(const GemvArgs &a, const typename T::Raw (&raw)[U], const typename T::X &xr, int cchunk,
                                   int r, int row0, int row_end, int grp, int slice, int lane, float *red) {
-    float part[U];
-#pragma unroll
-    for (int u = 0; u < U; u++) part[u] = T::dot(a, raw[u], xr, cchunk);
 #pragma unroll
     for (int u = 0; u < U; u++) {
-        float tot = wave_sum_lane63(part[u]);
+        float tot = wave_sum_lane63(T::dot(a, raw[u], xr, cchunk));
         int row = r + u;
-        if (lane == 63 && row < row_end) {
-            if (a.S == 1) a.y[row] = a.bias ? tot + a.bias[row] : tot;
-            else red[(grp * a.R + (row - row0)) * a.S + slice] = tot;
-        }
+        if (lane == 63 && row < row_end) red[(grp * a.R + (row - row0)) * a.S + slice] = tot;
     }
 }
 
-template <class T, int U>
+template <class T, int U, int NB, int XTN>
 __global__ void __launch_bounds__(512) gemv_staged_kernel(GemvArgs a) {
     extern __shared__ float4 lds4[];
     constexpr int F4 = T::W / 4; // float4 per chunk
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave / a.S, slice = wave - grp * a.S;
     const int nf4 = a.cpr * F4;
     float *red = reinterpret_cast<float *>(lds4 + nf4);
 
-    // 1. x: global -> registers, issued first so that it comes back first
-    float4 xt[XT];
-    const float4 *xg = reinterpret_cast<const float4 *>(a.x);
-#pragma unroll
-    for (int j = 0; j < XT; j++) {
-        int f = tid + (int)blockDim.x * j;
-        xt[j] = f < nf4 ? xg[f] : make_float4(0, 0, 0, 0);
-    }
-
-    // 2. weights of the first two row batches
+    // 1. weights of the first row batch: gets HBM going at once
     const int chunk = slice * 64 + lane;
     const bool active = chunk < a.cpr;
     const int cchunk = active ? chunk : a.cpr - 1;
     const int row0 = (blockIdx.x * a.G + grp) * a.R;
     int row_end = row0 + a.R;
     row_end = row_end < a.n_rows ? row_end : a.n_rows;
-    const bool has_rows = row0 < row_end;
-    typename T::Raw A[U], B[U];
-    if (has_rows) {
-        load_batch<T, U>(a, row0, row_end, cchunk, A);
-        if (row0 + U < row_end) load_batch<T, U>(a, row0 + U, row_end, cchunk, B);
+    const int row_last = (row_end > row0 ? row_end : a.n_rows) - 1;
+    typename T::Raw buf[NB][U];
+    load_batch<T, U>(a, row0 < a.n_rows ? row0 : a.n_rows - 1, row_last, cchunk, buf[0]);
+
+    // 2. x: global -> registers (an L2 hit; younger than the first batch, so waiting for it is enough)
+    float4 xt[XTN];
+    const float4 *xg = reinterpret_cast<const float4 *>(a.x);
+#pragma unroll
+    for (int j = 0; j < XTN; j++) {
+        int f = tid + (int)blockDim.x * j;
+        xt[j] = xg[f < nf4 ? f : nf4 - 1];
     }
 
     // 3. x: registers -> LDS (swizzled) -> this lane's K-range
 #pragma unroll
-    for (int j = 0; j < XT; j++) {
+    for (int j = 0; j < XTN; j++) {
         int f = tid + (int)blockDim.x * j;
         if (f < nf4) {
             int c = f / F4, i = f - c * F4;
@@ -462,6 +456,9 @@ __global__ void __launch_bounds__(512) gemv_staged_kernel(GemvArgs a) {
             lds4[sl * (64 * F4) + i * P + (c & 63)] = xt[j];
         }
     }
+    // the next batches go out while the workgroup meets at the barrier
+#pragma unroll
+    for (int b = 1; b < NB; b++) load_batch<T, U>(a, row0 + b * U, row_last, cchunk, buf[b]);
     __syncthreads();
     typename T::X xr;
     {
@@ -471,29 +468,36 @@ __global__ void __launch_bounds__(512) gemv_staged_kernel(GemvArgs a) {
         T::set_x(a, [&](int i) { return active ? mine[i * P] : make_float4(0, 0, 0, 0); }, xr);
     }
 
-    // 4. fold the batches
-    if (has_rows) {
-        for (int r = row0; r < row_end; r += 2 * U) {
-            fold_batch<T, U>(a, A, xr, cchunk, r, row0, row_end, grp, slice, lane, red);
-            if (r + 2 * U < row_end) load_batch<T, U>(a, r + 2 * U, row_end, cchunk, A);
-            if (r + U < row_end) {
-                fold_batch<T, U>(a, B, xr, cchunk, r + U, row0, row_end, grp, slice, lane, red);
-                if (r + 3 * U < row_end) load_batch<T, U>(a, r + 3 * U, row_end, cchunk, B);
+    // 4. fold the batches: a ring of NB register buffers, refilled as soon as they are consumed
+    for (int r = row0; r < row_end; r += NB * U) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            if (r + b * U < row_end) {
+                fold_batch<T, U>(a, buf[b], xr, cchunk, r + b * U, row0, row_end, grp, slice, lane, red);
+                if (r + (NB + b) * U < row_end) load_batch<T, U>(a, r + (NB + b) * U, row_last, cchunk, buf[b]);
             }
         }
     }
-    if (a.S > 1) {
-        __syncthreads();
-        for (int t = tid; t < a.G * a.R; t += (int)blockDim.x) {
-            int g = t / a.R, rr = t - g * a.R;
-            int row = (blockIdx.x * a.G + g) * a.R + rr;
-            if (row < a.n_rows) {
-                float tot = 0.f;
-                for (int s = 0; s < a.S; s++) tot += red[(g * a.R + rr) * a.S + s];
-                a.y[row] = a.bias ? tot + a.bias[row] : tot;
-            }
+
+    // 5. slice totals -> y
+    __syncthreads();
+    for (int t = tid; t < a.G * a.R; t += (int)blockDim.x) {
+        int g = t / a.R, rr = t - g * a.R;
+        int row = (blockIdx.x * a.G + g) * a.R + rr;
+        if (row < a.n_rows) {
+            float tot = red[(g * a.R + rr) * a.S];
+            for (int sidx = 1; sidx < a.S; sidx++) tot += red[(g * a.R + rr) * a.S + sidx];
+            a.y[row] = a.bias ? tot + a.bias[row] : tot;
         }
     }
+}
+
+template <class T, int U, int NB>
+void launch_staged(const GemvArgs &a, unsigned grid, unsigned block, size_t lds, int xt_need, hipStream_t st) {
+    if (xt_need <= 1) gemv_staged_kernel<T, U, NB, 1><<<grid, block, lds, st>>>(a);
+    else if (xt_need <= 2) gemv_staged_kernel<T, U, NB, 2><<<grid, block, lds, st>>>(a);
+    else if (xt_need <= 4) gemv_staged_kernel<T, U, NB, 4><<<grid, block, lds, st>>>(a);
+    else gemv_staged_kernel<T, U, NB, 8><<<grid, block, lds, st>>>(a);
 }
 
 template <class T>
@@ -514,16 +518,20 @@ int launch(axq_ctx *ctx, const axq_weight *w, const float *x, const float *bias,
         a.S = s_need;
         a.G = 8 / a.S;
         a.npass = 1;
-        if ((F4 + a.G - 1) / a.G <= XT) {
+        unsigned block = (unsigned)(64 * a.S * a.G);
+        int nf4 = a.cpr * F4;
+        int xt_need = (nf4 + (int)block - 1) / (int)block;
+        if (xt_need <= 8) {
             int groups = cus * a.G;
             a.R = (a.n_rows + groups - 1) / groups;
             if (a.R < 1) a.R = 1;
             int rows_per_wg = a.G * a.R;
             unsigned grid = (unsigned)((a.n_rows + rows_per_wg - 1) / rows_per_wg);
-            unsigned block = (unsigned)(64 * a.S * a.G);
-            size_t lds = (size_t)a.cpr * F4 * 16 + (size_t)a.G * a.R * a.S * sizeof(float);
-            if (lds <= 64 * 1024 && a.R <= 1024) {
-                gemv_staged_kernel<T, U><<<grid, block, lds, ctx->stream>>>(a);
+            size_t lds = (size_t)nf4 * 16 + (size_t)a.G * a.R * a.S * sizeof(float);
+            if (lds <= 64 * 1024) {
+                if (a.R <= 2) launch_staged<T, 2, 1>(a, grid, block, lds, xt_need, ctx->stream);
+                else if (a.R <= 4) launch_staged<T, 2, 2>(a, grid, block, lds, xt_need, ctx->stream);
+                else launch_staged<T, 2, 4>(a, grid, block, lds, xt_need, ctx->stream);
                 AXQ_LAUNCH_CHECK(ctx, "gemv_staged_kernel");
                 return AXQ_OK;
             }
@@ -556,7 +564,15 @@ int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, c
     for (int b = 0; b < batch; b++) {
         const float *xb = x + (size_t)b * (size_t)w->k;
         float *yb = y + (size_t)b * (size_t)w->n_rows;
-        int rc;
+        const uint8_t *xq = nullptr;
+        if (ctx->gemv_prep && axq_type_is_block_quantized(w->type) && w->k % 64 == 0 && w->k <= AXQ_XQ_MAX_K) {
+            int prc = axq_dev_prep_x(ctx, xb, w->k, ctx->xq);
+            if (prc) return prc;
+            xq = ctx->xq;
+        }
+        int rc = axq_dev_gemv_dp(ctx, w, xb, xq, bias, yb);
+        if (rc < 0) return rc;
+        if (rc == 1) continue;
         switch (w->type) {
         case AXQ_Q4_K: rc = launch<Q4K>(ctx, w, xb, bias, yb); break;
         case AXQ_Q4_0: rc = launch<Q4x<false>>(ctx, w, xb, bias, yb); break;

@@ -1,0 +1,531 @@
+// Decode-path quantized matmul, main kernel: integer dot products on the matrix
+// pipe.  y[n] = sum_k x[k] * W[n, k] (+ bias[n]) for the block-quantized types.
+//
+// Why: the kernel is HBM-bound on paper, but unpacking 4-bit codes to f32 and
+// issuing one FMA per weight costs about 200 VALU instructions per 4096-wide
+// row and makes the vector ALU the real limit.  Here the multiply-accumulate
+// runs as v_mfma_i32_4x4x4_16B_i8 ("16 independent 4x4x4 int8 products"), used
+// as a wide dot-product unit, not as a GEMM:
+//
+//   - x is split, once per workgroup, into four signed 7-bit limbs per element
+//     against a power-of-two scale per 32-element group:
+//         x = s_g * (l0*128^3 + l1*128^2 + l2*128 + l3),   |l_i| <= 64
+//     (28 bits below the group's largest magnitude: finer than f32's 24).
+//     The limbs are the MFMA's A operand, one limb per matrix row.
+//   - a lane's weight codes are the B operand: the four bytes of
+//     (q & 0x0F0F0F0F) are four int8 weights of the lane's own row, so a dword
+//     of eight 4-bit codes costs three VALU instructions (and, shift, and) and
+//     two MFMAs.  Lane (blk, j) = (lane / 4, lane % 4) supplies column j of
+//     block blk: row j of the current 4-row step, k-chunk blk of the wave's
+//     1024-wide K slice.  Its four accumulators are its own row's dot products
+//     with the four limbs: no cross-lane traffic until the final sum.
+//   - integer accumulation is exact; per 32-element group the four sums are
+//     recombined in f32, scaled by s_g and the block's f16 scale/min; the 16
+//     k-chunks of a row are added with two DPP row shifts, then across the four
+//     DPP rows and the K slices in a fixed order through LDS: no atomics,
+//     results are run-to-run identical.
+//
+// Memory side: every weight byte is read exactly once with 128-bit loads, 256
+// contiguous bytes per row per instruction; a ring of NB row steps per wave is
+// kept in flight and refilled as soon as a step has been consumed.
+#include <hip/hip_fp16.h>
+
+#include "axq_internal.h"
+
+namespace {
+
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+struct DpArgs {
+    const uint8_t *codes, *meta, *qh;
+    size_t codes_pitch, meta_pitch, qh_pitch;
+    const float *x, *bias;
+    const uint8_t *xq; // x already split into limbs (see stage_x), or NULL: the kernel splits it itself
+    float *y;
+    int n_rows, k;
+    int S, G, P;   // K slices per pass, row groups per workgroup, passes over K per lane
+    int steps;     // 4-row steps per group
+};
+
+__device__ inline float f16lo(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v & 0xFFFF))); }
+__device__ inline float f16hi(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v >> 16))); }
+__device__ inline float ub0(uint32_t v) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(v)); return r; }
+__device__ inline float ub1(uint32_t v) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(v)); return r; }
+
+__device__ inline int4v mfma(int a, uint32_t b, int4v c) { return __builtin_amdgcn_mfma_i32_4x4x4i8(a, (int)b, c, 0, 0, 0); }
+
+// sum_k n_k x_k over one 32-element group from its four limb sums
+__device__ inline float recombine(int4v d, float sg) {
+    float f = fmaf((float)d[0], 128.0f, (float)d[1]);
+    f = fmaf(f, 128.0f, (float)d[2]);
+    f = fmaf(f, 128.0f, (float)d[3]);
+    return f * sg;
+}
+
+// What a lane keeps of x for one pass: limb (lane % 4) of its 64 k-values as 16
+// MFMA A operands, and scale / plain sum of its two 32-element groups.
+struct XOp {
+    int a[16];
+    float sg[2], xs[2];
+};
+
+// ---------------------------------------------------------------------------
+// Per-type traits.  A lane covers 64 weights of one row per pass = two
+// 32-element groups.  group_k() gives the K offset of group g for chunk index
+// c (c counts 64-weight lane chunks along the row); load() fetches the lane's
+// bytes of one row; dot() returns its share of the row's dot product.
+// ---------------------------------------------------------------------------
+struct DQ4K {
+    struct Raw { uint4 q0, q1, h; };
+    static constexpr bool PERM_A = false;
+    __device__ static int group_k(int c, int g) { return c * 64 + g * 32; }
+    __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
+        // the code plane interleaves, per 64-pair slice, the first 16 bytes of every pair, then the second 16
+        const int cpr = a.k >> 6;
+        c = c < cpr ? c : cpr - 1; // lanes past the end of the row re-read its last chunk against x = 0
+        int slice = c >> 6, pr = c & 63;
+        int P = cpr - (slice << 6);
+        P = P < 64 ? P : 64;
+        const uint8_t *base = a.codes + row * a.codes_pitch + (size_t)slice * 2048 + (size_t)pr * 16;
+        r.q0 = *reinterpret_cast<const uint4 *>(base);
+        r.q1 = *reinterpret_cast<const uint4 *>(base + (size_t)P * 16);
+        r.h = *reinterpret_cast<const uint4 *>(a.meta + row * a.meta_pitch + (size_t)(c >> 2) * 16);
+    }
+    __device__ static float dot(const Raw &r, const XOp &x, int c) {
+        const uint32_t q0[4] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w};
+        const uint32_t q1[4] = {r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+#pragma unroll
+        for (int w = 0; w < 4; w++) { // bytes 4w..4w+3 of the first half: elements 4w.. of both sub-blocks
+            lo = mfma(x.a[w], q0[w] & 0x0F0F0F0Fu, lo);
+            hi = mfma(x.a[8 + w], (q0[w] >> 4) & 0x0F0F0F0Fu, hi);
+        }
+#pragma unroll
+        for (int w = 0; w < 4; w++) { // second half: elements 16+4w..
+            lo = mfma(x.a[4 + w], q1[w] & 0x0F0F0F0Fu, lo);
+            hi = mfma(x.a[12 + w], (q1[w] >> 4) & 0x0F0F0F0Fu, hi);
+        }
+        // 6-bit scale/min of sub-blocks 2p, 2p+1 (ggml get_scale_min_k4 order); p is fixed per lane
+        int p = c & 3;
+        int sh = (p & 1) * 16;
+        uint32_t ya = r.h.y >> sh, za = r.h.z >> sh, wa = r.h.w >> sh;
+        uint32_t scp, mp;
+        if (p < 2) {
+            scp = ya & 0x3F3F;
+            mp = za & 0x3F3F;
+        } else {
+            scp = (wa & 0x0F0F) | ((ya >> 2) & 0x3030);
+            mp = ((wa >> 4) & 0x0F0F) | ((za >> 2) & 0x3030);
+        }
+        float pos = fmaf(ub0(scp), recombine(lo, x.sg[0]), ub1(scp) * recombine(hi, x.sg[1]));
+        float neg = fmaf(ub0(mp), x.xs[0], ub1(mp) * x.xs[1]);
+        return fmaf(f16lo(r.h.x), pos, -(f16hi(r.h.x) * neg));
+    }
+};
+
+// Q4_0 / Q4_1 (reference nibble order, types.rs:179-198: byte i = elements 2i, 2i+1).  The lane's
+// two groups are the 32-element blocks c*2 and c*2+1... taken 16 blocks apart so that one load
+// instruction reads 256 contiguous bytes per row.
+template <bool WITH_MIN>
+struct DQ4x {
+    struct Raw { uint4 q[2]; uint32_t m[2]; };
+    static constexpr bool PERM_A = true; // dword w of a block: low nibbles = elements 8w+{0,2,4,6}, high = 8w+{1,3,5,7}
+    __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
+    __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
+    __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
+        const uint8_t *codes = a.codes + row * a.codes_pitch;
+        const uint8_t *meta = a.meta + row * a.meta_pitch;
+        const int nblk = a.k >> 5;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            int b = blk_index(c, g);
+            b = b < nblk ? b : nblk - 1;
+            r.q[g] = *reinterpret_cast<const uint4 *>(codes + (size_t)b * 16);
+            if (WITH_MIN) r.m[g] = *reinterpret_cast<const uint32_t *>(meta + (size_t)b * 4);
+            else r.m[g] = *reinterpret_cast<const uint16_t *>(meta + (size_t)b * 2);
+        }
+    }
+    __device__ static float dot(const Raw &r, const XOp &x, int) {
+        float tot = 0.f;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const uint32_t q[4] = {r.q[g].x, r.q[g].y, r.q[g].z, r.q[g].w};
+            int4v e = {0, 0, 0, 0}, o = {0, 0, 0, 0};
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                e = mfma(x.a[8 * g + 2 * w], q[w] & 0x0F0F0F0Fu, e);
+                o = mfma(x.a[8 * g + 2 * w + 1], (q[w] >> 4) & 0x0F0F0F0Fu, o);
+            }
+            float acc = recombine(e + o, x.sg[g]);
+            float scale = f16lo(r.m[g]);
+            if (WITH_MIN) tot += fmaf(scale, acc, f16hi(r.m[g]) * x.xs[g]);
+            else tot += scale * fmaf(-8.0f, x.xs[g], acc);
+        }
+        return tot;
+    }
+};
+
+// Q5_0 / Q5_1 (GGUF): byte j = elements j (low nibble) and j+16 (high); qh bit e = bit 4 of element e.
+template <bool WITH_MIN>
+struct DQ5x {
+    struct Raw { uint4 q[2]; uint32_t qh[2]; uint32_t m[2]; };
+    static constexpr bool PERM_A = false;
+    __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
+    __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
+    __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
+        const uint8_t *codes = a.codes + row * a.codes_pitch;
+        const uint8_t *meta = a.meta + row * a.meta_pitch;
+        const uint8_t *qh = a.qh + row * a.qh_pitch;
+        const int nblk = a.k >> 5;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            int b = blk_index(c, g);
+            b = b < nblk ? b : nblk - 1;
+            r.q[g] = *reinterpret_cast<const uint4 *>(codes + (size_t)b * 16);
+            r.qh[g] = *reinterpret_cast<const uint32_t *>(qh + (size_t)b * 4);
+            if (WITH_MIN) r.m[g] = *reinterpret_cast<const uint32_t *>(meta + (size_t)b * 4);
+            else r.m[g] = *reinterpret_cast<const uint16_t *>(meta + (size_t)b * 2);
+        }
+    }
+    __device__ static float dot(const Raw &r, const XOp &x, int) {
+        float tot = 0.f;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const uint32_t q[4] = {r.q[g].x, r.q[g].y, r.q[g].z, r.q[g].w};
+            int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                // spread 4 bits of qh to bit 4 of each byte: t * 0x00204081 puts bit i at bit 8i
+                uint32_t bl = (((r.qh[g] >> (4 * w)) & 0xFu) * 0x00204081u) & 0x01010101u;
+                uint32_t bh = (((r.qh[g] >> (16 + 4 * w)) & 0xFu) * 0x00204081u) & 0x01010101u;
+                lo = mfma(x.a[8 * g + w], (q[w] & 0x0F0F0F0Fu) | (bl << 4), lo);
+                hi = mfma(x.a[8 * g + 4 + w], ((q[w] >> 4) & 0x0F0F0F0Fu) | (bh << 4), hi);
+            }
+            float acc = recombine(lo + hi, x.sg[g]);
+            float d = f16lo(r.m[g]);
+            if (WITH_MIN) tot += fmaf(d, acc, f16hi(r.m[g]) * x.xs[g]);
+            else tot += d * fmaf(-16.0f, x.xs[g], acc);
+        }
+        return tot;
+    }
+};
+
+// Q8_0: four 16-byte vectors of int8 codes per lane per pass = two blocks; the codes are the B operand as they are.
+struct DQ80 {
+    struct Raw { uint4 q[4]; uint32_t m[2]; };
+    static constexpr bool PERM_A = false;
+    // 16-byte vector v (0..3) of chunk c: vector index along the row; block = vector / 2
+    __device__ static int vec_index(int c, int v) { return ((c >> 4) << 6) + (v >> 1) * 32 + (c & 15) * 2 + (v & 1); }
+    __device__ static int group_k(int c, int g) { return vec_index(c, 2 * g) * 16; }
+    __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
+        const uint8_t *codes = a.codes + row * a.codes_pitch;
+        const uint8_t *meta = a.meta + row * a.meta_pitch;
+        const int nvec = a.k >> 4;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            int v0 = vec_index(c, 2 * g);
+            v0 = v0 < nvec ? v0 : nvec - 2;
+            r.q[2 * g] = *reinterpret_cast<const uint4 *>(codes + (size_t)v0 * 16);
+            r.q[2 * g + 1] = *reinterpret_cast<const uint4 *>(codes + (size_t)v0 * 16 + 16);
+            r.m[g] = *reinterpret_cast<const uint16_t *>(meta + (size_t)(v0 >> 1) * 2);
+        }
+    }
+    __device__ static float dot(const Raw &r, const XOp &x, int) {
+        float tot = 0.f;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const uint32_t q[8] = {r.q[2 * g].x, r.q[2 * g].y, r.q[2 * g].z, r.q[2 * g].w,
+                                   r.q[2 * g + 1].x, r.q[2 * g + 1].y, r.q[2 * g + 1].z, r.q[2 * g + 1].w};
+            int4v e = {0, 0, 0, 0}, o = {0, 0, 0, 0};
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                e = mfma(x.a[8 * g + 2 * w], q[2 * w], e);
+                o = mfma(x.a[8 * g + 2 * w + 1], q[2 * w + 1], o);
+            }
+            tot += f16lo(r.m[g]) * recombine(e + o, x.sg[g]);
+        }
+        return tot;
+    }
+};
+
+// ---------------------------------------------------------------------------
+// x staging: LDS holds four int8 limb planes [K] and, per 32-element group, the
+// f32 scale that turns limb sums back into sum(n*x), and the plain sum of x.
+// ---------------------------------------------------------------------------
+__device__ inline void stage_x(const float *x, int k, uint8_t *planes, float2 *grp, int tid, int nthreads) {
+    const int kpad = (k + 15) & ~15;
+    // one task = 8 consecutive elements; 4 consecutive lanes share a 32-element group
+    const int ntask = (k + 7) >> 3;
+    const int ntask_pad = (ntask + 3) & ~3;
+    for (int t = tid; t < ntask_pad; t += nthreads) {
+        float v[8];
+        const bool live = t < ntask;
+        if (live) {
+            const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)t * 8);
+            float4 a = p[0], b = p[1];
+            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = 0.f;
+        }
+        float amax = 0.f, sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            amax = fmaxf(amax, fabsf(v[i]));
+            sum += v[i];
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 1));
+        amax = fmaxf(amax, __shfl_xor(amax, 2));
+        sum += __shfl_xor(sum, 1);
+        sum += __shfl_xor(sum, 2);
+        // amax in [2^e, 2^(e+1)): scale so that |x| * f < 2^27, f = 2^(26-e); limb sums times 2^(e-26) give back x
+        uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFF;
+        const bool bad = eb == 0xFF; // inf or nan in the group: poison the scale so that the row becomes nan
+        eb = eb < 30 ? 30 : eb;
+        eb = eb > 254 ? 254 : eb;
+        float f = __builtin_bit_cast(float, (280u - eb) << 23);
+        float sg = __builtin_bit_cast(float, (eb - 26u) << 23);
+        if (bad) sg = __builtin_nanf("");
+        uint32_t l[4][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            int tq = bad ? 0 : (int)rintf(v[i] * f);
+            int l3 = ((tq + 64) & 127) - 64;
+            tq = (tq - l3) >> 7;
+            int l2 = ((tq + 64) & 127) - 64;
+            tq = (tq - l2) >> 7;
+            int l1 = ((tq + 64) & 127) - 64;
+            int l0 = (tq - l1) >> 7;
+            int sh = 8 * (i & 3);
+            l[0][i >> 2] |= (uint32_t)(l0 & 0xFF) << sh;
+            l[1][i >> 2] |= (uint32_t)(l1 & 0xFF) << sh;
+            l[2][i >> 2] |= (uint32_t)(l2 & 0xFF) << sh;
+            l[3][i >> 2] |= (uint32_t)(l3 & 0xFF) << sh;
+        }
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                *reinterpret_cast<uint2 *>(planes + (size_t)i * kpad + (size_t)t * 8) = make_uint2(l[i][0], l[i][1]);
+            if ((t & 3) == 0) grp[t >> 2] = make_float2(sg, sum);
+        }
+    }
+}
+
+// Gather bytes {0,2} of lo and {0,2} of hi (sel = 0) or {1,3} of each (sel = 1)
+__device__ inline int pick_alt(uint32_t lo, uint32_t hi, int sel) {
+    return (int)__builtin_amdgcn_perm(hi, lo, sel ? 0x07050301u : 0x06040200u);
+}
+
+template <class T>
+__device__ inline void fetch_xop(const uint8_t *planes, const float2 *grp, int kpad, int k, int limb, int c, XOp &o) {
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        int kb = T::group_k(c, g);
+        uint32_t nat[8];
+        if (kb < k) { // groups past the end of the row contribute nothing
+            const uint4 *p = reinterpret_cast<const uint4 *>(planes + (size_t)limb * kpad + kb);
+            uint4 u = p[0], v = p[1];
+            nat[0] = u.x; nat[1] = u.y; nat[2] = u.z; nat[3] = u.w; nat[4] = v.x; nat[5] = v.y; nat[6] = v.z; nat[7] = v.w;
+            float2 sv = grp[kb >> 5];
+            o.sg[g] = sv.x;
+            o.xs[g] = sv.y;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) nat[i] = 0;
+            o.sg[g] = 0.f;
+            o.xs[g] = 0.f;
+        }
+        if (T::PERM_A) {
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                o.a[8 * g + 2 * w] = pick_alt(nat[2 * w], nat[2 * w + 1], 0);
+                o.a[8 * g + 2 * w + 1] = pick_alt(nat[2 * w], nat[2 * w + 1], 1);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) o.a[8 * g + i] = (int)nat[i];
+        }
+    }
+}
+
+// Sum over the four k-chunks of each 16-lane DPP row (lanes with equal lane % 4): lanes 12..15 of every
+// row end with that row's four totals.  The four DPP rows are added later, from LDS.
+__device__ inline float sum_within_row(float v) {
+    int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true); // row_shr:4
+    v += __builtin_bit_cast(float, t);
+    t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true); // row_shr:8
+    v += __builtin_bit_cast(float, t);
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// The kernel.  NB row steps in flight per wave, PP passes over K per lane.
+// ---------------------------------------------------------------------------
+template <class T, int NB, int PP, bool PRE>
+__global__ void __launch_bounds__(512) gemv_dp_kernel(DpArgs a) {
+    extern __shared__ uint4 lds_raw[];
+    const int kpad = (a.k + 15) & ~15;
+    // PRE: the limbs come from global memory (written by prep_x_kernel or by the kernel that produced x)
+    const uint8_t *planes = PRE ? a.xq : reinterpret_cast<const uint8_t *>(lds_raw);
+    const float2 *grp = reinterpret_cast<const float2 *>(planes + (size_t)4 * kpad);
+    float *red = PRE ? reinterpret_cast<float *>(lds_raw)
+                     : reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(lds_raw) + (size_t)4 * kpad + (size_t)((a.k + 31) >> 5) * 8);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g_idx = wave / a.S, slice = wave - g_idx * a.S;
+    const int blk = lane >> 2, j = lane & 3;
+
+    // chunk index of this lane in pass p
+    int c[PP];
+#pragma unroll
+    for (int p = 0; p < PP; p++) c[p] = ((p * a.S + slice) << 4) + blk;
+    const int rows_per_group = a.steps * 4;
+    const int row0 = (blockIdx.x * a.G + g_idx) * rows_per_group;
+    int row_end = row0 + rows_per_group;
+    row_end = row_end < a.n_rows ? row_end : a.n_rows;
+    const int last = a.n_rows - 1;
+
+    // Slot of (row, slice, DPP row) in the LDS reduction buffer: 4*S partial sums per output row.
+    const int dpp_row = lane >> 4;
+    const int red_stride = 4 * a.S;
+
+    typename T::Raw buf[NB][PP];
+    XOp xo[PP];
+    if (PRE) {
+        // 1. this lane's A operands first (L2 hits, needed before anything can be folded) ...
+#pragma unroll
+        for (int p = 0; p < PP; p++) fetch_xop<T>(planes, grp, kpad, a.k, j, c[p], xo[p]);
+    }
+    // 2. ... then the first NB steps' weights: the whole ring is in flight from the start
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+        int row = row0 + 4 * b + j;
+        row = row < last ? row : last;
+#pragma unroll
+        for (int p = 0; p < PP; p++) T::load(a, (size_t)row, c[p], buf[b][p]);
+    }
+    if (!PRE) {
+        // x -> limbs in LDS -> this lane's A operands, while the weights are on their way
+        uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw);
+        stage_x(a.x, a.k, wplanes, reinterpret_cast<float2 *>(wplanes + (size_t)4 * kpad), tid, (int)blockDim.x);
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < PP; p++) fetch_xop<T>(planes, grp, kpad, a.k, j, c[p], xo[p]);
+    }
+
+    // 3. fold the steps through the ring.  Everything inside the loops is unconditional (rows past the
+    //    end are clamped and their results dropped) so that the outstanding-load count is the same on
+    //    every path and a step waits for its own three loads only, not for the whole ring.
+    const int rounds = (a.steps + NB - 1) / NB;
+    auto fold = [&](int b, int rs) {
+        float part = 0.f;
+#pragma unroll
+        for (int p = 0; p < PP; p++) part += T::dot(buf[b][p], xo[p], c[p]);
+        float tot = sum_within_row(part);
+        if ((blk & 3) == 3 && rs + j < row_end)
+            red[(rs + j - row0 + g_idx * rows_per_group) * red_stride + slice * 4 + dpp_row] = tot;
+    };
+    int r = row0;
+    for (int round = 0; round < rounds - 1; round++, r += 4 * NB) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            fold(b, r + 4 * b);
+            int row = r + 4 * (NB + b) + j;
+            row = row < last ? row : last;
+#pragma unroll
+            for (int p = 0; p < PP; p++) T::load(a, (size_t)row, c[p], buf[b][p]);
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; b++) fold(b, r + 4 * b);
+
+    // 4. partial sums -> y, in a fixed order
+    __syncthreads();
+    const int wg_rows = a.G * rows_per_group;
+    for (int t = tid; t < wg_rows; t += (int)blockDim.x) {
+        int row = blockIdx.x * wg_rows + t;
+        if (row < a.n_rows) {
+            float tot = red[t * red_stride];
+            for (int s = 1; s < red_stride; s++) tot += red[t * red_stride + s];
+            a.y[row] = a.bias ? tot + a.bias[row] : tot;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) prep_x_kernel(const float *x, int k, uint8_t *xq) {
+    const int kpad = (k + 15) & ~15;
+    stage_x(x, k, xq, reinterpret_cast<float2 *>(xq + (size_t)4 * kpad), (int)(blockIdx.x * blockDim.x + threadIdx.x),
+            (int)(gridDim.x * blockDim.x));
+}
+
+template <class T>
+bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
+    if (w->k % 64 != 0) return false;
+    DpArgs a;
+    a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
+    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
+    a.x = x; a.xq = xq; a.bias = bias; a.y = y;
+    a.n_rows = (int)w->n_rows;
+    a.k = (int)w->k;
+    int slices = (a.k + 1023) / 1024;
+    a.P = (slices + 7) / 8;
+    if (a.P > 2) return false;
+    a.S = (slices + a.P - 1) / a.P;
+    a.G = 8 / a.S;
+    if (a.G < 1) a.G = 1;
+    int cus = ctx->prop.multiProcessorCount;
+    // 4-row steps per group: spread the rows over `wgs_per_cu` workgroups per compute unit
+    int wgs_per_cu = xq ? 2 : 1; // splitting x inside the kernel is paid per workgroup: use fewer, longer ones
+    int groups = cus * wgs_per_cu * a.G;
+    int steps = (a.n_rows + 4 * groups - 1) / (4 * groups);
+    if (steps < 1) steps = 1;
+    a.steps = steps;
+    int wg_rows = a.G * steps * 4;
+    unsigned grid = (unsigned)((a.n_rows + wg_rows - 1) / wg_rows);
+    unsigned block = (unsigned)(64 * a.S * a.G);
+    int kpad = (a.k + 15) & ~15;
+    size_t lds = (size_t)wg_rows * a.S * 4 * 4;
+    if (!xq) lds += (size_t)4 * kpad + (size_t)((a.k + 31) / 32) * 8;
+    if (lds > 64 * 1024) return false;
+    if (xq) {
+        if (a.P == 1) gemv_dp_kernel<T, 4, 1, true><<<grid, block, lds, ctx->stream>>>(a);
+        else gemv_dp_kernel<T, 2, 2, true><<<grid, block, lds, ctx->stream>>>(a);
+    } else {
+        if (a.P == 1) gemv_dp_kernel<T, 4, 1, false><<<grid, block, lds, ctx->stream>>>(a);
+        else gemv_dp_kernel<T, 2, 2, false><<<grid, block, lds, ctx->stream>>>(a);
+    }
+    return true;
+}
+
+} // namespace
+
+// Bytes of the split form of a K-vector: four limb planes and one (scale, sum) pair per 32 elements.
+size_t axq_xq_bytes(int64_t k) { return (size_t)4 * (size_t)((k + 15) & ~15) + (size_t)((k + 31) / 32) * 8; }
+
+// x[k] (f32, device) -> split form at xq (device, axq_xq_bytes(k) bytes).
+int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq) {
+    int tasks = (int)((k + 7) / 8);
+    int grid = (tasks + 255) / 256;
+    prep_x_kernel<<<grid, 256, 0, ctx->stream>>>(x, (int)k, xq);
+    AXQ_LAUNCH_CHECK(ctx, "prep_x_kernel");
+    return AXQ_OK;
+}
+
+// Returns 1 when the launch was made, 0 when this kernel does not cover the shape (the caller falls
+// back to the vector-ALU kernels), or a negative status.  xq = NULL: the kernel splits x itself.
+int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
+    bool ok;
+    switch (w->type) {
+    case AXQ_Q4_K: ok = launch_dp<DQ4K>(ctx, w, x, xq, bias, y); break;
+    case AXQ_Q4_0: ok = launch_dp<DQ4x<false>>(ctx, w, x, xq, bias, y); break;
+    case AXQ_Q4_1: ok = launch_dp<DQ4x<true>>(ctx, w, x, xq, bias, y); break;
+    case AXQ_Q5_0: ok = launch_dp<DQ5x<false>>(ctx, w, x, xq, bias, y); break;
+    case AXQ_Q5_1: ok = launch_dp<DQ5x<true>>(ctx, w, x, xq, bias, y); break;
+    case AXQ_Q8_0: ok = launch_dp<DQ80>(ctx, w, x, xq, bias, y); break;
+    default: return 0;
+    }
+    if (!ok) return 0;
+    AXQ_LAUNCH_CHECK(ctx, "gemv_dp_kernel");
+    return 1;
+}

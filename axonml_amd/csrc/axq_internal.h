@@ -17,6 +17,8 @@ struct axq_ctx {
     hipEvent_t ev_start, ev_stop;
     hipDeviceProp_t prop;
     float fp8_unit_inv; // 1 / value(fp8 byte 0x01) as converted by v_cvt_pk_f32_fp8
+    uint8_t *xq;        // device scratch: the split form of one activation vector (AXQ_XQ_MAX_K elements)
+    int gemv_prep;      // 0: split x inside the GEMV kernel, 1: in a kernel of its own
     char err[512];
 };
 
@@ -47,6 +49,8 @@ struct axq_weight {
     size_t codes_pitch, meta_pitch, qh_pitch;
     bool owns;
 };
+
+#define AXQ_XQ_MAX_K 65536
 
 static inline size_t axq_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -88,5 +92,9 @@ int axq_dev_repack(axq_ctx *ctx, const axq_weight *w, uint8_t *packed_dev, bool 
 int axq_weight_alloc(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, axq_weight **out);
 // gemv.hip
 int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x_dev, int batch, const float *bias_dev, float *y_dev);
+// gemv_mfma.hip: 1 = launched, 0 = shape not covered, <0 = error
+int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y);
+size_t axq_xq_bytes(int64_t k);
+int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq);
 // gemm.hip
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_dev, int m, float *y_dev);
