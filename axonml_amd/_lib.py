@@ -95,6 +95,7 @@ SIGNATURES = {
     "axq_model_generate": (_i, [_vp, _vp, _i, _i, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "axq_model_seq_len": (_i, [_vp]),
     "axq_fill_normal_f32": (_i, [_vp, _vp, _sz, C.c_float, C.c_float, C.c_float, C.c_float, C.c_uint64]),
+    "axq_bench_gemv_ring": (_i, [_vp, C.POINTER(_vp), _i, _vp, _i, _vp, _i]),
 }
 
 _lib = None

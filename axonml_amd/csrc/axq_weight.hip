@@ -276,4 +276,19 @@ int axq_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, f
     return AXQ_OK;
 }
 
+int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, const float *x_dev, int batch,
+                        float *y_dev, int iters) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_gemv_ring: NULL context");
+    if (!weights || n_weights <= 0 || !x_dev || !y_dev || batch <= 0)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_gemv_ring: bad argument");
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    for (int i = 0; i < iters; i++) {
+        const axq_weight *w = weights[i % n_weights];
+        if (!w) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_gemv_ring: NULL weight");
+        int rc = axq_dev_gemv(ctx, w, x_dev, batch, NULL, y_dev);
+        if (rc) return rc;
+    }
+    return AXQ_OK;
+}
+
 } // extern "C"

@@ -194,6 +194,11 @@ AXQ_API int axq_model_seq_len(const axq_model *m);
 AXQ_API int axq_fill_normal_f32(axq_ctx *ctx, float *dst_dev, size_t n, float mean, float std, float outlier_p,
                                 float outlier_mag, uint64_t seed);
 
+/* Enqueues `iters` GEMV launches back to back from C, launch i using weights[i % n_weights] (a ring
+ * of copies larger than the last-level cache keeps every launch streaming from HBM).  Device pointers. */
+AXQ_API int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, const float *x_dev,
+                                int batch, float *y_dev, int iters);
+
 #ifdef __cplusplus
 }
 #endif
