@@ -1,17 +1,727 @@
-// Decode model (placeholder; filled in after the GEMV path is verified).
+// Decode step of a LLaMA/Mistral-shape model with every linear block-quantized.
+//
+// Follows LLaMA::forward_with_cache (crates/axonml-llm/src/llama.rs:731-762) and
+// LLaMAForCausalLM::generate (llama.rs:900-977) for one sequence (batch 1):
+//   embedding lookup            crates/axonml-nn/src/layers/embedding.rs:103-146
+//   RMSNorm                     llama.rs:158-187
+//   q/k/v, o, gate/up/down      Linear::forward on quantized weights (the GEMV kernels)
+//   RoPE, half-split            llama.rs:223-252, 281-321 (tables built on the host as the reference does)
+//   KV cache append             crates/axonml-llm/src/attention.rs:46-70 (f16 here, grown in place)
+//   GQA causal attention        llama.rs:420-447 without the repeat_kv copy (llama.rs:450-480)
+//   SwiGLU                      llama.rs:562-567
+//   greedy argmax               llama.rs:1025-1030 (of equal maxima the last index wins)
+//
+// Device-side structure: q,k,v are one fused weight, gate and up another; every kernel that
+// produces a GEMV input also writes it in split (int8 limb) form, so the GEMV kernels never
+// re-split x; position and current token live in device memory so that the whole step is one
+// HIP graph replayed per token with no host round trip.
+#include <hip/hip_fp16.h>
+#include <math.h>
+#include <stdlib.h>
+
+#include <vector>
+
 #include "axq_internal.h"
+#include "axq_split.h"
+
+struct axq_model {
+    axq_ctx *ctx;
+    axq_model_config cfg;
+    int qkv_rows, q_dim, kv_dim;
+    // weights
+    uint16_t *emb;                  // f16 [vocab, hidden]
+    float *norm_attn, *norm_ffn;    // [layers, hidden]
+    float *norm_final;              // [hidden]
+    std::vector<axq_weight *> w_qkv, w_o, w_gu, w_down;
+    axq_weight *w_head;
+    std::vector<uint32_t> set_mask; // per layer: bit per axq_linear_id that has been set
+    bool head_set;
+    float *rope_cos, *rope_sin;     // [max_pos, head_dim / 2]
+    uint16_t *kcache, *vcache;      // f16 [layers, kv_heads, max_pos, head_dim]
+    // activations
+    float *h, *xn, *qkv, *att, *gu, *act, *logits;
+    uint8_t *xq_h, *xq_att, *xq_act;
+    // device-side state
+    int32_t *pos, *tok, *next, *gen, *prompt, *out;
+    int prompt_cap, out_cap;
+    int host_pos;
+    hipGraphExec_t graph;
+    bool graph_ok;
+};
+
+namespace {
+
+__device__ inline float block_sum(float v, float *scratch) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m);
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; i++) t += scratch[i];
+    return t;
+}
+
+__device__ inline float block_max(float v, float *scratch) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = -INFINITY;
+    for (int i = 0; i < nw; i++) t = fmaxf(t, scratch[i]);
+    return t;
+}
+
+// h = embedding[tok] (optional), then xn = rmsnorm(h) * w, written as f32 and in split form.
+// One workgroup; each thread owns 8-element tasks so that the split can be made from registers.
+__global__ void __launch_bounds__(1024) norm_kernel(const uint16_t *emb, const int32_t *tok, float *h, const float *w,
+                                                    int hidden, float eps, float *xn, uint8_t *xq) {
+    __shared__ float scratch[16];
+    const int ntask = hidden >> 3;
+    const int kpad = (hidden + 15) & ~15;
+    uint4 *grp = reinterpret_cast<uint4 *>(xq + (size_t)4 * kpad);
+    float ss = 0.f;
+    for (int t = threadIdx.x; t < ntask; t += blockDim.x) {
+        float v[8];
+        if (emb) {
+            const uint4 raw = *reinterpret_cast<const uint4 *>(emb + (size_t)tok[0] * hidden + (size_t)t * 8);
+            const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                v[2 * i] = __half2float(__ushort_as_half((unsigned short)(r[i] & 0xFFFF)));
+                v[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(r[i] >> 16)));
+            }
+            float4 *o = reinterpret_cast<float4 *>(h + (size_t)t * 8);
+            o[0] = make_float4(v[0], v[1], v[2], v[3]);
+            o[1] = make_float4(v[4], v[5], v[6], v[7]);
+        } else {
+            const float4 *p = reinterpret_cast<const float4 *>(h + (size_t)t * 8);
+            float4 a = p[0], b = p[1];
+            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) ss = fmaf(v[i], v[i], ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float rms = sqrtf(ss / (float)hidden + eps);
+    const int ntask_pad = (ntask + 3) & ~3;
+    for (int t = threadIdx.x; t < ntask_pad; t += blockDim.x) {
+        float v[8];
+        const bool live = t < ntask;
+        if (live) {
+            const float4 *p = reinterpret_cast<const float4 *>(h + (size_t)t * 8);
+            const float4 *pw = reinterpret_cast<const float4 *>(w + (size_t)t * 8);
+            float4 a = p[0], b = p[1], wa = pw[0], wb = pw[1];
+            v[0] = (a.x / rms) * wa.x; v[1] = (a.y / rms) * wa.y; v[2] = (a.z / rms) * wa.z; v[3] = (a.w / rms) * wa.w;
+            v[4] = (b.x / rms) * wb.x; v[5] = (b.y / rms) * wb.y; v[6] = (b.z / rms) * wb.z; v[7] = (b.w / rms) * wb.w;
+            float4 *o = reinterpret_cast<float4 *>(xn + (size_t)t * 8);
+            o[0] = make_float4(v[0], v[1], v[2], v[3]);
+            o[1] = make_float4(v[4], v[5], v[6], v[7]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = 0.f;
+        }
+        axq_split8(v, t, live, xq, grp, kpad);
+    }
+}
+
+// One workgroup per query head: RoPE on q (and on this head's new k), append k,v to the f16 cache
+// (by the first query head of each KV group), causal softmax(q.k / sqrt(d)) over positions 0..pos,
+// weighted sum of v; the head's output goes out as f32 and in split form.
+// Every position but the newest is read from the cache; the newest comes from registers, rounded
+// to f16 exactly as the cache holds it.
+__global__ void __launch_bounds__(256) attn_kernel(const float *qkv, const float *rope_cos, const float *rope_sin,
+                                                   uint16_t *kcache, uint16_t *vcache, const int32_t *pos_p, int n_heads,
+                                                   int n_kv, int d, int max_pos, float *att, uint8_t *xq_att) {
+    extern __shared__ float sm[];
+    float *q = sm;                // [d]
+    float *knew = q + d;          // [d]  (f16-rounded)
+    float *vnew = knew + d;       // [d]
+    float *scores = vnew + d;     // [max_pos]
+    float *outp = scores + max_pos; // [256 / d][d]
+    __shared__ float scratch[8];
+    const int head = blockIdx.x, kvh = head / (n_heads / n_kv);
+    const int pos = pos_p[0];
+    const int half = d >> 1;
+    const int q_dim = n_heads * d, kv_dim = n_kv * d;
+    const float *qh = qkv + (size_t)head * d;
+    const float *kh = qkv + q_dim + (size_t)kvh * d;
+    const float *vh = qkv + q_dim + kv_dim + (size_t)kvh * d;
+    uint16_t *kc = kcache + (size_t)kvh * max_pos * d;
+    uint16_t *vc = vcache + (size_t)kvh * max_pos * d;
+    const bool writer = head % (n_heads / n_kv) == 0;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
+        float x1 = qh[i], x2 = qh[i + half];
+        q[i] = x1 * c - x2 * s;
+        q[i + half] = x1 * s + x2 * c;
+        float k1 = kh[i], k2 = kh[i + half];
+        __half ka = __float2half_rn(k1 * c - k2 * s), kb = __float2half_rn(k1 * s + k2 * c);
+        __half va = __float2half_rn(vh[i]), vb = __float2half_rn(vh[i + half]);
+        knew[i] = __half2float(ka); knew[i + half] = __half2float(kb);
+        vnew[i] = __half2float(va); vnew[i + half] = __half2float(vb);
+        if (writer) {
+            kc[(size_t)pos * d + i] = __half_as_ushort(ka); kc[(size_t)pos * d + i + half] = __half_as_ushort(kb);
+            vc[(size_t)pos * d + i] = __half_as_ushort(va); vc[(size_t)pos * d + i + half] = __half_as_ushort(vb);
+        }
+    }
+    __syncthreads();
+    const float scale = 1.0f / sqrtf((float)d);
+    // scores: one thread per position
+    float lmax = -INFINITY;
+    for (int jpos = threadIdx.x; jpos <= pos; jpos += blockDim.x) {
+        float s = 0.f;
+        if (jpos == pos) {
+            for (int i = 0; i < d; i++) s = fmaf(q[i], knew[i], s);
+        } else {
+            const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)jpos * d);
+            for (int i8 = 0; i8 < d / 8; i8++) {
+                uint4 raw = kr[i8];
+                const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    s = fmaf(q[8 * i8 + 2 * e], __half2float(__ushort_as_half((unsigned short)(r[e] & 0xFFFF))), s);
+                    s = fmaf(q[8 * i8 + 2 * e + 1], __half2float(__ushort_as_half((unsigned short)(r[e] >> 16))), s);
+                }
+            }
+        }
+        s *= scale;
+        scores[jpos] = s;
+        lmax = fmaxf(lmax, s);
+    }
+    const float mx = block_max(lmax, scratch);
+    float lsum = 0.f;
+    for (int jpos = threadIdx.x; jpos <= pos; jpos += blockDim.x) {
+        float e = expf(scores[jpos] - mx);
+        scores[jpos] = e;
+        lsum += e;
+    }
+    const float denom = block_sum(lsum, scratch); // also orders the scores[] writes before the reads below
+    // weighted sum of v: thread (part, dim); two parts split the positions
+    const int dim = threadIdx.x % d, part = threadIdx.x / d, nparts = blockDim.x / d;
+    float acc = 0.f;
+    if (part < nparts) {
+        for (int jpos = part; jpos <= pos; jpos += nparts) {
+            float p = scores[jpos] / denom;
+            float vv = jpos == pos ? vnew[dim] : __half2float(__ushort_as_half(vc[(size_t)jpos * d + dim]));
+            acc = fmaf(p, vv, acc);
+        }
+        outp[part * d + dim] = acc;
+    }
+    __syncthreads();
+    // fold the parts, write f32 and the split form (d / 8 tasks, lane quads aligned)
+    const int ntask = d >> 3;
+    const int k_total = q_dim, kpad = (k_total + 15) & ~15;
+    uint4 *grp = reinterpret_cast<uint4 *>(xq_att + (size_t)4 * kpad);
+    if ((int)threadIdx.x < ((ntask + 3) & ~3)) {
+        const int t = threadIdx.x;
+        const bool live = t < ntask;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float a = 0.f;
+            if (live)
+                for (int p = 0; p < nparts; p++) a += outp[p * d + t * 8 + i];
+            v[i] = a;
+        }
+        if (live) {
+            float4 *o = reinterpret_cast<float4 *>(att + (size_t)head * d + (size_t)t * 8);
+            o[0] = make_float4(v[0], v[1], v[2], v[3]);
+            o[1] = make_float4(v[4], v[5], v[6], v[7]);
+        }
+        axq_split8(v, head * ntask + t, live, xq_att, grp, kpad);
+    }
+}
+
+// act = silu(gate) * up over [inter]; gu = [gate (inter) | up (inter)].
+__global__ void __launch_bounds__(256) swiglu_kernel(const float *gu, int inter, float *act, uint8_t *xq) {
+    const int ntask = inter >> 3;
+    const int kpad = (inter + 15) & ~15;
+    uint4 *grp = reinterpret_cast<uint4 *>(xq + (size_t)4 * kpad);
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool live = t < ntask;
+    float v[8];
+    if (live) {
+        const float4 *pg = reinterpret_cast<const float4 *>(gu + (size_t)t * 8);
+        const float4 *pu = reinterpret_cast<const float4 *>(gu + inter + (size_t)t * 8);
+        float4 ga = pg[0], gb = pg[1], ua = pu[0], ub = pu[1];
+        const float g[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+        const float u[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = (g[i] * (1.0f / (1.0f + expf(-g[i])))) * u[i];
+        float4 *o = reinterpret_cast<float4 *>(act + (size_t)t * 8);
+        o[0] = make_float4(v[0], v[1], v[2], v[3]);
+        o[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = 0.f;
+    }
+    axq_split8(v, t, live, xq, grp, kpad);
+}
+
+// argmax over the logits, last index among equal maxima (Iterator::max_by); then pos += 1.
+__global__ void __launch_bounds__(1024) argmax_kernel(const float *logits, int vocab, int32_t *next, int32_t *pos) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    float best = -INFINITY;
+    int idx = 0;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+        float v = logits[i];
+        if (v >= best) { best = v; idx = i; }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        float ov = __shfl_xor(best, m);
+        int oi = __shfl_xor(idx, m);
+        if (ov > best || (ov == best && oi > idx)) { best = ov; idx = oi; }
+    }
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { bv[wave] = best; bi[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++)
+            if (bv[w] > best || (bv[w] == best && bi[w] > idx)) { best = bv[w]; idx = bi[w]; }
+        next[0] = idx;
+        pos[0] = pos[0] + 1;
+    }
+}
+
+__global__ void pick_prompt_kernel(const int32_t *prompt, const int32_t *pos, int base, int32_t *tok) {
+    tok[0] = prompt[pos[0] - base];
+}
+__global__ void commit_next_kernel(const int32_t *next, int32_t *tok, int32_t *gen, int32_t *out, int out_cap) {
+    int g = gen[0];
+    tok[0] = next[0];
+    if (g < out_cap) out[g] = next[0];
+    gen[0] = g + 1;
+}
+__global__ void set_i32_kernel(int32_t *p, int32_t v) { p[0] = v; }
+__global__ void fill_f32_kernel(float *p, size_t n, float v) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+__global__ void f32_to_f16_kernel(const float *src, size_t n, uint16_t *dst) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = __half_as_ushort(__float2half_rn(src[i]));
+}
+
+int lin_dims(const axq_model *m, int layer, int which, int64_t *rows, int64_t *k) {
+    const axq_model_config &c = m->cfg;
+    if (layer < 0) { *rows = c.vocab_size; *k = c.hidden_size; return 0; }
+    switch (which) {
+    case AXQ_LIN_Q: *rows = m->q_dim; *k = c.hidden_size; break;
+    case AXQ_LIN_K: case AXQ_LIN_V: *rows = m->kv_dim; *k = c.hidden_size; break;
+    case AXQ_LIN_O: *rows = c.hidden_size; *k = m->q_dim; break;
+    case AXQ_LIN_GATE: case AXQ_LIN_UP: *rows = c.intermediate_size; *k = c.hidden_size; break;
+    case AXQ_LIN_DOWN: *rows = c.hidden_size; *k = c.intermediate_size; break;
+    default: return -1;
+    }
+    return 0;
+}
+
+// Copies all rows of src into dst starting at dst row `row_off` (same type and k): plane by plane.
+int copy_rows(axq_ctx *ctx, axq_weight *dst, const axq_weight *src, int64_t row_off) {
+    struct { uint8_t *d; const uint8_t *s; size_t pitch; } planes[3] = {
+        {dst->codes, src->codes, src->codes_pitch}, {dst->meta, src->meta, src->meta_pitch}, {dst->qh, src->qh, src->qh_pitch}};
+    for (auto &p : planes) {
+        if (p.pitch == 0) continue;
+        AXQ_HIP(ctx, hipMemcpyAsync(p.d + (size_t)row_off * p.pitch, p.s, p.pitch * (size_t)src->n_rows,
+                                    hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    }
+    return AXQ_OK;
+}
+
+// y = W x (+ bias): split-form GEMV when the shape is covered, else the f32 path.
+int gemv(axq_model *m, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
+    int rc = axq_dev_gemv_dp(m->ctx, w, x, xq, bias, y);
+    if (rc < 0) return rc;
+    if (rc == 1) return AXQ_OK;
+    return axq_dev_gemv(m->ctx, w, x, 1, bias, y);
+}
+
+// The kernels of one token, enqueued on the context's stream.
+int enqueue_step(axq_model *m) {
+    axq_ctx *ctx = m->ctx;
+    const axq_model_config &c = m->cfg;
+    hipStream_t st = ctx->stream;
+    const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim;
+    const size_t kv_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * d;
+    const size_t attn_lds = (size_t)(3 * d + c.max_position_embeddings + 256) * sizeof(float);
+    int rc;
+    for (int l = 0; l < c.num_hidden_layers; l++) {
+        norm_kernel<<<1, 1024, 0, st>>>(l == 0 ? m->emb : nullptr, m->tok, m->h, m->norm_attn + (size_t)l * H, H,
+                                        c.rms_norm_eps, m->xn, m->xq_h);
+        if ((rc = gemv(m, m->w_qkv[l], m->xn, m->xq_h, nullptr, m->qkv))) return rc;
+        attn_kernel<<<c.num_attention_heads, 256, attn_lds, st>>>(m->qkv, m->rope_cos, m->rope_sin,
+                                                                  m->kcache + (size_t)l * kv_layer,
+                                                                  m->vcache + (size_t)l * kv_layer, m->pos,
+                                                                  c.num_attention_heads, c.num_key_value_heads, d,
+                                                                  c.max_position_embeddings, m->att, m->xq_att);
+        if ((rc = gemv(m, m->w_o[l], m->att, m->xq_att, m->h, m->h))) return rc; // residual through the bias slot
+        norm_kernel<<<1, 1024, 0, st>>>(nullptr, m->tok, m->h, m->norm_ffn + (size_t)l * H, H, c.rms_norm_eps, m->xn,
+                                        m->xq_h);
+        if ((rc = gemv(m, m->w_gu[l], m->xn, m->xq_h, nullptr, m->gu))) return rc;
+        swiglu_kernel<<<(I / 8 + 255) / 256, 256, 0, st>>>(m->gu, I, m->act, m->xq_act);
+        if ((rc = gemv(m, m->w_down[l], m->act, m->xq_act, m->h, m->h))) return rc;
+    }
+    norm_kernel<<<1, 1024, 0, st>>>(c.num_hidden_layers == 0 ? m->emb : nullptr, m->tok, m->h, m->norm_final, H,
+                                    c.rms_norm_eps, m->xn, m->xq_h);
+    if ((rc = gemv(m, m->w_head, m->xn, m->xq_h, nullptr, m->logits))) return rc;
+    argmax_kernel<<<1, 1024, 0, st>>>(m->logits, c.vocab_size, m->next, m->pos);
+    AXQ_LAUNCH_CHECK(ctx, "decode step");
+    return AXQ_OK;
+}
+
+int check_ready(axq_model *m) {
+    if (!m->emb || !m->head_set) return axq_fail(m->ctx, AXQ_ERR_INVALID_DATA, "Invalid quantized data: embedding or lm_head not set");
+    for (int l = 0; l < m->cfg.num_hidden_layers; l++)
+        if (m->set_mask[l] != (1u << AXQ_LIN_COUNT) - 1)
+            return axq_fail(m->ctx, AXQ_ERR_INVALID_DATA, "Invalid quantized data: layer %d has unset linears (mask %#x)", l,
+                            m->set_mask[l]);
+    return AXQ_OK;
+}
+
+// Captures the step into a graph on first use; later calls replay it.
+int run_step(axq_model *m) {
+    axq_ctx *ctx = m->ctx;
+    static const bool no_graph = getenv("AXQ_DECODE_GRAPH") && getenv("AXQ_DECODE_GRAPH")[0] == '0';
+    if (no_graph) return enqueue_step(m); // development knob: plain launches instead of a graph replay
+    if (!m->graph_ok) {
+        hipGraph_t g = nullptr;
+        AXQ_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), AXQ_ERR_DRIVER);
+        int rc = enqueue_step(m);
+        hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+        if (rc) {
+            if (g) (void)hipGraphDestroy(g);
+            return rc;
+        }
+        if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipStreamEndCapture: %s", hipGetErrorString(e));
+        e = hipGraphInstantiate(&m->graph, g, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(g);
+        if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipGraphInstantiate: %s", hipGetErrorString(e));
+        m->graph_ok = true;
+    }
+    AXQ_HIP(ctx, hipGraphLaunch(m->graph, ctx->stream), AXQ_ERR_KERNEL_LAUNCH_FAILED);
+    return AXQ_OK;
+}
+
+template <class T>
+hipError_t dev_alloc(T **p, size_t count) { return hipMalloc((void **)p, (count ? count : 1) * sizeof(T)); }
+
+} // namespace
 
 extern "C" {
-int axq_model_create(axq_ctx *ctx, const axq_model_config *, axq_model **) {
-    return axq_fail(ctx, AXQ_ERR_KERNEL_LAUNCH_FAILED, "axq_model_create: not built yet");
+
+int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_create: NULL context");
+    if (!cfg || !out) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_create: NULL pointer");
+    *out = NULL;
+    const axq_model_config &c = *cfg;
+    if (c.vocab_size <= 0 || c.hidden_size <= 0 || c.intermediate_size <= 0 || c.num_hidden_layers < 0 ||
+        c.num_attention_heads <= 0 || c.num_key_value_heads <= 0 || c.head_dim <= 0 || c.max_position_embeddings <= 0)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: model dimensions must be positive");
+    if (c.num_attention_heads % c.num_key_value_heads != 0)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: %d query heads are not a multiple of %d kv heads",
+                        c.num_attention_heads, c.num_key_value_heads);
+    if (c.hidden_size % 32 || c.intermediate_size % 32 ||
+        (c.head_dim != 32 && c.head_dim != 64 && c.head_dim != 128 && c.head_dim != 256))
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH,
+                        "Shape mismatch: hidden and intermediate sizes must be multiples of 32 and head_dim one of 32, 64, "
+                        "128, 256");
+    if ((size_t)(3 * c.head_dim + 256 + c.max_position_embeddings) * 4 > 60 * 1024)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: max_position_embeddings %d does not fit the attention kernel",
+                        c.max_position_embeddings);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    axq_model *m = new (std::nothrow) axq_model();
+    if (!m) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "out of host memory");
+    m->ctx = ctx;
+    m->cfg = c;
+    m->q_dim = c.num_attention_heads * c.head_dim;
+    m->kv_dim = c.num_key_value_heads * c.head_dim;
+    m->qkv_rows = m->q_dim + 2 * m->kv_dim;
+    const int L = c.num_hidden_layers, H = c.hidden_size, I = c.intermediate_size;
+    m->w_qkv.assign(L, nullptr); m->w_o.assign(L, nullptr); m->w_gu.assign(L, nullptr); m->w_down.assign(L, nullptr);
+    m->set_mask.assign(L, 0);
+    m->prompt_cap = c.max_position_embeddings;
+    m->out_cap = c.max_position_embeddings;
+    const size_t kv = (size_t)L * c.num_key_value_heads * c.max_position_embeddings * c.head_dim;
+    hipError_t e = hipSuccess;
+#define TRY(x) if (e == hipSuccess) e = (x)
+    TRY(dev_alloc(&m->norm_attn, (size_t)L * H)); TRY(dev_alloc(&m->norm_ffn, (size_t)L * H)); TRY(dev_alloc(&m->norm_final, H));
+    TRY(dev_alloc(&m->rope_cos, (size_t)c.max_position_embeddings * c.head_dim / 2));
+    TRY(dev_alloc(&m->rope_sin, (size_t)c.max_position_embeddings * c.head_dim / 2));
+    TRY(dev_alloc(&m->kcache, kv)); TRY(dev_alloc(&m->vcache, kv));
+    TRY(dev_alloc(&m->h, H)); TRY(dev_alloc(&m->xn, H)); TRY(dev_alloc(&m->qkv, m->qkv_rows)); TRY(dev_alloc(&m->att, m->q_dim));
+    TRY(dev_alloc(&m->gu, (size_t)2 * I)); TRY(dev_alloc(&m->act, I)); TRY(dev_alloc(&m->logits, c.vocab_size));
+    TRY(dev_alloc(&m->xq_h, axq_split_bytes(H))); TRY(dev_alloc(&m->xq_att, axq_split_bytes(m->q_dim)));
+    TRY(dev_alloc(&m->xq_act, axq_split_bytes(I)));
+    TRY(dev_alloc(&m->pos, 1)); TRY(dev_alloc(&m->tok, 1)); TRY(dev_alloc(&m->next, 1)); TRY(dev_alloc(&m->gen, 1));
+    TRY(dev_alloc(&m->prompt, m->prompt_cap)); TRY(dev_alloc(&m->out, m->out_cap));
+#undef TRY
+    if (e != hipSuccess) {
+        int rc = axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "model buffers: %s", hipGetErrorString(e));
+        axq_model_free(m);
+        return rc;
+    }
+    // unit norms by default (RMSNorm::new, llama.rs:150-156); zeroed cache and state
+    size_t nn = (size_t)L * H;
+    if (nn) fill_f32_kernel<<<(unsigned)((nn + 255) / 256), 256, 0, ctx->stream>>>(m->norm_attn, nn, 1.0f);
+    if (nn) fill_f32_kernel<<<(unsigned)((nn + 255) / 256), 256, 0, ctx->stream>>>(m->norm_ffn, nn, 1.0f);
+    fill_f32_kernel<<<(H + 255) / 256, 256, 0, ctx->stream>>>(m->norm_final, H, 1.0f);
+    (void)hipMemsetAsync(m->kcache, 0, kv * 2, ctx->stream);
+    (void)hipMemsetAsync(m->vcache, 0, kv * 2, ctx->stream);
+    (void)hipMemsetAsync(m->pos, 0, 4, ctx->stream);
+    (void)hipMemsetAsync(m->gen, 0, 4, ctx->stream);
+    (void)hipMemsetAsync(m->tok, 0, 4, ctx->stream);
+    // RotaryEmbedding::new (llama.rs:223-252): inv_freq_i = 1 / theta^(2i/d), tables of cos/sin(pos * inv_freq_i)
+    {
+        const int half = c.head_dim / 2;
+        std::vector<float> hc((size_t)c.max_position_embeddings * half), hs(hc.size());
+        for (int i = 0; i < half; i++) {
+            float inv_freq = 1.0f / powf(c.rope_theta, 2.0f * (float)i / (float)c.head_dim);
+            for (int p = 0; p < c.max_position_embeddings; p++) {
+                float angle = (float)p * inv_freq;
+                hc[(size_t)p * half + i] = cosf(angle);
+                hs[(size_t)p * half + i] = sinf(angle);
+            }
+        }
+        e = hipMemcpyAsync(m->rope_cos, hc.data(), hc.size() * 4, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(m->rope_sin, hs.data(), hs.size() * 4, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) {
+            int rc = axq_fail(ctx, AXQ_ERR_COPY_FAILED, "rope tables: %s", hipGetErrorString(e));
+            axq_model_free(m);
+            return rc;
+        }
+    }
+    *out = m;
+    return AXQ_OK;
 }
-void axq_model_free(axq_model *) {}
-int axq_model_set_embedding_f16(axq_model *, const uint16_t *, int) { return AXQ_ERR_INVALID_ARGUMENT; }
-int axq_model_set_norm(axq_model *, int, int, const float *, int) { return AXQ_ERR_INVALID_ARGUMENT; }
-int axq_model_set_linear(axq_model *, int, int, const axq_weight *) { return AXQ_ERR_INVALID_ARGUMENT; }
-int axq_model_random_init(axq_model *, int, float, uint64_t) { return AXQ_ERR_INVALID_ARGUMENT; }
-int axq_model_reset(axq_model *) { return AXQ_ERR_INVALID_ARGUMENT; }
-int axq_model_forward(axq_model *, int32_t, float *, int32_t *) { return AXQ_ERR_INVALID_ARGUMENT; }
-int axq_model_generate(axq_model *, const int32_t *, int, int, int32_t *, float *, float *) { return AXQ_ERR_INVALID_ARGUMENT; }
-int axq_model_seq_len(const axq_model *) { return -1; }
+
+void axq_model_free(axq_model *m) {
+    if (!m) return;
+    axq_ctx *ctx = m->ctx;
+    (void)hipStreamSynchronize(ctx->stream);
+    if (m->graph_ok) (void)hipGraphExecDestroy(m->graph);
+    for (auto *w : m->w_qkv) axq_weight_free(ctx, w);
+    for (auto *w : m->w_o) axq_weight_free(ctx, w);
+    for (auto *w : m->w_gu) axq_weight_free(ctx, w);
+    for (auto *w : m->w_down) axq_weight_free(ctx, w);
+    axq_weight_free(ctx, m->w_head);
+    void *bufs[] = {m->emb, m->norm_attn, m->norm_ffn, m->norm_final, m->rope_cos, m->rope_sin, m->kcache, m->vcache, m->h,
+                    m->xn, m->qkv, m->att, m->gu, m->act, m->logits, m->xq_h, m->xq_att, m->xq_act, m->pos, m->tok,
+                    m->next, m->gen, m->prompt, m->out};
+    for (void *p : bufs)
+        if (p) (void)hipFree(p);
+    delete m;
 }
+
+int axq_model_set_embedding_f16(axq_model *m, const uint16_t *table, int mem) {
+    if (!m || !table) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    size_t n = (size_t)m->cfg.vocab_size * m->cfg.hidden_size;
+    if (!m->emb) AXQ_HIP(ctx, dev_alloc(&m->emb, n), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, hipMemcpyAsync(m->emb, table, n * 2, mem == AXQ_MEM_DEVICE ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
+                                ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_model_set_norm(axq_model *m, int layer, int which, const float *w, int mem) {
+    if (!m || !w) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    const int H = m->cfg.hidden_size;
+    if (layer >= m->cfg.num_hidden_layers || (layer >= 0 && (which < 0 || which > 1)))
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_set_norm: layer %d / which %d out of range", layer, which);
+    float *dst = layer < 0 ? m->norm_final : (which == 0 ? m->norm_attn : m->norm_ffn) + (size_t)layer * H;
+    AXQ_HIP(ctx, hipMemcpyAsync(dst, w, (size_t)H * 4, mem == AXQ_MEM_DEVICE ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
+                                ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_model_set_linear(axq_model *m, int layer, int which, const axq_weight *w) {
+    if (!m || !w) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    if (layer >= m->cfg.num_hidden_layers)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_set_linear: layer %d out of range", layer);
+    int64_t rows, k;
+    if (lin_dims(m, layer, which, &rows, &k))
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_set_linear: unknown linear %d", which);
+    if (w->n_rows != rows || w->k != k)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: expected [%lld, %lld], got [%lld, %lld]", (long long)rows,
+                        (long long)k, (long long)w->n_rows, (long long)w->k);
+    axq_weight **slot;
+    int64_t slot_rows = rows, row_off = 0;
+    if (layer < 0) {
+        slot = &m->w_head;
+    } else if (which <= AXQ_LIN_V) {
+        slot = &m->w_qkv[layer];
+        slot_rows = m->qkv_rows;
+        row_off = which == AXQ_LIN_Q ? 0 : (which == AXQ_LIN_K ? m->q_dim : m->q_dim + m->kv_dim);
+    } else if (which == AXQ_LIN_O) {
+        slot = &m->w_o[layer];
+    } else if (which == AXQ_LIN_DOWN) {
+        slot = &m->w_down[layer];
+    } else {
+        slot = &m->w_gu[layer];
+        slot_rows = 2 * (int64_t)m->cfg.intermediate_size;
+        row_off = which == AXQ_LIN_GATE ? 0 : m->cfg.intermediate_size;
+    }
+    int rc;
+    if (!*slot && (rc = axq_weight_alloc(ctx, w->type, slot_rows, k, slot))) return rc;
+    if ((*slot)->type != w->type)
+        return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: fused weight holds %s, got %s",
+                        axq_type_name((*slot)->type), axq_type_name(w->type));
+    if ((rc = copy_rows(ctx, *slot, w, row_off))) return rc;
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    if (layer < 0) m->head_set = true; else m->set_mask[layer] |= 1u << which;
+    return AXQ_OK;
+}
+
+int axq_model_random_init(axq_model *m, int type, float std, uint64_t seed) {
+    if (!m) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    const axq_model_config &c = m->cfg;
+    size_t max_elems = (size_t)c.vocab_size * c.hidden_size;
+    for (int which = 0; which < AXQ_LIN_COUNT; which++) {
+        int64_t r, k;
+        lin_dims(m, 0, which, &r, &k);
+        if ((size_t)(r * k) > max_elems) max_elems = (size_t)(r * k);
+    }
+    float *tmp = nullptr;
+    AXQ_HIP(ctx, dev_alloc(&tmp, max_elems), AXQ_ERR_ALLOCATION_FAILED);
+    int rc = AXQ_OK;
+    uint64_t s = seed;
+    auto one = [&](int layer, int which) {
+        int64_t r, k;
+        lin_dims(m, layer, which, &r, &k);
+        rc = axq_fill_normal_f32(ctx, tmp, (size_t)(r * k), 0.0f, std, 0.0f, 0.0f, ++s);
+        axq_weight *w = nullptr;
+        if (!rc) rc = axq_weight_quantize(ctx, type, r, k, tmp, AXQ_MEM_DEVICE, &w);
+        if (!rc) rc = axq_model_set_linear(m, layer, which, w);
+        axq_weight_free(ctx, w);
+    };
+    for (int l = 0; l < c.num_hidden_layers && !rc; l++)
+        for (int which = 0; which < AXQ_LIN_COUNT && !rc; which++) one(l, which);
+    if (!rc) one(-1, 0);
+    if (!rc) {
+        size_t n = (size_t)c.vocab_size * c.hidden_size;
+        rc = axq_fill_normal_f32(ctx, tmp, n, 0.0f, std, 0.0f, 0.0f, ++s);
+        if (!rc && !m->emb && dev_alloc(&m->emb, n) != hipSuccess) rc = axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "embedding");
+        if (!rc) f32_to_f16_kernel<<<(unsigned)((n + 255) / 256), 256, 0, ctx->stream>>>(tmp, n, m->emb);
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(tmp);
+    return rc;
+}
+
+int axq_model_reset(axq_model *m) {
+    if (!m) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->pos, 0);
+    set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->gen, 0);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    m->host_pos = 0;
+    return AXQ_OK;
+}
+
+int axq_model_seq_len(const axq_model *m) { return m ? m->host_pos : -1; }
+
+int axq_model_read_kv(axq_model *m, int layer, int which, uint16_t *out) {
+    if (!m || !out || layer < 0 || layer >= m->cfg.num_hidden_layers) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    size_t per_layer = (size_t)m->cfg.num_key_value_heads * m->cfg.max_position_embeddings * m->cfg.head_dim;
+    const uint16_t *src = (which ? m->vcache : m->kcache) + (size_t)layer * per_layer;
+    AXQ_HIP(ctx, hipMemcpyAsync(out, src, per_layer * 2, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_model_read_hidden(axq_model *m, float *hidden_out) {
+    if (!m || !hidden_out) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    AXQ_HIP(ctx, hipMemcpyAsync(hidden_out, m->h, (size_t)m->cfg.hidden_size * 4, hipMemcpyDeviceToHost, ctx->stream),
+            AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_t *next_token) {
+    if (!m) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    int rc;
+    if ((rc = check_ready(m))) return rc;
+    if (token < 0 || token >= m->cfg.vocab_size)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "token %d outside the vocabulary of %d", token, m->cfg.vocab_size);
+    if (m->host_pos >= m->cfg.max_position_embeddings)
+        return axq_fail(ctx, AXQ_ERR_OVERFLOW, "Numerical overflow during quantization: KV cache is full (%d positions)",
+                        m->cfg.max_position_embeddings);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->tok, token);
+    if ((rc = run_step(m))) return rc;
+    m->host_pos++;
+    if (logits)
+        AXQ_HIP(ctx, hipMemcpyAsync(logits, m->logits, (size_t)m->cfg.vocab_size * 4, hipMemcpyDeviceToHost, ctx->stream),
+                AXQ_ERR_COPY_FAILED);
+    if (next_token)
+        AXQ_HIP(ctx, hipMemcpyAsync(next_token, m->next, 4, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_model_generate(axq_model *m, const int32_t *prompt, int n_prompt, int max_new_tokens, int32_t *out_tokens,
+                       float *prefill_ms, float *decode_ms) {
+    if (!m || !prompt || (max_new_tokens > 0 && !out_tokens)) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    int rc;
+    if ((rc = check_ready(m))) return rc;
+    if (n_prompt <= 0 || max_new_tokens < 0)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: prompt must hold at least one token");
+    if (m->host_pos + n_prompt + max_new_tokens - 1 > m->cfg.max_position_embeddings || n_prompt > m->prompt_cap ||
+        max_new_tokens > m->out_cap)
+        return axq_fail(ctx, AXQ_ERR_OVERFLOW, "Numerical overflow during quantization: %d + %d + %d positions exceed the cache of %d",
+                        m->host_pos, n_prompt, max_new_tokens, m->cfg.max_position_embeddings);
+    for (int i = 0; i < n_prompt; i++)
+        if (prompt[i] < 0 || prompt[i] >= m->cfg.vocab_size)
+            return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "prompt token %d outside the vocabulary", prompt[i]);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipMemcpyAsync(m->prompt, prompt, (size_t)n_prompt * 4, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->gen, 0);
+    const int base = m->host_pos;
+    hipEvent_t e0, e1, e2;
+    AXQ_HIP(ctx, hipEventCreate(&e0), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipEventCreate(&e1), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipEventCreate(&e2), AXQ_ERR_DRIVER);
+    (void)hipEventRecord(e0, ctx->stream);
+    // prompt: one step per token (the cache fills position by position)
+    for (int i = 0; i < n_prompt && !rc; i++) {
+        pick_prompt_kernel<<<1, 1, 0, ctx->stream>>>(m->prompt, m->pos, base, m->tok);
+        rc = run_step(m);
+    }
+    (void)hipEventRecord(e1, ctx->stream);
+    // generation: the argmax of step i is the input of step i+1, on the device
+    for (int i = 0; i < max_new_tokens && !rc; i++) {
+        commit_next_kernel<<<1, 1, 0, ctx->stream>>>(m->next, m->tok, m->gen, m->out, m->out_cap);
+        if (i + 1 < max_new_tokens) rc = run_step(m);
+    }
+    (void)hipEventRecord(e2, ctx->stream);
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    float ms = 0.f;
+    if (!rc && e == hipSuccess) {
+        if (prefill_ms && hipEventElapsedTime(&ms, e0, e1) == hipSuccess) *prefill_ms = ms;
+        if (decode_ms && hipEventElapsedTime(&ms, e1, e2) == hipSuccess) *decode_ms = ms;
+    }
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); (void)hipEventDestroy(e2);
+    if (rc) return rc;
+    if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "generate: %s", hipGetErrorString(e));
+    m->host_pos = base + n_prompt + (max_new_tokens > 0 ? max_new_tokens - 1 : 0);
+    if (max_new_tokens > 0)
+        AXQ_HIP(ctx, hipMemcpy(out_tokens, m->out, (size_t)max_new_tokens * 4, hipMemcpyDeviceToHost), AXQ_ERR_COPY_FAILED);
+    return AXQ_OK;
+}
+
+} // extern "C"

@@ -66,13 +66,14 @@ __device__ inline float wave_sum_lane63(float v) {
 // The four bytes of `v` must each hold a value 0..15.  v_cvt_pk_f32_fp8 turns
 // such a byte n into n * unit (the 8-bit float with a 3-bit mantissa is linear
 // over 0..15), two bytes per instruction; x has been pre-multiplied by 1/unit.
-__device__ inline void fma_nibbles4(uint32_t v, const float *xs, float &acc) {
+// `c` = 8 * unit: the codes are centred (n - 8) before the multiply so that no large sums cancel later.
+__device__ inline void fma_nibbles4(uint32_t v, const float *xs, float c, float &acc) {
     float2v a = __builtin_amdgcn_cvt_pk_f32_fp8((int)v, false);
     float2v b = __builtin_amdgcn_cvt_pk_f32_fp8((int)v, true);
-    acc = fmaf(a[0], xs[0], acc);
-    acc = fmaf(a[1], xs[1], acc);
-    acc = fmaf(b[0], xs[2], acc);
-    acc = fmaf(b[1], xs[3], acc);
+    acc = fmaf(a[0] - c, xs[0], acc);
+    acc = fmaf(a[1] - c, xs[1], acc);
+    acc = fmaf(b[0] - c, xs[2], acc);
+    acc = fmaf(b[1] - c, xs[3], acc);
 }
 
 // ---------------------------------------------------------------------------
@@ -106,7 +107,8 @@ struct Q4K {
         r.q1 = *reinterpret_cast<const uint4 *>(base + (size_t)P * 16);
         r.h = *reinterpret_cast<const uint4 *>(a.meta + (size_t)row * a.meta_pitch + (size_t)(chunk >> 2) * 16);
     }
-    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int chunk) {
+    __device__ static float dot(const GemvArgs &a, const Raw &r, const X &x, int chunk) {
+        const float c8 = 8.0f / a.fp8_unit_inv;
         int p = chunk & 3;
         // 6-bit scale/min of sub-blocks 2p and 2p+1 (ggml get_scale_min_k4 order)
         int sh = (p & 1) * 16;
@@ -126,16 +128,17 @@ struct Q4K {
 #pragma unroll
         for (int w = 0; w < 4; w++) {
             // first half of the pair: bytes 4w..4w+3 -> elements 4w.. (low), 32+4w.. (high)
-            fma_nibbles4(q0[w] & 0x0F0F0F0Fu, &x.xs[4 * w], alo0);
-            fma_nibbles4((q0[w] >> 4) & 0x0F0F0F0Fu, &x.xs[32 + 4 * w], ahi0);
+            fma_nibbles4(q0[w] & 0x0F0F0F0Fu, &x.xs[4 * w], c8, alo0);
+            fma_nibbles4((q0[w] >> 4) & 0x0F0F0F0Fu, &x.xs[32 + 4 * w], c8, ahi0);
             // second half: bytes 16+4w.. -> elements 16+4w.. (low), 48+4w.. (high)
-            fma_nibbles4(q1[w] & 0x0F0F0F0Fu, &x.xs[16 + 4 * w], alo1);
-            fma_nibbles4((q1[w] >> 4) & 0x0F0F0F0Fu, &x.xs[48 + 4 * w], ahi1);
+            fma_nibbles4(q1[w] & 0x0F0F0F0Fu, &x.xs[16 + 4 * w], c8, alo1);
+            fma_nibbles4((q1[w] >> 4) & 0x0F0F0F0Fu, &x.xs[48 + 4 * w], c8, ahi1);
         }
-        float sc0 = ubyte0(scp), sc1 = ubyte1(scp), m0 = ubyte0(mp), m1 = ubyte1(mp);
-        float pos = fmaf(sc0, alo0 + alo1, sc1 * (ahi0 + ahi1));
-        float neg = fmaf(m0, x.sum_lo, m1 * x.sum_hi);
-        return fmaf(d, pos, -(dmin * neg));
+        float s0 = d * ubyte0(scp), s1 = d * ubyte1(scp);
+        float y = fmaf(s0, alo0 + alo1, s1 * (ahi0 + ahi1)); // sum d*sc*(q - 8)*x
+        y = fmaf(fmaf(8.0f, s0, -(dmin * ubyte0(mp))), x.sum_lo, y);
+        y = fmaf(fmaf(8.0f, s1, -(dmin * ubyte1(mp))), x.sum_hi, y);
+        return y;
     }
 };
 
@@ -162,8 +165,9 @@ struct Q4x { // Q4_0 / Q4_1: adjacent-pair nibble order (types.rs:179-198)
         if (WITH_MIN) r.m = *reinterpret_cast<const uint32_t *>(m + (size_t)chunk * 4);
         else r.m = *reinterpret_cast<const uint16_t *>(m + (size_t)chunk * 2);
     }
-    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int) {
+    __device__ static float dot(const GemvArgs &a, const Raw &r, const X &x, int) {
         const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        const float c8 = 8.0f / a.fp8_unit_inv;
         float a0 = 0.f, a1 = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
@@ -172,15 +176,15 @@ struct Q4x { // Q4_0 / Q4_1: adjacent-pair nibble order (types.rs:179-198)
             float2v la = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, false), lb = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, true);
             float2v ha = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, false), hb = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, true);
             const float *xs = &x.xs[8 * w];
-            a0 = fmaf(la[0], xs[0], a0); a1 = fmaf(ha[0], xs[1], a1);
-            a0 = fmaf(la[1], xs[2], a0); a1 = fmaf(ha[1], xs[3], a1);
-            a0 = fmaf(lb[0], xs[4], a0); a1 = fmaf(hb[0], xs[5], a1);
-            a0 = fmaf(lb[1], xs[6], a0); a1 = fmaf(hb[1], xs[7], a1);
+            a0 = fmaf(la[0] - c8, xs[0], a0); a1 = fmaf(ha[0] - c8, xs[1], a1);
+            a0 = fmaf(la[1] - c8, xs[2], a0); a1 = fmaf(ha[1] - c8, xs[3], a1);
+            a0 = fmaf(lb[0] - c8, xs[4], a0); a1 = fmaf(hb[0] - c8, xs[5], a1);
+            a0 = fmaf(lb[1] - c8, xs[6], a0); a1 = fmaf(hb[1] - c8, xs[7], a1);
         }
         float scale = f16_bits_to_f32(r.m & 0xFFFF);
-        float acc = a0 + a1;
-        if (WITH_MIN) return fmaf(scale, acc, f16_bits_to_f32(r.m >> 16) * x.sum);
-        return scale * fmaf(-8.0f, x.sum, acc);
+        float acc = a0 + a1; // sum (n - 8) x
+        if (WITH_MIN) return fmaf(scale, acc, fmaf(8.0f, scale, f16_bits_to_f32(r.m >> 16)) * x.sum);
+        return scale * acc;
     }
 };
 
@@ -218,15 +222,15 @@ struct Q5x { // Q5_0 / Q5_1: byte j = elements j (low nibble) and j+16 (high); q
             uint32_t lo = (q[w] & 0x0F0F0F0Fu) | (bl << 4);
             uint32_t hi = ((q[w] >> 4) & 0x0F0F0F0Fu) | (bh << 4);
             const float *xl = &x.xs[4 * w], *xh = &x.xs[16 + 4 * w];
-            a0 = fmaf(ubyte0(lo), xl[0], a0); a1 = fmaf(ubyte0(hi), xh[0], a1);
-            a0 = fmaf(ubyte1(lo), xl[1], a0); a1 = fmaf(ubyte1(hi), xh[1], a1);
-            a0 = fmaf(ubyte2(lo), xl[2], a0); a1 = fmaf(ubyte2(hi), xh[2], a1);
-            a0 = fmaf(ubyte3(lo), xl[3], a0); a1 = fmaf(ubyte3(hi), xh[3], a1);
+            a0 = fmaf(ubyte0(lo) - 16.0f, xl[0], a0); a1 = fmaf(ubyte0(hi) - 16.0f, xh[0], a1);
+            a0 = fmaf(ubyte1(lo) - 16.0f, xl[1], a0); a1 = fmaf(ubyte1(hi) - 16.0f, xh[1], a1);
+            a0 = fmaf(ubyte2(lo) - 16.0f, xl[2], a0); a1 = fmaf(ubyte2(hi) - 16.0f, xh[2], a1);
+            a0 = fmaf(ubyte3(lo) - 16.0f, xl[3], a0); a1 = fmaf(ubyte3(hi) - 16.0f, xh[3], a1);
         }
         float d = f16_bits_to_f32(r.m & 0xFFFF);
-        float acc = a0 + a1;
-        if (WITH_MIN) return fmaf(d, acc, f16_bits_to_f32(r.m >> 16) * x.sum);
-        return d * fmaf(-16.0f, x.sum, acc);
+        float acc = a0 + a1; // sum (u - 16) x
+        if (WITH_MIN) return fmaf(d, acc, fmaf(16.0f, d, f16_bits_to_f32(r.m >> 16)) * x.sum);
+        return d * acc;
     }
 };
 

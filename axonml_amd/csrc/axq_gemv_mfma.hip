@@ -31,6 +31,7 @@
 #include <hip/hip_fp16.h>
 
 #include "axq_internal.h"
+#include "axq_split.h"
 
 namespace {
 
@@ -67,6 +68,8 @@ __device__ inline float recombine(int4v d, float sg) {
 struct XOp {
     int a[16];
     float sg[2], xs[2];
+    int4v init[2]; // -(code centre) * (limb sums of the group): the accumulators start here, so that the
+                   // MFMAs sum (n - centre) * limb exactly and no large terms cancel in f32 afterwards
 };
 
 // ---------------------------------------------------------------------------
@@ -78,6 +81,7 @@ struct XOp {
 struct DQ4K {
     struct Raw { uint4 q0, q1, h; };
     static constexpr bool PERM_A = false;
+    static constexpr int CENTRE = 8; // w = d*sc*(q - 8) + (8*d*sc - dmin*m)
     __device__ static int group_k(int c, int g) { return c * 64 + g * 32; }
     __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
         // the code plane interleaves, per 64-pair slice, the first 16 bytes of every pair, then the second 16
@@ -94,7 +98,7 @@ struct DQ4K {
     __device__ static float dot(const Raw &r, const XOp &x, int c) {
         const uint32_t q0[4] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w};
         const uint32_t q1[4] = {r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-        int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+        int4v lo = x.init[0], hi = x.init[1];
 #pragma unroll
         for (int w = 0; w < 4; w++) { // bytes 4w..4w+3 of the first half: elements 4w.. of both sub-blocks
             lo = mfma(x.a[w], q0[w] & 0x0F0F0F0Fu, lo);
@@ -117,9 +121,13 @@ struct DQ4K {
             scp = (wa & 0x0F0F) | ((ya >> 2) & 0x3030);
             mp = ((wa >> 4) & 0x0F0F) | ((za >> 2) & 0x3030);
         }
-        float pos = fmaf(ub0(scp), recombine(lo, x.sg[0]), ub1(scp) * recombine(hi, x.sg[1]));
-        float neg = fmaf(ub0(mp), x.xs[0], ub1(mp) * x.xs[1]);
-        return fmaf(f16lo(r.h.x), pos, -(f16hi(r.h.x) * neg));
+        const float d = f16lo(r.h.x), dmin = f16hi(r.h.x);
+        const float s0 = d * ub0(scp), s1 = d * ub1(scp);
+        float y = fmaf(s0, recombine(lo, x.sg[0]), s1 * recombine(hi, x.sg[1]));
+        // what is left of the offsets after centring: small, since dmin*m ~ 8*d*sc for weights centred on zero
+        y = fmaf(fmaf(8.0f, s0, -(dmin * ub0(mp))), x.xs[0], y);
+        y = fmaf(fmaf(8.0f, s1, -(dmin * ub1(mp))), x.xs[1], y);
+        return y;
     }
 };
 
@@ -130,6 +138,7 @@ template <bool WITH_MIN>
 struct DQ4x {
     struct Raw { uint4 q[2]; uint32_t m[2]; };
     static constexpr bool PERM_A = true; // dword w of a block: low nibbles = elements 8w+{0,2,4,6}, high = 8w+{1,3,5,7}
+    static constexpr int CENTRE = 8;
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
     __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
@@ -150,16 +159,16 @@ struct DQ4x {
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             const uint32_t q[4] = {r.q[g].x, r.q[g].y, r.q[g].z, r.q[g].w};
-            int4v e = {0, 0, 0, 0}, o = {0, 0, 0, 0};
+            int4v e = x.init[g], o = {0, 0, 0, 0};
 #pragma unroll
             for (int w = 0; w < 4; w++) {
                 e = mfma(x.a[8 * g + 2 * w], q[w] & 0x0F0F0F0Fu, e);
                 o = mfma(x.a[8 * g + 2 * w + 1], (q[w] >> 4) & 0x0F0F0F0Fu, o);
             }
-            float acc = recombine(e + o, x.sg[g]);
+            float acc = recombine(e + o, x.sg[g]); // sum (n - 8) x
             float scale = f16lo(r.m[g]);
-            if (WITH_MIN) tot += fmaf(scale, acc, f16hi(r.m[g]) * x.xs[g]);
-            else tot += scale * fmaf(-8.0f, x.xs[g], acc);
+            if (WITH_MIN) tot += fmaf(scale, acc, fmaf(8.0f, scale, f16hi(r.m[g])) * x.xs[g]);
+            else tot += scale * acc;
         }
         return tot;
     }
@@ -170,6 +179,7 @@ template <bool WITH_MIN>
 struct DQ5x {
     struct Raw { uint4 q[2]; uint32_t qh[2]; uint32_t m[2]; };
     static constexpr bool PERM_A = false;
+    static constexpr int CENTRE = 16;
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
     __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
@@ -192,7 +202,7 @@ struct DQ5x {
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             const uint32_t q[4] = {r.q[g].x, r.q[g].y, r.q[g].z, r.q[g].w};
-            int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+            int4v lo = x.init[g], hi = {0, 0, 0, 0};
 #pragma unroll
             for (int w = 0; w < 4; w++) {
                 // spread 4 bits of qh to bit 4 of each byte: t * 0x00204081 puts bit i at bit 8i
@@ -201,10 +211,10 @@ struct DQ5x {
                 lo = mfma(x.a[8 * g + w], (q[w] & 0x0F0F0F0Fu) | (bl << 4), lo);
                 hi = mfma(x.a[8 * g + 4 + w], ((q[w] >> 4) & 0x0F0F0F0Fu) | (bh << 4), hi);
             }
-            float acc = recombine(lo + hi, x.sg[g]);
+            float acc = recombine(lo + hi, x.sg[g]); // sum (u - 16) x
             float d = f16lo(r.m[g]);
-            if (WITH_MIN) tot += fmaf(d, acc, f16hi(r.m[g]) * x.xs[g]);
-            else tot += d * fmaf(-16.0f, x.xs[g], acc);
+            if (WITH_MIN) tot += fmaf(d, acc, fmaf(16.0f, d, f16hi(r.m[g])) * x.xs[g]);
+            else tot += d * acc;
         }
         return tot;
     }
@@ -214,6 +224,7 @@ struct DQ5x {
 struct DQ80 {
     struct Raw { uint4 q[4]; uint32_t m[2]; };
     static constexpr bool PERM_A = false;
+    static constexpr int CENTRE = 0;
     // 16-byte vector v (0..3) of chunk c: vector index along the row; block = vector / 2
     __device__ static int vec_index(int c, int v) { return ((c >> 4) << 6) + (v >> 1) * 32 + (c & 15) * 2 + (v & 1); }
     __device__ static int group_k(int c, int g) { return vec_index(c, 2 * g) * 16; }
@@ -248,76 +259,13 @@ struct DQ80 {
     }
 };
 
-// ---------------------------------------------------------------------------
-// x staging: LDS holds four int8 limb planes [K] and, per 32-element group, the
-// f32 scale that turns limb sums back into sum(n*x), and the plain sum of x.
-// ---------------------------------------------------------------------------
-__device__ inline void stage_x(const float *x, int k, uint8_t *planes, float2 *grp, int tid, int nthreads) {
-    const int kpad = (k + 15) & ~15;
-    // one task = 8 consecutive elements; 4 consecutive lanes share a 32-element group
-    const int ntask = (k + 7) >> 3;
-    const int ntask_pad = (ntask + 3) & ~3;
-    for (int t = tid; t < ntask_pad; t += nthreads) {
-        float v[8];
-        const bool live = t < ntask;
-        if (live) {
-            const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)t * 8);
-            float4 a = p[0], b = p[1];
-            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = 0.f;
-        }
-        float amax = 0.f, sum = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            amax = fmaxf(amax, fabsf(v[i]));
-            sum += v[i];
-        }
-        amax = fmaxf(amax, __shfl_xor(amax, 1));
-        amax = fmaxf(amax, __shfl_xor(amax, 2));
-        sum += __shfl_xor(sum, 1);
-        sum += __shfl_xor(sum, 2);
-        // amax in [2^e, 2^(e+1)): scale so that |x| * f < 2^27, f = 2^(26-e); limb sums times 2^(e-26) give back x
-        uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFF;
-        const bool bad = eb == 0xFF; // inf or nan in the group: poison the scale so that the row becomes nan
-        eb = eb < 30 ? 30 : eb;
-        eb = eb > 254 ? 254 : eb;
-        float f = __builtin_bit_cast(float, (280u - eb) << 23);
-        float sg = __builtin_bit_cast(float, (eb - 26u) << 23);
-        if (bad) sg = __builtin_nanf("");
-        uint32_t l[4][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            int tq = bad ? 0 : (int)rintf(v[i] * f);
-            int l3 = ((tq + 64) & 127) - 64;
-            tq = (tq - l3) >> 7;
-            int l2 = ((tq + 64) & 127) - 64;
-            tq = (tq - l2) >> 7;
-            int l1 = ((tq + 64) & 127) - 64;
-            int l0 = (tq - l1) >> 7;
-            int sh = 8 * (i & 3);
-            l[0][i >> 2] |= (uint32_t)(l0 & 0xFF) << sh;
-            l[1][i >> 2] |= (uint32_t)(l1 & 0xFF) << sh;
-            l[2][i >> 2] |= (uint32_t)(l2 & 0xFF) << sh;
-            l[3][i >> 2] |= (uint32_t)(l3 & 0xFF) << sh;
-        }
-        if (live) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                *reinterpret_cast<uint2 *>(planes + (size_t)i * kpad + (size_t)t * 8) = make_uint2(l[i][0], l[i][1]);
-            if ((t & 3) == 0) grp[t >> 2] = make_float2(sg, sum);
-        }
-    }
-}
-
 // Gather bytes {0,2} of lo and {0,2} of hi (sel = 0) or {1,3} of each (sel = 1)
 __device__ inline int pick_alt(uint32_t lo, uint32_t hi, int sel) {
     return (int)__builtin_amdgcn_perm(hi, lo, sel ? 0x07050301u : 0x06040200u);
 }
 
 template <class T>
-__device__ inline void fetch_xop(const uint8_t *planes, const float2 *grp, int kpad, int k, int limb, int c, XOp &o) {
+__device__ inline void fetch_xop(const uint8_t *planes, const uint4 *grp, int kpad, int k, int limb, int c, XOp &o) {
 #pragma unroll
     for (int g = 0; g < 2; g++) {
         int kb = T::group_k(c, g);
@@ -326,14 +274,19 @@ __device__ inline void fetch_xop(const uint8_t *planes, const float2 *grp, int k
             const uint4 *p = reinterpret_cast<const uint4 *>(planes + (size_t)limb * kpad + kb);
             uint4 u = p[0], v = p[1];
             nat[0] = u.x; nat[1] = u.y; nat[2] = u.z; nat[3] = u.w; nat[4] = v.x; nat[5] = v.y; nat[6] = v.z; nat[7] = v.w;
-            float2 sv = grp[kb >> 5];
-            o.sg[g] = sv.x;
-            o.xs[g] = sv.y;
+            uint4 sv = grp[kb >> 5];
+            o.sg[g] = __builtin_bit_cast(float, sv.x);
+            o.xs[g] = __builtin_bit_cast(float, sv.y);
+            o.init[g][0] = -T::CENTRE * ((int)(sv.z << 16) >> 16);
+            o.init[g][1] = -T::CENTRE * ((int)sv.z >> 16);
+            o.init[g][2] = -T::CENTRE * ((int)(sv.w << 16) >> 16);
+            o.init[g][3] = -T::CENTRE * ((int)sv.w >> 16);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; i++) nat[i] = 0;
             o.sg[g] = 0.f;
             o.xs[g] = 0.f;
+            o.init[g] = int4v{0, 0, 0, 0};
         }
         if (T::PERM_A) {
 #pragma unroll
@@ -367,9 +320,9 @@ __global__ void __launch_bounds__(512) gemv_dp_kernel(DpArgs a) {
     const int kpad = (a.k + 15) & ~15;
     // PRE: the limbs come from global memory (written by prep_x_kernel or by the kernel that produced x)
     const uint8_t *planes = PRE ? a.xq : reinterpret_cast<const uint8_t *>(lds_raw);
-    const float2 *grp = reinterpret_cast<const float2 *>(planes + (size_t)4 * kpad);
+    const uint4 *grp = reinterpret_cast<const uint4 *>(planes + (size_t)4 * kpad);
     float *red = PRE ? reinterpret_cast<float *>(lds_raw)
-                     : reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(lds_raw) + (size_t)4 * kpad + (size_t)((a.k + 31) >> 5) * 8);
+                     : reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(lds_raw) + (size_t)4 * kpad + (size_t)((a.k + 31) >> 5) * 16);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -408,7 +361,7 @@ __global__ void __launch_bounds__(512) gemv_dp_kernel(DpArgs a) {
     if (!PRE) {
         // x -> limbs in LDS -> this lane's A operands, while the weights are on their way
         uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw);
-        stage_x(a.x, a.k, wplanes, reinterpret_cast<float2 *>(wplanes + (size_t)4 * kpad), tid, (int)blockDim.x);
+        stage_x(a.x, a.k, wplanes, reinterpret_cast<uint4 *>(wplanes + (size_t)4 * kpad), tid, (int)blockDim.x);
         __syncthreads();
 #pragma unroll
         for (int p = 0; p < PP; p++) fetch_xop<T>(planes, grp, kpad, a.k, j, c[p], xo[p]);
@@ -455,7 +408,7 @@ __global__ void __launch_bounds__(512) gemv_dp_kernel(DpArgs a) {
 
 __global__ void __launch_bounds__(256) prep_x_kernel(const float *x, int k, uint8_t *xq) {
     const int kpad = (k + 15) & ~15;
-    stage_x(x, k, xq, reinterpret_cast<float2 *>(xq + (size_t)4 * kpad), (int)(blockIdx.x * blockDim.x + threadIdx.x),
+    stage_x(x, k, xq, reinterpret_cast<uint4 *>(xq + (size_t)4 * kpad), (int)(blockIdx.x * blockDim.x + threadIdx.x),
             (int)(gridDim.x * blockDim.x));
 }
 
@@ -486,7 +439,7 @@ bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t 
     unsigned block = (unsigned)(64 * a.S * a.G);
     int kpad = (a.k + 15) & ~15;
     size_t lds = (size_t)wg_rows * a.S * 4 * 4;
-    if (!xq) lds += (size_t)4 * kpad + (size_t)((a.k + 31) / 32) * 8;
+    if (!xq) lds += (size_t)4 * kpad + (size_t)((a.k + 31) / 32) * 16;
     if (lds > 64 * 1024) return false;
     if (xq) {
         if (a.P == 1) gemv_dp_kernel<T, 4, 1, true><<<grid, block, lds, ctx->stream>>>(a);
@@ -501,7 +454,7 @@ bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t 
 } // namespace
 
 // Bytes of the split form of a K-vector: four limb planes and one (scale, sum) pair per 32 elements.
-size_t axq_xq_bytes(int64_t k) { return (size_t)4 * (size_t)((k + 15) & ~15) + (size_t)((k + 31) / 32) * 8; }
+size_t axq_xq_bytes(int64_t k) { return axq_split_bytes(k); }
 
 // x[k] (f32, device) -> split form at xq (device, axq_xq_bytes(k) bytes).
 int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq) {

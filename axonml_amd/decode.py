@@ -1,0 +1,160 @@
+"""Host-side mirror of the reference's LLaMA/Mistral decode loop over the axq C ABI.
+
+`QuantizedLlama` plays the part of LLaMAForCausalLM (crates/axonml-llm/src/llama.rs:834-1100) for one
+sequence: `forward_with_cache`-style single-token steps and greedy `generate`, with every linear a
+quantized, device-resident weight.  Config field names follow LLaMAConfig / MistralConfig.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import MEM_HOST
+from .quant import DeviceWeight, QuantType, default_context
+
+LINEARS = {"q": 0, "k": 1, "v": 2, "o": 3, "gate": 4, "up": 5, "down": 6}
+
+
+def mistral_7b_config(max_position_embeddings=640):
+    """MistralConfig::mistral_7b (crates/axonml-llm/src/mistral.rs:56-70), context capped to the cache size."""
+    return dict(vocab_size=32000, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32,
+                num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                max_position_embeddings=max_position_embeddings, rms_norm_eps=1e-5, rope_theta=10000.0)
+
+
+class QuantizedLlama:
+    def __init__(self, ctx=None, **cfg):
+        self.ctx = ctx or default_context()
+        self.cfg = _lib.ModelConfig(**cfg)
+        h = C.c_void_p()
+        self.ctx.check(self.ctx.lib.axq_model_create(self.ctx.handle, C.byref(self.cfg), C.byref(h)))
+        self.handle = h
+
+    # ---- weights
+    def set_embedding_f16(self, table_bits):
+        t = np.ascontiguousarray(table_bits, dtype=np.uint16)
+        assert t.size == self.cfg.vocab_size * self.cfg.hidden_size
+        self.ctx.check(self.ctx.lib.axq_model_set_embedding_f16(self.handle, t.ctypes.data, MEM_HOST))
+
+    def set_norm(self, layer, which, w):
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        self.ctx.check(self.ctx.lib.axq_model_set_norm(self.handle, layer, which, w.ctypes.data, MEM_HOST))
+
+    def set_linear(self, layer, name, weight):
+        """weight: QuantizedTensor or DeviceWeight of the linear's [out, in] shape; layer -1 = lm_head."""
+        dw = weight if isinstance(weight, DeviceWeight) else DeviceWeight.upload(weight, self.ctx)
+        try:
+            self.ctx.check(self.ctx.lib.axq_model_set_linear(self.handle, layer, LINEARS.get(name, 0), dw.handle))
+        finally:
+            if dw is not weight:
+                dw.free()
+
+    def random_init(self, quant_type=QuantType.Q4_K, std=0.02, seed=1):
+        self.ctx.check(self.ctx.lib.axq_model_random_init(self.handle, int(quant_type), std, seed))
+
+    # ---- stepping
+    def reset(self):
+        self.ctx.check(self.ctx.lib.axq_model_reset(self.handle))
+
+    def seq_len(self):
+        return self.ctx.lib.axq_model_seq_len(self.handle)
+
+    def forward(self, token, want_logits=True):
+        logits = np.empty(self.cfg.vocab_size, dtype=np.float32) if want_logits else None
+        nxt = C.c_int32()
+        self.ctx.check(self.ctx.lib.axq_model_forward(self.handle, int(token), logits.ctypes.data if want_logits else None,
+                                                      C.byref(nxt)))
+        return nxt.value, logits
+
+    def hidden(self):
+        out = np.empty(self.cfg.hidden_size, dtype=np.float32)
+        self.ctx.check(self.ctx.lib.axq_model_read_hidden(self.handle, out.ctypes.data))
+        return out
+
+    def kv(self, layer, which):
+        c = self.cfg
+        out = np.empty((c.num_key_value_heads, c.max_position_embeddings, c.head_dim), dtype=np.uint16)
+        self.ctx.check(self.ctx.lib.axq_model_read_kv(self.handle, layer, which, out.ctypes.data))
+        return out
+
+    def generate(self, prompt, max_new_tokens):
+        p = np.ascontiguousarray(prompt, dtype=np.int32)
+        out = np.empty(max_new_tokens, dtype=np.int32)
+        pre, dec = C.c_float(), C.c_float()
+        self.ctx.check(self.ctx.lib.axq_model_generate(self.handle, p.ctypes.data, p.size, max_new_tokens, out.ctypes.data,
+                                                       C.byref(pre), C.byref(dec)))
+        return out, pre.value, dec.value
+
+    def close(self):
+        if self.handle:
+            self.ctx.lib.axq_model_free(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def smoke(ctx):
+    """Two-layer model, a few tokens, against the CPU decode oracle (called from __graft_entry__.smoke)."""
+    import oracle as o
+
+    cfg = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+               num_key_value_heads=2, head_dim=64, max_position_embeddings=32, rms_norm_eps=1e-5, rope_theta=10000.0)
+    rng = np.random.default_rng(0)
+    gpu = QuantizedLlama(ctx, **cfg)
+    cpu = o.DecodeModel(vocab_size=512, hidden_size=256, intermediate_size=512, num_layers=2, num_heads=4, num_kv_heads=2,
+                        head_dim=64, max_seq_len=32, rms_norm_eps=1e-5, rope_theta=10000.0)
+    emb = (rng.standard_normal((512, 256)) * 0.5).astype(np.float16).view(np.uint16)
+    gpu.set_embedding_f16(emb)
+    cpu.set_embedding_f16(emb)
+    shapes = {"q": (256, 256), "k": (128, 256), "v": (128, 256), "o": (256, 256), "gate": (512, 256), "up": (512, 256),
+              "down": (256, 512)}
+    from .quant import QuantizedTensor
+
+    for layer in list(range(2)) + [-1]:
+        for name, (n, k) in (shapes.items() if layer >= 0 else [("q", (512, 256))]):
+            w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+            packed = o.quantize(o.Q4_K, w)
+            gpu.set_linear(layer, name, QuantizedTensor([n, k], QuantType.Q4_K, packed))
+            cpu.set_linear(layer, LINEARS[name], o.Q4_K, packed)
+    worst = 0.0
+    tok = 3
+    for pos in range(6):
+        g_next, g_logits = gpu.forward(tok)
+        c_next, c_logits = cpu.forward(tok, pos)
+        worst = max(worst, float(np.abs(g_logits - c_logits).max() / np.abs(c_logits).max()))
+        assert g_next == c_next, f"greedy token differs at position {pos}: {g_next} vs {c_next}"
+        tok = c_next
+    assert worst <= 1e-3, f"decode logits differ by {worst} of the logit range"
+    print(f"smoke: 2-layer Q4_K decode, 6 tokens, greedy ids equal, logits within {worst:.1e} of their range", flush=True)
+    gpu.close()
+    cpu.close()
+
+
+def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
+    """BASELINE config 4: Mistral-7B shape, random init, all linears Q4_K, f16 KV cache, greedy."""
+    cfg = mistral_7b_config(prompt_len + new_tokens)
+    m = QuantizedLlama(ctx, **cfg)
+    m.random_init(QuantType.Q4_K, 0.02, 1)
+    rng = np.random.default_rng(0)
+    prompt = rng.integers(0, cfg["vocab_size"], size=prompt_len, dtype=np.int32)
+    m.generate(prompt[:8], 4)  # warm-up: graph capture, first-touch
+    m.reset()
+    out, pre_ms, dec_ms = m.generate(prompt, new_tokens)
+    steps = new_tokens - 1
+    weights = 32 * (2 * 4096 * 4096 + 2 * 1024 * 4096 + 3 * 14336 * 4096) + 32000 * 4096
+    mean_ctx = prompt_len + new_tokens / 2
+    bytes_per_token = weights * 0.5625 + 131072 * mean_ctx + 131072
+    tok_s = steps / (dec_ms * 1e-3)
+    res = {"model": "Mistral-7B shape, random init, Q4_K linears, f16 KV cache", "prompt_tokens": prompt_len,
+           "generated_tokens": new_tokens, "prefill_ms": pre_ms, "prefill_tokens_per_s": prompt_len / (pre_ms * 1e-3),
+           "decode_ms": dec_ms, "decode_steps_timed": steps, "tokens_per_s": tok_s, "ms_per_token": dec_ms / steps,
+           "algorithmic_bytes_per_token": bytes_per_token, "gbps": bytes_per_token * tok_s / 1e9,
+           "frac_of_hbm_peak": bytes_per_token * tok_s / 8e12, "distinct_generated_ids": int(len(set(out.tolist())))}
+    log(f"  decode 7B-shape: {tok_s:.1f} tok/s ({res['ms_per_token']:.3f} ms/token, {res['gbps']:.0f} GB/s), "
+        f"prefill {res['prefill_tokens_per_s']:.0f} tok/s")
+    m.close()
+    return res

@@ -187,6 +187,10 @@ AXQ_API int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_
 AXQ_API int axq_model_generate(axq_model *m, const int32_t *prompt, int n_prompt, int max_new_tokens,
                                int32_t *out_tokens, float *prefill_ms, float *decode_ms);
 AXQ_API int axq_model_seq_len(const axq_model *m);
+/* The residual stream after the last step (f32[hidden], host): for intermediate checks in tests. */
+AXQ_API int axq_model_read_hidden(axq_model *m, float *hidden_out);
+/* One layer's f16 cache, [kv_heads][max_position_embeddings][head_dim] (host); which 0 = keys, 1 = values. */
+AXQ_API int axq_model_read_kv(axq_model *m, int layer, int which, uint16_t *out);
 
 /* ---- benchmark utilities ------------------------------------------------- */
 /* dst[i] ~ N(mean, std) from a counter-based generator (seed, i); with

@@ -57,6 +57,7 @@ def lib():
         L.axo_model_set_linear.restype, L.axo_model_set_linear.argtypes = i, [vp, i, i, i, vp]
         L.axo_model_forward.restype, L.axo_model_forward.argtypes = i, [vp, i, i, vp]
         L.axo_model_hidden.restype, L.axo_model_hidden.argtypes = C.POINTER(C.c_float), [vp]
+        L.axo_model_kv.restype, L.axo_model_kv.argtypes = C.POINTER(C.c_uint16), [vp, i, i]
         _lib = L
     return _lib
 
@@ -153,6 +154,11 @@ class DecodeModel:
 
     def hidden(self):
         return np.ctypeslib.as_array(lib().axo_model_hidden(self.h), shape=(self.cfg.hidden_size,)).copy()
+
+    def kv(self, layer, which):
+        c = self.cfg
+        shape = (c.num_kv_heads, c.max_seq_len, c.head_dim)
+        return np.ctypeslib.as_array(lib().axo_model_kv(self.h, layer, which), shape=shape).copy()
 
     def close(self):
         if self.h:

@@ -260,5 +260,10 @@ AXO_API int axo_model_forward(axo_model *m, int token, int pos, float *logits) {
     return best;
 }
 
+/* f16 cache of a layer, [kv_heads][max_seq][head_dim]; which = 0 keys (after RoPE), 1 values. */
+AXO_API const uint16_t *axo_model_kv(const axo_model *m, int layer, int which) {
+    return which ? m->layers[layer].vc : m->layers[layer].kc;
+}
+
 /* Hidden state after the last forward (for intermediate checks). */
 AXO_API const float *axo_model_hidden(const axo_model *m) { return m->h; }

@@ -1,0 +1,115 @@
+"""GPU parity: the decode step against the CPU decode oracle on small models.
+Bar: greedy token ids identical; logits within 1e-3 of the logit range (max|y - ref| / max|ref|, see
+tests/util.py for why the stack is compared normwise); f16 cache contents identical except for isolated
+one-ulp roundings."""
+import numpy as np
+import pytest
+
+import oracle as o
+from tests.decode_common import load_gpu, load_oracle, random_weights, tiny_config
+from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q4_0, o.Q8_0, o.Q5_1])
+def test_step_by_step_logits_and_tokens(ctx, qtype):
+    c = tiny_config()
+    w = random_weights(c, 10 + qtype, qtype=qtype)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    tok = 11
+    for pos in range(24):
+        c_next, c_logits = cpu.forward(tok, pos)
+        g_next, g_logits = gpu.forward(tok)
+        assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, (pos, o.TYPE_NAMES[qtype])
+        assert g_next == c_next, pos
+        tok = c_next
+    assert gpu.seq_len() == 24
+    gpu.close()
+
+
+def test_kv_cache_matches_oracle_up_to_isolated_f16_roundings(ctx):
+    c = tiny_config(num_layers=2)
+    w = random_weights(c, 50)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    tok, n = 3, 20
+    for pos in range(n):  # both sides are fed the oracle's tokens
+        gpu.forward(tok, want_logits=False)
+        tok, _ = cpu.forward(tok, pos)
+    for layer in range(2):
+        for which in (0, 1):
+            a, b = cpu.kv(layer, which)[:, :n], gpu.kv(layer, which)[:, :n]
+            differ = a != b
+            assert differ.mean() < 0.1, (layer, which, differ.mean())  # a few per cent once upstream noise reaches 1e-5
+            af, bf = a.view(np.float16).astype(np.float64), b.view(np.float16).astype(np.float64)
+            # one f16 ulp of the element; values that are small by cancellation (a rotated key is a difference
+            # of two products) carry the upstream f32 noise instead, ~1e-5 of the largest element
+            ulp = np.maximum(np.abs(af) * 2.0 ** -10, 5e-5 * np.abs(af).max())
+            bad = np.argwhere(np.abs(af - bf) > ulp)
+            assert bad.size == 0, f"cache element {bad[0]} differs by more than one f16 ulp: {af[tuple(bad[0])]} vs {bf[tuple(bad[0])]}"
+    gpu.close()
+
+
+def test_generate_matches_oracle_greedy_and_is_repeatable(ctx):
+    c = tiny_config(num_layers=3, max_seq_len=96)
+    w = random_weights(c, 20)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    rng = np.random.default_rng(0)
+    prompt = rng.integers(0, c["vocab_size"], size=17)
+    want, tok = [], None
+    for pos, t in enumerate(prompt):
+        tok, _ = cpu.forward(int(t), pos)
+    for i in range(40):
+        want.append(tok)
+        if i + 1 < 40:
+            tok, _ = cpu.forward(tok, len(prompt) + i)
+    got, pre_ms, dec_ms = gpu.generate(prompt, 40)
+    assert got.tolist() == want
+    assert gpu.seq_len() == len(prompt) + 39 and pre_ms > 0 and dec_ms > 0
+    gpu.reset()
+    again, _, _ = gpu.generate(prompt, 40)
+    assert again.tolist() == want  # graph replays are deterministic and the reset clears the position
+    gpu.close()
+
+
+def test_gqa_and_head_dim_variants(ctx):
+    for over in (dict(num_heads=8, num_kv_heads=2, head_dim=32), dict(num_heads=2, num_kv_heads=1, head_dim=128),
+                 dict(num_heads=4, num_kv_heads=4, head_dim=64, hidden_size=512, intermediate_size=768)):
+        c = tiny_config(**over)
+        w = random_weights(c, 30)
+        cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+        tok = 1
+        for pos in range(8):
+            c_next, c_logits = cpu.forward(tok, pos)
+            g_next, g_logits = gpu.forward(tok)
+            assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, (over, pos)
+            assert g_next == c_next
+            tok = c_next
+        gpu.close()
+
+
+def test_error_paths(ctx):
+    from axonml_amd import quant as q
+    from axonml_amd.decode import QuantizedLlama
+
+    with pytest.raises(q.ShapeMismatch):
+        QuantizedLlama(ctx, vocab_size=64, hidden_size=256, intermediate_size=512, num_hidden_layers=1,
+                       num_attention_heads=3, num_key_value_heads=2, head_dim=64, max_position_embeddings=16,
+                       rms_norm_eps=1e-5, rope_theta=1e4)
+    c = tiny_config(num_layers=1)
+    m = load_gpu(ctx, c, random_weights(c, 40))
+    with pytest.raises(q.ShapeMismatch):  # wrong linear shape
+        m.set_linear(0, "q", q.quantize_tensor(np.zeros((64, 256), np.float32), q.QuantType.Q4_K, ctx))
+    with pytest.raises(q.InvalidQuantType):  # fused q,k,v must share a type
+        m.set_linear(0, "k", q.quantize_tensor(np.zeros((128, 256), np.float32), q.QuantType.Q8_0, ctx))
+    with pytest.raises(q.QuantError):
+        m.forward(10 ** 6)
+    fresh = QuantizedLlama(ctx, vocab_size=64, hidden_size=256, intermediate_size=512, num_hidden_layers=1,
+                           num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=16,
+                           rms_norm_eps=1e-5, rope_theta=1e4)
+    with pytest.raises(q.InvalidData):  # weights not set
+        fresh.forward(1)
+    for _ in range(c["max_seq_len"]):
+        m.forward(1, want_logits=False)
+    with pytest.raises(q.Overflow):  # cache full
+        m.forward(1)

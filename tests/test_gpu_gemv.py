@@ -97,6 +97,26 @@ def test_linearity_and_determinism_at_full_size(ctx):
     dw.free()
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0])
+@pytest.mark.parametrize("k", [512, 4096, 32768 + 256])
+def test_activations_with_a_mean_do_not_cancel(ctx, qtype, k):
+    # post-softmax / post-SiLU activations are not zero-mean: offsets of the unsigned codes must be
+    # removed exactly, not by subtracting two large f32 sums.  Checked against the float64 product
+    # at the strict floor for a positive-mean, a tiny and a spiky input.
+    rng = np.random.default_rng(k + qtype)
+    n = 64
+    w = gen_weight(rng, n, k, std=0.06)
+    wq = o.quantize(qtype, w)
+    wd = o.dequantize(qtype, wq, n * k).reshape(n, k)
+    dw = q.DeviceWeight.upload(q.QuantizedTensor([n, k], qtype, wq), ctx)
+    for x in (0.3 + 0.05 * rng.standard_normal((1, k)), 1e-3 * rng.standard_normal((1, k)),
+              rng.standard_normal((1, k)) * np.where(np.arange(k) % 32 < 4, 10.0, 0.01)):
+        x = x.astype(np.float32)
+        got = q.quantized_matmul(x, dw, None, ctx)
+        assert max_rel_err(got, o.matmul_f64(wd, x), STRICT_FLOOR) <= 2e-4
+    dw.free()
+
+
 def test_quantized_linear_keeps_leading_dims(ctx):
     rng = np.random.default_rng(4)
     w = gen_weight(rng, 48, 512)

@@ -1,0 +1,73 @@
+"""Pins the CPU decode oracle (oracle/axq_decode_oracle.c) against closed forms and an independent
+numpy float64 forward.  The reference's own decode tests are shape-only (llama.rs:1123-1211) and its
+code cannot run here, so these are what stands behind the GPU decode parity tests."""
+import numpy as np
+
+import oracle as o
+from tests.decode_common import LIN_ID, NumpyDecoder, load_oracle, random_weights, tiny_config
+from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err
+
+
+def test_matches_independent_float64_forward():
+    c = tiny_config()
+    w = random_weights(c, 1)
+    cpu, ref = load_oracle(c, w), NumpyDecoder(c, w)
+    tok = 5
+    for pos in range(10):
+        nxt, logits = cpu.forward(tok, pos)
+        want = ref.forward(tok, pos)
+        assert max_rel_err(logits, want, DECODE_FLOOR) < DECODE_RTOL / 10, pos
+        assert nxt == int(np.flatnonzero(want == want.max())[-1])
+        tok = nxt
+
+
+def test_zero_linears_leave_embedding_and_give_zero_logits_closed_form():
+    # all layer linears zero: h = embedding; logits = head @ rmsnorm(h): a one-line closed form
+    c = tiny_config(num_layers=1)
+    w = random_weights(c, 2, qtype=o.F32)
+    for name in LIN_ID:
+        w["layers"][0][name] = np.zeros_like(w["layers"][0][name])
+    cpu = load_oracle(c, w)
+    _, logits = cpu.forward(7, 0)
+    e = w["emb"].view(np.float16)[7].astype(np.float64)
+    xn = e / np.sqrt(np.mean(e * e) + c["rms_norm_eps"]) * w["final_norm"]
+    want = w["head"].view(np.float32).reshape(c["vocab_size"], c["hidden_size"]).astype(np.float64) @ xn
+    assert max_rel_err(logits, want) < 1e-4  # f32 accumulation over 256 terms
+    assert np.allclose(cpu.hidden(), e, rtol=0, atol=0)
+
+
+def test_rmsnorm_of_constant_vector_returns_the_weight():
+    # x = const: x / sqrt(x^2 + eps) ~= sign(x); through a zero-layer model with identity-free head
+    c = tiny_config(num_layers=0, vocab_size=256, hidden_size=256)
+    w = random_weights(c, 3, qtype=o.F32)
+    w["emb"] = np.full((256, 256), 3.0, np.float16).view(np.uint16)
+    w["head"] = np.eye(256, dtype=np.float32).view(np.uint8).reshape(-1)
+    cpu = load_oracle(c, w)
+    _, logits = cpu.forward(0, 0)
+    assert np.allclose(logits, w["final_norm"], rtol=1e-5)
+
+
+def test_first_position_attention_returns_v_and_rope_is_identity_at_zero():
+    # pos 0: softmax over one position = 1, RoPE angle 0 -> attention output = f16(v); with o = identity,
+    # other linears crafted so the residual is checkable: h1 = e + f16(W_v rmsnorm(e)) (heads = kv heads)
+    c = tiny_config(num_layers=1, num_heads=4, num_kv_heads=4, head_dim=64, hidden_size=256)
+    w = random_weights(c, 4, qtype=o.F32)
+    L = w["layers"][0]
+    L["o"] = np.eye(256, dtype=np.float32).view(np.uint8).reshape(-1)
+    for n in ("gate", "up", "down"):
+        L[n] = np.zeros_like(L[n])
+    cpu = load_oracle(c, w)
+    cpu.forward(9, 0)
+    e = w["emb"].view(np.float16)[9].astype(np.float64)
+    xn = e / np.sqrt(np.mean(e * e) + c["rms_norm_eps"]) * L["norm0"]
+    v = (L["v"].view(np.float32).reshape(256, 256).astype(np.float64) @ xn).astype(np.float16).astype(np.float64)
+    assert np.allclose(cpu.hidden(), e + v, rtol=1e-5, atol=1e-5)
+
+
+def test_greedy_tie_takes_last_index():
+    c = tiny_config(num_layers=0, vocab_size=256, hidden_size=256)
+    w = random_weights(c, 5, qtype=o.F32)
+    w["head"] = np.zeros((256, 256), np.float32).view(np.uint8).reshape(-1)  # all logits equal
+    cpu = load_oracle(c, w)
+    nxt, _ = cpu.forward(1, 0)
+    assert nxt == 255  # Iterator::max_by keeps the last of equal maxima (llama.rs:1025-1030)

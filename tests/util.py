@@ -11,6 +11,14 @@ import numpy as np
 MATMUL_RTOL = 1e-3
 REL_FLOOR = 1e-2
 STRICT_FLOOR = 1e-3
+# Logits after a whole decoder stack are compared normwise: max|y - ref| / max|ref| <= 1e-3 (DECODE_FLOOR = 1
+# in max_rel_err).  The per-element floor metric is the wrong instrument there, because rounding k and v to
+# f16 for the cache is a discontinuity: two correct f32 evaluations that differ in the last bits upstream
+# round an occasional cache element to neighbouring f16 values (tests/test_gpu_decode.py counts them: a few
+# per thousand, one f16 ulp each), and each such flip moves every logit by ~1e-5 of the logit range --
+# invisible normwise (measured 6e-5), but several 1e-3 of a logit that happens to be near zero.
+DECODE_RTOL = 1e-3
+DECODE_FLOOR = 1.0
 
 
 def max_rel_err(got, want, floor=REL_FLOOR):
