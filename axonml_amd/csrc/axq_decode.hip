@@ -40,6 +40,8 @@ struct axq_model {
     uint16_t *kcache, *vcache;      // f16 [layers, kv_heads, max_pos, head_dim]
     // activations
     float *h, *xn, *qkv, *att, *gu, *act, *logits;
+    float *att_part;                // [kv_heads][max_splits][rep][head_dim + 2] partial attention results
+    int max_splits;
     uint8_t *xq_h, *xq_att, *xq_act;
     // device-side state
     int32_t *pos, *tok, *next, *gen, *prompt, *out;
@@ -60,18 +62,6 @@ __device__ inline float block_sum(float v, float *scratch) {
     __syncthreads();
     float t = 0.f;
     for (int i = 0; i < nw; i++) t += scratch[i];
-    return t;
-}
-
-__device__ inline float block_max(float v, float *scratch) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
-    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = (blockDim.x + 63) >> 6;
-    __syncthreads();
-    if (lane == 0) scratch[wave] = v;
-    __syncthreads();
-    float t = -INFINITY;
-    for (int i = 0; i < nw; i++) t = fmaxf(t, scratch[i]);
     return t;
 }
 
@@ -128,110 +118,167 @@ __global__ void __launch_bounds__(1024) norm_kernel(const uint16_t *emb, const i
     }
 }
 
-// One workgroup per query head: RoPE on q (and on this head's new k), append k,v to the f16 cache
-// (by the first query head of each KV group), causal softmax(q.k / sqrt(d)) over positions 0..pos,
-// weighted sum of v; the head's output goes out as f32 and in split form.
-// Every position but the newest is read from the cache; the newest comes from registers, rounded
-// to f16 exactly as the cache holds it.
-__global__ void __launch_bounds__(256) attn_kernel(const float *qkv, const float *rope_cos, const float *rope_sin,
-                                                   uint16_t *kcache, uint16_t *vcache, const int32_t *pos_p, int n_heads,
-                                                   int n_kv, int d, int max_pos, float *att, uint8_t *xq_att) {
+// Attention for one new token, split over the cached positions ("flash decoding"):
+//
+// attn_partial_kernel, grid (kv_heads, max_splits): workgroup (g, s) covers positions [s*CHUNK, (s+1)*CHUNK)
+// of KV head g for all the query heads that share it (GQA without the repeat_kv copy, llama.rs:450-480).
+// It applies RoPE to those query heads, computes q.k / sqrt(d) against the cached f16 keys with 16-byte
+// loads (d/8 lanes per position), keeps the chunk's running maximum m, exponentials and their sum l, and
+// accumulates sum_p exp(s_p - m) v_p.  The workgroup whose chunk holds the newest position also applies
+// RoPE to the new key, rounds k and v to f16, appends them to the cache and uses them from registers.
+// Workgroups whose chunk starts beyond the newest position leave at once (the grid is sized for the
+// longest context so that the launch can sit in a graph).
+//
+// attn_combine_kernel, grid (heads): merges the partial (m, l, o) triples of a head in a fixed order,
+// normalises, and writes the head's output as f32 and in split form.
+constexpr int ATT_CHUNK = 32;
+constexpr int ATT_MAX_REP = 8; // query heads per KV head
+
+__global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, const float *rope_cos, const float *rope_sin,
+                                                           uint16_t *kcache, uint16_t *vcache, const int32_t *pos_p,
+                                                           int n_heads, int n_kv, int d, int max_pos, int max_splits,
+                                                           float *part) {
     extern __shared__ float sm[];
-    float *q = sm;                // [d]
-    float *knew = q + d;          // [d]  (f16-rounded)
-    float *vnew = knew + d;       // [d]
-    float *scores = vnew + d;     // [max_pos]
-    float *outp = scores + max_pos; // [256 / d][d]
-    __shared__ float scratch[8];
-    const int head = blockIdx.x, kvh = head / (n_heads / n_kv);
+    const int rep = n_heads / n_kv;
+    float *qs = sm;                       // [rep][d]
+    float *knew = qs + rep * d;           // [d] f16-rounded
+    float *vnew = knew + d;               // [d]
+    float *sc = vnew + d;                 // [rep][ATT_CHUNK]
+    float *stat = sc + rep * ATT_CHUNK;   // [rep][2]: m, l
+    const int kvh = blockIdx.x, split = blockIdx.y;
     const int pos = pos_p[0];
+    const int p0 = split * ATT_CHUNK;
+    if (p0 > pos) return;
+    const int p1 = (p0 + ATT_CHUNK < pos + 1) ? p0 + ATT_CHUNK : pos + 1;
+    const int np = p1 - p0;
+    const bool has_new = pos < p1;
     const int half = d >> 1;
     const int q_dim = n_heads * d, kv_dim = n_kv * d;
-    const float *qh = qkv + (size_t)head * d;
-    const float *kh = qkv + q_dim + (size_t)kvh * d;
-    const float *vh = qkv + q_dim + kv_dim + (size_t)kvh * d;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     uint16_t *kc = kcache + (size_t)kvh * max_pos * d;
     uint16_t *vc = vcache + (size_t)kvh * max_pos * d;
-    const bool writer = head % (n_heads / n_kv) == 0;
-    for (int i = threadIdx.x; i < half; i += blockDim.x) {
-        float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
-        float x1 = qh[i], x2 = qh[i + half];
-        q[i] = x1 * c - x2 * s;
-        q[i + half] = x1 * s + x2 * c;
-        float k1 = kh[i], k2 = kh[i + half];
-        __half ka = __float2half_rn(k1 * c - k2 * s), kb = __float2half_rn(k1 * s + k2 * c);
-        __half va = __float2half_rn(vh[i]), vb = __float2half_rn(vh[i + half]);
-        knew[i] = __half2float(ka); knew[i + half] = __half2float(kb);
-        vnew[i] = __half2float(va); vnew[i + half] = __half2float(vb);
-        if (writer) {
-            kc[(size_t)pos * d + i] = __half_as_ushort(ka); kc[(size_t)pos * d + i + half] = __half_as_ushort(kb);
-            vc[(size_t)pos * d + i] = __half_as_ushort(va); vc[(size_t)pos * d + i + half] = __half_as_ushort(vb);
+    const float *cs = rope_cos + (size_t)pos * half, *sn = rope_sin + (size_t)pos * half;
+    for (int i = tid; i < rep * half; i += blockDim.x) {
+        int h = i / half, e = i - h * half;
+        const float *qh = qkv + (size_t)(kvh * rep + h) * d;
+        float c = cs[e], s = sn[e], x1 = qh[e], x2 = qh[e + half];
+        qs[h * d + e] = x1 * c - x2 * s;
+        qs[h * d + e + half] = x1 * s + x2 * c;
+    }
+    if (has_new) {
+        const float *kh = qkv + q_dim + (size_t)kvh * d;
+        const float *vh = qkv + q_dim + kv_dim + (size_t)kvh * d;
+        for (int e = tid; e < half; e += blockDim.x) {
+            float c = cs[e], s = sn[e], k1 = kh[e], k2 = kh[e + half];
+            __half ka = __float2half_rn(k1 * c - k2 * s), kb = __float2half_rn(k1 * s + k2 * c);
+            __half va = __float2half_rn(vh[e]), vb = __float2half_rn(vh[e + half]);
+            knew[e] = __half2float(ka); knew[e + half] = __half2float(kb);
+            vnew[e] = __half2float(va); vnew[e + half] = __half2float(vb);
+            kc[(size_t)pos * d + e] = __half_as_ushort(ka); kc[(size_t)pos * d + e + half] = __half_as_ushort(kb);
+            vc[(size_t)pos * d + e] = __half_as_ushort(va); vc[(size_t)pos * d + e + half] = __half_as_ushort(vb);
         }
     }
     __syncthreads();
+    // scores: d/8 lanes per position, 64/(d/8) positions per wave pass
+    const int lp = d >> 3, ppw = 64 / lp;
+    const int c8 = lane % lp, r = lane / lp;
     const float scale = 1.0f / sqrtf((float)d);
-    // scores: one thread per position
-    float lmax = -INFINITY;
-    for (int jpos = threadIdx.x; jpos <= pos; jpos += blockDim.x) {
-        float s = 0.f;
-        if (jpos == pos) {
-            for (int i = 0; i < d; i++) s = fmaf(q[i], knew[i], s);
-        } else {
-            const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)jpos * d);
-            for (int i8 = 0; i8 < d / 8; i8++) {
-                uint4 raw = kr[i8];
-                const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+    for (int pp = wave * ppw; pp < np; pp += 4 * ppw) {
+        const int pi = pp + r;          // position within the chunk
+        const int p = p0 + pi;
+        float kf[8];
+        if (pi < np && p != pos) {
+            const uint4 raw = *reinterpret_cast<const uint4 *>(kc + (size_t)p * d + c8 * 8);
+            const uint32_t rr[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    s = fmaf(q[8 * i8 + 2 * e], __half2float(__ushort_as_half((unsigned short)(r[e] & 0xFFFF))), s);
-                    s = fmaf(q[8 * i8 + 2 * e + 1], __half2float(__ushort_as_half((unsigned short)(r[e] >> 16))), s);
-                }
+            for (int e = 0; e < 4; e++) {
+                kf[2 * e] = __half2float(__ushort_as_half((unsigned short)(rr[e] & 0xFFFF)));
+                kf[2 * e + 1] = __half2float(__ushort_as_half((unsigned short)(rr[e] >> 16)));
             }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) kf[e] = (pi < np) ? knew[c8 * 8 + e] : 0.f;
         }
-        s *= scale;
-        scores[jpos] = s;
-        lmax = fmaxf(lmax, s);
-    }
-    const float mx = block_max(lmax, scratch);
-    float lsum = 0.f;
-    for (int jpos = threadIdx.x; jpos <= pos; jpos += blockDim.x) {
-        float e = expf(scores[jpos] - mx);
-        scores[jpos] = e;
-        lsum += e;
-    }
-    const float denom = block_sum(lsum, scratch); // also orders the scores[] writes before the reads below
-    // weighted sum of v: thread (part, dim); two parts split the positions
-    const int dim = threadIdx.x % d, part = threadIdx.x / d, nparts = blockDim.x / d;
-    float acc = 0.f;
-    if (part < nparts) {
-        for (int jpos = part; jpos <= pos; jpos += nparts) {
-            float p = scores[jpos] / denom;
-            float vv = jpos == pos ? vnew[dim] : __half2float(__ushort_as_half(vc[(size_t)jpos * d + dim]));
-            acc = fmaf(p, vv, acc);
+        for (int h = 0; h < rep; h++) {
+            const float *qh = qs + h * d + c8 * 8;
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) s = fmaf(qh[e], kf[e], s);
+            for (int m = 1; m < lp; m <<= 1) s += __shfl_xor(s, m);
+            if (c8 == 0 && pi < np) sc[h * ATT_CHUNK + pi] = s * scale;
         }
-        outp[part * d + dim] = acc;
     }
     __syncthreads();
-    // fold the parts, write f32 and the split form (d / 8 tasks, lane quads aligned)
+    // per head: chunk maximum, exponentials, their sum (one wave per head, heads strided over the 4 waves)
+    for (int h = wave; h < rep; h += 4) {
+        float v = lane < np ? sc[h * ATT_CHUNK + lane] : -INFINITY; // ATT_CHUNK <= 64
+        float mx = v;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
+        float e = lane < np ? expf(v - mx) : 0.f;
+        float sum = e;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
+        if (lane < np) sc[h * ATT_CHUNK + lane] = e;
+        if (lane == 0) { stat[2 * h] = mx; stat[2 * h + 1] = sum; }
+    }
+    __syncthreads();
+    // sum_p e_p v_p: thread = (head group, dim)
+    const int dim = tid % d, hg = tid / d, nhg = blockDim.x / d;
+    float acc[ATT_MAX_REP];
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_REP; i++) acc[i] = 0.f;
+    for (int pi = 0; pi < np; pi++) {
+        const int p = p0 + pi;
+        const float vv = (p == pos) ? vnew[dim] : __half2float(__ushort_as_half(vc[(size_t)p * d + dim]));
+#pragma unroll
+        for (int i = 0; i < ATT_MAX_REP; i++) {
+            int h = hg + i * nhg;
+            if (h < rep) acc[i] = fmaf(sc[h * ATT_CHUNK + pi], vv, acc[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_REP; i++) {
+        int h = hg + i * nhg;
+        if (h < rep) {
+            float *o = part + ((size_t)(kvh * max_splits + split) * rep + h) * (d + 2);
+            o[2 + dim] = acc[i];
+            if (dim == 0) { o[0] = stat[2 * h]; o[1] = stat[2 * h + 1]; }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, const int32_t *pos_p, int n_heads, int n_kv,
+                                                           int d, int max_splits, float *att, uint8_t *xq_att) {
+    __shared__ float outs[256];
+    const int head = blockIdx.x, rep = n_heads / n_kv, kvh = head / rep, h = head - kvh * rep;
+    const int nsplit = pos_p[0] / ATT_CHUNK + 1;
+    const int dim = threadIdx.x;
+    if (dim < d) {
+        const float *base = part + ((size_t)(kvh * max_splits) * rep + h) * (d + 2);
+        const size_t stride = (size_t)rep * (d + 2);
+        float mx = -INFINITY;
+        for (int s = 0; s < nsplit; s++) mx = fmaxf(mx, base[s * stride]);
+        float l = 0.f, o = 0.f;
+        for (int s = 0; s < nsplit; s++) {
+            float w = expf(base[s * stride] - mx);
+            l = fmaf(base[s * stride + 1], w, l);
+            o = fmaf(base[s * stride + 2 + dim], w, o);
+        }
+        float v = o / l;
+        outs[dim] = v;
+        att[(size_t)head * d + dim] = v;
+    }
+    __syncthreads();
     const int ntask = d >> 3;
-    const int k_total = q_dim, kpad = (k_total + 15) & ~15;
+    const int kpad = (n_heads * d + 15) & ~15;
     uint4 *grp = reinterpret_cast<uint4 *>(xq_att + (size_t)4 * kpad);
     if ((int)threadIdx.x < ((ntask + 3) & ~3)) {
         const int t = threadIdx.x;
         const bool live = t < ntask;
         float v[8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            float a = 0.f;
-            if (live)
-                for (int p = 0; p < nparts; p++) a += outp[p * d + t * 8 + i];
-            v[i] = a;
-        }
-        if (live) {
-            float4 *o = reinterpret_cast<float4 *>(att + (size_t)head * d + (size_t)t * 8);
-            o[0] = make_float4(v[0], v[1], v[2], v[3]);
-            o[1] = make_float4(v[4], v[5], v[6], v[7]);
-        }
+        for (int i = 0; i < 8; i++) v[i] = live ? outs[t * 8 + i] : 0.f;
         axq_split8(v, head * ntask + t, live, xq_att, grp, kpad);
     }
 }
@@ -349,17 +396,18 @@ int enqueue_step(axq_model *m) {
     hipStream_t st = ctx->stream;
     const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim;
     const size_t kv_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * d;
-    const size_t attn_lds = (size_t)(3 * d + c.max_position_embeddings + 256) * sizeof(float);
+    const int rep = c.num_attention_heads / c.num_key_value_heads;
+    const size_t attn_lds = (size_t)(rep * d + 2 * d + rep * ATT_CHUNK + 2 * rep) * sizeof(float);
     int rc;
     for (int l = 0; l < c.num_hidden_layers; l++) {
         norm_kernel<<<1, 1024, 0, st>>>(l == 0 ? m->emb : nullptr, m->tok, m->h, m->norm_attn + (size_t)l * H, H,
                                         c.rms_norm_eps, m->xn, m->xq_h);
         if ((rc = gemv(m, m->w_qkv[l], m->xn, m->xq_h, nullptr, m->qkv))) return rc;
-        attn_kernel<<<c.num_attention_heads, 256, attn_lds, st>>>(m->qkv, m->rope_cos, m->rope_sin,
-                                                                  m->kcache + (size_t)l * kv_layer,
-                                                                  m->vcache + (size_t)l * kv_layer, m->pos,
-                                                                  c.num_attention_heads, c.num_key_value_heads, d,
-                                                                  c.max_position_embeddings, m->att, m->xq_att);
+        attn_partial_kernel<<<dim3(c.num_key_value_heads, m->max_splits), 256, attn_lds, st>>>(
+            m->qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer, m->vcache + (size_t)l * kv_layer, m->pos,
+            c.num_attention_heads, c.num_key_value_heads, d, c.max_position_embeddings, m->max_splits, m->att_part);
+        attn_combine_kernel<<<c.num_attention_heads, 256, 0, st>>>(m->att_part, m->pos, c.num_attention_heads,
+                                                                   c.num_key_value_heads, d, m->max_splits, m->att, m->xq_att);
         if ((rc = gemv(m, m->w_o[l], m->att, m->xq_att, m->h, m->h))) return rc; // residual through the bias slot
         norm_kernel<<<1, 1024, 0, st>>>(nullptr, m->tok, m->h, m->norm_ffn + (size_t)l * H, H, c.rms_norm_eps, m->xn,
                                         m->xq_h);
@@ -431,9 +479,9 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH,
                         "Shape mismatch: hidden and intermediate sizes must be multiples of 32 and head_dim one of 32, 64, "
                         "128, 256");
-    if ((size_t)(3 * c.head_dim + 256 + c.max_position_embeddings) * 4 > 60 * 1024)
-        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: max_position_embeddings %d does not fit the attention kernel",
-                        c.max_position_embeddings);
+    if (c.num_attention_heads / c.num_key_value_heads > ATT_MAX_REP)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: at most %d query heads per KV head, got %d", ATT_MAX_REP,
+                        c.num_attention_heads / c.num_key_value_heads);
     AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
     axq_model *m = new (std::nothrow) axq_model();
     if (!m) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "out of host memory");
@@ -442,6 +490,7 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     m->q_dim = c.num_attention_heads * c.head_dim;
     m->kv_dim = c.num_key_value_heads * c.head_dim;
     m->qkv_rows = m->q_dim + 2 * m->kv_dim;
+    m->max_splits = (c.max_position_embeddings + ATT_CHUNK - 1) / ATT_CHUNK;
     const int L = c.num_hidden_layers, H = c.hidden_size, I = c.intermediate_size;
     m->w_qkv.assign(L, nullptr); m->w_o.assign(L, nullptr); m->w_gu.assign(L, nullptr); m->w_down.assign(L, nullptr);
     m->set_mask.assign(L, 0);
@@ -455,6 +504,7 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     TRY(dev_alloc(&m->rope_sin, (size_t)c.max_position_embeddings * c.head_dim / 2));
     TRY(dev_alloc(&m->kcache, kv)); TRY(dev_alloc(&m->vcache, kv));
     TRY(dev_alloc(&m->h, H)); TRY(dev_alloc(&m->xn, H)); TRY(dev_alloc(&m->qkv, m->qkv_rows)); TRY(dev_alloc(&m->att, m->q_dim));
+    TRY(dev_alloc(&m->att_part, (size_t)c.num_key_value_heads * m->max_splits * (c.num_attention_heads / c.num_key_value_heads) * (c.head_dim + 2)));
     TRY(dev_alloc(&m->gu, (size_t)2 * I)); TRY(dev_alloc(&m->act, I)); TRY(dev_alloc(&m->logits, c.vocab_size));
     TRY(dev_alloc(&m->xq_h, axq_split_bytes(H))); TRY(dev_alloc(&m->xq_att, axq_split_bytes(m->q_dim)));
     TRY(dev_alloc(&m->xq_act, axq_split_bytes(I)));
@@ -512,7 +562,7 @@ void axq_model_free(axq_model *m) {
     for (auto *w : m->w_down) axq_weight_free(ctx, w);
     axq_weight_free(ctx, m->w_head);
     void *bufs[] = {m->emb, m->norm_attn, m->norm_ffn, m->norm_final, m->rope_cos, m->rope_sin, m->kcache, m->vcache, m->h,
-                    m->xn, m->qkv, m->att, m->gu, m->act, m->logits, m->xq_h, m->xq_att, m->xq_act, m->pos, m->tok,
+                    m->xn, m->qkv, m->att, m->att_part, m->gu, m->act, m->logits, m->xq_h, m->xq_att, m->xq_act, m->pos, m->tok,
                     m->next, m->gen, m->prompt, m->out};
     for (void *p : bufs)
         if (p) (void)hipFree(p);
