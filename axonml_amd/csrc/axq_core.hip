@@ -203,6 +203,7 @@ void axq_destroy(axq_ctx *ctx) {
     (void)hipEventDestroy(ctx->ev_stop);
     (void)hipStreamDestroy(ctx->own_stream);
     (void)hipFree(ctx->xq);
+    if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
     free(ctx);
 }
 

@@ -1,0 +1,42 @@
+"""Prefill-path benchmark helper: quantized GEMM with bf16 activations (BASELINE config 5)."""
+import ctypes as C
+
+import numpy as np
+
+from ._lib import MEM_DEVICE
+from .quant import QuantType, f32_to_bf16_bits
+
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16, published
+
+
+def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(QuantType.Q4_K, QuantType.Q5_1), iters=20):
+    lib = ctx.lib
+    rng = np.random.default_rng(0)
+    out = []
+    for qt in types:
+        for n in ns:
+            f = ctx.malloc(n * k * 4)
+            ctx.check(lib.axq_fill_normal_f32(ctx.handle, f, n * k, 0.0, 0.02, 0.0, 0.0, 77))
+            h = C.c_void_p()
+            ctx.check(lib.axq_weight_quantize(ctx.handle, int(qt), n, k, f, MEM_DEVICE, C.byref(h)))
+            ctx.free(f)
+            for m in ms:
+                x = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+                xd = ctx.to_device(x)
+                yd = ctx.malloc(m * n * 4)
+                for _ in range(3):
+                    ctx.check(lib.axq_gemm_bf16(ctx.handle, h, xd, m, yd, MEM_DEVICE))
+                ctx.synchronize()
+                ctx.timer_start()
+                for _ in range(iters):
+                    ctx.check(lib.axq_gemm_bf16(ctx.handle, h, xd, m, yd, MEM_DEVICE))
+                t = ctx.timer_stop() / iters
+                flops = 2.0 * m * n * k
+                r = {"type": str(qt), "m": m, "n": n, "k": k, "ms": t, "tflops": flops / (t * 1e-3) / 1e12}
+                r["frac_of_mfma_f16_peak"] = r["tflops"] / MFMA_F16_PEAK_TFLOPS
+                out.append(r)
+                log(f"  prefill {r['type']} M={m} N={n}: {t * 1e3:.1f} us, {r['tflops']:.1f} TFLOP/s")
+                ctx.free(xd)
+                ctx.free(yd)
+            lib.axq_weight_free(ctx.handle, h)
+    return out

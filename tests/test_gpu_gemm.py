@@ -1,0 +1,81 @@
+"""GPU parity: the prefill-path quantized GEMM (bf16 activations, f32 accumulate) against the CPU oracle.
+
+Bar: max relative error <= 1e-3 against the reference f32 result (dequantise -> f32 sgemm on the same
+bf16 inputs widened exactly), relative error taken against max(|ref_i|, 1e-2 * max|ref|), and the same
+bound against the float64 product at the 1e-3 floor."""
+import numpy as np
+import pytest
+
+import oracle as o
+from axonml_amd import quant as q
+from tests.util import MATMUL_RTOL, STRICT_FLOOR, gen_weight, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.F16, o.F32]
+
+
+def _check(ctx, qtype, m, n, k, seed, xscale=1.0):
+    rng = np.random.default_rng(seed)
+    w = gen_weight(rng, n, k)
+    xb = q.f32_to_bf16_bits((rng.standard_normal((m, k)) * xscale).astype(np.float32))
+    x = q.bf16_bits_to_f32(xb)
+    wq = o.quantize(qtype, w)
+    want = o.matmul_ref(qtype, wq, x, n, k)
+    got = q.quantized_matmul_bf16(xb, q.QuantizedTensor([n, k], qtype, wq), ctx)
+    assert got.shape == (m, n)
+    err = max_rel_err(got, want)
+    assert err <= MATMUL_RTOL, f"{o.TYPE_NAMES[qtype]} M={m} N={n} K={k}: max rel err {err:.3e}"
+    exact = o.matmul_f64(o.dequantize(qtype, wq, n * k).reshape(n, k), x)
+    assert max_rel_err(got, exact, STRICT_FLOOR) <= MATMUL_RTOL
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("m,n,k", [(1, 128, 256), (7, 64, 256), (128, 128, 512), (130, 200, 1024), (300, 256, 768)])
+def test_gemm_small_shapes(ctx, qtype, m, n, k):
+    _check(ctx, qtype, m, n, k, seed=m + n + k + qtype)
+
+
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_1])
+@pytest.mark.parametrize("m", [128, 512])
+def test_config_prefill_k4096(ctx, qtype, m):
+    _check(ctx, qtype, m, 512, 4096, seed=m)
+
+
+@pytest.mark.parametrize("xscale", [1e-4, 1.0, 3e4])
+def test_row_scaling_keeps_extreme_activations_exact(ctx, xscale):
+    _check(ctx, o.Q4_K, 64, 128, 512, seed=9, xscale=xscale)
+
+
+def test_rows_with_different_magnitudes(ctx):
+    rng = np.random.default_rng(3)
+    m, n, k = 96, 128, 512
+    w = gen_weight(rng, n, k)
+    x = rng.standard_normal((m, k)).astype(np.float32) * (10.0 ** rng.integers(-6, 6, size=(m, 1))).astype(np.float32)
+    xb = q.f32_to_bf16_bits(x)
+    x = q.bf16_bits_to_f32(xb)
+    wq = o.quantize(o.Q4_K, w)
+    want = o.matmul_f64(o.dequantize(o.Q4_K, wq, n * k).reshape(n, k), x)
+    got = q.quantized_matmul_bf16(xb, q.QuantizedTensor([n, k], o.Q4_K, wq), ctx)
+    for r in range(m):  # per row: each row has its own scale
+        assert max_rel_err(got[r], want[r], STRICT_FLOOR) <= MATMUL_RTOL, r
+
+
+def test_gemm_matches_gemv_path(ctx):
+    rng = np.random.default_rng(5)
+    n, k = 256, 1024
+    dw = q.DeviceWeight.quantize(gen_weight(rng, n, k), q.QuantType.Q4_K, ctx)
+    xb = q.f32_to_bf16_bits(rng.standard_normal((4, k)).astype(np.float32))
+    y_gemm = q.quantized_matmul_bf16(xb, dw, ctx)
+    y_gemv = q.quantized_matmul(q.bf16_bits_to_f32(xb), dw, None, ctx)
+    assert max_rel_err(y_gemm, y_gemv) <= 1e-4
+    dw.free()
+
+
+def test_gemm_shape_errors(ctx):
+    w = q.quantize_tensor(np.zeros((4, 256), np.float32), q.QuantType.Q8_0, ctx)
+    with pytest.raises(q.ShapeMismatch):
+        q.quantized_matmul_bf16(np.zeros((2, 128), np.uint16), w, ctx)
+    w32 = q.quantize_tensor(np.zeros((4, 96), np.float32), q.QuantType.Q8_0, ctx)
+    with pytest.raises(q.InvalidBlockSize):  # the GEMM needs k % 64 == 0
+        q.quantized_matmul_bf16(np.zeros((2, 96), np.uint16), w32, ctx)
