@@ -98,6 +98,7 @@ SIGNATURES = {
     "axq_model_read_kv": (_i, [_vp, _i, _i, _vp]),
     "axq_fill_normal_f32": (_i, [_vp, _vp, _sz, C.c_float, C.c_float, C.c_float, C.c_float, C.c_uint64]),
     "axq_bench_gemv_ring": (_i, [_vp, C.POINTER(_vp), _i, _vp, _i, _vp, _i]),
+    "axq_bench_copy": (_i, [_vp, _vp, _vp, _sz, _i]),
 }
 
 _lib = None

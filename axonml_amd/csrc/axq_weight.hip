@@ -89,6 +89,13 @@ int axq_weight_alloc(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, axq_weig
     return AXQ_OK;
 }
 
+// Plain 16-byte-per-lane copy: reads `n16*16` bytes and writes as many.  Used to calibrate the memory
+// counters of a profiler run against a kernel whose traffic is known.
+__global__ void axq_copy16_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
 extern "C" {
 
 int axq_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, void *packed, int mem) {
@@ -287,6 +294,20 @@ int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_we
         if (!w) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_gemv_ring: NULL weight");
         int rc = axq_dev_gemv(ctx, w, x_dev, batch, NULL, y_dev);
         if (rc) return rc;
+    }
+    return AXQ_OK;
+}
+
+int axq_bench_copy(axq_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes, int iters) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_copy: NULL context");
+    if (!dst_dev || !src_dev || bytes == 0 || bytes % 16 || ((uintptr_t)dst_dev | (uintptr_t)src_dev) % 16)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_copy: pointers and size must be multiples of 16");
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    size_t n16 = bytes / 16;
+    int grid = (int)((n16 + 255) / 256 < 16384 ? (n16 + 255) / 256 : 16384);
+    for (int i = 0; i < iters; i++) {
+        axq_copy16_kernel<<<grid, 256, 0, ctx->stream>>>((uint4 *)dst_dev, (const uint4 *)src_dev, n16);
+        AXQ_LAUNCH_CHECK(ctx, "axq_bench_copy");
     }
     return AXQ_OK;
 }

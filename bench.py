@@ -132,6 +132,40 @@ def cpu_baseline(packed, qtype, n, k, x, budget_s=12.0):
             "ms_per_step": med * 1e3}
 
 
+COPY_PROBE_BYTES = 256 << 20
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemv_q4k_14336x4096_hbm_counters.txt")
+
+
+def counter_probe(ctx, steps):
+    """Work for a `rocprofv3 --pmc FETCH_SIZE` (or WRITE_SIZE) run: the copy kernel moves a known number of
+    bytes each way, which gives the factor between the counter and bytes; the GEMV launches follow."""
+    from axonml_amd import quant as q
+
+    src = ctx.malloc(COPY_PROBE_BYTES)
+    dst = ctx.malloc(COPY_PROBE_BYTES)
+    ctx.check(ctx.lib.axq_fill_normal_f32(ctx.handle, src, COPY_PROBE_BYTES // 4, 0.0, 1.0, 0.0, 0.0, 5))
+    ctx.check(ctx.lib.axq_bench_copy(ctx.handle, dst, src, COPY_PROBE_BYTES, 8))
+    ctx.synchronize()
+    ctx.free(src)
+    ctx.free(dst)
+    _, ws, _, x_dev, y_dev = gemv_case(ctx, q.QuantType.Q4_K, N_HEAD, K_HEAD, 1, steps, 20, outlier_p=0.01)
+    free_case(ctx, ws, x_dev, y_dev)
+    log(f"counter probe: 8 copies of {COPY_PROBE_BYTES} B, then {steps + 20} GEMV launches")
+
+
+def measured_traffic():
+    """HBM bytes per GEMV launch from the committed counter summary (a line `traffic_bytes_per_launch: N`),
+    or None when no summary is there."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -139,6 +173,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-extras", action="store_true", help="headline case only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--counter-probe", action="store_true",
+                    help="for profiler counter runs: a few launches of a 256 MiB plain copy kernel, then the "
+                         "headline GEMV ring; no oracle, no CPU leg, no JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path is built or measured)")
@@ -149,6 +186,10 @@ def main():
     info = ctx.device_info()
     log(f"device: {info.name.decode()} {info.arch.decode()} CUs={info.compute_units}")
     T = q.QuantType
+
+    if args.counter_probe:
+        counter_probe(ctx, args.steps)
+        return
 
     # ---- headline: Q4_K GEMV 14336 x 4096, batch 1
     head, ws, x, x_dev, y_dev = gemv_case(ctx, T.Q4_K, N_HEAD, K_HEAD, 1, args.steps, args.warmup, outlier_p=0.01)
@@ -210,7 +251,7 @@ def main():
                    "algorithmic_bytes_per_step": head["algorithmic_bytes"],
                    "inputs": "W~N(0,0.02) with 1% at +-0.5, x~N(0,1), generated and quantised on the device"},
         "roofline": {"bound": "hbm", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": head["gbps"] / HBM_PEAK_GBPS, "traffic": None},
+                     "frac": head["gbps"] / HBM_PEAK_GBPS, "traffic": measured_traffic()},
         "cpu_baseline": cpu,
         "extra": extra,
     }

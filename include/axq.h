@@ -203,6 +203,10 @@ AXQ_API int axq_fill_normal_f32(axq_ctx *ctx, float *dst_dev, size_t n, float me
 AXQ_API int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, const float *x_dev,
                                 int batch, float *y_dev, int iters);
 
+/* Enqueues `iters` launches of a plain copy kernel (reads `bytes`, writes `bytes`; both pointers and the
+ * size multiples of 16).  A kernel of known traffic against which profiler memory counters are scaled. */
+AXQ_API int axq_bench_copy(axq_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes, int iters);
+
 #ifdef __cplusplus
 }
 #endif
