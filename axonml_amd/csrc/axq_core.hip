@@ -190,6 +190,12 @@ int axq_init(int device, axq_ctx **out) {
     // hand over the split form instead.  AXQ_GEMV_PREP=separate forces the two-kernel form (development).
     const char *prep = getenv("AXQ_GEMV_PREP");
     ctx->gemv_prep = (prep && strcmp(prep, "separate") == 0) ? 1 : 0;
+    const char *mnb = getenv("AXQ_GEMV_MAX_NB");
+    ctx->gemv_max_nb = mnb ? atoi(mnb) : 4;
+    if (ctx->gemv_max_nb < 1 || ctx->gemv_max_nb > 8) ctx->gemv_max_nb = 4;
+    const char *wpc = getenv("AXQ_GEMV_WGS_PER_CU");
+    ctx->gemv_wgs_per_cu = wpc ? atoi(wpc) : 1;
+    if (ctx->gemv_wgs_per_cu < 1 || ctx->gemv_wgs_per_cu > 16) ctx->gemv_wgs_per_cu = 1;
 #undef INIT_HIP
     *out = ctx;
     return AXQ_OK;

@@ -82,6 +82,7 @@ struct DQ4K {
     struct Raw { uint4 q0, q1, h; };
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 8; // w = d*sc*(q - 8) + (8*d*sc - dmin*m)
+    static constexpr int BIG_NB = 4; // row steps a lane can hold within 128 registers
     __device__ static int group_k(int c, int g) { return c * 64 + g * 32; }
     __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
         // the code plane interleaves, per 64-pair slice, the first 16 bytes of every pair, then the second 16
@@ -139,6 +140,7 @@ struct DQ4x {
     struct Raw { uint4 q[2]; uint32_t m[2]; };
     static constexpr bool PERM_A = true; // dword w of a block: low nibbles = elements 8w+{0,2,4,6}, high = 8w+{1,3,5,7}
     static constexpr int CENTRE = 8;
+    static constexpr int BIG_NB = 4;
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
     __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
@@ -180,6 +182,7 @@ struct DQ5x {
     struct Raw { uint4 q[2]; uint32_t qh[2]; uint32_t m[2]; };
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 16;
+    static constexpr int BIG_NB = 4;
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
     __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
@@ -225,6 +228,7 @@ struct DQ80 {
     struct Raw { uint4 q[4]; uint32_t m[2]; };
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 0;
+    static constexpr int BIG_NB = 3;
     // 16-byte vector v (0..3) of chunk c: vector index along the row; block = vector / 2
     __device__ static int vec_index(int c, int v) { return ((c >> 4) << 6) + (v >> 1) * 32 + (c & 15) * 2 + (v & 1); }
     __device__ static int group_k(int c, int g) { return vec_index(c, 2 * g) * 16; }
@@ -312,95 +316,119 @@ __device__ inline float sum_within_row(float v) {
 }
 
 // ---------------------------------------------------------------------------
-// The kernel.  NB row steps in flight per wave, PP passes over K per lane.
+// The kernel.  A workgroup is G row groups of S waves; wave `slice` of a group covers k-chunks
+// [16*slice, 16*slice+16) of the row (1024 weights), so S = ceil(K / 1024) waves span K once.  A group
+// owns `steps` consecutive 4-row steps; each wave keeps a ring of NB of them in flight and refills a slot
+// as soon as it has been folded.
+//
+// Waves issue in order, a load that finds the memory pipeline full blocks its wave, and the pipeline is one
+// queue per compute unit.  So the order of the first instructions decides the ramp: every wave requests x
+// (or its split form) first, a barrier keeps all weight requests behind all x requests, and the split of x
+// runs while the first weights are on their way.
 // ---------------------------------------------------------------------------
-template <class T, int NB, int PP, bool PRE>
-__global__ void __launch_bounds__(512) gemv_dp_kernel(DpArgs a) {
+template <class T, int NB, bool PRE>
+__global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(DpArgs a) {
     extern __shared__ uint4 lds_raw[];
-    const int kpad = (a.k + 15) & ~15;
-    // PRE: the limbs come from global memory (written by prep_x_kernel or by the kernel that produced x)
-    const uint8_t *planes = PRE ? a.xq : reinterpret_cast<const uint8_t *>(lds_raw);
-    const uint4 *grp = reinterpret_cast<const uint4 *>(planes + (size_t)4 * kpad);
-    float *red = PRE ? reinterpret_cast<float *>(lds_raw)
-                     : reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(lds_raw) + (size_t)4 * kpad + (size_t)((a.k + 31) >> 5) * 16);
-
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g_idx = wave / a.S, slice = wave - g_idx * a.S;
     const int blk = lane >> 2, j = lane & 3;
+    const int c = (slice << 4) + blk; // this lane's 64-weight chunk of the row
 
-    // chunk index of this lane in pass p
-    int c[PP];
-#pragma unroll
-    for (int p = 0; p < PP; p++) c[p] = ((p * a.S + slice) << 4) + blk;
+    // LDS: the split form of x (limb planes, then group records), then the reduction buffer
+    uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw);
+    const int kpad = (a.k + 15) & ~15;
+    uint4 *wgrp = reinterpret_cast<uint4 *>(wplanes + (size_t)4 * kpad);
+    const int n16 = (int)(axq_split_bytes(a.k) >> 4);
+    float *red = reinterpret_cast<float *>(lds_raw + n16 + 1); // one spare 16-byte slot takes the surplus stores of step 3
     const int rows_per_group = a.steps * 4;
     const int row0 = (blockIdx.x * a.G + g_idx) * rows_per_group;
-    int row_end = row0 + rows_per_group;
-    row_end = row_end < a.n_rows ? row_end : a.n_rows;
     const int last = a.n_rows - 1;
+    const int red_stride = 4 * a.S; // partial sums per output row in the LDS reduction buffer
+    float *red_lane = red + (g_idx * rows_per_group + j) * red_stride + slice * 4 + (lane >> 4);
+    const int nthreads = (int)blockDim.x;
 
-    // Slot of (row, slice, DPP row) in the LDS reduction buffer: 4*S partial sums per output row.
-    const int dpp_row = lane >> 4;
-    const int red_stride = 4 * a.S;
-
-    typename T::Raw buf[NB][PP];
-    XOp xo[PP];
+    // 1. x first.  The compute unit's memory pipeline is one queue for all its waves, so the barrier makes
+    //    sure that no wave's x request stands behind another wave's weight requests.  A thread fetches at
+    //    most two 8-element split tasks of raw x (K <= 16 per thread by construction of the launch), or at
+    //    most five 16-byte pieces of an x that arrives already split.
+    uint4 x0, x1, x2, x3, x4 = {0, 0, 0, 0};
+    const int ntask = a.k >> 3; // K is a multiple of 64 here: whole quads of tasks
     if (PRE) {
-        // 1. this lane's A operands first (L2 hits, needed before anything can be folded) ...
-#pragma unroll
-        for (int p = 0; p < PP; p++) fetch_xop<T>(planes, grp, kpad, a.k, j, c[p], xo[p]);
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.xq);
+        auto piece = [&](int u) { int i = tid + u * nthreads; return src[i < n16 ? i : 0]; };
+        x0 = piece(0); x1 = piece(1); x2 = piece(2); x3 = piece(3); x4 = piece(4);
+    } else {
+        auto half = [&](int u, int h) {
+            int t = tid + u * nthreads;
+            t = t < ntask ? t : (t & 3);
+            return reinterpret_cast<const uint4 *>(a.x + (size_t)t * 8)[h];
+        };
+        x0 = half(0, 0); x1 = half(0, 1); x2 = half(1, 0); x3 = half(1, 1);
     }
-    // 2. ... then the first NB steps' weights: the whole ring is in flight from the start
-#pragma unroll
-    for (int b = 0; b < NB; b++) {
-        int row = row0 + 4 * b + j;
+    __builtin_amdgcn_s_barrier();
+    // 2. the ring: rows past the group's end re-read its first step (cache hits, no HBM traffic)
+    typename T::Raw buf[NB];
+    auto request = [&](int step, int b) {
+        int row = row0 + 4 * (step < a.steps ? step : 0) + j;
         row = row < last ? row : last;
-#pragma unroll
-        for (int p = 0; p < PP; p++) T::load(a, (size_t)row, c[p], buf[b][p]);
-    }
-    if (!PRE) {
-        // x -> limbs in LDS -> this lane's A operands, while the weights are on their way
-        uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw);
-        stage_x(a.x, a.k, wplanes, reinterpret_cast<uint4 *>(wplanes + (size_t)4 * kpad), tid, (int)blockDim.x);
-        __syncthreads();
-#pragma unroll
-        for (int p = 0; p < PP; p++) fetch_xop<T>(planes, grp, kpad, a.k, j, c[p], xo[p]);
-    }
-
-    // 3. fold the steps through the ring.  Everything inside the loops is unconditional (rows past the
-    //    end are clamped and their results dropped) so that the outstanding-load count is the same on
-    //    every path and a step waits for its own three loads only, not for the whole ring.
-    const int rounds = (a.steps + NB - 1) / NB;
-    auto fold = [&](int b, int rs) {
-        float part = 0.f;
-#pragma unroll
-        for (int p = 0; p < PP; p++) part += T::dot(buf[b][p], xo[p], c[p]);
-        float tot = sum_within_row(part);
-        if ((blk & 3) == 3 && rs + j < row_end)
-            red[(rs + j - row0 + g_idx * rows_per_group) * red_stride + slice * 4 + dpp_row] = tot;
+        T::load(a, (size_t)row, c, buf[b]);
     };
-    int r = row0;
-    for (int round = 0; round < rounds - 1; round++, r += 4 * NB) {
+#pragma unroll
+    for (int b = 0; b < NB; b++) request(b, b);
+    // 3. x -> LDS in split form -> this lane's A operands, while the weights are on their way
+    if (PRE) {
+        auto put = [&](int u, const uint4 &v) { int i = tid + u * nthreads; lds_raw[i < n16 ? i : n16] = v; };
+        put(0, x0); put(1, x1); put(2, x2); put(3, x3); put(4, x4);
+    } else {
+        auto split = [&](int u, const uint4 &lo, const uint4 &hi) {
+            const int t = tid + u * nthreads;
+            if (t < ntask) { // whole quads of lanes: K is a multiple of 64
+                const float xv[8] = {__builtin_bit_cast(float, lo.x), __builtin_bit_cast(float, lo.y),
+                                     __builtin_bit_cast(float, lo.z), __builtin_bit_cast(float, lo.w),
+                                     __builtin_bit_cast(float, hi.x), __builtin_bit_cast(float, hi.y),
+                                     __builtin_bit_cast(float, hi.z), __builtin_bit_cast(float, hi.w)};
+                axq_split8(xv, t, true, wplanes, wgrp, kpad);
+            }
+        };
+        split(0, x0, x1);
+        split(1, x2, x3);
+    }
+    __syncthreads();
+    XOp xo;
+    fetch_xop<T>(wplanes, wgrp, kpad, a.k, j, c, xo);
+
+    // 4. fold the steps through the ring
+    const bool writer = (blk & 3) == 3;
+    auto fold = [&](int b, int step) {
+        float tot = sum_within_row(T::dot(buf[b], xo, c));
+        if (writer) red_lane[step * 4 * red_stride] = tot;
+    };
+    const int rounds = (a.steps + NB - 1) / NB;
+    int step = 0;
+    for (int round = 0; round < rounds - 1; round++, step += NB) {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            fold(b, r + 4 * b);
-            int row = r + 4 * (NB + b) + j;
-            row = row < last ? row : last;
-#pragma unroll
-            for (int p = 0; p < PP; p++) T::load(a, (size_t)row, c[p], buf[b][p]);
+            fold(b, step + b);
+            request(step + NB + b, b);
         }
     }
 #pragma unroll
-    for (int b = 0; b < NB; b++) fold(b, r + 4 * b);
+    for (int b = 0; b < NB; b++)
+        if (step + b < a.steps) fold(b, step + b); // the last round may be short: its spare slots hold re-reads
 
-    // 4. partial sums -> y, in a fixed order
+    // partial sums -> y, in a fixed order
     __syncthreads();
     const int wg_rows = a.G * rows_per_group;
     for (int t = tid; t < wg_rows; t += (int)blockDim.x) {
         int row = blockIdx.x * wg_rows + t;
         if (row < a.n_rows) {
-            float tot = red[t * red_stride];
-            for (int s = 1; s < red_stride; s++) tot += red[t * red_stride + s];
+            const float4 *pr = reinterpret_cast<const float4 *>(red + (size_t)t * red_stride);
+            float tot = 0.f;
+            for (int s = 0; s < a.S; s++) { // slice by slice, the four DPP rows of each in order
+                float4 v = pr[s];
+                tot += (v.x + v.y) + (v.z + v.w);
+            }
             a.y[row] = a.bias ? tot + a.bias[row] : tot;
         }
     }
@@ -412,42 +440,61 @@ __global__ void __launch_bounds__(256) prep_x_kernel(const float *x, int k, uint
             (int)(gridDim.x * blockDim.x));
 }
 
+template <class T, int NB, bool PRE>
+void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
+    static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
+    if (lds > 64 * 1024 && !big_lds_allowed) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        big_lds_allowed = true;
+    }
+    gemv_dp_kernel<T, NB, PRE><<<grid, block, lds, ctx->stream>>>(a);
+}
+
+template <class T, bool PRE>
+void launch_nb(axq_ctx *ctx, const DpArgs &a, int nb, unsigned grid, unsigned block, size_t lds) {
+    switch (nb) {
+    case 1: launch_one<T, 1, PRE>(ctx, a, grid, block, lds); break;
+    case 2: launch_one<T, 2, PRE>(ctx, a, grid, block, lds); break;
+    case 3: launch_one<T, 3, PRE>(ctx, a, grid, block, lds); break;
+    case 4: launch_one<T, 4, PRE>(ctx, a, grid, block, lds); break;
+    case 5: launch_one<T, 5, PRE>(ctx, a, grid, block, lds); break;
+    case 6: launch_one<T, 6, PRE>(ctx, a, grid, block, lds); break;
+    case 7: launch_one<T, 7, PRE>(ctx, a, grid, block, lds); break;
+    default: launch_one<T, 8, PRE>(ctx, a, grid, block, lds); break;
+    }
+}
+
 template <class T>
 bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
-    if (w->k % 64 != 0) return false;
+    if (w->k % 64 != 0 || w->k > 16384) return false;
     DpArgs a;
     a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
     a.x = x; a.xq = xq; a.bias = bias; a.y = y;
     a.n_rows = (int)w->n_rows;
     a.k = (int)w->k;
-    int slices = (a.k + 1023) / 1024;
-    a.P = (slices + 7) / 8;
-    if (a.P > 2) return false;
-    a.S = (slices + a.P - 1) / a.P;
-    a.G = 8 / a.S;
-    if (a.G < 1) a.G = 1;
-    int cus = ctx->prop.multiProcessorCount;
-    // 4-row steps per group: spread the rows over `wgs_per_cu` workgroups per compute unit
-    int wgs_per_cu = xq ? 2 : 1; // splitting x inside the kernel is paid per workgroup: use fewer, longer ones
-    int groups = cus * wgs_per_cu * a.G;
-    int steps = (a.n_rows + 4 * groups - 1) / (4 * groups);
-    if (steps < 1) steps = 1;
+    a.S = (a.k + 1023) / 1024;            // waves that span K once (<= 16)
+    a.G = a.S <= 8 ? 8 / a.S : 1;         // row groups per workgroup
+    a.P = 1;
+    const unsigned block = (unsigned)(64 * a.S * a.G);
+    // 4-row steps per group: one workgroup per compute unit unless that makes a group's share of the
+    // reduction buffer too large; the ring depth is what a lane can hold in registers
+    const int rowsteps = (a.n_rows + 3) / 4;
+    const int cus = ctx->prop.multiProcessorCount;
+    int wgs = cus * ctx->gemv_wgs_per_cu;
+    int steps = (rowsteps + wgs * a.G - 1) / (wgs * a.G);
+    if (steps > 64) steps = 64;
     a.steps = steps;
-    int wg_rows = a.G * steps * 4;
-    unsigned grid = (unsigned)((a.n_rows + wg_rows - 1) / wg_rows);
-    unsigned block = (unsigned)(64 * a.S * a.G);
-    int kpad = (a.k + 15) & ~15;
-    size_t lds = (size_t)wg_rows * a.S * 4 * 4;
-    if (!xq) lds += (size_t)4 * kpad + (size_t)((a.k + 31) / 32) * 16;
-    if (lds > 64 * 1024) return false;
-    if (xq) {
-        if (a.P == 1) gemv_dp_kernel<T, 4, 1, true><<<grid, block, lds, ctx->stream>>>(a);
-        else gemv_dp_kernel<T, 2, 2, true><<<grid, block, lds, ctx->stream>>>(a);
-    } else {
-        if (a.P == 1) gemv_dp_kernel<T, 4, 1, false><<<grid, block, lds, ctx->stream>>>(a);
-        else gemv_dp_kernel<T, 2, 2, false><<<grid, block, lds, ctx->stream>>>(a);
-    }
+    int nb = block > 512 ? T::BIG_NB : 8;
+    if (nb > ctx->gemv_max_nb) nb = ctx->gemv_max_nb;
+    if (nb > steps) nb = steps;
+    const unsigned grid = (unsigned)((rowsteps + steps * a.G - 1) / (steps * a.G));
+    size_t lds = (size_t)a.G * steps * 4 * a.S * 4 * sizeof(float);
+    lds += axq_split_bytes(a.k) + 16;
+    if (lds > 160 * 1024) return false;
+    if (xq) launch_nb<T, true>(ctx, a, nb, grid, block, lds);
+    else launch_nb<T, false>(ctx, a, nb, grid, block, lds);
     return true;
 }
 

@@ -19,6 +19,8 @@ struct axq_ctx {
     float fp8_unit_inv; // 1 / value(fp8 byte 0x01) as converted by v_cvt_pk_f32_fp8
     uint8_t *xq;        // device scratch: the split form of one activation vector (AXQ_XQ_MAX_K elements)
     int gemv_prep;      // 0: split x inside the GEMV kernel, 1: in a kernel of its own
+    int gemv_max_nb;    // most 4-row steps a GEMV lane holds in flight (1..8)
+    int gemv_wgs_per_cu; // GEMV workgroups per compute unit that the rows are spread over
     void *gemm_scratch; // device scratch of the prefill GEMM (scaled f16 activations + row scales), grown on demand
     size_t gemm_scratch_bytes;
     char err[512];

@@ -15,9 +15,19 @@ __host__ __device__ static inline size_t axq_split_bytes(int64_t k) {
     return (size_t)4 * (size_t)((k + 15) & ~15) + (size_t)((k + 31) / 32) * 16;
 }
 
+// lane ^ 1 and lane ^ 2 within a quad, as one DPP move each
+__device__ inline float axq_quad_xor1(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
+}
+__device__ inline float axq_quad_xor2(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
+}
+__device__ inline int axq_quad_xor1(int v) { return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, true); }
+__device__ inline int axq_quad_xor2(int v) { return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, true); }
+
 // One task = 8 consecutive elements v[0..7] = x[8*task .. 8*task+7].  The four lanes of an aligned
 // lane quad must call this together with four consecutive tasks (task % 4 == lane % 4): they share a
-// 32-element group and exchange its maximum and sum through lane shuffles.  `live` = false lanes take
+// 32-element group and exchange its maximum and sum through DPP quad moves.  `live` = false lanes take
 // part in the shuffles (with zeros) and store nothing.
 __device__ inline void axq_split8(const float (&v)[8], int task, bool live, uint8_t *planes, uint4 *grp, int kpad) {
     float amax = 0.f, sum = 0.f;
@@ -26,10 +36,10 @@ __device__ inline void axq_split8(const float (&v)[8], int task, bool live, uint
         amax = fmaxf(amax, fabsf(v[i]));
         sum += v[i];
     }
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
+    amax = fmaxf(amax, axq_quad_xor1(amax));
+    amax = fmaxf(amax, axq_quad_xor2(amax));
+    sum += axq_quad_xor1(sum);
+    sum += axq_quad_xor2(sum);
     // amax in [2^e, 2^(e+1)): scale so that |x| * f < 2^27, f = 2^(26-e); limb sums times 2^(e-26) give back x
     uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFF;
     const bool bad = eb == 0xFF;
@@ -38,33 +48,32 @@ __device__ inline void axq_split8(const float (&v)[8], int task, bool live, uint
     float f = __builtin_bit_cast(float, (280u - eb) << 23);
     float sg = __builtin_bit_cast(float, (eb - 26u) << 23);
     if (bad) sg = __builtin_nanf("");
-    uint32_t l[4][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
-    int ls[4] = {0, 0, 0, 0};
+    // t = rint(x f) = sum_i l_i 128^i with balanced digits; adding 64 (1 + 128 + 128^2 + 128^3) makes every
+    // digit non-negative, d_i = l_i + 64 in 0..127 (the top one up to 128), so that plain bit fields extract
+    // them; bytes go back to l_i = d_i - 64 four at a time: (d + 64) ^ 0x80 is d - 64 modulo 256.
+    uint32_t pk[4][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}}; // [plane][dword]: plane 0 = most significant limb
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        int tq = bad ? 0 : (int)rintf(v[i] * f);
-        int l3 = ((tq + 64) & 127) - 64;
-        tq = (tq - l3) >> 7;
-        int l2 = ((tq + 64) & 127) - 64;
-        tq = (tq - l2) >> 7;
-        int l1 = ((tq + 64) & 127) - 64;
-        int l0 = (tq - l1) >> 7;
-        int sh = 8 * (i & 3);
-        l[0][i >> 2] |= (uint32_t)(l0 & 0xFF) << sh;
-        l[1][i >> 2] |= (uint32_t)(l1 & 0xFF) << sh;
-        l[2][i >> 2] |= (uint32_t)(l2 & 0xFF) << sh;
-        l[3][i >> 2] |= (uint32_t)(l3 & 0xFF) << sh;
-        ls[0] += l0; ls[1] += l1; ls[2] += l2; ls[3] += l3;
+        const uint32_t u = (uint32_t)((bad ? 0 : (int)rintf(v[i] * f)) + 135274560);
+        const int sh = 8 * (i & 3);
+        pk[3][i >> 2] |= (u & 127u) << sh;
+        pk[2][i >> 2] |= ((u >> 7) & 127u) << sh;
+        pk[1][i >> 2] |= ((u >> 14) & 127u) << sh;
+        pk[0][i >> 2] |= (u >> 21) << sh;
     }
+    int ls[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        ls[i] += __shfl_xor(ls[i], 1);
-        ls[i] += __shfl_xor(ls[i], 2);
+        ls[i] = (int)__builtin_amdgcn_sad_u8(pk[i][0], 0u, __builtin_amdgcn_sad_u8(pk[i][1], 0u, 0u)) - 512;
+        ls[i] += axq_quad_xor1(ls[i]);
+        ls[i] += axq_quad_xor2(ls[i]);
+        pk[i][0] = (pk[i][0] + 0x40404040u) ^ 0x80808080u;
+        pk[i][1] = (pk[i][1] + 0x40404040u) ^ 0x80808080u;
     }
     if (live) {
 #pragma unroll
         for (int i = 0; i < 4; i++)
-            *reinterpret_cast<uint2 *>(planes + (size_t)i * kpad + (size_t)task * 8) = make_uint2(l[i][0], l[i][1]);
+            *reinterpret_cast<uint2 *>(planes + (size_t)i * kpad + (size_t)task * 8) = make_uint2(pk[i][0], pk[i][1]);
         if ((task & 3) == 0)
             grp[task >> 2] = make_uint4(__builtin_bit_cast(uint32_t, sg), __builtin_bit_cast(uint32_t, sum),
                                         (uint32_t)(ls[0] & 0xFFFF) | ((uint32_t)ls[1] << 16),
