@@ -72,6 +72,15 @@ struct XOp {
                    // MFMAs sum (n - centre) * limb exactly and no large terms cancel in f32 afterwards
 };
 
+// Addressing.  A workgroup's rows lie within a few megabytes, so a lane addresses its bytes as
+// (uniform 64-bit plane base of the workgroup's first row) + (32-bit offset): one integer add per load.
+struct Bases { const uint8_t *codes, *meta, *qh; };  // planes at the workgroup's first row
+struct RowOff { uint32_t c, m, h; };                 // (row - first row) * pitch, per plane
+struct LaneOff { uint32_t c[2], m[2], h[2]; };       // the lane's byte offsets inside a row, per plane
+__device__ inline uint4 ld16(const uint8_t *base, uint32_t off) { return *reinterpret_cast<const uint4 *>(base + off); }
+__device__ inline uint32_t ld4(const uint8_t *base, uint32_t off) { return *reinterpret_cast<const uint32_t *>(base + off); }
+__device__ inline uint32_t ld2(const uint8_t *base, uint32_t off) { return *reinterpret_cast<const uint16_t *>(base + off); }
+
 // ---------------------------------------------------------------------------
 // Per-type traits.  A lane covers 64 weights of one row per pass = two
 // 32-element groups.  group_k() gives the K offset of group g for chunk index
@@ -84,31 +93,40 @@ struct DQ4K {
     static constexpr int CENTRE = 8; // w = d*sc*(q - 8) + (8*d*sc - dmin*m)
     static constexpr int BIG_NB = 4; // row steps a lane can hold within 128 registers
     __device__ static int group_k(int c, int g) { return c * 64 + g * 32; }
-    __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
+    __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
         // the code plane interleaves, per 64-pair slice, the first 16 bytes of every pair, then the second 16
         const int cpr = a.k >> 6;
         c = c < cpr ? c : cpr - 1; // lanes past the end of the row re-read its last chunk against x = 0
         int slice = c >> 6, pr = c & 63;
         int P = cpr - (slice << 6);
         P = P < 64 ? P : 64;
-        const uint8_t *base = a.codes + row * a.codes_pitch + (size_t)slice * 2048 + (size_t)pr * 16;
-        r.q0 = *reinterpret_cast<const uint4 *>(base);
-        r.q1 = *reinterpret_cast<const uint4 *>(base + (size_t)P * 16);
-        r.h = *reinterpret_cast<const uint4 *>(a.meta + row * a.meta_pitch + (size_t)(c >> 2) * 16);
+        o.c[0] = (uint32_t)(slice * 2048 + pr * 16);
+        o.c[1] = o.c[0] + (uint32_t)P * 16;
+        o.m[0] = (uint32_t)(c >> 2) * 16;
+    }
+    __device__ static void load(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+        r.q0 = ld16(b.codes, ro.c + o.c[0]);
+        r.q1 = ld16(b.codes, ro.c + o.c[1]);
+        r.h = ld16(b.meta, ro.m + o.m[0]);
     }
     __device__ static float dot(const Raw &r, const XOp &x, int c) {
         const uint32_t q0[4] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w};
         const uint32_t q1[4] = {r.q1.x, r.q1.y, r.q1.z, r.q1.w};
         int4v lo = x.init[0], hi = x.init[1];
+        // all sixteen B operands first, then the products: the matrix pipe must not read a register the
+        // vector ALU has just written
+        uint32_t ml[8], mh[8];
 #pragma unroll
-        for (int w = 0; w < 4; w++) { // bytes 4w..4w+3 of the first half: elements 4w.. of both sub-blocks
-            lo = mfma(x.a[w], q0[w] & 0x0F0F0F0Fu, lo);
-            hi = mfma(x.a[8 + w], (q0[w] >> 4) & 0x0F0F0F0Fu, hi);
+        for (int w = 0; w < 4; w++) {
+            ml[w] = q0[w] & 0x0F0F0F0Fu;            // first half: elements 4w.. of the low-nibble sub-block
+            mh[w] = (q0[w] >> 4) & 0x0F0F0F0Fu;     //             ... and of the high-nibble sub-block
+            ml[4 + w] = q1[w] & 0x0F0F0F0Fu;        // second half: elements 16+4w..
+            mh[4 + w] = (q1[w] >> 4) & 0x0F0F0F0Fu;
         }
 #pragma unroll
-        for (int w = 0; w < 4; w++) { // second half: elements 16+4w..
-            lo = mfma(x.a[4 + w], q1[w] & 0x0F0F0F0Fu, lo);
-            hi = mfma(x.a[12 + w], (q1[w] >> 4) & 0x0F0F0F0Fu, hi);
+        for (int w = 0; w < 8; w++) {
+            lo = mfma(x.a[w], ml[w], lo);
+            hi = mfma(x.a[8 + w], mh[w], hi);
         }
         // 6-bit scale/min of sub-blocks 2p, 2p+1 (ggml get_scale_min_k4 order); p is fixed per lane
         int p = c & 3;
@@ -143,17 +161,21 @@ struct DQ4x {
     static constexpr int BIG_NB = 4;
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
-    __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
-        const uint8_t *codes = a.codes + row * a.codes_pitch;
-        const uint8_t *meta = a.meta + row * a.meta_pitch;
+    __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
         const int nblk = a.k >> 5;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             int b = blk_index(c, g);
             b = b < nblk ? b : nblk - 1;
-            r.q[g] = *reinterpret_cast<const uint4 *>(codes + (size_t)b * 16);
-            if (WITH_MIN) r.m[g] = *reinterpret_cast<const uint32_t *>(meta + (size_t)b * 4);
-            else r.m[g] = *reinterpret_cast<const uint16_t *>(meta + (size_t)b * 2);
+            o.c[g] = (uint32_t)b * 16;
+            o.m[g] = (uint32_t)b * (WITH_MIN ? 4 : 2);
+        }
+    }
+    __device__ static void load(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            r.q[g] = ld16(b.codes, ro.c + o.c[g]);
+            r.m[g] = WITH_MIN ? ld4(b.meta, ro.m + o.m[g]) : ld2(b.meta, ro.m + o.m[g]);
         }
     }
     __device__ static float dot(const Raw &r, const XOp &x, int) {
@@ -185,19 +207,23 @@ struct DQ5x {
     static constexpr int BIG_NB = 4;
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
-    __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
-        const uint8_t *codes = a.codes + row * a.codes_pitch;
-        const uint8_t *meta = a.meta + row * a.meta_pitch;
-        const uint8_t *qh = a.qh + row * a.qh_pitch;
+    __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
         const int nblk = a.k >> 5;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             int b = blk_index(c, g);
             b = b < nblk ? b : nblk - 1;
-            r.q[g] = *reinterpret_cast<const uint4 *>(codes + (size_t)b * 16);
-            r.qh[g] = *reinterpret_cast<const uint32_t *>(qh + (size_t)b * 4);
-            if (WITH_MIN) r.m[g] = *reinterpret_cast<const uint32_t *>(meta + (size_t)b * 4);
-            else r.m[g] = *reinterpret_cast<const uint16_t *>(meta + (size_t)b * 2);
+            o.c[g] = (uint32_t)b * 16;
+            o.h[g] = (uint32_t)b * 4;
+            o.m[g] = (uint32_t)b * (WITH_MIN ? 4 : 2);
+        }
+    }
+    __device__ static void load(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            r.q[g] = ld16(b.codes, ro.c + o.c[g]);
+            r.qh[g] = ld4(b.qh, ro.h + o.h[g]);
+            r.m[g] = WITH_MIN ? ld4(b.meta, ro.m + o.m[g]) : ld2(b.meta, ro.m + o.m[g]);
         }
     }
     __device__ static float dot(const Raw &r, const XOp &x, int) {
@@ -232,17 +258,22 @@ struct DQ80 {
     // 16-byte vector v (0..3) of chunk c: vector index along the row; block = vector / 2
     __device__ static int vec_index(int c, int v) { return ((c >> 4) << 6) + (v >> 1) * 32 + (c & 15) * 2 + (v & 1); }
     __device__ static int group_k(int c, int g) { return vec_index(c, 2 * g) * 16; }
-    __device__ static void load(const DpArgs &a, size_t row, int c, Raw &r) {
-        const uint8_t *codes = a.codes + row * a.codes_pitch;
-        const uint8_t *meta = a.meta + row * a.meta_pitch;
+    __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
         const int nvec = a.k >> 4;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             int v0 = vec_index(c, 2 * g);
             v0 = v0 < nvec ? v0 : nvec - 2;
-            r.q[2 * g] = *reinterpret_cast<const uint4 *>(codes + (size_t)v0 * 16);
-            r.q[2 * g + 1] = *reinterpret_cast<const uint4 *>(codes + (size_t)v0 * 16 + 16);
-            r.m[g] = *reinterpret_cast<const uint16_t *>(meta + (size_t)(v0 >> 1) * 2);
+            o.c[g] = (uint32_t)v0 * 16;
+            o.m[g] = (uint32_t)(v0 >> 1) * 2;
+        }
+    }
+    __device__ static void load(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            r.q[2 * g] = ld16(b.codes, ro.c + o.c[g]);
+            r.q[2 * g + 1] = ld16(b.codes, ro.c + o.c[g] + 16);
+            r.m[g] = ld2(b.meta, ro.m + o.m[g]);
         }
     }
     __device__ static float dot(const Raw &r, const XOp &x, int) {
@@ -342,7 +373,6 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     const int n16 = (int)(axq_split_bytes(a.k) >> 4);
     float *red = reinterpret_cast<float *>(lds_raw + n16 + 1); // one spare 16-byte slot takes the surplus stores of step 3
     const int rows_per_group = a.steps * 4;
-    const int row0 = (blockIdx.x * a.G + g_idx) * rows_per_group;
     const int last = a.n_rows - 1;
     const int red_stride = 4 * a.S; // partial sums per output row in the LDS reduction buffer
     float *red_lane = red + (g_idx * rows_per_group + j) * red_stride + slice * 4 + (lane >> 4);
@@ -369,13 +399,23 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     __builtin_amdgcn_s_barrier();
     // 2. the ring: rows past the group's end re-read its first step (cache hits, no HBM traffic)
     typename T::Raw buf[NB];
+    LaneOff lo;
+    T::lane_offsets(a, c, lo);
+    const int wg_row0 = blockIdx.x * a.G * rows_per_group;
+    const Bases bases = {a.codes + (size_t)wg_row0 * a.codes_pitch, a.meta + (size_t)wg_row0 * a.meta_pitch,
+                         a.qh + (size_t)wg_row0 * a.qh_pitch};
+    const uint32_t cp = (uint32_t)a.codes_pitch, mp = (uint32_t)a.meta_pitch, qp = (uint32_t)a.qh_pitch;
+    const int rl0 = g_idx * rows_per_group + j, rl_last = last - wg_row0; // rows relative to the workgroup's first
     auto request = [&](int step, int b) {
-        int row = row0 + 4 * (step < a.steps ? step : 0) + j;
-        row = row < last ? row : last;
-        T::load(a, (size_t)row, c, buf[b]);
+        int rl = rl0 + 4 * (step < a.steps ? step : 0);
+        rl = rl < rl_last ? rl : rl_last;
+        const RowOff ro = {(uint32_t)rl * cp, (uint32_t)rl * mp, (uint32_t)rl * qp};
+        T::load(bases, ro, lo, buf[b]);
     };
+    constexpr int NB0 = NB < 2 ? NB : 2; // steps requested before x is staged: enough to start the stream,
+                                         // few enough that no wave is still blocked issuing them at the barrier
 #pragma unroll
-    for (int b = 0; b < NB; b++) request(b, b);
+    for (int b = 0; b < NB0; b++) request(b, b);
     // 3. x -> LDS in split form -> this lane's A operands, while the weights are on their way
     if (PRE) {
         auto put = [&](int u, const uint4 &v) { int i = tid + u * nthreads; lds_raw[i < n16 ? i : n16] = v; };
@@ -397,12 +437,15 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     __syncthreads();
     XOp xo;
     fetch_xop<T>(wplanes, wgrp, kpad, a.k, j, c, xo);
+#pragma unroll
+    for (int b = NB0; b < NB; b++) request(b, b);
 
     // 4. fold the steps through the ring
     const bool writer = (blk & 3) == 3;
+    const int red_step = 4 * red_stride;
     auto fold = [&](int b, int step) {
         float tot = sum_within_row(T::dot(buf[b], xo, c));
-        if (writer) red_lane[step * 4 * red_stride] = tot;
+        if (writer) red_lane[step * red_step] = tot;
     };
     const int rounds = (a.steps + NB - 1) / NB;
     int step = 0;
