@@ -42,7 +42,6 @@ struct axq_model {
     float *h, *xn, *qkv, *att, *gu, *act, *logits;
     float *att_part;                // [kv_heads][max_splits][rep][head_dim + 2] partial attention results
     int max_splits;
-    uint8_t *xq_h, *xq_att, *xq_act;
     // device-side state
     int32_t *pos, *tok, *next, *gen, *prompt, *out;
     int prompt_cap, out_cap;
@@ -65,56 +64,45 @@ __device__ inline float block_sum(float v, float *scratch) {
     return t;
 }
 
-// h = embedding[tok] (optional), then xn = rmsnorm(h) * w, written as f32 and in split form.
-// One workgroup; each thread owns 8-element tasks so that the split can be made from registers.
-__global__ void __launch_bounds__(1024) norm_kernel(const uint16_t *emb, const int32_t *tok, float *h, const float *w,
-                                                    int hidden, float eps, float *xn, uint8_t *xq) {
+// h = embedding[tok] widened to f32 (Embedding::lookup, nn/src/layers/embedding.rs:103-146).
+__global__ void __launch_bounds__(256) embed_kernel(const uint16_t *emb, const int32_t *tok, float *h, int hidden) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (hidden >> 3)) return;
+    const uint4 raw = *reinterpret_cast<const uint4 *>(emb + (size_t)tok[0] * hidden + (size_t)t * 8);
+    const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        v[2 * i] = __half2float(__ushort_as_half((unsigned short)(r[i] & 0xFFFF)));
+        v[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(r[i] >> 16)));
+    }
+    float4 *o = reinterpret_cast<float4 *>(h + (size_t)t * 8);
+    o[0] = make_float4(v[0], v[1], v[2], v[3]);
+    o[1] = make_float4(v[4], v[5], v[6], v[7]);
+}
+
+// xn = rmsnorm(h) * w (RMSNorm::forward, llm/src/llama.rs:158-187).  One workgroup.  Only used in front of
+// linears that the matrix-pipe GEMV does not cover; otherwise the GEMV normalises its input itself.
+__global__ void __launch_bounds__(1024) norm_kernel(const float *h, const float *w, int hidden, float eps, float *xn) {
     __shared__ float scratch[16];
     const int ntask = hidden >> 3;
-    const int kpad = (hidden + 15) & ~15;
-    uint4 *grp = reinterpret_cast<uint4 *>(xq + (size_t)4 * kpad);
     float ss = 0.f;
     for (int t = threadIdx.x; t < ntask; t += blockDim.x) {
-        float v[8];
-        if (emb) {
-            const uint4 raw = *reinterpret_cast<const uint4 *>(emb + (size_t)tok[0] * hidden + (size_t)t * 8);
-            const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                v[2 * i] = __half2float(__ushort_as_half((unsigned short)(r[i] & 0xFFFF)));
-                v[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(r[i] >> 16)));
-            }
-            float4 *o = reinterpret_cast<float4 *>(h + (size_t)t * 8);
-            o[0] = make_float4(v[0], v[1], v[2], v[3]);
-            o[1] = make_float4(v[4], v[5], v[6], v[7]);
-        } else {
-            const float4 *p = reinterpret_cast<const float4 *>(h + (size_t)t * 8);
-            float4 a = p[0], b = p[1];
-            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-        }
+        const float4 *p = reinterpret_cast<const float4 *>(h + (size_t)t * 8);
+        float4 a = p[0], b = p[1];
+        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
         for (int i = 0; i < 8; i++) ss = fmaf(v[i], v[i], ss);
     }
     ss = block_sum(ss, scratch);
-    const float rms = sqrtf(ss / (float)hidden + eps);
-    const int ntask_pad = (ntask + 3) & ~3;
-    for (int t = threadIdx.x; t < ntask_pad; t += blockDim.x) {
-        float v[8];
-        const bool live = t < ntask;
-        if (live) {
-            const float4 *p = reinterpret_cast<const float4 *>(h + (size_t)t * 8);
-            const float4 *pw = reinterpret_cast<const float4 *>(w + (size_t)t * 8);
-            float4 a = p[0], b = p[1], wa = pw[0], wb = pw[1];
-            v[0] = (a.x / rms) * wa.x; v[1] = (a.y / rms) * wa.y; v[2] = (a.z / rms) * wa.z; v[3] = (a.w / rms) * wa.w;
-            v[4] = (b.x / rms) * wb.x; v[5] = (b.y / rms) * wb.y; v[6] = (b.z / rms) * wb.z; v[7] = (b.w / rms) * wb.w;
-            float4 *o = reinterpret_cast<float4 *>(xn + (size_t)t * 8);
-            o[0] = make_float4(v[0], v[1], v[2], v[3]);
-            o[1] = make_float4(v[4], v[5], v[6], v[7]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = 0.f;
-        }
-        axq_split8(v, t, live, xq, grp, kpad);
+    const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+    for (int t = threadIdx.x; t < ntask; t += blockDim.x) {
+        const float4 *p = reinterpret_cast<const float4 *>(h + (size_t)t * 8);
+        const float4 *pw = reinterpret_cast<const float4 *>(w + (size_t)t * 8);
+        float4 a = p[0], b = p[1], wa = pw[0], wb = pw[1];
+        float4 *o = reinterpret_cast<float4 *>(xn + (size_t)t * 8);
+        o[0] = make_float4((a.x * inv) * wa.x, (a.y * inv) * wa.y, (a.z * inv) * wa.z, (a.w * inv) * wa.w);
+        o[1] = make_float4((b.x * inv) * wb.x, (b.y * inv) * wb.y, (b.z * inv) * wb.z, (b.w * inv) * wb.w);
     }
 }
 
@@ -132,7 +120,17 @@ __global__ void __launch_bounds__(1024) norm_kernel(const uint16_t *emb, const i
 // attn_combine_kernel, grid (heads): merges the partial (m, l, o) triples of a head in a fixed order,
 // normalises, and writes the head's output as f32 and in split form.
 constexpr int ATT_CHUNK = 32;
-constexpr int ATT_MAX_REP = 8; // query heads per KV head
+constexpr int ATT_MAX_REP = 8;  // query heads per KV head
+constexpr int ATT_MAX_PASS = 4; // 16-byte pieces of K (and of V) a thread fetches: 32 positions * d / 8 / 256 threads
+
+__device__ inline void halves_to_floats(const uint4 &raw, float (&f)[8]) {
+    const uint32_t rr[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        f[2 * e] = __half2float(__ushort_as_half((unsigned short)(rr[e] & 0xFFFF)));
+        f[2 * e + 1] = __half2float(__ushort_as_half((unsigned short)(rr[e] >> 16)));
+    }
+}
 
 __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, const float *rope_cos, const float *rope_sin,
                                                            uint16_t *kcache, uint16_t *vcache, const int32_t *pos_p,
@@ -145,6 +143,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
     float *vnew = knew + d;               // [d]
     float *sc = vnew + d;                 // [rep][ATT_CHUNK]
     float *stat = sc + rep * ATT_CHUNK;   // [rep][2]: m, l
+    float *vs = stat + 2 * rep;           // [ATT_CHUNK][d]: the chunk's values
     const int kvh = blockIdx.x, split = blockIdx.y;
     const int pos = pos_p[0];
     const int p0 = split * ATT_CHUNK;
@@ -157,6 +156,22 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     uint16_t *kc = kcache + (size_t)kvh * max_pos * d;
     uint16_t *vc = vcache + (size_t)kvh * max_pos * d;
+
+    // Every cached byte this workgroup needs is requested before anything else: d/8 lanes per position,
+    // 64/(d/8) positions per wave pass, at most ATT_MAX_PASS passes.  Positions outside the chunk and the
+    // newest position (still in registers) re-read the chunk's first row and are not used.
+    const int lp = d >> 3, ppw = 64 / lp;
+    const int c8 = lane % lp, r = lane / lp;
+    uint4 kraw[ATT_MAX_PASS], vraw[ATT_MAX_PASS];
+#pragma unroll
+    for (int it = 0; it < ATT_MAX_PASS; it++) {
+        const int pi = (it * 4 + wave) * ppw + r;
+        const int p = (pi < np && p0 + pi != pos) ? p0 + pi : p0;
+        const bool any = it * 4 * ppw < ATT_CHUNK; // uniform: this pass exists for this head size
+        kraw[it] = any ? *reinterpret_cast<const uint4 *>(kc + (size_t)p * d + c8 * 8) : make_uint4(0, 0, 0, 0);
+        vraw[it] = any ? *reinterpret_cast<const uint4 *>(vc + (size_t)p * d + c8 * 8) : make_uint4(0, 0, 0, 0);
+    }
+
     const float *cs = rope_cos + (size_t)pos * half, *sn = rope_sin + (size_t)pos * half;
     for (int i = tid; i < rep * half; i += blockDim.x) {
         int h = i / half, e = i - h * half;
@@ -179,33 +194,34 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
         }
     }
     __syncthreads();
-    // scores: d/8 lanes per position, 64/(d/8) positions per wave pass
-    const int lp = d >> 3, ppw = 64 / lp;
-    const int c8 = lane % lp, r = lane / lp;
+    // scores, and the chunk's values into LDS as f32
     const float scale = 1.0f / sqrtf((float)d);
-    for (int pp = wave * ppw; pp < np; pp += 4 * ppw) {
-        const int pi = pp + r;          // position within the chunk
-        const int p = p0 + pi;
-        float kf[8];
-        if (pi < np && p != pos) {
-            const uint4 raw = *reinterpret_cast<const uint4 *>(kc + (size_t)p * d + c8 * 8);
-            const uint32_t rr[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                kf[2 * e] = __half2float(__ushort_as_half((unsigned short)(rr[e] & 0xFFFF)));
-                kf[2 * e + 1] = __half2float(__ushort_as_half((unsigned short)(rr[e] >> 16)));
+    for (int it = 0; it < ATT_MAX_PASS; it++) {
+        const int pi = (it * 4 + wave) * ppw + r; // position within the chunk
+        if (it * 4 * ppw < ATT_CHUNK && pi < ATT_CHUNK) {
+            float kf[8], vf[8];
+            if (pi < np && p0 + pi != pos) {
+                halves_to_floats(kraw[it], kf);
+                halves_to_floats(vraw[it], vf);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    kf[e] = (pi < np) ? knew[c8 * 8 + e] : 0.f;
+                    vf[e] = (pi < np) ? vnew[c8 * 8 + e] : 0.f;
+                }
             }
-        } else {
+            float4 *dst = reinterpret_cast<float4 *>(vs + (size_t)pi * d + c8 * 8);
+            dst[0] = make_float4(vf[0], vf[1], vf[2], vf[3]);
+            dst[1] = make_float4(vf[4], vf[5], vf[6], vf[7]);
+            for (int h = 0; h < rep; h++) {
+                const float *qh = qs + h * d + c8 * 8;
+                float s = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; e++) kf[e] = (pi < np) ? knew[c8 * 8 + e] : 0.f;
-        }
-        for (int h = 0; h < rep; h++) {
-            const float *qh = qs + h * d + c8 * 8;
-            float s = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; e++) s = fmaf(qh[e], kf[e], s);
-            for (int m = 1; m < lp; m <<= 1) s += __shfl_xor(s, m);
-            if (c8 == 0 && pi < np) sc[h * ATT_CHUNK + pi] = s * scale;
+                for (int e = 0; e < 8; e++) s = fmaf(qh[e], kf[e], s);
+                for (int m = 1; m < lp; m <<= 1) s += __shfl_xor(s, m);
+                if (c8 == 0 && pi < np) sc[h * ATT_CHUNK + pi] = s * scale;
+            }
         }
     }
     __syncthreads();
@@ -219,18 +235,18 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
         float sum = e;
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
-        if (lane < np) sc[h * ATT_CHUNK + lane] = e;
+        if (lane < ATT_CHUNK) sc[h * ATT_CHUNK + lane] = e; // zero beyond the chunk's last position
         if (lane == 0) { stat[2 * h] = mx; stat[2 * h + 1] = sum; }
     }
     __syncthreads();
-    // sum_p e_p v_p: thread = (head group, dim)
+    // sum_p e_p v_p: thread = (head group, dim); positions in order, rows beyond np carry weight zero
     const int dim = tid % d, hg = tid / d, nhg = blockDim.x / d;
     float acc[ATT_MAX_REP];
 #pragma unroll
     for (int i = 0; i < ATT_MAX_REP; i++) acc[i] = 0.f;
-    for (int pi = 0; pi < np; pi++) {
-        const int p = p0 + pi;
-        const float vv = (p == pos) ? vnew[dim] : __half2float(__ushort_as_half(vc[(size_t)p * d + dim]));
+#pragma unroll 8
+    for (int pi = 0; pi < ATT_CHUNK; pi++) {
+        const float vv = vs[(size_t)pi * d + dim];
 #pragma unroll
         for (int i = 0; i < ATT_MAX_REP; i++) {
             int h = hg + i * nhg;
@@ -248,65 +264,70 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
     }
 }
 
+// grid (heads), 256 threads.  The (m, l) pairs of the head's splits go through LDS so that every thread
+// knows the weights exp(m_s - max) before it walks the splits; the walk itself has no dependent loads.
 __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, const int32_t *pos_p, int n_heads, int n_kv,
-                                                           int d, int max_splits, float *att, uint8_t *xq_att) {
-    __shared__ float outs[256];
+                                                           int d, int max_splits, float *att) {
+    extern __shared__ float cm[];
+    float *wgt = cm;                 // [max_splits] exp(m_s - max)
+    float *red = wgt + max_splits;   // [4] wave maxima, then [4] wave sums of l_s w_s
     const int head = blockIdx.x, rep = n_heads / n_kv, kvh = head / rep, h = head - kvh * rep;
     const int nsplit = pos_p[0] / ATT_CHUNK + 1;
-    const int dim = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float *base = part + ((size_t)(kvh * max_splits) * rep + h) * (d + 2);
+    const size_t stride = (size_t)rep * (d + 2);
+    // maxima
+    float mx = -INFINITY;
+    for (int s = tid; s < nsplit; s += 256) mx = fmaxf(mx, base[s * stride]);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    // weights and the normaliser, summed in split order by one thread so that the result does not depend on timing
+    for (int s = tid; s < nsplit; s += 256) wgt[s] = expf(base[s * stride] - mx);
+    __syncthreads();
+    const int dim = tid;
     if (dim < d) {
-        const float *base = part + ((size_t)(kvh * max_splits) * rep + h) * (d + 2);
-        const size_t stride = (size_t)rep * (d + 2);
-        float mx = -INFINITY;
-        for (int s = 0; s < nsplit; s++) mx = fmaxf(mx, base[s * stride]);
         float l = 0.f, o = 0.f;
-        for (int s = 0; s < nsplit; s++) {
-            float w = expf(base[s * stride] - mx);
-            l = fmaf(base[s * stride + 1], w, l);
-            o = fmaf(base[s * stride + 2 + dim], w, o);
+        int s = 0;
+        for (; s + 4 <= nsplit; s += 4) {
+            float l4[4], o4[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                l4[u] = base[(s + u) * stride + 1];
+                o4[u] = base[(s + u) * stride + 2 + dim];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                l = fmaf(l4[u], wgt[s + u], l);
+                o = fmaf(o4[u], wgt[s + u], o);
+            }
+        }
+        for (; s < nsplit; s++) {
+            l = fmaf(base[s * stride + 1], wgt[s], l);
+            o = fmaf(base[s * stride + 2 + dim], wgt[s], o);
         }
         float v = o / l;
-        outs[dim] = v;
         att[(size_t)head * d + dim] = v;
-    }
-    __syncthreads();
-    const int ntask = d >> 3;
-    const int kpad = (n_heads * d + 15) & ~15;
-    uint4 *grp = reinterpret_cast<uint4 *>(xq_att + (size_t)4 * kpad);
-    if ((int)threadIdx.x < ((ntask + 3) & ~3)) {
-        const int t = threadIdx.x;
-        const bool live = t < ntask;
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = live ? outs[t * 8 + i] : 0.f;
-        axq_split8(v, head * ntask + t, live, xq_att, grp, kpad);
     }
 }
 
 // act = silu(gate) * up over [inter]; gu = [gate (inter) | up (inter)].
-__global__ void __launch_bounds__(256) swiglu_kernel(const float *gu, int inter, float *act, uint8_t *xq) {
-    const int ntask = inter >> 3;
-    const int kpad = (inter + 15) & ~15;
-    uint4 *grp = reinterpret_cast<uint4 *>(xq + (size_t)4 * kpad);
+__global__ void __launch_bounds__(256) swiglu_kernel(const float *gu, int inter, float *act) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    const bool live = t < ntask;
+    if (t >= (inter >> 3)) return;
+    const float4 *pg = reinterpret_cast<const float4 *>(gu + (size_t)t * 8);
+    const float4 *pu = reinterpret_cast<const float4 *>(gu + inter + (size_t)t * 8);
+    float4 ga = pg[0], gb = pg[1], ua = pu[0], ub = pu[1];
+    const float g[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+    const float u[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
     float v[8];
-    if (live) {
-        const float4 *pg = reinterpret_cast<const float4 *>(gu + (size_t)t * 8);
-        const float4 *pu = reinterpret_cast<const float4 *>(gu + inter + (size_t)t * 8);
-        float4 ga = pg[0], gb = pg[1], ua = pu[0], ub = pu[1];
-        const float g[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
-        const float u[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = (g[i] * (1.0f / (1.0f + expf(-g[i])))) * u[i];
-        float4 *o = reinterpret_cast<float4 *>(act + (size_t)t * 8);
-        o[0] = make_float4(v[0], v[1], v[2], v[3]);
-        o[1] = make_float4(v[4], v[5], v[6], v[7]);
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = 0.f;
-    }
-    axq_split8(v, t, live, xq, grp, kpad);
+    for (int i = 0; i < 8; i++) v[i] = (g[i] * (1.0f / (1.0f + expf(-g[i])))) * u[i];
+    float4 *o = reinterpret_cast<float4 *>(act + (size_t)t * 8);
+    o[0] = make_float4(v[0], v[1], v[2], v[3]);
+    o[1] = make_float4(v[4], v[5], v[6], v[7]);
 }
 
 // argmax over the logits, last index among equal maxima (Iterator::max_by); then pos += 1.
@@ -381,15 +402,29 @@ int copy_rows(axq_ctx *ctx, axq_weight *dst, const axq_weight *src, int64_t row_
     return AXQ_OK;
 }
 
-// y = W x (+ bias): split-form GEMV when the shape is covered, else the f32 path.
-int gemv(axq_model *m, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
-    int rc = axq_dev_gemv_dp(m->ctx, w, x, xq, bias, y);
-    if (rc < 0) return rc;
-    if (rc == 1) return AXQ_OK;
-    return axq_dev_gemv(m->ctx, w, x, 1, bias, y);
+// y = W f(x) (+ bias), f = identity, RMSNorm with weights `aux`, or SwiGLU with `aux` as the `up` vector.
+// The matrix-pipe GEMV applies f while it stages x; for a linear it does not cover (other weight types,
+// K not a multiple of 64 or beyond 16384) f runs as a kernel of its own into `tmp` and the f32 GEMV follows.
+int linear(axq_model *m, const axq_weight *w, const float *x, int mode, const float *aux, float *tmp, const float *bias,
+           float *y) {
+    axq_ctx *ctx = m->ctx;
+    if (axq_dev_gemv_dp_covers(w)) {
+        int rc = axq_dev_gemv_dp_ex(ctx, w, x, nullptr, mode, aux, m->cfg.rms_norm_eps, bias, y);
+        return rc < 0 ? rc : AXQ_OK;
+    }
+    const int k = (int)w->k;
+    if (mode == AXQ_X_RMSNORM) {
+        norm_kernel<<<1, 1024, 0, ctx->stream>>>(x, aux, k, m->cfg.rms_norm_eps, tmp);
+        x = tmp;
+    } else if (mode == AXQ_X_SWIGLU) {
+        swiglu_kernel<<<(k / 8 + 255) / 256, 256, 0, ctx->stream>>>(x, k, tmp); // x = [gate | up]
+        x = tmp;
+    }
+    return axq_dev_gemv(ctx, w, x, 1, bias, y);
 }
 
-// The kernels of one token, enqueued on the context's stream.
+// The kernels of one token, enqueued on the context's stream: six per layer when every linear is covered
+// by the matrix-pipe GEMV (norms and SwiGLU ride in the GEMVs, residual adds in their bias slot).
 int enqueue_step(axq_model *m) {
     axq_ctx *ctx = m->ctx;
     const axq_model_config &c = m->cfg;
@@ -397,27 +432,23 @@ int enqueue_step(axq_model *m) {
     const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim;
     const size_t kv_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * d;
     const int rep = c.num_attention_heads / c.num_key_value_heads;
-    const size_t attn_lds = (size_t)(rep * d + 2 * d + rep * ATT_CHUNK + 2 * rep) * sizeof(float);
+    const size_t attn_lds = (size_t)(rep * d + 2 * d + rep * ATT_CHUNK + 2 * rep + ATT_CHUNK * d) * sizeof(float);
+    const size_t comb_lds = (size_t)(m->max_splits + 8) * sizeof(float);
     int rc;
+    embed_kernel<<<(H / 8 + 255) / 256, 256, 0, st>>>(m->emb, m->tok, m->h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
-        norm_kernel<<<1, 1024, 0, st>>>(l == 0 ? m->emb : nullptr, m->tok, m->h, m->norm_attn + (size_t)l * H, H,
-                                        c.rms_norm_eps, m->xn, m->xq_h);
-        if ((rc = gemv(m, m->w_qkv[l], m->xn, m->xq_h, nullptr, m->qkv))) return rc;
+        if ((rc = linear(m, m->w_qkv[l], m->h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, m->xn, nullptr, m->qkv))) return rc;
         attn_partial_kernel<<<dim3(c.num_key_value_heads, m->max_splits), 256, attn_lds, st>>>(
             m->qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer, m->vcache + (size_t)l * kv_layer, m->pos,
             c.num_attention_heads, c.num_key_value_heads, d, c.max_position_embeddings, m->max_splits, m->att_part);
-        attn_combine_kernel<<<c.num_attention_heads, 256, 0, st>>>(m->att_part, m->pos, c.num_attention_heads,
-                                                                   c.num_key_value_heads, d, m->max_splits, m->att, m->xq_att);
-        if ((rc = gemv(m, m->w_o[l], m->att, m->xq_att, m->h, m->h))) return rc; // residual through the bias slot
-        norm_kernel<<<1, 1024, 0, st>>>(nullptr, m->tok, m->h, m->norm_ffn + (size_t)l * H, H, c.rms_norm_eps, m->xn,
-                                        m->xq_h);
-        if ((rc = gemv(m, m->w_gu[l], m->xn, m->xq_h, nullptr, m->gu))) return rc;
-        swiglu_kernel<<<(I / 8 + 255) / 256, 256, 0, st>>>(m->gu, I, m->act, m->xq_act);
-        if ((rc = gemv(m, m->w_down[l], m->act, m->xq_act, m->h, m->h))) return rc;
+        attn_combine_kernel<<<c.num_attention_heads, 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
+                                                                          c.num_key_value_heads, d, m->max_splits, m->att);
+        // residual adds go through the bias slot, in place
+        if ((rc = linear(m, m->w_o[l], m->att, AXQ_X_PLAIN, nullptr, nullptr, m->h, m->h))) return rc;
+        if ((rc = linear(m, m->w_gu[l], m->h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, m->xn, nullptr, m->gu))) return rc;
+        if ((rc = linear(m, m->w_down[l], m->gu, AXQ_X_SWIGLU, m->gu + I, m->act, m->h, m->h))) return rc;
     }
-    norm_kernel<<<1, 1024, 0, st>>>(c.num_hidden_layers == 0 ? m->emb : nullptr, m->tok, m->h, m->norm_final, H,
-                                    c.rms_norm_eps, m->xn, m->xq_h);
-    if ((rc = gemv(m, m->w_head, m->xn, m->xq_h, nullptr, m->logits))) return rc;
+    if ((rc = linear(m, m->w_head, m->h, AXQ_X_RMSNORM, m->norm_final, m->xn, nullptr, m->logits))) return rc;
     argmax_kernel<<<1, 1024, 0, st>>>(m->logits, c.vocab_size, m->next, m->pos);
     AXQ_LAUNCH_CHECK(ctx, "decode step");
     return AXQ_OK;
@@ -506,8 +537,6 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     TRY(dev_alloc(&m->h, H)); TRY(dev_alloc(&m->xn, H)); TRY(dev_alloc(&m->qkv, m->qkv_rows)); TRY(dev_alloc(&m->att, m->q_dim));
     TRY(dev_alloc(&m->att_part, (size_t)c.num_key_value_heads * m->max_splits * (c.num_attention_heads / c.num_key_value_heads) * (c.head_dim + 2)));
     TRY(dev_alloc(&m->gu, (size_t)2 * I)); TRY(dev_alloc(&m->act, I)); TRY(dev_alloc(&m->logits, c.vocab_size));
-    TRY(dev_alloc(&m->xq_h, axq_split_bytes(H))); TRY(dev_alloc(&m->xq_att, axq_split_bytes(m->q_dim)));
-    TRY(dev_alloc(&m->xq_act, axq_split_bytes(I)));
     TRY(dev_alloc(&m->pos, 1)); TRY(dev_alloc(&m->tok, 1)); TRY(dev_alloc(&m->next, 1)); TRY(dev_alloc(&m->gen, 1));
     TRY(dev_alloc(&m->prompt, m->prompt_cap)); TRY(dev_alloc(&m->out, m->out_cap));
 #undef TRY
@@ -562,7 +591,7 @@ void axq_model_free(axq_model *m) {
     for (auto *w : m->w_down) axq_weight_free(ctx, w);
     axq_weight_free(ctx, m->w_head);
     void *bufs[] = {m->emb, m->norm_attn, m->norm_ffn, m->norm_final, m->rope_cos, m->rope_sin, m->kcache, m->vcache, m->h,
-                    m->xn, m->qkv, m->att, m->att_part, m->gu, m->act, m->logits, m->xq_h, m->xq_att, m->xq_act, m->pos, m->tok,
+                    m->xn, m->qkv, m->att, m->att_part, m->gu, m->act, m->logits, m->pos, m->tok,
                     m->next, m->gen, m->prompt, m->out};
     for (void *p : bufs)
         if (p) (void)hipFree(p);

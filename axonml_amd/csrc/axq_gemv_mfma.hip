@@ -46,6 +46,9 @@ struct DpArgs {
     int n_rows, k;
     int S, G, P;   // K slices per pass, row groups per workgroup, passes over K per lane
     int steps;     // 4-row steps per group
+    int mode;      // what x is: AXQ_X_PLAIN, or a vector still to be normalised / gated (see axq_internal.h)
+    const float *aux; // AXQ_X_RMSNORM: the norm weights; AXQ_X_SWIGLU: the `up` vector (x is `gate`)
+    float eps;
 };
 
 __device__ inline float f16lo(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v & 0xFFFF))); }
@@ -371,7 +374,8 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     const int kpad = (a.k + 15) & ~15;
     uint4 *wgrp = reinterpret_cast<uint4 *>(wplanes + (size_t)4 * kpad);
     const int n16 = (int)(axq_split_bytes(a.k) >> 4);
-    float *red = reinterpret_cast<float *>(lds_raw + n16 + 1); // one spare 16-byte slot takes the surplus stores of step 3
+    // one spare 16-byte slot takes the surplus stores of step 3, 64 bytes hold per-wave sums of a fused RMSNorm
+    float *red = reinterpret_cast<float *>(lds_raw + n16 + 1 + 4);
     const int rows_per_group = a.steps * 4;
     const int last = a.n_rows - 1;
     const int red_stride = 4 * a.S; // partial sums per output row in the LDS reduction buffer
@@ -383,6 +387,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     //    most two 8-element split tasks of raw x (K <= 16 per thread by construction of the launch), or at
     //    most five 16-byte pieces of an x that arrives already split.
     uint4 x0, x1, x2, x3, x4 = {0, 0, 0, 0};
+    uint4 e0 = {0, 0, 0, 0}, e1 = e0, e2 = e0, e3 = e0; // second operand of a fused prologue
     const int ntask = a.k >> 3; // K is a multiple of 64 here: whole quads of tasks
     if (PRE) {
         const uint4 *src = reinterpret_cast<const uint4 *>(a.xq);
@@ -395,6 +400,14 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
             return reinterpret_cast<const uint4 *>(a.x + (size_t)t * 8)[h];
         };
         x0 = half(0, 0); x1 = half(0, 1); x2 = half(1, 0); x3 = half(1, 1);
+        if (a.mode != AXQ_X_PLAIN) {
+            auto half2 = [&](int u, int h) {
+                int t = tid + u * nthreads;
+                t = t < ntask ? t : (t & 3);
+                return reinterpret_cast<const uint4 *>(a.aux + (size_t)t * 8)[h];
+            };
+            e0 = half2(0, 0); e1 = half2(0, 1); e2 = half2(1, 0); e3 = half2(1, 1);
+        }
     }
     __builtin_amdgcn_s_barrier();
     // 2. the ring: rows past the group's end re-read its first step (cache hits, no HBM traffic)
@@ -421,18 +434,51 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
         auto put = [&](int u, const uint4 &v) { int i = tid + u * nthreads; lds_raw[i < n16 ? i : n16] = v; };
         put(0, x0); put(1, x1); put(2, x2); put(3, x3); put(4, x4);
     } else {
-        auto split = [&](int u, const uint4 &lo, const uint4 &hi) {
-            const int t = tid + u * nthreads;
-            if (t < ntask) { // whole quads of lanes: K is a multiple of 64
-                const float xv[8] = {__builtin_bit_cast(float, lo.x), __builtin_bit_cast(float, lo.y),
-                                     __builtin_bit_cast(float, lo.z), __builtin_bit_cast(float, lo.w),
-                                     __builtin_bit_cast(float, hi.x), __builtin_bit_cast(float, hi.y),
-                                     __builtin_bit_cast(float, hi.z), __builtin_bit_cast(float, hi.w)};
-                axq_split8(xv, t, true, wplanes, wgrp, kpad);
-            }
+        auto unpack = [](const uint4 &lo, const uint4 &hi, float (&v)[8]) {
+            v[0] = __builtin_bit_cast(float, lo.x); v[1] = __builtin_bit_cast(float, lo.y);
+            v[2] = __builtin_bit_cast(float, lo.z); v[3] = __builtin_bit_cast(float, lo.w);
+            v[4] = __builtin_bit_cast(float, hi.x); v[5] = __builtin_bit_cast(float, hi.y);
+            v[6] = __builtin_bit_cast(float, hi.z); v[7] = __builtin_bit_cast(float, hi.w);
         };
-        split(0, x0, x1);
-        split(1, x2, x3);
+        float xv[2][8], ev[2][8];
+        unpack(x0, x1, xv[0]);
+        unpack(x2, x3, xv[1]);
+        const bool live0 = tid < ntask, live1 = tid + nthreads < ntask; // whole quads of lanes: K is a multiple of 64
+        if (a.mode == AXQ_X_RMSNORM) {
+            // RMSNorm::forward (llm/src/llama.rs:158-187) of the whole vector, by every workgroup for itself
+            unpack(e0, e1, ev[0]);
+            unpack(e2, e3, ev[1]);
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                if (live0) ss = fmaf(xv[0][i], xv[0][i], ss);
+                if (live1) ss = fmaf(xv[1][i], xv[1][i], ss);
+            }
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+            float *wsum = reinterpret_cast<float *>(lds_raw + n16 + 1); // 16 floats kept for this between x and `red`
+            if (lane == 0) wsum[wave] = ss;
+            __syncthreads();
+            float tot = 0.f;
+            for (int i = 0; i < (nthreads >> 6); i++) tot += wsum[i];
+            const float inv = 1.0f / sqrtf(tot / (float)a.k + a.eps);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                xv[0][i] = (xv[0][i] * inv) * ev[0][i];
+                xv[1][i] = (xv[1][i] * inv) * ev[1][i];
+            }
+        } else if (a.mode == AXQ_X_SWIGLU) {
+            // LLaMAMLP::forward (llm/src/llama.rs:562-567): silu(gate) * up, silu(v) = v * 1 / (1 + exp(-v))
+            unpack(e0, e1, ev[0]);
+            unpack(e2, e3, ev[1]);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                xv[0][i] = (xv[0][i] * (1.0f / (1.0f + expf(-xv[0][i])))) * ev[0][i];
+                xv[1][i] = (xv[1][i] * (1.0f / (1.0f + expf(-xv[1][i])))) * ev[1][i];
+            }
+        }
+        if (live0) axq_split8(xv[0], tid, true, wplanes, wgrp, kpad);
+        if (live1) axq_split8(xv[1], tid + nthreads, true, wplanes, wgrp, kpad);
     }
     __syncthreads();
     XOp xo;
@@ -509,12 +555,14 @@ void launch_nb(axq_ctx *ctx, const DpArgs &a, int nb, unsigned grid, unsigned bl
 }
 
 template <class T>
-bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
+bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux, float eps,
+               const float *bias, float *y) {
     if (w->k % 64 != 0 || w->k > 16384) return false;
     DpArgs a;
     a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
     a.x = x; a.xq = xq; a.bias = bias; a.y = y;
+    a.mode = mode; a.aux = aux; a.eps = eps;
     a.n_rows = (int)w->n_rows;
     a.k = (int)w->k;
     a.S = (a.k + 1023) / 1024;            // waves that span K once (<= 16)
@@ -534,7 +582,7 @@ bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t 
     if (nb > steps) nb = steps;
     const unsigned grid = (unsigned)((rowsteps + steps * a.G - 1) / (steps * a.G));
     size_t lds = (size_t)a.G * steps * 4 * a.S * 4 * sizeof(float);
-    lds += axq_split_bytes(a.k) + 16;
+    lds += axq_split_bytes(a.k) + 16 + 64;
     if (lds > 160 * 1024) return false;
     if (xq) launch_nb<T, true>(ctx, a, nb, grid, block, lds);
     else launch_nb<T, false>(ctx, a, nb, grid, block, lds);
@@ -556,19 +604,35 @@ int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq) {
 }
 
 // Returns 1 when the launch was made, 0 when this kernel does not cover the shape (the caller falls
-// back to the vector-ALU kernels), or a negative status.  xq = NULL: the kernel splits x itself.
-int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
+// back to the vector-ALU kernels), or a negative status.  xq = NULL: the kernel splits x itself, after
+// applying the prologue `mode` (axq_internal.h) with its second operand `aux`.
+int axq_dev_gemv_dp_ex(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux,
+                       float eps, const float *bias, float *y) {
     bool ok;
+    if (xq && mode != AXQ_X_PLAIN) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "a fused prologue needs the raw x");
     switch (w->type) {
-    case AXQ_Q4_K: ok = launch_dp<DQ4K>(ctx, w, x, xq, bias, y); break;
-    case AXQ_Q4_0: ok = launch_dp<DQ4x<false>>(ctx, w, x, xq, bias, y); break;
-    case AXQ_Q4_1: ok = launch_dp<DQ4x<true>>(ctx, w, x, xq, bias, y); break;
-    case AXQ_Q5_0: ok = launch_dp<DQ5x<false>>(ctx, w, x, xq, bias, y); break;
-    case AXQ_Q5_1: ok = launch_dp<DQ5x<true>>(ctx, w, x, xq, bias, y); break;
-    case AXQ_Q8_0: ok = launch_dp<DQ80>(ctx, w, x, xq, bias, y); break;
+    case AXQ_Q4_K: ok = launch_dp<DQ4K>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
+    case AXQ_Q4_0: ok = launch_dp<DQ4x<false>>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
+    case AXQ_Q4_1: ok = launch_dp<DQ4x<true>>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
+    case AXQ_Q5_0: ok = launch_dp<DQ5x<false>>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
+    case AXQ_Q5_1: ok = launch_dp<DQ5x<true>>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
+    case AXQ_Q8_0: ok = launch_dp<DQ80>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
     default: return 0;
     }
     if (!ok) return 0;
     AXQ_LAUNCH_CHECK(ctx, "gemv_dp_kernel");
     return 1;
+}
+
+int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
+    return axq_dev_gemv_dp_ex(ctx, w, x, xq, AXQ_X_PLAIN, nullptr, 0.f, bias, y);
+}
+
+// Whether axq_dev_gemv_dp_ex covers a weight of this type and width.
+bool axq_dev_gemv_dp_covers(const axq_weight *w) {
+    switch (w->type) {
+    case AXQ_Q4_K: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q8_0:
+        return w->k % 64 == 0 && w->k <= 16384;
+    default: return false;
+    }
 }
