@@ -121,7 +121,6 @@ __global__ void __launch_bounds__(1024) norm_kernel(const float *h, const float 
 // normalises, and writes the head's output as f32 and in split form.
 constexpr int ATT_CHUNK = 32;
 constexpr int ATT_MAX_REP = 8;  // query heads per KV head
-constexpr int ATT_MAX_PASS = 4; // 16-byte pieces of K (and of V) a thread fetches: 32 positions * d / 8 / 256 threads
 
 __device__ inline void halves_to_floats(const uint4 &raw, float (&f)[8]) {
     const uint32_t rr[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -132,18 +131,38 @@ __device__ inline void halves_to_floats(const uint4 &raw, float (&f)[8]) {
     }
 }
 
+// Sum over aligned groups of LP lanes (4, 8, 16 or 32), every lane of the group gets the total: DPP quad
+// permutes and row mirrors inside a 16-lane row, one lane exchange beyond it.
+template <int LP>
+__device__ inline float group_sum(float s) {
+    s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0xB1, 0xf, 0xf, true));
+    s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0x4E, 0xf, 0xf, true));
+    if (LP >= 8) s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0x141, 0xf, 0xf, true));
+    if (LP >= 16) s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0x140, 0xf, 0xf, true));
+    if (LP >= 32) s += __shfl_xor(s, 16);
+    return s;
+}
+
+// D = head size (32, 64, 128, 256), REP = query heads per KV head rounded up to a power of two (the real
+// count `rep` may be smaller).  Specialised so that the code is short and straight: a kernel that runs once
+// per layer is fetched cold, and its instruction fetch is part of its run time.
+template <int D, int REP>
 __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, const float *rope_cos, const float *rope_sin,
                                                            uint16_t *kcache, uint16_t *vcache, const int32_t *pos_p,
-                                                           int n_heads, int n_kv, int d, int max_pos, int max_splits,
-                                                           float *part) {
-    extern __shared__ float sm[];
+                                                           int n_heads, int n_kv, int max_pos, int max_splits, float *part) {
+    constexpr int HALF = D / 2;
+    constexpr int LP = D / 8, PPW = 64 / LP;                 // lanes per position, positions per wave pass
+    constexpr int NPASS = (ATT_CHUNK + 4 * PPW - 1) / (4 * PPW); // passes of the four waves over the chunk
+    constexpr int NQ = (REP * HALF + 255) / 256;             // rotation pairs of the query heads per thread
+    constexpr int NHG = 256 / D > 0 ? 256 / D : 1;           // head groups in the value sum (threads = NHG * D)
+    constexpr int HPT = (REP + NHG - 1) / NHG;               // heads per thread in the value sum
+    static_assert(D <= 256 && ATT_CHUNK <= 64 && REP <= ATT_MAX_REP, "shape limits");
+    __shared__ float qs[REP * D];            // rotated query heads
+    __shared__ float knew[D], vnew[D];       // the new key and value, f16-rounded
+    __shared__ __attribute__((aligned(16))) float sc[ATT_CHUNK * REP]; // scores, then exp(score - max), head-minor
+    __shared__ float stat[2 * REP];          // per head: m, l
+    __shared__ __attribute__((aligned(16))) float vs[ATT_CHUNK * D];   // the chunk's values
     const int rep = n_heads / n_kv;
-    float *qs = sm;                       // [rep][d]
-    float *knew = qs + rep * d;           // [d] f16-rounded
-    float *vnew = knew + d;               // [d]
-    float *sc = vnew + d;                 // [rep][ATT_CHUNK]
-    float *stat = sc + rep * ATT_CHUNK;   // [rep][2]: m, l
-    float *vs = stat + 2 * rep;           // [ATT_CHUNK][d]: the chunk's values
     const int kvh = blockIdx.x, split = blockIdx.y;
     const int pos = pos_p[0];
     const int p0 = split * ATT_CHUNK;
@@ -151,83 +170,99 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
     const int p1 = (p0 + ATT_CHUNK < pos + 1) ? p0 + ATT_CHUNK : pos + 1;
     const int np = p1 - p0;
     const bool has_new = pos < p1;
-    const int half = d >> 1;
-    const int q_dim = n_heads * d, kv_dim = n_kv * d;
+    const int q_dim = n_heads * D, kv_dim = n_kv * D;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    uint16_t *kc = kcache + (size_t)kvh * max_pos * d;
-    uint16_t *vc = vcache + (size_t)kvh * max_pos * d;
+    uint16_t *kc = kcache + (size_t)kvh * max_pos * D;
+    uint16_t *vc = vcache + (size_t)kvh * max_pos * D;
 
-    // Every cached byte this workgroup needs is requested before anything else: d/8 lanes per position,
-    // 64/(d/8) positions per wave pass, at most ATT_MAX_PASS passes.  Positions outside the chunk and the
-    // newest position (still in registers) re-read the chunk's first row and are not used.
-    const int lp = d >> 3, ppw = 64 / lp;
-    const int c8 = lane % lp, r = lane / lp;
-    uint4 kraw[ATT_MAX_PASS], vraw[ATT_MAX_PASS];
+    // Everything this workgroup reads from memory is requested here, so that the kernel pays one memory
+    // latency and not one per stage.  Positions outside the chunk and the newest one (still in registers)
+    // re-read the chunk's first row and are not used.
+    const int c8 = lane % LP, r = lane / LP;
+    uint4 kraw[NPASS], vraw[NPASS];
 #pragma unroll
-    for (int it = 0; it < ATT_MAX_PASS; it++) {
-        const int pi = (it * 4 + wave) * ppw + r;
+    for (int it = 0; it < NPASS; it++) {
+        const int pi = (it * 4 + wave) * PPW + r;
         const int p = (pi < np && p0 + pi != pos) ? p0 + pi : p0;
-        const bool any = it * 4 * ppw < ATT_CHUNK; // uniform: this pass exists for this head size
-        kraw[it] = any ? *reinterpret_cast<const uint4 *>(kc + (size_t)p * d + c8 * 8) : make_uint4(0, 0, 0, 0);
-        vraw[it] = any ? *reinterpret_cast<const uint4 *>(vc + (size_t)p * d + c8 * 8) : make_uint4(0, 0, 0, 0);
+        kraw[it] = *reinterpret_cast<const uint4 *>(kc + (size_t)p * D + c8 * 8);
+        vraw[it] = *reinterpret_cast<const uint4 *>(vc + (size_t)p * D + c8 * 8);
     }
+    const float *cs = rope_cos + (size_t)pos * HALF, *sn = rope_sin + (size_t)pos * HALF;
+    float qx1[NQ], qx2[NQ], qc[NQ], qn[NQ];
+#pragma unroll
+    for (int u = 0; u < NQ; u++) {
+        int i = tid + u * 256;
+        i = i < rep * HALF ? i : 0;
+        const int h = i / HALF, e = i % HALF;
+        const float *qh = qkv + (size_t)(kvh * rep + h) * D;
+        qc[u] = cs[e]; qn[u] = sn[e]; qx1[u] = qh[e]; qx2[u] = qh[e + HALF];
+    }
+    const int en = tid < HALF ? tid : 0;
+    const float *kh = qkv + q_dim + (size_t)kvh * D;
+    const float *vh = qkv + q_dim + kv_dim + (size_t)kvh * D;
+    const float nc = cs[en], ns = sn[en], k1 = kh[en], k2 = kh[en + HALF], v1 = vh[en], v2 = vh[en + HALF];
 
-    const float *cs = rope_cos + (size_t)pos * half, *sn = rope_sin + (size_t)pos * half;
-    for (int i = tid; i < rep * half; i += blockDim.x) {
-        int h = i / half, e = i - h * half;
-        const float *qh = qkv + (size_t)(kvh * rep + h) * d;
-        float c = cs[e], s = sn[e], x1 = qh[e], x2 = qh[e + half];
-        qs[h * d + e] = x1 * c - x2 * s;
-        qs[h * d + e + half] = x1 * s + x2 * c;
-    }
-    if (has_new) {
-        const float *kh = qkv + q_dim + (size_t)kvh * d;
-        const float *vh = qkv + q_dim + kv_dim + (size_t)kvh * d;
-        for (int e = tid; e < half; e += blockDim.x) {
-            float c = cs[e], s = sn[e], k1 = kh[e], k2 = kh[e + half];
-            __half ka = __float2half_rn(k1 * c - k2 * s), kb = __float2half_rn(k1 * s + k2 * c);
-            __half va = __float2half_rn(vh[e]), vb = __float2half_rn(vh[e + half]);
-            knew[e] = __half2float(ka); knew[e + half] = __half2float(kb);
-            vnew[e] = __half2float(va); vnew[e + half] = __half2float(vb);
-            kc[(size_t)pos * d + e] = __half_as_ushort(ka); kc[(size_t)pos * d + e + half] = __half_as_ushort(kb);
-            vc[(size_t)pos * d + e] = __half_as_ushort(va); vc[(size_t)pos * d + e + half] = __half_as_ushort(vb);
+    // RoPE (RotaryEmbedding::rotate_tensor, llm/src/llama.rs:281-321: half-split pairs) on the query heads ...
+#pragma unroll
+    for (int u = 0; u < NQ; u++) {
+        const int i = tid + u * 256;
+        if (i < rep * HALF) {
+            const int h = i / HALF, e = i % HALF;
+            qs[h * D + e] = qx1[u] * qc[u] - qx2[u] * qn[u];
+            qs[h * D + e + HALF] = qx1[u] * qn[u] + qx2[u] * qc[u];
         }
+    }
+    // ... and on the new key, which goes to the cache with the new value, rounded to f16
+    if (has_new && tid < HALF) {
+        const int e = tid;
+        __half ka = __float2half_rn(k1 * nc - k2 * ns), kb = __float2half_rn(k1 * ns + k2 * nc);
+        __half va = __float2half_rn(v1), vb = __float2half_rn(v2);
+        knew[e] = __half2float(ka); knew[e + HALF] = __half2float(kb);
+        vnew[e] = __half2float(va); vnew[e + HALF] = __half2float(vb);
+        kc[(size_t)pos * D + e] = __half_as_ushort(ka); kc[(size_t)pos * D + e + HALF] = __half_as_ushort(kb);
+        vc[(size_t)pos * D + e] = __half_as_ushort(va); vc[(size_t)pos * D + e + HALF] = __half_as_ushort(vb);
     }
     __syncthreads();
     // scores, and the chunk's values into LDS as f32
-    const float scale = 1.0f / sqrtf((float)d);
+    const float scale = 1.0f / sqrtf((float)D);
 #pragma unroll
-    for (int it = 0; it < ATT_MAX_PASS; it++) {
-        const int pi = (it * 4 + wave) * ppw + r; // position within the chunk
-        if (it * 4 * ppw < ATT_CHUNK && pi < ATT_CHUNK) {
+    for (int it = 0; it < NPASS; it++) {
+        const int pi = (it * 4 + wave) * PPW + r; // position within the chunk
+        if (pi < ATT_CHUNK) {
             float kf[8], vf[8];
-            if (pi < np && p0 + pi != pos) {
-                halves_to_floats(kraw[it], kf);
-                halves_to_floats(vraw[it], vf);
-            } else {
+            halves_to_floats(kraw[it], kf);
+            halves_to_floats(vraw[it], vf);
+            const bool cached = pi < np && p0 + pi != pos;
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    kf[e] = (pi < np) ? knew[c8 * 8 + e] : 0.f;
-                    vf[e] = (pi < np) ? vnew[c8 * 8 + e] : 0.f;
-                }
+            for (int e = 0; e < 8; e++) {
+                kf[e] = cached ? kf[e] : (pi < np ? knew[c8 * 8 + e] : 0.f);
+                vf[e] = cached ? vf[e] : (pi < np ? vnew[c8 * 8 + e] : 0.f);
             }
-            float4 *dst = reinterpret_cast<float4 *>(vs + (size_t)pi * d + c8 * 8);
+            float4 *dst = reinterpret_cast<float4 *>(vs + pi * D + c8 * 8);
             dst[0] = make_float4(vf[0], vf[1], vf[2], vf[3]);
             dst[1] = make_float4(vf[4], vf[5], vf[6], vf[7]);
-            for (int h = 0; h < rep; h++) {
-                const float *qh = qs + h * d + c8 * 8;
-                float s = 0.f;
+            float sh[REP];
 #pragma unroll
-                for (int e = 0; e < 8; e++) s = fmaf(qh[e], kf[e], s);
-                for (int m = 1; m < lp; m <<= 1) s += __shfl_xor(s, m);
-                if (c8 == 0 && pi < np) sc[h * ATT_CHUNK + pi] = s * scale;
+            for (int h = 0; h < REP; h++) {
+                const float4 *qh = reinterpret_cast<const float4 *>(qs + h * D + c8 * 8);
+                const float4 qa = qh[0], qb = qh[1];
+                float s = qa.x * kf[0];
+                s = fmaf(qa.y, kf[1], s); s = fmaf(qa.z, kf[2], s); s = fmaf(qa.w, kf[3], s);
+                s = fmaf(qb.x, kf[4], s); s = fmaf(qb.y, kf[5], s); s = fmaf(qb.z, kf[6], s); s = fmaf(qb.w, kf[7], s);
+                sh[h] = s;
+            }
+#pragma unroll
+            for (int h = 0; h < REP; h++) sh[h] = group_sum<LP>(sh[h]);
+            if (c8 == 0) {
+#pragma unroll
+                for (int h = 0; h < REP; h++) sc[pi * REP + h] = (pi < np && h < rep) ? sh[h] * scale : -INFINITY;
             }
         }
     }
     __syncthreads();
     // per head: chunk maximum, exponentials, their sum (one wave per head, heads strided over the 4 waves)
     for (int h = wave; h < rep; h += 4) {
-        float v = lane < np ? sc[h * ATT_CHUNK + lane] : -INFINITY; // ATT_CHUNK <= 64
+        float v = lane < ATT_CHUNK ? sc[lane * REP + h] : -INFINITY;
         float mx = v;
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
@@ -235,29 +270,30 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
         float sum = e;
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
-        if (lane < ATT_CHUNK) sc[h * ATT_CHUNK + lane] = e; // zero beyond the chunk's last position
+        if (lane < ATT_CHUNK) sc[lane * REP + h] = e; // zero beyond the chunk's last position
         if (lane == 0) { stat[2 * h] = mx; stat[2 * h + 1] = sum; }
     }
     __syncthreads();
-    // sum_p e_p v_p: thread = (head group, dim); positions in order, rows beyond np carry weight zero
-    const int dim = tid % d, hg = tid / d, nhg = blockDim.x / d;
-    float acc[ATT_MAX_REP];
+    // sum_p e_p v_p: thread = (head group, dim), heads hg, hg + NHG, ...; positions in order, rows beyond
+    // np carry weight zero
+    const int dim = tid % D, hg = tid / D;
+    float acc[HPT];
 #pragma unroll
-    for (int i = 0; i < ATT_MAX_REP; i++) acc[i] = 0.f;
+    for (int i = 0; i < HPT; i++) acc[i] = 0.f;
 #pragma unroll 8
     for (int pi = 0; pi < ATT_CHUNK; pi++) {
-        const float vv = vs[(size_t)pi * d + dim];
+        const float vv = vs[pi * D + dim];
 #pragma unroll
-        for (int i = 0; i < ATT_MAX_REP; i++) {
-            int h = hg + i * nhg;
-            if (h < rep) acc[i] = fmaf(sc[h * ATT_CHUNK + pi], vv, acc[i]);
+        for (int i = 0; i < HPT; i++) {
+            const int h = hg + i * NHG;
+            acc[i] = fmaf(sc[pi * REP + (h < REP ? h : 0)], vv, acc[i]);
         }
     }
 #pragma unroll
-    for (int i = 0; i < ATT_MAX_REP; i++) {
-        int h = hg + i * nhg;
-        if (h < rep) {
-            float *o = part + ((size_t)(kvh * max_splits + split) * rep + h) * (d + 2);
+    for (int i = 0; i < HPT; i++) {
+        const int h = hg + i * NHG;
+        if (h < rep && tid < NHG * D) {
+            float *o = part + ((size_t)(kvh * max_splits + split) * rep + h) * (D + 2);
             o[2 + dim] = acc[i];
             if (dim == 0) { o[0] = stat[2 * h]; o[1] = stat[2 * h + 1]; }
         }
@@ -402,6 +438,33 @@ int copy_rows(axq_ctx *ctx, axq_weight *dst, const axq_weight *src, int64_t row_
     return AXQ_OK;
 }
 
+template <int D, int REP>
+void launch_attn_partial_t(axq_model *m, int l, hipStream_t st) {
+    const axq_model_config &c = m->cfg;
+    const size_t kv_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * D;
+    attn_partial_kernel<D, REP><<<dim3(c.num_key_value_heads, m->max_splits), 256, 0, st>>>(
+        m->qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer, m->vcache + (size_t)l * kv_layer, m->pos,
+        c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, m->max_splits, m->att_part);
+}
+
+template <int D>
+void launch_attn_partial_d(axq_model *m, int l, hipStream_t st) {
+    const int rep = m->cfg.num_attention_heads / m->cfg.num_key_value_heads;
+    if (rep == 1) launch_attn_partial_t<D, 1>(m, l, st);
+    else if (rep == 2) launch_attn_partial_t<D, 2>(m, l, st);
+    else if (rep <= 4) launch_attn_partial_t<D, 4>(m, l, st);
+    else launch_attn_partial_t<D, 8>(m, l, st);
+}
+
+void launch_attn_partial(axq_model *m, int l, hipStream_t st) {
+    switch (m->cfg.head_dim) { // axq_model_create admits these four sizes only
+    case 32: launch_attn_partial_d<32>(m, l, st); break;
+    case 64: launch_attn_partial_d<64>(m, l, st); break;
+    case 128: launch_attn_partial_d<128>(m, l, st); break;
+    default: launch_attn_partial_d<256>(m, l, st); break;
+    }
+}
+
 // y = W f(x) (+ bias), f = identity, RMSNorm with weights `aux`, or SwiGLU with `aux` as the `up` vector.
 // The matrix-pipe GEMV applies f while it stages x; for a linear it does not cover (other weight types,
 // K not a multiple of 64 or beyond 16384) f runs as a kernel of its own into `tmp` and the f32 GEMV follows.
@@ -430,17 +493,12 @@ int enqueue_step(axq_model *m) {
     const axq_model_config &c = m->cfg;
     hipStream_t st = ctx->stream;
     const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim;
-    const size_t kv_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * d;
-    const int rep = c.num_attention_heads / c.num_key_value_heads;
-    const size_t attn_lds = (size_t)(rep * d + 2 * d + rep * ATT_CHUNK + 2 * rep + ATT_CHUNK * d) * sizeof(float);
     const size_t comb_lds = (size_t)(m->max_splits + 8) * sizeof(float);
     int rc;
     embed_kernel<<<(H / 8 + 255) / 256, 256, 0, st>>>(m->emb, m->tok, m->h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
         if ((rc = linear(m, m->w_qkv[l], m->h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, m->xn, nullptr, m->qkv))) return rc;
-        attn_partial_kernel<<<dim3(c.num_key_value_heads, m->max_splits), 256, attn_lds, st>>>(
-            m->qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer, m->vcache + (size_t)l * kv_layer, m->pos,
-            c.num_attention_heads, c.num_key_value_heads, d, c.max_position_embeddings, m->max_splits, m->att_part);
+        launch_attn_partial(m, l, st);
         attn_combine_kernel<<<c.num_attention_heads, 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
                                                                           c.num_key_value_heads, d, m->max_splits, m->att);
         // residual adds go through the bias slot, in place
