@@ -13,9 +13,9 @@
 //     element that matters inside f16's normal range; the row scale is undone on the output.
 // Accumulation is f32 inside the MFMA, in K order.
 //
-// Tiling: a workgroup computes BM x 128 outputs (BM = 128 or 256) with BM/32 waves, one 64 x 64 block
-// (2 x 2 MFMA tiles) per wave; K advances 64 at a time through one LDS stage holding the x tile and
-// the two weight tiles; two workgroups share a compute unit and fill each other's load/dequant gaps.
+// Tiling: a workgroup computes BM x 128 outputs (BM = 128 or 256); K advances 64 at a time through two LDS
+// stages, each holding the x tile and the two weight tiles.  Half of the waves multiply, the other half
+// feed (see gemm_kernel).
 #include <hip/hip_fp16.h>
 
 #include "axq_internal.h"
@@ -24,6 +24,7 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4))); // a 16-byte register quad (arrays of HIP's uint4 struct end up in scratch)
 
 constexpr int BN = 128;  // output columns (weight rows) per workgroup
 constexpr int BK = 64;   // K per stage
@@ -39,6 +40,20 @@ struct GemmArgs {
 };
 
 __device__ inline float h2f(uint32_t bits) { return __half2float(__ushort_as_half((unsigned short)bits)); }
+template <int B>
+__device__ inline float ubyte(uint32_t v) { // byte B of v as a float, one instruction
+    float r;
+    if (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(v));
+    else if (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(v));
+    else if (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(v));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+
+// Weights go through the matrix pipe as WSCALE * w = wh + wl with wh, wl in f16: the power-of-two factor
+// keeps the low part of ordinary weights (|w| > 5e-4) out of f16's subnormal range; the epilogue divides
+// it out again.  A trait names its factor WS, and says PRESCALED when its convert step applies it already.
+constexpr float WSCALE = 256.0f;
 
 // ---------------------------------------------------------------------------
 // Dequantisation units.  A unit is 16 weights of one weight row inside the current 64-wide K step:
@@ -47,7 +62,10 @@ __device__ inline float h2f(uint32_t bits) { return __half2float(__ushort_as_hal
 // or of the GGUF spec (Q5_0, Q5_1, Q4_K), rounding as the f32 reference does (multiply, then add).
 // ---------------------------------------------------------------------------
 struct GQ4K {
-    __device__ static void deq16(const GemmArgs &a, size_t row, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+    static constexpr bool PRESCALED = true;
+    static constexpr float WS = WSCALE;
+    struct Raw { uint2 q; uint4 h; };
+    __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
         const int cpr = a.k >> 6;          // pairs per row
         const int pair = kstep;            // one pair of sub-blocks per K step
         const int slice = pair >> 6, pr = pair & 63;
@@ -55,8 +73,13 @@ struct GQ4K {
         P = P < 64 ? P : 64;
         const int half = u4 >> 1, part = u4 & 1;
         const uint8_t *base = a.codes + row * a.codes_pitch + (size_t)slice * 2048 + (size_t)half * 16 * P + (size_t)pr * 16 + part * 8;
-        const uint2 q = *reinterpret_cast<const uint2 *>(base);
-        const uint4 h = *reinterpret_cast<const uint4 *>(a.meta + row * a.meta_pitch + (size_t)(pair >> 2) * 16);
+        r.q = *reinterpret_cast<const uint2 *>(base);
+        r.h = *reinterpret_cast<const uint4 *>(a.meta + row * a.meta_pitch + (size_t)(pair >> 2) * 16);
+    }
+    __device__ static void cvt16(const Raw &r, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+        const uint2 q = r.q;
+        const uint4 h = r.h;
+        const int pair = kstep, half = u4 >> 1, part = u4 & 1;
         const int p = pair & 3, sh = (p & 1) * 16;
         const uint32_t ya = h.y >> sh, za = h.z >> sh, wa = h.w >> sh;
         uint32_t scp, mp;
@@ -67,16 +90,18 @@ struct GQ4K {
             scp = (wa & 0x0F0F) | ((ya >> 2) & 0x3030);
             mp = ((wa >> 4) & 0x0F0F) | ((za >> 2) & 0x3030);
         }
-        const float d = h2f(h.x & 0xFFFF), dmin = h2f(h.x >> 16);
-        const float sd0 = d * (float)(scp & 0xFF), sd1 = d * (float)(scp >> 8);
-        const float sm0 = dmin * (float)(mp & 0xFF), sm1 = dmin * (float)(mp >> 8);
-        const uint32_t qq[2] = {q.x, q.y};
+        const float d = WSCALE * h2f(h.x & 0xFFFF), dmin = WSCALE * h2f(h.x >> 16);
+        const float sd0 = d * ubyte<0>(scp), sd1 = d * ubyte<1>(scp);
+        const float sm0 = dmin * ubyte<0>(mp), sm1 = dmin * ubyte<1>(mp);
+        // one rounding per weight (fma) where the f32 reference has two: far below what f16 pairs resolve
+        const uint32_t ml[2] = {q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu};
+        const uint32_t mh[2] = {(q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu};
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            uint32_t byte = (qq[i >> 2] >> (8 * (i & 3))) & 0xFF;
-            float lo = sd0 * (float)(byte & 0xF), hi = sd1 * (float)(byte >> 4);
-            w[i] = lo - sm0;
-            w[8 + i] = hi - sm1;
+        for (int j = 0; j < 2; j++) {
+            w[4 * j + 0] = fmaf(sd0, ubyte<0>(ml[j]), -sm0); w[4 * j + 1] = fmaf(sd0, ubyte<1>(ml[j]), -sm0);
+            w[4 * j + 2] = fmaf(sd0, ubyte<2>(ml[j]), -sm0); w[4 * j + 3] = fmaf(sd0, ubyte<3>(ml[j]), -sm0);
+            w[8 + 4 * j + 0] = fmaf(sd1, ubyte<0>(mh[j]), -sm1); w[8 + 4 * j + 1] = fmaf(sd1, ubyte<1>(mh[j]), -sm1);
+            w[8 + 4 * j + 2] = fmaf(sd1, ubyte<2>(mh[j]), -sm1); w[8 + 4 * j + 3] = fmaf(sd1, ubyte<3>(mh[j]), -sm1);
         }
         k0 = half * 16 + part * 8;
         k1 = 32 + k0;
@@ -85,19 +110,20 @@ struct GQ4K {
 
 template <bool WITH_MIN>
 struct GQ4x { // reference nibble order: byte i = elements 2i (low), 2i+1 (high)
-    __device__ static void deq16(const GemmArgs &a, size_t row, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+    static constexpr bool PRESCALED = false;
+    static constexpr float WS = WSCALE;
+    struct Raw { uint2 q; uint32_t m; };
+    __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
         const int blk = kstep * 2 + (u4 >> 1), part = u4 & 1;
-        const uint2 q = *reinterpret_cast<const uint2 *>(a.codes + row * a.codes_pitch + (size_t)blk * 16 + part * 8);
+        r.q = *reinterpret_cast<const uint2 *>(a.codes + row * a.codes_pitch + (size_t)blk * 16 + part * 8);
         const uint8_t *mp = a.meta + row * a.meta_pitch;
-        float scale, mn = 0.f;
-        if (WITH_MIN) {
-            uint32_t m = *reinterpret_cast<const uint32_t *>(mp + (size_t)blk * 4);
-            scale = h2f(m & 0xFFFF);
-            mn = h2f(m >> 16);
-        } else {
-            scale = h2f(*reinterpret_cast<const uint16_t *>(mp + (size_t)blk * 2));
-        }
-        const uint32_t qq[2] = {q.x, q.y};
+        r.m = WITH_MIN ? *reinterpret_cast<const uint32_t *>(mp + (size_t)blk * 4)
+                       : (uint32_t) * reinterpret_cast<const uint16_t *>(mp + (size_t)blk * 2);
+    }
+    __device__ static void cvt16(const Raw &r, int, int u4, float (&w)[16], int &k0, int &k1) {
+        const int part = u4 & 1;
+        const float scale = h2f(r.m & 0xFFFF), mn = WITH_MIN ? h2f(r.m >> 16) : 0.f;
+        const uint32_t qq[2] = {r.q.x, r.q.y};
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             uint32_t nib = (qq[i >> 3] >> (4 * (i & 7))) & 0xF;
@@ -115,20 +141,22 @@ struct GQ4x { // reference nibble order: byte i = elements 2i (low), 2i+1 (high)
 
 template <bool WITH_MIN>
 struct GQ5x { // byte j = elements j (low nibble) and j + 16 (high); qh bit e = bit 4 of element e
-    __device__ static void deq16(const GemmArgs &a, size_t row, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+    static constexpr bool PRESCALED = false;
+    static constexpr float WS = WSCALE;
+    struct Raw { uint2 q; uint32_t qh, m; };
+    __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
         const int blk = kstep * 2 + (u4 >> 1), part = u4 & 1;
-        const uint2 q = *reinterpret_cast<const uint2 *>(a.codes + row * a.codes_pitch + (size_t)blk * 16 + part * 8);
-        const uint32_t qh = *reinterpret_cast<const uint32_t *>(a.qh + row * a.qh_pitch + (size_t)blk * 4);
+        r.q = *reinterpret_cast<const uint2 *>(a.codes + row * a.codes_pitch + (size_t)blk * 16 + part * 8);
+        r.qh = *reinterpret_cast<const uint32_t *>(a.qh + row * a.qh_pitch + (size_t)blk * 4);
         const uint8_t *mp = a.meta + row * a.meta_pitch;
-        float d, mn = 0.f;
-        if (WITH_MIN) {
-            uint32_t m = *reinterpret_cast<const uint32_t *>(mp + (size_t)blk * 4);
-            d = h2f(m & 0xFFFF);
-            mn = h2f(m >> 16);
-        } else {
-            d = h2f(*reinterpret_cast<const uint16_t *>(mp + (size_t)blk * 2));
-        }
-        const uint32_t qq[2] = {q.x, q.y};
+        r.m = WITH_MIN ? *reinterpret_cast<const uint32_t *>(mp + (size_t)blk * 4)
+                       : (uint32_t) * reinterpret_cast<const uint16_t *>(mp + (size_t)blk * 2);
+    }
+    __device__ static void cvt16(const Raw &r, int, int u4, float (&w)[16], int &k0, int &k1) {
+        const int part = u4 & 1;
+        const uint32_t qh = r.qh;
+        const float d = h2f(r.m & 0xFFFF), mn = WITH_MIN ? h2f(r.m >> 16) : 0.f;
+        const uint32_t qq[2] = {r.q.x, r.q.y};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const int e = part * 8 + i;
@@ -150,11 +178,18 @@ struct GQ5x { // byte j = elements j (low nibble) and j + 16 (high); qh bit e = 
 };
 
 struct GQ80 {
-    __device__ static void deq16(const GemmArgs &a, size_t row, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+    static constexpr bool PRESCALED = false;
+    static constexpr float WS = WSCALE;
+    struct Raw { uint4 q; uint32_t m; };
+    __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
         const int blk = kstep * 2 + (u4 >> 1), part = u4 & 1;
-        const uint4 q = *reinterpret_cast<const uint4 *>(a.codes + row * a.codes_pitch + (size_t)blk * 32 + part * 16);
-        const float scale = h2f(*reinterpret_cast<const uint16_t *>(a.meta + row * a.meta_pitch + (size_t)blk * 2));
-        const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
+        r.q = *reinterpret_cast<const uint4 *>(a.codes + row * a.codes_pitch + (size_t)blk * 32 + part * 16);
+        r.m = *reinterpret_cast<const uint16_t *>(a.meta + row * a.meta_pitch + (size_t)blk * 2);
+    }
+    __device__ static void cvt16(const Raw &r, int, int u4, float (&w)[16], int &k0, int &k1) {
+        const int part = u4 & 1;
+        const float scale = h2f(r.m);
+        const uint32_t qq[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
 #pragma unroll
         for (int i = 0; i < 16; i++) w[i] = (float)(signed char)((qq[i >> 2] >> (8 * (i & 3))) & 0xFF) * scale;
         k0 = (u4 >> 1) * 32 + part * 16;
@@ -163,9 +198,16 @@ struct GQ80 {
 };
 
 struct GF16 {
-    __device__ static void deq16(const GemmArgs &a, size_t row, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+    static constexpr bool PRESCALED = false;
+    static constexpr float WS = 1.0f; // plain weights may be large: no headroom to give away
+    struct Raw { uint4 v0, v1; };
+    __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
         const uint4 *p = reinterpret_cast<const uint4 *>(a.codes + row * a.codes_pitch + ((size_t)kstep * 64 + u4 * 16) * 2);
-        const uint4 v0 = p[0], v1 = p[1];
+        r.v0 = p[0];
+        r.v1 = p[1];
+    }
+    __device__ static void cvt16(const Raw &r, int, int u4, float (&w)[16], int &k0, int &k1) {
+        const uint4 v0 = r.v0, v1 = r.v1;
         const uint32_t qq[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -178,11 +220,18 @@ struct GF16 {
 };
 
 struct GF32 {
-    __device__ static void deq16(const GemmArgs &a, size_t row, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+    static constexpr bool PRESCALED = false;
+    static constexpr float WS = 1.0f; // plain weights may be large: no headroom to give away
+    struct Raw { float4 v[4]; };
+    __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
         const float4 *p = reinterpret_cast<const float4 *>(a.codes + row * a.codes_pitch + ((size_t)kstep * 64 + u4 * 16) * 4);
 #pragma unroll
+        for (int i = 0; i < 4; i++) r.v[i] = p[i];
+    }
+    __device__ static void cvt16(const Raw &r, int, int u4, float (&w)[16], int &k0, int &k1) {
+#pragma unroll
         for (int i = 0; i < 4; i++) {
-            float4 v = p[i];
+            float4 v = r.v[i];
             w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
         }
         k0 = u4 * 16;
@@ -190,117 +239,160 @@ struct GF32 {
     }
 };
 
-__device__ inline uint32_t pack_h2(_Float16 a, _Float16 b) {
-    return (uint32_t)__builtin_bit_cast(unsigned short, a) | ((uint32_t)__builtin_bit_cast(unsigned short, b) << 16);
-}
-
-// w[0..7] -> eight f16 "high" parts and eight f16 remainders, as two 16-byte vectors
-__device__ inline void split8_f16(const float *w, uint4 &hi, uint4 &lo) {
+// Eight values times `scale` -> eight f16 high parts and eight f16 remainders, as
+// two 16-byte vectors.  The high part is the value with its mantissa cut to f16's eleven bits, a mask, exact in
+// f16; the remainder is exact in f32 and keeps its own top eleven bits.
+__device__ inline void split8_f16(const float *w, float scale, uint4 &hi, uint4 &lo) {
     uint32_t h[4], l[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        _Float16 h0 = (_Float16)w[2 * i], h1 = (_Float16)w[2 * i + 1];
-        _Float16 l0 = (_Float16)(w[2 * i] - (float)h0), l1 = (_Float16)(w[2 * i + 1] - (float)h1);
-        h[i] = pack_h2(h0, h1);
-        l[i] = pack_h2(l0, l1);
+        const float a = w[2 * i] * scale, b = w[2 * i + 1] * scale; // scale 1 folds away
+        const float ah = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, a) & 0xFFFFE000u);
+        const float bh = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, b) & 0xFFFFE000u);
+        h[i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(ah, bh));
+        l[i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a - ah, b - bh));
     }
     hi = make_uint4(h[0], h[1], h[2], h[3]);
     lo = make_uint4(l[0], l[1], l[2], l[3]);
 }
 
-template <class T, int BM>
-__global__ void __launch_bounds__(2 * BM) gemm_kernel(GemmArgs a) {
+// WM = 1 or 2: the workgroup computes (128 * WM) x 128 outputs with 4 * WM waves of two kinds.
+//   - 2 * WM "multiplier" waves each own a 128 x 64 block (4 x 2 MFMA tiles, 128 accumulator registers) and
+//     do nothing but read the current LDS stage and issue MFMAs;
+//   - 2 * WM "feeder" waves fetch the x tile and the packed weights of the step after next, convert the
+//     next step's weights (dequantise, split into two f16) and write the other LDS stage.
+// Waves are dealt to the four SIMDs in turn, so with WM = 2 every SIMD holds one wave of each kind and its
+// vector ALU converts while its matrix pipe multiplies; one barrier per K step hands the stages over.
+template <class T, int WM>
+__global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
+    constexpr int BM = 128 * WM, NTF = 128 * WM; // rows of x per tile; feeder threads
+    constexpr int XV = BM * 8 / NTF;             // 16-byte x vectors per feeder thread and K step (= 8)
+    constexpr int UNITS = BN * 4 / NTF;          // 16-weight units per feeder thread and K step (2 or 4)
+    constexpr int STAGE = (BM + 2 * BN) * LDK;   // halfs per LDS stage
     extern __shared__ _Float16 lds[];
-    _Float16 *As = lds;               // [BM][LDK]
-    _Float16 *Bh = As + BM * LDK;     // [BN][LDK]
-    _Float16 *Bl = Bh + BN * LDK;     // [BN][LDK]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int nthreads = 2 * BM;
-    const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
-    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64; // this wave's 64 x 64 block inside the tile
-    const int li = lane & 31, lk = (lane >> 5) * 8;
+    const bool feeder = tid >= NTF;
+    // Workgroups of one XCD (those with equal id modulo 8) take consecutive tiles, N fastest: the x tile is
+    // the big operand of a step (BM x 64 halfs against 128 x 64 packed weights), so the workgroups that share
+    // an x tile should share an L2.
+    const int nt = (a.n + BN - 1) / BN, total = (int)gridDim.x;
+    int tile = blockIdx.x;
+    if (total % 8 == 0) tile = (tile & 7) * (total >> 3) + (tile >> 3);
+    const int m0 = (tile / nt) * BM, n0 = (tile % nt) * BN;
+    const int ksteps = a.k / BK;
 
-    float16v acc[2][2];
+    if (feeder) {
+        const int ft = tid - NTF;
+        u32x4 xa[XV];
+        typename T::Raw raw[UNITS];
+        // row addresses do not change from step to step
+        const _Float16 *xrow[XV];
+        size_t wrow[UNITS];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+        for (int i = 0; i < XV; i++) {
+            int v = ft + i * NTF;
+            int gm = m0 + (v >> 3);
+            gm = gm < a.m ? gm : a.m - 1;
+            xrow[i] = a.xh + (size_t)gm * a.k + (v & 7) * 8;
+        }
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            int gn = n0 + ((ft + u * NTF) >> 2);
+            wrow[u] = (size_t)(gn < a.n ? gn : a.n - 1);
+        }
+        auto fetch = [&](int ks) { // clamped: past the last step the feeders re-read it and nobody looks
+            ks = ks < ksteps ? ks : ksteps - 1;
+#pragma unroll
+            for (int i = 0; i < XV; i++) xa[i] = *reinterpret_cast<const u32x4 *>(xrow[i] + (size_t)ks * BK);
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) T::load16(a, wrow[u], ks, (ft + u * NTF) & 3, raw[u]);
+        };
+        fetch(0);
+        for (int ks = 0; ks <= ksteps; ks++) {
+            // registers hold step ks: convert it into stage ks & 1, with step ks + 1 already requested
+            _Float16 *As = lds + (ks & 1) * STAGE, *Bh = As + BM * LDK, *Bl = Bh + BN * LDK;
+            const int kcur = ks < ksteps ? ks : ksteps - 1;
+            u32x4 xs[XV];
+            float w[UNITS][16];
+            int k0[UNITS], k1[UNITS];
+#pragma unroll
+            for (int i = 0; i < XV; i++) xs[i] = xa[i];
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) T::cvt16(raw[u], kcur, (ft + u * NTF) & 3, w[u], k0[u], k1[u]);
+            fetch(ks + 1);
+            if (ks < ksteps) {
+#pragma unroll
+                for (int i = 0; i < XV; i++) {
+                    int v = ft + i * NTF;
+                    int row = v >> 3, c = v & 7;
+                    *reinterpret_cast<u32x4 *>(As + row * LDK + c * 8) = xs[i];
+                }
+#pragma unroll
+                for (int u = 0; u < UNITS; u++) {
+                    int row = (ft + u * NTF) >> 2;
+                    uint4 h0, l0, h1, l1;
+                    split8_f16(w[u], T::PRESCALED ? 1.0f : T::WS, h0, l0);
+                    split8_f16(w[u] + 8, T::PRESCALED ? 1.0f : T::WS, h1, l1);
+                    *reinterpret_cast<uint4 *>(Bh + row * LDK + k0[u]) = h0;
+                    *reinterpret_cast<uint4 *>(Bh + row * LDK + k1[u]) = h1;
+                    *reinterpret_cast<uint4 *>(Bl + row * LDK + k0[u]) = l0;
+                    *reinterpret_cast<uint4 *>(Bl + row * LDK + k1[u]) = l1;
+                }
+            }
+            __syncthreads(); // barrier ks: stage ks & 1 is complete, stage (ks + 1) & 1 has been read
+        }
+        return;
+    }
+
+    const int wm = (wave >> 1) * 128, wn = (wave & 1) * 64; // this wave's block inside the tile
+    const int li = lane & 31, lk = (lane >> 5) * 8;
+    float16v acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-
-    const int ksteps = a.k / BK;
+    __syncthreads(); // barrier 0
     for (int ks = 0; ks < ksteps; ks++) {
-        // x tile: BM rows of 64 halfs = 8 vectors of 16 bytes per row
-        uint4 xa[4];
+        const _Float16 *As = lds + (ks & 1) * STAGE, *Bh = As + BM * LDK, *Bl = Bh + BN * LDK;
+        // fragments of sub-step kk + 1 are read from LDS while the sixteen MFMAs of sub-step kk run
+        half8 af[2][4], bh[2][2], bl[2][2];
+        auto read_frags = [&](int kk, int slot) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int v = tid + i * nthreads; // BM * 8 vectors in all = 4 per thread
-            int row = v >> 3, c = v & 7;
-            int gm = m0 + row;
-            gm = gm < a.m ? gm : a.m - 1;
-            xa[i] = *reinterpret_cast<const uint4 *>(a.xh + (size_t)gm * a.k + (size_t)ks * BK + c * 8);
-        }
-        // weight tile: 128 rows x 4 units of 16 weights
-        constexpr int UNITS = BN * 4 / (2 * BM); // per thread: 2 (BM = 128) or 1 (BM = 256)
-        uint4 wh[UNITS][2], wl[UNITS][2];
-        int wk0[UNITS], wk1[UNITS];
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            int unit = tid + u * nthreads;
-            int row = unit >> 2, u4 = unit & 3;
-            int gn = n0 + row;
-            gn = gn < a.n ? gn : a.n - 1;
-            float w[16];
-            T::deq16(a, (size_t)gn, ks, u4, w, wk0[u], wk1[u]);
-            split8_f16(w, wh[u][0], wl[u][0]);
-            split8_f16(w + 8, wh[u][1], wl[u][1]);
-        }
-        __syncthreads(); // the previous step's MFMAs have read the stage
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int v = tid + i * nthreads;
-            int row = v >> 3, c = v & 7;
-            *reinterpret_cast<uint4 *>(As + row * LDK + c * 8) = xa[i];
-        }
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            int unit = tid + u * nthreads;
-            int row = unit >> 2;
-            *reinterpret_cast<uint4 *>(Bh + row * LDK + wk0[u]) = wh[u][0];
-            *reinterpret_cast<uint4 *>(Bh + row * LDK + wk1[u]) = wh[u][1];
-            *reinterpret_cast<uint4 *>(Bl + row * LDK + wk0[u]) = wl[u][0];
-            *reinterpret_cast<uint4 *>(Bl + row * LDK + wk1[u]) = wl[u][1];
-        }
-        __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 16) {
-            half8 af[2], bh[2], bl[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) af[i] = *reinterpret_cast<const half8 *>(As + (wm + i * 32 + li) * LDK + kk + lk);
+            for (int i = 0; i < 4; i++) af[slot][i] = *reinterpret_cast<const half8 *>(As + (wm + i * 32 + li) * LDK + kk + lk);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                bh[j] = *reinterpret_cast<const half8 *>(Bh + (wn + j * 32 + li) * LDK + kk + lk);
-                bl[j] = *reinterpret_cast<const half8 *>(Bl + (wn + j * 32 + li) * LDK + kk + lk);
+                bh[slot][j] = *reinterpret_cast<const half8 *>(Bh + (wn + j * 32 + li) * LDK + kk + lk);
+                bl[slot][j] = *reinterpret_cast<const half8 *>(Bl + (wn + j * 32 + li) * LDK + kk + lk);
             }
+        };
+        read_frags(0, 0);
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+        for (int t = 0; t < BK / 16; t++) {
+            if (t + 1 < BK / 16) read_frags((t + 1) * 16, (t + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bl[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bh[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t & 1][i], bl[t & 1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t & 1][i], bh[t & 1][j], acc[i][j], 0, 0, 0);
                 }
+            __builtin_amdgcn_sched_barrier(0);
         }
+        __syncthreads(); // barrier ks + 1
     }
     // D layout: lane -> column li; register r -> row 8 * (r / 4) + 4 * (lane / 32) + r % 4
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int gn = n0 + wn + j * 32 + li;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int gm = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (gm < a.m && gn < a.n) a.y[(size_t)gm * a.n + gn] = acc[i][j][r] * a.rowscale[gm];
+                if (gm < a.m && gn < a.n) a.y[(size_t)gm * a.n + gn] = acc[i][j][r] * (a.rowscale[gm] * (1.0f / T::WS));
             }
         }
 }
@@ -337,16 +429,18 @@ __global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int
 template <class T>
 int launch_gemm(axq_ctx *ctx, const GemmArgs &a) {
     static bool attr_set = false;
-    const int bm = a.m > 128 ? 256 : 128;
-    dim3 grid((a.n + BN - 1) / BN, (a.m + bm - 1) / bm);
-    size_t lds = (size_t)(bm + 2 * BN) * LDK * sizeof(_Float16);
+    const int wm = a.m > 128 ? 2 : 1, bm = 128 * wm;
+    const unsigned grid = (unsigned)(((a.n + BN - 1) / BN) * ((a.m + bm - 1) / bm));
+    const size_t lds = (size_t)2 * (bm + 2 * BN) * LDK * sizeof(_Float16); // two stages
     if (!attr_set) {
-        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, 256>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)((256 + 2 * BN) * LDK * 2)), AXQ_ERR_DRIVER);
+        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, 2>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * (256 + 2 * BN) * LDK * 2)), AXQ_ERR_DRIVER);
+        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, 1>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * (128 + 2 * BN) * LDK * 2)), AXQ_ERR_DRIVER);
         attr_set = true;
     }
-    if (bm == 256) gemm_kernel<T, 256><<<grid, 512, lds, ctx->stream>>>(a);
-    else gemm_kernel<T, 128><<<grid, 256, lds, ctx->stream>>>(a);
+    if (wm == 2) gemm_kernel<T, 2><<<grid, 512, lds, ctx->stream>>>(a);
+    else gemm_kernel<T, 1><<<grid, 256, lds, ctx->stream>>>(a);
     AXQ_LAUNCH_CHECK(ctx, "gemm_kernel");
     return AXQ_OK;
 }
