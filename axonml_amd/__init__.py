@@ -13,6 +13,8 @@ from .quant import (  # noqa: F401
     QuantizedLinear,
     QuantizedTensor,
     QuantType,
+    compute_quantization_error,
+    compute_quantization_stats,
     default_context,
     dequantize_block,
     dequantize_tensor,

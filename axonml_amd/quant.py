@@ -387,6 +387,27 @@ def compute_quantization_error(original, dequantized):
     return float(np.sqrt(np.float32(np.sum(d * d, dtype=np.float32)) / np.float32(a.size)))
 
 
+class QuantizationStats:
+    """rmse, max_error, mean_error, compression_ratio (quantize.rs:251-261)."""
+
+    def __init__(self, rmse, max_error, mean_error, compression_ratio):
+        self.rmse, self.max_error, self.mean_error, self.compression_ratio = rmse, max_error, mean_error, compression_ratio
+
+
+def compute_quantization_stats(original, dequantized, quant_type):
+    """quantize.rs:264-284: error statistics in f32 over the zipped pairs."""
+    a = np.asarray(original, dtype=np.float32).reshape(-1)
+    b = np.asarray(dequantized, dtype=np.float32).reshape(-1)
+    n = min(a.size, b.size)
+    err = np.abs(a[:n] - b[:n])
+    cnt = np.float32(n)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        mse = np.sum(err * err, dtype=np.float32) / cnt
+        mean = np.sum(err, dtype=np.float32) / cnt
+    return QuantizationStats(float(np.sqrt(mse)), float(err.max()) if n else 0.0, float(mean),
+                             QuantType(quant_type).compression_ratio())
+
+
 def f32_to_bf16_bits(x):
     """Round-to-nearest-even f32 -> bf16 bit patterns (uint16)."""
     u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
