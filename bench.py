@@ -166,6 +166,49 @@ def measured_traffic():
     return None
 
 
+def cpu_decode_baseline(budget_tokens=8):
+    """Same-run host figure for the 7B-shape decode: the CPU decode oracle (f32 weights dequantised once, all
+    threads in the matrix-vector products) on a TWO-layer slice of the Mistral-7B shape plus the full lm_head,
+    timed per token at a short context and EXTRAPOLATED to 32 layers by the f32 weight bytes a token streams
+    (the host path is memory-bound): t_32 = t_2 * bytes_32 / bytes_2.  A full 32-layer f32 model (28 GB) is not
+    practical to build and time inside the benchmark."""
+    import oracle as o
+
+    H, I, V, NH, NKV, D = 4096, 14336, 32000, 32, 8, 128
+    rng = np.random.default_rng(7)
+
+    def packed(n, k):
+        nsb = n * k // 256
+        b = rng.integers(0, 256, size=(nsb, 144), dtype=np.uint8)
+        b[:, 0:2] = np.frombuffer(np.float16(8e-4).tobytes(), np.uint8)
+        b[:, 2:4] = np.frombuffer(np.float16(6e-3).tobytes(), np.uint8)
+        return b.reshape(-1)
+
+    layers = 2
+    m = o.DecodeModel(vocab_size=V, hidden_size=H, intermediate_size=I, num_layers=layers, num_heads=NH,
+                      num_kv_heads=NKV, head_dim=D, max_seq_len=16, rms_norm_eps=1e-5, rope_theta=10000.0)
+    m.set_embedding_f16((rng.standard_normal((V, H)) * 0.02).astype(np.float16).view(np.uint16))
+    shapes = {"q": (H, H), "k": (NKV * D, H), "v": (NKV * D, H), "o": (H, H), "gate": (I, H), "up": (I, H), "down": (H, I)}
+    for layer in range(layers):
+        for name, (n, k) in shapes.items():
+            m.set_linear(layer, o.DecodeModel.LIN[name], o.Q4_K, packed(n, k))
+    m.set_linear(-1, 0, o.Q4_K, packed(V, H))
+    m.forward(1, 0, want_logits=False)  # first touch
+    times = []
+    for pos in range(1, 1 + budget_tokens):
+        t0 = time.perf_counter()
+        m.forward(pos, pos, want_logits=False)
+        times.append(time.perf_counter() - t0)
+    m.close()
+    t2 = float(np.median(times))
+    per_layer = 2 * H * H + 2 * NKV * D * H + 3 * I * H
+    scale = (32 * per_layer + V * H) / (layers * per_layer + V * H)
+    t32 = t2 * scale
+    return {"tokens_per_s": 1.0 / t32, "ms_per_token": t32 * 1e3, "kind": "port, extrapolated from a 2-layer slice",
+            "cores": int(o.lib().axo_num_threads()), "ms_per_token_2_layers_plus_head": t2 * 1e3, "extrapolation_factor": scale,
+            "sample": f"median of {budget_tokens} tokens on a 2-layer model of the Mistral-7B shape with the full lm_head, context < 16"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -224,6 +267,9 @@ def main():
             from axonml_amd import decode as d
 
             extra["decode"] = d.bench_7b(ctx, log)
+            if not args.no_cpu:
+                extra["decode"]["cpu_baseline"] = cpu_decode_baseline()
+                log(f"  decode cpu baseline (extrapolated): {extra['decode']['cpu_baseline']['tokens_per_s']:.2f} tok/s")
         except ImportError:
             pass
         try:
