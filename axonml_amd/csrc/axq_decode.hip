@@ -349,21 +349,19 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, co
     }
 }
 
-// act = silu(gate) * up over [inter]; gu = [gate (inter) | up (inter)].
+// act = silu(gate) * up over [inter]; gu alternates four gate values with the four up values of the same indices
+// (the row order of the fused gate/up weight).
 __global__ void __launch_bounds__(256) swiglu_kernel(const float *gu, int inter, float *act) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= (inter >> 3)) return;
-    const float4 *pg = reinterpret_cast<const float4 *>(gu + (size_t)t * 8);
-    const float4 *pu = reinterpret_cast<const float4 *>(gu + inter + (size_t)t * 8);
-    float4 ga = pg[0], gb = pg[1], ua = pu[0], ub = pu[1];
-    const float g[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
-    const float u[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
-    float v[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = (g[i] * (1.0f / (1.0f + expf(-g[i])))) * u[i];
-    float4 *o = reinterpret_cast<float4 *>(act + (size_t)t * 8);
-    o[0] = make_float4(v[0], v[1], v[2], v[3]);
-    o[1] = make_float4(v[4], v[5], v[6], v[7]);
+    const int t = blockIdx.x * blockDim.x + threadIdx.x; // four consecutive outputs
+    if (t >= (inter >> 2)) return;
+    const float4 g = *reinterpret_cast<const float4 *>(gu + (size_t)t * 8);
+    const float4 u = *reinterpret_cast<const float4 *>(gu + (size_t)t * 8 + 4);
+    float4 o;
+    o.x = (g.x * (1.0f / (1.0f + expf(-g.x)))) * u.x;
+    o.y = (g.y * (1.0f / (1.0f + expf(-g.y)))) * u.y;
+    o.z = (g.z * (1.0f / (1.0f + expf(-g.z)))) * u.z;
+    o.w = (g.w * (1.0f / (1.0f + expf(-g.w)))) * u.w;
+    *reinterpret_cast<float4 *>(act + (size_t)t * 4) = o;
 }
 
 // argmax over the logits, last index among equal maxima (Iterator::max_by); then pos += 1.
@@ -438,6 +436,20 @@ int copy_rows(axq_ctx *ctx, axq_weight *dst, const axq_weight *src, int64_t row_
     return AXQ_OK;
 }
 
+// Rows of `src` into every other group of four rows of `dst`, starting at group `first` (0 or 1): the fused
+// gate/up weight alternates four gate rows with the four up rows of the same indices, so that a GEMV
+// workgroup holds both halves of every pair it needs for silu(gate) * up.
+int copy_rows_interleaved(axq_ctx *ctx, axq_weight *dst, const axq_weight *src, int first) {
+    struct { uint8_t *d; const uint8_t *s; size_t pitch; } planes[3] = {
+        {dst->codes, src->codes, src->codes_pitch}, {dst->meta, src->meta, src->meta_pitch}, {dst->qh, src->qh, src->qh_pitch}};
+    for (auto &p : planes) {
+        if (p.pitch == 0) continue;
+        AXQ_HIP(ctx, hipMemcpy2DAsync(p.d + (size_t)first * 4 * p.pitch, 8 * p.pitch, p.s, 4 * p.pitch, 4 * p.pitch,
+                                      (size_t)src->n_rows / 4, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    }
+    return AXQ_OK;
+}
+
 template <int D, int REP>
 void launch_attn_partial_t(axq_model *m, int l, hipStream_t st) {
     const axq_model_config &c = m->cfg;
@@ -465,23 +477,27 @@ void launch_attn_partial(axq_model *m, int l, hipStream_t st) {
     }
 }
 
-// y = W f(x) (+ bias), f = identity, RMSNorm with weights `aux`, or SwiGLU with `aux` as the `up` vector.
-// The matrix-pipe GEMV applies f while it stages x; for a linear it does not cover (other weight types,
-// K not a multiple of 64 or beyond 16384) f runs as a kernel of its own into `tmp` and the f32 GEMV follows.
-int linear(axq_model *m, const axq_weight *w, const float *x, int mode, const float *aux, float *tmp, const float *bias,
-           float *y) {
+// y = g(W f(x) (+ bias)): f = identity or RMSNorm with weights `aux`; g = identity, or, for the fused gate/up
+// weight, silu(gate) * up over its row pairs (y then has half as many entries as W has rows).  The matrix-pipe
+// GEMV applies f while it stages x and g while it writes y; for a linear it does not cover (other weight types,
+// K not a multiple of 64 or beyond 16384) f and g run as kernels of their own around the f32 GEMV, through `tmp`.
+int linear(axq_model *m, const axq_weight *w, const float *x, int xmode, const float *aux, int ymode, float *tmp,
+           const float *bias, float *y) {
     axq_ctx *ctx = m->ctx;
     if (axq_dev_gemv_dp_covers(w)) {
-        int rc = axq_dev_gemv_dp_ex(ctx, w, x, nullptr, mode, aux, m->cfg.rms_norm_eps, bias, y);
+        int rc = axq_dev_gemv_dp_ex(ctx, w, x, nullptr, xmode, aux, m->cfg.rms_norm_eps, ymode, bias, y);
         return rc < 0 ? rc : AXQ_OK;
     }
-    const int k = (int)w->k;
-    if (mode == AXQ_X_RMSNORM) {
+    const int k = (int)w->k, n = (int)w->n_rows;
+    if (xmode == AXQ_X_RMSNORM) {
         norm_kernel<<<1, 1024, 0, ctx->stream>>>(x, aux, k, m->cfg.rms_norm_eps, tmp);
         x = tmp;
-    } else if (mode == AXQ_X_SWIGLU) {
-        swiglu_kernel<<<(k / 8 + 255) / 256, 256, 0, ctx->stream>>>(x, k, tmp); // x = [gate | up]
-        x = tmp;
+    }
+    if (ymode == AXQ_Y_SWIGLU) {
+        int rc = axq_dev_gemv(ctx, w, x, 1, bias, m->gu);
+        if (rc) return rc;
+        swiglu_kernel<<<(n / 8 + 255) / 256, 256, 0, ctx->stream>>>(m->gu, n / 2, y);
+        return AXQ_OK;
     }
     return axq_dev_gemv(ctx, w, x, 1, bias, y);
 }
@@ -492,21 +508,23 @@ int enqueue_step(axq_model *m) {
     axq_ctx *ctx = m->ctx;
     const axq_model_config &c = m->cfg;
     hipStream_t st = ctx->stream;
-    const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim;
+    const int H = c.hidden_size, d = c.head_dim;
     const size_t comb_lds = (size_t)(m->max_splits + 8) * sizeof(float);
     int rc;
     embed_kernel<<<(H / 8 + 255) / 256, 256, 0, st>>>(m->emb, m->tok, m->h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
-        if ((rc = linear(m, m->w_qkv[l], m->h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, m->xn, nullptr, m->qkv))) return rc;
+        if ((rc = linear(m, m->w_qkv[l], m->h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, AXQ_Y_PLAIN, m->xn, nullptr, m->qkv)))
+            return rc;
         launch_attn_partial(m, l, st);
         attn_combine_kernel<<<c.num_attention_heads, 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
                                                                           c.num_key_value_heads, d, m->max_splits, m->att);
         // residual adds go through the bias slot, in place
-        if ((rc = linear(m, m->w_o[l], m->att, AXQ_X_PLAIN, nullptr, nullptr, m->h, m->h))) return rc;
-        if ((rc = linear(m, m->w_gu[l], m->h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, m->xn, nullptr, m->gu))) return rc;
-        if ((rc = linear(m, m->w_down[l], m->gu, AXQ_X_SWIGLU, m->gu + I, m->act, m->h, m->h))) return rc;
+        if ((rc = linear(m, m->w_o[l], m->att, AXQ_X_PLAIN, nullptr, AXQ_Y_PLAIN, nullptr, m->h, m->h))) return rc;
+        if ((rc = linear(m, m->w_gu[l], m->h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, AXQ_Y_SWIGLU, m->xn, nullptr, m->act)))
+            return rc;
+        if ((rc = linear(m, m->w_down[l], m->act, AXQ_X_PLAIN, nullptr, AXQ_Y_PLAIN, nullptr, m->h, m->h))) return rc;
     }
-    if ((rc = linear(m, m->w_head, m->h, AXQ_X_RMSNORM, m->norm_final, m->xn, nullptr, m->logits))) return rc;
+    if ((rc = linear(m, m->w_head, m->h, AXQ_X_RMSNORM, m->norm_final, AXQ_Y_PLAIN, m->xn, nullptr, m->logits))) return rc;
     argmax_kernel<<<1, 1024, 0, st>>>(m->logits, c.vocab_size, m->next, m->pos);
     AXQ_LAUNCH_CHECK(ctx, "decode step");
     return AXQ_OK;
@@ -713,7 +731,8 @@ int axq_model_set_linear(axq_model *m, int layer, int which, const axq_weight *w
     if ((*slot)->type != w->type)
         return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: fused weight holds %s, got %s",
                         axq_type_name((*slot)->type), axq_type_name(w->type));
-    if ((rc = copy_rows(ctx, *slot, w, row_off))) return rc;
+    const bool pair = layer >= 0 && (which == AXQ_LIN_GATE || which == AXQ_LIN_UP);
+    if ((rc = pair ? copy_rows_interleaved(ctx, *slot, w, which == AXQ_LIN_UP) : copy_rows(ctx, *slot, w, row_off))) return rc;
     AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
     if (layer < 0) m->head_set = true; else m->set_mask[layer] |= 1u << which;
     return AXQ_OK;

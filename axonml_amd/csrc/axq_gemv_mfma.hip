@@ -46,9 +46,10 @@ struct DpArgs {
     int n_rows, k;
     int S, G, P;   // K slices per pass, row groups per workgroup, passes over K per lane
     int steps;     // 4-row steps per group
-    int mode;      // what x is: AXQ_X_PLAIN, or a vector still to be normalised / gated (see axq_internal.h)
-    const float *aux; // AXQ_X_RMSNORM: the norm weights; AXQ_X_SWIGLU: the `up` vector (x is `gate`)
+    int mode;      // what x is: AXQ_X_PLAIN, or a vector still to be normalised (see axq_internal.h)
+    const float *aux; // AXQ_X_RMSNORM: the norm weights
     float eps;
+    int ymode;     // AXQ_Y_PLAIN or AXQ_Y_SWIGLU
 };
 
 __device__ inline float f16lo(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v & 0xFFFF))); }
@@ -467,15 +468,6 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
                 xv[0][i] = (xv[0][i] * inv) * ev[0][i];
                 xv[1][i] = (xv[1][i] * inv) * ev[1][i];
             }
-        } else if (a.mode == AXQ_X_SWIGLU) {
-            // LLaMAMLP::forward (llm/src/llama.rs:562-567): silu(gate) * up, silu(v) = v * 1 / (1 + exp(-v))
-            unpack(e0, e1, ev[0]);
-            unpack(e2, e3, ev[1]);
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                xv[0][i] = (xv[0][i] * (1.0f / (1.0f + expf(-xv[0][i])))) * ev[0][i];
-                xv[1][i] = (xv[1][i] * (1.0f / (1.0f + expf(-xv[1][i])))) * ev[1][i];
-            }
         }
         if (live0) axq_split8(xv[0], tid, true, wplanes, wgrp, kpad);
         if (live1) axq_split8(xv[1], tid + nthreads, true, wplanes, wgrp, kpad);
@@ -509,15 +501,31 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     // partial sums -> y, in a fixed order
     __syncthreads();
     const int wg_rows = a.G * rows_per_group;
-    for (int t = tid; t < wg_rows; t += (int)blockDim.x) {
+    auto row_total = [&](int t) { // slice by slice, the four DPP rows of each in order
+        const float4 *pr = reinterpret_cast<const float4 *>(red + (size_t)t * red_stride);
+        float tot = 0.f;
+        for (int s = 0; s < a.S; s++) {
+            float4 v = pr[s];
+            tot += (v.x + v.y) + (v.z + v.w);
+        }
+        return tot;
+    };
+    if (a.ymode == AXQ_Y_SWIGLU) {
+        // rows 8b..8b+3 are gate rows, 8b+4..8b+7 the up rows of the same outputs (wg_rows is a multiple of 8)
+        for (int t = tid; t < (wg_rows >> 1); t += nthreads) {
+            const int lg = ((t >> 2) << 3) + (t & 3);
+            const int row = blockIdx.x * wg_rows + lg;
+            if (row + 4 < a.n_rows) {
+                const float g = row_total(lg), u = row_total(lg + 4);
+                a.y[(blockIdx.x * wg_rows >> 1) + t] = (g * (1.0f / (1.0f + expf(-g)))) * u;
+            }
+        }
+        return;
+    }
+    for (int t = tid; t < wg_rows; t += nthreads) {
         int row = blockIdx.x * wg_rows + t;
         if (row < a.n_rows) {
-            const float4 *pr = reinterpret_cast<const float4 *>(red + (size_t)t * red_stride);
-            float tot = 0.f;
-            for (int s = 0; s < a.S; s++) { // slice by slice, the four DPP rows of each in order
-                float4 v = pr[s];
-                tot += (v.x + v.y) + (v.z + v.w);
-            }
+            const float tot = row_total(t);
             a.y[row] = a.bias ? tot + a.bias[row] : tot;
         }
     }
@@ -556,13 +564,13 @@ void launch_nb(axq_ctx *ctx, const DpArgs &a, int nb, unsigned grid, unsigned bl
 
 template <class T>
 bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux, float eps,
-               const float *bias, float *y) {
+               int ymode, const float *bias, float *y) {
     if (w->k % 64 != 0 || w->k > 16384) return false;
     DpArgs a;
     a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
     a.x = x; a.xq = xq; a.bias = bias; a.y = y;
-    a.mode = mode; a.aux = aux; a.eps = eps;
+    a.mode = mode; a.aux = aux; a.eps = eps; a.ymode = ymode;
     a.n_rows = (int)w->n_rows;
     a.k = (int)w->k;
     a.S = (a.k + 1023) / 1024;            // waves that span K once (<= 16)
@@ -576,6 +584,7 @@ bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t 
     int wgs = cus * ctx->gemv_wgs_per_cu;
     int steps = (rowsteps + wgs * a.G - 1) / (wgs * a.G);
     if (steps > 64) steps = 64;
+    if (ymode == AXQ_Y_SWIGLU && ((a.G * steps) & 1)) steps++; // a workgroup must hold whole gate/up groups of 8 rows
     a.steps = steps;
     int nb = block > 512 ? T::BIG_NB : 8;
     if (nb > ctx->gemv_max_nb) nb = ctx->gemv_max_nb;
@@ -607,16 +616,18 @@ int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq) {
 // back to the vector-ALU kernels), or a negative status.  xq = NULL: the kernel splits x itself, after
 // applying the prologue `mode` (axq_internal.h) with its second operand `aux`.
 int axq_dev_gemv_dp_ex(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux,
-                       float eps, const float *bias, float *y) {
+                       float eps, int ymode, const float *bias, float *y) {
     bool ok;
     if (xq && mode != AXQ_X_PLAIN) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "a fused prologue needs the raw x");
+    if (ymode == AXQ_Y_SWIGLU && (w->n_rows % 8 != 0 || bias))
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "the SwiGLU epilogue needs whole groups of 8 rows and no bias");
     switch (w->type) {
-    case AXQ_Q4_K: ok = launch_dp<DQ4K>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
-    case AXQ_Q4_0: ok = launch_dp<DQ4x<false>>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
-    case AXQ_Q4_1: ok = launch_dp<DQ4x<true>>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
-    case AXQ_Q5_0: ok = launch_dp<DQ5x<false>>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
-    case AXQ_Q5_1: ok = launch_dp<DQ5x<true>>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
-    case AXQ_Q8_0: ok = launch_dp<DQ80>(ctx, w, x, xq, mode, aux, eps, bias, y); break;
+    case AXQ_Q4_K: ok = launch_dp<DQ4K>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
+    case AXQ_Q4_0: ok = launch_dp<DQ4x<false>>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
+    case AXQ_Q4_1: ok = launch_dp<DQ4x<true>>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
+    case AXQ_Q5_0: ok = launch_dp<DQ5x<false>>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
+    case AXQ_Q5_1: ok = launch_dp<DQ5x<true>>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
+    case AXQ_Q8_0: ok = launch_dp<DQ80>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
     default: return 0;
     }
     if (!ok) return 0;
@@ -625,7 +636,7 @@ int axq_dev_gemv_dp_ex(axq_ctx *ctx, const axq_weight *w, const float *x, const 
 }
 
 int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y) {
-    return axq_dev_gemv_dp_ex(ctx, w, x, xq, AXQ_X_PLAIN, nullptr, 0.f, bias, y);
+    return axq_dev_gemv_dp_ex(ctx, w, x, xq, AXQ_X_PLAIN, nullptr, 0.f, AXQ_Y_PLAIN, bias, y);
 }
 
 // Whether axq_dev_gemv_dp_ex covers a weight of this type and width.

@@ -100,10 +100,13 @@ int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x_dev, int batc
 int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y);
 // What the GEMV does to x before it uses it (xq must be NULL for the fused forms):
 enum { AXQ_X_PLAIN = 0,    // nothing
-       AXQ_X_RMSNORM = 1,  // x <- x / sqrt(mean(x^2) + eps) * aux   (aux = norm weights, K floats)
-       AXQ_X_SWIGLU = 2 }; // x <- silu(x) * aux                      (x = gate, aux = up, K floats each)
+       AXQ_X_RMSNORM = 1 }; // x <- x / sqrt(mean(x^2) + eps) * aux   (aux = norm weights, K floats)
+// ... and to its result before it writes it:
+enum { AXQ_Y_PLAIN = 0,    // y[row] = dot (+ bias[row])
+       AXQ_Y_SWIGLU = 1 }; // rows come in groups of four "gate" rows followed by their four "up" rows:
+                           // y[i] = silu(gate_i) * up_i, half as many outputs as rows (no bias)
 int axq_dev_gemv_dp_ex(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux,
-                       float eps, const float *bias, float *y);
+                       float eps, int ymode, const float *bias, float *y);
 bool axq_dev_gemv_dp_covers(const axq_weight *w);
 size_t axq_xq_bytes(int64_t k);
 int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq);
