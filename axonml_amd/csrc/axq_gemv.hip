@@ -565,6 +565,15 @@ int launch(axq_ctx *ctx, const axq_weight *w, const float *x, const float *bias,
 int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y) {
     if (w->n_rows > INT32_MAX || w->k > INT32_MAX)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
+    // small batches: eight vectors at a time against one pass over the weights, where that kernel applies
+    while (batch >= 2 && axq_dev_gemv_batch_covers(w, batch < 8 ? batch : 8)) {
+        const int nb = batch < 8 ? batch : 8;
+        int rc = axq_dev_gemv_batch(ctx, w, x, nb, bias, y);
+        if (rc) return rc;
+        x += (size_t)nb * (size_t)w->k;
+        y += (size_t)nb * (size_t)w->n_rows;
+        batch -= nb;
+    }
     for (int b = 0; b < batch; b++) {
         const float *xb = x + (size_t)b * (size_t)w->k;
         float *yb = y + (size_t)b * (size_t)w->n_rows;

@@ -1,0 +1,311 @@
+// Decode-path quantized matmul for a small batch (2..8 activation vectors): y[b, n] = sum_k x[b, k] W[n, k].
+//
+// The weights are read once for the whole batch.  The dot products run on v_mfma_i32_32x32x32_i8 with
+//   A (32 x 32): row 4 b + l = limb l of activation vector b (the split form of axq_split.h), 32 k of one block,
+//   B (32 x 32): column n = one of 32 weight rows, the block's 32 codes as signed bytes,
+// so one instruction multiplies a 32-element block of 32 weight rows with all vectors and limbs.  Lane
+// (n, h) = (lane % 32, lane / 32) supplies 16 of the block's codes of row n and receives D[4 b + l][n] for
+// b = h, h + 2, h + 4, h + 6: all four limbs of four vectors, which it recombines and scales by itself.
+//
+// A workgroup owns 32 weight rows; its S = K / 512 <= 8 waves split K (16 blocks each) and keep their A operands
+// in registers; the partial sums of the waves meet in LDS and are added in a fixed order.  The split form of
+// the batch is made once, by a small kernel in front (a workgroup could not afford to split eight vectors
+// for its 32 rows).
+#include <hip/hip_fp16.h>
+
+#include "axq_internal.h"
+#include "axq_split.h"
+
+namespace {
+
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int UNITS = 16;      // 32-element blocks per wave
+constexpr int WAVE_K = 32 * UNITS;
+constexpr int MAX_BATCH = 8;
+
+struct MbArgs {
+    const uint8_t *codes, *meta;
+    size_t codes_pitch, meta_pitch;
+    const uint8_t *xa;  // the batch's limbs as MFMA A operands: [block][h][row 4 b + l] x 16 bytes (pack_x_kernel)
+    const float *xsg;   // [block][h][4]: group scales of vectors h, h + 2, h + 4, h + 6; then the plain sums, same layout
+    const float *bias;
+    float *y;
+    int n_rows, k, batch;
+};
+
+__device__ inline float f16lo(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v & 0xFFFF))); }
+__device__ inline float f16hi(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v >> 16))); }
+// four unsigned nibble codes in the low nibbles of the four bytes -> four signed bytes (code - 8)
+__device__ inline int minus8(uint32_t t) { return (int)((((t | 0x80808080u) - 0x08080808u)) ^ 0x80808080u); }
+__device__ inline u32x4 ldg16(const uint8_t *p) { return *reinterpret_cast<const u32x4 *>(p); }
+
+// sum_k n_k x_k over one 32-element block of one vector from its four limb sums (limb 0 most significant)
+__device__ inline float recombine4(int d0, int d1, int d2, int d3) {
+    float f = fmaf((float)d0, 128.0f, (float)d1);
+    f = fmaf(f, 128.0f, (float)d2);
+    return fmaf(f, 128.0f, (float)d3);
+}
+
+// ---------------------------------------------------------------------------
+// Per-type traits.  `u` counts the wave's blocks 0..15, `blk0` is the wave's first block in the row,
+// h = lane / 32 says which 16 of a block's 32 codes the lane supplies.
+//   EVEN_ODD : h = 0 supplies the even elements, h = 1 the odd ones (reference nibble order); otherwise
+//              h = 0 supplies elements 0..15, h = 1 elements 16..31
+//   coef()   : w = d * (code - CENTRE) + mo, CENTRE = 8 for the 4-bit types
+// ---------------------------------------------------------------------------
+template <bool WITH_MIN>
+struct MQ4x {
+    static constexpr bool EVEN_ODD = true;
+    static constexpr bool OFFSET = WITH_MIN;
+    struct Raw { u32x4 q[UNITS]; u32x4 m[WITH_MIN ? 4 : 2]; };
+    __device__ static void load(const MbArgs &a, size_t row, int blk0, int, Raw &r) {
+        const uint8_t *codes = a.codes + row * a.codes_pitch + (size_t)blk0 * 16;
+        const uint8_t *meta = a.meta + row * a.meta_pitch + (size_t)blk0 * (WITH_MIN ? 4 : 2);
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) r.q[u] = ldg16(codes + u * 16);
+#pragma unroll
+        for (int i = 0; i < (WITH_MIN ? 4 : 2); i++) r.m[i] = ldg16(meta + i * 16);
+    }
+    __device__ static int4v operand(const Raw &r, int u, int h) {
+        const int sh = 4 * h;
+        int4v b;
+#pragma unroll
+        for (int i = 0; i < 4; i++) b[i] = minus8((r.q[u][i] >> sh) & 0x0F0F0F0Fu);
+        return b;
+    }
+    __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
+        if (WITH_MIN) {
+            const uint32_t v = r.m[u >> 2][u & 3];
+            d = f16lo(v);
+            mo = fmaf(8.0f, d, f16hi(v));
+        } else {
+            const uint32_t v = r.m[u >> 3][(u >> 1) & 3];
+            d = (u & 1) ? f16hi(v) : f16lo(v);
+            mo = 0.f;
+        }
+    }
+};
+
+struct MQ80 {
+    static constexpr bool EVEN_ODD = false;
+    static constexpr bool OFFSET = false;
+    struct Raw { u32x4 q[UNITS]; u32x4 m[2]; };
+    __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, Raw &r) {
+        const uint8_t *codes = a.codes + row * a.codes_pitch + (size_t)blk0 * 32 + h * 16;
+        const uint8_t *meta = a.meta + row * a.meta_pitch + (size_t)blk0 * 2;
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) r.q[u] = ldg16(codes + u * 32);
+        r.m[0] = ldg16(meta);
+        r.m[1] = ldg16(meta + 16);
+    }
+    __device__ static int4v operand(const Raw &r, int u, int) {
+        int4v b = {(int)r.q[u][0], (int)r.q[u][1], (int)r.q[u][2], (int)r.q[u][3]};
+        return b;
+    }
+    __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
+        const uint32_t v = r.m[u >> 3][(u >> 1) & 3];
+        d = (u & 1) ? f16hi(v) : f16lo(v);
+        mo = 0.f;
+    }
+};
+
+// Q4_K: a block is a sub-block; the lane's 16-byte piece of pair p (first half for h = 0, second for h = 1)
+// holds its codes of sub-block 2p in the low nibbles and of sub-block 2p + 1 in the high ones.
+struct MQ4K {
+    static constexpr bool EVEN_ODD = false;
+    static constexpr bool OFFSET = true;
+    struct Raw { u32x4 q[UNITS / 2]; u32x4 h[UNITS / 8]; };
+    __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, Raw &r) {
+        const int cpr = a.k >> 6;          // pairs per row
+        const int pair0 = blk0 >> 1;       // the wave's first pair; 8 pairs = 2 superblocks, inside one 64-pair slice
+        const int slice = pair0 >> 6, pr = pair0 & 63;
+        int P = cpr - (slice << 6);
+        P = P < 64 ? P : 64;
+        const uint8_t *codes = a.codes + row * a.codes_pitch + (size_t)slice * 2048 + (size_t)h * 16 * P + (size_t)pr * 16;
+        const uint8_t *meta = a.meta + row * a.meta_pitch + (size_t)(pair0 >> 2) * 16;
+#pragma unroll
+        for (int p = 0; p < UNITS / 2; p++) r.q[p] = ldg16(codes + p * 16);
+#pragma unroll
+        for (int s = 0; s < UNITS / 8; s++) r.h[s] = ldg16(meta + s * 16);
+    }
+    __device__ static int4v operand(const Raw &r, int u, int) {
+        const int sh = 4 * (u & 1);
+        int4v b;
+#pragma unroll
+        for (int i = 0; i < 4; i++) b[i] = minus8((r.q[u >> 1][i] >> sh) & 0x0F0F0F0Fu);
+        return b;
+    }
+    __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
+        // 6-bit scale and min of sub-block j = u % 8 of superblock u / 8 (ggml get_scale_min_k4 order)
+        const u32x4 h = r.h[u >> 3];
+        const int j = u & 7;
+        const uint32_t sc_lo = (j & 4) ? h[3] : h[1], mn_lo = (j & 4) ? h[3] : h[2];
+        const int sh = 8 * (j & 3);
+        uint32_t sc, mn;
+        if (j < 4) {
+            sc = (h[1] >> sh) & 63;
+            mn = (h[2] >> sh) & 63;
+        } else {
+            sc = ((sc_lo >> sh) & 0xF) | (((h[1] >> sh) >> 6 & 3) << 4);
+            mn = ((mn_lo >> sh) >> 4 & 0xF) | (((h[2] >> sh) >> 6 & 3) << 4);
+        }
+        const float dd = f16lo(h[0]), dmin = f16hi(h[0]);
+        d = dd * (float)sc;
+        mo = fmaf(8.0f, d, -(dmin * (float)mn));
+    }
+};
+
+// bytes {0, 2} of lo and of hi (sel = 0) or bytes {1, 3} of each (sel = 1)
+__device__ inline int pick_alt(uint32_t lo, uint32_t hi, int sel) {
+    return (int)__builtin_amdgcn_perm(hi, lo, sel ? 0x07050301u : 0x06040200u);
+}
+
+template <class T>
+__global__ void __launch_bounds__(512) gemv_mb_kernel(MbArgs a) {
+    extern __shared__ float lds_f[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int S = (int)blockDim.x >> 6;
+    const int n = lane & 31, h = lane >> 5;
+    const int nblk = a.k >> 5;
+    float *sgs = lds_f;                    // [block of the row][h][4]: group scales of vectors h, h+2, h+4, h+6
+    float *xss = sgs + (size_t)nblk * 8;   // same layout: plain sums of x over the group (contiguous with sgs)
+    float *red = xss + (size_t)nblk * 8;   // [wave][vector][row]
+
+    // 1. this lane's A operands for the wave's 16 blocks: one contiguous kilobyte per wave and block
+    int4v A[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) {
+        const u32x4 v = ldg16(a.xa + ((size_t)((wave * UNITS + u) * 2 + h) * 32 + n) * 16);
+        A[u] = int4v{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
+    }
+    // scales and sums of all vectors -> LDS (already in the order the lanes read them)
+    for (int t = tid; t < nblk * 4; t += (int)blockDim.x)
+        reinterpret_cast<float4 *>(lds_f)[t] = reinterpret_cast<const float4 *>(a.xsg)[t];
+    // 2. the weights of this wave: 32 rows x 16 blocks, all requested at once
+    const int row0 = blockIdx.x * 32;
+    int row = row0 + n;
+    row = row < a.n_rows ? row : a.n_rows - 1;
+    typename T::Raw raw;
+    T::load(a, (size_t)row, wave * UNITS, h, raw);
+    __syncthreads();
+
+    // 3. one MFMA per block; the lane scales and adds its four vectors
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) {
+        const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        const int16v D = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[u], T::operand(raw, u, h), zero, 0, 0, 0);
+        float d, mo;
+        T::coef(raw, u, d, mo);
+        const int g = wave * UNITS + u;
+        const float4 sg4 = *reinterpret_cast<const float4 *>(sgs + (size_t)(g * 2 + h) * 4);
+        const float sgv[4] = {sg4.x, sg4.y, sg4.z, sg4.w};
+#pragma unroll
+        for (int bi = 0; bi < 4; bi++)
+            acc[bi] = fmaf(d * sgv[bi], recombine4(D[4 * bi], D[4 * bi + 1], D[4 * bi + 2], D[4 * bi + 3]), acc[bi]);
+        if (T::OFFSET) {
+            const float4 xs4 = *reinterpret_cast<const float4 *>(xss + (size_t)(g * 2 + h) * 4);
+            acc[0] = fmaf(mo, xs4.x, acc[0]); acc[1] = fmaf(mo, xs4.y, acc[1]);
+            acc[2] = fmaf(mo, xs4.z, acc[2]); acc[3] = fmaf(mo, xs4.w, acc[3]);
+        }
+    }
+    // 4. partial sums of the waves -> y, in wave order
+#pragma unroll
+    for (int bi = 0; bi < 4; bi++) red[((size_t)wave * MAX_BATCH + (2 * bi + h)) * 32 + n] = acc[bi];
+    __syncthreads();
+    for (int t = tid; t < a.batch * 32; t += (int)blockDim.x) {
+        const int b = t >> 5, r = t & 31;
+        if (row0 + r < a.n_rows) {
+            float tot = 0.f;
+            for (int w = 0; w < S; w++) tot += red[((size_t)w * MAX_BATCH + b) * 32 + r];
+            if (a.bias) tot += a.bias[row0 + r];
+            a.y[(size_t)b * a.n_rows + row0 + r] = tot;
+        }
+    }
+}
+
+// x[batch, k] -> A operands and group records.  Thread = (8-element task, vector b); vectors beyond the batch
+// are written as zeros.  EVEN_ODD: the h = 0 half of a block's operand holds its even elements, h = 1 the odd.
+template <bool EVEN_ODD>
+__global__ void __launch_bounds__(256) pack_x_kernel(const float *x, int k, int batch, uint8_t *xa, float *xsg) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    const int ntask = k >> 3, nblk = k >> 5;
+    if (t >= ntask) return; // k is a multiple of 512: whole quads of tasks
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (b < batch) {
+        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)b * k + (size_t)t * 8);
+        const float4 v0 = p[0], v1 = p[1];
+        v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w; v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
+    }
+    uint32_t pk[4][2];
+    float sg, sum;
+    int ls[4];
+    axq_split8_compute(v, pk, sg, sum, ls);
+    if (b >= batch) { sg = 0.f; sum = 0.f; }
+    const int blk = t >> 2, e0 = (t & 3) * 8; // first element of the task inside its block
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+        const int row = 4 * b + l;
+        if (EVEN_ODD) {
+            uint8_t *d0 = xa + ((size_t)(blk * 2 + 0) * 32 + row) * 16 + (e0 >> 1);
+            uint8_t *d1 = xa + ((size_t)(blk * 2 + 1) * 32 + row) * 16 + (e0 >> 1);
+            *reinterpret_cast<uint32_t *>(d0) = (uint32_t)pick_alt(pk[l][0], pk[l][1], 0);
+            *reinterpret_cast<uint32_t *>(d1) = (uint32_t)pick_alt(pk[l][0], pk[l][1], 1);
+        } else {
+            uint8_t *d = xa + ((size_t)(blk * 2 + (e0 >> 4)) * 32 + row) * 16 + (e0 & 15);
+            *reinterpret_cast<uint2 *>(d) = make_uint2(pk[l][0], pk[l][1]);
+        }
+    }
+    if ((t & 3) == 0) {
+        const int slot = (blk * 2 + (b & 1)) * 4 + (b >> 1);
+        xsg[slot] = sg;
+        xsg[(size_t)nblk * 8 + slot] = sum;
+    }
+}
+
+template <class T>
+void launch_mb(axq_ctx *ctx, const MbArgs &a, const float *x) {
+    const dim3 pgrid((unsigned)((a.k / 8 + 255) / 256), MAX_BATCH);
+    pack_x_kernel<T::EVEN_ODD><<<pgrid, 256, 0, ctx->stream>>>(x, a.k, a.batch, const_cast<uint8_t *>(a.xa),
+                                                               const_cast<float *>(a.xsg));
+    const unsigned S = (unsigned)(a.k / WAVE_K);
+    const unsigned grid = (unsigned)((a.n_rows + 31) / 32);
+    const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float);
+    gemv_mb_kernel<T><<<grid, 64 * S, lds, ctx->stream>>>(a);
+}
+
+} // namespace
+
+// Whether the batched kernel covers this call.
+bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch) {
+    if (batch < 2 || batch > MAX_BATCH) return false;
+    // at most 8 waves: a lane holds 64 registers of A operands and 64 of weights, more than a 16-wave workgroup may
+    if (w->k % WAVE_K != 0 || w->k > 8 * WAVE_K) return false; // 34 k bytes of scratch fit the context's x buffer
+    return w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q8_0 || w->type == AXQ_Q4_K;
+}
+
+// y[batch, n_rows] = x[batch, k] W^T (+ bias) for 2 <= batch <= 8: split the batch, then one pass over W.
+int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y) {
+    const int k = (int)w->k;
+    // scratch (the context's x buffer): 32 k bytes of A operands, then 2 * (k / 32) * 8 floats of scales and sums
+    uint8_t *xa = ctx->xq;
+    float *xsg = reinterpret_cast<float *>(ctx->xq + (size_t)32 * k);
+    MbArgs a;
+    a.codes = w->codes; a.meta = w->meta;
+    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch;
+    a.xa = xa; a.xsg = xsg;
+    a.bias = bias; a.y = y;
+    a.n_rows = (int)w->n_rows; a.k = k; a.batch = batch;
+    switch (w->type) {
+    case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, x); break;
+    case AXQ_Q4_1: launch_mb<MQ4x<true>>(ctx, a, x); break;
+    case AXQ_Q8_0: launch_mb<MQ80>(ctx, a, x); break;
+    case AXQ_Q4_K: launch_mb<MQ4K>(ctx, a, x); break;
+    default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
+    }
+    AXQ_LAUNCH_CHECK(ctx, "gemv_mb_kernel");
+    return AXQ_OK;
+}

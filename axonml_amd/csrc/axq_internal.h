@@ -110,5 +110,8 @@ int axq_dev_gemv_dp_ex(axq_ctx *ctx, const axq_weight *w, const float *x, const 
 bool axq_dev_gemv_dp_covers(const axq_weight *w);
 size_t axq_xq_bytes(int64_t k);
 int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq);
+// gemv_batch.hip: batches of 2..8 vectors against one pass over the weights
+bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch);
+int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y);
 // gemm.hip
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_dev, int m, float *y_dev);

@@ -29,8 +29,11 @@ __device__ inline int axq_quad_xor2(int v) { return __builtin_amdgcn_update_dpp(
 // lane quad must call this together with four consecutive tasks (task % 4 == lane % 4): they share a
 // 32-element group and exchange its maximum and sum through DPP quad moves.  `live` = false lanes take
 // part in the shuffles (with zeros) and store nothing.
-__device__ inline void axq_split8(const float (&v)[8], int task, bool live, uint8_t *planes, uint4 *grp, int kpad) {
-    float amax = 0.f, sum = 0.f;
+// The arithmetic of a task: limb bytes pk[limb][dword] (limb 0 most significant; dword 0 = elements 0..3),
+// the group's scale, plain sum and limb sums (the latter three equal in the four lanes of the quad).
+__device__ inline void axq_split8_compute(const float (&v)[8], uint32_t (&pk)[4][2], float &sg, float &sum, int (&ls)[4]) {
+    float amax = 0.f;
+    sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         amax = fmaxf(amax, fabsf(v[i]));
@@ -46,12 +49,13 @@ __device__ inline void axq_split8(const float (&v)[8], int task, bool live, uint
     eb = eb < 30 ? 30 : eb;
     eb = eb > 254 ? 254 : eb;
     float f = __builtin_bit_cast(float, (280u - eb) << 23);
-    float sg = __builtin_bit_cast(float, (eb - 26u) << 23);
+    sg = __builtin_bit_cast(float, (eb - 26u) << 23);
     if (bad) sg = __builtin_nanf("");
     // t = rint(x f) = sum_i l_i 128^i with balanced digits; adding 64 (1 + 128 + 128^2 + 128^3) makes every
     // digit non-negative, d_i = l_i + 64 in 0..127 (the top one up to 128), so that plain bit fields extract
     // them; bytes go back to l_i = d_i - 64 four at a time: (d + 64) ^ 0x80 is d - 64 modulo 256.
-    uint32_t pk[4][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}}; // [plane][dword]: plane 0 = most significant limb
+#pragma unroll
+    for (int i = 0; i < 4; i++) pk[i][0] = pk[i][1] = 0;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const uint32_t u = (uint32_t)((bad ? 0 : (int)rintf(v[i] * f)) + 135274560);
@@ -61,7 +65,6 @@ __device__ inline void axq_split8(const float (&v)[8], int task, bool live, uint
         pk[1][i >> 2] |= ((u >> 14) & 127u) << sh;
         pk[0][i >> 2] |= (u >> 21) << sh;
     }
-    int ls[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         ls[i] = (int)__builtin_amdgcn_sad_u8(pk[i][0], 0u, __builtin_amdgcn_sad_u8(pk[i][1], 0u, 0u)) - 512;
@@ -70,6 +73,13 @@ __device__ inline void axq_split8(const float (&v)[8], int task, bool live, uint
         pk[i][0] = (pk[i][0] + 0x40404040u) ^ 0x80808080u;
         pk[i][1] = (pk[i][1] + 0x40404040u) ^ 0x80808080u;
     }
+}
+
+__device__ inline void axq_split8(const float (&v)[8], int task, bool live, uint8_t *planes, uint4 *grp, int kpad) {
+    uint32_t pk[4][2];
+    float sg, sum;
+    int ls[4];
+    axq_split8_compute(v, pk, sg, sum, ls);
     if (live) {
 #pragma unroll
         for (int i = 0; i < 4; i++)

@@ -134,3 +134,41 @@ def test_gemv_shape_errors(ctx):
         q.quantized_matmul(np.zeros((1, 128), np.float32), w, None, ctx)
     with pytest.raises(q.ShapeMismatch):
         q.quantized_matmul(np.zeros((1, 256), np.float32), w, np.zeros(3, np.float32), ctx)
+
+
+# ---- small batches: one pass over the weights for up to eight vectors (v_mfma_i32_32x32x32_i8 path)
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q8_0, o.Q4_K])
+@pytest.mark.parametrize("batch,n,k", [(2, 32, 512), (3, 100, 1024), (8, 96, 4096), (8, 33, 512), (11, 64, 2048), (16, 40, 4096)])
+def test_small_batch_reads_weights_once(ctx, qtype, batch, n, k):
+    rng = np.random.default_rng(batch * 1000 + n + k + qtype)
+    w = gen_weight(rng, n, k)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    x[1] = 0.3 + 0.05 * x[1]  # one vector with a mean: code offsets must cancel exactly for it too
+    bias = rng.standard_normal(n).astype(np.float32)
+    wq = o.quantize(qtype, w)
+    want = o.matmul_ref(qtype, wq, x, n, k, bias)
+    dw = q.DeviceWeight.upload(q.QuantizedTensor([n, k], qtype, wq), ctx)
+    got = q.quantized_matmul(x, dw, bias, ctx)
+    assert got.shape == (batch, n)
+    assert max_rel_err(got, want) <= MATMUL_RTOL
+    exact = o.matmul_f64(o.dequantize(qtype, wq, n * k).reshape(n, k), x) + bias.astype(np.float64)
+    assert max_rel_err(got, exact, STRICT_FLOOR) <= MATMUL_RTOL
+    # the batched kernel and the one-vector kernel agree far inside the tolerance
+    one = np.stack([q.quantized_matmul(x[i:i + 1], dw, bias, ctx)[0] for i in range(batch)])
+    assert max_rel_err(got, one, STRICT_FLOOR) <= 1e-4
+    dw.free()
+
+
+def test_small_batch_config_shape(ctx):
+    # BASELINE config 2: 11008 x 4096, batch 8, Q4_0 and Q4_1
+    rng = np.random.default_rng(82)
+    n, k, batch = 11008, 4096, 8
+    w = gen_weight(rng, n, k)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    for qtype in (o.Q4_0, o.Q4_1):
+        wq = o.quantize(qtype, w)
+        dw = q.DeviceWeight.upload(q.QuantizedTensor([n, k], qtype, wq), ctx)
+        got = q.quantized_matmul(x, dw, None, ctx)
+        exact = o.matmul_f64(o.dequantize(qtype, wq, n * k).reshape(n, k), x)
+        assert max_rel_err(got, exact, STRICT_FLOOR) <= MATMUL_RTOL
+        dw.free()
