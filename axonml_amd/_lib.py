@@ -99,6 +99,9 @@ SIGNATURES = {
     "axq_fill_normal_f32": (_i, [_vp, _vp, _sz, C.c_float, C.c_float, C.c_float, C.c_float, C.c_uint64]),
     "axq_bench_gemv_ring": (_i, [_vp, C.POINTER(_vp), _i, _vp, _i, _vp, _i]),
     "axq_bench_copy": (_i, [_vp, _vp, _vp, _sz, _i]),
+    "axq_type_from_ggml": (_i, [_i]),
+    "axq_type_to_ggml": (_i, [_i]),
+    "axq_gguf_convert_blocks": (_i, [_vp, _i, _vp, _vp, _sz, _i, _i]),
 }
 
 _lib = None

@@ -278,6 +278,12 @@ def main():
             extra["prefill_gemm"] = pf.bench(ctx, log)
         except ImportError:
             pass
+        try:
+            from axonml_amd import gguf
+
+            extra["gguf_convert"] = gguf.bench(ctx, log)
+        except ImportError:
+            pass
 
     out = {
         "metric": "q4k_gemv_effective_hbm_gbps",

@@ -127,6 +127,23 @@ AXQ_API int axq_quantize(axq_ctx *ctx, int type, const float *src, size_t numel,
 /* dst: numel f32 (the tail block is truncated, dequantize.rs:44-50). */
 AXQ_API int axq_dequantize(axq_ctx *ctx, int type, const void *packed, size_t numel, float *dst, int mem);
 
+/* ---- GGUF interop.  The reference names GGUF only as a file extension
+ *      (crates/axonml-cli/src/commands/quant.rs:218) and has no reader; the
+ *      block layouts are those of the GGUF / ggml specification.  Q8_0, Q5_0,
+ *      Q5_1, Q4_K, F16 and F32 images are the same on both sides; Q4_0 and
+ *      Q4_1 keep their scales and permute the 32 nibbles of a block (ggml: byte
+ *      j = elements j, j+16; reference pack(), types.rs:190-198: byte i =
+ *      elements 2i, 2i+1).  Element formulas agree, so a converted tensor
+ *      dequantises (dequantize.rs:116-121, 145-151) to ggml's values. ------- */
+enum { AXQ_GGUF_TO_NATIVE = 0, AXQ_NATIVE_TO_GGUF = 1 };
+/* ggml_type number of a GGUF tensor table entry -> axq_quant_type, -1 if this library has no such type. */
+AXQ_API int axq_type_from_ggml(int ggml_type);
+AXQ_API int axq_type_to_ggml(int type);
+/* Converts nblocks block images between the two orders; src == dst is allowed.
+ * Device pointers must be 16-byte aligned. */
+AXQ_API int axq_gguf_convert_blocks(axq_ctx *ctx, int type, const void *src, void *dst, size_t nblocks, int direction,
+                                    int mem);
+
 /* ---- device-resident weights: QuantizedTensor (types.rs:296-334) of shape
  *      [n_rows, k] as a Linear weight (nn/src/layers/linear.rs:41-42) -------- */
 /* Copies `packed` (bytes must equal axq_packed_bytes(type, n_rows*k)); the

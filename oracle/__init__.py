@@ -58,6 +58,8 @@ def lib():
         L.axo_model_forward.restype, L.axo_model_forward.argtypes = i, [vp, i, i, vp]
         L.axo_model_hidden.restype, L.axo_model_hidden.argtypes = C.POINTER(C.c_float), [vp]
         L.axo_model_kv.restype, L.axo_model_kv.argtypes = C.POINTER(C.c_uint16), [vp, i, i]
+        L.axo_gguf_convert.restype, L.axo_gguf_convert.argtypes = i, [i, vp, vp, sz, sz, i]
+        L.axo_ggml_dequantize.restype, L.axo_ggml_dequantize.argtypes = i, [i, vp, sz, vp]
         _lib = L
     return _lib
 
@@ -170,3 +172,26 @@ class DecodeModel:
             self.close()
         except Exception:
             pass
+
+
+def gguf_convert(qtype, blocks, to_gguf):
+    """Block images between ggml's order and the reference's (Q4_0 / Q4_1 permute nibbles, the rest copy)."""
+    src = np.ascontiguousarray(blocks, dtype=np.uint8).reshape(-1)
+    bb = lib().axo_bytes_per_block(qtype)
+    assert src.size % bb == 0
+    out = np.empty_like(src)
+    rc = lib().axo_gguf_convert(qtype, src.ctypes.data, out.ctypes.data, src.size // bb, bb, 1 if to_gguf else 0)
+    if rc:
+        raise ValueError(f"axo_gguf_convert: {rc}")
+    return out
+
+
+def ggml_dequantize(qtype, blocks):
+    """ggml's own row dequantiser on Q4_0 / Q4_1 blocks in ggml order."""
+    src = np.ascontiguousarray(blocks, dtype=np.uint8).reshape(-1)
+    nb = src.size // lib().axo_bytes_per_block(qtype)
+    out = np.empty(nb * 32, dtype=np.float32)
+    rc = lib().axo_ggml_dequantize(qtype, src.ctypes.data, nb, out.ctypes.data)
+    if rc:
+        raise ValueError(f"axo_ggml_dequantize: {rc}")
+    return out
