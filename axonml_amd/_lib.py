@@ -34,6 +34,11 @@ class DeviceInfo(C.Structure):
     ]
 
 
+class SamplingConfig(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_k", C.c_int32), ("top_p", C.c_float), ("repetition_penalty", C.c_float),
+                ("do_sample", C.c_int32)]
+
+
 class ModelConfig(C.Structure):
     _fields_ = [
         ("vocab_size", C.c_int32),
@@ -99,6 +104,8 @@ SIGNATURES = {
     "axq_fill_normal_f32": (_i, [_vp, _vp, _sz, C.c_float, C.c_float, C.c_float, C.c_float, C.c_uint64]),
     "axq_bench_gemv_ring": (_i, [_vp, C.POINTER(_vp), _i, _vp, _i, _vp, _i]),
     "axq_bench_copy": (_i, [_vp, _vp, _vp, _sz, _i]),
+    "axq_sample_token": (_i, [_vp, _vp, _i, _vp, _i, C.POINTER(SamplingConfig), C.c_float, C.POINTER(C.c_int32), _vp, _i]),
+    "axq_model_set_sampling": (_i, [_vp, C.POINTER(SamplingConfig), C.c_uint64]),
     "axq_type_from_ggml": (_i, [_i]),
     "axq_type_to_ggml": (_i, [_i]),
     "axq_gguf_convert_blocks": (_i, [_vp, _i, _vp, _vp, _sz, _i, _i]),

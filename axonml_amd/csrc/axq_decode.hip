@@ -44,6 +44,11 @@ struct axq_model {
     int max_splits;
     // device-side state
     int32_t *pos, *tok, *next, *gen, *prompt, *out;
+    int32_t *hist;                  // every token fed so far, by position (what a repetition penalty looks at)
+    void *sample_scratch;           // scratch of the sampler, allocated when one is set
+    bool sampling;                  // next token by axq_sampling_config instead of the plain argmax
+    axq_sampling_config sampler;
+    uint64_t sample_seed;
     int prompt_cap, out_cap;
     int host_pos;
     hipGraphExec_t graph;
@@ -401,6 +406,7 @@ __global__ void commit_next_kernel(const int32_t *next, int32_t *tok, int32_t *g
     gen[0] = g + 1;
 }
 __global__ void set_i32_kernel(int32_t *p, int32_t v) { p[0] = v; }
+__global__ void record_token_kernel(int32_t *hist, const int32_t *pos, const int32_t *tok) { hist[pos[0]] = tok[0]; }
 __global__ void fill_f32_kernel(float *p, size_t n, float v) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -540,7 +546,7 @@ int check_ready(axq_model *m) {
 }
 
 // Captures the step into a graph on first use; later calls replay it.
-int run_step(axq_model *m) {
+int run_step_graph(axq_model *m) {
     axq_ctx *ctx = m->ctx;
     static const bool no_graph = getenv("AXQ_DECODE_GRAPH") && getenv("AXQ_DECODE_GRAPH")[0] == '0';
     if (no_graph) return enqueue_step(m); // development knob: plain launches instead of a graph replay
@@ -561,6 +567,17 @@ int run_step(axq_model *m) {
     }
     AXQ_HIP(ctx, hipGraphLaunch(m->graph, ctx->stream), AXQ_ERR_KERNEL_LAUNCH_FAILED);
     return AXQ_OK;
+}
+
+// One token: note it in the history, run the step, and when a sampler is set let it replace the step's argmax.
+// The uniform variate of a draw comes from (seed, position), so a run is repeatable.
+int run_token(axq_model *m) {
+    axq_ctx *ctx = m->ctx;
+    record_token_kernel<<<1, 1, 0, ctx->stream>>>(m->hist, m->pos, m->tok);
+    int rc = run_step_graph(m);
+    if (rc || !m->sampling) return rc;
+    return axq_dev_sample(ctx, m->logits, m->cfg.vocab_size, m->hist, m->pos, 0, &m->sampler, 0.f, m->pos, m->sample_seed,
+                          m->sample_scratch, m->next, nullptr);
 }
 
 template <class T>
@@ -615,6 +632,7 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     TRY(dev_alloc(&m->gu, (size_t)2 * I)); TRY(dev_alloc(&m->act, I)); TRY(dev_alloc(&m->logits, c.vocab_size));
     TRY(dev_alloc(&m->pos, 1)); TRY(dev_alloc(&m->tok, 1)); TRY(dev_alloc(&m->next, 1)); TRY(dev_alloc(&m->gen, 1));
     TRY(dev_alloc(&m->prompt, m->prompt_cap)); TRY(dev_alloc(&m->out, m->out_cap));
+    TRY(dev_alloc(&m->hist, c.max_position_embeddings));
 #undef TRY
     if (e != hipSuccess) {
         int rc = axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "model buffers: %s", hipGetErrorString(e));
@@ -668,7 +686,7 @@ void axq_model_free(axq_model *m) {
     axq_weight_free(ctx, m->w_head);
     void *bufs[] = {m->emb, m->norm_attn, m->norm_ffn, m->norm_final, m->rope_cos, m->rope_sin, m->kcache, m->vcache, m->h,
                     m->xn, m->qkv, m->att, m->att_part, m->gu, m->act, m->logits, m->pos, m->tok,
-                    m->next, m->gen, m->prompt, m->out};
+                    m->next, m->gen, m->prompt, m->out, m->hist, m->sample_scratch};
     for (void *p : bufs)
         if (p) (void)hipFree(p);
     delete m;
@@ -785,6 +803,22 @@ int axq_model_reset(axq_model *m) {
     return AXQ_OK;
 }
 
+int axq_model_set_sampling(axq_model *m, const axq_sampling_config *cfg, uint64_t seed) {
+    if (!m) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    if (!cfg) { // back to the greedy argmax of the step itself
+        m->sampling = false;
+        return AXQ_OK;
+    }
+    int rc;
+    if ((rc = axq_check_sampling_config(ctx, cfg))) return rc;
+    if (!m->sample_scratch) AXQ_HIP(ctx, hipMalloc(&m->sample_scratch, axq_sample_scratch_bytes(m->cfg.vocab_size)), AXQ_ERR_ALLOCATION_FAILED);
+    m->sampler = *cfg;
+    m->sample_seed = seed;
+    m->sampling = true;
+    return AXQ_OK;
+}
+
 int axq_model_seq_len(const axq_model *m) { return m ? m->host_pos : -1; }
 
 int axq_model_read_kv(axq_model *m, int layer, int which, uint16_t *out) {
@@ -818,7 +852,7 @@ int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_t *next_
                         m->cfg.max_position_embeddings);
     AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
     set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->tok, token);
-    if ((rc = run_step(m))) return rc;
+    if ((rc = run_token(m))) return rc;
     m->host_pos++;
     if (logits)
         AXQ_HIP(ctx, hipMemcpyAsync(logits, m->logits, (size_t)m->cfg.vocab_size * 4, hipMemcpyDeviceToHost, ctx->stream),
@@ -856,13 +890,13 @@ int axq_model_generate(axq_model *m, const int32_t *prompt, int n_prompt, int ma
     // prompt: one step per token (the cache fills position by position)
     for (int i = 0; i < n_prompt && !rc; i++) {
         pick_prompt_kernel<<<1, 1, 0, ctx->stream>>>(m->prompt, m->pos, base, m->tok);
-        rc = run_step(m);
+        rc = run_token(m);
     }
     (void)hipEventRecord(e1, ctx->stream);
     // generation: the argmax of step i is the input of step i+1, on the device
     for (int i = 0; i < max_new_tokens && !rc; i++) {
         commit_next_kernel<<<1, 1, 0, ctx->stream>>>(m->next, m->tok, m->gen, m->out, m->out_cap);
-        if (i + 1 < max_new_tokens) rc = run_step(m);
+        if (i + 1 < max_new_tokens) rc = run_token(m);
     }
     (void)hipEventRecord(e2, ctx->stream);
     hipError_t e = hipStreamSynchronize(ctx->stream);

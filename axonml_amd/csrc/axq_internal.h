@@ -113,5 +113,11 @@ int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq);
 // gemv_batch.hip: batches of 2..8 vectors against one pass over the weights
 bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch);
 int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y);
+// sample.hip: every pointer a device pointer; scratch = axq_sample_scratch_bytes(vocab)
+size_t axq_sample_scratch_bytes(int vocab);
+int axq_check_sampling_config(axq_ctx *ctx, const axq_sampling_config *cfg);
+int axq_dev_sample(axq_ctx *ctx, const float *logits, int vocab, const int32_t *hist, const int32_t *hist_len_dev, int hist_len,
+                   const axq_sampling_config *cfg, float u, const int32_t *counter_dev, uint64_t seed, void *scratch,
+                   int32_t *out, float *filtered_out);
 // gemm.hip
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_dev, int m, float *y_dev);

@@ -52,6 +52,12 @@ class QuantizedLlama:
     def random_init(self, quant_type=QuantType.Q4_K, std=0.02, seed=1):
         self.ctx.check(self.ctx.lib.axq_model_random_init(self.handle, int(quant_type), std, seed))
 
+    def set_sampling(self, config=None, seed=0):
+        """Next tokens by a GenerationConfig (temperature, top-k, top-p, repetition penalty over every token fed so
+        far, draws from (seed, position)) instead of the plain argmax; None goes back to greedy."""
+        cfg = config.to_c() if config is not None else None
+        self.ctx.check(self.ctx.lib.axq_model_set_sampling(self.handle, C.byref(cfg) if cfg is not None else None, int(seed)))
+
     # ---- stepping
     def reset(self):
         self.ctx.check(self.ctx.lib.axq_model_reset(self.handle))
@@ -156,5 +162,16 @@ def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
            "frac_of_hbm_peak": bytes_per_token * tok_s / 8e12, "distinct_generated_ids": int(len(set(out.tolist())))}
     log(f"  decode 7B-shape: {tok_s:.1f} tok/s ({res['ms_per_token']:.3f} ms/token, {res['gbps']:.0f} GB/s), "
         f"prefill {res['prefill_tokens_per_s']:.0f} tok/s")
+    # the same with the sampler in the loop (temperature 0.8, top-k 40, top-p 0.9, repetition penalty 1.1)
+    from .generation import GenerationConfig
+
+    m.reset()
+    m.set_sampling(GenerationConfig(temperature=0.8, top_k=40, top_p=0.9, repetition_penalty=1.1), seed=7)
+    m.generate(prompt[:8], 4)
+    m.reset()
+    _, _, dec_s = m.generate(prompt, new_tokens)
+    res["sampled_tokens_per_s"] = steps / (dec_s * 1e-3)
+    res["sampler_us_per_token"] = (dec_s - dec_ms) / steps * 1e3
+    log(f"  with top-k/top-p sampling: {res['sampled_tokens_per_s']:.1f} tok/s (sampler {res['sampler_us_per_token']:.0f} us per token)")
     m.close()
     return res

@@ -209,6 +209,30 @@ AXQ_API int axq_model_read_hidden(axq_model *m, float *hidden_out);
 /* One layer's f16 cache, [kv_heads][max_position_embeddings][head_dim] (host); which 0 = keys, 1 = values. */
 AXQ_API int axq_model_read_kv(axq_model *m, int layer, int which, uint16_t *out);
 
+/* ---- next-token selection: TextGenerator::get_next_token (llm/src/generation.rs:258-269) =
+ *      apply_repetition_penalty (:145-158, once per occurrence), apply_temperature (:136-142),
+ *      apply_top_k (:161-180), apply_top_p (:183-214), then sample (:217-245) or argmax (:248-255),
+ *      on the device.  Penalty, temperature and top-k are bit-exact; the softmax sums of top-p
+ *      and of the draw are exact where the reference adds f32 sequentially, so a decision may
+ *      differ when a cumulative probability comes within ~1e-5 of its threshold. ---------- */
+/* The GenerationConfig fields that get_next_token reads (generation.rs:11-35). */
+typedef struct {
+    float temperature;        /* > 0; 1.0 leaves the logits alone */
+    int32_t top_k;            /* 0 = None */
+    float top_p;              /* negative = None */
+    float repetition_penalty; /* > 0; 1.0 = none */
+    int32_t do_sample;        /* 0: argmax of the filtered logits (ties: the last, as Iterator::max_by) */
+} axq_sampling_config;
+/* logits: f32[vocab]; generated: the ids the penalty looks at (may be NULL when n_generated = 0);
+ * u in [0, 1) stands for the reference's rand::thread_rng draw; token: one id; filtered_logits
+ * (optional, f32[vocab]): the logits after all filters, dropped entries -inf. */
+AXQ_API int axq_sample_token(axq_ctx *ctx, const float *logits, int vocab, const int32_t *generated, int n_generated,
+                             const axq_sampling_config *cfg, float u, int32_t *token, float *filtered_logits, int mem);
+/* Makes axq_model_forward / axq_model_generate choose the next token this way instead of by the plain
+ * argmax; the penalty sees every token fed so far, the draw of a step comes from (seed, position).
+ * cfg = NULL: back to greedy. */
+AXQ_API int axq_model_set_sampling(axq_model *m, const axq_sampling_config *cfg, uint64_t seed);
+
 /* ---- benchmark utilities ------------------------------------------------- */
 /* dst[i] ~ N(mean, std) from a counter-based generator (seed, i); with
  * outlier_p > 0 each element is instead +/-outlier_mag with that probability. */

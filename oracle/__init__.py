@@ -22,6 +22,11 @@ class ModelConfig(C.Structure):
                                                                                          ("rope_theta", C.c_float)]
 
 
+class SamplingConfig(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_k", C.c_int32), ("top_p", C.c_float), ("repetition_penalty", C.c_float),
+                ("do_sample", C.c_int32)]
+
+
 _lib = None
 
 
@@ -60,6 +65,7 @@ def lib():
         L.axo_model_kv.restype, L.axo_model_kv.argtypes = C.POINTER(C.c_uint16), [vp, i, i]
         L.axo_gguf_convert.restype, L.axo_gguf_convert.argtypes = i, [i, vp, vp, sz, sz, i]
         L.axo_ggml_dequantize.restype, L.axo_ggml_dequantize.argtypes = i, [i, vp, sz, vp]
+        L.axo_get_next_token.restype, L.axo_get_next_token.argtypes = i, [vp, i, vp, i, C.POINTER(SamplingConfig), C.c_float]
         _lib = L
     return _lib
 
@@ -195,3 +201,12 @@ def ggml_dequantize(qtype, blocks):
     if rc:
         raise ValueError(f"axo_ggml_dequantize: {rc}")
     return out
+
+
+def get_next_token(logits, generated=(), temperature=1.0, top_k=None, top_p=None, repetition_penalty=1.0, do_sample=True, u=0.0):
+    """TextGenerator::get_next_token with the uniform variate given; returns (token, filtered logits)."""
+    work = np.array(logits, dtype=np.float32).reshape(-1)
+    gen = np.ascontiguousarray(generated, dtype=np.int32).reshape(-1)
+    cfg = SamplingConfig(temperature, top_k or 0, -1.0 if top_p is None else top_p, repetition_penalty, 1 if do_sample else 0)
+    tok = lib().axo_get_next_token(work.ctypes.data, work.size, gen.ctypes.data if gen.size else None, gen.size, C.byref(cfg), u)
+    return tok, work
