@@ -375,7 +375,28 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const float *logits, int v
     __shared__ int bi[16];
     float best = -INFINITY;
     int idx = 0;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    // eight 16-byte loads per thread in flight at a time; a thread's indices rise, and `>=` keeps the last maximum
+    const int n4 = vocab >> 2;
+    const float4 *l4 = reinterpret_cast<const float4 *>(logits);
+    for (int base = threadIdx.x; base < n4; base += 8 * 1024) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int f = base + u * 1024;
+            v[u] = l4[f < n4 ? f : n4 - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int f = base + u * 1024;
+            if (f < n4) {
+                const float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (e[c] >= best) { best = e[c]; idx = 4 * f + c; }
+            }
+        }
+    }
+    for (int i = 4 * n4 + threadIdx.x; i < vocab; i += 1024) {
         float v = logits[i];
         if (v >= best) { best = v; idx = i; }
     }
