@@ -36,7 +36,9 @@ struct GemmArgs {
     const _Float16 *xh;    // [M, K] row-scaled f16
     const float *rowscale; // [M]
     float *y;              // [M, N]
+    float *ypart;          // split K: [splits, M, N] unscaled partial sums (NULL when one workgroup covers all of K)
     int m, n, k;
+    int steps_per_split;   // K steps per workgroup (grid.y of them cover K)
 };
 
 __device__ inline float h2f(uint32_t bits) { return __half2float(__ushort_as_half((unsigned short)bits)); }
@@ -279,7 +281,9 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
     int tile = blockIdx.x;
     if (total % 8 == 0) tile = (tile & 7) * (total >> 3) + (tile >> 3);
     const int m0 = (tile / nt) * BM, n0 = (tile % nt) * BN;
-    const int ksteps = a.k / BK;
+    // split K: workgroup (x, y) covers K steps [kbeg, kbeg + ksteps)
+    const int kbeg = (int)blockIdx.y * a.steps_per_split;
+    const int ksteps = a.k / BK - kbeg < a.steps_per_split ? a.k / BK - kbeg : a.steps_per_split;
 
     if (feeder) {
         const int ft = tid - NTF;
@@ -303,9 +307,9 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
         auto fetch = [&](int ks) { // clamped: past the last step the feeders re-read it and nobody looks
             ks = ks < ksteps ? ks : ksteps - 1;
 #pragma unroll
-            for (int i = 0; i < XV; i++) xa[i] = *reinterpret_cast<const u32x4 *>(xrow[i] + (size_t)ks * BK);
+            for (int i = 0; i < XV; i++) xa[i] = *reinterpret_cast<const u32x4 *>(xrow[i] + (size_t)(kbeg + ks) * BK);
 #pragma unroll
-            for (int u = 0; u < UNITS; u++) T::load16(a, wrow[u], ks, (ft + u * NTF) & 3, raw[u]);
+            for (int u = 0; u < UNITS; u++) T::load16(a, wrow[u], kbeg + ks, (ft + u * NTF) & 3, raw[u]);
         };
         fetch(0);
         for (int ks = 0; ks <= ksteps; ks++) {
@@ -318,7 +322,7 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
 #pragma unroll
             for (int i = 0; i < XV; i++) xs[i] = xa[i];
 #pragma unroll
-            for (int u = 0; u < UNITS; u++) T::cvt16(raw[u], kcur, (ft + u * NTF) & 3, w[u], k0[u], k1[u]);
+            for (int u = 0; u < UNITS; u++) T::cvt16(raw[u], kbeg + kcur, (ft + u * NTF) & 3, w[u], k0[u], k1[u]);
             fetch(ks + 1);
             if (ks < ksteps) {
 #pragma unroll
@@ -392,7 +396,10 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int gm = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (gm < a.m && gn < a.n) a.y[(size_t)gm * a.n + gn] = acc[i][j][r] * (a.rowscale[gm] * (1.0f / T::WS));
+                if (gm < a.m && gn < a.n) {
+                    if (a.ypart) a.ypart[((size_t)blockIdx.y * a.m + gm) * a.n + gn] = acc[i][j][r];
+                    else a.y[(size_t)gm * a.n + gn] = acc[i][j][r] * (a.rowscale[gm] * (1.0f / T::WS));
+                }
             }
         }
 }
@@ -426,11 +433,26 @@ __global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int
     if (threadIdx.x == 0) rowscale[row] = 1.0f / f;
 }
 
+// y = (sum over the splits, in order) * rowscale / ws: four outputs per thread
+__global__ void __launch_bounds__(256) gemm_reduce_kernel(const float *ypart, const float *rowscale, int m, int n, int splits,
+                                                          float inv_ws, float *y) {
+    const size_t i4 = (size_t)blockIdx.x * blockDim.x + threadIdx.x, total4 = (size_t)m * n / 4;
+    if (i4 >= total4) return;
+    float4 acc = reinterpret_cast<const float4 *>(ypart)[i4];
+    for (int s = 1; s < splits; s++) {
+        const float4 v = reinterpret_cast<const float4 *>(ypart + (size_t)s * m * n)[i4];
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    const float f = rowscale[(i4 * 4) / (size_t)n] * inv_ws; // n is a multiple of 4: the four share a row
+    reinterpret_cast<float4 *>(y)[i4] = make_float4(acc.x * f, acc.y * f, acc.z * f, acc.w * f);
+}
+
 template <class T>
-int launch_gemm(axq_ctx *ctx, const GemmArgs &a) {
+int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
     static bool attr_set = false;
     const int wm = a.m > 128 ? 2 : 1, bm = 128 * wm;
-    const unsigned grid = (unsigned)(((a.n + BN - 1) / BN) * ((a.m + bm - 1) / bm));
+    const unsigned tiles = (unsigned)(((a.n + BN - 1) / BN) * ((a.m + bm - 1) / bm));
+    const dim3 grid(tiles, (unsigned)splits);
     const size_t lds = (size_t)2 * (bm + 2 * BN) * LDK * sizeof(_Float16); // two stages
     if (!attr_set) {
         AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, 2>),
@@ -442,6 +464,12 @@ int launch_gemm(axq_ctx *ctx, const GemmArgs &a) {
     if (wm == 2) gemm_kernel<T, 2><<<grid, 512, lds, ctx->stream>>>(a);
     else gemm_kernel<T, 1><<<grid, 256, lds, ctx->stream>>>(a);
     AXQ_LAUNCH_CHECK(ctx, "gemm_kernel");
+    if (splits > 1) {
+        const size_t total4 = (size_t)a.m * a.n / 4;
+        gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(a.ypart, a.rowscale, a.m, a.n, splits,
+                                                                                    1.0f / T::WS, a.y);
+        AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
+    }
     return AXQ_OK;
 }
 
@@ -453,8 +481,20 @@ int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int 
                         (long long)w->k);
     if (w->n_rows > INT32_MAX || w->k > INT32_MAX)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
-    // scratch: f16 activations [m, k] then the row scales [m]; kept in the context and grown on demand
-    const size_t xh_bytes = axq_align_up((size_t)m * (size_t)w->k * 2, 256), need = xh_bytes + (size_t)m * 4;
+    // scratch: f16 activations [m, k], the row scales [m], the partial sums of a split K; kept in the context, grown on demand
+    // split K when the output tiles alone leave most compute units idle (short prompts): the splits' partial
+    // sums go through scratch and are added in order by a second kernel
+    const int bm = m > 128 ? 256 : 128;
+    const long tiles = (long)((w->n_rows + BN - 1) / BN) * ((m + bm - 1) / bm);
+    const int ksteps = (int)(w->k / BK), cus = ctx->prop.multiProcessorCount;
+    int splits = (int)(cus / tiles);
+    splits = splits > 8 ? 8 : splits;
+    if (splits > ksteps / 4) splits = ksteps / 4;
+    if (splits < 2 || w->n_rows % 4 != 0) splits = 1;
+    const int steps_per_split = (ksteps + splits - 1) / splits;
+    splits = (ksteps + steps_per_split - 1) / steps_per_split;
+    const size_t xh_bytes = axq_align_up((size_t)m * (size_t)w->k * 2, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
+    const size_t need = xh_bytes + rs_bytes + (splits > 1 ? (size_t)splits * m * (size_t)w->n_rows * 4 : 0);
     if (ctx->gemm_scratch_bytes < need) {
         AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
         if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
@@ -470,17 +510,19 @@ int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int 
     a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
     a.xh = xh; a.rowscale = rowscale; a.y = y;
+    a.ypart = splits > 1 ? reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(ctx->gemm_scratch) + xh_bytes + rs_bytes) : nullptr;
     a.m = m; a.n = (int)w->n_rows; a.k = (int)w->k;
+    a.steps_per_split = steps_per_split;
     int rc;
     switch (w->type) {
-    case AXQ_Q4_K: rc = launch_gemm<GQ4K>(ctx, a); break;
-    case AXQ_Q4_0: rc = launch_gemm<GQ4x<false>>(ctx, a); break;
-    case AXQ_Q4_1: rc = launch_gemm<GQ4x<true>>(ctx, a); break;
-    case AXQ_Q5_0: rc = launch_gemm<GQ5x<false>>(ctx, a); break;
-    case AXQ_Q5_1: rc = launch_gemm<GQ5x<true>>(ctx, a); break;
-    case AXQ_Q8_0: rc = launch_gemm<GQ80>(ctx, a); break;
-    case AXQ_F16: rc = launch_gemm<GF16>(ctx, a); break;
-    case AXQ_F32: rc = launch_gemm<GF32>(ctx, a); break;
+    case AXQ_Q4_K: rc = launch_gemm<GQ4K>(ctx, a, splits); break;
+    case AXQ_Q4_0: rc = launch_gemm<GQ4x<false>>(ctx, a, splits); break;
+    case AXQ_Q4_1: rc = launch_gemm<GQ4x<true>>(ctx, a, splits); break;
+    case AXQ_Q5_0: rc = launch_gemm<GQ5x<false>>(ctx, a, splits); break;
+    case AXQ_Q5_1: rc = launch_gemm<GQ5x<true>>(ctx, a, splits); break;
+    case AXQ_Q8_0: rc = launch_gemm<GQ80>(ctx, a, splits); break;
+    case AXQ_F16: rc = launch_gemm<GF16>(ctx, a, splits); break;
+    case AXQ_F32: rc = launch_gemm<GF32>(ctx, a, splits); break;
     default: rc = axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
     }
     return rc;
