@@ -32,19 +32,26 @@ __device__ inline int axq_quad_xor2(int v) { return __builtin_amdgcn_update_dpp(
 // The arithmetic of a task: limb bytes pk[limb][dword] (limb 0 most significant; dword 0 = elements 0..3),
 // the group's scale, plain sum and limb sums (the latter three equal in the four lanes of the quad).
 __device__ inline void axq_split8_compute(const float (&v)[8], uint32_t (&pk)[4][2], float &sg, float &sum, int (&ls)[4]) {
-    float amax = 0.f;
+    // largest magnitude as an integer maximum of the sign-less bit patterns: a nan ranks above everything
+    // (a float maximum would drop it, and the nan would then count as zero)
+    uint32_t amax = 0;
     sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        amax = fmaxf(amax, fabsf(v[i]));
+        const uint32_t m = __builtin_bit_cast(uint32_t, v[i]) & 0x7FFFFFFFu;
+        amax = amax > m ? amax : m;
         sum += v[i];
     }
-    amax = fmaxf(amax, axq_quad_xor1(amax));
-    amax = fmaxf(amax, axq_quad_xor2(amax));
+    {
+        const uint32_t o1 = (uint32_t)axq_quad_xor1((int)amax);
+        amax = amax > o1 ? amax : o1;
+        const uint32_t o2 = (uint32_t)axq_quad_xor2((int)amax);
+        amax = amax > o2 ? amax : o2;
+    }
     sum += axq_quad_xor1(sum);
     sum += axq_quad_xor2(sum);
     // amax in [2^e, 2^(e+1)): scale so that |x| * f < 2^27, f = 2^(26-e); limb sums times 2^(e-26) give back x
-    uint32_t eb = (__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFF;
+    uint32_t eb = amax >> 23;
     const bool bad = eb == 0xFF;
     eb = eb < 30 ? 30 : eb;
     eb = eb > 254 ? 254 : eb;

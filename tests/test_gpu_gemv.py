@@ -172,3 +172,23 @@ def test_small_batch_config_shape(ctx):
         exact = o.matmul_f64(o.dequantize(qtype, wq, n * k).reshape(n, k), x)
         assert max_rel_err(got, exact, STRICT_FLOOR) <= MATMUL_RTOL
         dw.free()
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("batch", [1, 8])
+def test_non_finite_activation_reaches_every_output(ctx, qtype, batch):
+    # a nan (or an infinity) in x makes every f32 dot product of the reference non-finite; the integer limb
+    # split must not lose it (a float maximum ignores nan operands)
+    rng = np.random.default_rng(17)
+    n, k = 64, 4096
+    dw = q.DeviceWeight.quantize(gen_weight(rng, n, k), q.QuantType(qtype), ctx)
+    for bad in (np.nan, np.inf, -np.inf):
+        x = rng.standard_normal((batch, k)).astype(np.float32)
+        x[0, 1234] = bad
+        y = q.quantized_matmul(x, dw, None, ctx)
+        assert not np.isfinite(y[0]).any(), (o.TYPE_NAMES[qtype], bad)
+        if np.isnan(bad):
+            assert np.isnan(y[0]).all()
+        if batch > 1:
+            assert np.isfinite(y[1:]).all()  # the other vectors of the batch are untouched
+    dw.free()
