@@ -51,6 +51,7 @@ class ModelConfig(C.Structure):
         ("max_position_embeddings", C.c_int32),
         ("rms_norm_eps", C.c_float),
         ("rope_theta", C.c_float),
+        ("sliding_window", C.c_int32),
     ]
 
 

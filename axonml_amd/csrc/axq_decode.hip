@@ -154,7 +154,8 @@ __device__ inline float group_sum(float s) {
 template <int D, int REP>
 __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, const float *rope_cos, const float *rope_sin,
                                                            uint16_t *kcache, uint16_t *vcache, const int32_t *pos_p,
-                                                           int n_heads, int n_kv, int max_pos, int max_splits, float *part) {
+                                                           int n_heads, int n_kv, int max_pos, int max_splits, int window,
+                                                           float *part) {
     constexpr int HALF = D / 2;
     constexpr int LP = D / 8, PPW = 64 / LP;                 // lanes per position, positions per wave pass
     constexpr int NPASS = (ATT_CHUNK + 4 * PPW - 1) / (4 * PPW); // passes of the four waves over the chunk
@@ -171,7 +172,9 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
     const int kvh = blockIdx.x, split = blockIdx.y;
     const int pos = pos_p[0];
     const int p0 = split * ATT_CHUNK;
-    if (p0 > pos) return;
+    // sliding window (MistralAttention, mistral.rs:204-238): positions before p_lo are not attended to
+    const int p_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+    if (p0 > pos || p0 + ATT_CHUNK <= p_lo) return;
     const int p1 = (p0 + ATT_CHUNK < pos + 1) ? p0 + ATT_CHUNK : pos + 1;
     const int np = p1 - p0;
     const bool has_new = pos < p1;
@@ -260,7 +263,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
             for (int h = 0; h < REP; h++) sh[h] = group_sum<LP>(sh[h]);
             if (c8 == 0) {
 #pragma unroll
-                for (int h = 0; h < REP; h++) sc[pi * REP + h] = (pi < np && h < rep) ? sh[h] * scale : -INFINITY;
+                for (int h = 0; h < REP; h++) sc[pi * REP + h] = (pi < np && p0 + pi >= p_lo && h < rep) ? sh[h] * scale : -INFINITY;
             }
         }
     }
@@ -271,7 +274,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
         float mx = v;
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
-        float e = lane < np ? expf(v - mx) : 0.f;
+        float e = (lane < np && p0 + lane >= p_lo) ? expf(v - mx) : 0.f;
         float sum = e;
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
@@ -308,14 +311,16 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
 // grid (heads), 256 threads.  The (m, l) pairs of the head's splits go through LDS so that every thread
 // knows the weights exp(m_s - max) before it walks the splits; the walk itself has no dependent loads.
 __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, const int32_t *pos_p, int n_heads, int n_kv,
-                                                           int d, int max_splits, float *att) {
+                                                           int d, int max_splits, int window, float *att) {
     extern __shared__ float cm[];
     float *wgt = cm;                 // [max_splits] exp(m_s - max)
     float *red = wgt + max_splits;   // [4] wave maxima, then [4] wave sums of l_s w_s
     const int head = blockIdx.x, rep = n_heads / n_kv, kvh = head / rep, h = head - kvh * rep;
-    const int nsplit = pos_p[0] / ATT_CHUNK + 1;
+    const int pos = pos_p[0];
+    const int s_lo = (window > 0 && pos + 1 > window) ? (pos + 1 - window) / ATT_CHUNK : 0; // first split inside the window
+    const int nsplit = pos / ATT_CHUNK + 1 - s_lo;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const float *base = part + ((size_t)(kvh * max_splits) * rep + h) * (d + 2);
+    const float *base = part + ((size_t)(kvh * max_splits + s_lo) * rep + h) * (d + 2);
     const size_t stride = (size_t)rep * (d + 2);
     // maxima
     float mx = -INFINITY;
@@ -483,7 +488,7 @@ void launch_attn_partial_t(axq_model *m, int l, hipStream_t st) {
     const size_t kv_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * D;
     attn_partial_kernel<D, REP><<<dim3(c.num_key_value_heads, m->max_splits), 256, 0, st>>>(
         m->qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer, m->vcache + (size_t)l * kv_layer, m->pos,
-        c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, m->max_splits, m->att_part);
+        c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, m->max_splits, c.sliding_window, m->att_part);
 }
 
 template <int D>
@@ -544,7 +549,7 @@ int enqueue_step(axq_model *m) {
             return rc;
         launch_attn_partial(m, l, st);
         attn_combine_kernel<<<c.num_attention_heads, 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
-                                                                          c.num_key_value_heads, d, m->max_splits, m->att);
+                                                                          c.num_key_value_heads, d, m->max_splits, c.sliding_window, m->att);
         // residual adds go through the bias slot, in place
         if ((rc = linear(m, m->w_o[l], m->att, AXQ_X_PLAIN, nullptr, AXQ_Y_PLAIN, nullptr, m->h, m->h))) return rc;
         if ((rc = linear(m, m->w_gu[l], m->h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, AXQ_Y_SWIGLU, m->xn, nullptr, m->act)))
@@ -614,7 +619,8 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     *out = NULL;
     const axq_model_config &c = *cfg;
     if (c.vocab_size <= 0 || c.hidden_size <= 0 || c.intermediate_size <= 0 || c.num_hidden_layers < 0 ||
-        c.num_attention_heads <= 0 || c.num_key_value_heads <= 0 || c.head_dim <= 0 || c.max_position_embeddings <= 0)
+        c.num_attention_heads <= 0 || c.num_key_value_heads <= 0 || c.head_dim <= 0 || c.max_position_embeddings <= 0 ||
+        c.sliding_window < 0)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: model dimensions must be positive");
     if (c.num_attention_heads % c.num_key_value_heads != 0)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: %d query heads are not a multiple of %d kv heads",

@@ -19,7 +19,7 @@ def mistral_7b_config(max_position_embeddings=640):
     """MistralConfig::mistral_7b (crates/axonml-llm/src/mistral.rs:56-70), context capped to the cache size."""
     return dict(vocab_size=32000, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32,
                 num_attention_heads=32, num_key_value_heads=8, head_dim=128,
-                max_position_embeddings=max_position_embeddings, rms_norm_eps=1e-5, rope_theta=10000.0)
+                max_position_embeddings=max_position_embeddings, rms_norm_eps=1e-5, rope_theta=10000.0, sliding_window=4096)
 
 
 class QuantizedLlama:

@@ -327,7 +327,8 @@ def llama_config_from_metadata(md, max_position_embeddings=None):
                 head_dim=int(md.get("llama.attention.key_length", hidden // heads)),
                 max_position_embeddings=int(max_position_embeddings or min(ctx_len, 4096)),
                 rms_norm_eps=float(md.get("llama.attention.layer_norm_rms_epsilon", 1e-5)),
-                rope_theta=float(md.get("llama.rope.freq_base", 10000.0)))
+                rope_theta=float(md.get("llama.rope.freq_base", 10000.0)),
+                sliding_window=int(md.get("llama.attention.sliding_window", 0)))
 
 
 def load_llama(path, ctx=None, max_position_embeddings=None, permuted_qk=True):

@@ -154,7 +154,8 @@ def parse_llama_config_from_json(cfg, max_position_embeddings=None):
                 num_key_value_heads=int(cfg.get("num_key_value_heads") or heads),
                 head_dim=int(cfg.get("head_dim") or hidden // heads),
                 max_position_embeddings=int(max_position_embeddings or cfg.get("max_position_embeddings", 4096)),
-                rms_norm_eps=float(cfg.get("rms_norm_eps", 1e-5)), rope_theta=float(cfg.get("rope_theta", 10000.0)))
+                rms_norm_eps=float(cfg.get("rms_norm_eps", 1e-5)), rope_theta=float(cfg.get("rope_theta", 10000.0)),
+                sliding_window=int(cfg.get("sliding_window") or 0))  # Mistral's window (parse_mistral_config, :557-572); none for LLaMA
 
 
 _PROJ = {"q": "self_attn.q_proj", "k": "self_attn.k_proj", "v": "self_attn.v_proj", "o": "self_attn.o_proj",

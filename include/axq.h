@@ -174,6 +174,10 @@ typedef struct {
     int32_t vocab_size, hidden_size, intermediate_size, num_hidden_layers;
     int32_t num_attention_heads, num_key_value_heads, head_dim, max_position_embeddings;
     float rms_norm_eps, rope_theta;
+    /* MistralConfig::sliding_window (mistral.rs:56-70): a token attends to the last `sliding_window`
+     * cache positions only (MistralAttention::forward_with_cache slices the cache, mistral.rs:204-238);
+     * 0 = the whole cache (LLaMA). */
+    int32_t sliding_window;
 } axq_model_config;
 
 typedef enum {

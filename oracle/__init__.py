@@ -19,7 +19,8 @@ TYPE_NAMES = {Q8_0: "Q8_0", Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_
 class ModelConfig(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("vocab_size", "hidden_size", "intermediate_size", "num_layers", "num_heads",
                                           "num_kv_heads", "head_dim", "max_seq_len")] + [("rms_norm_eps", C.c_float),
-                                                                                         ("rope_theta", C.c_float)]
+                                                                                         ("rope_theta", C.c_float),
+                                                                                         ("sliding_window", C.c_int32)]
 
 
 class SamplingConfig(C.Structure):

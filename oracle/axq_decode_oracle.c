@@ -48,6 +48,7 @@ typedef struct {
     int32_t vocab_size, hidden_size, intermediate_size, num_layers;
     int32_t num_heads, num_kv_heads, head_dim, max_seq_len;
     float rms_norm_eps, rope_theta;
+    int32_t sliding_window; /* 0 = attend to the whole cache; else the last sliding_window positions (mistral.rs:204-238) */
 } axo_model_config;
 
 enum { AXO_LIN_Q = 0, AXO_LIN_K, AXO_LIN_V, AXO_LIN_O, AXO_LIN_GATE, AXO_LIN_UP, AXO_LIN_DOWN, AXO_LIN_COUNT };
@@ -212,7 +213,8 @@ AXO_API int axo_model_forward(axo_model *m, int token, int pos, float *logits) {
             int kh = h / group;
             const float *qh = m->q + (size_t)h * d;
             float mx = -INFINITY;
-            for (int j = 0; j <= pos; j++) {
+            const int j0 = (c->sliding_window > 0 && pos + 1 > c->sliding_window) ? pos + 1 - c->sliding_window : 0;
+            for (int j = j0; j <= pos; j++) {
                 const uint16_t *kr = L->kc + ((size_t)kh * c->max_seq_len + (size_t)j) * d;
                 float s = 0.0f;
                 for (int i = 0; i < d; i++) s += qh[i] * axo_f16_to_f32(kr[i]);
@@ -221,13 +223,13 @@ AXO_API int axo_model_forward(axo_model *m, int token, int pos, float *logits) {
                 if (s > mx) mx = s;
             }
             float sum = 0.0f;
-            for (int j = 0; j <= pos; j++) {
+            for (int j = j0; j <= pos; j++) {
                 m->scores[j] = expf(m->scores[j] - mx);
                 sum += m->scores[j];
             }
             float *oh = m->att + (size_t)h * d;
             for (int i = 0; i < d; i++) oh[i] = 0.0f;
-            for (int j = 0; j <= pos; j++) {
+            for (int j = j0; j <= pos; j++) {
                 const uint16_t *vr = L->vc + ((size_t)kh * c->max_seq_len + (size_t)j) * d;
                 float p = m->scores[j] / sum;
                 for (int i = 0; i < d; i++) oh[i] += p * axo_f16_to_f32(vr[i]);

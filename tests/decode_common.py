@@ -18,7 +18,7 @@ LIN_ID = {"q": 0, "k": 1, "v": 2, "o": 3, "gate": 4, "up": 5, "down": 6}
 
 def tiny_config(**over):
     c = dict(vocab_size=320, hidden_size=256, intermediate_size=512, num_layers=2, num_heads=4, num_kv_heads=2,
-             head_dim=64, max_seq_len=48, rms_norm_eps=1e-5, rope_theta=10000.0)
+             head_dim=64, max_seq_len=48, rms_norm_eps=1e-5, rope_theta=10000.0, sliding_window=0)
     c.update(over)
     return c
 
@@ -57,7 +57,8 @@ def load_gpu(ctx, c, w):
     m = QuantizedLlama(ctx, vocab_size=c["vocab_size"], hidden_size=c["hidden_size"],
                        intermediate_size=c["intermediate_size"], num_hidden_layers=c["num_layers"],
                        num_attention_heads=c["num_heads"], num_key_value_heads=c["num_kv_heads"], head_dim=c["head_dim"],
-                       max_position_embeddings=c["max_seq_len"], rms_norm_eps=c["rms_norm_eps"], rope_theta=c["rope_theta"])
+                       max_position_embeddings=c["max_seq_len"], rms_norm_eps=c["rms_norm_eps"], rope_theta=c["rope_theta"],
+                       sliding_window=c.get("sliding_window", 0))
     m.set_embedding_f16(w["emb"])
     m.set_norm(-1, 0, w["final_norm"])
     shapes = LIN_SHAPES(c)
@@ -111,8 +112,10 @@ class NumpyDecoder:
             v = (L["v"] @ xn).reshape(nkv, d)
             self.k[l].append(k.astype(np.float16).astype(np.float64))
             self.v[l].append(v.astype(np.float16).astype(np.float64))
-            K = np.stack(self.k[l], 1)  # [nkv, T, d]
-            V = np.stack(self.v[l], 1)
+            win = c.get("sliding_window", 0)
+            first = max(0, len(self.k[l]) - win) if win else 0  # Mistral: the last `win` positions only
+            K = np.stack(self.k[l][first:], 1)  # [nkv, T, d]
+            V = np.stack(self.v[l][first:], 1)
             out = np.zeros((nh, d))
             for hd in range(nh):
                 kv = hd // (nh // nkv)

@@ -28,6 +28,22 @@ def test_step_by_step_logits_and_tokens(ctx, qtype):
     gpu.close()
 
 
+@pytest.mark.parametrize("window", [1, 5, 32, 40])
+def test_sliding_window_attention(ctx, window):
+    # windows inside one 32-position split, ending exactly on a split, and spanning two splits
+    c = tiny_config(sliding_window=window, max_seq_len=100)
+    w = random_weights(c, 60 + window)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    tok = 2
+    for pos in range(90):
+        c_next, c_logits = cpu.forward(tok, pos)
+        g_next, g_logits = gpu.forward(tok)
+        assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, pos
+        assert g_next == c_next, pos
+        tok = c_next
+    gpu.close()
+
+
 def test_kv_cache_matches_oracle_up_to_isolated_f16_roundings(ctx):
     c = tiny_config(num_layers=2)
     w = random_weights(c, 50)

@@ -86,11 +86,14 @@ def test_config_defaults_follow_the_reference():
     # parse_llama_config_from_json (hf_loader.rs:511-530): every key optional, LLaMA-2-7B defaults
     c = hf.parse_llama_config_from_json({})
     assert c == dict(vocab_size=32000, hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
-                     num_key_value_heads=32, head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=10000.0)
+                     num_key_value_heads=32, head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=10000.0,
+                     sliding_window=0)
     c = hf.parse_llama_config_from_json({"num_attention_heads": 8, "hidden_size": 512, "num_key_value_heads": 2, "rope_theta": 1e6},
                                         max_position_embeddings=64)
     assert c["num_key_value_heads"] == 2 and c["head_dim"] == 64 and c["max_position_embeddings"] == 64 and c["rope_theta"] == 1e6
     assert hf.parse_llama_config_from_json({"num_attention_heads": 8})["num_key_value_heads"] == 8  # falls back to the head count
+    assert hf.parse_llama_config_from_json({"sliding_window": 4096})["sliding_window"] == 4096  # Mistral's config.json
+    assert hf.parse_llama_config_from_json({"sliding_window": None})["sliding_window"] == 0
 
 
 def _tiny_checkpoint(tmp_path, c, seed, sharded, tied, prefix="model."):

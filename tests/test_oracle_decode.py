@@ -21,6 +21,25 @@ def test_matches_independent_float64_forward():
         tok = nxt
 
 
+def test_sliding_window_matches_independent_forward_and_differs_from_full_attention():
+    # MistralAttention::forward_with_cache (mistral.rs:204-238): only the last `sliding_window` cache rows are attended to
+    c = tiny_config(sliding_window=6)
+    w = random_weights(c, 4)
+    cpu, ref, full = load_oracle(c, w), NumpyDecoder(c, w), load_oracle(tiny_config(), w)
+    tok, differs = 5, False
+    for pos in range(16):
+        nxt, logits = cpu.forward(tok, pos)
+        want = ref.forward(tok, pos)
+        assert max_rel_err(logits, want, DECODE_FLOOR) < DECODE_RTOL / 10, pos
+        _, logits_full = full.forward(tok, pos)
+        if pos < 6:
+            assert np.array_equal(logits, logits_full)  # the window is not full yet
+        else:
+            differs |= not np.array_equal(logits, logits_full)
+        tok = nxt
+    assert differs
+
+
 def test_zero_linears_leave_embedding_and_give_zero_logits_closed_form():
     # all layer linears zero: h = embedding; logits = head @ rmsnorm(h): a one-line closed form
     c = tiny_config(num_layers=1)
