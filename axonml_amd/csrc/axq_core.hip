@@ -185,7 +185,10 @@ int axq_init(int device, axq_ctx **out) {
         return AXQ_ERR_DRIVER;
     }
     ctx->fp8_unit_inv = 1.0f / h[0];
-    INIT_HIP(hipMalloc((void **)&ctx->xq, axq_xq_bytes(AXQ_XQ_MAX_K)));
+    {
+        size_t xq_bytes = axq_xq_bytes(AXQ_XQ_MAX_K), mb_bytes = (size_t)34 * AXQ_BATCH_MAX_K; // one vector split, or a small batch packed
+        INIT_HIP(hipMalloc((void **)&ctx->xq, xq_bytes > mb_bytes ? xq_bytes : mb_bytes));
+    }
     // A lone GEMV call splits x inside the kernel (one launch); callers that produce x on the device
     // hand over the split form instead.  AXQ_GEMV_PREP=separate forces the two-kernel form (development).
     const char *prep = getenv("AXQ_GEMV_PREP");

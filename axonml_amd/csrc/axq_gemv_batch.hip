@@ -7,8 +7,9 @@
 // (n, h) = (lane % 32, lane / 32) supplies 16 of the block's codes of row n and receives D[4 b + l][n] for
 // b = h, h + 2, h + 4, h + 6: all four limbs of four vectors, which it recombines and scales by itself.
 //
-// A workgroup owns 32 weight rows; its S = K / 512 <= 8 waves split K (16 blocks each) and keep their A operands
-// in registers; the partial sums of the waves meet in LDS and are added in a fixed order.  The split form of
+// A workgroup owns 32 weight rows; its up to 8 waves take the row's chunks of 16 blocks (512 weights) in turn,
+// the A operands of a chunk in registers; the partial sums of the waves meet in LDS and are added in a fixed
+// order.  K is a multiple of 256, so a row's last chunk holds 16 or 8 blocks.  The split form of
 // the batch is made once, by a small kernel in front (a workgroup could not afford to split eight vectors
 // for its 32 rows).
 #include <hip/hip_fp16.h>
@@ -61,13 +62,18 @@ struct MQ4x {
     static constexpr bool EVEN_ODD = true;
     static constexpr bool OFFSET = WITH_MIN;
     struct Raw { u32x4 q[UNITS]; u32x4 m[WITH_MIN ? 4 : 2]; };
-    __device__ static void load(const MbArgs &a, size_t row, int blk0, int, Raw &r) {
-        const uint8_t *codes = a.codes + row * a.codes_pitch + (size_t)blk0 * 16;
-        const uint8_t *meta = a.meta + row * a.meta_pitch + (size_t)blk0 * (WITH_MIN ? 4 : 2);
+    // blocks past the end of the row (the second half of a short last chunk) re-read its last block / vector
+    __device__ static void load(const MbArgs &a, size_t row, int blk0, int, int nblk, Raw &r) {
+        const uint8_t *codes = a.codes + row * a.codes_pitch;
+        const uint8_t *meta = a.meta + row * a.meta_pitch;
+        constexpr int PER = WITH_MIN ? 4 : 8; // blocks per 16-byte vector of scales
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) r.q[u] = ldg16(codes + u * 16);
+        for (int u = 0; u < UNITS; u++) { const int b = blk0 + u < nblk ? blk0 + u : nblk - 1; r.q[u] = ldg16(codes + (size_t)b * 16); }
 #pragma unroll
-        for (int i = 0; i < (WITH_MIN ? 4 : 2); i++) r.m[i] = ldg16(meta + i * 16);
+        for (int i = 0; i < (WITH_MIN ? 4 : 2); i++) {
+            const int v = blk0 / PER + i < nblk / PER ? blk0 / PER + i : nblk / PER - 1;
+            r.m[i] = ldg16(meta + (size_t)v * 16);
+        }
     }
     __device__ static int4v operand(const Raw &r, int u, int h) {
         const int sh = 4 * h;
@@ -93,13 +99,16 @@ struct MQ80 {
     static constexpr bool EVEN_ODD = false;
     static constexpr bool OFFSET = false;
     struct Raw { u32x4 q[UNITS]; u32x4 m[2]; };
-    __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, Raw &r) {
-        const uint8_t *codes = a.codes + row * a.codes_pitch + (size_t)blk0 * 32 + h * 16;
-        const uint8_t *meta = a.meta + row * a.meta_pitch + (size_t)blk0 * 2;
+    __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, int nblk, Raw &r) {
+        const uint8_t *codes = a.codes + row * a.codes_pitch + h * 16;
+        const uint8_t *meta = a.meta + row * a.meta_pitch;
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) r.q[u] = ldg16(codes + u * 32);
-        r.m[0] = ldg16(meta);
-        r.m[1] = ldg16(meta + 16);
+        for (int u = 0; u < UNITS; u++) { const int b = blk0 + u < nblk ? blk0 + u : nblk - 1; r.q[u] = ldg16(codes + (size_t)b * 32); }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int v = blk0 / 8 + i < nblk / 8 ? blk0 / 8 + i : nblk / 8 - 1;
+            r.m[i] = ldg16(meta + (size_t)v * 16);
+        }
     }
     __device__ static int4v operand(const Raw &r, int u, int) {
         int4v b = {(int)r.q[u][0], (int)r.q[u][1], (int)r.q[u][2], (int)r.q[u][3]};
@@ -118,18 +127,19 @@ struct MQ4K {
     static constexpr bool EVEN_ODD = false;
     static constexpr bool OFFSET = true;
     struct Raw { u32x4 q[UNITS / 2]; u32x4 h[UNITS / 8]; };
-    __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, Raw &r) {
+    __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, int nblk, Raw &r) {
         const int cpr = a.k >> 6;          // pairs per row
-        const int pair0 = blk0 >> 1;       // the wave's first pair; 8 pairs = 2 superblocks, inside one 64-pair slice
+        const int pair0 = blk0 >> 1;       // the chunk's first pair; 8 pairs = 2 superblocks, inside one 64-pair slice
         const int slice = pair0 >> 6, pr = pair0 & 63;
         int P = cpr - (slice << 6);
         P = P < 64 ? P : 64;
+        const int np = (nblk - blk0) >> 1; // pairs of the chunk inside the row: 8, or 4 for a short last chunk
         const uint8_t *codes = a.codes + row * a.codes_pitch + (size_t)slice * 2048 + (size_t)h * 16 * P + (size_t)pr * 16;
         const uint8_t *meta = a.meta + row * a.meta_pitch + (size_t)(pair0 >> 2) * 16;
 #pragma unroll
-        for (int p = 0; p < UNITS / 2; p++) r.q[p] = ldg16(codes + p * 16);
+        for (int p = 0; p < UNITS / 2; p++) r.q[p] = ldg16(codes + (p < np ? p : np - 1) * 16);
 #pragma unroll
-        for (int s = 0; s < UNITS / 8; s++) r.h[s] = ldg16(meta + s * 16);
+        for (int s = 0; s < UNITS / 8; s++) r.h[s] = ldg16(meta + (4 * s < np ? s : 0) * 16);
     }
     __device__ static int4v operand(const Raw &r, int u, int) {
         const int sh = 4 * (u & 1);
@@ -174,42 +184,50 @@ __global__ void __launch_bounds__(512) gemv_mb_kernel(MbArgs a) {
     float *xss = sgs + (size_t)nblk * 8;   // same layout: plain sums of x over the group (contiguous with sgs)
     float *red = xss + (size_t)nblk * 8;   // [wave][vector][row]
 
-    // 1. this lane's A operands for the wave's 16 blocks: one contiguous kilobyte per wave and block
-    int4v A[UNITS];
-#pragma unroll
-    for (int u = 0; u < UNITS; u++) {
-        const u32x4 v = ldg16(a.xa + ((size_t)((wave * UNITS + u) * 2 + h) * 32 + n) * 16);
-        A[u] = int4v{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
-    }
     // scales and sums of all vectors -> LDS (already in the order the lanes read them)
     for (int t = tid; t < nblk * 4; t += (int)blockDim.x)
         reinterpret_cast<float4 *>(lds_f)[t] = reinterpret_cast<const float4 *>(a.xsg)[t];
-    // 2. the weights of this wave: 32 rows x 16 blocks, all requested at once
     const int row0 = blockIdx.x * 32;
     int row = row0 + n;
     row = row < a.n_rows ? row : a.n_rows - 1;
-    typename T::Raw raw;
-    T::load(a, (size_t)row, wave * UNITS, h, raw);
     __syncthreads();
 
-    // 3. one MFMA per block; the lane scales and adds its four vectors
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const int nchunks = (nblk + UNITS - 1) / UNITS;
+    for (int c = wave; c < nchunks; c += S) {
+        const int blk0 = c * UNITS;
+        const int nu = nblk - blk0 < UNITS ? nblk - blk0 : UNITS;
+        // 1. this lane's A operands for the chunk's blocks: one contiguous kilobyte per wave and block
+        int4v A[UNITS];
 #pragma unroll
-    for (int u = 0; u < UNITS; u++) {
-        const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        const int16v D = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[u], T::operand(raw, u, h), zero, 0, 0, 0);
-        float d, mo;
-        T::coef(raw, u, d, mo);
-        const int g = wave * UNITS + u;
-        const float4 sg4 = *reinterpret_cast<const float4 *>(sgs + (size_t)(g * 2 + h) * 4);
-        const float sgv[4] = {sg4.x, sg4.y, sg4.z, sg4.w};
+        for (int u = 0; u < UNITS; u++) {
+            const int b = u < nu ? blk0 + u : blk0;
+            const u32x4 v = ldg16(a.xa + ((size_t)(b * 2 + h) * 32 + n) * 16);
+            A[u] = int4v{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
+        }
+        // 2. the weights of the chunk: 32 rows x 16 blocks, all requested at once
+        typename T::Raw raw;
+        T::load(a, (size_t)row, blk0, h, nblk, raw);
+        // 3. one MFMA per block; the lane scales and adds its four vectors
 #pragma unroll
-        for (int bi = 0; bi < 4; bi++)
-            acc[bi] = fmaf(d * sgv[bi], recombine4(D[4 * bi], D[4 * bi + 1], D[4 * bi + 2], D[4 * bi + 3]), acc[bi]);
-        if (T::OFFSET) {
-            const float4 xs4 = *reinterpret_cast<const float4 *>(xss + (size_t)(g * 2 + h) * 4);
-            acc[0] = fmaf(mo, xs4.x, acc[0]); acc[1] = fmaf(mo, xs4.y, acc[1]);
-            acc[2] = fmaf(mo, xs4.z, acc[2]); acc[3] = fmaf(mo, xs4.w, acc[3]);
+        for (int u = 0; u < UNITS; u++) {
+            if (u < nu) {
+                const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                const int16v D = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[u], T::operand(raw, u, h), zero, 0, 0, 0);
+                float d, mo;
+                T::coef(raw, u, d, mo);
+                const int g = blk0 + u;
+                const float4 sg4 = *reinterpret_cast<const float4 *>(sgs + (size_t)(g * 2 + h) * 4);
+                const float sgv[4] = {sg4.x, sg4.y, sg4.z, sg4.w};
+#pragma unroll
+                for (int bi = 0; bi < 4; bi++)
+                    acc[bi] = fmaf(d * sgv[bi], recombine4(D[4 * bi], D[4 * bi + 1], D[4 * bi + 2], D[4 * bi + 3]), acc[bi]);
+                if (T::OFFSET) {
+                    const float4 xs4 = *reinterpret_cast<const float4 *>(xss + (size_t)(g * 2 + h) * 4);
+                    acc[0] = fmaf(mo, xs4.x, acc[0]); acc[1] = fmaf(mo, xs4.y, acc[1]);
+                    acc[2] = fmaf(mo, xs4.z, acc[2]); acc[3] = fmaf(mo, xs4.w, acc[3]);
+                }
+            }
         }
     }
     // 4. partial sums of the waves -> y, in wave order
@@ -271,7 +289,7 @@ void launch_mb(axq_ctx *ctx, const MbArgs &a, const float *x) {
     const dim3 pgrid((unsigned)((a.k / 8 + 255) / 256), MAX_BATCH);
     pack_x_kernel<T::EVEN_ODD><<<pgrid, 256, 0, ctx->stream>>>(x, a.k, a.batch, const_cast<uint8_t *>(a.xa),
                                                                const_cast<float *>(a.xsg));
-    const unsigned S = (unsigned)(a.k / WAVE_K);
+    const unsigned chunks = (unsigned)((a.k + WAVE_K - 1) / WAVE_K), S = chunks < 8 ? chunks : 8;
     const unsigned grid = (unsigned)((a.n_rows + 31) / 32);
     const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float);
     gemv_mb_kernel<T><<<grid, 64 * S, lds, ctx->stream>>>(a);
@@ -282,8 +300,7 @@ void launch_mb(axq_ctx *ctx, const MbArgs &a, const float *x) {
 // Whether the batched kernel covers this call.
 bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch) {
     if (batch < 2 || batch > MAX_BATCH) return false;
-    // at most 8 waves: a lane holds 64 registers of A operands and 64 of weights, more than a 16-wave workgroup may
-    if (w->k % WAVE_K != 0 || w->k > 8 * WAVE_K) return false; // 34 k bytes of scratch fit the context's x buffer
+    if (w->k % 256 != 0 || w->k > AXQ_BATCH_MAX_K) return false; // 34 k bytes of scratch: the context's x buffer holds that much
     return w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q8_0 || w->type == AXQ_Q4_K;
 }
 

@@ -255,7 +255,8 @@ def main():
     if not args.no_extras:
         cases = [(T.Q4_K, 4096, 14336, 1, 0.01), (T.Q8_0, 4096, 4096, 1, 0.0), (T.Q4_0, 11008, 4096, 1, 0.0),
                  (T.Q4_0, 4096, 11008, 1, 0.0), (T.Q4_1, 11008, 4096, 1, 0.0), (T.Q4_1, 4096, 11008, 1, 0.0),
-                 (T.Q4_0, 11008, 4096, 8, 0.0), (T.Q4_1, 11008, 4096, 8, 0.0)]
+                 (T.Q4_0, 11008, 4096, 8, 0.0), (T.Q4_1, 11008, 4096, 8, 0.0), (T.Q4_0, 4096, 11008, 8, 0.0),
+                 (T.Q4_1, 4096, 11008, 8, 0.0)]
         gem = []
         for qt, n, k, b, op in cases:
             r, ws2, _, xd, yd = gemv_case(ctx, qt, n, k, b, max(200, args.steps // 4), 50, outlier_p=op)

@@ -138,7 +138,8 @@ def test_gemv_shape_errors(ctx):
 
 # ---- small batches: one pass over the weights for up to eight vectors (v_mfma_i32_32x32x32_i8 path)
 @pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q8_0, o.Q4_K])
-@pytest.mark.parametrize("batch,n,k", [(2, 32, 512), (3, 100, 1024), (8, 96, 4096), (8, 33, 512), (11, 64, 2048), (16, 40, 4096)])
+@pytest.mark.parametrize("batch,n,k", [(2, 32, 512), (3, 100, 1024), (8, 96, 4096), (8, 33, 512), (11, 64, 2048), (16, 40, 4096),
+                                       (2, 32, 256), (8, 33, 768), (8, 40, 11008), (5, 64, 14336), (8, 32, 16384)])
 def test_small_batch_reads_weights_once(ctx, qtype, batch, n, k):
     rng = np.random.default_rng(batch * 1000 + n + k + qtype)
     w = gen_weight(rng, n, k)
@@ -155,14 +156,15 @@ def test_small_batch_reads_weights_once(ctx, qtype, batch, n, k):
     assert max_rel_err(got, exact, STRICT_FLOOR) <= MATMUL_RTOL
     # the batched kernel and the one-vector kernel agree far inside the tolerance
     one = np.stack([q.quantized_matmul(x[i:i + 1], dw, bias, ctx)[0] for i in range(batch)])
-    assert max_rel_err(got, one, STRICT_FLOOR) <= 1e-4
+    assert max_rel_err(got, one, STRICT_FLOOR) <= 3e-4  # f32 summation orders differ; at this floor that is the noise
     dw.free()
 
 
-def test_small_batch_config_shape(ctx):
-    # BASELINE config 2: 11008 x 4096, batch 8, Q4_0 and Q4_1
+@pytest.mark.parametrize("n,k", [(11008, 4096), (4096, 11008)])
+def test_small_batch_config_shape(ctx, n, k):
+    # BASELINE config 2: 11008 x 4096 and the transposed down-projection shape, batch 8, Q4_0 and Q4_1
     rng = np.random.default_rng(82)
-    n, k, batch = 11008, 4096, 8
+    batch = 8
     w = gen_weight(rng, n, k)
     x = rng.standard_normal((batch, k)).astype(np.float32)
     for qtype in (o.Q4_0, o.Q4_1):
