@@ -186,7 +186,8 @@ int axq_init(int device, axq_ctx **out) {
     }
     ctx->fp8_unit_inv = 1.0f / h[0];
     {
-        size_t xq_bytes = axq_xq_bytes(AXQ_XQ_MAX_K), mb_bytes = (size_t)34 * AXQ_BATCH_MAX_K; // one vector split, or a small batch packed
+        // one vector split, or a small batch packed plus the partial sums of its split K
+        size_t xq_bytes = axq_xq_bytes(AXQ_XQ_MAX_K), mb_bytes = (size_t)34 * AXQ_BATCH_MAX_K + (size_t)4 * 8 * AXQ_BATCH_SPLIT_ROWS * 4;
         INIT_HIP(hipMalloc((void **)&ctx->xq, xq_bytes > mb_bytes ? xq_bytes : mb_bytes));
     }
     // A lone GEMV call splits x inside the kernel (one launch); callers that produce x on the device

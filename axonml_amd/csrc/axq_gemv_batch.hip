@@ -2,7 +2,7 @@
 //
 // The weights are read once for the whole batch.  The dot products run on v_mfma_i32_32x32x32_i8 with
 //   A (32 x 32): row 4 b + l = limb l of activation vector b (the split form of axq_split.h), 32 k of one block,
-//   B (32 x 32): column n = one of 32 weight rows, the block's 32 codes as signed bytes,
+//   B (32 x 32): column n = one of 32 weight rows, the block's 32 codes as bytes (4-bit codes as they are, 0..15),
 // so one instruction multiplies a 32-element block of 32 weight rows with all vectors and limbs.  Lane
 // (n, h) = (lane % 32, lane / 32) supplies 16 of the block's codes of row n and receives D[4 b + l][n] for
 // b = h, h + 2, h + 4, h + 6: all four limbs of four vectors, which it recombines and scales by itself.
@@ -23,7 +23,7 @@ typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int UNITS = 16;      // 32-element blocks per wave
+constexpr int UNITS = 8;       // 32-element blocks per wave and chunk
 constexpr int WAVE_K = 32 * UNITS;
 constexpr int MAX_BATCH = 8;
 
@@ -34,20 +34,19 @@ struct MbArgs {
     const float *xsg;   // [block][h][4]: group scales of vectors h, h + 2, h + 4, h + 6; then the plain sums, same layout
     const float *bias;
     float *y;
+    float *ypart; // K split over several workgroups: [split][batch][n_rows] partial sums, added by mb_reduce_kernel
     int n_rows, k, batch;
+    int chunks_per_split; // chunks of a row that one workgroup (blockIdx.y) takes
 };
 
 __device__ inline float f16lo(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v & 0xFFFF))); }
 __device__ inline float f16hi(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v >> 16))); }
-// four unsigned nibble codes in the low nibbles of the four bytes -> four signed bytes (code - 8)
-__device__ inline int minus8(uint32_t t) { return (int)((((t | 0x80808080u) - 0x08080808u)) ^ 0x80808080u); }
 __device__ inline u32x4 ldg16(const uint8_t *p) { return *reinterpret_cast<const u32x4 *>(p); }
 
 // sum_k n_k x_k over one 32-element block of one vector from its four limb sums (limb 0 most significant)
 __device__ inline float recombine4(int d0, int d1, int d2, int d3) {
-    float f = fmaf((float)d0, 128.0f, (float)d1);
-    f = fmaf(f, 128.0f, (float)d2);
-    return fmaf(f, 128.0f, (float)d3);
+    // |d_i| <= 32 * 127 * 64 < 2^18: two limbs combine exactly in an integer (< 2^25 ... the f32 of it rounds like the fma chain would)
+    return fmaf((float)(d0 * 128 + d1), 16384.0f, (float)(d2 * 128 + d3));
 }
 
 // ---------------------------------------------------------------------------
@@ -55,13 +54,15 @@ __device__ inline float recombine4(int d0, int d1, int d2, int d3) {
 // h = lane / 32 says which 16 of a block's 32 codes the lane supplies.
 //   EVEN_ODD : h = 0 supplies the even elements, h = 1 the odd ones (reference nibble order); otherwise
 //              h = 0 supplies elements 0..15, h = 1 elements 16..31
-//   coef()   : w = d * (code - CENTRE) + mo, CENTRE = 8 for the 4-bit types
+//   coef()   : w = d * code + mo (the 4-bit codes unsigned: the integer sums are exact, and the two f32 terms
+//              that then cancel for an activation with a mean are each rounded once)
 // ---------------------------------------------------------------------------
 template <bool WITH_MIN>
 struct MQ4x {
     static constexpr bool EVEN_ODD = true;
-    static constexpr bool OFFSET = WITH_MIN;
-    struct Raw { u32x4 q[UNITS]; u32x4 m[WITH_MIN ? 4 : 2]; };
+    static constexpr bool OFFSET = true; // w = d * code + mo with mo = min (Q4_1) or -8 d (Q4_0): the codes stay unsigned
+    static constexpr int NV = UNITS * (WITH_MIN ? 4 : 2) / 16 > 0 ? UNITS * (WITH_MIN ? 4 : 2) / 16 : 1; // 16-byte vectors of scales per chunk
+    struct Raw { u32x4 q[UNITS]; u32x4 m[NV]; };
     // blocks past the end of the row (the second half of a short last chunk) re-read its last block / vector
     __device__ static void load(const MbArgs &a, size_t row, int blk0, int, int nblk, Raw &r) {
         const uint8_t *codes = a.codes + row * a.codes_pitch;
@@ -70,7 +71,7 @@ struct MQ4x {
 #pragma unroll
         for (int u = 0; u < UNITS; u++) { const int b = blk0 + u < nblk ? blk0 + u : nblk - 1; r.q[u] = ldg16(codes + (size_t)b * 16); }
 #pragma unroll
-        for (int i = 0; i < (WITH_MIN ? 4 : 2); i++) {
+        for (int i = 0; i < NV; i++) {
             const int v = blk0 / PER + i < nblk / PER ? blk0 / PER + i : nblk / PER - 1;
             r.m[i] = ldg16(meta + (size_t)v * 16);
         }
@@ -79,18 +80,18 @@ struct MQ4x {
         const int sh = 4 * h;
         int4v b;
 #pragma unroll
-        for (int i = 0; i < 4; i++) b[i] = minus8((r.q[u][i] >> sh) & 0x0F0F0F0Fu);
+        for (int i = 0; i < 4; i++) b[i] = (int)((r.q[u][i] >> sh) & 0x0F0F0F0Fu);
         return b;
     }
     __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
         if (WITH_MIN) {
             const uint32_t v = r.m[u >> 2][u & 3];
             d = f16lo(v);
-            mo = fmaf(8.0f, d, f16hi(v));
+            mo = f16hi(v);
         } else {
             const uint32_t v = r.m[u >> 3][(u >> 1) & 3];
             d = (u & 1) ? f16hi(v) : f16lo(v);
-            mo = 0.f;
+            mo = -8.0f * d;
         }
     }
 };
@@ -98,14 +99,15 @@ struct MQ4x {
 struct MQ80 {
     static constexpr bool EVEN_ODD = false;
     static constexpr bool OFFSET = false;
-    struct Raw { u32x4 q[UNITS]; u32x4 m[2]; };
+    static constexpr int NV = UNITS / 8 > 0 ? UNITS / 8 : 1;
+    struct Raw { u32x4 q[UNITS]; u32x4 m[NV]; };
     __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, int nblk, Raw &r) {
         const uint8_t *codes = a.codes + row * a.codes_pitch + h * 16;
         const uint8_t *meta = a.meta + row * a.meta_pitch;
 #pragma unroll
         for (int u = 0; u < UNITS; u++) { const int b = blk0 + u < nblk ? blk0 + u : nblk - 1; r.q[u] = ldg16(codes + (size_t)b * 32); }
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < NV; i++) {
             const int v = blk0 / 8 + i < nblk / 8 ? blk0 / 8 + i : nblk / 8 - 1;
             r.m[i] = ldg16(meta + (size_t)v * 16);
         }
@@ -145,7 +147,7 @@ struct MQ4K {
         const int sh = 4 * (u & 1);
         int4v b;
 #pragma unroll
-        for (int i = 0; i < 4; i++) b[i] = minus8((r.q[u >> 1][i] >> sh) & 0x0F0F0F0Fu);
+        for (int i = 0; i < 4; i++) b[i] = (int)((r.q[u >> 1][i] >> sh) & 0x0F0F0F0Fu);
         return b;
     }
     __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
@@ -164,7 +166,7 @@ struct MQ4K {
         }
         const float dd = f16lo(h[0]), dmin = f16hi(h[0]);
         d = dd * (float)sc;
-        mo = fmaf(8.0f, d, -(dmin * (float)mn));
+        mo = -(dmin * (float)mn);
     }
 };
 
@@ -174,7 +176,7 @@ __device__ inline int pick_alt(uint32_t lo, uint32_t hi, int sel) {
 }
 
 template <class T>
-__global__ void __launch_bounds__(512) gemv_mb_kernel(MbArgs a) {
+__global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
     extern __shared__ float lds_f[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int S = (int)blockDim.x >> 6;
@@ -194,7 +196,8 @@ __global__ void __launch_bounds__(512) gemv_mb_kernel(MbArgs a) {
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     const int nchunks = (nblk + UNITS - 1) / UNITS;
-    for (int c = wave; c < nchunks; c += S) {
+    const int c_lo = (int)blockIdx.y * a.chunks_per_split, c_hi = c_lo + a.chunks_per_split < nchunks ? c_lo + a.chunks_per_split : nchunks;
+    for (int c = c_lo + wave; c < c_hi; c += S) {
         const int blk0 = c * UNITS;
         const int nu = nblk - blk0 < UNITS ? nblk - blk0 : UNITS;
         // 1. this lane's A operands for the chunk's blocks: one contiguous kilobyte per wave and block
@@ -239,8 +242,12 @@ __global__ void __launch_bounds__(512) gemv_mb_kernel(MbArgs a) {
         if (row0 + r < a.n_rows) {
             float tot = 0.f;
             for (int w = 0; w < S; w++) tot += red[((size_t)w * MAX_BATCH + b) * 32 + r];
-            if (a.bias) tot += a.bias[row0 + r];
-            a.y[(size_t)b * a.n_rows + row0 + r] = tot;
+            if (a.ypart) {
+                a.ypart[((size_t)blockIdx.y * a.batch + b) * a.n_rows + row0 + r] = tot;
+            } else {
+                if (a.bias) tot += a.bias[row0 + r];
+                a.y[(size_t)b * a.n_rows + row0 + r] = tot;
+            }
         }
     }
 }
@@ -284,15 +291,38 @@ __global__ void __launch_bounds__(256) pack_x_kernel(const float *x, int k, int 
     }
 }
 
+// y = sum over the splits, in order (+ bias)
+__global__ void __launch_bounds__(256) mb_reduce_kernel(const float *ypart, const float *bias, int n_rows, int batch, int splits, float *y) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x, total = n_rows * batch;
+    if (i >= total) return;
+    float tot = ypart[i];
+    for (int z = 1; z < splits; z++) tot += ypart[(size_t)z * total + i];
+    if (bias) tot += bias[i % n_rows];
+    y[i] = tot;
+}
+
 template <class T>
-void launch_mb(axq_ctx *ctx, const MbArgs &a, const float *x) {
+void launch_mb(axq_ctx *ctx, MbArgs a, const float *x) {
     const dim3 pgrid((unsigned)((a.k / 8 + 255) / 256), MAX_BATCH);
     pack_x_kernel<T::EVEN_ODD><<<pgrid, 256, 0, ctx->stream>>>(x, a.k, a.batch, const_cast<uint8_t *>(a.xa),
                                                                const_cast<float *>(a.xsg));
-    const unsigned chunks = (unsigned)((a.k + WAVE_K - 1) / WAVE_K), S = chunks < 8 ? chunks : 8;
-    const unsigned grid = (unsigned)((a.n_rows + 31) / 32);
+    const unsigned chunks = (unsigned)((a.k + WAVE_K - 1) / WAVE_K);
+    const unsigned tiles = (unsigned)((a.n_rows + 31) / 32);
+    // few row tiles (a narrow output): split K over up to four workgroups per tile so that the chip is full
+    unsigned splits = (unsigned)ctx->prop.multiProcessorCount / tiles;
+    splits = splits > 4 ? 4 : splits;
+    if (splits > chunks / 8) splits = chunks / 8;
+    if (splits < 2) splits = 1;
+    a.chunks_per_split = (int)((chunks + splits - 1) / splits);
+    splits = (chunks + a.chunks_per_split - 1) / a.chunks_per_split;
+    if (splits < 2) a.ypart = nullptr;
+    const unsigned S = (unsigned)a.chunks_per_split < 8 ? (unsigned)a.chunks_per_split : 8;
     const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float);
-    gemv_mb_kernel<T><<<grid, 64 * S, lds, ctx->stream>>>(a);
+    gemv_mb_kernel<T><<<dim3(tiles, splits), 64 * S, lds, ctx->stream>>>(a);
+    if (splits > 1) {
+        const int total = a.n_rows * a.batch;
+        mb_reduce_kernel<<<(total + 255) / 256, 256, 0, ctx->stream>>>(a.ypart, a.bias, a.n_rows, a.batch, (int)splits, a.y);
+    }
 }
 
 } // namespace
@@ -315,6 +345,8 @@ int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int ba
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch;
     a.xa = xa; a.xsg = xsg;
     a.bias = bias; a.y = y;
+    // partial sums of a split K behind the x operands (splits only happen below AXQ_BATCH_SPLIT_ROWS rows)
+    a.ypart = w->n_rows <= AXQ_BATCH_SPLIT_ROWS ? reinterpret_cast<float *>(ctx->xq + (size_t)34 * AXQ_BATCH_MAX_K) : nullptr;
     a.n_rows = (int)w->n_rows; a.k = k; a.batch = batch;
     switch (w->type) {
     case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, x); break;

@@ -56,6 +56,7 @@ struct axq_weight {
 
 #define AXQ_XQ_MAX_K 65536
 #define AXQ_BATCH_MAX_K 16384 // widest weight of the small-batch GEMV: its x operands take 34 bytes per element of K
+#define AXQ_BATCH_SPLIT_ROWS 8192 // it splits K only for weights of at most this many rows: 4 splits x 8 vectors of partial sums
 
 static inline size_t axq_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
