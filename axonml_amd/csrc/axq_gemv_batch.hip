@@ -63,13 +63,13 @@ struct MQ4x {
     static constexpr bool OFFSET = true; // w = d * code + mo with mo = min (Q4_1) or -8 d (Q4_0): the codes stay unsigned
     static constexpr int NV = UNITS * (WITH_MIN ? 4 : 2) / 16 > 0 ? UNITS * (WITH_MIN ? 4 : 2) / 16 : 1; // 16-byte vectors of scales per chunk
     struct Raw { u32x4 q[UNITS]; u32x4 m[NV]; };
-    // blocks past the end of the row (the second half of a short last chunk) re-read its last block / vector
-    __device__ static void load(const MbArgs &a, size_t row, int blk0, int, int nblk, Raw &r) {
-        const uint8_t *codes = a.codes + row * a.codes_pitch;
+    // the chunk's codes of one row: NP 16-byte pieces, piece p = block blk0 + p; a lane wants piece u for block u
+    static constexpr int NP = UNITS, NQ = UNITS;
+    __device__ static size_t piece_off(const MbArgs &, int blk0, int p) { return (size_t)(blk0 + p) * 16; }
+    __device__ static int want(int j, int) { return j; }
+    __device__ static void load_meta(const MbArgs &a, size_t row, int blk0, int nblk, Raw &r) {
         const uint8_t *meta = a.meta + row * a.meta_pitch;
         constexpr int PER = WITH_MIN ? 4 : 8; // blocks per 16-byte vector of scales
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) { const int b = blk0 + u < nblk ? blk0 + u : nblk - 1; r.q[u] = ldg16(codes + (size_t)b * 16); }
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             const int v = blk0 / PER + i < nblk / PER ? blk0 / PER + i : nblk / PER - 1;
@@ -101,11 +101,12 @@ struct MQ80 {
     static constexpr bool OFFSET = false;
     static constexpr int NV = UNITS / 8 > 0 ? UNITS / 8 : 1;
     struct Raw { u32x4 q[UNITS]; u32x4 m[NV]; };
-    __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, int nblk, Raw &r) {
-        const uint8_t *codes = a.codes + row * a.codes_pitch + h * 16;
+    // 32 code bytes per block: piece 2u + h = the h-th half of block blk0 + u
+    static constexpr int NP = 2 * UNITS, NQ = UNITS;
+    __device__ static size_t piece_off(const MbArgs &, int blk0, int p) { return (size_t)blk0 * 32 + (size_t)p * 16; }
+    __device__ static int want(int j, int h) { return 2 * j + h; }
+    __device__ static void load_meta(const MbArgs &a, size_t row, int blk0, int nblk, Raw &r) {
         const uint8_t *meta = a.meta + row * a.meta_pitch;
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) { const int b = blk0 + u < nblk ? blk0 + u : nblk - 1; r.q[u] = ldg16(codes + (size_t)b * 32); }
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             const int v = blk0 / 8 + i < nblk / 8 ? blk0 / 8 + i : nblk / 8 - 1;
@@ -129,19 +130,20 @@ struct MQ4K {
     static constexpr bool EVEN_ODD = false;
     static constexpr bool OFFSET = true;
     struct Raw { u32x4 q[UNITS / 2]; u32x4 h[UNITS / 8]; };
-    __device__ static void load(const MbArgs &a, size_t row, int blk0, int h, int nblk, Raw &r) {
+    // a chunk is one superblock = 4 pairs: pieces 0..3 = the first 16 bytes of its pairs, 4..7 = their second 16 bytes
+    static_assert(UNITS == 8, "one superblock per chunk");
+    static constexpr int NP = 8, NQ = 4;
+    __device__ static size_t piece_off(const MbArgs &a, int blk0, int p) {
         const int cpr = a.k >> 6;          // pairs per row
-        const int pair0 = blk0 >> 1;       // the chunk's first pair; 8 pairs = 2 superblocks, inside one 64-pair slice
+        const int pair0 = blk0 >> 1;       // the chunk's first pair; its 4 pairs lie inside one 64-pair slice
         const int slice = pair0 >> 6, pr = pair0 & 63;
         int P = cpr - (slice << 6);
         P = P < 64 ? P : 64;
-        const int np = (nblk - blk0) >> 1; // pairs of the chunk inside the row: 8, or 4 for a short last chunk
-        const uint8_t *codes = a.codes + row * a.codes_pitch + (size_t)slice * 2048 + (size_t)h * 16 * P + (size_t)pr * 16;
-        const uint8_t *meta = a.meta + row * a.meta_pitch + (size_t)(pair0 >> 2) * 16;
-#pragma unroll
-        for (int p = 0; p < UNITS / 2; p++) r.q[p] = ldg16(codes + (p < np ? p : np - 1) * 16);
-#pragma unroll
-        for (int s = 0; s < UNITS / 8; s++) r.h[s] = ldg16(meta + (4 * s < np ? s : 0) * 16);
+        return (size_t)slice * 2048 + (size_t)(p >> 2) * 16 * P + (size_t)(pr + (p & 3)) * 16;
+    }
+    __device__ static int want(int j, int h) { return 4 * h + j; }
+    __device__ static void load_meta(const MbArgs &a, size_t row, int blk0, int, Raw &r) {
+        r.h[0] = ldg16(a.meta + row * a.meta_pitch + (size_t)(blk0 >> 3) * 16);
     }
     __device__ static int4v operand(const Raw &r, int u, int) {
         const int sh = 4 * (u & 1);
@@ -185,6 +187,7 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
     float *sgs = lds_f;                    // [block of the row][h][4]: group scales of vectors h, h+2, h+4, h+6
     float *xss = sgs + (size_t)nblk * 8;   // same layout: plain sums of x over the group (contiguous with sgs)
     float *red = xss + (size_t)nblk * 8;   // [wave][vector][row]
+    u32x4 *patch = reinterpret_cast<u32x4 *>(red + (size_t)S * MAX_BATCH * 32) + (size_t)wave * 32 * T::NP; // this wave's 32 x NP pieces
 
     // scales and sums of all vectors -> LDS (already in the order the lanes read them)
     for (int t = tid; t < nblk * 4; t += (int)blockDim.x)
@@ -208,9 +211,30 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
             const u32x4 v = ldg16(a.xa + ((size_t)(b * 2 + h) * 32 + n) * 16);
             A[u] = int4v{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
         }
-        // 2. the weights of the chunk: 32 rows x 16 blocks, all requested at once
+        // 2. the weights of the chunk.  Codes: the wave fetches its 32 rows' pieces with whole runs per row (eight
+        //    or sixteen lanes side by side on one row) and turns them into "lane = row" through its LDS patch;
+        //    a lane reading 16 bytes of its own row per load would touch 32 cache lines per instruction.
+        constexpr int NP = T::NP, NI = NP / 2;
+        u32x4 stage[NI];
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const int idx = i * 64 + lane, r = idx / NP, pc = idx % NP;
+            const int gr = row0 + r < a.n_rows ? row0 + r : a.n_rows - 1;
+            stage[i] = ldg16(a.codes + (size_t)gr * a.codes_pitch + T::piece_off(a, blk0, pc));
+        }
         typename T::Raw raw;
-        T::load(a, (size_t)row, blk0, h, nblk, raw);
+        T::load_meta(a, (size_t)row, blk0, nblk, raw);
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const int idx = i * 64 + lane, r = idx / NP, pc = idx % NP;
+            patch[r * NP + (pc ^ (r & (NP - 1)))] = stage[i]; // rotated per row: the reads below spread over the banks
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the wave's LDS writes have landed
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int j = 0; j < T::NQ; j++) raw.q[j] = patch[n * NP + (T::want(j, h) ^ (n & (NP - 1)))];
         // 3. one MFMA per block; the lane scales and adds its four vectors
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
@@ -317,7 +341,12 @@ void launch_mb(axq_ctx *ctx, MbArgs a, const float *x) {
     splits = (chunks + a.chunks_per_split - 1) / a.chunks_per_split;
     if (splits < 2) a.ypart = nullptr;
     const unsigned S = (unsigned)a.chunks_per_split < 8 ? (unsigned)a.chunks_per_split : 8;
-    const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float);
+    const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float) + (size_t)S * 32 * T::NP * 16;
+    static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
+    if (lds > 64 * 1024 && !big_lds_allowed) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        big_lds_allowed = true;
+    }
     gemv_mb_kernel<T><<<dim3(tiles, splits), 64 * S, lds, ctx->stream>>>(a);
     if (splits > 1) {
         const int total = a.n_rows * a.batch;
