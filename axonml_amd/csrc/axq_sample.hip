@@ -36,8 +36,12 @@ struct SampleArgs {
     float *filtered_out;        // optional: the logits after all filters
 };
 
+constexpr int FAST_K = 128;   // top-k up to here takes the short path below ...
+constexpr int MAX_CAND = 256; // ... as long as its first cut leaves at most this many candidates
+
 struct Shared {
-    u64 hist[BINS];
+    u64 hist[BINS];        // radix histogram; the short path keeps its candidate list here afterwards
+    uint32_t tk[ST];       // one key per thread (the short path's thread maxima)
     u64 part[17];
     float fpart[16];
     int ipart[16];
@@ -222,10 +226,103 @@ __global__ void __launch_bounds__(ST) sample_kernel(SampleArgs a) {
         for (int i = tid; i < n; i += ST) w[ix(i)] = w[ix(i)] / a.temperature;
     __syncthreads();
     auto wkey = [&](int i) { return order_key(w[ix(i)]); };
-    float mx = -INFINITY;
+    float tmax = -INFINITY; // this thread's maximum over its strided share
 #pragma unroll 8
-    for (int i = tid; i < n; i += ST) mx = fmaxf(mx, w[ix(i)]);
-    mx = block_max(mx, sh);
+    for (int i = tid; i < n; i += ST) tmax = fmaxf(tmax, w[ix(i)]);
+    const float mx = block_max(tmax, sh);
+    // Short path for a small top-k (the usual 20 ... 100): the k largest logits lie among the elements that
+    // reach the k-th largest of the 1024 thread maxima (each thread's maximum over its strided share), usually
+    // little more than k of them.  Those candidates go into a list, one per thread, and everything after that
+    // -- exact top-k with ties by index, softmax, top-p, the draw -- works on the list with the same rules and
+    // the same exact sums as the long path, in a few loops over at most MAX_CAND entries.
+    if (a.top_k > 0 && a.top_k <= FAST_K && a.top_k < n) {
+        sh.tk[tid] = order_key(tmax);
+        if (tid == 0) sh.bc_i32[2] = 0;
+        __syncthreads();
+        uint32_t cut;
+        u64 unused;
+        (void)radix_select<false>(ST, (u64)a.top_k, [&](int i) { return sh.tk[i]; }, [](int) { return (u64)1; }, sh, &cut, &unused);
+        uint32_t *ckey = reinterpret_cast<uint32_t *>(sh.hist);
+        int *cidx = reinterpret_cast<int *>(ckey + MAX_CAND);
+        u64 *cfx = reinterpret_cast<u64 *>(cidx + MAX_CAND);
+#pragma unroll 8
+        for (int i = tid; i < n; i += ST) {
+            const uint32_t k = wkey(i);
+            if (k >= cut) {
+                const int slot = atomicAdd(&sh.bc_i32[2], 1);
+                if (slot < MAX_CAND) { ckey[slot] = k; cidx[slot] = i; }
+            }
+        }
+        __syncthreads();
+        const int m = sh.bc_i32[2];
+        if (m <= MAX_CAND) { // else: too many ties at the cut; the long path below handles it
+            const bool mine = tid < m;
+            const uint32_t key = mine ? ckey[tid] : 0;
+            const int idx = mine ? cidx[tid] : 0;
+            // exact top-k: rank in the reference's stable descending order
+            int rank = 0;
+            if (mine)
+                for (int j = 0; j < m; j++) rank += (ckey[j] > key) || (ckey[j] == key && cidx[j] < idx);
+            bool keep = mine && rank < a.top_k;
+            const float val = mine ? w[ix(idx)] : -INFINITY;
+            float ev = keep ? expf(val - mx) : 0.0f;
+            u64 total;
+            if (a.top_p >= 0.0f) {
+                (void)block_excl_scan(fx_of(ev), sh, &total);
+                const float sum = (float)((double)total * (1.0 / 1099511627776.0));
+                if (keep) ev = ev / sum; // now a probability; the draw below uses what is left of these
+                __syncthreads();
+                if (tid < MAX_CAND) ckey[tid] = keep ? __builtin_bit_cast(uint32_t, ev) : 0u;
+                __syncthreads();
+                // mass of everything that precedes this entry in descending order of probability (ties by index)
+                u64 before = 0;
+                if (keep)
+                    for (int j = 0; j < m; j++) {
+                        const uint32_t pj = ckey[j];
+                        const uint32_t pt = __builtin_bit_cast(uint32_t, ev);
+                        if (pj > pt || (pj == pt && pj != 0 && cidx[j] < idx)) before += fx_of(__builtin_bit_cast(float, pj));
+                    }
+                const u64 target = (u64)((double)a.top_p * 1099511627776.0);
+                if (keep && before > target) { keep = false; ev = 0.0f; } // the entry that crosses p itself stays
+                __syncthreads();
+            }
+            if (a.filtered_out) {
+#pragma unroll 8
+                for (int i = tid; i < n; i += ST) a.filtered_out[i] = -INFINITY;
+                __syncthreads();
+                if (keep) a.filtered_out[idx] = val;
+            }
+            if (!a.do_sample) { // the last of the equal maxima; the maximum is always kept
+                int best = (keep && val == mx) ? idx : -1;
+#pragma unroll
+                for (int s2 = 32; s2 >= 1; s2 >>= 1) { const int o = __shfl_xor(best, s2); best = o > best ? o : best; }
+                __syncthreads();
+                if ((tid & 63) == 0) sh.ipart[tid >> 6] = best;
+                __syncthreads();
+                if (tid == 0) {
+                    for (int wv = 1; wv < ST / 64; wv++) best = sh.ipart[wv] > best ? sh.ipart[wv] : best;
+                    a.out[0] = best < 0 ? 0 : best;
+                }
+                return;
+            }
+            // the draw: first entry in index order whose cumulative weight exceeds u times the total
+            (void)block_excl_scan(fx_of(ev), sh, &total);
+            __syncthreads();
+            if (tid < MAX_CAND) cfx[tid] = fx_of(ev);
+            __syncthreads();
+            const float u = a.counter_dev ? uniform_from(a.seed, (u64)*a.counter_dev) : a.u;
+            const u64 target = (u64)((double)u * (double)total);
+            u64 before = 0;
+            if (keep)
+                for (int j = 0; j < m; j++) before += cidx[j] < idx ? cfx[j] : 0;
+            if (tid == 0) sh.bc_i32[1] = n - 1; // the reference's fallback: the last token
+            __syncthreads();
+            if (keep && before <= target && target < before + fx_of(ev)) sh.bc_i32[1] = idx;
+            __syncthreads();
+            if (tid == 0) a.out[0] = sh.bc_i32[1];
+            return;
+        }
+    }
     // top-k: the k largest stay (ties: lower index first), the rest become -inf
     if (a.top_k > 0 && a.top_k < n) {
         uint32_t thr;

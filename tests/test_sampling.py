@@ -234,3 +234,33 @@ def test_model_generates_with_the_sampler(ctx, cfg):
     gpu.set_sampling(GenerationConfig.greedy(), 0)
     assert np.array_equal(gpu.generate(prompt, 8)[0], plain)
     gpu.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [300, 32000])
+def test_small_top_k_with_ties_at_the_cut(ctx, n):
+    # the short candidate-list path: six equal logits straddle rank k, the lower indices must win; then top-p and draws
+    rng = np.random.default_rng(n)
+    lg = _logits(rng, n, spread=2.0)
+    order = np.argsort(-lg, kind="stable")
+    tied = np.sort(order[36:42])
+    lg[tied] = lg[order[38]]
+    for top_p in (None, 0.7):
+        cfg = GenerationConfig(temperature=1.3, top_k=40, top_p=top_p, repetition_penalty=1.2, do_sample=True)
+        gen = rng.integers(0, n, size=50)
+        _, want = o.get_next_token(lg, gen, temperature=1.3, top_k=40, top_p=top_p, repetition_penalty=1.2, u=0.5)
+        g = TextGenerator(cfg, ctx)
+        _, f = g.get_next_token(lg, gen, u=0.5, return_filtered=True)
+        if top_p is None:
+            assert np.array_equal(f.view(np.uint32), want.view(np.uint32))
+            assert np.isfinite(f).sum() == 40
+        else:
+            _, pre = o.get_next_token(lg, gen, temperature=1.3, top_k=40, repetition_penalty=1.2, u=0.5)
+            cs = np.cumsum(np.sort(np.diff(np.concatenate([[0.0], _cdf64(pre)])))[::-1])
+            if np.abs(cs - top_p).min() >= MARGIN:
+                assert np.array_equal(np.isfinite(f), np.isfinite(want))
+        cdf = _cdf64(want)
+        for u in (0.01, 0.3, 0.62, 0.97):
+            if np.abs(cdf - u).min() >= MARGIN:
+                assert g.get_next_token(lg, gen, u=u) == o.get_next_token(lg, gen, temperature=1.3, top_k=40, top_p=top_p,
+                                                                           repetition_penalty=1.2, u=u)[0], (top_p, u)
