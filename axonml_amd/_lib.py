@@ -98,6 +98,7 @@ SIGNATURES = {
     "axq_model_random_init": (_i, [_vp, _i, C.c_float, C.c_uint64]),
     "axq_model_reset": (_i, [_vp]),
     "axq_model_forward": (_i, [_vp, C.c_int32, _vp, C.POINTER(C.c_int32)]),
+    "axq_model_forward_tokens": (_i, [_vp, _vp, _i, _vp, C.POINTER(C.c_int32)]),
     "axq_model_generate": (_i, [_vp, _vp, _i, _i, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "axq_model_seq_len": (_i, [_vp]),
     "axq_model_read_hidden": (_i, [_vp, _vp]),

@@ -41,6 +41,7 @@ struct axq_model {
     // activations
     float *h, *xn, *qkv, *att, *gu, *act, *logits;
     float *att_part;                // [kv_heads][max_splits][rep][head_dim + 2] partial attention results
+    float *pb_h, *pb_xn, *pb_qkv, *pb_att, *pb_gu, *pb_act; // the same activations for eight prompt tokens at a time
     int max_splits;
     // device-side state
     int32_t *pos, *tok, *next, *gen, *prompt, *out;
@@ -69,11 +70,12 @@ __device__ inline float block_sum(float v, float *scratch) {
     return t;
 }
 
-// h = embedding[tok] widened to f32 (Embedding::lookup, nn/src/layers/embedding.rs:103-146).
+// h = embedding[tok] widened to f32 (Embedding::lookup, nn/src/layers/embedding.rs:103-146); grid.y = tokens.
 __global__ void __launch_bounds__(256) embed_kernel(const uint16_t *emb, const int32_t *tok, float *h, int hidden) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (hidden >> 3)) return;
-    const uint4 raw = *reinterpret_cast<const uint4 *>(emb + (size_t)tok[0] * hidden + (size_t)t * 8);
+    h += (size_t)blockIdx.y * hidden;
+    const uint4 raw = *reinterpret_cast<const uint4 *>(emb + (size_t)tok[blockIdx.y] * hidden + (size_t)t * 8);
     const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
     float v[8];
 #pragma unroll
@@ -86,11 +88,14 @@ __global__ void __launch_bounds__(256) embed_kernel(const uint16_t *emb, const i
     o[1] = make_float4(v[4], v[5], v[6], v[7]);
 }
 
-// xn = rmsnorm(h) * w (RMSNorm::forward, llm/src/llama.rs:158-187).  One workgroup.  Only used in front of
-// linears that the matrix-pipe GEMV does not cover; otherwise the GEMV normalises its input itself.
+// xn = rmsnorm(h) * w (RMSNorm::forward, llm/src/llama.rs:158-187).  One workgroup per vector.  Used in front of
+// linears that the matrix-pipe GEMV does not cover (otherwise the GEMV normalises its input itself) and for
+// prompt tokens that go through the layers several at a time.
 __global__ void __launch_bounds__(1024) norm_kernel(const float *h, const float *w, int hidden, float eps, float *xn) {
     __shared__ float scratch[16];
     const int ntask = hidden >> 3;
+    h += (size_t)blockIdx.x * hidden;
+    xn += (size_t)blockIdx.x * hidden;
     float ss = 0.f;
     for (int t = threadIdx.x; t < ntask; t += blockDim.x) {
         const float4 *p = reinterpret_cast<const float4 *>(h + (size_t)t * 8);
@@ -359,11 +364,145 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, co
     }
 }
 
+// Prompt tokens go through the layers up to eight at a time (one pass over the weights serves all of them).
+// rope_append_kernel, grid (kv_heads, tokens), head_dim / 2 threads: RoPE on the new keys, keys and values
+// rounded to f16 into the cache at positions pos0 + b, exactly as the one-token kernel above writes them.
+constexpr int PROMPT_BATCH = 8;
+
+__global__ void __launch_bounds__(128) rope_append_kernel(const float *qkv, int qkv_rows, int q_dim, int kv_dim,
+                                                          const float *rope_cos, const float *rope_sin, uint16_t *kcache,
+                                                          uint16_t *vcache, int pos0, int max_pos, int d) {
+    const int half = d >> 1, e = threadIdx.x, kvh = blockIdx.x, p = pos0 + (int)blockIdx.y;
+    const float *row = qkv + (size_t)blockIdx.y * qkv_rows;
+    const float *kh = row + q_dim + (size_t)kvh * d, *vh = row + q_dim + kv_dim + (size_t)kvh * d;
+    const float nc = rope_cos[(size_t)p * half + e], ns = rope_sin[(size_t)p * half + e];
+    const float k1 = kh[e], k2 = kh[e + half];
+    uint16_t *kc = kcache + ((size_t)kvh * max_pos + p) * d, *vc = vcache + ((size_t)kvh * max_pos + p) * d;
+    kc[e] = __half_as_ushort(__float2half_rn(k1 * nc - k2 * ns));
+    kc[e + half] = __half_as_ushort(__float2half_rn(k1 * ns + k2 * nc));
+    vc[e] = __half_as_ushort(__float2half_rn(vh[e]));
+    vc[e + half] = __half_as_ushort(__float2half_rn(vh[e + half]));
+}
+
+// attn_prompt_kernel, grid (heads, tokens), 1024 threads: the query of head `head` at position p = pos0 + b
+// against the cached keys lo..p (causal, llama.rs:420-447; lo > 0 under a sliding window), all read from the
+// cache: scores into LDS, their maximum, exponentials and sum, then sum_j e_j v_j / sum.  Keys and values
+// are read 16 bytes per lane, head_dim / 8 lanes per position.
+template <int D>
+__global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int qkv_rows, const float *rope_cos,
+                                                           const float *rope_sin, const uint16_t *kcache,
+                                                           const uint16_t *vcache, int pos0, int n_heads, int n_kv,
+                                                           int max_pos, int window, float *att) {
+    constexpr int HALF = D / 2, LP = D / 8, PPB = 1024 / LP; // lanes per position, positions per pass of the workgroup
+    extern __shared__ float sc[];                            // scores, then exp(score - max)
+    __shared__ __attribute__((aligned(16))) float qs[D];
+    __shared__ float red[16];
+    __shared__ __attribute__((aligned(16))) float osum[16 * D];
+    const int head = blockIdx.x, b = blockIdx.y, p = pos0 + b;
+    const int rep = n_heads / n_kv, kvh = head / rep;
+    const int p_lo = (window > 0 && p + 1 > window) ? p + 1 - window : 0;
+    const int span = p + 1 - p_lo;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint16_t *kc = kcache + ((size_t)kvh * max_pos + p_lo) * D;
+    const uint16_t *vc = vcache + ((size_t)kvh * max_pos + p_lo) * D;
+    if (tid < HALF) {
+        const float *qh = qkv + (size_t)b * qkv_rows + (size_t)head * D;
+        const float c = rope_cos[(size_t)p * HALF + tid], s = rope_sin[(size_t)p * HALF + tid];
+        const float q1 = qh[tid], q2 = qh[tid + HALF];
+        qs[tid] = q1 * c - q2 * s;
+        qs[tid + HALF] = q1 * s + q2 * c;
+    }
+    __syncthreads();
+    const int c8 = tid % LP, r = tid / LP;
+    float qf[8];
+    {
+        const float4 *qp = reinterpret_cast<const float4 *>(qs + c8 * 8);
+        const float4 qa = qp[0], qb = qp[1];
+        qf[0] = qa.x; qf[1] = qa.y; qf[2] = qa.z; qf[3] = qa.w; qf[4] = qb.x; qf[5] = qb.y; qf[6] = qb.z; qf[7] = qb.w;
+    }
+    const float scale = 1.0f / sqrtf((float)D);
+    constexpr int UN = 4;
+    for (int j0 = 0; j0 < span; j0 += UN * PPB) {
+        uint4 raw[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int j = j0 + u * PPB + r;
+            raw[u] = *reinterpret_cast<const uint4 *>(kc + (size_t)(j < span ? j : 0) * D + c8 * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int j = j0 + u * PPB + r;
+            float kf[8];
+            halves_to_floats(raw[u], kf);
+            float s = qf[0] * kf[0];
+#pragma unroll
+            for (int e = 1; e < 8; e++) s = fmaf(qf[e], kf[e], s);
+            s = group_sum<LP>(s);
+            if (j < span && c8 == 0) sc[j] = s * scale;
+        }
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int j = tid; j < span; j += 1024) mx = fmaxf(mx, sc[j]);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = red[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) mx = fmaxf(mx, red[w]);
+    float sum = 0.f;
+    for (int j = tid; j < span; j += 1024) {
+        const float e = expf(sc[j] - mx);
+        sc[j] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, red); // its barriers also publish the exponentials
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j0 = 0; j0 < span; j0 += UN * PPB) {
+        uint4 raw[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int j = j0 + u * PPB + r;
+            raw[u] = *reinterpret_cast<const uint4 *>(vc + (size_t)(j < span ? j : 0) * D + c8 * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int j = j0 + u * PPB + r;
+            const float e = j < span ? sc[j] : 0.f;
+            float vf[8];
+            halves_to_floats(raw[u], vf);
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] = fmaf(e, vf[i], acc[i]);
+        }
+    }
+    // lanes of a wave that hold the same dims, then the sixteen waves in order
+#pragma unroll
+    for (int m = LP; m < 64; m <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] += __shfl_xor(acc[i], m);
+    }
+    if (lane < LP) {
+        float4 *dst = reinterpret_cast<float4 *>(osum + wave * D + c8 * 8);
+        dst[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    }
+    __syncthreads();
+    if (tid < D) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 16; w++) o += osum[w * D + tid];
+        att[(size_t)b * n_heads * D + (size_t)head * D + tid] = o / sum;
+    }
+}
+
 // act = silu(gate) * up over [inter]; gu alternates four gate values with the four up values of the same indices
-// (the row order of the fused gate/up weight).
+// (the row order of the fused gate/up weight); grid.y = vectors.
 __global__ void __launch_bounds__(256) swiglu_kernel(const float *gu, int inter, float *act) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x; // four consecutive outputs
     if (t >= (inter >> 2)) return;
+    gu += (size_t)blockIdx.y * 2 * inter;
+    act += (size_t)blockIdx.y * inter;
     const float4 g = *reinterpret_cast<const float4 *>(gu + (size_t)t * 8);
     const float4 u = *reinterpret_cast<const float4 *>(gu + (size_t)t * 8 + 4);
     float4 o;
@@ -432,6 +571,8 @@ __global__ void commit_next_kernel(const int32_t *next, int32_t *tok, int32_t *g
     gen[0] = g + 1;
 }
 __global__ void set_i32_kernel(int32_t *p, int32_t v) { p[0] = v; }
+__global__ void add_i32_kernel(int32_t *p, int32_t v) { p[0] += v; }
+__global__ void record_tokens_kernel(int32_t *hist, int pos0, const int32_t *toks) { hist[pos0 + threadIdx.x] = toks[threadIdx.x]; }
 __global__ void record_token_kernel(int32_t *hist, const int32_t *pos, const int32_t *tok) { hist[pos[0]] = tok[0]; }
 __global__ void fill_f32_kernel(float *p, size_t n, float v) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -606,6 +747,93 @@ int run_token(axq_model *m) {
                           m->sample_scratch, m->next, nullptr);
 }
 
+// Whether `nb` prompt tokens starting at position pos0 can go through the layers together: every linear of
+// the layers within the small-batch GEMV's reach, and the scores of the longest query within LDS.
+size_t prompt_attn_lds(const axq_model *m, int pos0, int nb) {
+    int span = pos0 + nb;
+    if (m->cfg.sliding_window > 0 && span > m->cfg.sliding_window) span = m->cfg.sliding_window;
+    return (size_t)((span + 255) / 256 * 256) * sizeof(float);
+}
+
+bool prompt_batch_covers(const axq_model *m, int pos0, int nb) {
+    if (nb < 2 || nb > PROMPT_BATCH) return false;
+    if (prompt_attn_lds(m, pos0, nb) > 128 * 1024) return false;
+    for (int l = 0; l < m->cfg.num_hidden_layers; l++)
+        for (const axq_weight *w : {m->w_qkv[l], m->w_o[l], m->w_gu[l], m->w_down[l]})
+            if (!axq_dev_gemv_batch_covers(w, nb)) return false;
+    return true;
+}
+
+template <int D>
+void launch_attn_prompt_d(axq_model *m, int l, int pos0, int nb, hipStream_t st) {
+    const axq_model_config &c = m->cfg;
+    const size_t per_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * D;
+    const size_t lds = prompt_attn_lds(m, pos0, nb);
+    static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
+    if (lds > 48 * 1024 && !big_lds_allowed) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prompt_kernel<D>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        big_lds_allowed = true;
+    }
+    attn_prompt_kernel<D><<<dim3(c.num_attention_heads, nb), 1024, lds, st>>>(
+        m->pb_qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + l * per_layer, m->vcache + l * per_layer, pos0,
+        c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, c.sliding_window, m->pb_att);
+}
+
+// The layers for prompt tokens toks[0..nb) (device memory) at positions pos0.., 2 <= nb <= 8: what nb steps
+// would leave in the KV cache, the history and the position counter, without the final norm and lm_head
+// (LLaMA::forward_with_cache on a multi-token input, llama.rs:731-762; its logits for all but the last
+// position are never looked at by generate, llama.rs:900-977).
+int enqueue_prompt_batch(axq_model *m, const int32_t *toks, int nb, int pos0) {
+    axq_ctx *ctx = m->ctx;
+    const axq_model_config &c = m->cfg;
+    hipStream_t st = ctx->stream;
+    const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim;
+    int rc;
+    record_tokens_kernel<<<1, nb, 0, st>>>(m->hist, pos0, toks);
+    embed_kernel<<<dim3((H / 8 + 255) / 256, nb), 256, 0, st>>>(m->emb, toks, m->pb_h, H);
+    for (int l = 0; l < c.num_hidden_layers; l++) {
+        const size_t per_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * d;
+        norm_kernel<<<nb, 1024, 0, st>>>(m->pb_h, m->norm_attn + (size_t)l * H, H, c.rms_norm_eps, m->pb_xn);
+        if ((rc = axq_dev_gemv_batch(ctx, m->w_qkv[l], m->pb_xn, nb, nullptr, nullptr, m->pb_qkv))) return rc;
+        rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
+            m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + l * per_layer,
+            m->vcache + l * per_layer, pos0, c.max_position_embeddings, d);
+        switch (d) {
+        case 32: launch_attn_prompt_d<32>(m, l, pos0, nb, st); break;
+        case 64: launch_attn_prompt_d<64>(m, l, pos0, nb, st); break;
+        case 128: launch_attn_prompt_d<128>(m, l, pos0, nb, st); break;
+        default: launch_attn_prompt_d<256>(m, l, pos0, nb, st); break;
+        }
+        if ((rc = axq_dev_gemv_batch(ctx, m->w_o[l], m->pb_att, nb, nullptr, m->pb_h, m->pb_h))) return rc;
+        norm_kernel<<<nb, 1024, 0, st>>>(m->pb_h, m->norm_ffn + (size_t)l * H, H, c.rms_norm_eps, m->pb_xn);
+        if ((rc = axq_dev_gemv_batch(ctx, m->w_gu[l], m->pb_xn, nb, nullptr, nullptr, m->pb_gu))) return rc;
+        swiglu_kernel<<<dim3((I / 4 + 255) / 256, nb), 256, 0, st>>>(m->pb_gu, I, m->pb_act);
+        if ((rc = axq_dev_gemv_batch(ctx, m->w_down[l], m->pb_act, nb, nullptr, m->pb_h, m->pb_h))) return rc;
+    }
+    add_i32_kernel<<<1, 1, 0, st>>>(m->pos, nb);
+    AXQ_LAUNCH_CHECK(ctx, "prompt batch");
+    return AXQ_OK;
+}
+
+// Feeds prompt[first..n) (already in m->prompt) from position base + first on: all but the last token in
+// batches where the batch path covers them, the rest (and always the last, whose logits are wanted) one by one.
+int feed_prompt(axq_model *m, int base, int n_prompt) {
+    axq_ctx *ctx = m->ctx;
+    static const bool no_batch = getenv("AXQ_PROMPT_BATCH") && getenv("AXQ_PROMPT_BATCH")[0] == '0'; // development knob
+    int i = 0, rc = AXQ_OK;
+    while (!no_batch && n_prompt - 1 - i >= 2) {
+        const int nb = n_prompt - 1 - i < PROMPT_BATCH ? n_prompt - 1 - i : PROMPT_BATCH;
+        if (!prompt_batch_covers(m, base + i, nb)) break;
+        if ((rc = enqueue_prompt_batch(m, m->prompt + i, nb, base + i))) return rc;
+        i += nb;
+    }
+    for (; i < n_prompt && !rc; i++) {
+        pick_prompt_kernel<<<1, 1, 0, ctx->stream>>>(m->prompt, m->pos, base, m->tok);
+        rc = run_token(m);
+    }
+    return rc;
+}
+
 template <class T>
 hipError_t dev_alloc(T **p, size_t count) { return hipMalloc((void **)p, (count ? count : 1) * sizeof(T)); }
 
@@ -657,6 +885,9 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     TRY(dev_alloc(&m->h, H)); TRY(dev_alloc(&m->xn, H)); TRY(dev_alloc(&m->qkv, m->qkv_rows)); TRY(dev_alloc(&m->att, m->q_dim));
     TRY(dev_alloc(&m->att_part, (size_t)c.num_key_value_heads * m->max_splits * (c.num_attention_heads / c.num_key_value_heads) * (c.head_dim + 2)));
     TRY(dev_alloc(&m->gu, (size_t)2 * I)); TRY(dev_alloc(&m->act, I)); TRY(dev_alloc(&m->logits, c.vocab_size));
+    TRY(dev_alloc(&m->pb_h, (size_t)PROMPT_BATCH * H)); TRY(dev_alloc(&m->pb_xn, (size_t)PROMPT_BATCH * H));
+    TRY(dev_alloc(&m->pb_qkv, (size_t)PROMPT_BATCH * m->qkv_rows)); TRY(dev_alloc(&m->pb_att, (size_t)PROMPT_BATCH * m->q_dim));
+    TRY(dev_alloc(&m->pb_gu, (size_t)PROMPT_BATCH * 2 * I)); TRY(dev_alloc(&m->pb_act, (size_t)PROMPT_BATCH * I));
     TRY(dev_alloc(&m->pos, 1)); TRY(dev_alloc(&m->tok, 1)); TRY(dev_alloc(&m->next, 1)); TRY(dev_alloc(&m->gen, 1));
     TRY(dev_alloc(&m->prompt, m->prompt_cap)); TRY(dev_alloc(&m->out, m->out_cap));
     TRY(dev_alloc(&m->hist, c.max_position_embeddings));
@@ -713,7 +944,8 @@ void axq_model_free(axq_model *m) {
     axq_weight_free(ctx, m->w_head);
     void *bufs[] = {m->emb, m->norm_attn, m->norm_ffn, m->norm_final, m->rope_cos, m->rope_sin, m->kcache, m->vcache, m->h,
                     m->xn, m->qkv, m->att, m->att_part, m->gu, m->act, m->logits, m->pos, m->tok,
-                    m->next, m->gen, m->prompt, m->out, m->hist, m->sample_scratch};
+                    m->next, m->gen, m->prompt, m->out, m->hist, m->sample_scratch, m->pb_h, m->pb_xn, m->pb_qkv, m->pb_att,
+                    m->pb_gu, m->pb_act};
     for (void *p : bufs)
         if (p) (void)hipFree(p);
     delete m;
@@ -890,6 +1122,36 @@ int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_t *next_
     return AXQ_OK;
 }
 
+int axq_model_forward_tokens(axq_model *m, const int32_t *tokens, int n, float *logits, int32_t *next_token) {
+    if (!m || !tokens) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    int rc;
+    if ((rc = check_ready(m))) return rc;
+    if (n <= 0) return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: at least one token is needed");
+    if (m->host_pos + n > m->cfg.max_position_embeddings || n > m->prompt_cap)
+        return axq_fail(ctx, AXQ_ERR_OVERFLOW, "Numerical overflow during quantization: %d + %d positions exceed the cache of %d",
+                        m->host_pos, n, m->cfg.max_position_embeddings);
+    for (int i = 0; i < n; i++)
+        if (tokens[i] < 0 || tokens[i] >= m->cfg.vocab_size)
+            return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "token %d outside the vocabulary of %d", tokens[i], m->cfg.vocab_size);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipMemcpyAsync(m->prompt, tokens, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    rc = feed_prompt(m, m->host_pos, n);
+    if (rc) { // the device-side position may have moved: bring both sides back to where the call started
+        set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->pos, m->host_pos);
+        (void)hipStreamSynchronize(ctx->stream);
+        return rc;
+    }
+    m->host_pos += n;
+    if (logits)
+        AXQ_HIP(ctx, hipMemcpyAsync(logits, m->logits, (size_t)m->cfg.vocab_size * 4, hipMemcpyDeviceToHost, ctx->stream),
+                AXQ_ERR_COPY_FAILED);
+    if (next_token)
+        AXQ_HIP(ctx, hipMemcpyAsync(next_token, m->next, 4, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
 int axq_model_generate(axq_model *m, const int32_t *prompt, int n_prompt, int max_new_tokens, int32_t *out_tokens,
                        float *prefill_ms, float *decode_ms) {
     if (!m || !prompt || (max_new_tokens > 0 && !out_tokens)) return AXQ_ERR_INVALID_ARGUMENT;
@@ -914,11 +1176,8 @@ int axq_model_generate(axq_model *m, const int32_t *prompt, int n_prompt, int ma
     AXQ_HIP(ctx, hipEventCreate(&e1), AXQ_ERR_DRIVER);
     AXQ_HIP(ctx, hipEventCreate(&e2), AXQ_ERR_DRIVER);
     (void)hipEventRecord(e0, ctx->stream);
-    // prompt: one step per token (the cache fills position by position)
-    for (int i = 0; i < n_prompt && !rc; i++) {
-        pick_prompt_kernel<<<1, 1, 0, ctx->stream>>>(m->prompt, m->pos, base, m->tok);
-        rc = run_token(m);
-    }
+    // prompt: up to eight tokens per pass over the weights, the last one by the step that also yields logits
+    rc = feed_prompt(m, base, n_prompt);
     (void)hipEventRecord(e1, ctx->stream);
     // generation: the argmax of step i is the input of step i+1, on the device
     for (int i = 0; i < max_new_tokens && !rc; i++) {

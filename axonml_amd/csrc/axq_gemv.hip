@@ -568,7 +568,7 @@ int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, c
     // small batches: eight vectors at a time against one pass over the weights, where that kernel applies
     while (batch >= 2 && axq_dev_gemv_batch_covers(w, batch < 8 ? batch : 8)) {
         const int nb = batch < 8 ? batch : 8;
-        int rc = axq_dev_gemv_batch(ctx, w, x, nb, bias, y);
+        int rc = axq_dev_gemv_batch(ctx, w, x, nb, bias, nullptr, y);
         if (rc) return rc;
         x += (size_t)nb * (size_t)w->k;
         y += (size_t)nb * (size_t)w->n_rows;

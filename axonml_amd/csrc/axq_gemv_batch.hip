@@ -33,6 +33,7 @@ struct MbArgs {
     const uint8_t *xa;  // the batch's limbs as MFMA A operands: [block][h][row 4 b + l] x 16 bytes (pack_x_kernel)
     const float *xsg;   // [block][h][4]: group scales of vectors h, h + 2, h + 4, h + 6; then the plain sums, same layout
     const float *bias;
+    const float *resid; // [batch, n_rows] added to y (may be y itself), or null
     float *y;
     float *ypart; // K split over several workgroups: [split][batch][n_rows] partial sums, added by mb_reduce_kernel
     int n_rows, k, batch;
@@ -270,6 +271,7 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
                 a.ypart[((size_t)blockIdx.y * a.batch + b) * a.n_rows + row0 + r] = tot;
             } else {
                 if (a.bias) tot += a.bias[row0 + r];
+                if (a.resid) tot += a.resid[(size_t)b * a.n_rows + row0 + r];
                 a.y[(size_t)b * a.n_rows + row0 + r] = tot;
             }
         }
@@ -315,13 +317,15 @@ __global__ void __launch_bounds__(256) pack_x_kernel(const float *x, int k, int 
     }
 }
 
-// y = sum over the splits, in order (+ bias)
-__global__ void __launch_bounds__(256) mb_reduce_kernel(const float *ypart, const float *bias, int n_rows, int batch, int splits, float *y) {
+// y = sum over the splits, in order (+ bias, + resid)
+__global__ void __launch_bounds__(256) mb_reduce_kernel(const float *ypart, const float *bias, const float *resid, int n_rows, int batch,
+                                                        int splits, float *y) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x, total = n_rows * batch;
     if (i >= total) return;
     float tot = ypart[i];
     for (int z = 1; z < splits; z++) tot += ypart[(size_t)z * total + i];
     if (bias) tot += bias[i % n_rows];
+    if (resid) tot += resid[i];
     y[i] = tot;
 }
 
@@ -350,7 +354,7 @@ void launch_mb(axq_ctx *ctx, MbArgs a, const float *x) {
     gemv_mb_kernel<T><<<dim3(tiles, splits), 64 * S, lds, ctx->stream>>>(a);
     if (splits > 1) {
         const int total = a.n_rows * a.batch;
-        mb_reduce_kernel<<<(total + 255) / 256, 256, 0, ctx->stream>>>(a.ypart, a.bias, a.n_rows, a.batch, (int)splits, a.y);
+        mb_reduce_kernel<<<(total + 255) / 256, 256, 0, ctx->stream>>>(a.ypart, a.bias, a.resid, a.n_rows, a.batch, (int)splits, a.y);
     }
 }
 
@@ -363,8 +367,9 @@ bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch) {
     return w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q8_0 || w->type == AXQ_Q4_K;
 }
 
-// y[batch, n_rows] = x[batch, k] W^T (+ bias) for 2 <= batch <= 8: split the batch, then one pass over W.
-int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y) {
+// y[batch, n_rows] = x[batch, k] W^T (+ bias per row of W) (+ resid[batch, n_rows], which may be y) for
+// 2 <= batch <= 8: split the batch, then one pass over W.
+int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, const float *resid, float *y) {
     const int k = (int)w->k;
     // scratch (the context's x buffer): 32 k bytes of A operands, then 2 * (k / 32) * 8 floats of scales and sums
     uint8_t *xa = ctx->xq;
@@ -373,7 +378,7 @@ int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int ba
     a.codes = w->codes; a.meta = w->meta;
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch;
     a.xa = xa; a.xsg = xsg;
-    a.bias = bias; a.y = y;
+    a.bias = bias; a.resid = resid; a.y = y;
     // partial sums of a split K behind the x operands (splits only happen below AXQ_BATCH_SPLIT_ROWS rows)
     a.ypart = w->n_rows <= AXQ_BATCH_SPLIT_ROWS ? reinterpret_cast<float *>(ctx->xq + (size_t)34 * AXQ_BATCH_MAX_K) : nullptr;
     a.n_rows = (int)w->n_rows; a.k = k; a.batch = batch;

@@ -114,7 +114,7 @@ size_t axq_xq_bytes(int64_t k);
 int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq);
 // gemv_batch.hip: batches of 2..8 vectors against one pass over the weights
 bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch);
-int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y);
+int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, const float *resid, float *y);
 // sample.hip: every pointer a device pointer; scratch = axq_sample_scratch_bytes(vocab)
 size_t axq_sample_scratch_bytes(int vocab);
 int axq_check_sampling_config(axq_ctx *ctx, const axq_sampling_config *cfg);

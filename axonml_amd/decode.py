@@ -72,6 +72,15 @@ class QuantizedLlama:
                                                       C.byref(nxt)))
         return nxt.value, logits
 
+    def forward_tokens(self, tokens, want_logits=True):
+        """forward_with_cache on several tokens (a prompt): the last position's next token and logits."""
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        logits = np.empty(self.cfg.vocab_size, dtype=np.float32) if want_logits else None
+        nxt = C.c_int32()
+        self.ctx.check(self.ctx.lib.axq_model_forward_tokens(self.handle, t.ctypes.data, t.size,
+                                                             logits.ctypes.data if want_logits else None, C.byref(nxt)))
+        return nxt.value, logits
+
     def hidden(self):
         out = np.empty(self.cfg.hidden_size, dtype=np.float32)
         self.ctx.check(self.ctx.lib.axq_model_read_hidden(self.handle, out.ctypes.data))

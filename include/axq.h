@@ -201,7 +201,13 @@ AXQ_API int axq_model_reset(axq_model *m);
 /* forward_with_cache for one token at the cache's current length; appends to
  * the cache.  logits (f32[vocab], host) may be NULL.  next_token (host) may be NULL. */
 AXQ_API int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_t *next_token);
-/* generate (llama.rs:900-977), greedy: feeds the prompt, then max_new_tokens
+/* forward_with_cache (llama.rs:731-762) for n >= 1 tokens at once (a prompt): appends n positions to the
+ * cache; logits / next_token are those of the last position.  Tokens before the last go through the
+ * layers up to eight per pass over the weights when every linear of the layers is Q4_0, Q4_1, Q8_0 or
+ * Q4_K with K a multiple of 256 up to 16384, else one by one; results agree with n calls of
+ * axq_model_forward to rounding (sums are taken in another order). */
+AXQ_API int axq_model_forward_tokens(axq_model *m, const int32_t *tokens, int n, float *logits, int32_t *next_token);
+/* generate (llama.rs:900-977), greedy: feeds the prompt (as axq_model_forward_tokens does), then max_new_tokens
  * steps, each consuming the previous argmax on the device.  out_tokens gets
  * max_new_tokens ids (host).  Timings (ms, may be NULL) cover prompt and
  * generation separately. */

@@ -88,6 +88,73 @@ def test_generate_matches_oracle_greedy_and_is_repeatable(ctx):
     gpu.close()
 
 
+@pytest.mark.parametrize("over,qtype,n_first,n_prompt", [
+    (dict(), o.Q4_K, 0, 2), (dict(), o.Q4_K, 0, 3), (dict(), o.Q4_K, 0, 9), (dict(), o.Q4_0, 0, 10), (dict(), o.Q8_0, 5, 26),
+    (dict(num_layers=3), o.Q4_1, 3, 17),
+    (dict(), o.Q5_1, 0, 12),  # a type outside the small-batch GEMV: fed one by one, same results
+    (dict(num_heads=8, num_kv_heads=2, head_dim=32), o.Q4_K, 1, 20),
+    (dict(num_heads=2, num_kv_heads=1, head_dim=128), o.Q4_K, 0, 19),
+    (dict(num_heads=1, num_kv_heads=1, head_dim=256), o.Q4_K, 2, 11),
+    (dict(sliding_window=5), o.Q4_K, 0, 30), (dict(sliding_window=12, max_seq_len=100), o.Q4_K, 7, 60),
+])
+def test_prompt_fed_at_once_matches_the_oracle_token_by_token(ctx, over, qtype, n_first, n_prompt):
+    """forward_tokens (up to eight prompt tokens per pass over the weights) against the oracle's one-token steps:
+    last logits and next token to the decode bar, and the KV cache against the GPU's own one-token path."""
+    c = tiny_config(**over)
+    w = random_weights(c, 70 + n_prompt, qtype=qtype)
+    cpu, gpu, one = load_oracle(c, w), load_gpu(ctx, c, w), load_gpu(ctx, c, w)
+    rng = np.random.default_rng(n_prompt)
+    toks = rng.integers(0, c["vocab_size"], size=n_first + n_prompt)
+    for pos, t in enumerate(toks):
+        c_next, c_logits = cpu.forward(int(t), pos)
+        one.forward(int(t), want_logits=False)
+    for t in toks[:n_first]:
+        gpu.forward(int(t), want_logits=False)
+    g_next, g_logits = gpu.forward_tokens(toks[n_first:])
+    assert gpu.seq_len() == len(toks)
+    assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL
+    assert g_next == c_next
+    n = len(toks)
+    for layer in range(c["num_layers"]):
+        for which in (0, 1):
+            a, b = one.kv(layer, which)[:, :n], gpu.kv(layer, which)[:, :n]
+            af, bf = a.view(np.float16).astype(np.float64), b.view(np.float16).astype(np.float64)
+            ulp = np.maximum(np.abs(af) * 2.0 ** -10, 5e-5 * np.abs(af).max())  # as in the cache test above
+            bad = np.argwhere(np.abs(af - bf) > ulp)
+            assert bad.size == 0, (layer, which, bad[0])
+    # the two paths go on alike: a few more steps, one token at a time
+    tok = c_next
+    for pos in range(n, min(n + 4, c["max_seq_len"])):
+        c_next, c_logits = cpu.forward(tok, pos)
+        g_next, g_logits = gpu.forward(tok)
+        assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, pos
+        assert g_next == c_next, pos
+        tok = c_next
+    for m in (gpu, one):
+        m.close()
+
+
+def test_forward_tokens_errors_leave_the_model_usable(ctx):
+    from axonml_amd import quant as q
+
+    c = tiny_config(num_layers=1)
+    w = random_weights(c, 41)
+    cpu, m = load_oracle(c, w), load_gpu(ctx, c, w)
+    with pytest.raises(q.ShapeMismatch):
+        m.forward_tokens([])
+    with pytest.raises(q.QuantError):
+        m.forward_tokens([1, 2, 10 ** 6])
+    with pytest.raises(q.Overflow):
+        m.forward_tokens(np.zeros(c["max_seq_len"] + 1, np.int32))
+    assert m.seq_len() == 0
+    toks = [4, 5, 6, 7, 8]
+    for pos, t in enumerate(toks):
+        c_next, c_logits = cpu.forward(t, pos)
+    g_next, g_logits = m.forward_tokens(toks)
+    assert g_next == c_next and max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL
+    m.close()
+
+
 def test_gqa_and_head_dim_variants(ctx):
     for over in (dict(num_heads=8, num_kv_heads=2, head_dim=32), dict(num_heads=2, num_kv_heads=1, head_dim=128),
                  dict(num_heads=4, num_kv_heads=4, head_dim=64, hidden_size=512, intermediate_size=768)):
