@@ -101,6 +101,7 @@ SIGNATURES = {
     "axq_model_forward_tokens": (_i, [_vp, _vp, _i, _vp, C.POINTER(C.c_int32)]),
     "axq_model_generate": (_i, [_vp, _vp, _i, _i, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "axq_model_seq_len": (_i, [_vp]),
+    "axq_model_truncate": (_i, [_vp, _i]),
     "axq_model_read_hidden": (_i, [_vp, _vp]),
     "axq_model_read_kv": (_i, [_vp, _i, _i, _vp]),
     "axq_fill_normal_f32": (_i, [_vp, _vp, _sz, C.c_float, C.c_float, C.c_float, C.c_float, C.c_uint64]),

@@ -1062,6 +1062,18 @@ int axq_model_reset(axq_model *m) {
     return AXQ_OK;
 }
 
+int axq_model_truncate(axq_model *m, int n_positions) {
+    if (!m) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    if (n_positions < 0 || n_positions > m->host_pos)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_truncate: %d positions asked, the cache holds %d", n_positions,
+                        m->host_pos);
+    set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->pos, n_positions);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    m->host_pos = n_positions;
+    return AXQ_OK;
+}
+
 int axq_model_set_sampling(axq_model *m, const axq_sampling_config *cfg, uint64_t seed) {
     if (!m) return AXQ_ERR_INVALID_ARGUMENT;
     axq_ctx *ctx = m->ctx;

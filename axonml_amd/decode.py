@@ -81,6 +81,10 @@ class QuantizedLlama:
                                                              logits.ctypes.data if want_logits else None, C.byref(nxt)))
         return nxt.value, logits
 
+    def truncate(self, n_positions):
+        """Rewind the cache to its first n_positions."""
+        self.ctx.check(self.ctx.lib.axq_model_truncate(self.handle, int(n_positions)))
+
     def hidden(self):
         out = np.empty(self.cfg.hidden_size, dtype=np.float32)
         self.ctx.check(self.ctx.lib.axq_model_read_hidden(self.handle, out.ctypes.data))

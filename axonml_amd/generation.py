@@ -2,7 +2,9 @@
 device sampler: `GenerationConfig` with its constructors and builders (:11-121) and `TextGenerator`
 (:124-277), whose `get_next_token` runs as one device kernel (`axq_sample_token`).  The reference draws its
 uniform variate from `rand::thread_rng`; here the caller passes `u`, or a numpy Generator supplies it.
-Beam search (:279-400) needs several sequences in flight and is not mirrored: the decode model holds one.
+`Beam` and `BeamSearch` (:277-400) are the reference's bookkeeping over per-beam logits; `beam_search_generate`
+drives them with the one-sequence decode model by rewinding its cache to the prefix a beam shares with what the
+cache holds and feeding the rest of the beam's tokens at once.
 """
 import ctypes as C
 import dataclasses
@@ -82,3 +84,89 @@ class TextGenerator:
 
     def should_stop(self, token):  # :272-274
         return int(token) in self.config.eos_token_ids
+
+
+@dataclasses.dataclass
+class Beam:
+    """Beam (generation.rs:277-304).  `score` adds raw logits in f32, as the reference does."""
+    tokens: List[int]
+    score: np.float32 = np.float32(0.0)
+    finished: bool = False
+
+    def normalized_score(self, length_penalty):
+        return np.float32(self.score) / np.power(np.float32(len(self.tokens)), np.float32(length_penalty))
+
+
+class BeamSearch:
+    """BeamSearch (generation.rs:306-400)."""
+
+    def __init__(self, num_beams, length_penalty, early_stopping, eos_token_ids):
+        self.num_beams, self.length_penalty = int(num_beams), float(length_penalty)
+        self.early_stopping, self.eos_token_ids = bool(early_stopping), [int(t) for t in eos_token_ids]
+
+    def init_beams(self, input_ids):
+        return [Beam([int(t) for t in np.asarray(input_ids).reshape(-1)])]
+
+    def expand_beams(self, beams, next_token_logits):
+        """Each live beam grows by its 2 * num_beams largest logits (equal logits: lower ids first, a stable
+        sort), finished beams stay as they are; the num_beams best by normalised score go on (equal
+        scores: in candidate order)."""
+        candidates = []
+        for beam, logits in zip(beams, next_token_logits):
+            if beam.finished:
+                candidates.append(beam)
+                continue
+            logits = np.asarray(logits, dtype=np.float32)
+            if np.isnan(logits).any():
+                raise ValueError("NaN among the logits")  # partial_cmp(..).unwrap() panics
+            order = np.argsort(-logits, kind="stable")[: self.num_beams * 2]
+            for token in order:
+                token = int(token)
+                candidates.append(Beam(beam.tokens + [token], np.float32(beam.score + logits[token]), token in self.eos_token_ids))
+        keys = np.array([c.normalized_score(self.length_penalty) for c in candidates], dtype=np.float32)
+        if np.isnan(keys).any():
+            raise ValueError("NaN among the beam scores")
+        keep = np.argsort(-keys, kind="stable")[: self.num_beams]
+        return [candidates[i] for i in keep]
+
+    def should_stop(self, beams):
+        return self.early_stopping and all(b.finished for b in beams)
+
+    def best_sequence(self, beams):
+        """Tokens of the best finished beam (of equal scores the last, Iterator::max_by), else of the first beam."""
+        best = None
+        for b in beams:
+            if b.finished and (best is None or b.normalized_score(self.length_penalty) >= best.normalized_score(self.length_penalty)):
+                best = b
+        if best is None:
+            best = beams[0] if beams else None
+        return None if best is None else list(best.tokens)
+
+
+def beam_search_generate(model, input_ids, beam_search, max_new_tokens):
+    """Beam search over a `QuantizedLlama`: per step every live beam's next-token logits, then
+    `expand_beams`, until `max_new_tokens` or `should_stop`.  The model keeps one sequence, so a beam is
+    brought in by rewinding the cache to the prefix it shares with the cached tokens and feeding the rest
+    (`truncate`, `forward_tokens`).  Returns (best_sequence, beams)."""
+    beams = beam_search.init_beams(input_ids)
+    cached = []  # tokens whose keys and values the model's cache holds now
+    if model.seq_len():
+        model.reset()
+    for _ in range(max_new_tokens):
+        per_beam = []
+        for b in beams:
+            if b.finished:
+                per_beam.append(None)
+                continue
+            shared = 0
+            limit = min(len(cached), len(b.tokens) - 1)  # at least the last token is fed: its logits are wanted
+            while shared < limit and cached[shared] == b.tokens[shared]:
+                shared += 1
+            model.truncate(shared)
+            _, logits = model.forward_tokens(b.tokens[shared:])
+            cached = list(b.tokens)
+            per_beam.append(logits)
+        beams = beam_search.expand_beams(beams, per_beam)
+        if beam_search.should_stop(beams):
+            break
+    return beam_search.best_sequence(beams), beams

@@ -198,6 +198,10 @@ AXQ_API int axq_model_set_linear(axq_model *m, int layer, int which, const axq_w
 AXQ_API int axq_model_random_init(axq_model *m, int type, float std, uint64_t seed);
 /* KVCache::clear (attention.rs:80-83). */
 AXQ_API int axq_model_reset(axq_model *m);
+/* Rewind the cache to its first n_positions (KVCache.seq_len is a public field, attention.rs:18-26: a caller
+ * that tries several continuations of one prefix, beam search for one, sets it back); the rows beyond are
+ * overwritten by the next tokens.  n_positions <= axq_model_seq_len. */
+AXQ_API int axq_model_truncate(axq_model *m, int n_positions);
 /* forward_with_cache for one token at the cache's current length; appends to
  * the cache.  logits (f32[vocab], host) may be NULL.  next_token (host) may be NULL. */
 AXQ_API int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_t *next_token);
