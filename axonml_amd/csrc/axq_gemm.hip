@@ -473,17 +473,85 @@ int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
     return AXQ_OK;
 }
 
-} // namespace
+// f32 rows, optionally RMS-normalised on the way ((x * inv_rms) * norm_w, RMSNorm::forward, llm/src/llama.rs:158-187),
+// -> two f16 rows each under one power-of-two scale: row t holds the leading 11 bits of every element, row m + t
+// what those leave, so that their GEMM results add up to the f32 product.
+__global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, const float *norm_w, float eps, int m, int k,
+                                                              _Float16 *xh, float *rowscale) {
+    __shared__ float red[4];
+    const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float *xr = x + (size_t)row * k;
+    float inv = 1.0f;
+    if (norm_w) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < k; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) ss += __shfl_xor(ss, s);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        ss = (red[0] + red[1]) + (red[2] + red[3]);
+        __syncthreads();
+        inv = 1.0f / sqrtf(ss / (float)k + eps);
+    }
+    uint32_t amax_bits = 0; // of |v| as integers: a NaN ranks above everything and is not dropped
+    for (int i = threadIdx.x; i < k; i += blockDim.x) {
+        const float v = norm_w ? (xr[i] * inv) * norm_w[i] : xr[i];
+        const uint32_t b = __builtin_bit_cast(uint32_t, v) & 0x7FFFFFFFu;
+        amax_bits = b > amax_bits ? b : amax_bits;
+    }
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)amax_bits, s);
+        amax_bits = o > amax_bits ? o : amax_bits;
+    }
+    if (lane == 0) red[wave] = __builtin_bit_cast(float, amax_bits);
+    __syncthreads();
+    uint32_t ab = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t o = __builtin_bit_cast(uint32_t, red[i]);
+        ab = o > ab ? o : ab;
+    }
+    // amax in [2^e, 2^(e+1)) -> multiply by 2^(14 - e); inf/nan rows are passed through unscaled
+    int eb = (int)((ab >> 23) & 0xFF);
+    if (eb == 0 || eb == 0xFF) eb = 127 + 14;
+    int sb = 127 + 14 - (eb - 127);
+    sb = sb < 1 ? 1 : (sb > 254 ? 254 : sb);
+    const float f = __builtin_bit_cast(float, (uint32_t)sb << 23);
+    for (int i = threadIdx.x; i < k; i += blockDim.x) {
+        const float v = (norm_w ? (xr[i] * inv) * norm_w[i] : xr[i]) * f;
+        const _Float16 hi = (_Float16)v;
+        xh[(size_t)row * k + i] = hi;
+        xh[(size_t)(m + row) * k + i] = (_Float16)(v - (float)hi);
+    }
+    if (threadIdx.x == 0) { rowscale[row] = 1.0f / f; rowscale[m + row] = 1.0f / f; }
+}
 
-int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
+// y[t] = y2[t] + y2[m + t] (+ bias) (+ resid[t]): the two halves of every activation row meet again
+__global__ void __launch_bounds__(256) gemm_pair_sum_kernel(const float *y2, const float *bias, const float *resid, size_t total, int n,
+                                                            float *y) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    float v = y2[i] + y2[total + i];
+    if (bias) v += bias[i % (size_t)n];
+    if (resid) v += resid[i];
+    y[i] = v;
+}
+
+struct GemmPlan {
+    int splits, steps_per_split;
+    size_t xh_bytes, rs_bytes, part_bytes;
+};
+
+// Split K when the output tiles alone leave most compute units idle (short prompts): the splits' partial sums go
+// through scratch and are added in order by a second kernel.  Scratch (kept in the context, grown on demand):
+// f16 activations [m, k] | row scales [m] | partial sums of a split K | `extra` bytes for the caller.
+int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, size_t extra, GemmPlan *p) {
     if (w->k % BK != 0)
         return axq_fail(ctx, AXQ_ERR_INVALID_BLOCK_SIZE, "Invalid block size: the prefill GEMM needs k %% 64 == 0, got %lld",
                         (long long)w->k);
     if (w->n_rows > INT32_MAX || w->k > INT32_MAX)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
-    // scratch: f16 activations [m, k], the row scales [m], the partial sums of a split K; kept in the context, grown on demand
-    // split K when the output tiles alone leave most compute units idle (short prompts): the splits' partial
-    // sums go through scratch and are added in order by a second kernel
     const int bm = m > 128 ? 256 : 128;
     const long tiles = (long)((w->n_rows + BN - 1) / BN) * ((m + bm - 1) / bm);
     const int ksteps = (int)(w->k / BK), cus = ctx->prop.multiProcessorCount;
@@ -491,10 +559,12 @@ int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int 
     splits = splits > 8 ? 8 : splits;
     if (splits > ksteps / 4) splits = ksteps / 4;
     if (splits < 2 || w->n_rows % 4 != 0) splits = 1;
-    const int steps_per_split = (ksteps + splits - 1) / splits;
-    splits = (ksteps + steps_per_split - 1) / steps_per_split;
-    const size_t xh_bytes = axq_align_up((size_t)m * (size_t)w->k * 2, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
-    const size_t need = xh_bytes + rs_bytes + (splits > 1 ? (size_t)splits * m * (size_t)w->n_rows * 4 : 0);
+    p->steps_per_split = (ksteps + splits - 1) / splits;
+    p->splits = (ksteps + p->steps_per_split - 1) / p->steps_per_split;
+    p->xh_bytes = axq_align_up((size_t)m * (size_t)w->k * 2, 256);
+    p->rs_bytes = axq_align_up((size_t)m * 4, 256);
+    p->part_bytes = axq_align_up(p->splits > 1 ? (size_t)p->splits * m * (size_t)w->n_rows * 4 : 0, 256);
+    const size_t need = p->xh_bytes + p->rs_bytes + p->part_bytes + extra;
     if (ctx->gemm_scratch_bytes < need) {
         AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
         if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
@@ -503,27 +573,63 @@ int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int 
         AXQ_HIP(ctx, hipMalloc(&ctx->gemm_scratch, need), AXQ_ERR_ALLOCATION_FAILED);
         ctx->gemm_scratch_bytes = need;
     }
-    _Float16 *xh = reinterpret_cast<_Float16 *>(ctx->gemm_scratch);
-    float *rowscale = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(ctx->gemm_scratch) + xh_bytes);
-    gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, (int)w->k, xh, rowscale);
+    return AXQ_OK;
+}
+
+// The GEMM proper over activations that already sit in scratch as scaled f16 rows.
+int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float *y) {
+    uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     GemmArgs a;
     a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
-    a.xh = xh; a.rowscale = rowscale; a.y = y;
-    a.ypart = splits > 1 ? reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(ctx->gemm_scratch) + xh_bytes + rs_bytes) : nullptr;
+    a.xh = reinterpret_cast<_Float16 *>(base); a.rowscale = reinterpret_cast<float *>(base + p.xh_bytes); a.y = y;
+    a.ypart = p.splits > 1 ? reinterpret_cast<float *>(base + p.xh_bytes + p.rs_bytes) : nullptr;
     a.m = m; a.n = (int)w->n_rows; a.k = (int)w->k;
-    a.steps_per_split = steps_per_split;
-    int rc;
+    a.steps_per_split = p.steps_per_split;
     switch (w->type) {
-    case AXQ_Q4_K: rc = launch_gemm<GQ4K>(ctx, a, splits); break;
-    case AXQ_Q4_0: rc = launch_gemm<GQ4x<false>>(ctx, a, splits); break;
-    case AXQ_Q4_1: rc = launch_gemm<GQ4x<true>>(ctx, a, splits); break;
-    case AXQ_Q5_0: rc = launch_gemm<GQ5x<false>>(ctx, a, splits); break;
-    case AXQ_Q5_1: rc = launch_gemm<GQ5x<true>>(ctx, a, splits); break;
-    case AXQ_Q8_0: rc = launch_gemm<GQ80>(ctx, a, splits); break;
-    case AXQ_F16: rc = launch_gemm<GF16>(ctx, a, splits); break;
-    case AXQ_F32: rc = launch_gemm<GF32>(ctx, a, splits); break;
-    default: rc = axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
+    case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);
+    case AXQ_Q4_0: return launch_gemm<GQ4x<false>>(ctx, a, p.splits);
+    case AXQ_Q4_1: return launch_gemm<GQ4x<true>>(ctx, a, p.splits);
+    case AXQ_Q5_0: return launch_gemm<GQ5x<false>>(ctx, a, p.splits);
+    case AXQ_Q5_1: return launch_gemm<GQ5x<true>>(ctx, a, p.splits);
+    case AXQ_Q8_0: return launch_gemm<GQ80>(ctx, a, p.splits);
+    case AXQ_F16: return launch_gemm<GF16>(ctx, a, p.splits);
+    case AXQ_F32: return launch_gemm<GF32>(ctx, a, p.splits);
+    default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
     }
-    return rc;
+}
+
+} // namespace
+
+int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
+    GemmPlan p;
+    int rc;
+    if ((rc = plan_gemm(ctx, w, m, 0, &p))) return rc;
+    uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
+    gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
+                                                   reinterpret_cast<float *>(base + p.xh_bytes));
+    return run_gemm(ctx, w, m, p, y);
+}
+
+bool axq_dev_gemm_f32_covers(const axq_weight *w, int m) {
+    return w->k % BK == 0 && m >= 1 && m <= AXQ_GEMM_F32_MAX_ROWS && w->n_rows <= INT32_MAX && w->k <= INT32_MAX;
+}
+
+// y[m, n] = f(x)[m, k] W^T (+ bias[n]) (+ resid[m, n], which may be y) with f32 activations: each row goes through the
+// matrix pipe as two f16 rows (2m rows in all), and the two results are added.  f = RMSNorm with weight norm_w
+// when that is given.
+int axq_dev_gemm_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int m, const float *norm_w, float eps, const float *bias,
+                     const float *resid, float *y) {
+    GemmPlan p;
+    int rc;
+    const size_t total = (size_t)m * (size_t)w->n_rows;
+    if ((rc = plan_gemm(ctx, w, 2 * m, 2 * total * sizeof(float), &p))) return rc;
+    uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
+    float *y2 = reinterpret_cast<float *>(base + p.xh_bytes + p.rs_bytes + p.part_bytes);
+    gemm_prep_x_f32_kernel<<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
+                                                       reinterpret_cast<float *>(base + p.xh_bytes));
+    if ((rc = run_gemm(ctx, w, 2 * m, p, y2))) return rc;
+    gemm_pair_sum_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(y2, bias, resid, total, (int)w->n_rows, y);
+    AXQ_LAUNCH_CHECK(ctx, "gemm_pair_sum_kernel");
+    return AXQ_OK;
 }

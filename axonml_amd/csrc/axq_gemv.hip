@@ -22,6 +22,8 @@
 //     outstanding.
 #include <hip/hip_fp16.h>
 
+#include <stdlib.h>
+
 #include "axq_internal.h"
 
 namespace {
@@ -565,6 +567,17 @@ int launch(axq_ctx *ctx, const axq_weight *w, const float *x, const float *bias,
 int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y) {
     if (w->n_rows > INT32_MAX || w->k > INT32_MAX)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
+    // many vectors: through the matrix-pipe GEMM, each f32 row as two f16 rows; worth it from about 40 rows where the
+    // small-batch kernel below is the alternative, from 8 where single-vector passes are
+    static const bool no_gemm = getenv("AXQ_GEMV_GEMM") && getenv("AXQ_GEMV_GEMM")[0] == '0'; // development knob
+    while (!no_gemm && batch >= (axq_dev_gemv_batch_covers(w, 8) ? 40 : 8) && axq_dev_gemm_f32_covers(w, 1)) {
+        const int nb = batch < AXQ_GEMM_F32_MAX_ROWS ? batch : AXQ_GEMM_F32_MAX_ROWS;
+        int rc = axq_dev_gemm_f32(ctx, w, x, nb, nullptr, 0.f, bias, nullptr, y);
+        if (rc) return rc;
+        x += (size_t)nb * (size_t)w->k;
+        y += (size_t)nb * (size_t)w->n_rows;
+        batch -= nb;
+    }
     // small batches: eight vectors at a time against one pass over the weights, where that kernel applies
     while (batch >= 2 && axq_dev_gemv_batch_covers(w, batch < 8 ? batch : 8)) {
         const int nb = batch < 8 ? batch : 8;

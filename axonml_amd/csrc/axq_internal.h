@@ -123,3 +123,7 @@ int axq_dev_sample(axq_ctx *ctx, const float *logits, int vocab, const int32_t *
                    int32_t *out, float *filtered_out);
 // gemm.hip
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_dev, int m, float *y_dev);
+#define AXQ_GEMM_F32_MAX_ROWS 2048 // rows per call of the f32-activation GEMM (its scratch grows with them)
+bool axq_dev_gemm_f32_covers(const axq_weight *w, int m);
+int axq_dev_gemm_f32(axq_ctx *ctx, const axq_weight *w, const float *x_dev, int m, const float *norm_w, float eps,
+                     const float *bias, const float *resid, float *y_dev);

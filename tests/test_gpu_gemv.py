@@ -160,6 +160,47 @@ def test_small_batch_reads_weights_once(ctx, qtype, batch, n, k):
     dw.free()
 
 
+# ---- many vectors: f32 rows through the matrix-pipe GEMM as two f16 rows each
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.F16, o.F32])
+@pytest.mark.parametrize("batch,n,k", [(40, 96, 512), (64, 100, 1024), (130, 33, 4096), (9, 64, 2048), (300, 257, 768)])
+def test_many_vectors_go_through_the_gemm_at_f32_accuracy(ctx, qtype, batch, n, k):
+    rng = np.random.default_rng(batch * 7 + n + k + qtype)
+    w = gen_weight(rng, n, k)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    x[1] = 0.3 + 0.05 * x[1]
+    x[2] *= 1e-3                      # rows of very different magnitude: every row has its own scale
+    x[3, ::7] *= 1e-4                 # small elements beside large ones inside a row
+    x[4] *= 3e4
+    bias = rng.standard_normal(n).astype(np.float32)
+    wq = o.quantize(qtype, w)
+    dw = q.DeviceWeight.upload(q.QuantizedTensor([n, k], qtype, wq), ctx)
+    got = q.quantized_matmul(x, dw, bias, ctx)
+    assert got.shape == (batch, n)
+    exact = o.matmul_f64(o.dequantize(qtype, wq, n * k).reshape(n, k), x) + bias.astype(np.float64)
+    # row by row, so that the large rows do not hide the small ones
+    for r in range(batch):
+        assert max_rel_err(got[r], exact[r], STRICT_FLOOR) <= MATMUL_RTOL, r
+    # far inside the tolerance: the split of a row into two f16 rows keeps 22 bits
+    rel = np.abs(got - exact).max(axis=1) / np.abs(exact).max(axis=1)
+    assert rel.max() <= 2e-5, rel.max()
+    dw.free()
+
+
+def test_many_vectors_non_finite_row(ctx):
+    rng = np.random.default_rng(5)
+    n, k, batch = 64, 512, 48
+    wq = o.quantize(o.Q4_K, gen_weight(rng, n, k))
+    dw = q.DeviceWeight.upload(q.QuantizedTensor([n, k], o.Q4_K, wq), ctx)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    x[5, 100] = np.nan
+    x[7, 3] = np.inf
+    y = q.quantized_matmul(x, dw, None, ctx)
+    assert not np.isfinite(y[5]).any() and not np.isfinite(y[7]).any()
+    keep = [r for r in range(batch) if r not in (5, 7)]
+    assert np.isfinite(y[keep]).all()
+    dw.free()
+
+
 @pytest.mark.parametrize("n,k", [(11008, 4096), (4096, 11008)])
 def test_small_batch_config_shape(ctx, n, k):
     # BASELINE config 2: 11008 x 4096 and the transposed down-projection shape, batch 8, Q4_0 and Q4_1
