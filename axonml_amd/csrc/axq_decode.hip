@@ -41,7 +41,8 @@ struct axq_model {
     // activations
     float *h, *xn, *qkv, *att, *gu, *act, *logits;
     float *att_part;                // [kv_heads][max_splits][rep][head_dim + 2] partial attention results
-    float *pb_h, *pb_xn, *pb_qkv, *pb_att, *pb_gu, *pb_act; // the same activations for eight prompt tokens at a time
+    float *pb_h, *pb_xn, *pb_qkv, *pb_att, *pb_gu, *pb_act; // the same activations for pb_cap prompt tokens at a time
+    int pb_cap;
     int max_splits;
     // device-side state
     int32_t *pos, *tok, *next, *gen, *prompt, *out;
@@ -747,21 +748,53 @@ int run_token(axq_model *m) {
                           m->sample_scratch, m->next, nullptr);
 }
 
-// Whether `nb` prompt tokens starting at position pos0 can go through the layers together: every linear of
-// the layers within the small-batch GEMV's reach, and the scores of the longest query within LDS.
+// Prompt tokens go through the layers several at a time: up to PROMPT_BATCH with the small-batch GEMV (one pass over
+// the weights for eight vectors), up to PROMPT_CHUNK with the matrix-pipe GEMM on f32 activations once there are
+// enough of them to fill its tiles.
+constexpr int PROMPT_CHUNK = 512;
+constexpr int PROMPT_GEMM_MIN = 32;
+
 size_t prompt_attn_lds(const axq_model *m, int pos0, int nb) {
     int span = pos0 + nb;
     if (m->cfg.sliding_window > 0 && span > m->cfg.sliding_window) span = m->cfg.sliding_window;
     return (size_t)((span + 255) / 256 * 256) * sizeof(float);
 }
 
-bool prompt_batch_covers(const axq_model *m, int pos0, int nb) {
-    if (nb < 2 || nb > PROMPT_BATCH) return false;
-    if (prompt_attn_lds(m, pos0, nb) > 128 * 1024) return false;
+enum PromptMode { PROMPT_SINGLE = 0, PROMPT_GEMV = 1, PROMPT_GEMM = 2 };
+
+// How `nb` prompt tokens starting at position pos0 can go through the layers together: every linear of the layers
+// within reach of the kernel in question, and the scores of the longest query within LDS.
+bool prompt_mode_covers(const axq_model *m, int mode, int pos0, int nb) {
+    if (nb < 2 || prompt_attn_lds(m, pos0, nb) > 128 * 1024) return false;
+    if (mode == PROMPT_GEMV && nb > PROMPT_BATCH) return false;
     for (int l = 0; l < m->cfg.num_hidden_layers; l++)
         for (const axq_weight *w : {m->w_qkv[l], m->w_o[l], m->w_gu[l], m->w_down[l]})
-            if (!axq_dev_gemv_batch_covers(w, nb)) return false;
+            if (mode == PROMPT_GEMV ? !axq_dev_gemv_batch_covers(w, nb) : !axq_dev_gemm_f32_covers(w, nb)) return false;
     return true;
+}
+
+template <class T>
+hipError_t dev_alloc(T **p, size_t count);
+
+// Activation rows for `cap` prompt tokens (the model starts with PROMPT_BATCH of them).
+int reserve_prompt_rows(axq_model *m, int cap) {
+    if (cap <= m->pb_cap) return AXQ_OK;
+    axq_ctx *ctx = m->ctx;
+    const int H = m->cfg.hidden_size, I = m->cfg.intermediate_size;
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    for (float **p : {&m->pb_h, &m->pb_qkv, &m->pb_att, &m->pb_gu, &m->pb_act}) {
+        if (*p) (void)hipFree(*p);
+        *p = nullptr;
+    }
+    m->pb_cap = 0;
+    hipError_t e = dev_alloc(&m->pb_h, (size_t)cap * H);
+    if (e == hipSuccess) e = dev_alloc(&m->pb_qkv, (size_t)cap * m->qkv_rows);
+    if (e == hipSuccess) e = dev_alloc(&m->pb_att, (size_t)cap * m->q_dim);
+    if (e == hipSuccess) e = dev_alloc(&m->pb_gu, (size_t)cap * 2 * I);
+    if (e == hipSuccess) e = dev_alloc(&m->pb_act, (size_t)cap * I);
+    if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "prompt activations for %d tokens: %s", cap, hipGetErrorString(e));
+    m->pb_cap = cap;
+    return AXQ_OK;
 }
 
 template <int D>
@@ -779,22 +812,31 @@ void launch_attn_prompt_d(axq_model *m, int l, int pos0, int nb, hipStream_t st)
         c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, c.sliding_window, m->pb_att);
 }
 
-// The layers for prompt tokens toks[0..nb) (device memory) at positions pos0.., 2 <= nb <= 8: what nb steps
-// would leave in the KV cache, the history and the position counter, without the final norm and lm_head
-// (LLaMA::forward_with_cache on a multi-token input, llama.rs:731-762; its logits for all but the last
-// position are never looked at by generate, llama.rs:900-977).
-int enqueue_prompt_batch(axq_model *m, const int32_t *toks, int nb, int pos0) {
+// The layers for prompt tokens toks[0..nb) (device memory) at positions pos0..: what nb steps would leave in the
+// KV cache, the history and the position counter, without the final norm and lm_head (LLaMA::forward_with_cache
+// on a multi-token input, llama.rs:731-762; its logits for all but the last position are never looked at by
+// generate, llama.rs:900-977).  mode: PROMPT_GEMV (nb <= 8) or PROMPT_GEMM.
+int enqueue_prompt_rows(axq_model *m, int mode, const int32_t *toks, int nb, int pos0) {
     axq_ctx *ctx = m->ctx;
     const axq_model_config &c = m->cfg;
     hipStream_t st = ctx->stream;
     const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim;
     int rc;
-    record_tokens_kernel<<<1, nb, 0, st>>>(m->hist, pos0, toks);
+    if ((rc = reserve_prompt_rows(m, nb))) return rc;
+    // y = f(x) W^T (+ resid): f = RMSNorm when norm_w is given
+    auto lin = [&](const axq_weight *w, const float *x, const float *norm_w, const float *resid, float *y) -> int {
+        if (mode == PROMPT_GEMM) return axq_dev_gemm_f32(ctx, w, x, nb, norm_w, c.rms_norm_eps, nullptr, resid, y);
+        if (norm_w) {
+            norm_kernel<<<nb, 1024, 0, st>>>(x, norm_w, (int)w->k, c.rms_norm_eps, m->pb_xn);
+            x = m->pb_xn;
+        }
+        return axq_dev_gemv_batch(ctx, w, x, nb, nullptr, resid, y);
+    };
+    for (int t0 = 0; t0 < nb; t0 += 1024) record_tokens_kernel<<<1, nb - t0 < 1024 ? nb - t0 : 1024, 0, st>>>(m->hist, pos0 + t0, toks + t0);
     embed_kernel<<<dim3((H / 8 + 255) / 256, nb), 256, 0, st>>>(m->emb, toks, m->pb_h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
         const size_t per_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * d;
-        norm_kernel<<<nb, 1024, 0, st>>>(m->pb_h, m->norm_attn + (size_t)l * H, H, c.rms_norm_eps, m->pb_xn);
-        if ((rc = axq_dev_gemv_batch(ctx, m->w_qkv[l], m->pb_xn, nb, nullptr, nullptr, m->pb_qkv))) return rc;
+        if ((rc = lin(m->w_qkv[l], m->pb_h, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv))) return rc;
         rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
             m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + l * per_layer,
             m->vcache + l * per_layer, pos0, c.max_position_embeddings, d);
@@ -804,27 +846,38 @@ int enqueue_prompt_batch(axq_model *m, const int32_t *toks, int nb, int pos0) {
         case 128: launch_attn_prompt_d<128>(m, l, pos0, nb, st); break;
         default: launch_attn_prompt_d<256>(m, l, pos0, nb, st); break;
         }
-        if ((rc = axq_dev_gemv_batch(ctx, m->w_o[l], m->pb_att, nb, nullptr, m->pb_h, m->pb_h))) return rc;
-        norm_kernel<<<nb, 1024, 0, st>>>(m->pb_h, m->norm_ffn + (size_t)l * H, H, c.rms_norm_eps, m->pb_xn);
-        if ((rc = axq_dev_gemv_batch(ctx, m->w_gu[l], m->pb_xn, nb, nullptr, nullptr, m->pb_gu))) return rc;
+        if ((rc = lin(m->w_o[l], m->pb_att, nullptr, m->pb_h, m->pb_h))) return rc;
+        if ((rc = lin(m->w_gu[l], m->pb_h, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu))) return rc;
         swiglu_kernel<<<dim3((I / 4 + 255) / 256, nb), 256, 0, st>>>(m->pb_gu, I, m->pb_act);
-        if ((rc = axq_dev_gemv_batch(ctx, m->w_down[l], m->pb_act, nb, nullptr, m->pb_h, m->pb_h))) return rc;
+        if ((rc = lin(m->w_down[l], m->pb_act, nullptr, m->pb_h, m->pb_h))) return rc;
     }
     add_i32_kernel<<<1, 1, 0, st>>>(m->pos, nb);
-    AXQ_LAUNCH_CHECK(ctx, "prompt batch");
+    AXQ_LAUNCH_CHECK(ctx, "prompt rows");
     return AXQ_OK;
 }
 
-// Feeds prompt[first..n) (already in m->prompt) from position base + first on: all but the last token in
-// batches where the batch path covers them, the rest (and always the last, whose logits are wanted) one by one.
+// Feeds prompt[0..n) (already in m->prompt) from position base on: all but the last token several at a time
+// where a batched path covers them, the rest (and always the last, whose logits are wanted) one by one.
 int feed_prompt(axq_model *m, int base, int n_prompt) {
     axq_ctx *ctx = m->ctx;
-    static const bool no_batch = getenv("AXQ_PROMPT_BATCH") && getenv("AXQ_PROMPT_BATCH")[0] == '0'; // development knob
+    static const char *knob = getenv("AXQ_PROMPT_BATCH"); // development knob: 0 = one by one, 1 = no GEMM
+    const int allow = knob ? atoi(knob) : 2;
     int i = 0, rc = AXQ_OK;
-    while (!no_batch && n_prompt - 1 - i >= 2) {
-        const int nb = n_prompt - 1 - i < PROMPT_BATCH ? n_prompt - 1 - i : PROMPT_BATCH;
-        if (!prompt_batch_covers(m, base + i, nb)) break;
-        if ((rc = enqueue_prompt_batch(m, m->prompt + i, nb, base + i))) return rc;
+    while (allow >= 1 && n_prompt - 1 - i >= 2) {
+        const int left = n_prompt - 1 - i;
+        int mode = PROMPT_SINGLE, nb = 0;
+        // enough rows to fill GEMM tiles (fewer where the small-batch GEMV does not apply and single steps are the alternative)
+        if (allow >= 2) {
+            nb = left < PROMPT_CHUNK ? left : PROMPT_CHUNK;
+            const bool gemv_ok = prompt_mode_covers(m, PROMPT_GEMV, base + i, left < PROMPT_BATCH ? left : PROMPT_BATCH);
+            if (nb >= (gemv_ok ? PROMPT_GEMM_MIN : PROMPT_BATCH) && prompt_mode_covers(m, PROMPT_GEMM, base + i, nb)) mode = PROMPT_GEMM;
+        }
+        if (mode == PROMPT_SINGLE) {
+            nb = left < PROMPT_BATCH ? left : PROMPT_BATCH;
+            if (prompt_mode_covers(m, PROMPT_GEMV, base + i, nb)) mode = PROMPT_GEMV;
+        }
+        if (mode == PROMPT_SINGLE) break;
+        if ((rc = enqueue_prompt_rows(m, mode, m->prompt + i, nb, base + i))) return rc;
         i += nb;
     }
     for (; i < n_prompt && !rc; i++) {
@@ -885,7 +938,8 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     TRY(dev_alloc(&m->h, H)); TRY(dev_alloc(&m->xn, H)); TRY(dev_alloc(&m->qkv, m->qkv_rows)); TRY(dev_alloc(&m->att, m->q_dim));
     TRY(dev_alloc(&m->att_part, (size_t)c.num_key_value_heads * m->max_splits * (c.num_attention_heads / c.num_key_value_heads) * (c.head_dim + 2)));
     TRY(dev_alloc(&m->gu, (size_t)2 * I)); TRY(dev_alloc(&m->act, I)); TRY(dev_alloc(&m->logits, c.vocab_size));
-    TRY(dev_alloc(&m->pb_h, (size_t)PROMPT_BATCH * H)); TRY(dev_alloc(&m->pb_xn, (size_t)PROMPT_BATCH * H));
+    m->pb_cap = PROMPT_BATCH;
+    TRY(dev_alloc(&m->pb_h, (size_t)PROMPT_BATCH * H)); TRY(dev_alloc(&m->pb_xn, (size_t)PROMPT_BATCH * (H > I ? H : I)));
     TRY(dev_alloc(&m->pb_qkv, (size_t)PROMPT_BATCH * m->qkv_rows)); TRY(dev_alloc(&m->pb_att, (size_t)PROMPT_BATCH * m->q_dim));
     TRY(dev_alloc(&m->pb_gu, (size_t)PROMPT_BATCH * 2 * I)); TRY(dev_alloc(&m->pb_act, (size_t)PROMPT_BATCH * I));
     TRY(dev_alloc(&m->pos, 1)); TRY(dev_alloc(&m->tok, 1)); TRY(dev_alloc(&m->next, 1)); TRY(dev_alloc(&m->gen, 1));

@@ -160,7 +160,7 @@ def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
     m.random_init(QuantType.Q4_K, 0.02, 1)
     rng = np.random.default_rng(0)
     prompt = rng.integers(0, cfg["vocab_size"], size=prompt_len, dtype=np.int32)
-    m.generate(prompt[:8], 4)  # warm-up: graph capture, first-touch
+    m.generate(prompt, 4)  # warm-up: graph capture, scratch buffers of the prompt path, first touch
     m.reset()
     out, pre_ms, dec_ms = m.generate(prompt, new_tokens)
     steps = new_tokens - 1

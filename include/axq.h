@@ -162,7 +162,9 @@ AXQ_API void axq_weight_free(axq_ctx *ctx, axq_weight *w);
  *      (tensor/src/tensor.rs:1020-1045) behind Linear::forward
  *      (nn/src/layers/linear.rs:104-140), fused ------------------------------ */
 /* y[batch, n_rows] = x[batch, k] * W^T (+ bias[n_rows] if non-NULL), f32.
- * Decode path (batch small); bias lives where x and y live. */
+ * Any batch: one vector and 2..8 vectors per pass over the weights (decode), from 40 rows on (k a
+ * multiple of 64) the matrix-pipe GEMM with every f32 row carried as two f16 rows, so that the result
+ * keeps f32 accuracy.  bias lives where x and y live. */
 AXQ_API int axq_gemv_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y,
                          int mem);
 /* y[m, n_rows] = x[m, k] * W^T, x in bf16 (raw uint16), y f32.  Prefill path. */
@@ -207,9 +209,10 @@ AXQ_API int axq_model_truncate(axq_model *m, int n_positions);
 AXQ_API int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_t *next_token);
 /* forward_with_cache (llama.rs:731-762) for n >= 1 tokens at once (a prompt): appends n positions to the
  * cache; logits / next_token are those of the last position.  Tokens before the last go through the
- * layers up to eight per pass over the weights when every linear of the layers is Q4_0, Q4_1, Q8_0 or
- * Q4_K with K a multiple of 256 up to 16384, else one by one; results agree with n calls of
- * axq_model_forward to rounding (sums are taken in another order). */
+ * layers together: from 32 on through the GEMM (f32 activations, K a multiple of 64), fewer up to eight
+ * per pass over the weights when every linear of the layers is Q4_0, Q4_1, Q8_0 or Q4_K with K a
+ * multiple of 256 up to 16384, else one by one; results agree with n calls of axq_model_forward to
+ * rounding (sums are taken in another order). */
 AXQ_API int axq_model_forward_tokens(axq_model *m, const int32_t *tokens, int n, float *logits, int32_t *next_token);
 /* generate (llama.rs:900-977), greedy: feeds the prompt (as axq_model_forward_tokens does), then max_new_tokens
  * steps, each consuming the previous argmax on the device.  out_tokens gets

@@ -91,11 +91,15 @@ def test_generate_matches_oracle_greedy_and_is_repeatable(ctx):
 @pytest.mark.parametrize("over,qtype,n_first,n_prompt", [
     (dict(), o.Q4_K, 0, 2), (dict(), o.Q4_K, 0, 3), (dict(), o.Q4_K, 0, 9), (dict(), o.Q4_0, 0, 10), (dict(), o.Q8_0, 5, 26),
     (dict(num_layers=3), o.Q4_1, 3, 17),
-    (dict(), o.Q5_1, 0, 12),  # a type outside the small-batch GEMV: fed one by one, same results
+    (dict(), o.Q5_1, 0, 12), (dict(), o.Q5_1, 0, 6),  # a type outside the small-batch GEMV: GEMM from 8 rows, else one by one
     (dict(num_heads=8, num_kv_heads=2, head_dim=32), o.Q4_K, 1, 20),
     (dict(num_heads=2, num_kv_heads=1, head_dim=128), o.Q4_K, 0, 19),
     (dict(num_heads=1, num_kv_heads=1, head_dim=256), o.Q4_K, 2, 11),
     (dict(sliding_window=5), o.Q4_K, 0, 30), (dict(sliding_window=12, max_seq_len=100), o.Q4_K, 7, 60),
+    # from 33 tokens on the rows before the last go through the GEMM (f32 activations as two f16 rows each)
+    (dict(max_seq_len=100), o.Q4_K, 0, 70), (dict(max_seq_len=100), o.Q4_0, 3, 45), (dict(max_seq_len=100), o.Q5_0, 0, 34),
+    (dict(max_seq_len=128, num_heads=8, num_kv_heads=2, head_dim=32), o.Q8_0, 10, 100),
+    (dict(max_seq_len=100, num_heads=2, num_kv_heads=1, head_dim=128, num_layers=3), o.Q4_1, 0, 41),
 ])
 def test_prompt_fed_at_once_matches_the_oracle_token_by_token(ctx, over, qtype, n_first, n_prompt):
     """forward_tokens (up to eight prompt tokens per pass over the weights) against the oracle's one-token steps:
