@@ -37,6 +37,18 @@ def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(
                 out.append(r)
                 log(f"  prefill {r['type']} M={m} N={n}: {t * 1e3:.1f} us, {r['tflops']:.1f} TFLOP/s")
                 ctx.free(xd)
+                # the same product from f32 rows (axq_gemv_f32 sends 40 rows or more through the GEMM as two f16 rows each)
+                xf = ctx.to_device(rng.standard_normal((m, k)).astype(np.float32))
+                for _ in range(3):
+                    ctx.check(lib.axq_gemv_f32(ctx.handle, h, xf, m, None, yd, MEM_DEVICE))
+                ctx.synchronize()
+                ctx.timer_start()
+                for _ in range(iters):
+                    ctx.check(lib.axq_gemv_f32(ctx.handle, h, xf, m, None, yd, MEM_DEVICE))
+                t32 = ctx.timer_stop() / iters
+                r["f32_rows_ms"], r["f32_rows_tflops"] = t32, flops / (t32 * 1e-3) / 1e12
+                log(f"          f32 rows      : {t32 * 1e3:.1f} us, {r['f32_rows_tflops']:.1f} TFLOP/s of useful work")
+                ctx.free(xf)
                 ctx.free(yd)
             lib.axq_weight_free(ctx.handle, h)
     return out
