@@ -43,6 +43,12 @@ struct axq_model {
     float *att_part;                // [kv_heads][max_splits][rep][head_dim + 2] partial attention results
     float *pb_h, *pb_xn, *pb_qkv, *pb_att, *pb_gu, *pb_act; // the same activations for pb_cap prompt tokens at a time
     int pb_cap;
+    int n_seq;                      // sequences the caches and the per-sequence state hold (axq_model_set_batch)
+    size_t seq_stride;              // cache elements of one sequence: layers * kv_heads * max_pos * head_dim
+    std::vector<int> seq_pos;       // host mirror of pos[s] for the batched calls (sequence 0: host_pos)
+    int32_t *bprompt, *boffsets, *bout; // prompts, their offsets and the generated ids of a batched generate
+    hipGraphExec_t graph_b;
+    bool graph_b_ok;
     int max_splits;
     // device-side state
     int32_t *pos, *tok, *next, *gen, *prompt, *out;
@@ -372,9 +378,13 @@ constexpr int PROMPT_BATCH = 8;
 
 __global__ void __launch_bounds__(128) rope_append_kernel(const float *qkv, int qkv_rows, int q_dim, int kv_dim,
                                                           const float *rope_cos, const float *rope_sin, uint16_t *kcache,
-                                                          uint16_t *vcache, int pos0, int max_pos, int d) {
-    const int half = d >> 1, e = threadIdx.x, kvh = blockIdx.x, p = pos0 + (int)blockIdx.y;
-    const float *row = qkv + (size_t)blockIdx.y * qkv_rows;
+                                                          uint16_t *vcache, int pos0, const int32_t *pos_arr,
+                                                          size_t seq_stride, int max_pos, int d) {
+    const int half = d >> 1, e = threadIdx.x, kvh = blockIdx.x, b = blockIdx.y;
+    // rows of one sequence at consecutive positions, or (pos_arr given) one row per sequence at that sequence's position
+    const int p = pos_arr ? pos_arr[b] : pos0 + b;
+    if (pos_arr) { kcache += (size_t)b * seq_stride; vcache += (size_t)b * seq_stride; }
+    const float *row = qkv + (size_t)b * qkv_rows;
     const float *kh = row + q_dim + (size_t)kvh * d, *vh = row + q_dim + kv_dim + (size_t)kvh * d;
     const float nc = rope_cos[(size_t)p * half + e], ns = rope_sin[(size_t)p * half + e];
     const float k1 = kh[e], k2 = kh[e + half];
@@ -392,14 +402,17 @@ __global__ void __launch_bounds__(128) rope_append_kernel(const float *qkv, int 
 template <int D>
 __global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int qkv_rows, const float *rope_cos,
                                                            const float *rope_sin, const uint16_t *kcache,
-                                                           const uint16_t *vcache, int pos0, int n_heads, int n_kv,
-                                                           int max_pos, int window, float *att) {
+                                                           const uint16_t *vcache, int pos0, const int32_t *pos_arr,
+                                                           size_t seq_stride, int n_heads, int n_kv, int max_pos, int window,
+                                                           float *att) {
     constexpr int HALF = D / 2, LP = D / 8, PPB = 1024 / LP; // lanes per position, positions per pass of the workgroup
     extern __shared__ float sc[];                            // scores, then exp(score - max)
     __shared__ __attribute__((aligned(16))) float qs[D];
     __shared__ float red[16];
     __shared__ __attribute__((aligned(16))) float osum[16 * D];
-    const int head = blockIdx.x, b = blockIdx.y, p = pos0 + b;
+    const int head = blockIdx.x, b = blockIdx.y;
+    const int p = pos_arr ? pos_arr[b] : pos0 + b; // as in rope_append_kernel
+    if (pos_arr) { kcache += (size_t)b * seq_stride; vcache += (size_t)b * seq_stride; }
     const int rep = n_heads / n_kv, kvh = head / rep;
     const int p_lo = (window > 0 && p + 1 > window) ? p + 1 - window : 0;
     const int span = p + 1 - p_lo;
@@ -518,6 +531,9 @@ __global__ void __launch_bounds__(256) swiglu_kernel(const float *gu, int inter,
 __global__ void __launch_bounds__(1024) argmax_kernel(const float *logits, int vocab, int32_t *next, int32_t *pos) {
     __shared__ float bv[16];
     __shared__ int bi[16];
+    logits += (size_t)blockIdx.x * vocab; // one workgroup per sequence
+    next += blockIdx.x;
+    pos += blockIdx.x;
     float best = -INFINITY;
     int idx = 0;
     // eight 16-byte loads per thread in flight at a time; a thread's indices rise, and `>=` keeps the last maximum
@@ -575,6 +591,17 @@ __global__ void set_i32_kernel(int32_t *p, int32_t v) { p[0] = v; }
 __global__ void add_i32_kernel(int32_t *p, int32_t v) { p[0] += v; }
 __global__ void record_tokens_kernel(int32_t *hist, int pos0, const int32_t *toks) { hist[pos0 + threadIdx.x] = toks[threadIdx.x]; }
 __global__ void record_token_kernel(int32_t *hist, const int32_t *pos, const int32_t *tok) { hist[pos[0]] = tok[0]; }
+// one thread per sequence
+__global__ void record_rows_kernel(int32_t *hist, int max_pos, const int32_t *pos, const int32_t *tok) {
+    hist[(size_t)threadIdx.x * max_pos + pos[threadIdx.x]] = tok[threadIdx.x];
+}
+__global__ void last_tokens_kernel(const int32_t *prompts, const int32_t *offsets, int32_t *tok) {
+    tok[threadIdx.x] = prompts[offsets[threadIdx.x + 1] - 1];
+}
+__global__ void commit_rows_kernel(const int32_t *next, int32_t *tok, int32_t *out, int step, int out_cap) {
+    tok[threadIdx.x] = next[threadIdx.x];
+    out[(size_t)threadIdx.x * out_cap + step] = next[threadIdx.x];
+}
 __global__ void fill_f32_kernel(float *p, size_t n, float v) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -748,35 +775,46 @@ int run_token(axq_model *m) {
                           m->sample_scratch, m->next, nullptr);
 }
 
-// Prompt tokens go through the layers several at a time: up to PROMPT_BATCH with the small-batch GEMV (one pass over
-// the weights for eight vectors), up to PROMPT_CHUNK with the matrix-pipe GEMM on f32 activations once there are
-// enough of them to fill its tiles.
+// Rows go through the layers several at a time: prompt tokens of one sequence at consecutive positions, or one token
+// of each of several sequences (a batched step).  Up to PROMPT_BATCH rows use the small-batch GEMV (one pass over the
+// weights for eight vectors), up to PROMPT_CHUNK the matrix-pipe GEMM on f32 activations once there are enough of
+// them to fill its tiles.
 constexpr int PROMPT_CHUNK = 512;
 constexpr int PROMPT_GEMM_MIN = 32;
 
-size_t prompt_attn_lds(const axq_model *m, int pos0, int nb) {
-    int span = pos0 + nb;
+// LDS of attn_prompt_kernel for queries up to position `last` (exclusive)
+size_t prompt_attn_lds(const axq_model *m, int last) {
+    int span = last;
     if (m->cfg.sliding_window > 0 && span > m->cfg.sliding_window) span = m->cfg.sliding_window;
     return (size_t)((span + 255) / 256 * 256) * sizeof(float);
 }
 
-enum PromptMode { PROMPT_SINGLE = 0, PROMPT_GEMV = 1, PROMPT_GEMM = 2 };
+enum RowsMode { ROWS_NONE = 0, ROWS_GEMV = 1, ROWS_GEMM = 2 };
 
-// How `nb` prompt tokens starting at position pos0 can go through the layers together: every linear of the layers
-// within reach of the kernel in question, and the scores of the longest query within LDS.
-bool prompt_mode_covers(const axq_model *m, int mode, int pos0, int nb) {
-    if (nb < 2 || prompt_attn_lds(m, pos0, nb) > 128 * 1024) return false;
-    if (mode == PROMPT_GEMV && nb > PROMPT_BATCH) return false;
+// Whether `nb` rows ending before position `last` can go through the layers together in that mode: the scores of the
+// longest query within LDS; for the GEMM every linear of the layers within its reach.  (The GEMV mode takes any
+// weight: what the small-batch kernel does not cover goes row by row.)
+bool rows_mode_covers(const axq_model *m, int mode, int last, int nb) {
+    if (nb < 1 || prompt_attn_lds(m, last) > 128 * 1024) return false;
+    if (mode == ROWS_GEMV) return nb <= PROMPT_BATCH;
     for (int l = 0; l < m->cfg.num_hidden_layers; l++)
         for (const axq_weight *w : {m->w_qkv[l], m->w_o[l], m->w_gu[l], m->w_down[l]})
-            if (mode == PROMPT_GEMV ? !axq_dev_gemv_batch_covers(w, nb) : !axq_dev_gemm_f32_covers(w, nb)) return false;
+            if (!axq_dev_gemm_f32_covers(w, nb)) return false;
+    return true;
+}
+
+bool all_layers_in_small_batch_reach(const axq_model *m, int nb) {
+    if (nb < 2) return false;
+    for (int l = 0; l < m->cfg.num_hidden_layers; l++)
+        for (const axq_weight *w : {m->w_qkv[l], m->w_o[l], m->w_gu[l], m->w_down[l]})
+            if (!axq_dev_gemv_batch_covers(w, nb < PROMPT_BATCH ? nb : PROMPT_BATCH)) return false;
     return true;
 }
 
 template <class T>
 hipError_t dev_alloc(T **p, size_t count);
 
-// Activation rows for `cap` prompt tokens (the model starts with PROMPT_BATCH of them).
+// Activation rows for `cap` tokens (the model starts with PROMPT_BATCH of them).
 int reserve_prompt_rows(axq_model *m, int cap) {
     if (cap <= m->pb_cap) return AXQ_OK;
     axq_ctx *ctx = m->ctx;
@@ -792,98 +830,175 @@ int reserve_prompt_rows(axq_model *m, int cap) {
     if (e == hipSuccess) e = dev_alloc(&m->pb_att, (size_t)cap * m->q_dim);
     if (e == hipSuccess) e = dev_alloc(&m->pb_gu, (size_t)cap * 2 * I);
     if (e == hipSuccess) e = dev_alloc(&m->pb_act, (size_t)cap * I);
-    if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "prompt activations for %d tokens: %s", cap, hipGetErrorString(e));
+    if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "activations for %d rows: %s", cap, hipGetErrorString(e));
     m->pb_cap = cap;
     return AXQ_OK;
 }
 
+// What a call of enqueue_rows works on.
+struct Rows {
+    int mode;            // ROWS_GEMV or ROWS_GEMM
+    const int32_t *toks; // [nb] device
+    int nb;
+    bool per_seq;        // false: rows pos0.. of sequence `seq`; true: row b is the next token of sequence b (nb = n_seq)
+    int seq, pos0;
+    size_t lds;          // of the attention kernel
+};
+
 template <int D>
-void launch_attn_prompt_d(axq_model *m, int l, int pos0, int nb, hipStream_t st) {
+void launch_attn_prompt_d(axq_model *m, int l, const Rows &r, hipStream_t st) {
     const axq_model_config &c = m->cfg;
     const size_t per_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * D;
-    const size_t lds = prompt_attn_lds(m, pos0, nb);
+    const size_t off = l * per_layer + (r.per_seq ? 0 : (size_t)r.seq * m->seq_stride);
     static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
-    if (lds > 48 * 1024 && !big_lds_allowed) {
+    if (r.lds > 48 * 1024 && !big_lds_allowed) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prompt_kernel<D>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
         big_lds_allowed = true;
     }
-    attn_prompt_kernel<D><<<dim3(c.num_attention_heads, nb), 1024, lds, st>>>(
-        m->pb_qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + l * per_layer, m->vcache + l * per_layer, pos0,
-        c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, c.sliding_window, m->pb_att);
+    attn_prompt_kernel<D><<<dim3(c.num_attention_heads, r.nb), 1024, r.lds, st>>>(
+        m->pb_qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0, r.per_seq ? m->pos : nullptr,
+        m->seq_stride, c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, c.sliding_window, m->pb_att);
 }
 
-// The layers for prompt tokens toks[0..nb) (device memory) at positions pos0..: what nb steps would leave in the
-// KV cache, the history and the position counter, without the final norm and lm_head (LLaMA::forward_with_cache
-// on a multi-token input, llama.rs:731-762; its logits for all but the last position are never looked at by
-// generate, llama.rs:900-977).  mode: PROMPT_GEMV (nb <= 8) or PROMPT_GEMM.
-int enqueue_prompt_rows(axq_model *m, int mode, const int32_t *toks, int nb, int pos0) {
+// The layers for `nb` rows (LLaMA::forward_with_cache on [batch, seq] input ids, llama.rs:731-762, for seq > 1 with
+// batch 1, or batch > 1 with seq 1).  Prompt rows of one sequence leave what nb steps would leave in that sequence's KV
+// cache, history and position counter, without the final norm and lm_head (generate never looks at the logits of
+// prompt positions before the last, llama.rs:900-977).  A batched step goes on to the logits and the argmax of
+// every sequence, as the one-token step does for one.
+int enqueue_rows(axq_model *m, const Rows &r) {
     axq_ctx *ctx = m->ctx;
     const axq_model_config &c = m->cfg;
     hipStream_t st = ctx->stream;
-    const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim;
+    const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim, nb = r.nb;
     int rc;
-    if ((rc = reserve_prompt_rows(m, nb))) return rc;
     // y = f(x) W^T (+ resid): f = RMSNorm when norm_w is given
     auto lin = [&](const axq_weight *w, const float *x, const float *norm_w, const float *resid, float *y) -> int {
-        if (mode == PROMPT_GEMM) return axq_dev_gemm_f32(ctx, w, x, nb, norm_w, c.rms_norm_eps, nullptr, resid, y);
+        if (r.mode == ROWS_GEMM) return axq_dev_gemm_f32(ctx, w, x, nb, norm_w, c.rms_norm_eps, nullptr, resid, y);
         if (norm_w) {
             norm_kernel<<<nb, 1024, 0, st>>>(x, norm_w, (int)w->k, c.rms_norm_eps, m->pb_xn);
             x = m->pb_xn;
         }
-        return axq_dev_gemv_batch(ctx, w, x, nb, nullptr, resid, y);
+        if (axq_dev_gemv_batch_covers(w, nb)) return axq_dev_gemv_batch(ctx, w, x, nb, nullptr, resid, y);
+        for (int b = 0; b < nb; b++) { // row by row, the residual row in the bias slot
+            int e = axq_dev_gemv(ctx, w, x + (size_t)b * w->k, 1, resid ? resid + (size_t)b * w->n_rows : nullptr, y + (size_t)b * w->n_rows);
+            if (e) return e;
+        }
+        return AXQ_OK;
     };
-    for (int t0 = 0; t0 < nb; t0 += 1024) record_tokens_kernel<<<1, nb - t0 < 1024 ? nb - t0 : 1024, 0, st>>>(m->hist, pos0 + t0, toks + t0);
-    embed_kernel<<<dim3((H / 8 + 255) / 256, nb), 256, 0, st>>>(m->emb, toks, m->pb_h, H);
+    const size_t seq_off = r.per_seq ? 0 : (size_t)r.seq * m->seq_stride;
+    if (r.per_seq) {
+        record_rows_kernel<<<1, nb, 0, st>>>(m->hist, c.max_position_embeddings, m->pos, r.toks);
+    } else {
+        int32_t *hist = m->hist + (size_t)r.seq * c.max_position_embeddings;
+        for (int t0 = 0; t0 < nb; t0 += 1024) record_tokens_kernel<<<1, nb - t0 < 1024 ? nb - t0 : 1024, 0, st>>>(hist, r.pos0 + t0, r.toks + t0);
+    }
+    embed_kernel<<<dim3((H / 8 + 255) / 256, nb), 256, 0, st>>>(m->emb, r.toks, m->pb_h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
-        const size_t per_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * d;
+        const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * d + seq_off;
         if ((rc = lin(m->w_qkv[l], m->pb_h, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv))) return rc;
         rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
-            m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + l * per_layer,
-            m->vcache + l * per_layer, pos0, c.max_position_embeddings, d);
+            m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0,
+            r.per_seq ? m->pos : nullptr, m->seq_stride, c.max_position_embeddings, d);
         switch (d) {
-        case 32: launch_attn_prompt_d<32>(m, l, pos0, nb, st); break;
-        case 64: launch_attn_prompt_d<64>(m, l, pos0, nb, st); break;
-        case 128: launch_attn_prompt_d<128>(m, l, pos0, nb, st); break;
-        default: launch_attn_prompt_d<256>(m, l, pos0, nb, st); break;
+        case 32: launch_attn_prompt_d<32>(m, l, r, st); break;
+        case 64: launch_attn_prompt_d<64>(m, l, r, st); break;
+        case 128: launch_attn_prompt_d<128>(m, l, r, st); break;
+        default: launch_attn_prompt_d<256>(m, l, r, st); break;
         }
         if ((rc = lin(m->w_o[l], m->pb_att, nullptr, m->pb_h, m->pb_h))) return rc;
         if ((rc = lin(m->w_gu[l], m->pb_h, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu))) return rc;
         swiglu_kernel<<<dim3((I / 4 + 255) / 256, nb), 256, 0, st>>>(m->pb_gu, I, m->pb_act);
         if ((rc = lin(m->w_down[l], m->pb_act, nullptr, m->pb_h, m->pb_h))) return rc;
     }
-    add_i32_kernel<<<1, 1, 0, st>>>(m->pos, nb);
-    AXQ_LAUNCH_CHECK(ctx, "prompt rows");
+    if (r.per_seq) {
+        norm_kernel<<<nb, 1024, 0, st>>>(m->pb_h, m->norm_final, H, c.rms_norm_eps, m->pb_xn);
+        if ((rc = axq_dev_gemv(ctx, m->w_head, m->pb_xn, nb, nullptr, m->logits))) return rc;
+        argmax_kernel<<<nb, 1024, 0, st>>>(m->logits, c.vocab_size, m->next, m->pos);
+    } else {
+        add_i32_kernel<<<1, 1, 0, st>>>(m->pos + r.seq, nb);
+    }
+    AXQ_LAUNCH_CHECK(ctx, "rows through the layers");
     return AXQ_OK;
 }
 
-// Feeds prompt[0..n) (already in m->prompt) from position base on: all but the last token several at a time
-// where a batched path covers them, the rest (and always the last, whose logits are wanted) one by one.
+// Feeds toks[0..n) (device memory) to sequence `seq` from position pos0 on as rows, several at a time; returns how many
+// went in (all, unless the attention scores of so long a context do not fit LDS: then none from there on).
+int feed_rows(axq_model *m, int seq, const int32_t *toks, int n, int pos0, int *fed) {
+    static const char *knob = getenv("AXQ_PROMPT_BATCH"); // development knob: 0 = no rows at all, 1 = no GEMM
+    const int allow = knob ? atoi(knob) : 2;
+    int i = 0, rc;
+    *fed = 0;
+    while (allow >= 1 && i < n) {
+        const int left = n - i;
+        Rows r;
+        r.mode = ROWS_NONE; r.toks = toks + i; r.per_seq = false; r.seq = seq; r.pos0 = pos0 + i;
+        // enough rows to fill GEMM tiles (fewer where the small-batch GEMV does not apply and single rows are the alternative)
+        r.nb = left < PROMPT_CHUNK ? left : PROMPT_CHUNK;
+        if (allow >= 2 && r.nb >= (all_layers_in_small_batch_reach(m, left) ? PROMPT_GEMM_MIN : PROMPT_BATCH) &&
+            rows_mode_covers(m, ROWS_GEMM, r.pos0 + r.nb, r.nb))
+            r.mode = ROWS_GEMM;
+        if (r.mode == ROWS_NONE) {
+            r.nb = left < PROMPT_BATCH ? left : PROMPT_BATCH;
+            if (rows_mode_covers(m, ROWS_GEMV, r.pos0 + r.nb, r.nb)) r.mode = ROWS_GEMV;
+        }
+        if (r.mode == ROWS_NONE) break;
+        r.lds = prompt_attn_lds(m, r.pos0 + r.nb);
+        if ((rc = reserve_prompt_rows(m, r.nb))) return rc;
+        if ((rc = enqueue_rows(m, r))) return rc;
+        i += r.nb;
+        *fed = i;
+    }
+    return AXQ_OK;
+}
+
+// Feeds prompt[0..n) (already in m->prompt) to sequence 0 from position base on: all but the last token as rows,
+// the last (and whatever the rows could not take) by the one-token step, which also yields the logits.
 int feed_prompt(axq_model *m, int base, int n_prompt) {
     axq_ctx *ctx = m->ctx;
-    static const char *knob = getenv("AXQ_PROMPT_BATCH"); // development knob: 0 = one by one, 1 = no GEMM
-    const int allow = knob ? atoi(knob) : 2;
-    int i = 0, rc = AXQ_OK;
-    while (allow >= 1 && n_prompt - 1 - i >= 2) {
-        const int left = n_prompt - 1 - i;
-        int mode = PROMPT_SINGLE, nb = 0;
-        // enough rows to fill GEMM tiles (fewer where the small-batch GEMV does not apply and single steps are the alternative)
-        if (allow >= 2) {
-            nb = left < PROMPT_CHUNK ? left : PROMPT_CHUNK;
-            const bool gemv_ok = prompt_mode_covers(m, PROMPT_GEMV, base + i, left < PROMPT_BATCH ? left : PROMPT_BATCH);
-            if (nb >= (gemv_ok ? PROMPT_GEMM_MIN : PROMPT_BATCH) && prompt_mode_covers(m, PROMPT_GEMM, base + i, nb)) mode = PROMPT_GEMM;
-        }
-        if (mode == PROMPT_SINGLE) {
-            nb = left < PROMPT_BATCH ? left : PROMPT_BATCH;
-            if (prompt_mode_covers(m, PROMPT_GEMV, base + i, nb)) mode = PROMPT_GEMV;
-        }
-        if (mode == PROMPT_SINGLE) break;
-        if ((rc = enqueue_prompt_rows(m, mode, m->prompt + i, nb, base + i))) return rc;
-        i += nb;
-    }
+    int i = 0, rc;
+    if ((rc = feed_rows(m, 0, m->prompt, n_prompt - 1, base, &i))) return rc;
     for (; i < n_prompt && !rc; i++) {
         pick_prompt_kernel<<<1, 1, 0, ctx->stream>>>(m->prompt, m->pos, base, m->tok);
         rc = run_token(m);
     }
+    return rc;
+}
+
+// One token of every sequence: a graph of its own, captured on first use.
+int run_batch_step(axq_model *m) {
+    axq_ctx *ctx = m->ctx;
+    Rows r;
+    r.mode = ROWS_GEMV; r.toks = m->tok; r.nb = m->n_seq; r.per_seq = true; r.seq = 0; r.pos0 = 0;
+    // sized for the longest context, so that the launch can sit in a graph
+    r.lds = prompt_attn_lds(m, m->cfg.max_position_embeddings);
+    static const bool no_graph = getenv("AXQ_DECODE_GRAPH") && getenv("AXQ_DECODE_GRAPH")[0] == '0';
+    int rc;
+    if (no_graph) {
+        rc = enqueue_rows(m, r);
+    } else {
+        if (!m->graph_b_ok) {
+            hipGraph_t g = nullptr;
+            AXQ_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), AXQ_ERR_DRIVER);
+            rc = enqueue_rows(m, r);
+            hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+            if (rc) {
+                if (g) (void)hipGraphDestroy(g);
+                return rc;
+            }
+            if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipStreamEndCapture: %s", hipGetErrorString(e));
+            e = hipGraphInstantiate(&m->graph_b, g, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(g);
+            if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipGraphInstantiate: %s", hipGetErrorString(e));
+            m->graph_b_ok = true;
+        }
+        AXQ_HIP(ctx, hipGraphLaunch(m->graph_b, ctx->stream), AXQ_ERR_KERNEL_LAUNCH_FAILED);
+        rc = AXQ_OK;
+    }
+    if (rc || !m->sampling) return rc;
+    const int V = m->cfg.vocab_size, P = m->cfg.max_position_embeddings;
+    for (int s = 0; s < m->n_seq && !rc; s++) // the draw of sequence s comes from (seed + s * odd constant, position)
+        rc = axq_dev_sample(ctx, m->logits + (size_t)s * V, V, m->hist + (size_t)s * P, m->pos + s, 0, &m->sampler, 0.f, m->pos + s,
+                            m->sample_seed + 0x9E3779B97F4A7C15ull * (uint64_t)s, m->sample_scratch, m->next + s, nullptr);
     return rc;
 }
 
@@ -923,6 +1038,9 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     m->kv_dim = c.num_key_value_heads * c.head_dim;
     m->qkv_rows = m->q_dim + 2 * m->kv_dim;
     m->max_splits = (c.max_position_embeddings + ATT_CHUNK - 1) / ATT_CHUNK;
+    m->n_seq = 1;
+    m->seq_stride = (size_t)c.num_hidden_layers * c.num_key_value_heads * c.max_position_embeddings * c.head_dim;
+    m->seq_pos.assign(1, 0);
     const int L = c.num_hidden_layers, H = c.hidden_size, I = c.intermediate_size;
     m->w_qkv.assign(L, nullptr); m->w_o.assign(L, nullptr); m->w_gu.assign(L, nullptr); m->w_down.assign(L, nullptr);
     m->set_mask.assign(L, 0);
@@ -991,6 +1109,9 @@ void axq_model_free(axq_model *m) {
     axq_ctx *ctx = m->ctx;
     (void)hipStreamSynchronize(ctx->stream);
     if (m->graph_ok) (void)hipGraphExecDestroy(m->graph);
+    if (m->graph_b_ok) (void)hipGraphExecDestroy(m->graph_b);
+    for (void *p : {(void *)m->bprompt, (void *)m->boffsets, (void *)m->bout})
+        if (p) (void)hipFree(p);
     for (auto *w : m->w_qkv) axq_weight_free(ctx, w);
     for (auto *w : m->w_o) axq_weight_free(ctx, w);
     for (auto *w : m->w_gu) axq_weight_free(ctx, w);
@@ -1109,10 +1230,11 @@ int axq_model_random_init(axq_model *m, int type, float std, uint64_t seed) {
 int axq_model_reset(axq_model *m) {
     if (!m) return AXQ_ERR_INVALID_ARGUMENT;
     axq_ctx *ctx = m->ctx;
-    set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->pos, 0);
+    for (int s = 0; s < m->n_seq; s++) set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->pos + s, 0);
     set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->gen, 0);
     AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
     m->host_pos = 0;
+    m->seq_pos.assign(m->n_seq, 0);
     return AXQ_OK;
 }
 
@@ -1125,6 +1247,155 @@ int axq_model_truncate(axq_model *m, int n_positions) {
     set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->pos, n_positions);
     AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
     m->host_pos = n_positions;
+    return AXQ_OK;
+}
+
+int axq_model_set_batch(axq_model *m, int n_seq) {
+    if (!m) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    const axq_model_config &c = m->cfg;
+    if (n_seq < 1 || n_seq > PROMPT_BATCH)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_set_batch: 1 to %d sequences, got %d", PROMPT_BATCH, n_seq);
+    if (n_seq > 1 && (c.vocab_size % 4 != 0 || prompt_attn_lds(m, c.max_position_embeddings) > 128 * 1024))
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH,
+                        "Shape mismatch: batched steps need a vocabulary that is a multiple of 4 and at most 32768 positions "
+                        "(or a sliding window) per sequence");
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    // the graphs hold the old addresses
+    if (m->graph_ok) (void)hipGraphExecDestroy(m->graph);
+    if (m->graph_b_ok) (void)hipGraphExecDestroy(m->graph_b);
+    m->graph_ok = m->graph_b_ok = false;
+    const size_t P = c.max_position_embeddings, S = (size_t)n_seq;
+    for (void **p : {(void **)&m->kcache, (void **)&m->vcache, (void **)&m->pos, (void **)&m->tok, (void **)&m->next, (void **)&m->hist,
+                     (void **)&m->logits, (void **)&m->bprompt, (void **)&m->boffsets, (void **)&m->bout}) {
+        if (*p) (void)hipFree(*p);
+        *p = nullptr;
+    }
+    m->n_seq = 1; // what the pointers can back until everything below has worked
+    hipError_t e = dev_alloc(&m->kcache, S * m->seq_stride);
+    if (e == hipSuccess) e = dev_alloc(&m->vcache, S * m->seq_stride);
+    if (e == hipSuccess) e = dev_alloc(&m->pos, S);
+    if (e == hipSuccess) e = dev_alloc(&m->tok, S);
+    if (e == hipSuccess) e = dev_alloc(&m->next, S);
+    if (e == hipSuccess) e = dev_alloc(&m->hist, S * P);
+    if (e == hipSuccess) e = dev_alloc(&m->logits, S * c.vocab_size);
+    if (e == hipSuccess) e = dev_alloc(&m->bprompt, S * P);
+    if (e == hipSuccess) e = dev_alloc(&m->boffsets, S + 1);
+    if (e == hipSuccess) e = dev_alloc(&m->bout, S * m->out_cap);
+    if (e == hipSuccess) e = hipMemsetAsync(m->kcache, 0, S * m->seq_stride * 2, ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(m->vcache, 0, S * m->seq_stride * 2, ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(m->pos, 0, S * 4, ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(m->tok, 0, S * 4, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess)
+        return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "caches and state for %d sequences: %s (the model is unusable until a call of "
+                        "axq_model_set_batch succeeds)", n_seq, hipGetErrorString(e));
+    m->n_seq = n_seq;
+    m->host_pos = 0;
+    m->seq_pos.assign(n_seq, 0);
+    return AXQ_OK;
+}
+
+int axq_model_batch(const axq_model *m) { return m ? m->n_seq : -1; }
+
+int axq_model_seq_len_of(const axq_model *m, int seq) {
+    if (!m || seq < 0 || seq >= m->n_seq) return -1;
+    return seq == 0 ? m->host_pos : m->seq_pos[seq];
+}
+
+int axq_model_forward_batch(axq_model *m, const int32_t *tokens, float *logits, int32_t *next_tokens) {
+    if (!m || !tokens) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    int rc;
+    if ((rc = check_ready(m))) return rc;
+    const int S = m->n_seq, V = m->cfg.vocab_size;
+    m->seq_pos[0] = m->host_pos;
+    for (int s = 0; s < S; s++) {
+        if (tokens[s] < 0 || tokens[s] >= V)
+            return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "token %d outside the vocabulary of %d", tokens[s], V);
+        if (m->seq_pos[s] >= m->cfg.max_position_embeddings)
+            return axq_fail(ctx, AXQ_ERR_OVERFLOW, "Numerical overflow during quantization: KV cache of sequence %d is full (%d positions)", s,
+                            m->cfg.max_position_embeddings);
+    }
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipMemcpyAsync(m->tok, tokens, (size_t)S * 4, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    if ((rc = run_batch_step(m))) return rc;
+    for (int s = 0; s < S; s++) m->seq_pos[s]++;
+    m->host_pos = m->seq_pos[0];
+    if (logits)
+        AXQ_HIP(ctx, hipMemcpyAsync(logits, m->logits, (size_t)S * V * 4, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    if (next_tokens)
+        AXQ_HIP(ctx, hipMemcpyAsync(next_tokens, m->next, (size_t)S * 4, hipMemcpyDeviceToHost, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_model_generate_batch(axq_model *m, const int32_t *prompts, const int32_t *offsets, int max_new_tokens, int32_t *out_tokens,
+                             float *prefill_ms, float *decode_ms) {
+    if (!m || !prompts || !offsets || !out_tokens) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    int rc;
+    if ((rc = check_ready(m))) return rc;
+    const int S = m->n_seq, P = m->cfg.max_position_embeddings;
+    if (max_new_tokens < 1 || max_new_tokens > m->out_cap || offsets[0] != 0)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: 1 to %d new tokens, offsets starting at 0", m->out_cap);
+    for (int s = 0; s < S; s++) {
+        const int n = offsets[s + 1] - offsets[s];
+        if (n < 1) return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: prompt %d must hold at least one token", s);
+        if (n + max_new_tokens - 1 > P)
+            return axq_fail(ctx, AXQ_ERR_OVERFLOW, "Numerical overflow during quantization: %d + %d positions of sequence %d exceed the cache of %d",
+                            n, max_new_tokens, s, P);
+        for (int i = offsets[s]; i < offsets[s + 1]; i++)
+            if (prompts[i] < 0 || prompts[i] >= m->cfg.vocab_size)
+                return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "prompt token %d outside the vocabulary", prompts[i]);
+    }
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    if ((rc = axq_model_reset(m))) return rc;
+    if (!m->bprompt) { // a model that never saw axq_model_set_batch: one sequence
+        hipError_t e = dev_alloc(&m->bprompt, (size_t)P);
+        if (e == hipSuccess) e = dev_alloc(&m->boffsets, 2);
+        if (e == hipSuccess) e = dev_alloc(&m->bout, (size_t)m->out_cap);
+        if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "prompt buffers: %s", hipGetErrorString(e));
+    }
+    AXQ_HIP(ctx, hipMemcpyAsync(m->bprompt, prompts, (size_t)offsets[S] * 4, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipMemcpyAsync(m->boffsets, offsets, (size_t)(S + 1) * 4, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    hipEvent_t e0, e1, e2;
+    AXQ_HIP(ctx, hipEventCreate(&e0), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipEventCreate(&e1), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipEventCreate(&e2), AXQ_ERR_DRIVER);
+    (void)hipEventRecord(e0, ctx->stream);
+    // every prompt but its last token, sequence by sequence; the last tokens are the input of the first batched step
+    for (int s = 0; s < S && !rc; s++) {
+        const int n = offsets[s + 1] - offsets[s] - 1;
+        int fed = 0;
+        rc = feed_rows(m, s, m->bprompt + offsets[s], n, 0, &fed);
+        if (!rc && fed != n) rc = axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: prompt %d cannot go through the layers as rows", s);
+    }
+    if (!rc) last_tokens_kernel<<<1, S, 0, ctx->stream>>>(m->bprompt, m->boffsets, m->tok);
+    (void)hipEventRecord(e1, ctx->stream);
+    for (int i = 0; i < max_new_tokens && !rc; i++) {
+        rc = run_batch_step(m);
+        if (!rc) commit_rows_kernel<<<1, S, 0, ctx->stream>>>(m->next, m->tok, m->bout, i, m->out_cap);
+    }
+    (void)hipEventRecord(e2, ctx->stream);
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    float ms = 0.f;
+    if (!rc && e == hipSuccess) {
+        if (prefill_ms && hipEventElapsedTime(&ms, e0, e1) == hipSuccess) *prefill_ms = ms;
+        if (decode_ms && hipEventElapsedTime(&ms, e1, e2) == hipSuccess) *decode_ms = ms;
+    }
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); (void)hipEventDestroy(e2);
+    if (rc || e != hipSuccess) { // positions on the device may have moved: start over
+        (void)axq_model_reset(m);
+        return rc ? rc : axq_fail(ctx, AXQ_ERR_DRIVER, "generate: %s", hipGetErrorString(e));
+    }
+    for (int s = 0; s < S; s++) {
+        m->seq_pos[s] = offsets[s + 1] - offsets[s] + max_new_tokens - 1;
+        AXQ_HIP(ctx, hipMemcpy(out_tokens + (size_t)s * max_new_tokens, m->bout + (size_t)s * m->out_cap, (size_t)max_new_tokens * 4,
+                               hipMemcpyDeviceToHost), AXQ_ERR_COPY_FAILED);
+    }
+    m->host_pos = m->seq_pos[0];
     return AXQ_OK;
 }
 

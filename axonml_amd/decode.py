@@ -81,6 +81,42 @@ class QuantizedLlama:
                                                              logits.ctypes.data if want_logits else None, C.byref(nxt)))
         return nxt.value, logits
 
+    def set_batch(self, n_seq):
+        """Caches and positions for n_seq sequences side by side (1..8); starts all of them afresh."""
+        self.ctx.check(self.ctx.lib.axq_model_set_batch(self.handle, int(n_seq)))
+
+    def batch(self):
+        return self.ctx.lib.axq_model_batch(self.handle)
+
+    def seq_len_of(self, seq):
+        return self.ctx.lib.axq_model_seq_len_of(self.handle, int(seq))
+
+    def forward_batch(self, tokens, want_logits=True):
+        """One token of every sequence: (next tokens [n_seq], logits [n_seq, vocab])."""
+        n = self.batch()
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        if t.shape != (n,):
+            raise ValueError(f"{n} tokens wanted, one per sequence")
+        logits = np.empty((n, self.cfg.vocab_size), dtype=np.float32) if want_logits else None
+        nxt = np.empty(n, dtype=np.int32)
+        self.ctx.check(self.ctx.lib.axq_model_forward_batch(self.handle, t.ctypes.data, logits.ctypes.data if want_logits else None,
+                                                            nxt.ctypes.data))
+        return nxt, logits
+
+    def generate_batch(self, prompts, max_new_tokens):
+        """prompts: n_seq token lists of any lengths -> (ids [n_seq, max_new_tokens], prompt ms, generation ms)."""
+        n = self.batch()
+        if len(prompts) != n:
+            raise ValueError(f"{n} prompts wanted, one per sequence")
+        flat = np.ascontiguousarray(np.concatenate([np.asarray(p, dtype=np.int32).reshape(-1) for p in prompts]), dtype=np.int32)
+        offsets = np.zeros(n + 1, dtype=np.int32)
+        offsets[1:] = np.cumsum([len(p) for p in prompts])
+        out = np.empty((n, max_new_tokens), dtype=np.int32)
+        pre, dec = C.c_float(), C.c_float()
+        self.ctx.check(self.ctx.lib.axq_model_generate_batch(self.handle, flat.ctypes.data, offsets.ctypes.data, max_new_tokens,
+                                                             out.ctypes.data, C.byref(pre), C.byref(dec)))
+        return out, pre.value, dec.value
+
     def truncate(self, n_positions):
         """Rewind the cache to its first n_positions."""
         self.ctx.check(self.ctx.lib.axq_model_truncate(self.handle, int(n_positions)))
@@ -186,5 +222,17 @@ def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
     res["sampled_tokens_per_s"] = steps / (dec_s * 1e-3)
     res["sampler_us_per_token"] = (dec_s - dec_ms) / steps * 1e3
     log(f"  with top-k/top-p sampling: {res['sampled_tokens_per_s']:.1f} tok/s (sampler {res['sampler_us_per_token']:.0f} us per token)")
+    # eight sequences side by side, greedy: one pass over the weights per step serves all of them
+    m.set_sampling(None)
+    for n_seq in (2, 4, 8):
+        m.set_batch(n_seq)
+        prompts = [rng.integers(0, cfg["vocab_size"], size=prompt_len, dtype=np.int32) for _ in range(n_seq)]
+        m.generate_batch(prompts, 4)
+        _, pre_b, dec_b = m.generate_batch(prompts, new_tokens)
+        res[f"batch{n_seq}_tokens_per_s"] = n_seq * new_tokens / (dec_b * 1e-3)
+        res[f"batch{n_seq}_ms_per_step"] = dec_b / new_tokens
+        res[f"batch{n_seq}_prefill_tokens_per_s"] = n_seq * (prompt_len - 1) / (pre_b * 1e-3)
+        log(f"  {n_seq} sequences: {res[f'batch{n_seq}_tokens_per_s']:.0f} tok/s in all ({res[f'batch{n_seq}_ms_per_step']:.3f} ms per step), "
+            f"prompts {res[f'batch{n_seq}_prefill_tokens_per_s']:.0f} tok/s")
     m.close()
     return res

@@ -214,6 +214,22 @@ AXQ_API int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_
  * multiple of 256 up to 16384, else one by one; results agree with n calls of axq_model_forward to
  * rounding (sums are taken in another order). */
 AXQ_API int axq_model_forward_tokens(axq_model *m, const int32_t *tokens, int n, float *logits, int32_t *next_token);
+/* Several sequences side by side (the batch dimension of forward_with_cache's input ids and of KVCache,
+ * llama.rs:731-762, attention.rs:28-35): n_seq = 1..8 caches and position counters; a batched step feeds
+ * one token of every sequence and reads the weights once for all of them.  Calling it discards every
+ * cache and starts all sequences at position 0.  The one-sequence calls above keep working on sequence 0. */
+AXQ_API int axq_model_set_batch(axq_model *m, int n_seq);
+AXQ_API int axq_model_batch(const axq_model *m);
+AXQ_API int axq_model_seq_len_of(const axq_model *m, int seq);
+/* tokens: int32[n_seq]; logits (host, may be NULL): f32[n_seq, vocab]; next_tokens (host, may be NULL): int32[n_seq].
+ * Sequences may stand at different positions. */
+AXQ_API int axq_model_forward_batch(axq_model *m, const int32_t *tokens, float *logits, int32_t *next_tokens);
+/* generate for n_seq prompts of any lengths at once: prompts holds them back to back, prompt s is
+ * prompts[offsets[s] .. offsets[s+1]) (offsets: int32[n_seq + 1], offsets[0] = 0).  Starts every sequence
+ * afresh.  out_tokens: int32[n_seq, max_new_tokens].  Each sequence gets what axq_model_generate gives for
+ * its prompt alone, to rounding (sums are taken in another order). */
+AXQ_API int axq_model_generate_batch(axq_model *m, const int32_t *prompts, const int32_t *offsets, int max_new_tokens,
+                                     int32_t *out_tokens, float *prefill_ms, float *decode_ms);
 /* generate (llama.rs:900-977), greedy: feeds the prompt (as axq_model_forward_tokens does), then max_new_tokens
  * steps, each consuming the previous argmax on the device.  out_tokens gets
  * max_new_tokens ids (host).  Timings (ms, may be NULL) cover prompt and
@@ -247,7 +263,7 @@ AXQ_API int axq_sample_token(axq_ctx *ctx, const float *logits, int vocab, const
                              const axq_sampling_config *cfg, float u, int32_t *token, float *filtered_logits, int mem);
 /* Makes axq_model_forward / axq_model_generate choose the next token this way instead of by the plain
  * argmax; the penalty sees every token fed so far, the draw of a step comes from (seed, position).
- * cfg = NULL: back to greedy. */
+ * cfg = NULL: back to greedy.  In batched steps sequence s draws from (seed + s * 0x9E3779B97F4A7C15, position). */
 AXQ_API int axq_model_set_sampling(axq_model *m, const axq_sampling_config *cfg, uint64_t seed);
 
 /* ---- benchmark utilities ------------------------------------------------- */

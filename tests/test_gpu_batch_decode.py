@@ -1,0 +1,141 @@
+"""GPU parity: several sequences side by side (batched steps, one pass over the weights for all of them)
+against the CPU decode oracle walking every sequence on its own.  Bar as for the one-sequence step: greedy
+token ids identical, logits within 1e-3 of the logit range."""
+import numpy as np
+import pytest
+
+import oracle as o
+from tests.decode_common import load_gpu, load_oracle, random_weights, tiny_config
+from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_walk(cpu, prompt, n_new):
+    """Greedy ids and the logits of every step for one prompt (the oracle overwrites cache rows by position)."""
+    ids, logits = [], []
+    for pos, t in enumerate(prompt):
+        nxt, lg = cpu.forward(int(t), pos)
+    for i in range(n_new):
+        ids.append(nxt)
+        logits.append(lg)
+        if i + 1 < n_new:
+            nxt, lg = cpu.forward(nxt, len(prompt) + i)
+    return ids, logits
+
+
+@pytest.mark.parametrize("n_seq,qtype,over", [(2, o.Q4_K, {}), (8, o.Q4_K, {}), (5, o.Q4_0, dict(num_layers=3)), (3, o.Q8_0, {}),
+                                              (4, o.Q5_1, {}),  # outside the small-batch GEMV: rows go one by one
+                                              (8, o.Q4_K, dict(num_heads=8, num_kv_heads=2, head_dim=32)),
+                                              (3, o.Q4_1, dict(num_heads=2, num_kv_heads=1, head_dim=128)),
+                                              (4, o.Q4_K, dict(sliding_window=6)), (1, o.Q4_K, {})])
+def test_generate_batch_matches_the_oracle_sequence_by_sequence(ctx, n_seq, qtype, over):
+    c = tiny_config(max_seq_len=96, **over)
+    w = random_weights(c, 200 + n_seq + qtype, qtype=qtype)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    gpu.set_batch(n_seq)
+    rng = np.random.default_rng(n_seq)
+    lengths = [1, 2, 9, 40, 17, 3, 64, 10][:n_seq]  # ragged: one token, GEMV rows, GEMM rows
+    prompts = [rng.integers(0, c["vocab_size"], size=n) for n in lengths]
+    n_new = 14
+    got, pre_ms, dec_ms = gpu.generate_batch(prompts, n_new)
+    assert got.shape == (n_seq, n_new) and pre_ms >= 0 and dec_ms > 0
+    for s, p in enumerate(prompts):
+        want, _ = _oracle_walk(cpu, p, n_new)
+        assert got[s].tolist() == want, s
+        assert gpu.seq_len_of(s) == len(p) + n_new - 1
+    again, _, _ = gpu.generate_batch(prompts, n_new)  # starts afresh; graph replays are deterministic
+    assert np.array_equal(again, got)
+    gpu.close()
+    cpu.close()
+
+
+def test_forward_batch_logits_at_different_positions(ctx):
+    c = tiny_config(max_seq_len=64)
+    w = random_weights(c, 300)
+    gpu = load_gpu(ctx, c, w)
+    n_seq = 4
+    gpu.set_batch(n_seq)
+    cpus = [load_oracle(c, w) for _ in range(n_seq)]
+    # bring the sequences to different positions: sequence 0 through the one-sequence calls, which work on it
+    rng = np.random.default_rng(1)
+    head = rng.integers(0, c["vocab_size"], size=5)
+    for pos, t in enumerate(head):
+        cpus[0].forward(int(t), pos)
+    gpu.forward_tokens(head, want_logits=False)
+    assert gpu.seq_len_of(0) == 5 and gpu.seq_len_of(1) == 0
+    toks = [3, 7, 11, 13]
+    pos = [5, 0, 0, 0]
+    for step in range(12):
+        g_next, g_logits = gpu.forward_batch(toks)
+        for s in range(n_seq):
+            c_next, c_logits = cpus[s].forward(int(toks[s]), pos[s])
+            assert max_rel_err(g_logits[s], c_logits, DECODE_FLOOR) <= DECODE_RTOL, (step, s)
+            assert g_next[s] == c_next, (step, s)
+            pos[s] += 1
+        toks = g_next.tolist()
+    assert [gpu.seq_len_of(s) for s in range(n_seq)] == pos and gpu.seq_len() == pos[0]
+    # the one-sequence step goes on from where the batched ones left sequence 0
+    c_next, c_logits = cpus[0].forward(int(toks[0]), pos[0])
+    g_next1, g_logits1 = gpu.forward(int(toks[0]))
+    assert g_next1 == c_next and max_rel_err(g_logits1, c_logits, DECODE_FLOOR) <= DECODE_RTOL
+    gpu.reset()
+    assert [gpu.seq_len_of(s) for s in range(n_seq)] == [0] * n_seq
+    gpu.close()
+    for m in cpus:
+        m.close()
+
+
+def test_batched_sampling_follows_each_sequences_own_history(ctx):
+    from axonml_amd.generation import GenerationConfig
+
+    c = tiny_config(max_seq_len=64)
+    w = random_weights(c, 310)
+    gpu, one = load_gpu(ctx, c, w), load_gpu(ctx, c, w)
+    gpu.set_batch(3)
+    cfg = GenerationConfig(temperature=0.9, top_k=12, top_p=0.95, repetition_penalty=1.3)
+    seed = 99
+    gpu.set_sampling(cfg, seed)
+    rng = np.random.default_rng(2)
+    prompts = [rng.integers(0, c["vocab_size"], size=n) for n in (6, 11, 2)]
+    got, _, _ = gpu.generate_batch(prompts, 10)
+    for s, p in enumerate(prompts):  # sequence s draws from (seed + s * odd constant, position)
+        one.reset()
+        one.set_sampling(cfg, (seed + 0x9E3779B97F4A7C15 * s) % (1 << 64))
+        want, _, _ = one.generate(p, 10)
+        assert got[s].tolist() == want.tolist(), s
+    gpu.close()
+    one.close()
+
+
+def test_batch_errors(ctx):
+    from axonml_amd import quant as q
+
+    c = tiny_config(num_layers=1)
+    m = load_gpu(ctx, c, random_weights(c, 320))
+    assert m.batch() == 1
+    with pytest.raises(q.QuantError):
+        m.set_batch(0)
+    with pytest.raises(q.QuantError):
+        m.set_batch(9)
+    m.set_batch(2)
+    assert m.batch() == 2
+    with pytest.raises(ValueError):
+        m.forward_batch([1])
+    with pytest.raises(q.QuantError):
+        m.forward_batch([1, 10 ** 6])
+    with pytest.raises(q.ShapeMismatch):
+        m.generate_batch([[1, 2], []], 3)
+    with pytest.raises(q.Overflow):
+        m.generate_batch([[1, 2], [3] * c["max_seq_len"]], 3)
+    with pytest.raises(q.ShapeMismatch):
+        m.generate_batch([[1], [2]], 0)
+    for _ in range(c["max_seq_len"]):
+        m.forward_batch([1, 2], want_logits=False)
+    with pytest.raises(q.Overflow):
+        m.forward_batch([1, 2])
+    m.set_batch(1)  # back to one sequence, afresh
+    assert m.seq_len() == 0
+    nxt, _ = m.forward(3)
+    assert 0 <= nxt < c["vocab_size"]
+    m.close()
