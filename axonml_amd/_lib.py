@@ -103,6 +103,7 @@ SIGNATURES = {
     "axq_model_seq_len": (_i, [_vp]),
     "axq_model_set_batch": (_i, [_vp, _i]),
     "axq_model_batch": (_i, [_vp]),
+    "axq_model_copy_sequence": (_i, [_vp, _i, _i]),
     "axq_model_seq_len_of": (_i, [_vp, _i]),
     "axq_model_forward_batch": (_i, [_vp, _vp, _vp, _vp]),
     "axq_model_generate_batch": (_i, [_vp, _vp, _vp, _i, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float)]),

@@ -1304,6 +1304,34 @@ int axq_model_seq_len_of(const axq_model *m, int seq) {
     return seq == 0 ? m->host_pos : m->seq_pos[seq];
 }
 
+int axq_model_copy_sequence(axq_model *m, int src, int dst) {
+    if (!m) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    const axq_model_config &c = m->cfg;
+    if (src < 0 || src >= m->n_seq || dst < 0 || dst >= m->n_seq)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_copy_sequence: sequences %d -> %d of %d", src, dst, m->n_seq);
+    if (src == dst) return AXQ_OK;
+    m->seq_pos[0] = m->host_pos;
+    const int n = m->seq_pos[src];
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    if (n > 0) {
+        // per (layer, kv head): the first n rows of max_pos
+        const size_t pitch = (size_t)c.max_position_embeddings * c.head_dim * 2, width = (size_t)n * c.head_dim * 2;
+        const size_t rows = (size_t)c.num_hidden_layers * c.num_key_value_heads;
+        AXQ_HIP(ctx, hipMemcpy2DAsync(m->kcache + (size_t)dst * m->seq_stride, pitch, m->kcache + (size_t)src * m->seq_stride, pitch, width,
+                                      rows, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+        AXQ_HIP(ctx, hipMemcpy2DAsync(m->vcache + (size_t)dst * m->seq_stride, pitch, m->vcache + (size_t)src * m->seq_stride, pitch, width,
+                                      rows, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+        AXQ_HIP(ctx, hipMemcpyAsync(m->hist + (size_t)dst * c.max_position_embeddings, m->hist + (size_t)src * c.max_position_embeddings,
+                                    (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
+    }
+    set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->pos + dst, n);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    m->seq_pos[dst] = n;
+    m->host_pos = m->seq_pos[0];
+    return AXQ_OK;
+}
+
 int axq_model_forward_batch(axq_model *m, const int32_t *tokens, float *logits, int32_t *next_tokens) {
     if (!m || !tokens) return AXQ_ERR_INVALID_ARGUMENT;
     axq_ctx *ctx = m->ctx;

@@ -91,6 +91,10 @@ class QuantizedLlama:
     def seq_len_of(self, seq):
         return self.ctx.lib.axq_model_seq_len_of(self.handle, int(seq))
 
+    def copy_sequence(self, src, dst):
+        """Sequence dst becomes a copy of sequence src (cache, history, position)."""
+        self.ctx.check(self.ctx.lib.axq_model_copy_sequence(self.handle, int(src), int(dst)))
+
     def forward_batch(self, tokens, want_logits=True):
         """One token of every sequence: (next tokens [n_seq], logits [n_seq, vocab])."""
         n = self.batch()

@@ -143,11 +143,18 @@ class BeamSearch:
         return None if best is None else list(best.tokens)
 
 
-def beam_search_generate(model, input_ids, beam_search, max_new_tokens):
+def beam_search_generate(model, input_ids, beam_search, max_new_tokens, batched=None):
     """Beam search over a `QuantizedLlama`: per step every live beam's next-token logits, then
-    `expand_beams`, until `max_new_tokens` or `should_stop`.  The model keeps one sequence, so a beam is
-    brought in by rewinding the cache to the prefix it shares with the cached tokens and feeding the rest
-    (`truncate`, `forward_tokens`).  Returns (best_sequence, beams)."""
+    `expand_beams`, until `max_new_tokens` or `should_stop`.  Returns (best_sequence, beams).
+
+    batched (default: when the model can and there are 2..8 beams): every beam lives in a sequence slot of the
+    model and one batched step serves all of them; a beam that forks copies its slot (`copy_sequence`).
+    Otherwise the model keeps one sequence, and a beam is brought in by rewinding the cache to the prefix it
+    shares with the cached tokens and feeding the rest (`truncate`, `forward_tokens`)."""
+    if batched is None:
+        batched = hasattr(model, "forward_batch") and 2 <= beam_search.num_beams <= 8
+    if batched:
+        return _beam_search_batched(model, input_ids, beam_search, max_new_tokens)
     beams = beam_search.init_beams(input_ids)
     cached = []  # tokens whose keys and values the model's cache holds now
     if model.seq_len():
@@ -168,5 +175,44 @@ def beam_search_generate(model, input_ids, beam_search, max_new_tokens):
             per_beam.append(logits)
         beams = beam_search.expand_beams(beams, per_beam)
         if beam_search.should_stop(beams):
+            break
+    return beam_search.best_sequence(beams), beams
+
+
+def _beam_search_batched(model, input_ids, beam_search, max_new_tokens):
+    n_slots = beam_search.num_beams
+    if model.batch() != n_slots:
+        model.set_batch(n_slots)
+    else:
+        model.reset()
+    beams = beam_search.init_beams(input_ids)
+    prompt = beams[0].tokens
+    if len(prompt) > 1:
+        model.forward_tokens(prompt[:-1], want_logits=False)  # sequence 0
+    for s in range(1, n_slots):  # all slots march in step, so idle ones never run ahead of the live ones
+        model.copy_sequence(0, s)
+    slot_of = {0: 0}  # index into `beams` -> slot, live beams only
+    for _ in range(max_new_tokens):
+        feed = [0] * n_slots
+        for i, slot in slot_of.items():
+            feed[slot] = beams[i].tokens[-1]
+        _, logits = model.forward_batch(feed)
+        per_beam = [logits[slot_of[i]] if i in slot_of else None for i in range(len(beams))]
+        grown = beam_search.expand_beams(beams, per_beam)
+        # a live beam of the new set continues the old live beam whose tokens it extends by one
+        by_tokens = {tuple(beams[i].tokens): slot for i, slot in slot_of.items()}
+        parents = [None if b.finished else by_tokens[tuple(b.tokens[:-1])] for b in grown]
+        first_child, new_slots = {}, {}
+        for j, parent in enumerate(parents):
+            if parent is not None and parent not in first_child:
+                first_child[parent] = j
+                new_slots[j] = parent
+        free = [s for s in range(n_slots) if s not in first_child]
+        for j, parent in enumerate(parents):
+            if parent is not None and j not in new_slots:
+                new_slots[j] = free.pop()
+                model.copy_sequence(parent, new_slots[j])
+        beams, slot_of = grown, new_slots
+        if beam_search.should_stop(beams) or not slot_of:
             break
     return beam_search.best_sequence(beams), beams

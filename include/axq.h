@@ -221,6 +221,9 @@ AXQ_API int axq_model_forward_tokens(axq_model *m, const int32_t *tokens, int n,
 AXQ_API int axq_model_set_batch(axq_model *m, int n_seq);
 AXQ_API int axq_model_batch(const axq_model *m);
 AXQ_API int axq_model_seq_len_of(const axq_model *m, int seq);
+/* Sequence dst becomes a copy of sequence src (cache rows, token history, position): two continuations of one
+ * prefix, as beam search forks them. */
+AXQ_API int axq_model_copy_sequence(axq_model *m, int src, int dst);
 /* tokens: int32[n_seq]; logits (host, may be NULL): f32[n_seq, vocab]; next_tokens (host, may be NULL): int32[n_seq].
  * Sequences may stand at different positions. */
 AXQ_API int axq_model_forward_batch(axq_model *m, const int32_t *tokens, float *logits, int32_t *next_tokens);

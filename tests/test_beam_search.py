@@ -83,8 +83,13 @@ class _OracleSequenceModel:
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("num_beams,length_penalty", [(1, 1.0), (3, 1.0), (4, 0.0)])
-def test_driver_against_the_oracle(ctx, num_beams, length_penalty):
+@pytest.mark.parametrize("batched", [False, True])
+@pytest.mark.parametrize("num_beams,length_penalty", [(1, 1.0), (3, 1.0), (4, 0.0), (8, 1.5), (2, 1.0)])
+def test_driver_against_the_oracle(ctx, num_beams, length_penalty, batched):
+    """batched: every beam in a sequence slot of the model, one batched step per search step, forks copy their slot;
+    otherwise one sequence, rewound and re-fed per beam.  Both against the same bookkeeping over the CPU oracle."""
+    if batched and num_beams == 1:
+        pytest.skip("one beam needs no slots")
     from tests.decode_common import load_gpu, load_oracle, random_weights, tiny_config
 
     c = tiny_config(num_layers=2, max_seq_len=64)
@@ -93,7 +98,7 @@ def test_driver_against_the_oracle(ctx, num_beams, length_penalty):
     prompt = np.random.default_rng(num_beams).integers(0, c["vocab_size"], size=11)
     eos = [5, 17]
     want_seq, want_beams = beam_search_generate(_OracleSequenceModel(cpu), prompt, BeamSearch(num_beams, length_penalty, True, eos), 12)
-    got_seq, got_beams = beam_search_generate(gpu, prompt, BeamSearch(num_beams, length_penalty, True, eos), 12)
+    got_seq, got_beams = beam_search_generate(gpu, prompt, BeamSearch(num_beams, length_penalty, True, eos), 12, batched=batched)
     assert got_seq == want_seq
     assert [b.tokens for b in got_beams] == [b.tokens for b in want_beams]
     for g, r in zip(got_beams, want_beams):

@@ -139,3 +139,32 @@ def test_batch_errors(ctx):
     nxt, _ = m.forward(3)
     assert 0 <= nxt < c["vocab_size"]
     m.close()
+
+
+def test_copy_sequence_forks_a_prefix(ctx):
+    c = tiny_config(max_seq_len=64)
+    w = random_weights(c, 330)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    gpu.set_batch(3)
+    rng = np.random.default_rng(3)
+    prefix = rng.integers(0, c["vocab_size"], size=13)
+    gpu.forward_tokens(prefix, want_logits=False)  # sequence 0
+    gpu.copy_sequence(0, 2)
+    assert [gpu.seq_len_of(s) for s in range(3)] == [13, 0, 13]
+    # sequences 0 and 2 go on with different tokens, sequence 1 starts from nothing
+    conts = [[5, 6, 7, 8], [9, 10, 11, 12], [200, 201, 202, 203]]
+    want = []
+    for s, cont in enumerate(conts):
+        seq = (list(prefix) if s != 1 else []) + cont
+        for pos, t in enumerate(seq):
+            nxt, lg = cpu.forward(int(t), pos)
+        want.append((nxt, lg))
+    for i in range(4):
+        g_next, g_logits = gpu.forward_batch([conts[s][i] for s in range(3)])
+    for s in range(3):
+        assert g_next[s] == want[s][0], s
+        assert max_rel_err(g_logits[s], want[s][1], DECODE_FLOOR) <= DECODE_RTOL, s
+    with pytest.raises(Exception):
+        gpu.copy_sequence(0, 3)
+    gpu.close()
+    cpu.close()
