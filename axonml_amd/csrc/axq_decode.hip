@@ -820,6 +820,10 @@ int reserve_prompt_rows(axq_model *m, int cap) {
     axq_ctx *ctx = m->ctx;
     const int H = m->cfg.hidden_size, I = m->cfg.intermediate_size;
     AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    if (m->graph_b_ok) { // the batched step's graph holds the old addresses
+        (void)hipGraphExecDestroy(m->graph_b);
+        m->graph_b_ok = false;
+    }
     for (float **p : {&m->pb_h, &m->pb_qkv, &m->pb_att, &m->pb_gu, &m->pb_act}) {
         if (*p) (void)hipFree(*p);
         *p = nullptr;
@@ -1557,8 +1561,11 @@ int axq_model_generate(axq_model *m, const int32_t *prompt, int n_prompt, int ma
         if (decode_ms && hipEventElapsedTime(&ms, e1, e2) == hipSuccess) *decode_ms = ms;
     }
     (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); (void)hipEventDestroy(e2);
-    if (rc) return rc;
-    if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "generate: %s", hipGetErrorString(e));
+    if (rc || e != hipSuccess) { // the device-side position may have moved: bring both sides back to where the call started
+        set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->pos, base);
+        (void)hipStreamSynchronize(ctx->stream);
+        return rc ? rc : axq_fail(ctx, AXQ_ERR_DRIVER, "generate: %s", hipGetErrorString(e));
+    }
     m->host_pos = base + n_prompt + (max_new_tokens > 0 ? max_new_tokens - 1 : 0);
     if (max_new_tokens > 0)
         AXQ_HIP(ctx, hipMemcpy(out_tokens, m->out, (size_t)max_new_tokens * 4, hipMemcpyDeviceToHost), AXQ_ERR_COPY_FAILED);

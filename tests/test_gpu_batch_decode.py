@@ -46,6 +46,12 @@ def test_generate_batch_matches_the_oracle_sequence_by_sequence(ctx, n_seq, qtyp
         assert gpu.seq_len_of(s) == len(p) + n_new - 1
     again, _, _ = gpu.generate_batch(prompts, n_new)  # starts afresh; graph replays are deterministic
     assert np.array_equal(again, got)
+    if n_seq == 2:  # longer prompts after the step's graph exists: the row buffers grow, and the graph is taken anew
+        longer = [rng.integers(0, c["vocab_size"], size=n) for n in (70, 33)]
+        got2, _, _ = gpu.generate_batch(longer, 6)
+        for s, p in enumerate(longer):
+            want, _ = _oracle_walk(cpu, p, 6)
+            assert got2[s].tolist() == want, s
     gpu.close()
     cpu.close()
 
