@@ -174,3 +174,38 @@ def test_copy_sequence_forks_a_prefix(ctx):
         gpu.copy_sequence(0, 3)
     gpu.close()
     cpu.close()
+
+
+def test_one_layer_at_the_7b_shape(ctx):
+    """The real layer shape (hidden 4096, intermediate 14336, 32 query heads over 8 KV heads of 128, Q4_K) with a
+    small vocabulary and one layer, so that the CPU oracle finishes in seconds: the one-token step, a prompt
+    through the GEMM rows, the small-batch rows, and batched steps of eight sequences, all against the oracle."""
+    c = tiny_config(vocab_size=1024, hidden_size=4096, intermediate_size=14336, num_layers=1, num_heads=32, num_kv_heads=8,
+                    head_dim=128, max_seq_len=96)
+    w = random_weights(c, 400, std=0.02)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    rng = np.random.default_rng(4)
+    prompt = rng.integers(0, c["vocab_size"], size=50)  # 49 rows through the GEMM, the last by the one-token step
+    for pos, t in enumerate(prompt):
+        c_next, c_logits = cpu.forward(int(t), pos)
+    g_next, g_logits = gpu.forward_tokens(prompt)
+    assert g_next == c_next and max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL
+    tok = c_next
+    for pos in range(50, 56):  # one-token steps on top of the cache the rows left
+        c_next, c_logits = cpu.forward(tok, pos)
+        g_next, g_logits = gpu.forward(tok)
+        assert g_next == c_next and max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, pos
+        tok = c_next
+    gpu.reset()
+    g_next, g_logits = gpu.forward_tokens(prompt[:9])  # eight rows through the small-batch GEMV
+    for pos, t in enumerate(prompt[:9]):
+        c_next, c_logits = cpu.forward(int(t), pos)
+    assert g_next == c_next and max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL
+    gpu.set_batch(8)
+    prompts = [rng.integers(0, c["vocab_size"], size=n) for n in (3, 40, 1, 12, 9, 2, 35, 5)]
+    got, _, _ = gpu.generate_batch(prompts, 5)
+    for s, p in enumerate(prompts):
+        want, _ = _oracle_walk(cpu, p, 5)
+        assert got[s].tolist() == want, s
+    gpu.close()
+    cpu.close()
