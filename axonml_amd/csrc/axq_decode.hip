@@ -875,14 +875,21 @@ int enqueue_rows(axq_model *m, const Rows &r) {
     hipStream_t st = ctx->stream;
     const int H = c.hidden_size, I = c.intermediate_size, d = c.head_dim, nb = r.nb;
     int rc;
-    // y = f(x) W^T (+ resid): f = RMSNorm when norm_w is given
-    auto lin = [&](const axq_weight *w, const float *x, const float *norm_w, const float *resid, float *y) -> int {
-        if (r.mode == ROWS_GEMM) return axq_dev_gemm_f32(ctx, w, x, nb, norm_w, c.rms_norm_eps, nullptr, resid, y);
-        if (norm_w) {
-            norm_kernel<<<nb, 1024, 0, st>>>(x, norm_w, (int)w->k, c.rms_norm_eps, m->pb_xn);
+    // y = f(x) W^T (+ resid): f = RMSNorm with weights aux, or SwiGLU over the gate/up rows in x, or nothing.  The
+    // small-batch GEMV applies f while it packs x; elsewhere f runs as a kernel of its own (the GEMM normalises itself).
+    auto lin = [&](const axq_weight *w, const float *x, int xmode, const float *aux, const float *resid, float *y) -> int {
+        const bool batch_kernel = r.mode == ROWS_GEMV && axq_dev_gemv_batch_covers(w, nb);
+        if (batch_kernel) return axq_dev_gemv_batch_ex(ctx, w, x, xmode, aux, c.rms_norm_eps, nb, nullptr, resid, y);
+        if (xmode == AXQ_X_SWIGLU) {
+            swiglu_kernel<<<dim3((I / 4 + 255) / 256, nb), 256, 0, st>>>(x, I, m->pb_act);
+            x = m->pb_act;
+        }
+        if (r.mode == ROWS_GEMM)
+            return axq_dev_gemm_f32(ctx, w, x, nb, xmode == AXQ_X_RMSNORM ? aux : nullptr, c.rms_norm_eps, nullptr, resid, y);
+        if (xmode == AXQ_X_RMSNORM) {
+            norm_kernel<<<nb, 1024, 0, st>>>(x, aux, (int)w->k, c.rms_norm_eps, m->pb_xn);
             x = m->pb_xn;
         }
-        if (axq_dev_gemv_batch_covers(w, nb)) return axq_dev_gemv_batch(ctx, w, x, nb, nullptr, resid, y);
         for (int b = 0; b < nb; b++) { // row by row, the residual row in the bias slot
             int e = axq_dev_gemv(ctx, w, x + (size_t)b * w->k, 1, resid ? resid + (size_t)b * w->n_rows : nullptr, y + (size_t)b * w->n_rows);
             if (e) return e;
@@ -899,7 +906,7 @@ int enqueue_rows(axq_model *m, const Rows &r) {
     embed_kernel<<<dim3((H / 8 + 255) / 256, nb), 256, 0, st>>>(m->emb, r.toks, m->pb_h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
         const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * d + seq_off;
-        if ((rc = lin(m->w_qkv[l], m->pb_h, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv))) return rc;
+        if ((rc = lin(m->w_qkv[l], m->pb_h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv))) return rc;
         rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
             m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0,
             r.per_seq ? m->pos : nullptr, m->seq_stride, c.max_position_embeddings, d);
@@ -909,10 +916,9 @@ int enqueue_rows(axq_model *m, const Rows &r) {
         case 128: launch_attn_prompt_d<128>(m, l, r, st); break;
         default: launch_attn_prompt_d<256>(m, l, r, st); break;
         }
-        if ((rc = lin(m->w_o[l], m->pb_att, nullptr, m->pb_h, m->pb_h))) return rc;
-        if ((rc = lin(m->w_gu[l], m->pb_h, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu))) return rc;
-        swiglu_kernel<<<dim3((I / 4 + 255) / 256, nb), 256, 0, st>>>(m->pb_gu, I, m->pb_act);
-        if ((rc = lin(m->w_down[l], m->pb_act, nullptr, m->pb_h, m->pb_h))) return rc;
+        if ((rc = lin(m->w_o[l], m->pb_att, AXQ_X_PLAIN, nullptr, m->pb_h, m->pb_h))) return rc;
+        if ((rc = lin(m->w_gu[l], m->pb_h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu))) return rc;
+        if ((rc = lin(m->w_down[l], m->pb_gu, AXQ_X_SWIGLU, nullptr, m->pb_h, m->pb_h))) return rc;
     }
     if (r.per_seq) {
         norm_kernel<<<nb, 1024, 0, st>>>(m->pb_h, m->norm_final, H, c.rms_norm_eps, m->pb_xn);

@@ -278,18 +278,57 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
     }
 }
 
-// x[batch, k] -> A operands and group records.  Thread = (8-element task, vector b); vectors beyond the batch
+// f(x)[batch, k] -> A operands and group records.  Thread = (8-element task, vector b); vectors beyond the batch
 // are written as zeros.  EVEN_ODD: the h = 0 half of a block's operand holds its even elements, h = 1 the odd.
-template <bool EVEN_ODD>
-__global__ void __launch_bounds__(256) pack_x_kernel(const float *x, int k, int batch, uint8_t *xa, float *xsg) {
+// XMODE: AXQ_X_PLAIN; AXQ_X_RMSNORM: f = x / sqrt(mean(x^2) + eps) * aux (every workgroup sums its vector's squares
+// itself); AXQ_X_SWIGLU: x holds [batch, 2k] gate/up values, four gate values followed by the four up values of the
+// same indices, and f = silu(gate) * up.
+template <bool EVEN_ODD, int XMODE>
+__global__ void __launch_bounds__(256) pack_x_kernel(const float *x, const float *aux, float eps, int k, int batch, uint8_t *xa,
+                                                     float *xsg) {
+    __shared__ float red[4];
     const int t = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
     const int ntask = k >> 3, nblk = k >> 5;
-    if (t >= ntask) return; // k is a multiple of 512: whole quads of tasks
+    float inv = 1.0f;
+    if (XMODE == AXQ_X_RMSNORM && b < batch) { // before any thread leaves: the sum needs the whole workgroup
+        const float4 *row = reinterpret_cast<const float4 *>(x + (size_t)b * k);
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < (k >> 2); i += 256) {
+            const float4 v = row[i];
+            ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        ss = (red[0] + red[1]) + (red[2] + red[3]);
+        inv = 1.0f / sqrtf(ss / (float)k + eps);
+    }
+    if (t >= ntask) return; // k is a multiple of 256: whole quads of tasks
     float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (b < batch) {
-        const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)b * k + (size_t)t * 8);
-        const float4 v0 = p[0], v1 = p[1];
-        v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w; v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
+        if (XMODE == AXQ_X_SWIGLU) {
+            const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)b * 2 * k + (size_t)t * 16);
+#pragma unroll
+            for (int g = 0; g < 2; g++) {
+                const float4 gt = p[2 * g], up = p[2 * g + 1];
+                v[4 * g + 0] = (gt.x * (1.0f / (1.0f + expf(-gt.x)))) * up.x;
+                v[4 * g + 1] = (gt.y * (1.0f / (1.0f + expf(-gt.y)))) * up.y;
+                v[4 * g + 2] = (gt.z * (1.0f / (1.0f + expf(-gt.z)))) * up.z;
+                v[4 * g + 3] = (gt.w * (1.0f / (1.0f + expf(-gt.w)))) * up.w;
+            }
+        } else {
+            const float4 *p = reinterpret_cast<const float4 *>(x + (size_t)b * k + (size_t)t * 8);
+            const float4 v0 = p[0], v1 = p[1];
+            v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w; v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
+            if (XMODE == AXQ_X_RMSNORM) {
+                const float4 *pw = reinterpret_cast<const float4 *>(aux + (size_t)t * 8);
+                const float4 w0 = pw[0], w1 = pw[1];
+                const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = (v[i] * inv) * wv[i];
+            }
+        }
     }
     uint32_t pk[4][2];
     float sg, sum;
@@ -330,10 +369,13 @@ __global__ void __launch_bounds__(256) mb_reduce_kernel(const float *ypart, cons
 }
 
 template <class T>
-void launch_mb(axq_ctx *ctx, MbArgs a, const float *x) {
+void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *aux, float eps) {
     const dim3 pgrid((unsigned)((a.k / 8 + 255) / 256), MAX_BATCH);
-    pack_x_kernel<T::EVEN_ODD><<<pgrid, 256, 0, ctx->stream>>>(x, a.k, a.batch, const_cast<uint8_t *>(a.xa),
-                                                               const_cast<float *>(a.xsg));
+    uint8_t *xa = const_cast<uint8_t *>(a.xa);
+    float *xsg = const_cast<float *>(a.xsg);
+    if (xmode == AXQ_X_RMSNORM) pack_x_kernel<T::EVEN_ODD, AXQ_X_RMSNORM><<<pgrid, 256, 0, ctx->stream>>>(x, aux, eps, a.k, a.batch, xa, xsg);
+    else if (xmode == AXQ_X_SWIGLU) pack_x_kernel<T::EVEN_ODD, AXQ_X_SWIGLU><<<pgrid, 256, 0, ctx->stream>>>(x, aux, eps, a.k, a.batch, xa, xsg);
+    else pack_x_kernel<T::EVEN_ODD, AXQ_X_PLAIN><<<pgrid, 256, 0, ctx->stream>>>(x, aux, eps, a.k, a.batch, xa, xsg);
     const unsigned chunks = (unsigned)((a.k + WAVE_K - 1) / WAVE_K);
     const unsigned tiles = (unsigned)((a.n_rows + 31) / 32);
     // few row tiles (a narrow output): split K over up to four workgroups per tile so that the chip is full
@@ -367,9 +409,14 @@ bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch) {
     return w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q8_0 || w->type == AXQ_Q4_K;
 }
 
-// y[batch, n_rows] = x[batch, k] W^T (+ bias per row of W) (+ resid[batch, n_rows], which may be y) for
-// 2 <= batch <= 8: split the batch, then one pass over W.
 int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, const float *resid, float *y) {
+    return axq_dev_gemv_batch_ex(ctx, w, x, AXQ_X_PLAIN, nullptr, 0.f, batch, bias, resid, y);
+}
+
+// y[batch, n_rows] = f(x)[batch, k] W^T (+ bias per row of W) (+ resid[batch, n_rows], which may be y) for
+// 2 <= batch <= 8: split the batch (f = xmode, see pack_x_kernel), then one pass over W.
+int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
+                          const float *bias, const float *resid, float *y) {
     const int k = (int)w->k;
     // scratch (the context's x buffer): 32 k bytes of A operands, then 2 * (k / 32) * 8 floats of scales and sums
     uint8_t *xa = ctx->xq;
@@ -383,10 +430,10 @@ int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int ba
     a.ypart = w->n_rows <= AXQ_BATCH_SPLIT_ROWS ? reinterpret_cast<float *>(ctx->xq + (size_t)34 * AXQ_BATCH_MAX_K) : nullptr;
     a.n_rows = (int)w->n_rows; a.k = k; a.batch = batch;
     switch (w->type) {
-    case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, x); break;
-    case AXQ_Q4_1: launch_mb<MQ4x<true>>(ctx, a, x); break;
-    case AXQ_Q8_0: launch_mb<MQ80>(ctx, a, x); break;
-    case AXQ_Q4_K: launch_mb<MQ4K>(ctx, a, x); break;
+    case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, x, xmode, aux, eps); break;
+    case AXQ_Q4_1: launch_mb<MQ4x<true>>(ctx, a, x, xmode, aux, eps); break;
+    case AXQ_Q8_0: launch_mb<MQ80>(ctx, a, x, xmode, aux, eps); break;
+    case AXQ_Q4_K: launch_mb<MQ4K>(ctx, a, x, xmode, aux, eps); break;
     default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
     }
     AXQ_LAUNCH_CHECK(ctx, "gemv_mb_kernel");

@@ -102,7 +102,8 @@ int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x_dev, int batc
 int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, const float *bias, float *y);
 // What the GEMV does to x before it uses it (xq must be NULL for the fused forms):
 enum { AXQ_X_PLAIN = 0,    // nothing
-       AXQ_X_RMSNORM = 1 }; // x <- x / sqrt(mean(x^2) + eps) * aux   (aux = norm weights, K floats)
+       AXQ_X_RMSNORM = 1,  // x <- x / sqrt(mean(x^2) + eps) * aux   (aux = norm weights, K floats)
+       AXQ_X_SWIGLU = 2 }; // small-batch GEMV only: x holds 2K gate/up values (groups of four and four), x <- silu(gate) * up
 // ... and to its result before it writes it:
 enum { AXQ_Y_PLAIN = 0,    // y[row] = dot (+ bias[row])
        AXQ_Y_SWIGLU = 1 }; // rows come in groups of four "gate" rows followed by their four "up" rows:
@@ -115,6 +116,8 @@ int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq);
 // gemv_batch.hip: batches of 2..8 vectors against one pass over the weights
 bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch);
 int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, const float *resid, float *y);
+int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
+                          const float *bias, const float *resid, float *y);
 // sample.hip: every pointer a device pointer; scratch = axq_sample_scratch_bytes(vocab)
 size_t axq_sample_scratch_bytes(int vocab);
 int axq_check_sampling_config(axq_ctx *ctx, const axq_sampling_config *cfg);
