@@ -1005,11 +1005,10 @@ int run_batch_step(axq_model *m) {
         rc = AXQ_OK;
     }
     if (rc || !m->sampling) return rc;
-    const int V = m->cfg.vocab_size, P = m->cfg.max_position_embeddings;
-    for (int s = 0; s < m->n_seq && !rc; s++) // the draw of sequence s comes from (seed + s * odd constant, position)
-        rc = axq_dev_sample(ctx, m->logits + (size_t)s * V, V, m->hist + (size_t)s * P, m->pos + s, 0, &m->sampler, 0.f, m->pos + s,
-                            m->sample_seed + 0x9E3779B97F4A7C15ull * (uint64_t)s, m->sample_scratch, m->next + s, nullptr);
-    return rc;
+    // one workgroup per sequence; the draw of sequence s comes from (seed + s * odd constant, position)
+    return axq_dev_sample_rows(ctx, m->n_seq, m->logits, (size_t)m->cfg.vocab_size, m->cfg.vocab_size, m->hist,
+                               (size_t)m->cfg.max_position_embeddings, m->pos, 0, &m->sampler, 0.f, m->pos, m->sample_seed,
+                               0x9E3779B97F4A7C15ull, m->sample_scratch, m->next, nullptr);
 }
 
 template <class T>
@@ -1304,6 +1303,11 @@ int axq_model_set_batch(axq_model *m, int n_seq) {
     m->n_seq = n_seq;
     m->host_pos = 0;
     m->seq_pos.assign(n_seq, 0);
+    if (m->sample_scratch) { // the sampler's scratch goes by sequences too
+        (void)hipFree(m->sample_scratch);
+        m->sample_scratch = nullptr;
+        AXQ_HIP(ctx, hipMalloc(&m->sample_scratch, (size_t)n_seq * axq_sample_scratch_bytes(c.vocab_size)), AXQ_ERR_ALLOCATION_FAILED);
+    }
     return AXQ_OK;
 }
 
@@ -1446,7 +1450,8 @@ int axq_model_set_sampling(axq_model *m, const axq_sampling_config *cfg, uint64_
     }
     int rc;
     if ((rc = axq_check_sampling_config(ctx, cfg))) return rc;
-    if (!m->sample_scratch) AXQ_HIP(ctx, hipMalloc(&m->sample_scratch, axq_sample_scratch_bytes(m->cfg.vocab_size)), AXQ_ERR_ALLOCATION_FAILED);
+    if (!m->sample_scratch) // a row of scratch per sequence
+        AXQ_HIP(ctx, hipMalloc(&m->sample_scratch, (size_t)m->n_seq * axq_sample_scratch_bytes(m->cfg.vocab_size)), AXQ_ERR_ALLOCATION_FAILED);
     m->sampler = *cfg;
     m->sample_seed = seed;
     m->sampling = true;

@@ -124,6 +124,10 @@ int axq_check_sampling_config(axq_ctx *ctx, const axq_sampling_config *cfg);
 int axq_dev_sample(axq_ctx *ctx, const float *logits, int vocab, const int32_t *hist, const int32_t *hist_len_dev, int hist_len,
                    const axq_sampling_config *cfg, float u, const int32_t *counter_dev, uint64_t seed, void *scratch,
                    int32_t *out, float *filtered_out);
+int axq_dev_sample_rows(axq_ctx *ctx, int rows, const float *logits, size_t logits_stride, int vocab, const int32_t *hist,
+                        size_t hist_stride, const int32_t *hist_len_dev, int hist_len, const axq_sampling_config *cfg, float u,
+                        const int32_t *counter_dev, uint64_t seed, uint64_t seed_stride, void *scratch, int32_t *out,
+                        float *filtered_out);
 // gemm.hip
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_dev, int m, float *y_dev);
 #define AXQ_GEMM_F32_MAX_ROWS 2048 // rows per call of the f32-activation GEMM (its scratch grows with them)

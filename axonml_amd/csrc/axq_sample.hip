@@ -34,6 +34,10 @@ struct SampleArgs {
     u64 seed;
     int32_t *out;
     float *filtered_out;        // optional: the logits after all filters
+    // one workgroup per row: row r reads logits + r * logits_stride, hist + r * hist_stride, hist_len_dev[r],
+    // counter_dev[r], works in work + r * work_stride, draws with seed + r * seed_stride and writes out[r]
+    size_t logits_stride, hist_stride, work_stride;
+    u64 seed_stride;
 };
 
 constexpr int FAST_K = 128;   // top-k up to here takes the short path below ...
@@ -196,6 +200,17 @@ __global__ void __launch_bounds__(ST) sample_kernel(SampleArgs a) {
     __shared__ Shared sh;
     extern __shared__ float lds_w[];
     const int tid = threadIdx.x, n = a.vocab;
+    if (blockIdx.x) {
+        const size_t r = blockIdx.x;
+        a.logits += r * a.logits_stride;
+        a.work += r * a.work_stride;
+        if (a.hist) a.hist += r * a.hist_stride;
+        if (a.hist_len_dev) a.hist_len_dev += r;
+        if (a.counter_dev) a.counter_dev += r;
+        a.seed += r * a.seed_stride;
+        a.out += r;
+        if (a.filtered_out) a.filtered_out += r * (size_t)n;
+    }
     constexpr bool in_lds = IN_LDS;
     float *const w = IN_LDS ? lds_w : a.work; // the working copy of the logits (address space known at compile time)
 #pragma unroll 8
@@ -423,6 +438,17 @@ struct Temp {
 int axq_dev_sample(axq_ctx *ctx, const float *logits, int vocab, const int32_t *hist, const int32_t *hist_len_dev, int hist_len,
                    const axq_sampling_config *cfg, float u, const int32_t *counter_dev, uint64_t seed, void *scratch,
                    int32_t *out, float *filtered_out) {
+    return axq_dev_sample_rows(ctx, 1, logits, 0, vocab, hist, 0, hist_len_dev, hist_len, cfg, u, counter_dev, seed, 0, scratch, out,
+                               filtered_out);
+}
+
+// `rows` independent draws in one launch, one workgroup each: row r takes logits + r * logits_stride,
+// hist + r * hist_stride, hist_len_dev[r], counter_dev[r], the seed seed + r * seed_stride and
+// axq_sample_scratch_bytes(vocab) bytes of scratch of its own, and writes out[r].
+int axq_dev_sample_rows(axq_ctx *ctx, int rows, const float *logits, size_t logits_stride, int vocab, const int32_t *hist,
+                        size_t hist_stride, const int32_t *hist_len_dev, int hist_len, const axq_sampling_config *cfg, float u,
+                        const int32_t *counter_dev, uint64_t seed, uint64_t seed_stride, void *scratch, int32_t *out,
+                        float *filtered_out) {
     SampleArgs a;
     a.logits = logits;
     a.work = reinterpret_cast<float *>(scratch);
@@ -433,14 +459,15 @@ int axq_dev_sample(axq_ctx *ctx, const float *logits, int vocab, const int32_t *
     a.top_k = cfg->top_k; a.do_sample = cfg->do_sample;
     a.u = u; a.counter_dev = counter_dev; a.seed = seed;
     a.out = out; a.filtered_out = filtered_out;
+    a.logits_stride = logits_stride; a.hist_stride = hist_stride; a.work_stride = 2 * padded_words(vocab); a.seed_stride = seed_stride;
     static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once
     if (!big_lds_allowed) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&sample_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)(padded_words(LDS_VOCAB) * 4));
         big_lds_allowed = true;
     }
-    if (vocab <= LDS_VOCAB) sample_kernel<true><<<1, ST, padded_words(vocab) * 4, ctx->stream>>>(a);
-    else sample_kernel<false><<<1, ST, 0, ctx->stream>>>(a);
+    if (vocab <= LDS_VOCAB) sample_kernel<true><<<rows, ST, padded_words(vocab) * 4, ctx->stream>>>(a);
+    else sample_kernel<false><<<rows, ST, 0, ctx->stream>>>(a);
     AXQ_LAUNCH_CHECK(ctx, "sample_kernel");
     return AXQ_OK;
 }

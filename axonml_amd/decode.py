@@ -238,5 +238,10 @@ def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
         res[f"batch{n_seq}_prefill_tokens_per_s"] = n_seq * (prompt_len - 1) / (pre_b * 1e-3)
         log(f"  {n_seq} sequences: {res[f'batch{n_seq}_tokens_per_s']:.0f} tok/s in all ({res[f'batch{n_seq}_ms_per_step']:.3f} ms per step), "
             f"prompts {res[f'batch{n_seq}_prefill_tokens_per_s']:.0f} tok/s")
+    m.set_sampling(GenerationConfig(temperature=0.8, top_k=40, top_p=0.9, repetition_penalty=1.1), seed=7)
+    m.generate_batch(prompts, 4)
+    _, _, dec_bs = m.generate_batch(prompts, new_tokens)
+    res["batch8_sampled_tokens_per_s"] = 8 * new_tokens / (dec_bs * 1e-3)
+    log(f"  8 sequences with top-k/top-p sampling: {res['batch8_sampled_tokens_per_s']:.0f} tok/s in all")
     m.close()
     return res
