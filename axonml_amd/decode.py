@@ -194,7 +194,8 @@ def smoke(ctx):
 
 
 def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
-    """BASELINE config 4: Mistral-7B shape, random init, all linears Q4_K, f16 KV cache, greedy."""
+    """Decode benchmark: Mistral-7B shape, random init, all linears Q4_K, f16 KV cache; greedy, sampled, and several
+    sequences side by side."""
     cfg = mistral_7b_config(prompt_len + new_tokens)
     m = QuantizedLlama(ctx, **cfg)
     m.random_init(QuantType.Q4_K, 0.02, 1)

@@ -1,4 +1,4 @@
-"""Prefill-path benchmark helper: quantized GEMM with bf16 activations (BASELINE config 5)."""
+"""Prefill-path benchmark helper: quantized GEMM with bf16 and f32 activations at the 7B model's projection shapes."""
 import ctypes as C
 
 import numpy as np

@@ -203,7 +203,7 @@ def test_many_vectors_non_finite_row(ctx):
 
 @pytest.mark.parametrize("n,k", [(11008, 4096), (4096, 11008)])
 def test_small_batch_config_shape(ctx, n, k):
-    # BASELINE config 2: 11008 x 4096 and the transposed down-projection shape, batch 8, Q4_0 and Q4_1
+    # the 7B LLaMA feed-forward shapes: 11008 x 4096 and the transposed down-projection, batch 8, Q4_0 and Q4_1
     rng = np.random.default_rng(82)
     batch = 8
     w = gen_weight(rng, n, k)
