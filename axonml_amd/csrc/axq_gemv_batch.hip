@@ -14,6 +14,8 @@
 // for its 32 rows).
 #include <hip/hip_fp16.h>
 
+#include <stdlib.h>
+
 #include "axq_internal.h"
 #include "axq_split.h"
 
@@ -386,7 +388,8 @@ void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *a
     a.chunks_per_split = (int)((chunks + splits - 1) / splits);
     splits = (chunks + a.chunks_per_split - 1) / a.chunks_per_split;
     if (splits < 2) a.ypart = nullptr;
-    const unsigned S = (unsigned)a.chunks_per_split < 8 ? (unsigned)a.chunks_per_split : 8;
+    static const unsigned smax = getenv("AXQ_BATCH_WAVES") ? (unsigned)atoi(getenv("AXQ_BATCH_WAVES")) : 8; // development knob (1..8)
+    const unsigned S = (unsigned)a.chunks_per_split < smax ? (unsigned)a.chunks_per_split : smax;
     const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float) + (size_t)S * 32 * T::NP * 16;
     static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
     if (lds > 64 * 1024 && !big_lds_allowed) {

@@ -67,7 +67,7 @@ def test_kv_cache_matches_oracle_up_to_isolated_f16_roundings(ctx):
 
 
 def test_generate_matches_oracle_greedy_and_is_repeatable(ctx):
-    c = tiny_config(num_layers=3, max_seq_len=96)
+    c = tiny_config(num_layers=3, max_seq_len=160)
     w = random_weights(c, 20)
     cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
     rng = np.random.default_rng(0)
@@ -75,15 +75,15 @@ def test_generate_matches_oracle_greedy_and_is_repeatable(ctx):
     want, tok = [], None
     for pos, t in enumerate(prompt):
         tok, _ = cpu.forward(int(t), pos)
-    for i in range(40):
+    for i in range(128):
         want.append(tok)
-        if i + 1 < 40:
+        if i + 1 < 128:
             tok, _ = cpu.forward(tok, len(prompt) + i)
-    got, pre_ms, dec_ms = gpu.generate(prompt, 40)
+    got, pre_ms, dec_ms = gpu.generate(prompt, 128)
     assert got.tolist() == want
-    assert gpu.seq_len() == len(prompt) + 39 and pre_ms > 0 and dec_ms > 0
+    assert gpu.seq_len() == len(prompt) + 127 and pre_ms > 0 and dec_ms > 0
     gpu.reset()
-    again, _, _ = gpu.generate(prompt, 40)
+    again, _, _ = gpu.generate(prompt, 128)
     assert again.tolist() == want  # graph replays are deterministic and the reset clears the position
     gpu.close()
 
