@@ -59,8 +59,11 @@ struct axq_model {
     uint64_t sample_seed;
     int prompt_cap, out_cap;
     int host_pos;
-    hipGraphExec_t graph;
+    hipGraphExec_t graph;           // the one-token step with the attention split over the positions
     bool graph_ok;
+    hipGraphExec_t graph_f;         // the same with one attention workgroup per head (short contexts)
+    bool graph_f_ok;
+    int fused_max;                  // contexts up to this many positions take graph_f
 };
 
 namespace {
@@ -396,18 +399,20 @@ __global__ void __launch_bounds__(128) rope_append_kernel(const float *qkv, int 
 }
 
 // attn_prompt_kernel, grid (heads, tokens), 1024 threads: the query of head `head` at position p = pos0 + b
-// against the cached keys lo..p (causal, llama.rs:420-447; lo > 0 under a sliding window), all read from the
-// cache: scores into LDS, their maximum, exponentials and sum, then sum_j e_j v_j / sum.  Keys and values
-// are read 16 bytes per lane, head_dim / 8 lanes per position.
-template <int D>
+// against the cached keys lo..p (causal, llama.rs:420-447; lo > 0 under a sliding window): scores into LDS, their
+// maximum, exponentials and sum, then sum_j e_j v_j / sum.  Keys and values are read 16 bytes per lane,
+// head_dim / 8 lanes per position.  APPEND (rows of different sequences only, pos_arr given): the row's own key and
+// value are not in the cache yet; every workgroup rotates the key itself, uses both from LDS (rounded to f16 as the
+// cache holds them), and the first query head of each KV head writes them to the cache.
+template <int D, bool APPEND>
 __global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int qkv_rows, const float *rope_cos,
-                                                           const float *rope_sin, const uint16_t *kcache,
-                                                           const uint16_t *vcache, int pos0, const int32_t *pos_arr,
-                                                           size_t seq_stride, int n_heads, int n_kv, int max_pos, int window,
-                                                           float *att) {
+                                                           const float *rope_sin, uint16_t *kcache, uint16_t *vcache, int pos0,
+                                                           const int32_t *pos_arr, size_t seq_stride, int n_heads, int n_kv,
+                                                           int max_pos, int window, float *att) {
     constexpr int HALF = D / 2, LP = D / 8, PPB = 1024 / LP; // lanes per position, positions per pass of the workgroup
     extern __shared__ float sc[];                            // scores, then exp(score - max)
     __shared__ __attribute__((aligned(16))) float qs[D];
+    __shared__ __attribute__((aligned(16))) float knew[APPEND ? D : 4], vnew[APPEND ? D : 4];
     __shared__ float red[16];
     __shared__ __attribute__((aligned(16))) float osum[16 * D];
     const int head = blockIdx.x, b = blockIdx.y;
@@ -425,6 +430,21 @@ __global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int
         const float q1 = qh[tid], q2 = qh[tid + HALF];
         qs[tid] = q1 * c - q2 * s;
         qs[tid + HALF] = q1 * s + q2 * c;
+    } else if (APPEND && tid >= 512 && tid < 512 + HALF) { // other waves: the new key and value (arithmetic of rope_append_kernel)
+        const int e = tid - 512, q_dim = n_heads * D, kv_dim = n_kv * D;
+        const float *row = qkv + (size_t)b * qkv_rows;
+        const float *kh = row + q_dim + (size_t)kvh * D, *vh = row + q_dim + kv_dim + (size_t)kvh * D;
+        const float nc = rope_cos[(size_t)p * HALF + e], ns = rope_sin[(size_t)p * HALF + e];
+        const float k1 = kh[e], k2 = kh[e + HALF];
+        const __half ka = __float2half_rn(k1 * nc - k2 * ns), kb = __float2half_rn(k1 * ns + k2 * nc);
+        const __half va = __float2half_rn(vh[e]), vb = __float2half_rn(vh[e + HALF]);
+        knew[e] = __half2float(ka); knew[e + HALF] = __half2float(kb);
+        vnew[e] = __half2float(va); vnew[e + HALF] = __half2float(vb);
+        if (head == kvh * rep) {
+            uint16_t *kw = kcache + ((size_t)kvh * max_pos + p) * D, *vw = vcache + ((size_t)kvh * max_pos + p) * D;
+            kw[e] = __half_as_ushort(ka); kw[e + HALF] = __half_as_ushort(kb);
+            vw[e] = __half_as_ushort(va); vw[e + HALF] = __half_as_ushort(vb);
+        }
     }
     __syncthreads();
     const int c8 = tid % LP, r = tid / LP;
@@ -435,19 +455,23 @@ __global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int
         qf[0] = qa.x; qf[1] = qa.y; qf[2] = qa.z; qf[3] = qa.w; qf[4] = qb.x; qf[5] = qb.y; qf[6] = qb.z; qf[7] = qb.w;
     }
     const float scale = 1.0f / sqrtf((float)D);
-    constexpr int UN = 4;
+    constexpr int UN = 4; // 16-byte loads in flight per lane (8 was slower at every context, 16 spills)
     for (int j0 = 0; j0 < span; j0 += UN * PPB) {
         uint4 raw[UN];
 #pragma unroll
         for (int u = 0; u < UN; u++) {
             const int j = j0 + u * PPB + r;
-            raw[u] = *reinterpret_cast<const uint4 *>(kc + (size_t)(j < span ? j : 0) * D + c8 * 8);
+            raw[u] = *reinterpret_cast<const uint4 *>(kc + (size_t)(j < span - (APPEND ? 1 : 0) ? j : 0) * D + c8 * 8);
         }
 #pragma unroll
         for (int u = 0; u < UN; u++) {
             const int j = j0 + u * PPB + r;
             float kf[8];
             halves_to_floats(raw[u], kf);
+            if (APPEND && j == span - 1) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) kf[e] = knew[c8 * 8 + e];
+            }
             float s = qf[0] * kf[0];
 #pragma unroll
             for (int e = 1; e < 8; e++) s = fmaf(qf[e], kf[e], s);
@@ -478,7 +502,7 @@ __global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int
 #pragma unroll
         for (int u = 0; u < UN; u++) {
             const int j = j0 + u * PPB + r;
-            raw[u] = *reinterpret_cast<const uint4 *>(vc + (size_t)(j < span ? j : 0) * D + c8 * 8);
+            raw[u] = *reinterpret_cast<const uint4 *>(vc + (size_t)(j < span - (APPEND ? 1 : 0) ? j : 0) * D + c8 * 8);
         }
 #pragma unroll
         for (int u = 0; u < UN; u++) {
@@ -486,6 +510,10 @@ __global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int
             const float e = j < span ? sc[j] : 0.f;
             float vf[8];
             halves_to_floats(raw[u], vf);
+            if (APPEND && j == span - 1) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) vf[i] = vnew[c8 * 8 + i];
+            }
 #pragma unroll
             for (int i = 0; i < 8; i++) acc[i] = fmaf(e, vf[i], acc[i]);
         }
@@ -705,7 +733,13 @@ int linear(axq_model *m, const axq_weight *w, const float *x, int xmode, const f
 
 // The kernels of one token, enqueued on the context's stream: six per layer when every linear is covered
 // by the matrix-pipe GEMV (norms and SwiGLU ride in the GEMVs, residual adds in their bias slot).
-int enqueue_step(axq_model *m) {
+void launch_attn_rows(axq_model *m, int l, const float *qkv, int nb, int pos0, const int32_t *pos_arr, size_t cache_off, size_t lds,
+                      float *att, hipStream_t st);
+size_t prompt_attn_lds(const axq_model *m, int last);
+
+// short: the context is at most m->fused_max positions: one attention workgroup per head does everything (the new key
+// and value included); otherwise the positions are split over workgroups and a second kernel merges them.
+int enqueue_step(axq_model *m, bool short_ctx) {
     axq_ctx *ctx = m->ctx;
     const axq_model_config &c = m->cfg;
     hipStream_t st = ctx->stream;
@@ -716,9 +750,13 @@ int enqueue_step(axq_model *m) {
     for (int l = 0; l < c.num_hidden_layers; l++) {
         if ((rc = linear(m, m->w_qkv[l], m->h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, AXQ_Y_PLAIN, m->xn, nullptr, m->qkv)))
             return rc;
-        launch_attn_partial(m, l, st);
-        attn_combine_kernel<<<c.num_attention_heads, 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
-                                                                          c.num_key_value_heads, d, m->max_splits, c.sliding_window, m->att);
+        if (short_ctx) {
+            launch_attn_rows(m, l, m->qkv, 1, 0, m->pos, 0, prompt_attn_lds(m, m->fused_max), m->att, st);
+        } else {
+            launch_attn_partial(m, l, st);
+            attn_combine_kernel<<<c.num_attention_heads, 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
+                                                                              c.num_key_value_heads, d, m->max_splits, c.sliding_window, m->att);
+        }
         // residual adds go through the bias slot, in place
         if ((rc = linear(m, m->w_o[l], m->att, AXQ_X_PLAIN, nullptr, AXQ_Y_PLAIN, nullptr, m->h, m->h))) return rc;
         if ((rc = linear(m, m->w_gu[l], m->h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, AXQ_Y_SWIGLU, m->xn, nullptr, m->act)))
@@ -740,36 +778,39 @@ int check_ready(axq_model *m) {
     return AXQ_OK;
 }
 
-// Captures the step into a graph on first use; later calls replay it.
-int run_step_graph(axq_model *m) {
+// Captures the step into a graph on first use; later calls replay it.  pos: the position of the token being fed.
+int run_step_graph(axq_model *m, int pos) {
     axq_ctx *ctx = m->ctx;
+    const bool short_ctx = pos < m->fused_max;
     static const bool no_graph = getenv("AXQ_DECODE_GRAPH") && getenv("AXQ_DECODE_GRAPH")[0] == '0';
-    if (no_graph) return enqueue_step(m); // development knob: plain launches instead of a graph replay
-    if (!m->graph_ok) {
+    if (no_graph) return enqueue_step(m, short_ctx); // development knob: plain launches instead of a graph replay
+    hipGraphExec_t &exec = short_ctx ? m->graph_f : m->graph;
+    bool &ok = short_ctx ? m->graph_f_ok : m->graph_ok;
+    if (!ok) {
         hipGraph_t g = nullptr;
         AXQ_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), AXQ_ERR_DRIVER);
-        int rc = enqueue_step(m);
+        int rc = enqueue_step(m, short_ctx);
         hipError_t e = hipStreamEndCapture(ctx->stream, &g);
         if (rc) {
             if (g) (void)hipGraphDestroy(g);
             return rc;
         }
         if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipStreamEndCapture: %s", hipGetErrorString(e));
-        e = hipGraphInstantiate(&m->graph, g, nullptr, nullptr, 0);
+        e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
         (void)hipGraphDestroy(g);
         if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipGraphInstantiate: %s", hipGetErrorString(e));
-        m->graph_ok = true;
+        ok = true;
     }
-    AXQ_HIP(ctx, hipGraphLaunch(m->graph, ctx->stream), AXQ_ERR_KERNEL_LAUNCH_FAILED);
+    AXQ_HIP(ctx, hipGraphLaunch(exec, ctx->stream), AXQ_ERR_KERNEL_LAUNCH_FAILED);
     return AXQ_OK;
 }
 
 // One token: note it in the history, run the step, and when a sampler is set let it replace the step's argmax.
 // The uniform variate of a draw comes from (seed, position), so a run is repeatable.
-int run_token(axq_model *m) {
+int run_token(axq_model *m, int pos) {
     axq_ctx *ctx = m->ctx;
     record_token_kernel<<<1, 1, 0, ctx->stream>>>(m->hist, m->pos, m->tok);
-    int rc = run_step_graph(m);
+    int rc = run_step_graph(m, pos);
     if (rc || !m->sampling) return rc;
     return axq_dev_sample(ctx, m->logits, m->cfg.vocab_size, m->hist, m->pos, 0, &m->sampler, 0.f, m->pos, m->sample_seed,
                           m->sample_scratch, m->next, nullptr);
@@ -849,19 +890,38 @@ struct Rows {
     size_t lds;          // of the attention kernel
 };
 
-template <int D>
-void launch_attn_prompt_d(axq_model *m, int l, const Rows &r, hipStream_t st) {
+template <int D, bool APPEND>
+void launch_attn_rows_t(axq_model *m, int l, const float *qkv, int nb, int pos0, const int32_t *pos_arr, size_t cache_off, size_t lds,
+                        float *att, hipStream_t st) {
     const axq_model_config &c = m->cfg;
-    const size_t per_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * D;
-    const size_t off = l * per_layer + (r.per_seq ? 0 : (size_t)r.seq * m->seq_stride);
     static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
-    if (r.lds > 48 * 1024 && !big_lds_allowed) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prompt_kernel<D>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+    if (lds > 48 * 1024 && !big_lds_allowed) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prompt_kernel<D, APPEND>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  128 * 1024);
         big_lds_allowed = true;
     }
-    attn_prompt_kernel<D><<<dim3(c.num_attention_heads, r.nb), 1024, r.lds, st>>>(
-        m->pb_qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0, r.per_seq ? m->pos : nullptr,
-        m->seq_stride, c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, c.sliding_window, m->pb_att);
+    const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * D + cache_off;
+    attn_prompt_kernel<D, APPEND><<<dim3(c.num_attention_heads, nb), 1024, lds, st>>>(
+        qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, pos0, pos_arr, m->seq_stride, c.num_attention_heads,
+        c.num_key_value_heads, c.max_position_embeddings, c.sliding_window, att);
+}
+
+// Attention of `nb` rows of layer l.  pos_arr == NULL: rows of one sequence (cache at cache_off) at positions pos0.., whose
+// keys and values rope_append_kernel has put into the cache.  Otherwise row b belongs to sequence b at position
+// pos_arr[b], and the kernel appends that row's key and value itself.
+void launch_attn_rows(axq_model *m, int l, const float *qkv, int nb, int pos0, const int32_t *pos_arr, size_t cache_off, size_t lds,
+                      float *att, hipStream_t st) {
+    const bool ap = pos_arr != nullptr;
+    switch (m->cfg.head_dim) {
+    case 32: ap ? launch_attn_rows_t<32, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st)
+                : launch_attn_rows_t<32, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st); break;
+    case 64: ap ? launch_attn_rows_t<64, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st)
+                : launch_attn_rows_t<64, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st); break;
+    case 128: ap ? launch_attn_rows_t<128, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st)
+                 : launch_attn_rows_t<128, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st); break;
+    default: ap ? launch_attn_rows_t<256, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st)
+                : launch_attn_rows_t<256, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st); break;
+    }
 }
 
 // The layers for `nb` rows (LLaMA::forward_with_cache on [batch, seq] input ids, llama.rs:731-762, for seq > 1 with
@@ -907,15 +967,11 @@ int enqueue_rows(axq_model *m, const Rows &r) {
     for (int l = 0; l < c.num_hidden_layers; l++) {
         const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * d + seq_off;
         if ((rc = lin(m->w_qkv[l], m->pb_h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv))) return rc;
-        rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
-            m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0,
-            r.per_seq ? m->pos : nullptr, m->seq_stride, c.max_position_embeddings, d);
-        switch (d) {
-        case 32: launch_attn_prompt_d<32>(m, l, r, st); break;
-        case 64: launch_attn_prompt_d<64>(m, l, r, st); break;
-        case 128: launch_attn_prompt_d<128>(m, l, r, st); break;
-        default: launch_attn_prompt_d<256>(m, l, r, st); break;
-        }
+        if (!r.per_seq)
+            rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
+                m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0, nullptr,
+                m->seq_stride, c.max_position_embeddings, d);
+        launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st);
         if ((rc = lin(m->w_o[l], m->pb_att, AXQ_X_PLAIN, nullptr, m->pb_h, m->pb_h))) return rc;
         if ((rc = lin(m->w_gu[l], m->pb_h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu))) return rc;
         if ((rc = lin(m->w_down[l], m->pb_gu, AXQ_X_SWIGLU, nullptr, m->pb_h, m->pb_h))) return rc;
@@ -969,7 +1025,7 @@ int feed_prompt(axq_model *m, int base, int n_prompt) {
     if ((rc = feed_rows(m, 0, m->prompt, n_prompt - 1, base, &i))) return rc;
     for (; i < n_prompt && !rc; i++) {
         pick_prompt_kernel<<<1, 1, 0, ctx->stream>>>(m->prompt, m->pos, base, m->tok);
-        rc = run_token(m);
+        rc = run_token(m, base + i);
     }
     return rc;
 }
@@ -1047,6 +1103,11 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     m->kv_dim = c.num_key_value_heads * c.head_dim;
     m->qkv_rows = m->q_dim + 2 * m->kv_dim;
     m->max_splits = (c.max_position_embeddings + ATT_CHUNK - 1) / ATT_CHUNK;
+    {
+        const char *knob = getenv("AXQ_ATTN_FUSED_MAX"); // development knob: 0 = always split the positions
+        m->fused_max = knob ? atoi(knob) : 384; // measured at the 7B shape: 670 against 645 tokens/s up to 224 positions, even at 384, behind from 512
+        if (m->fused_max > 32768) m->fused_max = 32768;
+    }
     m->n_seq = 1;
     m->seq_stride = (size_t)c.num_hidden_layers * c.num_key_value_heads * c.max_position_embeddings * c.head_dim;
     m->seq_pos.assign(1, 0);
@@ -1118,6 +1179,7 @@ void axq_model_free(axq_model *m) {
     axq_ctx *ctx = m->ctx;
     (void)hipStreamSynchronize(ctx->stream);
     if (m->graph_ok) (void)hipGraphExecDestroy(m->graph);
+    if (m->graph_f_ok) (void)hipGraphExecDestroy(m->graph_f);
     if (m->graph_b_ok) (void)hipGraphExecDestroy(m->graph_b);
     for (void *p : {(void *)m->bprompt, (void *)m->boffsets, (void *)m->bout})
         if (p) (void)hipFree(p);
@@ -1273,8 +1335,9 @@ int axq_model_set_batch(axq_model *m, int n_seq) {
     AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
     // the graphs hold the old addresses
     if (m->graph_ok) (void)hipGraphExecDestroy(m->graph);
+    if (m->graph_f_ok) (void)hipGraphExecDestroy(m->graph_f);
     if (m->graph_b_ok) (void)hipGraphExecDestroy(m->graph_b);
-    m->graph_ok = m->graph_b_ok = false;
+    m->graph_ok = m->graph_f_ok = m->graph_b_ok = false;
     const size_t P = c.max_position_embeddings, S = (size_t)n_seq;
     for (void **p : {(void **)&m->kcache, (void **)&m->vcache, (void **)&m->pos, (void **)&m->tok, (void **)&m->next, (void **)&m->hist,
                      (void **)&m->logits, (void **)&m->bprompt, (void **)&m->boffsets, (void **)&m->bout}) {
@@ -1491,7 +1554,7 @@ int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_t *next_
                         m->cfg.max_position_embeddings);
     AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
     set_i32_kernel<<<1, 1, 0, ctx->stream>>>(m->tok, token);
-    if ((rc = run_token(m))) return rc;
+    if ((rc = run_token(m, m->host_pos))) return rc;
     m->host_pos++;
     if (logits)
         AXQ_HIP(ctx, hipMemcpyAsync(logits, m->logits, (size_t)m->cfg.vocab_size * 4, hipMemcpyDeviceToHost, ctx->stream),
@@ -1562,7 +1625,7 @@ int axq_model_generate(axq_model *m, const int32_t *prompt, int n_prompt, int ma
     // generation: the argmax of step i is the input of step i+1, on the device
     for (int i = 0; i < max_new_tokens && !rc; i++) {
         commit_next_kernel<<<1, 1, 0, ctx->stream>>>(m->next, m->tok, m->gen, m->out, m->out_cap);
-        if (i + 1 < max_new_tokens) rc = run_token(m);
+        if (i + 1 < max_new_tokens) rc = run_token(m, base + n_prompt + i);
     }
     (void)hipEventRecord(e2, ctx->stream);
     hipError_t e = hipStreamSynchronize(ctx->stream);

@@ -44,6 +44,35 @@ def test_sliding_window_attention(ctx, window):
     gpu.close()
 
 
+@pytest.mark.parametrize("fused_max", ["0", "20", "1000"])
+def test_both_attention_forms_of_the_step(ctx, monkeypatch, fused_max):
+    """Short contexts take one attention workgroup per head, longer ones split the positions over workgroups and
+    merge; the switch-over (normally at 1024 positions) is moved into the walk here."""
+    monkeypatch.setenv("AXQ_ATTN_FUSED_MAX", fused_max)
+    c = tiny_config(max_seq_len=64, sliding_window=0)
+    w = random_weights(c, 95)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    tok = 4
+    for pos in range(40):
+        c_next, c_logits = cpu.forward(tok, pos)
+        g_next, g_logits = gpu.forward(tok)
+        assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, pos
+        assert g_next == c_next, pos
+        tok = c_next
+    gpu.reset()
+    prompt = np.random.default_rng(5).integers(0, c["vocab_size"], size=12)
+    want = []
+    for pos, t in enumerate(prompt):
+        nxt, _ = cpu.forward(int(t), pos)
+    for i in range(30):
+        want.append(nxt)
+        nxt, _ = cpu.forward(nxt, len(prompt) + i)
+    got, _, _ = gpu.generate(prompt, 30)  # crosses position 20 inside the generation loop
+    assert got.tolist() == want
+    gpu.close()
+    cpu.close()
+
+
 def test_kv_cache_matches_oracle_up_to_isolated_f16_roundings(ctx):
     c = tiny_config(num_layers=2)
     w = random_weights(c, 50)
