@@ -7,6 +7,8 @@
 // multiply, divide, add and subtract separately (f32), and so do these kernels.
 #include <hip/hip_fp16.h>
 
+#include <stdint.h>
+
 #include "axq_internal.h"
 
 namespace {
@@ -473,6 +475,77 @@ __global__ void repack_kernel(PlanarDesc d, uint8_t *packed, bool to_planar) {
     }
 }
 
+// The same copy for images whose base is 16-byte aligned: a workgroup takes 128 consecutive blocks, whose images
+// form one contiguous, 16-byte aligned run (128 times any image size is a multiple of 16), moves that run between
+// memory and LDS with 16-byte accesses, and serves the planes from LDS: one thread per block for the scales (and
+// the high bits), one thread per 16 bytes of codes.  Every access to memory is as wide as its alignment allows
+// and consecutive threads touch consecutive addresses.
+template <int IMG, int META, int QH, int CODE>
+__global__ void __launch_bounds__(256) repack_lds_kernel(PlanarDesc d, uint8_t *packed, bool to_planar, int64_t total) {
+    constexpr int NB = 128, CU = CODE / 16;
+    __shared__ __attribute__((aligned(16))) uint8_t img[NB * IMG];
+    const int tid = threadIdx.x;
+    const int64_t t0 = (int64_t)blockIdx.x * NB;
+    const int nb = total - t0 < NB ? (int)(total - t0) : NB;
+    const int nbytes = nb * IMG;
+    uint8_t *g = packed + (size_t)t0 * IMG;
+    if (to_planar) {
+        for (int o = tid * 16; o + 16 <= nbytes; o += 256 * 16) *reinterpret_cast<uint4 *>(img + o) = *reinterpret_cast<const uint4 *>(g + o);
+        for (int o = (nbytes & ~15) + tid * 2; o < nbytes; o += 512) store_u16(img + o, load_u16(g + o)); // a last run's tail
+        __syncthreads();
+    }
+    for (int u = tid; u < nb; u += 256) {
+        const int64_t t = t0 + u, row = t / d.blocks_per_row, blk = t - row * d.blocks_per_row;
+        uint8_t *li = img + u * IMG;
+        uint8_t *pm = d.meta + (size_t)row * d.meta_pitch + (size_t)blk * META;
+        if (META == 2) {
+            if (to_planar) store_u16(pm, load_u16(li)); else store_u16(li, load_u16(pm));
+        } else if (META == 4) {
+            if (to_planar) {
+                *reinterpret_cast<uint32_t *>(pm) = (uint32_t)load_u16(li) | ((uint32_t)load_u16(li + 2) << 16);
+            } else {
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(pm);
+                store_u16(li, (uint16_t)v); store_u16(li + 2, (uint16_t)(v >> 16));
+            }
+        } else { // 16: IMG is a multiple of 16 too, so the LDS side is aligned as well
+            if (to_planar) *reinterpret_cast<uint4 *>(pm) = *reinterpret_cast<const uint4 *>(li);
+            else *reinterpret_cast<uint4 *>(li) = *reinterpret_cast<const uint4 *>(pm);
+        }
+        if (QH) {
+            uint8_t *ph = d.qh + (size_t)row * d.qh_pitch + (size_t)blk * 4;
+            if (to_planar) {
+                *reinterpret_cast<uint32_t *>(ph) = (uint32_t)load_u16(li + META) | ((uint32_t)load_u16(li + META + 2) << 16);
+            } else {
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(ph);
+                store_u16(li + META, (uint16_t)v); store_u16(li + META + 2, (uint16_t)(v >> 16));
+            }
+        }
+    }
+    for (int v = tid; v < nb * CU; v += 256) {
+        const int u = v / CU, c = v - u * CU;
+        const int64_t t = t0 + u, row = t / d.blocks_per_row, blk = t - row * d.blocks_per_row;
+        uint8_t *li = img + u * IMG + META + QH + 16 * c; // 2-byte aligned
+        uint8_t *pc = d.codes + (size_t)row * d.codes_pitch +
+                      (d.type == AXQ_Q4_K ? q4k_code_offset(d.blocks_per_row, blk, 16 * c) : (size_t)blk * CODE + 16 * c);
+        if (to_planar) {
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) w[i] = (uint32_t)load_u16(li + 4 * i) | ((uint32_t)load_u16(li + 4 * i + 2) << 16);
+            *reinterpret_cast<uint4 *>(pc) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+            const uint4 q = *reinterpret_cast<const uint4 *>(pc);
+            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) { store_u16(li + 4 * i, (uint16_t)w[i]); store_u16(li + 4 * i + 2, (uint16_t)(w[i] >> 16)); }
+        }
+    }
+    if (!to_planar) {
+        __syncthreads();
+        for (int o = tid * 16; o + 16 <= nbytes; o += 256 * 16) *reinterpret_cast<uint4 *>(g + o) = *reinterpret_cast<const uint4 *>(img + o);
+        for (int o = (nbytes & ~15) + tid * 2; o < nbytes; o += 512) store_u16(g + o, load_u16(img + o));
+    }
+}
+
 inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
 
 } // namespace
@@ -533,7 +606,20 @@ int axq_dev_repack(axq_ctx *ctx, const axq_weight *w, uint8_t *packed, bool to_p
     d.type = w->type;
     size_t total = (size_t)(d.n_rows * d.blocks_per_row);
     if (total == 0) return AXQ_OK;
-    repack_kernel<<<grid_for(total, 128), 128, 0, ctx->stream>>>(d, packed, to_planar);
+    if ((reinterpret_cast<uintptr_t>(packed) & 15) == 0) { // the usual case: allocations are aligned far beyond that
+        const unsigned grid = grid_for(total, 128);
+        const int64_t n = (int64_t)total;
+        switch (w->type) {
+        case AXQ_Q8_0: repack_lds_kernel<34, 2, 0, 32><<<grid, 256, 0, ctx->stream>>>(d, packed, to_planar, n); break;
+        case AXQ_Q4_0: repack_lds_kernel<18, 2, 0, 16><<<grid, 256, 0, ctx->stream>>>(d, packed, to_planar, n); break;
+        case AXQ_Q4_1: repack_lds_kernel<20, 4, 0, 16><<<grid, 256, 0, ctx->stream>>>(d, packed, to_planar, n); break;
+        case AXQ_Q5_0: repack_lds_kernel<22, 2, 4, 16><<<grid, 256, 0, ctx->stream>>>(d, packed, to_planar, n); break;
+        case AXQ_Q5_1: repack_lds_kernel<24, 4, 4, 16><<<grid, 256, 0, ctx->stream>>>(d, packed, to_planar, n); break;
+        default: repack_lds_kernel<144, 16, 0, 128><<<grid, 256, 0, ctx->stream>>>(d, packed, to_planar, n); break;
+        }
+    } else {
+        repack_kernel<<<grid_for(total, 128), 128, 0, ctx->stream>>>(d, packed, to_planar);
+    }
     AXQ_LAUNCH_CHECK(ctx, "repack kernel");
     return AXQ_OK;
 }
