@@ -48,24 +48,37 @@ __device__ inline void store_u16(uint8_t *p, uint16_t v) { *reinterpret_cast<uin
 __device__ inline uint16_t load_u16(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
 
 // ---- Q8_0: quantize.rs:82-114, image types.rs:142-147 ---------------------
-__global__ void quant_q8_0_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
-    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= nblk) return;
-    float x[32];
-    int len;
-    load_block32(src, numel, b, x, len);
-    float max_abs = 0.0f;
+// The 34-byte images of a workgroup's 128 blocks are put together in LDS and leave as one run of 16-byte stores
+// (a thread writing its own image would store 2 bytes at a time, 34 bytes from its neighbour's).
+__global__ void __launch_bounds__(128) quant_q8_0_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
+    __shared__ __attribute__((aligned(16))) uint8_t img[128 * 34];
+    const size_t b0 = (size_t)blockIdx.x * 128, b = b0 + threadIdx.x;
+    if (b < nblk) {
+        float x[32];
+        int len;
+        load_block32(src, numel, b, x, len);
+        float max_abs = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 32; i++)
-        if (i < len) max_abs = fmaxf(max_abs, fabsf(x[i]));
-    float scale = max_abs > 0.0f ? max_abs / 127.0f : 1.0f;
-    uint8_t *o = out + b * 34;
-    store_u16(o, f32_to_f16_bits(scale));
+        for (int i = 0; i < 32; i++)
+            if (i < len) max_abs = fmaxf(max_abs, fabsf(x[i]));
+        float scale = max_abs > 0.0f ? max_abs / 127.0f : 1.0f;
+        uint8_t *o = img + threadIdx.x * 34;
+        store_u16(o, f32_to_f16_bits(scale));
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        int q0 = (2 * i) < len ? round_clamp(x[2 * i] / scale, -127.0f, 127.0f) : 0;
-        int q1 = (2 * i + 1) < len ? round_clamp(x[2 * i + 1] / scale, -127.0f, 127.0f) : 0;
-        store_u16(o + 2 + 2 * i, (uint16_t)((q0 & 0xFF) | ((q1 & 0xFF) << 8)));
+        for (int i = 0; i < 16; i++) {
+            int q0 = (2 * i) < len ? round_clamp(x[2 * i] / scale, -127.0f, 127.0f) : 0;
+            int q1 = (2 * i + 1) < len ? round_clamp(x[2 * i + 1] / scale, -127.0f, 127.0f) : 0;
+            store_u16(o + 2 + 2 * i, (uint16_t)((q0 & 0xFF) | ((q1 & 0xFF) << 8)));
+        }
+    }
+    __syncthreads();
+    const int nb = nblk - b0 < 128 ? (int)(nblk - b0) : 128, nbytes = nb * 34;
+    uint8_t *g = out + b0 * 34; // 128 * 34 is a multiple of 16: as aligned as `out`
+    if ((reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        for (int o = threadIdx.x * 16; o + 16 <= nbytes; o += 128 * 16) *reinterpret_cast<uint4 *>(g + o) = *reinterpret_cast<const uint4 *>(img + o);
+        for (int o = (nbytes & ~15) + threadIdx.x * 2; o < nbytes; o += 256) store_u16(g + o, load_u16(img + o));
+    } else {
+        for (int o = threadIdx.x * 2; o < nbytes; o += 256) store_u16(g + o, load_u16(img + o));
     }
 }
 
@@ -298,20 +311,50 @@ __global__ void quant_q4_k_kernel(const float *src, size_t numel, size_t nsb, ui
 }
 
 // ---- F16: quantize.rs:212-218 --------------------------------------------
+// eight elements per thread where both sides are 16-byte aligned, one by one otherwise and for the last few
 __global__ void quant_f16_kernel(const float *src, size_t numel, uint16_t *out) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < numel) out[i] = f32_to_f16_bits(src[i]);
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x, i = t * 8;
+    if (i >= numel) return;
+    if (i + 8 <= numel && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+        const float4 a = reinterpret_cast<const float4 *>(src + i)[0], b = reinterpret_cast<const float4 *>(src + i)[1];
+        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) w[j] = (uint32_t)f32_to_f16_bits(v[2 * j]) | ((uint32_t)f32_to_f16_bits(v[2 * j + 1]) << 16);
+        *reinterpret_cast<uint4 *>(out + i) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+        for (size_t j = i; j < numel && j < i + 8; j++) out[j] = f32_to_f16_bits(src[j]);
+    }
 }
 __global__ void dequant_f16_kernel(const uint16_t *src, size_t numel, float *out) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < numel) out[i] = f16_bits_to_f32(src[i]);
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x, i = t * 8;
+    if (i >= numel) return;
+    if (i + 8 <= numel && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(src + i);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[2 * j] = f16_bits_to_f32((uint16_t)w[j]);
+            v[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
+        }
+        reinterpret_cast<float4 *>(out + i)[0] = make_float4(v[0], v[1], v[2], v[3]);
+        reinterpret_cast<float4 *>(out + i)[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        for (size_t j = i; j < numel && j < i + 8; j++) out[j] = f16_bits_to_f32(src[j]);
+    }
 }
 
 // ---- dequantisers: dequantize.rs:89-92, 116-121, 145-151 -------------------
 // One thread per 32 elements; for Q4_K a thread handles one sub-block.
-__global__ void dequant_kernel(int type, const uint8_t *packed, size_t numel, size_t n32, float *out) {
-    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n32) return;
+// The 32 values of a thread go through an LDS tile (rows padded to 33 floats), so that the workgroup's 16 KB of
+// output leave as consecutive 16-byte stores instead of 128-byte strides between neighbouring threads.
+__global__ void __launch_bounds__(128) dequant_kernel(int type, const uint8_t *packed, size_t numel, size_t n32, float *out) {
+    __shared__ float tile[128 * 33];
+    const size_t t0 = (size_t)blockIdx.x * 128;
+    size_t t = t0 + threadIdx.x;
+    const bool live = t < n32;
+    if (!live) t = n32 - 1; // computes a block again, stores nothing: every thread has to reach the barrier
     float y[32];
     switch (type) {
     case AXQ_Q8_0: {
@@ -414,15 +457,25 @@ __global__ void dequant_kernel(int type, const uint8_t *packed, size_t numel, si
     default:
         return;
     }
-    size_t start = t * 32;
-    if (start + 32 <= numel) {
-        float4 *o = reinterpret_cast<float4 *>(out + start);
+    if (live) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) o[i] = make_float4(y[4 * i], y[4 * i + 1], y[4 * i + 2], y[4 * i + 3]);
-    } else {
+        for (int i = 0; i < 32; i++) tile[threadIdx.x * 33 + i] = y[i];
+    }
+    __syncthreads();
+    const size_t start = t0 * 32; // of the workgroup
+    const bool vec = (reinterpret_cast<uintptr_t>(out) & 15) == 0;
 #pragma unroll
-        for (int i = 0; i < 32; i++)
-            if (start + i < numel) out[start + i] = y[i];
+    for (int r = 0; r < 8; r++) {
+        const int e4 = r * 128 + threadIdx.x, row = e4 >> 3, col = (e4 & 7) * 4;
+        const size_t g = start + (size_t)e4 * 4;
+        const float *src = tile + row * 33 + col;
+        if (vec && g + 4 <= numel) {
+            *reinterpret_cast<float4 *>(out + g) = make_float4(src[0], src[1], src[2], src[3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (g + i < numel) out[g + i] = src[i];
+        }
     }
 }
 
@@ -561,7 +614,7 @@ int axq_dev_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, uin
     case AXQ_Q5_0: quant_q5_kernel<false><<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_Q5_1: quant_q5_kernel<true><<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_Q4_K: quant_q4_k_kernel<<<grid_for(nblk * 8, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
-    case AXQ_F16: quant_f16_kernel<<<grid_for(numel, 256), 256, 0, ctx->stream>>>(src, numel, (uint16_t *)packed); break;
+    case AXQ_F16: quant_f16_kernel<<<grid_for((numel + 7) / 8, 256), 256, 0, ctx->stream>>>(src, numel, (uint16_t *)packed); break;
     case AXQ_F32:
         AXQ_HIP(ctx, hipMemcpyAsync(packed, src, numel * 4, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
         return AXQ_OK;
@@ -580,7 +633,7 @@ int axq_dev_dequantize(axq_ctx *ctx, int type, const uint8_t *packed, size_t num
         break;
     }
     case AXQ_F16:
-        dequant_f16_kernel<<<grid_for(numel, 256), 256, 0, ctx->stream>>>((const uint16_t *)packed, numel, dst);
+        dequant_f16_kernel<<<grid_for((numel + 7) / 8, 256), 256, 0, ctx->stream>>>((const uint16_t *)packed, numel, dst);
         break;
     case AXQ_F32:
         AXQ_HIP(ctx, hipMemcpyAsync(dst, packed, numel * 4, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);

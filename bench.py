@@ -209,6 +209,41 @@ def cpu_decode_baseline(budget_tokens=8):
             "sample": f"median of {budget_tokens} tokens on a 2-layer model of the Mistral-7B shape with the full lm_head, context < 16"}
 
 
+def codec_rates(ctx, n=N_HEAD, k=K_HEAD, iters=20):
+    """quantize_tensor / dequantize_tensor on the device for one weight of the headline shape, per type: time per call
+    and the bytes it has to move (4 B per element on the f32 side, the packed image on the other)."""
+    from axonml_amd import quant as q
+    from axonml_amd._lib import MEM_DEVICE
+
+    lib, numel = ctx.lib, n * k
+    f = ctx.malloc(numel * 4)
+    g = ctx.malloc(numel * 4)
+    ctx.check(lib.axq_fill_normal_f32(ctx.handle, f, numel, 0.0, 0.02, 0.01, 0.5, 99))
+    out = []
+    for qt in (q.QuantType.Q8_0, q.QuantType.Q4_0, q.QuantType.Q4_1, q.QuantType.Q5_0, q.QuantType.Q5_1, q.QuantType.Q4_K, q.QuantType.F16):
+        nbytes = lib.axq_packed_bytes(int(qt), numel)
+        p = ctx.malloc(nbytes)
+        r = {"type": str(qt), "numel": numel, "packed_bytes": nbytes}
+        for name, call in (("quantize", lambda: lib.axq_quantize(ctx.handle, int(qt), f, numel, p, MEM_DEVICE)),
+                           ("dequantize", lambda: lib.axq_dequantize(ctx.handle, int(qt), p, numel, g, MEM_DEVICE))):
+            for _ in range(3):
+                ctx.check(call())
+            ctx.synchronize()
+            ctx.timer_start()
+            for _ in range(iters):
+                ctx.check(call())
+            t = ctx.timer_stop() / iters
+            r[f"{name}_us"] = t * 1e3
+            r[f"{name}_gbps"] = (numel * 4 + nbytes) / (t * 1e-3) / 1e9
+        log(f"  codec {r['type']}: quantize {r['quantize_us']:.1f} us ({r['quantize_gbps']:.0f} GB/s), "
+            f"dequantize {r['dequantize_us']:.1f} us ({r['dequantize_gbps']:.0f} GB/s)")
+        out.append(r)
+        ctx.free(p)
+    ctx.free(f)
+    ctx.free(g)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -264,6 +299,7 @@ def main():
             gem.append(r)
             log(f"  {r['type']} [{n},{k}] b={b}: {r['us_per_step']:.2f} us, {r['gbps']:.0f} GB/s")
         extra["gemv"] = gem
+        extra["codecs"] = codec_rates(ctx)
         try:
             from axonml_amd import decode as d
 
