@@ -880,6 +880,11 @@ int reserve_prompt_rows(axq_model *m, int cap) {
     return AXQ_OK;
 }
 
+bool attn_mfma_allowed() {
+    static const bool off = getenv("AXQ_ATTN_MFMA") && getenv("AXQ_ATTN_MFMA")[0] == '0'; // development knob
+    return !off;
+}
+
 // What a call of enqueue_rows works on.
 struct Rows {
     int mode;            // ROWS_GEMV or ROWS_GEMM
@@ -971,7 +976,15 @@ int enqueue_rows(axq_model *m, const Rows &r) {
             rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
                 m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0, nullptr,
                 m->seq_stride, c.max_position_embeddings, d);
-        launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st);
+        // many rows of one sequence: attention on the matrix pipe, a tile of rows against every key once
+        int on_mfma = 0;
+        if (!r.per_seq && nb >= PROMPT_GEMM_MIN && attn_mfma_allowed()) {
+            on_mfma = axq_dev_attn_rows_mfma(ctx, m->pb_qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0,
+                                             nb, c.num_attention_heads, c.num_key_value_heads, d, c.max_position_embeddings,
+                                             c.sliding_window, m->pb_att);
+            if (on_mfma < 0) return on_mfma;
+        }
+        if (!on_mfma) launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st);
         if ((rc = lin(m->w_o[l], m->pb_att, AXQ_X_PLAIN, nullptr, m->pb_h, m->pb_h))) return rc;
         if ((rc = lin(m->w_gu[l], m->pb_h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu))) return rc;
         if ((rc = lin(m->w_down[l], m->pb_gu, AXQ_X_SWIGLU, nullptr, m->pb_h, m->pb_h))) return rc;

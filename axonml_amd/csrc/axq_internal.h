@@ -128,6 +128,10 @@ int axq_dev_sample_rows(axq_ctx *ctx, int rows, const float *logits, size_t logi
                         size_t hist_stride, const int32_t *hist_len_dev, int hist_len, const axq_sampling_config *cfg, float u,
                         const int32_t *counter_dev, uint64_t seed, uint64_t seed_stride, void *scratch, int32_t *out,
                         float *filtered_out);
+// attn.hip: causal attention of T prompt rows of one sequence on the matrix pipe; 1 = launched, 0 = shape not covered
+int axq_dev_attn_rows_mfma(axq_ctx *ctx, const float *qkv, int qkv_rows, const float *rope_cos, const float *rope_sin,
+                           const uint16_t *kcache, const uint16_t *vcache, int pos0, int T, int n_heads, int n_kv, int head_dim,
+                           int max_pos, int window, float *att);
 // gemm.hip
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_dev, int m, float *y_dev);
 #define AXQ_GEMM_F32_MAX_ROWS 2048 // rows per call of the f32-activation GEMM (its scratch grows with them)

@@ -129,6 +129,13 @@ def test_generate_matches_oracle_greedy_and_is_repeatable(ctx):
     (dict(max_seq_len=100), o.Q4_K, 0, 70), (dict(max_seq_len=100), o.Q4_0, 3, 45), (dict(max_seq_len=100), o.Q5_0, 0, 34),
     (dict(max_seq_len=128, num_heads=8, num_kv_heads=2, head_dim=32), o.Q8_0, 10, 100),
     (dict(max_seq_len=100, num_heads=2, num_kv_heads=1, head_dim=128, num_layers=3), o.Q4_1, 0, 41),
+    # many rows: attention on the matrix pipe; several key tiles per wave, every ratio of query to KV heads, windows
+    (dict(max_seq_len=320), o.Q4_K, 0, 300), (dict(max_seq_len=320), o.Q4_K, 37, 270),
+    (dict(max_seq_len=200, num_heads=8, num_kv_heads=1, head_dim=32), o.Q4_K, 0, 190),
+    (dict(max_seq_len=200, num_heads=4, num_kv_heads=4, head_dim=64), o.Q4_0, 5, 150),
+    (dict(max_seq_len=200, num_heads=2, num_kv_heads=2, head_dim=128), o.Q8_0, 0, 130),
+    (dict(max_seq_len=260, sliding_window=40), o.Q4_K, 0, 250), (dict(max_seq_len=260, sliding_window=33, num_heads=8, num_kv_heads=2, head_dim=32), o.Q4_K, 9, 240),
+    (dict(max_seq_len=200, num_heads=3, num_kv_heads=1, head_dim=64, hidden_size=192), o.Q8_0, 0, 120),  # three query heads per KV head: the general kernel
 ])
 def test_prompt_fed_at_once_matches_the_oracle_token_by_token(ctx, over, qtype, n_first, n_prompt):
     """forward_tokens (up to eight prompt tokens per pass over the weights) against the oracle's one-token steps:
