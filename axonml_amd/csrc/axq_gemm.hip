@@ -39,6 +39,10 @@ struct GemmArgs {
     float *ypart;          // split K: [splits, M, N] unscaled partial sums (NULL when one workgroup covers all of K)
     int m, n, k;
     int steps_per_split;   // K steps per workgroup (grid.y of them cover K)
+    // pair mode (f32 activations): rows 2t and 2t + 1 of xh are the two f16 parts of activation row t, and their results
+    // are added into output row t (+ bias[n] + resid[t, n]); y, ypart and resid then have m / 2 rows
+    int pair;
+    const float *bias, *resid;
 };
 
 __device__ inline float h2f(uint32_t bits) { return __half2float(__ushort_as_half((unsigned short)bits)); }
@@ -397,8 +401,21 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
             for (int r = 0; r < 16; r++) {
                 const int gm = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (gm < a.m && gn < a.n) {
-                    if (a.ypart) a.ypart[((size_t)blockIdx.y * a.m + gm) * a.n + gn] = acc[i][j][r];
-                    else a.y[(size_t)gm * a.n + gn] = acc[i][j][r] * (a.rowscale[gm] * (1.0f / T::WS));
+                    if (!a.pair) {
+                        if (a.ypart) a.ypart[((size_t)blockIdx.y * a.m + gm) * a.n + gn] = acc[i][j][r];
+                        else a.y[(size_t)gm * a.n + gn] = acc[i][j][r] * (a.rowscale[gm] * (1.0f / T::WS));
+                    } else if ((r & 1) == 0) { // gm is even: this register and the next hold the two parts of row gm / 2
+                        const size_t t = (size_t)(gm >> 1);
+                        const float v = acc[i][j][r] + acc[i][j][r + 1];
+                        if (a.ypart) {
+                            a.ypart[((size_t)blockIdx.y * (a.m >> 1) + t) * a.n + gn] = v;
+                        } else {
+                            float out = v * (a.rowscale[gm] * (1.0f / T::WS));
+                            if (a.bias) out += a.bias[gn];
+                            if (a.resid) out += a.resid[t * a.n + gn];
+                            a.y[t * a.n + gn] = out;
+                        }
+                    }
                 }
             }
         }
@@ -433,18 +450,28 @@ __global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int
     if (threadIdx.x == 0) rowscale[row] = 1.0f / f;
 }
 
-// y = (sum over the splits, in order) * rowscale / ws: four outputs per thread
-__global__ void __launch_bounds__(256) gemm_reduce_kernel(const float *ypart, const float *rowscale, int m, int n, int splits,
-                                                          float inv_ws, float *y) {
-    const size_t i4 = (size_t)blockIdx.x * blockDim.x + threadIdx.x, total4 = (size_t)m * n / 4;
+// y = (sum over the splits, in order) * rowscale / ws (+ bias + resid): four outputs per thread.  `rows` output rows;
+// row_mul = 2 in pair mode (output row t was scaled as activation rows 2t, 2t + 1).
+__global__ void __launch_bounds__(256) gemm_reduce_kernel(const float *ypart, const float *rowscale, int rows, int n, int splits,
+                                                          float inv_ws, int row_mul, const float *bias, const float *resid, float *y) {
+    const size_t i4 = (size_t)blockIdx.x * blockDim.x + threadIdx.x, total4 = (size_t)rows * n / 4;
     if (i4 >= total4) return;
     float4 acc = reinterpret_cast<const float4 *>(ypart)[i4];
     for (int s = 1; s < splits; s++) {
-        const float4 v = reinterpret_cast<const float4 *>(ypart + (size_t)s * m * n)[i4];
+        const float4 v = reinterpret_cast<const float4 *>(ypart + (size_t)s * rows * n)[i4];
         acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
     }
-    const float f = rowscale[(i4 * 4) / (size_t)n] * inv_ws; // n is a multiple of 4: the four share a row
-    reinterpret_cast<float4 *>(y)[i4] = make_float4(acc.x * f, acc.y * f, acc.z * f, acc.w * f);
+    const size_t row = (i4 * 4) / (size_t)n, col = (i4 * 4) % (size_t)n; // n is a multiple of 4: the four share a row
+    const float f = rowscale[row * row_mul] * inv_ws;
+    float4 out = make_float4(acc.x * f, acc.y * f, acc.z * f, acc.w * f);
+    if (bias) {
+        out.x += bias[col]; out.y += bias[col + 1]; out.z += bias[col + 2]; out.w += bias[col + 3];
+    }
+    if (resid) {
+        const float4 r = reinterpret_cast<const float4 *>(resid)[i4];
+        out.x += r.x; out.y += r.y; out.z += r.z; out.w += r.w;
+    }
+    reinterpret_cast<float4 *>(y)[i4] = out;
 }
 
 template <class T>
@@ -465,17 +492,18 @@ int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
     else gemm_kernel<T, 1><<<grid, 256, lds, ctx->stream>>>(a);
     AXQ_LAUNCH_CHECK(ctx, "gemm_kernel");
     if (splits > 1) {
-        const size_t total4 = (size_t)a.m * a.n / 4;
-        gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(a.ypart, a.rowscale, a.m, a.n, splits,
-                                                                                    1.0f / T::WS, a.y);
+        const int rows = a.pair ? a.m / 2 : a.m;
+        const size_t total4 = (size_t)rows * a.n / 4;
+        gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(a.ypart, a.rowscale, rows, a.n, splits, 1.0f / T::WS,
+                                                                                    a.pair ? 2 : 1, a.bias, a.resid, a.y);
         AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
     }
     return AXQ_OK;
 }
 
 // f32 rows, optionally RMS-normalised on the way ((x * inv_rms) * norm_w, RMSNorm::forward, llm/src/llama.rs:158-187),
-// -> two f16 rows each under one power-of-two scale: row t holds the leading 11 bits of every element, row m + t
-// what those leave, so that their GEMM results add up to the f32 product.
+// -> two f16 rows each under one power-of-two scale: row 2t holds the leading 11 bits of every element, row 2t + 1
+// what those leave, so that their GEMM results add up to the f32 product (the GEMM's epilogue adds them: pair mode).
 __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, const float *norm_w, float eps, int m, int k,
                                                               _Float16 *xh, float *rowscale) {
     __shared__ float red[4];
@@ -521,21 +549,10 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
     for (int i = threadIdx.x; i < k; i += blockDim.x) {
         const float v = (norm_w ? (xr[i] * inv) * norm_w[i] : xr[i]) * f;
         const _Float16 hi = (_Float16)v;
-        xh[(size_t)row * k + i] = hi;
-        xh[(size_t)(m + row) * k + i] = (_Float16)(v - (float)hi);
+        xh[(size_t)(2 * row) * k + i] = hi;
+        xh[(size_t)(2 * row + 1) * k + i] = (_Float16)(v - (float)hi);
     }
-    if (threadIdx.x == 0) { rowscale[row] = 1.0f / f; rowscale[m + row] = 1.0f / f; }
-}
-
-// y[t] = y2[t] + y2[m + t] (+ bias) (+ resid[t]): the two halves of every activation row meet again
-__global__ void __launch_bounds__(256) gemm_pair_sum_kernel(const float *y2, const float *bias, const float *resid, size_t total, int n,
-                                                            float *y) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= total) return;
-    float v = y2[i] + y2[total + i];
-    if (bias) v += bias[i % (size_t)n];
-    if (resid) v += resid[i];
-    y[i] = v;
+    if (threadIdx.x == 0) { rowscale[2 * row] = 1.0f / f; rowscale[2 * row + 1] = 1.0f / f; }
 }
 
 struct GemmPlan {
@@ -577,7 +594,8 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, size_t extra, GemmPlan *
 }
 
 // The GEMM proper over activations that already sit in scratch as scaled f16 rows.
-int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float *y) {
+int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float *y, bool pair = false, const float *bias = nullptr,
+             const float *resid = nullptr) {
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     GemmArgs a;
     a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
@@ -586,6 +604,7 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     a.ypart = p.splits > 1 ? reinterpret_cast<float *>(base + p.xh_bytes + p.rs_bytes) : nullptr;
     a.m = m; a.n = (int)w->n_rows; a.k = (int)w->k;
     a.steps_per_split = p.steps_per_split;
+    a.pair = pair ? 1 : 0; a.bias = bias; a.resid = resid;
     switch (w->type) {
     case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);
     case AXQ_Q4_0: return launch_gemm<GQ4x<false>>(ctx, a, p.splits);
@@ -616,20 +635,15 @@ bool axq_dev_gemm_f32_covers(const axq_weight *w, int m) {
 }
 
 // y[m, n] = f(x)[m, k] W^T (+ bias[n]) (+ resid[m, n], which may be y) with f32 activations: each row goes through the
-// matrix pipe as two f16 rows (2m rows in all), and the two results are added.  f = RMSNorm with weight norm_w
+// matrix pipe as two adjacent f16 rows (2m rows in all), and the GEMM's epilogue adds the two results.  f = RMSNorm with weight norm_w
 // when that is given.
 int axq_dev_gemm_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int m, const float *norm_w, float eps, const float *bias,
                      const float *resid, float *y) {
     GemmPlan p;
     int rc;
-    const size_t total = (size_t)m * (size_t)w->n_rows;
-    if ((rc = plan_gemm(ctx, w, 2 * m, 2 * total * sizeof(float), &p))) return rc;
+    if ((rc = plan_gemm(ctx, w, 2 * m, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
-    float *y2 = reinterpret_cast<float *>(base + p.xh_bytes + p.rs_bytes + p.part_bytes);
     gemm_prep_x_f32_kernel<<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
                                                        reinterpret_cast<float *>(base + p.xh_bytes));
-    if ((rc = run_gemm(ctx, w, 2 * m, p, y2))) return rc;
-    gemm_pair_sum_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(y2, bias, resid, total, (int)w->n_rows, y);
-    AXQ_LAUNCH_CHECK(ctx, "gemm_pair_sum_kernel");
-    return AXQ_OK;
+    return run_gemm(ctx, w, 2 * m, p, y, true, bias, resid);
 }
