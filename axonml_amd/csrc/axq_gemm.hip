@@ -506,13 +506,32 @@ int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
 // what those leave, so that their GEMM results add up to the f32 product (the GEMM's epilogue adds them: pair mode).
 __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, const float *norm_w, float eps, int m, int k,
                                                               _Float16 *xh, float *rowscale) {
+    // the row stays in registers between the passes: 16 bytes per thread and step, up to 16 steps (k <= 16384);
+    // longer rows (or k not a multiple of 4) take the plain loops below
+    constexpr int STEPS = 16;
     __shared__ float red[4];
     const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float *xr = x + (size_t)row * k;
+    const bool in_regs = (k & 3) == 0 && k <= STEPS * 256 * 4;
+    float4 v[STEPS];
+    if (in_regs) {
+#pragma unroll
+        for (int c = 0; c < STEPS; c++) {
+            const int i4 = c * 256 + threadIdx.x;
+            v[c] = i4 * 4 < k ? reinterpret_cast<const float4 *>(xr)[i4] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     float inv = 1.0f;
     if (norm_w) {
         float ss = 0.f;
-        for (int i = threadIdx.x; i < k; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
+        if (in_regs) {
+#pragma unroll
+            for (int c = 0; c < STEPS; c++) {
+                ss = fmaf(v[c].x, v[c].x, ss); ss = fmaf(v[c].y, v[c].y, ss); ss = fmaf(v[c].z, v[c].z, ss); ss = fmaf(v[c].w, v[c].w, ss);
+            }
+        } else {
+            for (int i = threadIdx.x; i < k; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
+        }
 #pragma unroll
         for (int s = 32; s >= 1; s >>= 1) ss += __shfl_xor(ss, s);
         if (lane == 0) red[wave] = ss;
@@ -520,12 +539,27 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
         ss = (red[0] + red[1]) + (red[2] + red[3]);
         __syncthreads();
         inv = 1.0f / sqrtf(ss / (float)k + eps);
+        if (in_regs) {
+#pragma unroll
+            for (int c = 0; c < STEPS; c++) {
+                const int i4 = c * 256 + threadIdx.x;
+                if (i4 * 4 < k) {
+                    const float4 w = reinterpret_cast<const float4 *>(norm_w)[i4];
+                    v[c] = make_float4((v[c].x * inv) * w.x, (v[c].y * inv) * w.y, (v[c].z * inv) * w.z, (v[c].w * inv) * w.w);
+                }
+            }
+        }
     }
     uint32_t amax_bits = 0; // of |v| as integers: a NaN ranks above everything and is not dropped
-    for (int i = threadIdx.x; i < k; i += blockDim.x) {
-        const float v = norm_w ? (xr[i] * inv) * norm_w[i] : xr[i];
-        const uint32_t b = __builtin_bit_cast(uint32_t, v) & 0x7FFFFFFFu;
+    auto note = [&](float f) {
+        const uint32_t b = __builtin_bit_cast(uint32_t, f) & 0x7FFFFFFFu;
         amax_bits = b > amax_bits ? b : amax_bits;
+    };
+    if (in_regs) {
+#pragma unroll
+        for (int c = 0; c < STEPS; c++) { note(v[c].x); note(v[c].y); note(v[c].z); note(v[c].w); }
+    } else {
+        for (int i = threadIdx.x; i < k; i += blockDim.x) note(norm_w ? (xr[i] * inv) * norm_w[i] : xr[i]);
     }
 #pragma unroll
     for (int s = 32; s >= 1; s >>= 1) {
@@ -546,11 +580,28 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
     int sb = 127 + 14 - (eb - 127);
     sb = sb < 1 ? 1 : (sb > 254 ? 254 : sb);
     const float f = __builtin_bit_cast(float, (uint32_t)sb << 23);
-    for (int i = threadIdx.x; i < k; i += blockDim.x) {
-        const float v = (norm_w ? (xr[i] * inv) * norm_w[i] : xr[i]) * f;
-        const _Float16 hi = (_Float16)v;
-        xh[(size_t)(2 * row) * k + i] = hi;
-        xh[(size_t)(2 * row + 1) * k + i] = (_Float16)(v - (float)hi);
+    _Float16 *hi_row = xh + (size_t)(2 * row) * k, *lo_row = hi_row + k;
+    if (in_regs) {
+#pragma unroll
+        for (int c = 0; c < STEPS; c++) {
+            const int i4 = c * 256 + threadIdx.x;
+            if (i4 * 4 < k) {
+                const float e[4] = {v[c].x * f, v[c].y * f, v[c].z * f, v[c].w * f};
+                _Float16 h[4], l[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) { h[j] = (_Float16)e[j]; l[j] = (_Float16)(e[j] - (float)h[j]); }
+                typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+                reinterpret_cast<half4 *>(hi_row)[i4] = half4{h[0], h[1], h[2], h[3]};
+                reinterpret_cast<half4 *>(lo_row)[i4] = half4{l[0], l[1], l[2], l[3]};
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < k; i += blockDim.x) {
+            const float e = (norm_w ? (xr[i] * inv) * norm_w[i] : xr[i]) * f;
+            const _Float16 hi = (_Float16)e;
+            hi_row[i] = hi;
+            lo_row[i] = (_Float16)(e - (float)hi);
+        }
     }
     if (threadIdx.x == 0) { rowscale[2 * row] = 1.0f / f; rowscale[2 * row + 1] = 1.0f / f; }
 }
