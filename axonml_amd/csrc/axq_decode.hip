@@ -45,10 +45,11 @@ struct axq_model {
     int pb_cap;
     int n_seq;                      // sequences the caches and the per-sequence state hold (axq_model_set_batch)
     size_t seq_stride;              // cache elements of one sequence: layers * kv_heads * max_pos * head_dim
+    size_t part_stride;             // floats of att_part per sequence
     std::vector<int> seq_pos;       // host mirror of pos[s] for the batched calls (sequence 0: host_pos)
     int32_t *bprompt, *boffsets, *bout; // prompts, their offsets and the generated ids of a batched generate
-    hipGraphExec_t graph_b;
-    bool graph_b_ok;
+    hipGraphExec_t graph_b, graph_bf; // batched step: split attention / one attention workgroup per head (short contexts)
+    bool graph_b_ok, graph_bf_ok;
     int max_splits;
     // device-side state
     int32_t *pos, *tok, *next, *gen, *prompt, *out;
@@ -170,7 +171,7 @@ template <int D, int REP>
 __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, const float *rope_cos, const float *rope_sin,
                                                            uint16_t *kcache, uint16_t *vcache, const int32_t *pos_p,
                                                            int n_heads, int n_kv, int max_pos, int max_splits, int window,
-                                                           float *part) {
+                                                           float *part, int qkv_stride, size_t seq_stride, size_t part_stride) {
     constexpr int HALF = D / 2;
     constexpr int LP = D / 8, PPW = 64 / LP;                 // lanes per position, positions per wave pass
     constexpr int NPASS = (ATT_CHUNK + 4 * PPW - 1) / (4 * PPW); // passes of the four waves over the chunk
@@ -185,7 +186,12 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
     __shared__ __attribute__((aligned(16))) float vs[ATT_CHUNK * D];   // the chunk's values
     const int rep = n_heads / n_kv;
     const int kvh = blockIdx.x, split = blockIdx.y;
-    const int pos = pos_p[0];
+    // blockIdx.z: the sequence (batched steps: its own row of qkv, position counter, cache and partial results)
+    qkv += (size_t)blockIdx.z * qkv_stride;
+    kcache += (size_t)blockIdx.z * seq_stride;
+    vcache += (size_t)blockIdx.z * seq_stride;
+    part += (size_t)blockIdx.z * part_stride;
+    const int pos = pos_p[blockIdx.z];
     const int p0 = split * ATT_CHUNK;
     // sliding window (MistralAttention, mistral.rs:204-238): positions before p_lo are not attended to
     const int p_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
@@ -326,12 +332,14 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
 // grid (heads), 256 threads.  The (m, l) pairs of the head's splits go through LDS so that every thread
 // knows the weights exp(m_s - max) before it walks the splits; the walk itself has no dependent loads.
 __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, const int32_t *pos_p, int n_heads, int n_kv,
-                                                           int d, int max_splits, int window, float *att) {
+                                                           int d, int max_splits, int window, float *att, size_t part_stride) {
     extern __shared__ float cm[];
     float *wgt = cm;                 // [max_splits] exp(m_s - max)
     float *red = wgt + max_splits;   // [4] wave maxima, then [4] wave sums of l_s w_s
     const int head = blockIdx.x, rep = n_heads / n_kv, kvh = head / rep, h = head - kvh * rep;
-    const int pos = pos_p[0];
+    part += (size_t)blockIdx.y * part_stride; // blockIdx.y: the sequence
+    att += (size_t)blockIdx.y * n_heads * d;
+    const int pos = pos_p[blockIdx.y];
     const int s_lo = (window > 0 && pos + 1 > window) ? (pos + 1 - window) / ATT_CHUNK : 0; // first split inside the window
     const int nsplit = pos / ATT_CHUNK + 1 - s_lo;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -679,31 +687,39 @@ int copy_rows_interleaved(axq_ctx *ctx, axq_weight *dst, const axq_weight *src, 
     return AXQ_OK;
 }
 
+// Attention of the newest token of `nseq` sequences (rows of qkv, qkv_rows apart), split over the positions, and the
+// merge of the splits; results to att (rows n_heads * d apart).
 template <int D, int REP>
-void launch_attn_partial_t(axq_model *m, int l, hipStream_t st) {
+void launch_attn_partial_t(axq_model *m, int l, const float *qkv, int nseq, hipStream_t st) {
     const axq_model_config &c = m->cfg;
     const size_t kv_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * D;
-    attn_partial_kernel<D, REP><<<dim3(c.num_key_value_heads, m->max_splits), 256, 0, st>>>(
-        m->qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer, m->vcache + (size_t)l * kv_layer, m->pos,
-        c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, m->max_splits, c.sliding_window, m->att_part);
+    attn_partial_kernel<D, REP><<<dim3(c.num_key_value_heads, m->max_splits, nseq), 256, 0, st>>>(
+        qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer, m->vcache + (size_t)l * kv_layer, m->pos,
+        c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, m->max_splits, c.sliding_window, m->att_part,
+        m->qkv_rows, m->seq_stride, m->part_stride);
 }
 
 template <int D>
-void launch_attn_partial_d(axq_model *m, int l, hipStream_t st) {
+void launch_attn_partial_d(axq_model *m, int l, const float *qkv, int nseq, hipStream_t st) {
     const int rep = m->cfg.num_attention_heads / m->cfg.num_key_value_heads;
-    if (rep == 1) launch_attn_partial_t<D, 1>(m, l, st);
-    else if (rep == 2) launch_attn_partial_t<D, 2>(m, l, st);
-    else if (rep <= 4) launch_attn_partial_t<D, 4>(m, l, st);
-    else launch_attn_partial_t<D, 8>(m, l, st);
+    if (rep == 1) launch_attn_partial_t<D, 1>(m, l, qkv, nseq, st);
+    else if (rep == 2) launch_attn_partial_t<D, 2>(m, l, qkv, nseq, st);
+    else if (rep <= 4) launch_attn_partial_t<D, 4>(m, l, qkv, nseq, st);
+    else launch_attn_partial_t<D, 8>(m, l, qkv, nseq, st);
 }
 
-void launch_attn_partial(axq_model *m, int l, hipStream_t st) {
-    switch (m->cfg.head_dim) { // axq_model_create admits these four sizes only
-    case 32: launch_attn_partial_d<32>(m, l, st); break;
-    case 64: launch_attn_partial_d<64>(m, l, st); break;
-    case 128: launch_attn_partial_d<128>(m, l, st); break;
-    default: launch_attn_partial_d<256>(m, l, st); break;
+void launch_attn_split(axq_model *m, int l, const float *qkv, int nseq, float *att, hipStream_t st) {
+    const axq_model_config &c = m->cfg;
+    switch (c.head_dim) { // axq_model_create admits these four sizes only
+    case 32: launch_attn_partial_d<32>(m, l, qkv, nseq, st); break;
+    case 64: launch_attn_partial_d<64>(m, l, qkv, nseq, st); break;
+    case 128: launch_attn_partial_d<128>(m, l, qkv, nseq, st); break;
+    default: launch_attn_partial_d<256>(m, l, qkv, nseq, st); break;
     }
+    const size_t comb_lds = (size_t)(m->max_splits + 8) * sizeof(float);
+    attn_combine_kernel<<<dim3(c.num_attention_heads, nseq), 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
+                                                                                c.num_key_value_heads, c.head_dim, m->max_splits,
+                                                                                c.sliding_window, att, m->part_stride);
 }
 
 // y = g(W f(x) (+ bias)): f = identity or RMSNorm with weights `aux`; g = identity, or, for the fused gate/up
@@ -743,8 +759,7 @@ int enqueue_step(axq_model *m, bool short_ctx) {
     axq_ctx *ctx = m->ctx;
     const axq_model_config &c = m->cfg;
     hipStream_t st = ctx->stream;
-    const int H = c.hidden_size, d = c.head_dim;
-    const size_t comb_lds = (size_t)(m->max_splits + 8) * sizeof(float);
+    const int H = c.hidden_size;
     int rc;
     embed_kernel<<<(H / 8 + 255) / 256, 256, 0, st>>>(m->emb, m->tok, m->h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
@@ -753,9 +768,7 @@ int enqueue_step(axq_model *m, bool short_ctx) {
         if (short_ctx) {
             launch_attn_rows(m, l, m->qkv, 1, 0, m->pos, 0, prompt_attn_lds(m, m->fused_max), m->att, st);
         } else {
-            launch_attn_partial(m, l, st);
-            attn_combine_kernel<<<c.num_attention_heads, 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
-                                                                              c.num_key_value_heads, d, m->max_splits, c.sliding_window, m->att);
+            launch_attn_split(m, l, m->qkv, 1, m->att, st);
         }
         // residual adds go through the bias slot, in place
         if ((rc = linear(m, m->w_o[l], m->att, AXQ_X_PLAIN, nullptr, AXQ_Y_PLAIN, nullptr, m->h, m->h))) return rc;
@@ -861,10 +874,10 @@ int reserve_prompt_rows(axq_model *m, int cap) {
     axq_ctx *ctx = m->ctx;
     const int H = m->cfg.hidden_size, I = m->cfg.intermediate_size;
     AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
-    if (m->graph_b_ok) { // the batched step's graph holds the old addresses
-        (void)hipGraphExecDestroy(m->graph_b);
-        m->graph_b_ok = false;
-    }
+    // the batched step's graphs hold the old addresses
+    if (m->graph_b_ok) (void)hipGraphExecDestroy(m->graph_b);
+    if (m->graph_bf_ok) (void)hipGraphExecDestroy(m->graph_bf);
+    m->graph_b_ok = m->graph_bf_ok = false;
     for (float **p : {&m->pb_h, &m->pb_qkv, &m->pb_att, &m->pb_gu, &m->pb_act}) {
         if (*p) (void)hipFree(*p);
         *p = nullptr;
@@ -893,6 +906,7 @@ struct Rows {
     bool per_seq;        // false: rows pos0.. of sequence `seq`; true: row b is the next token of sequence b (nb = n_seq)
     int seq, pos0;
     size_t lds;          // of the attention kernel
+    bool split_attn;     // per_seq: the positions split over workgroups and merged (long contexts) instead of one workgroup per head
 };
 
 template <int D, bool APPEND>
@@ -984,7 +998,8 @@ int enqueue_rows(axq_model *m, const Rows &r) {
                                              c.sliding_window, m->pb_att);
             if (on_mfma < 0) return on_mfma;
         }
-        if (!on_mfma) launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st);
+        if (r.per_seq && r.split_attn) launch_attn_split(m, l, m->pb_qkv, nb, m->pb_att, st);
+        else if (!on_mfma) launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st);
         if ((rc = lin(m->w_o[l], m->pb_att, AXQ_X_PLAIN, nullptr, m->pb_h, m->pb_h))) return rc;
         if ((rc = lin(m->w_gu[l], m->pb_h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu))) return rc;
         if ((rc = lin(m->w_down[l], m->pb_gu, AXQ_X_SWIGLU, nullptr, m->pb_h, m->pb_h))) return rc;
@@ -1010,7 +1025,7 @@ int feed_rows(axq_model *m, int seq, const int32_t *toks, int n, int pos0, int *
     while (allow >= 1 && i < n) {
         const int left = n - i;
         Rows r;
-        r.mode = ROWS_NONE; r.toks = toks + i; r.per_seq = false; r.seq = seq; r.pos0 = pos0 + i;
+        r.mode = ROWS_NONE; r.toks = toks + i; r.per_seq = false; r.seq = seq; r.pos0 = pos0 + i; r.split_attn = false;
         // enough rows to fill GEMM tiles (fewer where the small-batch GEMV does not apply and single rows are the alternative)
         r.nb = left < PROMPT_CHUNK ? left : PROMPT_CHUNK;
         if (allow >= 2 && r.nb >= (all_layers_in_small_batch_reach(m, left) ? PROMPT_GEMM_MIN : PROMPT_BATCH) &&
@@ -1043,19 +1058,23 @@ int feed_prompt(axq_model *m, int base, int n_prompt) {
     return rc;
 }
 
-// One token of every sequence: a graph of its own, captured on first use.
-int run_batch_step(axq_model *m) {
+// One token of every sequence: graphs of their own, captured on first use.  max_pos_now: the largest position any
+// sequence feeds a token at in this step (contexts beyond m->fused_max take the split form of the attention).
+int run_batch_step(axq_model *m, int max_pos_now) {
     axq_ctx *ctx = m->ctx;
     Rows r;
     r.mode = ROWS_GEMV; r.toks = m->tok; r.nb = m->n_seq; r.per_seq = true; r.seq = 0; r.pos0 = 0;
-    // sized for the longest context, so that the launch can sit in a graph
-    r.lds = prompt_attn_lds(m, m->cfg.max_position_embeddings);
+    r.split_attn = max_pos_now >= m->fused_max;
+    // sized for the longest context this form serves, so that the launch can sit in a graph
+    r.lds = prompt_attn_lds(m, r.split_attn ? 1 : m->fused_max);
     static const bool no_graph = getenv("AXQ_DECODE_GRAPH") && getenv("AXQ_DECODE_GRAPH")[0] == '0';
     int rc;
     if (no_graph) {
         rc = enqueue_rows(m, r);
     } else {
-        if (!m->graph_b_ok) {
+        hipGraphExec_t &exec = r.split_attn ? m->graph_b : m->graph_bf;
+        bool &ok = r.split_attn ? m->graph_b_ok : m->graph_bf_ok;
+        if (!ok) {
             hipGraph_t g = nullptr;
             AXQ_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), AXQ_ERR_DRIVER);
             rc = enqueue_rows(m, r);
@@ -1065,12 +1084,12 @@ int run_batch_step(axq_model *m) {
                 return rc;
             }
             if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipStreamEndCapture: %s", hipGetErrorString(e));
-            e = hipGraphInstantiate(&m->graph_b, g, nullptr, nullptr, 0);
+            e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
             (void)hipGraphDestroy(g);
             if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipGraphInstantiate: %s", hipGetErrorString(e));
-            m->graph_b_ok = true;
+            ok = true;
         }
-        AXQ_HIP(ctx, hipGraphLaunch(m->graph_b, ctx->stream), AXQ_ERR_KERNEL_LAUNCH_FAILED);
+        AXQ_HIP(ctx, hipGraphLaunch(exec, ctx->stream), AXQ_ERR_KERNEL_LAUNCH_FAILED);
         rc = AXQ_OK;
     }
     if (rc || !m->sampling) return rc;
@@ -1137,7 +1156,8 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     TRY(dev_alloc(&m->rope_sin, (size_t)c.max_position_embeddings * c.head_dim / 2));
     TRY(dev_alloc(&m->kcache, kv)); TRY(dev_alloc(&m->vcache, kv));
     TRY(dev_alloc(&m->h, H)); TRY(dev_alloc(&m->xn, H)); TRY(dev_alloc(&m->qkv, m->qkv_rows)); TRY(dev_alloc(&m->att, m->q_dim));
-    TRY(dev_alloc(&m->att_part, (size_t)c.num_key_value_heads * m->max_splits * (c.num_attention_heads / c.num_key_value_heads) * (c.head_dim + 2)));
+    m->part_stride = (size_t)c.num_key_value_heads * m->max_splits * (c.num_attention_heads / c.num_key_value_heads) * (c.head_dim + 2);
+    TRY(dev_alloc(&m->att_part, m->part_stride));
     TRY(dev_alloc(&m->gu, (size_t)2 * I)); TRY(dev_alloc(&m->act, I)); TRY(dev_alloc(&m->logits, c.vocab_size));
     m->pb_cap = PROMPT_BATCH;
     TRY(dev_alloc(&m->pb_h, (size_t)PROMPT_BATCH * H)); TRY(dev_alloc(&m->pb_xn, (size_t)PROMPT_BATCH * (H > I ? H : I)));
@@ -1194,6 +1214,7 @@ void axq_model_free(axq_model *m) {
     if (m->graph_ok) (void)hipGraphExecDestroy(m->graph);
     if (m->graph_f_ok) (void)hipGraphExecDestroy(m->graph_f);
     if (m->graph_b_ok) (void)hipGraphExecDestroy(m->graph_b);
+    if (m->graph_bf_ok) (void)hipGraphExecDestroy(m->graph_bf);
     for (void *p : {(void *)m->bprompt, (void *)m->boffsets, (void *)m->bout})
         if (p) (void)hipFree(p);
     for (auto *w : m->w_qkv) axq_weight_free(ctx, w);
@@ -1350,10 +1371,11 @@ int axq_model_set_batch(axq_model *m, int n_seq) {
     if (m->graph_ok) (void)hipGraphExecDestroy(m->graph);
     if (m->graph_f_ok) (void)hipGraphExecDestroy(m->graph_f);
     if (m->graph_b_ok) (void)hipGraphExecDestroy(m->graph_b);
-    m->graph_ok = m->graph_f_ok = m->graph_b_ok = false;
+    if (m->graph_bf_ok) (void)hipGraphExecDestroy(m->graph_bf);
+    m->graph_ok = m->graph_f_ok = m->graph_b_ok = m->graph_bf_ok = false;
     const size_t P = c.max_position_embeddings, S = (size_t)n_seq;
     for (void **p : {(void **)&m->kcache, (void **)&m->vcache, (void **)&m->pos, (void **)&m->tok, (void **)&m->next, (void **)&m->hist,
-                     (void **)&m->logits, (void **)&m->bprompt, (void **)&m->boffsets, (void **)&m->bout}) {
+                     (void **)&m->logits, (void **)&m->bprompt, (void **)&m->boffsets, (void **)&m->bout, (void **)&m->att_part}) {
         if (*p) (void)hipFree(*p);
         *p = nullptr;
     }
@@ -1368,6 +1390,7 @@ int axq_model_set_batch(axq_model *m, int n_seq) {
     if (e == hipSuccess) e = dev_alloc(&m->bprompt, S * P);
     if (e == hipSuccess) e = dev_alloc(&m->boffsets, S + 1);
     if (e == hipSuccess) e = dev_alloc(&m->bout, S * m->out_cap);
+    if (e == hipSuccess) e = dev_alloc(&m->att_part, S * m->part_stride);
     if (e == hipSuccess) e = hipMemsetAsync(m->kcache, 0, S * m->seq_stride * 2, ctx->stream);
     if (e == hipSuccess) e = hipMemsetAsync(m->vcache, 0, S * m->seq_stride * 2, ctx->stream);
     if (e == hipSuccess) e = hipMemsetAsync(m->pos, 0, S * 4, ctx->stream);
@@ -1438,7 +1461,9 @@ int axq_model_forward_batch(axq_model *m, const int32_t *tokens, float *logits, 
     }
     AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
     AXQ_HIP(ctx, hipMemcpyAsync(m->tok, tokens, (size_t)S * 4, hipMemcpyHostToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
-    if ((rc = run_batch_step(m))) return rc;
+    int max_pos_now = 0;
+    for (int s = 0; s < S; s++) max_pos_now = m->seq_pos[s] > max_pos_now ? m->seq_pos[s] : max_pos_now;
+    if ((rc = run_batch_step(m, max_pos_now))) return rc;
     for (int s = 0; s < S; s++) m->seq_pos[s]++;
     m->host_pos = m->seq_pos[0];
     if (logits)
@@ -1492,8 +1517,10 @@ int axq_model_generate_batch(axq_model *m, const int32_t *prompts, const int32_t
     }
     if (!rc) last_tokens_kernel<<<1, S, 0, ctx->stream>>>(m->bprompt, m->boffsets, m->tok);
     (void)hipEventRecord(e1, ctx->stream);
+    int longest = 0;
+    for (int s = 0; s < S; s++) longest = offsets[s + 1] - offsets[s] > longest ? offsets[s + 1] - offsets[s] : longest;
     for (int i = 0; i < max_new_tokens && !rc; i++) {
-        rc = run_batch_step(m);
+        rc = run_batch_step(m, longest - 1 + i); // step i feeds sequence s its token at position n_s - 1 + i
         if (!rc) commit_rows_kernel<<<1, S, 0, ctx->stream>>>(m->next, m->tok, m->bout, i, m->out_cap);
     }
     (void)hipEventRecord(e2, ctx->stream);

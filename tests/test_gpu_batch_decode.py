@@ -209,3 +209,42 @@ def test_one_layer_at_the_7b_shape(ctx):
         assert got[s].tolist() == want, s
     gpu.close()
     cpu.close()
+
+
+@pytest.mark.parametrize("fused_max", ["0", "25", "1000"])
+def test_batched_steps_in_both_attention_forms(ctx, monkeypatch, fused_max):
+    """Short contexts: one attention workgroup per sequence and head; longer ones: the positions split over workgroups
+    and merged, for all sequences in one launch.  The switch-over (normally at 384 positions) is moved into the walk."""
+    monkeypatch.setenv("AXQ_ATTN_FUSED_MAX", fused_max)
+    c = tiny_config(max_seq_len=80)
+    w = random_weights(c, 340)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    gpu.set_batch(5)
+    rng = np.random.default_rng(8)
+    prompts = [rng.integers(0, c["vocab_size"], size=n) for n in (3, 22, 40, 1, 17)]
+    got, _, _ = gpu.generate_batch(prompts, 20)
+    for s, p in enumerate(prompts):
+        want, _ = _oracle_walk(cpu, p, 20)
+        assert got[s].tolist() == want, s
+    # logits of single batched steps on top of that, sequences at different positions on both sides of the switch
+    toks = got[:, -1].tolist()
+    pos = [len(p) + 19 for p in prompts]
+    cpus = []
+    for s, p in enumerate(prompts):
+        m = load_oracle(c, w)
+        seq = list(p) + got[s, :-1].tolist()
+        for i, t in enumerate(seq):
+            m.forward(int(t), i)
+        cpus.append(m)
+    for step in range(3):
+        g_next, g_logits = gpu.forward_batch(toks)
+        for s in range(5):
+            c_next, c_logits = cpus[s].forward(int(toks[s]), pos[s])
+            assert max_rel_err(g_logits[s], c_logits, DECODE_FLOOR) <= DECODE_RTOL, (step, s)
+            assert g_next[s] == c_next
+            pos[s] += 1
+        toks = g_next.tolist()
+    gpu.close()
+    cpu.close()
+    for m in cpus:
+        m.close()
