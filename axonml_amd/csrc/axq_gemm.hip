@@ -18,6 +18,8 @@
 // feed (see gemm_kernel).
 #include <hip/hip_fp16.h>
 
+#include <stdlib.h>
+
 #include "axq_internal.h"
 
 namespace {
@@ -43,6 +45,7 @@ struct GemmArgs {
     // are added into output row t (+ bias[n] + resid[t, n]); y, ypart and resid then have m / 2 rows
     int pair;
     const float *bias, *resid;
+    int wm;                // 1: 128-row tiles, 2: 256-row tiles
 };
 
 __device__ inline float h2f(uint32_t bits) { return __half2float(__ushort_as_half((unsigned short)bits)); }
@@ -477,7 +480,7 @@ __global__ void __launch_bounds__(256) gemm_reduce_kernel(const float *ypart, co
 template <class T>
 int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
     static bool attr_set = false;
-    const int wm = a.m > 128 ? 2 : 1, bm = 128 * wm;
+    const int wm = a.wm, bm = 128 * wm;
     const unsigned tiles = (unsigned)(((a.n + BN - 1) / BN) * ((a.m + bm - 1) / bm));
     const dim3 grid(tiles, (unsigned)splits);
     const size_t lds = (size_t)2 * (bm + 2 * BN) * LDK * sizeof(_Float16); // two stages
@@ -607,7 +610,7 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
 }
 
 struct GemmPlan {
-    int splits, steps_per_split;
+    int splits, steps_per_split, wm;
     size_t xh_bytes, rs_bytes, part_bytes;
 };
 
@@ -620,7 +623,9 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, size_t extra, GemmPlan *
                         (long long)w->k);
     if (w->n_rows > INT32_MAX || w->k > INT32_MAX)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
-    const int bm = m > 128 ? 256 : 128;
+    static const int bm_knob = getenv("AXQ_GEMM_BM") ? atoi(getenv("AXQ_GEMM_BM")) : 0; // development knob: 128 or 256 for every shape
+    const int bm = bm_knob ? bm_knob : (m > 128 ? 256 : 128);
+    p->wm = bm / 128;
     const long tiles = (long)((w->n_rows + BN - 1) / BN) * ((m + bm - 1) / bm);
     const int ksteps = (int)(w->k / BK), cus = ctx->prop.multiProcessorCount;
     int splits = (int)(cus / tiles);
@@ -655,7 +660,7 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     a.ypart = p.splits > 1 ? reinterpret_cast<float *>(base + p.xh_bytes + p.rs_bytes) : nullptr;
     a.m = m; a.n = (int)w->n_rows; a.k = (int)w->k;
     a.steps_per_split = p.steps_per_split;
-    a.pair = pair ? 1 : 0; a.bias = bias; a.resid = resid;
+    a.pair = pair ? 1 : 0; a.bias = bias; a.resid = resid; a.wm = p.wm;
     switch (w->type) {
     case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);
     case AXQ_Q4_0: return launch_gemm<GQ4x<false>>(ctx, a, p.splits);
