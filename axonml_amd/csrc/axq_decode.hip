@@ -65,6 +65,7 @@ struct axq_model {
     hipGraphExec_t graph_f;         // the same with one attention workgroup per head (short contexts)
     bool graph_f_ok;
     int fused_max;                  // contexts up to this many positions take graph_f
+    bool attn_mfma;                 // prompt attention of many rows on the matrix pipe (development knob AXQ_ATTN_MFMA=0: off)
 };
 
 namespace {
@@ -893,11 +894,6 @@ int reserve_prompt_rows(axq_model *m, int cap) {
     return AXQ_OK;
 }
 
-bool attn_mfma_allowed() {
-    static const bool off = getenv("AXQ_ATTN_MFMA") && getenv("AXQ_ATTN_MFMA")[0] == '0'; // development knob
-    return !off;
-}
-
 // What a call of enqueue_rows works on.
 struct Rows {
     int mode;            // ROWS_GEMV or ROWS_GEMM
@@ -992,7 +988,7 @@ int enqueue_rows(axq_model *m, const Rows &r) {
                 m->seq_stride, c.max_position_embeddings, d);
         // many rows of one sequence: attention on the matrix pipe, a tile of rows against every key once
         int on_mfma = 0;
-        if (!r.per_seq && nb >= PROMPT_GEMM_MIN && attn_mfma_allowed()) {
+        if (!r.per_seq && nb >= PROMPT_GEMM_MIN && m->attn_mfma) {
             on_mfma = axq_dev_attn_rows_mfma(ctx, m->pb_qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0,
                                              nb, c.num_attention_heads, c.num_key_value_heads, d, c.max_position_embeddings,
                                              c.sliding_window, m->pb_att);
@@ -1139,6 +1135,7 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
         const char *knob = getenv("AXQ_ATTN_FUSED_MAX"); // development knob: 0 = always split the positions
         m->fused_max = knob ? atoi(knob) : 384; // measured at the 7B shape: 670 against 645 tokens/s up to 224 positions, even at 384, behind from 512
         if (m->fused_max > 32768) m->fused_max = 32768;
+        m->attn_mfma = !(getenv("AXQ_ATTN_MFMA") && getenv("AXQ_ATTN_MFMA")[0] == '0');
     }
     m->n_seq = 1;
     m->seq_stride = (size_t)c.num_hidden_layers * c.num_key_value_heads * c.max_position_embeddings * c.head_dim;

@@ -236,3 +236,30 @@ def test_error_paths(ctx):
         m.forward(1, want_logits=False)
     with pytest.raises(q.Overflow):  # cache full
         m.forward(1)
+
+
+@pytest.mark.parametrize("over,n_first,n_prompt", [(dict(max_seq_len=400), 0, 390), (dict(max_seq_len=400, sliding_window=70), 11, 300),
+                                                    (dict(max_seq_len=300, num_heads=8, num_kv_heads=1, head_dim=32), 3, 257),
+                                                    (dict(max_seq_len=300, num_heads=2, num_kv_heads=2, head_dim=128), 0, 33)])
+def test_the_two_prompt_attention_kernels_agree(ctx, monkeypatch, over, n_first, n_prompt):
+    """The matrix-pipe attention of prompt rows against the per-query kernel on the same model and tokens: last logits,
+    hidden state and the KV cache (rows written by layer 2 depend on layer 1's attention output)."""
+    c = tiny_config(num_layers=3, **over)
+    w = random_weights(c, 99)
+    toks = np.random.default_rng(n_prompt).integers(0, c["vocab_size"], size=n_first + n_prompt)
+    out = []
+    for knob in ("1", "0"):
+        monkeypatch.setenv("AXQ_ATTN_MFMA", knob)
+        m = load_gpu(ctx, c, w)
+        for t in toks[:n_first]:
+            m.forward(int(t), want_logits=False)
+        nxt, logits = m.forward_tokens(toks[n_first:])
+        out.append((nxt, logits, m.hidden(), [m.kv(l, which)[:, :len(toks)].copy() for l in range(3) for which in (0, 1)]))
+        m.close()
+    (n1, l1, h1, kv1), (n0, l0, h0, kv0) = out
+    assert n1 == n0
+    assert max_rel_err(l1, l0, DECODE_FLOOR) <= 1e-4   # both are f32-accurate: they agree far inside the decode bar
+    assert max_rel_err(h1, h0, 1e-2) <= 2e-3   # an f16 cache element that rounds the other way moves the last layers by about 1e-5
+    for a, b in zip(kv1, kv0):
+        af, bf = a.view(np.float16).astype(np.float64), b.view(np.float16).astype(np.float64)
+        assert np.abs(af - bf).max() <= 2.0 ** -9 * np.abs(af).max()  # isolated one-ulp f16 roundings at most
