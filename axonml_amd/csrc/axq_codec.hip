@@ -48,8 +48,22 @@ __device__ inline void store_u16(uint8_t *p, uint16_t v) { *reinterpret_cast<uin
 __device__ inline uint16_t load_u16(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
 
 // ---- Q8_0: quantize.rs:82-114, image types.rs:142-147 ---------------------
-// The 34-byte images of a workgroup's 128 blocks are put together in LDS and leave as one run of 16-byte stores
-// (a thread writing its own image would store 2 bytes at a time, 34 bytes from its neighbour's).
+// The images of a workgroup's 128 blocks are put together in LDS and leave as one run of 16-byte stores (a thread
+// writing its own image would store 2 bytes at a time, IMG bytes from its neighbour's).  Called by every thread of
+// the workgroup; 128 * IMG is a multiple of 16, so the run is as aligned as `out`.
+template <int IMG>
+__device__ inline void flush_images(const uint8_t *img, uint8_t *out, size_t b0, size_t nblk) {
+    __syncthreads();
+    const int nb = nblk - b0 < 128 ? (int)(nblk - b0) : 128, nbytes = nb * IMG;
+    uint8_t *g = out + b0 * IMG;
+    if ((reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        for (int o = threadIdx.x * 16; o + 16 <= nbytes; o += 128 * 16) *reinterpret_cast<uint4 *>(g + o) = *reinterpret_cast<const uint4 *>(img + o);
+        for (int o = (nbytes & ~15) + threadIdx.x * 2; o < nbytes; o += 256) store_u16(g + o, load_u16(img + o));
+    } else {
+        for (int o = threadIdx.x * 2; o < nbytes; o += 256) store_u16(g + o, load_u16(img + o));
+    }
+}
+
 __global__ void __launch_bounds__(128) quant_q8_0_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
     __shared__ __attribute__((aligned(16))) uint8_t img[128 * 34];
     const size_t b0 = (size_t)blockIdx.x * 128, b = b0 + threadIdx.x;
@@ -71,132 +85,133 @@ __global__ void __launch_bounds__(128) quant_q8_0_kernel(const float *src, size_
             store_u16(o + 2 + 2 * i, (uint16_t)((q0 & 0xFF) | ((q1 & 0xFF) << 8)));
         }
     }
-    __syncthreads();
-    const int nb = nblk - b0 < 128 ? (int)(nblk - b0) : 128, nbytes = nb * 34;
-    uint8_t *g = out + b0 * 34; // 128 * 34 is a multiple of 16: as aligned as `out`
-    if ((reinterpret_cast<uintptr_t>(out) & 15) == 0) {
-        for (int o = threadIdx.x * 16; o + 16 <= nbytes; o += 128 * 16) *reinterpret_cast<uint4 *>(g + o) = *reinterpret_cast<const uint4 *>(img + o);
-        for (int o = (nbytes & ~15) + threadIdx.x * 2; o < nbytes; o += 256) store_u16(g + o, load_u16(img + o));
-    } else {
-        for (int o = threadIdx.x * 2; o < nbytes; o += 256) store_u16(g + o, load_u16(img + o));
-    }
+    flush_images<34>(img, out, b0, nblk);
 }
 
 // ---- Q4_0: quantize.rs:121-156, pack types.rs:190-198 ---------------------
-__global__ void quant_q4_0_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
-    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= nblk) return;
-    float x[32];
-    int len;
-    load_block32(src, numel, b, x, len);
-    float max_abs = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 32; i++)
-        if (i < len) max_abs = fmaxf(max_abs, fabsf(x[i]));
-    float scale = max_abs > 0.0f ? max_abs / 7.0f : 1.0f;
-    uint8_t *o = out + b * 18;
-    store_u16(o, f32_to_f16_bits(scale));
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        uint32_t w = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            int e = 4 * i + j;
-            int q = e < len ? round_clamp(x[e] / scale, -8.0f, 7.0f) : 0;
-            w |= (uint32_t)((q + 8) & 0x0F) << (4 * j);
-        }
-        store_u16(o + 2 + 2 * i, (uint16_t)w);
-    }
-}
-
-// ---- Q4_1: quantize.rs:163-205, image types.rs:249-255 --------------------
-__global__ void quant_q4_1_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
-    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= nblk) return;
-    float x[32];
-    int len;
-    load_block32(src, numel, b, x, len);
-    float mn = INFINITY, mx = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 32; i++)
-        if (i < len) {
-            mn = fminf(mn, x[i]);
-            mx = fmaxf(mx, x[i]);
-        }
-    float scale = mx > mn ? (mx - mn) / 15.0f : 1.0f;
-    uint8_t *o = out + b * 20;
-    store_u16(o, f32_to_f16_bits(scale));
-    store_u16(o + 2, f32_to_f16_bits(mn));
-    int nbytes = len / 2 < 16 ? len / 2 : 16; // the reference's pack loop bound
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        uint32_t w = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            int e = 4 * i + j;
-            int q = e < len ? round_clamp((x[e] - mn) / scale, 0.0f, 15.0f) : 0;
-            if ((e >> 1) >= nbytes) q = 0;
-            w |= (uint32_t)(q & 0x0F) << (4 * j);
-        }
-        store_u16(o + 4 + 2 * i, (uint16_t)w);
-    }
-}
-
-// ---- Q5_0 / Q5_1: GGUF layouts; scale rules max_abs/15 and (max-min)/31 ---
-template <bool WITH_MIN>
-__global__ void quant_q5_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
-    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= nblk) return;
-    float x[32];
-    int len;
-    load_block32(src, numel, b, x, len);
-    float scale, mn = 0.0f;
-    if (WITH_MIN) {
-        float lo = INFINITY, hi = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 32; i++)
-            if (i < len) {
-                lo = fminf(lo, x[i]);
-                hi = fmaxf(hi, x[i]);
-            }
-        scale = hi > lo ? (hi - lo) / 31.0f : 1.0f;
-        mn = lo;
-    } else {
+__global__ void __launch_bounds__(128) quant_q4_0_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
+    __shared__ __attribute__((aligned(16))) uint8_t img[128 * 18];
+    const size_t b0 = (size_t)blockIdx.x * 128, b = b0 + threadIdx.x;
+    if (b < nblk) {
+        float x[32];
+        int len;
+        load_block32(src, numel, b, x, len);
         float max_abs = 0.0f;
 #pragma unroll
         for (int i = 0; i < 32; i++)
             if (i < len) max_abs = fmaxf(max_abs, fabsf(x[i]));
-        scale = max_abs > 0.0f ? max_abs / 15.0f : 1.0f;
-    }
-    uint32_t u[32];
+        float scale = max_abs > 0.0f ? max_abs / 7.0f : 1.0f;
+        uint8_t *o = img + threadIdx.x * 18;
+        store_u16(o, f32_to_f16_bits(scale));
 #pragma unroll
-    for (int i = 0; i < 32; i++) {
-        if (WITH_MIN)
-            u[i] = i < len ? (uint32_t)round_clamp((x[i] - mn) / scale, 0.0f, 31.0f) : 0u;
-        else
-            u[i] = i < len ? (uint32_t)(round_clamp(x[i] / scale, -16.0f, 15.0f) + 16) : 16u;
+        for (int i = 0; i < 8; i++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                int e = 4 * i + j;
+                int q = e < len ? round_clamp(x[e] / scale, -8.0f, 7.0f) : 0;
+                w |= (uint32_t)((q + 8) & 0x0F) << (4 * j);
+            }
+            store_u16(o + 2 + 2 * i, (uint16_t)w);
+        }
     }
-    uint8_t *o = out + b * (WITH_MIN ? 24 : 22);
-    store_u16(o, f32_to_f16_bits(scale));
-    int off = 2;
-    if (WITH_MIN) {
+    flush_images<18>(img, out, b0, nblk);
+}
+
+// ---- Q4_1: quantize.rs:163-205, image types.rs:249-255 --------------------
+__global__ void __launch_bounds__(128) quant_q4_1_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
+    __shared__ __attribute__((aligned(16))) uint8_t img[128 * 20];
+    const size_t b0 = (size_t)blockIdx.x * 128, b = b0 + threadIdx.x;
+    if (b < nblk) {
+        float x[32];
+        int len;
+        load_block32(src, numel, b, x, len);
+        float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 32; i++)
+            if (i < len) {
+                mn = fminf(mn, x[i]);
+                mx = fmaxf(mx, x[i]);
+            }
+        float scale = mx > mn ? (mx - mn) / 15.0f : 1.0f;
+        uint8_t *o = img + threadIdx.x * 20;
+        store_u16(o, f32_to_f16_bits(scale));
         store_u16(o + 2, f32_to_f16_bits(mn));
-        off = 4;
-    }
-    uint32_t qh = 0;
+        int nbytes = len / 2 < 16 ? len / 2 : 16; // the reference's pack loop bound
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
-        qh |= ((u[j] >> 4) & 1u) << j;
-        qh |= ((u[j + 16] >> 4) & 1u) << (j + 16);
-    }
-    store_u16(o + off, (uint16_t)qh);
-    store_u16(o + off + 2, (uint16_t)(qh >> 16));
+        for (int i = 0; i < 8; i++) {
+            uint32_t w = 0;
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-        uint32_t b0 = (u[2 * j] & 0x0F) | ((u[2 * j + 16] & 0x0F) << 4);
-        uint32_t b1 = (u[2 * j + 1] & 0x0F) | ((u[2 * j + 17] & 0x0F) << 4);
-        store_u16(o + off + 4 + 2 * j, (uint16_t)(b0 | (b1 << 8)));
+            for (int j = 0; j < 4; j++) {
+                int e = 4 * i + j;
+                int q = e < len ? round_clamp((x[e] - mn) / scale, 0.0f, 15.0f) : 0;
+                if ((e >> 1) >= nbytes) q = 0;
+                w |= (uint32_t)(q & 0x0F) << (4 * j);
+            }
+            store_u16(o + 4 + 2 * i, (uint16_t)w);
+        }
     }
+    flush_images<20>(img, out, b0, nblk);
+}
+
+// ---- Q5_0 / Q5_1: GGUF layouts; scale rules max_abs/15 and (max-min)/31 ---
+template <bool WITH_MIN>
+__global__ void __launch_bounds__(128) quant_q5_kernel(const float *src, size_t numel, size_t nblk, uint8_t *out) {
+    __shared__ __attribute__((aligned(16))) uint8_t img[128 * 24];
+    const size_t b0 = (size_t)blockIdx.x * 128, b = b0 + threadIdx.x;
+    if (b < nblk) {
+        float x[32];
+        int len;
+        load_block32(src, numel, b, x, len);
+        float scale, mn = 0.0f;
+        if (WITH_MIN) {
+            float lo = INFINITY, hi = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 32; i++)
+                if (i < len) {
+                    lo = fminf(lo, x[i]);
+                    hi = fmaxf(hi, x[i]);
+                }
+            scale = hi > lo ? (hi - lo) / 31.0f : 1.0f;
+            mn = lo;
+        } else {
+            float max_abs = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; i++)
+                if (i < len) max_abs = fmaxf(max_abs, fabsf(x[i]));
+            scale = max_abs > 0.0f ? max_abs / 15.0f : 1.0f;
+        }
+        uint32_t u[32];
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            if (WITH_MIN)
+                u[i] = i < len ? (uint32_t)round_clamp((x[i] - mn) / scale, 0.0f, 31.0f) : 0u;
+            else
+                u[i] = i < len ? (uint32_t)(round_clamp(x[i] / scale, -16.0f, 15.0f) + 16) : 16u;
+        }
+        uint8_t *o = img + threadIdx.x * (WITH_MIN ? 24 : 22);
+        store_u16(o, f32_to_f16_bits(scale));
+        int off = 2;
+        if (WITH_MIN) {
+            store_u16(o + 2, f32_to_f16_bits(mn));
+            off = 4;
+        }
+        uint32_t qh = 0;
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            qh |= ((u[j] >> 4) & 1u) << j;
+            qh |= ((u[j + 16] >> 4) & 1u) << (j + 16);
+        }
+        store_u16(o + off, (uint16_t)qh);
+        store_u16(o + off + 2, (uint16_t)(qh >> 16));
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            uint32_t b0 = (u[2 * j] & 0x0F) | ((u[2 * j + 16] & 0x0F) << 4);
+            uint32_t b1 = (u[2 * j + 1] & 0x0F) | ((u[2 * j + 17] & 0x0F) << 4);
+            store_u16(o + off + 4 + 2 * j, (uint16_t)(b0 | (b1 << 8)));
+        }
+    }
+    flush_images<(WITH_MIN ? 24 : 22)>(img, out, b0, nblk);
 }
 
 // ---- Q4_K: one lane per 32-element sub-block, 8 lanes per superblock -------
