@@ -952,9 +952,20 @@ int enqueue_rows(axq_model *m, const Rows &r) {
     int rc;
     // y = f(x) W^T (+ resid): f = RMSNorm with weights aux, or SwiGLU over the gate/up rows in x, or nothing.  The
     // small-batch GEMV applies f while it packs x; elsewhere f runs as a kernel of its own (the GEMM normalises itself).
-    auto lin = [&](const axq_weight *w, const float *x, int xmode, const float *aux, const float *resid, float *y) -> int {
+    // `next` (with RMSNorm weights next_aux): the linear that takes y next; where both are small-batch GEMVs, the first
+    // one's reduction prepares the second one's operands, which then skips its own packing.
+    const axq_weight *packed_for = nullptr; // the weight whose operands the GEMV scratch holds, if any
+    auto lin = [&](const axq_weight *w, const float *x, int xmode, const float *aux, const float *resid, float *y, const axq_weight *next,
+                   const float *next_aux) -> int {
         const bool batch_kernel = r.mode == ROWS_GEMV && axq_dev_gemv_batch_covers(w, nb);
-        if (batch_kernel) return axq_dev_gemv_batch_ex(ctx, w, x, xmode, aux, c.rms_norm_eps, nb, nullptr, resid, y);
+        if (batch_kernel) {
+            const bool ready = packed_for == w;
+            const bool chain = next && axq_dev_gemv_batch_covers(next, nb);
+            packed_for = chain ? next : nullptr;
+            return axq_dev_gemv_batch_chain(ctx, w, x, ready ? AXQ_X_PACKED : xmode, aux, c.rms_norm_eps, nb, nullptr, resid, y,
+                                            chain ? next : nullptr, chain ? next_aux : nullptr);
+        }
+        packed_for = nullptr;
         if (xmode == AXQ_X_SWIGLU) {
             swiglu_kernel<<<dim3((I / 4 + 255) / 256, nb), 256, 0, st>>>(x, I, m->pb_act);
             x = m->pb_act;
@@ -981,7 +992,7 @@ int enqueue_rows(axq_model *m, const Rows &r) {
     embed_kernel<<<dim3((H / 8 + 255) / 256, nb), 256, 0, st>>>(m->emb, r.toks, m->pb_h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
         const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * d + seq_off;
-        if ((rc = lin(m->w_qkv[l], m->pb_h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv))) return rc;
+        if ((rc = lin(m->w_qkv[l], m->pb_h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv, nullptr, nullptr))) return rc;
         if (!r.per_seq)
             rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
                 m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0, nullptr,
@@ -996,9 +1007,10 @@ int enqueue_rows(axq_model *m, const Rows &r) {
         }
         if (r.per_seq && r.split_attn) launch_attn_split(m, l, m->pb_qkv, nb, m->pb_att, st);
         else if (!on_mfma) launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st);
-        if ((rc = lin(m->w_o[l], m->pb_att, AXQ_X_PLAIN, nullptr, m->pb_h, m->pb_h))) return rc;
-        if ((rc = lin(m->w_gu[l], m->pb_h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu))) return rc;
-        if ((rc = lin(m->w_down[l], m->pb_gu, AXQ_X_SWIGLU, nullptr, m->pb_h, m->pb_h))) return rc;
+        if ((rc = lin(m->w_o[l], m->pb_att, AXQ_X_PLAIN, nullptr, m->pb_h, m->pb_h, m->w_gu[l], m->norm_ffn + (size_t)l * H))) return rc;
+        if ((rc = lin(m->w_gu[l], m->pb_h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu, nullptr, nullptr))) return rc;
+        if ((rc = lin(m->w_down[l], m->pb_gu, AXQ_X_SWIGLU, nullptr, m->pb_h, m->pb_h, l + 1 < c.num_hidden_layers ? m->w_qkv[l + 1] : nullptr,
+                      m->norm_attn + (size_t)(l + 1 < c.num_hidden_layers ? l + 1 : l) * H))) return rc;
     }
     if (r.per_seq) {
         norm_kernel<<<nb, 1024, 0, st>>>(m->pb_h, m->norm_final, H, c.rms_norm_eps, m->pb_xn);

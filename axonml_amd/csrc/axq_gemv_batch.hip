@@ -280,6 +280,37 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
     }
 }
 
+// Eight consecutive elements (task t) of vector b -> their limbs in the A operands and, from the first task of a
+// 32-element block, the block's scale and sum.  The four tasks of a block sit in four consecutive lanes, which
+// all have to call this together.
+template <bool EVEN_ODD>
+__device__ inline void store_packed(const float (&v)[8], int t, int b, int batch, int nblk, uint8_t *xa, float *xsg) {
+    uint32_t pk[4][2];
+    float sg, sum;
+    int ls[4];
+    axq_split8_compute(v, pk, sg, sum, ls);
+    if (b >= batch) { sg = 0.f; sum = 0.f; }
+    const int blk = t >> 2, e0 = (t & 3) * 8; // first element of the task inside its block
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+        const int row = 4 * b + l;
+        if (EVEN_ODD) {
+            uint8_t *d0 = xa + ((size_t)(blk * 2 + 0) * 32 + row) * 16 + (e0 >> 1);
+            uint8_t *d1 = xa + ((size_t)(blk * 2 + 1) * 32 + row) * 16 + (e0 >> 1);
+            *reinterpret_cast<uint32_t *>(d0) = (uint32_t)pick_alt(pk[l][0], pk[l][1], 0);
+            *reinterpret_cast<uint32_t *>(d1) = (uint32_t)pick_alt(pk[l][0], pk[l][1], 1);
+        } else {
+            uint8_t *d = xa + ((size_t)(blk * 2 + (e0 >> 4)) * 32 + row) * 16 + (e0 & 15);
+            *reinterpret_cast<uint2 *>(d) = make_uint2(pk[l][0], pk[l][1]);
+        }
+    }
+    if ((t & 3) == 0) {
+        const int slot = (blk * 2 + (b & 1)) * 4 + (b >> 1);
+        xsg[slot] = sg;
+        xsg[(size_t)nblk * 8 + slot] = sum;
+    }
+}
+
 // f(x)[batch, k] -> A operands and group records.  Thread = (8-element task, vector b); vectors beyond the batch
 // are written as zeros.  EVEN_ODD: the h = 0 half of a block's operand holds its even elements, h = 1 the odd.
 // XMODE: AXQ_X_PLAIN; AXQ_X_RMSNORM: f = x / sqrt(mean(x^2) + eps) * aux (every workgroup sums its vector's squares
@@ -332,30 +363,7 @@ __global__ void __launch_bounds__(256) pack_x_kernel(const float *x, const float
             }
         }
     }
-    uint32_t pk[4][2];
-    float sg, sum;
-    int ls[4];
-    axq_split8_compute(v, pk, sg, sum, ls);
-    if (b >= batch) { sg = 0.f; sum = 0.f; }
-    const int blk = t >> 2, e0 = (t & 3) * 8; // first element of the task inside its block
-#pragma unroll
-    for (int l = 0; l < 4; l++) {
-        const int row = 4 * b + l;
-        if (EVEN_ODD) {
-            uint8_t *d0 = xa + ((size_t)(blk * 2 + 0) * 32 + row) * 16 + (e0 >> 1);
-            uint8_t *d1 = xa + ((size_t)(blk * 2 + 1) * 32 + row) * 16 + (e0 >> 1);
-            *reinterpret_cast<uint32_t *>(d0) = (uint32_t)pick_alt(pk[l][0], pk[l][1], 0);
-            *reinterpret_cast<uint32_t *>(d1) = (uint32_t)pick_alt(pk[l][0], pk[l][1], 1);
-        } else {
-            uint8_t *d = xa + ((size_t)(blk * 2 + (e0 >> 4)) * 32 + row) * 16 + (e0 & 15);
-            *reinterpret_cast<uint2 *>(d) = make_uint2(pk[l][0], pk[l][1]);
-        }
-    }
-    if ((t & 3) == 0) {
-        const int slot = (blk * 2 + (b & 1)) * 4 + (b >> 1);
-        xsg[slot] = sg;
-        xsg[(size_t)nblk * 8 + slot] = sum;
-    }
+    store_packed<EVEN_ODD>(v, t, b, batch, nblk, xa, xsg);
 }
 
 // y = sum over the splits, in order (+ bias, + resid)
@@ -370,12 +378,92 @@ __global__ void __launch_bounds__(256) mb_reduce_kernel(const float *ypart, cons
     y[i] = tot;
 }
 
+// The same reduction for a result that is the input of the next small-batch GEMV (its n_rows are that GEMV's k):
+// one workgroup per vector adds the splits (+ bias, + resid), writes y, and goes on to what pack_x_kernel would do
+// with y next (RMSNorm with the weights next_aux when those are given, then the split into limbs), with the row in
+// registers in between.  splits = 0: `src` is the finished y already.  n <= 16384, a multiple of 256.
+template <bool EVEN_ODD>
+__global__ void __launch_bounds__(512) mb_reduce_pack_kernel(const float *src, int splits, const float *bias, const float *resid, int n,
+                                                             int batch, float *y, const float *next_aux, float eps, uint8_t *xa,
+                                                             float *xsg) {
+    constexpr int TPT = 4; // tasks of eight elements per thread
+    __shared__ float red[8];
+    const int b = blockIdx.x, ntask = n >> 3, nblk = n >> 5;
+    const size_t total = (size_t)n * batch;
+    float v[TPT][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int q = 0; q < TPT; q++) {
+        const int t = q * 512 + (int)threadIdx.x;
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[q][i] = 0.f;
+        if (t < ntask && b < batch) {
+            const size_t at = (size_t)b * n + (size_t)t * 8;
+            const float4 *p = reinterpret_cast<const float4 *>(src + at);
+            float4 a0 = p[0], a1 = p[1];
+            for (int z = 1; z < splits; z++) {
+                const float4 *pz = reinterpret_cast<const float4 *>(src + (size_t)z * total + at);
+                const float4 c0 = pz[0], c1 = pz[1];
+                a0.x += c0.x; a0.y += c0.y; a0.z += c0.z; a0.w += c0.w;
+                a1.x += c1.x; a1.y += c1.y; a1.z += c1.z; a1.w += c1.w;
+            }
+            if (splits > 0) {
+                if (bias) {
+                    const float *pb = bias + (size_t)t * 8;
+                    a0.x += pb[0]; a0.y += pb[1]; a0.z += pb[2]; a0.w += pb[3];
+                    a1.x += pb[4]; a1.y += pb[5]; a1.z += pb[6]; a1.w += pb[7];
+                }
+                if (resid) {
+                    const float4 *pr = reinterpret_cast<const float4 *>(resid + at);
+                    const float4 r0 = pr[0], r1 = pr[1];
+                    a0.x += r0.x; a0.y += r0.y; a0.z += r0.z; a0.w += r0.w;
+                    a1.x += r1.x; a1.y += r1.y; a1.z += r1.z; a1.w += r1.w;
+                }
+                reinterpret_cast<float4 *>(y + at)[0] = a0;
+                reinterpret_cast<float4 *>(y + at)[1] = a1;
+            }
+            v[q][0] = a0.x; v[q][1] = a0.y; v[q][2] = a0.z; v[q][3] = a0.w;
+            v[q][4] = a1.x; v[q][5] = a1.y; v[q][6] = a1.z; v[q][7] = a1.w;
+#pragma unroll
+            for (int i = 0; i < 8; i++) ss = fmaf(v[q][i], v[q][i], ss);
+        }
+    }
+    if (next_aux) { // RMSNorm of the whole row (RMSNorm::forward, llm/src/llama.rs:158-187)
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        ss = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
+        const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll
+        for (int q = 0; q < TPT; q++) {
+            const int t = q * 512 + (int)threadIdx.x;
+            if (t < ntask && b < batch) {
+                const float4 *pw = reinterpret_cast<const float4 *>(next_aux + (size_t)t * 8);
+                const float4 w0 = pw[0], w1 = pw[1];
+                const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[q][i] = (v[q][i] * inv) * wv[i];
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < TPT; q++) {
+        const int t = q * 512 + (int)threadIdx.x;
+        if (t < ntask) store_packed<EVEN_ODD>(v[q], t, b, batch, nblk, xa, xsg); // ntask is a multiple of 4: whole quads
+    }
+}
+
+// next_even_odd < 0: nothing follows.  Otherwise y is the input of another small-batch GEMV whose operands
+// (EVEN_ODD as given, RMSNorm with next_aux when that is not null) are prepared here, in the same scratch.
 template <class T>
-void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *aux, float eps) {
+void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *aux, float eps, int next_even_odd, const float *next_aux) {
     const dim3 pgrid((unsigned)((a.k / 8 + 255) / 256), MAX_BATCH);
     uint8_t *xa = const_cast<uint8_t *>(a.xa);
     float *xsg = const_cast<float *>(a.xsg);
-    if (xmode == AXQ_X_RMSNORM) pack_x_kernel<T::EVEN_ODD, AXQ_X_RMSNORM><<<pgrid, 256, 0, ctx->stream>>>(x, aux, eps, a.k, a.batch, xa, xsg);
+    if (xmode == AXQ_X_PACKED) {
+        // the operands are in place already (the previous call prepared them)
+    } else if (xmode == AXQ_X_RMSNORM) pack_x_kernel<T::EVEN_ODD, AXQ_X_RMSNORM><<<pgrid, 256, 0, ctx->stream>>>(x, aux, eps, a.k, a.batch, xa, xsg);
     else if (xmode == AXQ_X_SWIGLU) pack_x_kernel<T::EVEN_ODD, AXQ_X_SWIGLU><<<pgrid, 256, 0, ctx->stream>>>(x, aux, eps, a.k, a.batch, xa, xsg);
     else pack_x_kernel<T::EVEN_ODD, AXQ_X_PLAIN><<<pgrid, 256, 0, ctx->stream>>>(x, aux, eps, a.k, a.batch, xa, xsg);
     const unsigned chunks = (unsigned)((a.k + WAVE_K - 1) / WAVE_K);
@@ -397,7 +485,17 @@ void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *a
         big_lds_allowed = true;
     }
     gemv_mb_kernel<T><<<dim3(tiles, splits), 64 * S, lds, ctx->stream>>>(a);
-    if (splits > 1) {
+    if (next_even_odd >= 0) {
+        // y's operands for the next GEMV (k' = n_rows): the scratch layout of that call
+        uint8_t *nxa = ctx->xq;
+        float *nxsg = reinterpret_cast<float *>(ctx->xq + (size_t)32 * a.n_rows);
+        const float *src = splits > 1 ? a.ypart : a.y;
+        const int nsp = splits > 1 ? (int)splits : 0;
+        if (next_even_odd)
+            mb_reduce_pack_kernel<true><<<MAX_BATCH, 512, 0, ctx->stream>>>(src, nsp, a.bias, a.resid, a.n_rows, a.batch, a.y, next_aux, eps, nxa, nxsg);
+        else
+            mb_reduce_pack_kernel<false><<<MAX_BATCH, 512, 0, ctx->stream>>>(src, nsp, a.bias, a.resid, a.n_rows, a.batch, a.y, next_aux, eps, nxa, nxsg);
+    } else if (splits > 1) {
         const int total = a.n_rows * a.batch;
         mb_reduce_kernel<<<(total + 255) / 256, 256, 0, ctx->stream>>>(a.ypart, a.bias, a.resid, a.n_rows, a.batch, (int)splits, a.y);
     }
@@ -420,7 +518,21 @@ int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int ba
 // 2 <= batch <= 8: split the batch (f = xmode, see pack_x_kernel), then one pass over W.
 int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
                           const float *bias, const float *resid, float *y) {
+    return axq_dev_gemv_batch_chain(ctx, w, x, xmode, aux, eps, batch, bias, resid, y, nullptr, nullptr);
+}
+
+// The same, and when `next` is given (a weight with k = w's n_rows that the small-batch kernel covers), y's operands for
+// the GEMV with `next` are prepared on the way (RMSNorm with next_aux when that is not null): that call then takes
+// xmode = AXQ_X_PACKED and no x.  The eps of a following RMSNorm is this call's eps.
+int axq_dev_gemv_batch_chain(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
+                             const float *bias, const float *resid, float *y, const axq_weight *next, const float *next_aux) {
     const int k = (int)w->k;
+    int next_even_odd = -1;
+    if (next) {
+        if (next->k != w->n_rows || !axq_dev_gemv_batch_covers(next, batch))
+            return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: the next weight does not take this one's output");
+        next_even_odd = (next->type == AXQ_Q4_0 || next->type == AXQ_Q4_1) ? 1 : 0;
+    }
     // scratch (the context's x buffer): 32 k bytes of A operands, then 2 * (k / 32) * 8 floats of scales and sums
     uint8_t *xa = ctx->xq;
     float *xsg = reinterpret_cast<float *>(ctx->xq + (size_t)32 * k);
@@ -433,10 +545,10 @@ int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int
     a.ypart = w->n_rows <= AXQ_BATCH_SPLIT_ROWS ? reinterpret_cast<float *>(ctx->xq + (size_t)34 * AXQ_BATCH_MAX_K) : nullptr;
     a.n_rows = (int)w->n_rows; a.k = k; a.batch = batch;
     switch (w->type) {
-    case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, x, xmode, aux, eps); break;
-    case AXQ_Q4_1: launch_mb<MQ4x<true>>(ctx, a, x, xmode, aux, eps); break;
-    case AXQ_Q8_0: launch_mb<MQ80>(ctx, a, x, xmode, aux, eps); break;
-    case AXQ_Q4_K: launch_mb<MQ4K>(ctx, a, x, xmode, aux, eps); break;
+    case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q4_1: launch_mb<MQ4x<true>>(ctx, a, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q8_0: launch_mb<MQ80>(ctx, a, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q4_K: launch_mb<MQ4K>(ctx, a, x, xmode, aux, eps, next_even_odd, next_aux); break;
     default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
     }
     AXQ_LAUNCH_CHECK(ctx, "gemv_mb_kernel");

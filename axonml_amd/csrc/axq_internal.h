@@ -103,7 +103,8 @@ int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uin
 // What the GEMV does to x before it uses it (xq must be NULL for the fused forms):
 enum { AXQ_X_PLAIN = 0,    // nothing
        AXQ_X_RMSNORM = 1,  // x <- x / sqrt(mean(x^2) + eps) * aux   (aux = norm weights, K floats)
-       AXQ_X_SWIGLU = 2 }; // small-batch GEMV only: x holds 2K gate/up values (groups of four and four), x <- silu(gate) * up
+       AXQ_X_SWIGLU = 2,   // small-batch GEMV only: x holds 2K gate/up values (groups of four and four), x <- silu(gate) * up
+       AXQ_X_PACKED = 3 }; // small-batch GEMV only: the previous call of a chain has prepared this call's operands
 // ... and to its result before it writes it:
 enum { AXQ_Y_PLAIN = 0,    // y[row] = dot (+ bias[row])
        AXQ_Y_SWIGLU = 1 }; // rows come in groups of four "gate" rows followed by their four "up" rows:
@@ -118,6 +119,8 @@ bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch);
 int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, const float *resid, float *y);
 int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
                           const float *bias, const float *resid, float *y);
+int axq_dev_gemv_batch_chain(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
+                             const float *bias, const float *resid, float *y, const axq_weight *next, const float *next_aux);
 // sample.hip: every pointer a device pointer; scratch = axq_sample_scratch_bytes(vocab)
 size_t axq_sample_scratch_bytes(int vocab);
 int axq_check_sampling_config(axq_ctx *ctx, const axq_sampling_config *cfg);
