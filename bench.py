@@ -119,7 +119,7 @@ def cpu_baseline(packed, qtype, n, k, x, budget_s=12.0):
     L.axo_matmul_ref(*args)  # warm-up (page faults of the scratch)
     times = []
     t_end = time.perf_counter() + budget_s
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 400):
         t0 = time.perf_counter()
         L.axo_matmul_ref(*args)
         times.append(time.perf_counter() - t0)
