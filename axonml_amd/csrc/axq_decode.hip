@@ -330,11 +330,39 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const float *qkv, con
     }
 }
 
+// Where an attention kernel leaves its output rows a second time, as the operands of the small-batch GEMV with the
+// output projection (which then skips its own packing pass): xa = nullptr for nothing.
+struct PackOut {
+    uint8_t *xa = nullptr;
+    float *xsg = nullptr;
+    int even_odd = 0;
+};
+
+// o[0 .. d) of head `head` of row b (LDS) -> operands; the first d / 8 threads of the workgroup, whole lane quads.
+// The workgroups of the last row also write the zeros of the rows that the batch does not have.
+__device__ inline void pack_head_out(const float *o, int d, int head, int n_heads, int b, int rows, const PackOut &pk) {
+    const int tid = threadIdx.x;
+    if (tid >= (d >> 3)) return;
+    const int t = head * (d >> 3) + tid, nblk = (n_heads * d) >> 5;
+    float v[8];
+    const float4 a0 = *reinterpret_cast<const float4 *>(o + tid * 8), a1 = *reinterpret_cast<const float4 *>(o + tid * 8 + 4);
+    v[0] = a0.x; v[1] = a0.y; v[2] = a0.z; v[3] = a0.w; v[4] = a1.x; v[5] = a1.y; v[6] = a1.z; v[7] = a1.w;
+    const int b_end = b == rows - 1 ? 8 : b + 1;
+    for (int bb = b; bb < b_end; bb++) {
+        if (pk.even_odd) axq_store_packed<true>(v, t, bb, rows, nblk, pk.xa, pk.xsg);
+        else axq_store_packed<false>(v, t, bb, rows, nblk, pk.xa, pk.xsg);
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = 0.f;
+    }
+}
+
 // grid (heads), 256 threads.  The (m, l) pairs of the head's splits go through LDS so that every thread
 // knows the weights exp(m_s - max) before it walks the splits; the walk itself has no dependent loads.
 __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, const int32_t *pos_p, int n_heads, int n_kv,
-                                                           int d, int max_splits, int window, float *att, size_t part_stride) {
+                                                           int d, int max_splits, int window, float *att, size_t part_stride,
+                                                           PackOut pk) {
     extern __shared__ float cm[];
+    __shared__ __attribute__((aligned(16))) float ov[256];
     float *wgt = cm;                 // [max_splits] exp(m_s - max)
     float *red = wgt + max_splits;   // [4] wave maxima, then [4] wave sums of l_s w_s
     const int head = blockIdx.x, rep = n_heads / n_kv, kvh = head / rep, h = head - kvh * rep;
@@ -380,6 +408,11 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, co
         }
         float v = o / l;
         att[(size_t)head * d + dim] = v;
+        ov[dim] = v;
+    }
+    if (pk.xa) {
+        __syncthreads();
+        pack_head_out(ov, d, head, n_heads, blockIdx.y, gridDim.y, pk);
     }
 }
 
@@ -417,7 +450,7 @@ template <int D, bool APPEND>
 __global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int qkv_rows, const float *rope_cos,
                                                            const float *rope_sin, uint16_t *kcache, uint16_t *vcache, int pos0,
                                                            const int32_t *pos_arr, size_t seq_stride, int n_heads, int n_kv,
-                                                           int max_pos, int window, float *att) {
+                                                           int max_pos, int window, float *att, PackOut pk) {
     constexpr int HALF = D / 2, LP = D / 8, PPB = 1024 / LP; // lanes per position, positions per pass of the workgroup
     extern __shared__ float sc[];                            // scores, then exp(score - max)
     __shared__ __attribute__((aligned(16))) float qs[D];
@@ -543,7 +576,13 @@ __global__ void __launch_bounds__(1024) attn_prompt_kernel(const float *qkv, int
         float o = 0.f;
 #pragma unroll
         for (int w = 0; w < 16; w++) o += osum[w * D + tid];
-        att[(size_t)b * n_heads * D + (size_t)head * D + tid] = o / sum;
+        o /= sum;
+        att[(size_t)b * n_heads * D + (size_t)head * D + tid] = o;
+        qs[tid] = o; // the query is in registers by now
+    }
+    if (pk.xa) {
+        __syncthreads();
+        pack_head_out(qs, D, head, n_heads, b, gridDim.y, pk);
     }
 }
 
@@ -709,7 +748,7 @@ void launch_attn_partial_d(axq_model *m, int l, const float *qkv, int nseq, hipS
     else launch_attn_partial_t<D, 8>(m, l, qkv, nseq, st);
 }
 
-void launch_attn_split(axq_model *m, int l, const float *qkv, int nseq, float *att, hipStream_t st) {
+void launch_attn_split(axq_model *m, int l, const float *qkv, int nseq, float *att, hipStream_t st, PackOut pk = PackOut()) {
     const axq_model_config &c = m->cfg;
     switch (c.head_dim) { // axq_model_create admits these four sizes only
     case 32: launch_attn_partial_d<32>(m, l, qkv, nseq, st); break;
@@ -720,7 +759,7 @@ void launch_attn_split(axq_model *m, int l, const float *qkv, int nseq, float *a
     const size_t comb_lds = (size_t)(m->max_splits + 8) * sizeof(float);
     attn_combine_kernel<<<dim3(c.num_attention_heads, nseq), 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
                                                                                 c.num_key_value_heads, c.head_dim, m->max_splits,
-                                                                                c.sliding_window, att, m->part_stride);
+                                                                                c.sliding_window, att, m->part_stride, pk);
 }
 
 // y = g(W f(x) (+ bias)): f = identity or RMSNorm with weights `aux`; g = identity, or, for the fused gate/up
@@ -751,7 +790,7 @@ int linear(axq_model *m, const axq_weight *w, const float *x, int xmode, const f
 // The kernels of one token, enqueued on the context's stream: six per layer when every linear is covered
 // by the matrix-pipe GEMV (norms and SwiGLU ride in the GEMVs, residual adds in their bias slot).
 void launch_attn_rows(axq_model *m, int l, const float *qkv, int nb, int pos0, const int32_t *pos_arr, size_t cache_off, size_t lds,
-                      float *att, hipStream_t st);
+                      float *att, hipStream_t st, PackOut pk = PackOut());
 size_t prompt_attn_lds(const axq_model *m, int last);
 
 // short: the context is at most m->fused_max positions: one attention workgroup per head does everything (the new key
@@ -907,7 +946,7 @@ struct Rows {
 
 template <int D, bool APPEND>
 void launch_attn_rows_t(axq_model *m, int l, const float *qkv, int nb, int pos0, const int32_t *pos_arr, size_t cache_off, size_t lds,
-                        float *att, hipStream_t st) {
+                        float *att, hipStream_t st, PackOut pk) {
     const axq_model_config &c = m->cfg;
     static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
     if (lds > 48 * 1024 && !big_lds_allowed) {
@@ -918,24 +957,24 @@ void launch_attn_rows_t(axq_model *m, int l, const float *qkv, int nb, int pos0,
     const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * D + cache_off;
     attn_prompt_kernel<D, APPEND><<<dim3(c.num_attention_heads, nb), 1024, lds, st>>>(
         qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, pos0, pos_arr, m->seq_stride, c.num_attention_heads,
-        c.num_key_value_heads, c.max_position_embeddings, c.sliding_window, att);
+        c.num_key_value_heads, c.max_position_embeddings, c.sliding_window, att, pk);
 }
 
 // Attention of `nb` rows of layer l.  pos_arr == NULL: rows of one sequence (cache at cache_off) at positions pos0.., whose
 // keys and values rope_append_kernel has put into the cache.  Otherwise row b belongs to sequence b at position
 // pos_arr[b], and the kernel appends that row's key and value itself.
 void launch_attn_rows(axq_model *m, int l, const float *qkv, int nb, int pos0, const int32_t *pos_arr, size_t cache_off, size_t lds,
-                      float *att, hipStream_t st) {
+                      float *att, hipStream_t st, PackOut pk) {
     const bool ap = pos_arr != nullptr;
     switch (m->cfg.head_dim) {
-    case 32: ap ? launch_attn_rows_t<32, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st)
-                : launch_attn_rows_t<32, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st); break;
-    case 64: ap ? launch_attn_rows_t<64, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st)
-                : launch_attn_rows_t<64, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st); break;
-    case 128: ap ? launch_attn_rows_t<128, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st)
-                 : launch_attn_rows_t<128, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st); break;
-    default: ap ? launch_attn_rows_t<256, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st)
-                : launch_attn_rows_t<256, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st); break;
+    case 32: ap ? launch_attn_rows_t<32, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st, pk)
+                : launch_attn_rows_t<32, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st, pk); break;
+    case 64: ap ? launch_attn_rows_t<64, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st, pk)
+                : launch_attn_rows_t<64, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st, pk); break;
+    case 128: ap ? launch_attn_rows_t<128, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st, pk)
+                 : launch_attn_rows_t<128, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st, pk); break;
+    default: ap ? launch_attn_rows_t<256, true>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st, pk)
+                : launch_attn_rows_t<256, false>(m, l, qkv, nb, pos0, pos_arr, cache_off, lds, att, st, pk); break;
     }
 }
 
@@ -1005,8 +1044,14 @@ int enqueue_rows(axq_model *m, const Rows &r) {
                                              c.sliding_window, m->pb_att);
             if (on_mfma < 0) return on_mfma;
         }
-        if (r.per_seq && r.split_attn) launch_attn_split(m, l, m->pb_qkv, nb, m->pb_att, st);
-        else if (!on_mfma) launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st);
+        // where the output projection is a small-batch GEMV, the attention kernels leave its operands as well
+        PackOut pk;
+        if (!on_mfma && r.mode == ROWS_GEMV && axq_dev_gemv_batch_covers(m->w_o[l], nb)) {
+            pk.even_odd = axq_dev_gemv_batch_operands(ctx, m->w_o[l], &pk.xa, &pk.xsg) ? 1 : 0;
+            packed_for = m->w_o[l];
+        }
+        if (r.per_seq && r.split_attn) launch_attn_split(m, l, m->pb_qkv, nb, m->pb_att, st, pk);
+        else if (!on_mfma) launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st, pk);
         if ((rc = lin(m->w_o[l], m->pb_att, AXQ_X_PLAIN, nullptr, m->pb_h, m->pb_h, m->w_gu[l], m->norm_ffn + (size_t)l * H))) return rc;
         if ((rc = lin(m->w_gu[l], m->pb_h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu, nullptr, nullptr))) return rc;
         if ((rc = lin(m->w_down[l], m->pb_gu, AXQ_X_SWIGLU, nullptr, m->pb_h, m->pb_h, l + 1 < c.num_hidden_layers ? m->w_qkv[l + 1] : nullptr,

@@ -175,11 +175,6 @@ struct MQ4K {
     }
 };
 
-// bytes {0, 2} of lo and of hi (sel = 0) or bytes {1, 3} of each (sel = 1)
-__device__ inline int pick_alt(uint32_t lo, uint32_t hi, int sel) {
-    return (int)__builtin_amdgcn_perm(hi, lo, sel ? 0x07050301u : 0x06040200u);
-}
-
 template <class T>
 __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
     extern __shared__ float lds_f[];
@@ -280,37 +275,6 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
     }
 }
 
-// Eight consecutive elements (task t) of vector b -> their limbs in the A operands and, from the first task of a
-// 32-element block, the block's scale and sum.  The four tasks of a block sit in four consecutive lanes, which
-// all have to call this together.
-template <bool EVEN_ODD>
-__device__ inline void store_packed(const float (&v)[8], int t, int b, int batch, int nblk, uint8_t *xa, float *xsg) {
-    uint32_t pk[4][2];
-    float sg, sum;
-    int ls[4];
-    axq_split8_compute(v, pk, sg, sum, ls);
-    if (b >= batch) { sg = 0.f; sum = 0.f; }
-    const int blk = t >> 2, e0 = (t & 3) * 8; // first element of the task inside its block
-#pragma unroll
-    for (int l = 0; l < 4; l++) {
-        const int row = 4 * b + l;
-        if (EVEN_ODD) {
-            uint8_t *d0 = xa + ((size_t)(blk * 2 + 0) * 32 + row) * 16 + (e0 >> 1);
-            uint8_t *d1 = xa + ((size_t)(blk * 2 + 1) * 32 + row) * 16 + (e0 >> 1);
-            *reinterpret_cast<uint32_t *>(d0) = (uint32_t)pick_alt(pk[l][0], pk[l][1], 0);
-            *reinterpret_cast<uint32_t *>(d1) = (uint32_t)pick_alt(pk[l][0], pk[l][1], 1);
-        } else {
-            uint8_t *d = xa + ((size_t)(blk * 2 + (e0 >> 4)) * 32 + row) * 16 + (e0 & 15);
-            *reinterpret_cast<uint2 *>(d) = make_uint2(pk[l][0], pk[l][1]);
-        }
-    }
-    if ((t & 3) == 0) {
-        const int slot = (blk * 2 + (b & 1)) * 4 + (b >> 1);
-        xsg[slot] = sg;
-        xsg[(size_t)nblk * 8 + slot] = sum;
-    }
-}
-
 // f(x)[batch, k] -> A operands and group records.  Thread = (8-element task, vector b); vectors beyond the batch
 // are written as zeros.  EVEN_ODD: the h = 0 half of a block's operand holds its even elements, h = 1 the odd.
 // XMODE: AXQ_X_PLAIN; AXQ_X_RMSNORM: f = x / sqrt(mean(x^2) + eps) * aux (every workgroup sums its vector's squares
@@ -363,7 +327,7 @@ __global__ void __launch_bounds__(256) pack_x_kernel(const float *x, const float
             }
         }
     }
-    store_packed<EVEN_ODD>(v, t, b, batch, nblk, xa, xsg);
+    axq_store_packed<EVEN_ODD>(v, t, b, batch, nblk, xa, xsg);
 }
 
 // y = sum over the splits, in order (+ bias, + resid)
@@ -450,7 +414,7 @@ __global__ void __launch_bounds__(512) mb_reduce_pack_kernel(const float *src, i
 #pragma unroll
     for (int q = 0; q < TPT; q++) {
         const int t = q * 512 + (int)threadIdx.x;
-        if (t < ntask) store_packed<EVEN_ODD>(v[q], t, b, batch, nblk, xa, xsg); // ntask is a multiple of 4: whole quads
+        if (t < ntask) axq_store_packed<EVEN_ODD>(v[q], t, b, batch, nblk, xa, xsg); // ntask is a multiple of 4: whole quads
     }
 }
 
@@ -508,6 +472,14 @@ bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch) {
     if (batch < 2 || batch > MAX_BATCH) return false;
     if (w->k % 256 != 0 || w->k > AXQ_BATCH_MAX_K) return false; // 34 k bytes of scratch: the context's x buffer holds that much
     return w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q8_0 || w->type == AXQ_Q4_K;
+}
+
+// Where a caller that prepares the operands of the call with w itself (axq_store_packed, then xmode = AXQ_X_PACKED) has
+// to put them; returns whether w takes the even and the odd elements of a block in separate halves.
+bool axq_dev_gemv_batch_operands(axq_ctx *ctx, const axq_weight *w, uint8_t **xa, float **xsg) {
+    *xa = ctx->xq;
+    *xsg = reinterpret_cast<float *>(ctx->xq + (size_t)32 * w->k);
+    return w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1;
 }
 
 int axq_dev_gemv_batch(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, const float *resid, float *y) {

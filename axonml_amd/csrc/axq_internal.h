@@ -121,6 +121,7 @@ int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int
                           const float *bias, const float *resid, float *y);
 int axq_dev_gemv_batch_chain(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
                              const float *bias, const float *resid, float *y, const axq_weight *next, const float *next_aux);
+bool axq_dev_gemv_batch_operands(axq_ctx *ctx, const axq_weight *w, uint8_t **xa, float **xsg);
 // sample.hip: every pointer a device pointer; scratch = axq_sample_scratch_bytes(vocab)
 size_t axq_sample_scratch_bytes(int vocab);
 int axq_check_sampling_config(axq_ctx *ctx, const axq_sampling_config *cfg);

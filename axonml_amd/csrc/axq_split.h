@@ -118,3 +118,43 @@ __device__ inline void stage_x(const float *x, int k, uint8_t *planes, uint4 *gr
         axq_split8(v, t, live, planes, grp, kpad);
     }
 }
+
+// ---- operands of the small-batch GEMV (2..8 vectors on the 32x32x32 int8 product) -------------------------
+// Scratch of a K-wide call: 32 K bytes of A operands (per 32-element block two halves of 32 rows x 16 bytes,
+// row 4 b + l = limb l of vector b), then 2 * (K / 32) * 8 floats: the blocks' scales, then their sums.
+
+// bytes {0, 2} of lo and of hi (sel = 0) or bytes {1, 3} of each (sel = 1)
+__device__ inline int axq_pick_alt(uint32_t lo, uint32_t hi, int sel) {
+    return (int)__builtin_amdgcn_perm(hi, lo, sel ? 0x07050301u : 0x06040200u);
+}
+
+// Eight consecutive elements (task t) of vector b -> their limbs in the A operands and, from the first task of a
+// 32-element block, the block's scale and sum.  The four tasks of a block sit in four consecutive lanes, which
+// all have to call this together.
+template <bool EVEN_ODD>
+__device__ inline void axq_store_packed(const float (&v)[8], int t, int b, int batch, int nblk, uint8_t *xa, float *xsg) {
+    uint32_t pk[4][2];
+    float sg, sum;
+    int ls[4];
+    axq_split8_compute(v, pk, sg, sum, ls);
+    if (b >= batch) { sg = 0.f; sum = 0.f; }
+    const int blk = t >> 2, e0 = (t & 3) * 8; // first element of the task inside its block
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+        const int row = 4 * b + l;
+        if (EVEN_ODD) {
+            uint8_t *d0 = xa + ((size_t)(blk * 2 + 0) * 32 + row) * 16 + (e0 >> 1);
+            uint8_t *d1 = xa + ((size_t)(blk * 2 + 1) * 32 + row) * 16 + (e0 >> 1);
+            *reinterpret_cast<uint32_t *>(d0) = (uint32_t)axq_pick_alt(pk[l][0], pk[l][1], 0);
+            *reinterpret_cast<uint32_t *>(d1) = (uint32_t)axq_pick_alt(pk[l][0], pk[l][1], 1);
+        } else {
+            uint8_t *d = xa + ((size_t)(blk * 2 + (e0 >> 4)) * 32 + row) * 16 + (e0 & 15);
+            *reinterpret_cast<uint2 *>(d) = make_uint2(pk[l][0], pk[l][1]);
+        }
+    }
+    if ((t & 3) == 0) {
+        const int slot = (blk * 2 + (b & 1)) * 4 + (b >> 1);
+        xsg[slot] = sg;
+        xsg[(size_t)nblk * 8 + slot] = sum;
+    }
+}
