@@ -1,0 +1,154 @@
+// Plain f16 GEMMs of the large prefill shapes on the vendor's GEMM library (hipBLASLt).
+//
+// A quantised weight that meets many activation rows is expanded once per call into two f16 planes
+// (axq_gemm.hip) and multiplied with the row-scaled f16 activations by two library GEMMs that accumulate in f32
+// into the same output.  The library is opened at first use (dlopen) and is not needed to load this one: where it
+// cannot be opened, or has no kernel for a shape, the caller stays on its own fused kernel.
+#include <dlfcn.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include "axq_internal.h"
+
+namespace {
+
+struct LtApi {
+    void *lib = nullptr;
+    bool tried = false, ok = false;
+    decltype(&hipblasLtCreate) create = nullptr;
+    decltype(&hipblasLtDestroy) destroy = nullptr;
+    decltype(&hipblasLtMatrixLayoutCreate) layout_create = nullptr;
+    decltype(&hipblasLtMatrixLayoutDestroy) layout_destroy = nullptr;
+    decltype(&hipblasLtMatmulDescCreate) desc_create = nullptr;
+    decltype(&hipblasLtMatmulDescDestroy) desc_destroy = nullptr;
+    decltype(&hipblasLtMatmulDescSetAttribute) desc_set = nullptr;
+    decltype(&hipblasLtMatmulPreferenceCreate) pref_create = nullptr;
+    decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
+    decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
+    decltype(&hipblasLtMatmulAlgoGetHeuristic) heuristic = nullptr;
+    decltype(&hipblasLtMatmul) matmul = nullptr;
+};
+
+LtApi g_api;
+
+template <class F>
+bool sym(F &f, const char *name) {
+    f = reinterpret_cast<F>(dlsym(g_api.lib, name));
+    return f != nullptr;
+}
+
+bool open_api() {
+    if (g_api.tried) return g_api.ok;
+    g_api.tried = true;
+    g_api.lib = dlopen("libhipblaslt.so.1", RTLD_NOW | RTLD_LOCAL);
+    if (!g_api.lib) g_api.lib = dlopen("libhipblaslt.so", RTLD_NOW | RTLD_LOCAL);
+    if (!g_api.lib) return false;
+    g_api.ok = sym(g_api.create, "hipblasLtCreate") && sym(g_api.destroy, "hipblasLtDestroy") &&
+               sym(g_api.layout_create, "hipblasLtMatrixLayoutCreate") && sym(g_api.layout_destroy, "hipblasLtMatrixLayoutDestroy") &&
+               sym(g_api.desc_create, "hipblasLtMatmulDescCreate") && sym(g_api.desc_destroy, "hipblasLtMatmulDescDestroy") &&
+               sym(g_api.desc_set, "hipblasLtMatmulDescSetAttribute") && sym(g_api.pref_create, "hipblasLtMatmulPreferenceCreate") &&
+               sym(g_api.pref_destroy, "hipblasLtMatmulPreferenceDestroy") && sym(g_api.pref_set, "hipblasLtMatmulPreferenceSetAttribute") &&
+               sym(g_api.heuristic, "hipblasLtMatmulAlgoGetHeuristic") && sym(g_api.matmul, "hipblasLtMatmul");
+    return g_api.ok;
+}
+
+constexpr size_t WORKSPACE_BYTES = 64u << 20;
+constexpr int PLAN_SLOTS = 16;
+
+// One (rows, n, k) shape: layouts and the algorithm the library's heuristic picked.
+struct LtPlan {
+    int m = 0, n = 0, k = 0;
+    bool usable = false;
+    hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
+    hipblasLtMatmulHeuristicResult_t heur;
+};
+
+struct LtState {
+    hipblasLtHandle_t handle = nullptr;
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    void *workspace = nullptr;
+    LtPlan plans[PLAN_SLOTS];
+    int n_plans = 0;
+    bool failed = false;
+};
+
+void drop_plan(LtPlan &p) {
+    if (p.la) (void)g_api.layout_destroy(p.la);
+    if (p.lb) (void)g_api.layout_destroy(p.lb);
+    if (p.lc) (void)g_api.layout_destroy(p.lc);
+    p = LtPlan();
+}
+
+LtState *state_of(axq_ctx *ctx) {
+    if (ctx->blaslt) return reinterpret_cast<LtState *>(ctx->blaslt);
+    if (!open_api()) return nullptr;
+    LtState *s = new LtState();
+    ctx->blaslt = s;
+    const hipblasOperation_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
+    const uint64_t ws = WORKSPACE_BYTES;
+    if (g_api.create(&s->handle) != HIPBLAS_STATUS_SUCCESS || g_api.desc_create(&s->desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS ||
+        g_api.desc_set(s->desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_t, sizeof op_t) != HIPBLAS_STATUS_SUCCESS ||
+        g_api.desc_set(s->desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof op_n) != HIPBLAS_STATUS_SUCCESS ||
+        g_api.pref_create(&s->pref) != HIPBLAS_STATUS_SUCCESS ||
+        g_api.pref_set(s->pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof ws) != HIPBLAS_STATUS_SUCCESS ||
+        hipMalloc(&s->workspace, WORKSPACE_BYTES) != hipSuccess) {
+        (void)hipGetLastError();
+        s->failed = true;
+    }
+    return s;
+}
+
+// In the library's column-major terms: D[n, m] = W[k, n]^T X[k, m], leading dimensions k, k and n, which is
+// y[m, n] = x[m, k] W[n, k]^T on row-major arrays.
+LtPlan *plan_for(LtState *s, int m, int n, int k) {
+    for (int i = 0; i < s->n_plans; i++)
+        if (s->plans[i].m == m && s->plans[i].n == n && s->plans[i].k == k) return &s->plans[i];
+    if (s->n_plans == PLAN_SLOTS) { // forget the oldest
+        drop_plan(s->plans[0]);
+        for (int i = 1; i < PLAN_SLOTS; i++) s->plans[i - 1] = s->plans[i];
+        s->plans[PLAN_SLOTS - 1] = LtPlan();
+        s->n_plans--;
+    }
+    LtPlan &p = s->plans[s->n_plans++];
+    p.m = m; p.n = n; p.k = k;
+    int found = 0;
+    if (g_api.layout_create(&p.la, HIP_R_16F, (uint64_t)k, (uint64_t)n, k) == HIPBLAS_STATUS_SUCCESS &&
+        g_api.layout_create(&p.lb, HIP_R_16F, (uint64_t)k, (uint64_t)m, k) == HIPBLAS_STATUS_SUCCESS &&
+        g_api.layout_create(&p.lc, HIP_R_32F, (uint64_t)n, (uint64_t)m, n) == HIPBLAS_STATUS_SUCCESS &&
+        g_api.heuristic(s->handle, s->desc, p.la, p.lb, p.lc, p.lc, s->pref, 1, &p.heur, &found) == HIPBLAS_STATUS_SUCCESS && found > 0 &&
+        p.heur.workspaceSize <= WORKSPACE_BYTES)
+        p.usable = true;
+    return &p;
+}
+
+} // namespace
+
+// y[m, n] (f32, row-major) = x[m, k] (w1 + w2)[n, k]^T, every operand f16 in device memory.
+// Returns 1 when both GEMMs were enqueued on the context's stream, 0 when the library is not there or has no kernel
+// for the shape (nothing was enqueued), a negative status when a launch failed.
+int axq_blaslt_gemm_f16(axq_ctx *ctx, const _Float16 *w1, const _Float16 *w2, const _Float16 *x, int m, int n, int k, float *y) {
+    LtState *s = state_of(ctx);
+    if (!s || s->failed) return 0;
+    LtPlan *p = plan_for(s, m, n, k);
+    if (!p->usable) return 0;
+    const float one = 1.0f, zero = 0.0f;
+    hipblasStatus_t st = g_api.matmul(s->handle, s->desc, &one, w1, p->la, x, p->lb, &zero, y, p->lc, y, p->lc, &p->heur.algo, s->workspace,
+                                      WORKSPACE_BYTES, ctx->stream);
+    if (st == HIPBLAS_STATUS_SUCCESS)
+        st = g_api.matmul(s->handle, s->desc, &one, w2, p->la, x, p->lb, &one, y, p->lc, y, p->lc, &p->heur.algo, s->workspace,
+                          WORKSPACE_BYTES, ctx->stream);
+    if (st != HIPBLAS_STATUS_SUCCESS) return axq_fail(ctx, AXQ_ERR_BLAS, "hipblasLtMatmul: status %d", (int)st);
+    return 1;
+}
+
+void axq_blaslt_release(axq_ctx *ctx) {
+    if (!ctx->blaslt) return;
+    LtState *s = reinterpret_cast<LtState *>(ctx->blaslt);
+    for (int i = 0; i < s->n_plans; i++) drop_plan(s->plans[i]);
+    if (s->pref) (void)g_api.pref_destroy(s->pref);
+    if (s->desc) (void)g_api.desc_destroy(s->desc);
+    if (s->handle) (void)g_api.destroy(s->handle);
+    if (s->workspace) (void)hipFree(s->workspace);
+    delete s;
+    ctx->blaslt = nullptr;
+}

@@ -117,6 +117,7 @@ const char *axq_status_str(int status) {
     case AXQ_ERR_COPY_FAILED: return "Memory copy failed";
     case AXQ_ERR_KERNEL_LAUNCH_FAILED: return "Kernel launch failed";
     case AXQ_ERR_DRIVER: return "Driver error";
+    case AXQ_ERR_BLAS: return "BLAS error";
     case AXQ_ERR_INVALID_ARGUMENT: return "Invalid argument";
     default: return "unknown status";
     }
@@ -214,6 +215,7 @@ void axq_destroy(axq_ctx *ctx) {
     (void)hipStreamDestroy(ctx->own_stream);
     (void)hipFree(ctx->xq);
     if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
+    axq_blaslt_release(ctx);
     free(ctx);
 }
 

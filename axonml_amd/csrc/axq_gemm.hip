@@ -609,6 +609,18 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
     if (threadIdx.x == 0) { rowscale[2 * row] = 1.0f / f; rowscale[2 * row + 1] = 1.0f / f; }
 }
 
+// The context's GEMM scratch, grown to `need` bytes (work that still uses the old one is waited for first).
+int reserve_scratch(axq_ctx *ctx, size_t need) {
+    if (ctx->gemm_scratch_bytes >= need) return AXQ_OK;
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
+    ctx->gemm_scratch = nullptr;
+    ctx->gemm_scratch_bytes = 0;
+    AXQ_HIP(ctx, hipMalloc(&ctx->gemm_scratch, need), AXQ_ERR_ALLOCATION_FAILED);
+    ctx->gemm_scratch_bytes = need;
+    return AXQ_OK;
+}
+
 struct GemmPlan {
     int splits, steps_per_split, wm;
     size_t xh_bytes, rs_bytes, part_bytes;
@@ -637,16 +649,7 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, size_t extra, GemmPlan *
     p->xh_bytes = axq_align_up((size_t)m * (size_t)w->k * 2, 256);
     p->rs_bytes = axq_align_up((size_t)m * 4, 256);
     p->part_bytes = axq_align_up(p->splits > 1 ? (size_t)p->splits * m * (size_t)w->n_rows * 4 : 0, 256);
-    const size_t need = p->xh_bytes + p->rs_bytes + p->part_bytes + extra;
-    if (ctx->gemm_scratch_bytes < need) {
-        AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
-        if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
-        ctx->gemm_scratch = nullptr;
-        ctx->gemm_scratch_bytes = 0;
-        AXQ_HIP(ctx, hipMalloc(&ctx->gemm_scratch, need), AXQ_ERR_ALLOCATION_FAILED);
-        ctx->gemm_scratch_bytes = need;
-    }
-    return AXQ_OK;
+    return reserve_scratch(ctx, p->xh_bytes + p->rs_bytes + p->part_bytes + extra);
 }
 
 // The GEMM proper over activations that already sit in scratch as scaled f16 rows.
@@ -674,11 +677,93 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Many rows: the weight expanded once per call into the two f16 planes that the kernel above builds tile by tile
+// (WS * w = wh + wl, split8_f16), for the GEMM library (axq_blaslt.hip), which multiplies both with the row-scaled f16
+// activations into the same f32 output; gemm_reduce_kernel then undoes the scales in place.
+// Thread = one 16-weight unit of the traits above; the planes are [n, k] row-major.
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ void __launch_bounds__(256) gemm_planes_kernel(GemmArgs a, _Float16 *wh, _Float16 *wl) {
+    const size_t unit = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int units_per_row = a.k >> 4;
+    const size_t row = unit / (size_t)units_per_row;
+    if (row >= (size_t)a.n) return;
+    const int in_row = (int)(unit - row * (size_t)units_per_row), kstep = in_row >> 2, u4 = in_row & 3;
+    typename T::Raw raw;
+    T::load16(a, row, kstep, u4, raw);
+    float w[16];
+    int k0, k1;
+    T::cvt16(raw, kstep, u4, w, k0, k1);
+    const float sc = T::PRESCALED ? 1.0f : T::WS;
+    uint4 h0, l0, h1, l1;
+    split8_f16(w, sc, h0, l0);
+    split8_f16(w + 8, sc, h1, l1);
+    const size_t at = row * (size_t)a.k + (size_t)kstep * BK;
+    *reinterpret_cast<uint4 *>(wh + at + k0) = h0;
+    *reinterpret_cast<uint4 *>(wh + at + k1) = h1;
+    *reinterpret_cast<uint4 *>(wl + at + k0) = l0;
+    *reinterpret_cast<uint4 *>(wl + at + k1) = l1;
+}
+
+template <class T>
+float launch_planes(axq_ctx *ctx, const GemmArgs &a, _Float16 *wh, _Float16 *wl) {
+    const size_t units = (size_t)a.n * (size_t)(a.k >> 4);
+    gemm_planes_kernel<T><<<(unsigned)((units + 255) / 256), 256, 0, ctx->stream>>>(a, wh, wl);
+    return T::WS;
+}
+
+// From how many rows on a bf16 call goes to the GEMM library (0: never).  Below, expanding the weight and the extra
+// pass over the output cost more than the library's faster multiplication saves (at 512 rows the kernel above wins
+// by 15 %, at 2048 the library by 19 %).
+int lib_min_rows() {
+    static const int v = getenv("AXQ_GEMM_LIB_MIN_ROWS") ? atoi(getenv("AXQ_GEMM_LIB_MIN_ROWS")) : 1024; // development knob
+    return v;
+}
+
+// 1 = done by the library, 0 = not (nothing that matters was enqueued), negative = error
+int gemm_bf16_on_library(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
+    if (w->k % BK != 0 || w->n_rows % 4 != 0 || w->n_rows > INT32_MAX || w->k > INT32_MAX) return 0;
+    const int n = (int)w->n_rows, k = (int)w->k;
+    const size_t xh_bytes = axq_align_up((size_t)m * k * 2, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
+    const size_t plane = axq_align_up((size_t)n * k * 2, 256);
+    int rc;
+    if ((rc = reserve_scratch(ctx, xh_bytes + rs_bytes + 2 * plane))) return rc;
+    uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
+    _Float16 *xh = reinterpret_cast<_Float16 *>(base);
+    float *rowscale = reinterpret_cast<float *>(base + xh_bytes);
+    _Float16 *wh = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes), *wl = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes + plane);
+    GemmArgs a = {};
+    a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
+    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
+    a.n = n; a.k = k;
+    float ws;
+    switch (w->type) {
+    case AXQ_Q4_K: ws = launch_planes<GQ4K>(ctx, a, wh, wl); break;
+    case AXQ_Q4_0: ws = launch_planes<GQ4x<false>>(ctx, a, wh, wl); break;
+    case AXQ_Q4_1: ws = launch_planes<GQ4x<true>>(ctx, a, wh, wl); break;
+    case AXQ_Q5_0: ws = launch_planes<GQ5x<false>>(ctx, a, wh, wl); break;
+    case AXQ_Q5_1: ws = launch_planes<GQ5x<true>>(ctx, a, wh, wl); break;
+    case AXQ_Q8_0: ws = launch_planes<GQ80>(ctx, a, wh, wl); break;
+    default: return 0; // plain f16 / f32 weights stay on the fused kernel
+    }
+    gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, k, xh, rowscale);
+    AXQ_LAUNCH_CHECK(ctx, "gemm_planes_kernel");
+    if ((rc = axq_blaslt_gemm_f16(ctx, wh, wl, xh, m, n, k, y)) <= 0) return rc;
+    const size_t total4 = (size_t)m * n / 4;
+    gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(y, rowscale, m, n, 1, 1.0f / ws, 1, nullptr, nullptr, y);
+    AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
+    return 1;
+}
+
 } // namespace
 
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
     GemmPlan p;
     int rc;
+    if (lib_min_rows() > 0 && m >= lib_min_rows()) {
+        if ((rc = gemm_bf16_on_library(ctx, w, x, m, y)) != 0) return rc < 0 ? rc : AXQ_OK;
+    }
     if ((rc = plan_gemm(ctx, w, m, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, (int)w->k, reinterpret_cast<_Float16 *>(base),

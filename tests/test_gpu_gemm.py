@@ -42,6 +42,18 @@ def test_config_prefill_k4096(ctx, qtype, m):
     _check(ctx, qtype, m, 512, 4096, seed=m)
 
 
+@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K])
+@pytest.mark.parametrize("m,n,k", [(1024, 136, 512), (1100, 520, 1024)])
+def test_many_rows_through_the_gemm_library(ctx, qtype, m, n, k):
+    """From 1024 rows on the weight is expanded into two bf16 planes and multiplied by the GEMM library."""
+    _check(ctx, qtype, m, n, k, seed=m + qtype)
+
+
+@pytest.mark.parametrize("xscale", [1e-30, 1e30])
+def test_many_rows_of_extreme_magnitude(ctx, xscale):
+    _check(ctx, o.Q4_K, 1030, 128, 512, seed=11, xscale=xscale)
+
+
 @pytest.mark.parametrize("xscale", [1e-4, 1.0, 3e4])
 def test_row_scaling_keeps_extreme_activations_exact(ctx, xscale):
     _check(ctx, o.Q4_K, 64, 128, 512, seed=9, xscale=xscale)
