@@ -433,10 +433,12 @@ void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *a
     const unsigned chunks = (unsigned)((a.k + WAVE_K - 1) / WAVE_K);
     const unsigned tiles = (unsigned)((a.n_rows + 31) / 32);
     // few row tiles (a narrow output): split K over up to four workgroups per tile so that the chip is full
+    // (twice as many, for two workgroups per compute unit, was slower: 2.36 against 2.32 ms per batched 7B step; so were
+    // 64-row workgroups that fetch the A operands once for two row tiles: 1 % faster on the gate/up shape, slower elsewhere)
     unsigned splits = (unsigned)ctx->prop.multiProcessorCount / tiles;
     splits = splits > 4 ? 4 : splits;
     if (splits > chunks / 8) splits = chunks / 8;
-    if (splits < 2) splits = 1;
+    if (splits < 2 || !a.ypart) splits = 1;
     a.chunks_per_split = (int)((chunks + splits - 1) / splits);
     splits = (chunks + a.chunks_per_split - 1) / a.chunks_per_split;
     if (splits < 2) a.ypart = nullptr;
