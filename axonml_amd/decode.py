@@ -156,43 +156,6 @@ class QuantizedLlama:
             pass
 
 
-def smoke(ctx):
-    """Two-layer model, a few tokens, against the CPU decode oracle (called from __graft_entry__.smoke)."""
-    import oracle as o
-
-    cfg = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
-               num_key_value_heads=2, head_dim=64, max_position_embeddings=32, rms_norm_eps=1e-5, rope_theta=10000.0)
-    rng = np.random.default_rng(0)
-    gpu = QuantizedLlama(ctx, **cfg)
-    cpu = o.DecodeModel(vocab_size=512, hidden_size=256, intermediate_size=512, num_layers=2, num_heads=4, num_kv_heads=2,
-                        head_dim=64, max_seq_len=32, rms_norm_eps=1e-5, rope_theta=10000.0)
-    emb = (rng.standard_normal((512, 256)) * 0.5).astype(np.float16).view(np.uint16)
-    gpu.set_embedding_f16(emb)
-    cpu.set_embedding_f16(emb)
-    shapes = {"q": (256, 256), "k": (128, 256), "v": (128, 256), "o": (256, 256), "gate": (512, 256), "up": (512, 256),
-              "down": (256, 512)}
-    from .quant import QuantizedTensor
-
-    for layer in list(range(2)) + [-1]:
-        for name, (n, k) in (shapes.items() if layer >= 0 else [("q", (512, 256))]):
-            w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
-            packed = o.quantize(o.Q4_K, w)
-            gpu.set_linear(layer, name, QuantizedTensor([n, k], QuantType.Q4_K, packed))
-            cpu.set_linear(layer, LINEARS[name], o.Q4_K, packed)
-    worst = 0.0
-    tok = 3
-    for pos in range(6):
-        g_next, g_logits = gpu.forward(tok)
-        c_next, c_logits = cpu.forward(tok, pos)
-        worst = max(worst, float(np.abs(g_logits - c_logits).max() / np.abs(c_logits).max()))
-        assert g_next == c_next, f"greedy token differs at position {pos}: {g_next} vs {c_next}"
-        tok = c_next
-    assert worst <= 1e-3, f"decode logits differ by {worst} of the logit range"
-    print(f"smoke: 2-layer Q4_K decode, 6 tokens, greedy ids equal, logits within {worst:.1e} of their range", flush=True)
-    gpu.close()
-    cpu.close()
-
-
 def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
     """Decode benchmark: Mistral-7B shape, random init, all linears Q4_K, f16 KV cache; greedy, sampled, and several
     sequences side by side."""
