@@ -357,14 +357,19 @@ __device__ inline void pack_head_out(const float *o, int d, int head, int n_head
 }
 
 // grid (heads), 256 threads.  The (m, l) pairs of the head's splits go through LDS so that every thread
-// knows the weights exp(m_s - max) before it walks the splits; the walk itself has no dependent loads.
+// knows the weights exp(m_s - max) before it walks the splits.  Everything the first COMB_PRE splits need is
+// requested before the first barrier (a context of up to COMB_PRE * ATT_CHUNK positions pays one memory latency, not
+// three); the walk over further splits has no dependent loads either.
+constexpr int COMB_PRE = 16;
+
 __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, const int32_t *pos_p, int n_heads, int n_kv,
                                                            int d, int max_splits, int window, float *att, size_t part_stride,
                                                            PackOut pk) {
     extern __shared__ float cm[];
     __shared__ __attribute__((aligned(16))) float ov[256];
     float *wgt = cm;                 // [max_splits] exp(m_s - max)
-    float *red = wgt + max_splits;   // [4] wave maxima, then [4] wave sums of l_s w_s
+    float *lv = wgt + max_splits;    // [max_splits] l_s
+    float *red = lv + max_splits;    // [4] wave maxima
     const int head = blockIdx.x, rep = n_heads / n_kv, kvh = head / rep, h = head - kvh * rep;
     part += (size_t)blockIdx.y * part_stride; // blockIdx.y: the sequence
     att += (size_t)blockIdx.y * n_heads * d;
@@ -374,41 +379,54 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, co
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const float *base = part + ((size_t)(kvh * max_splits + s_lo) * rep + h) * (d + 2);
     const size_t stride = (size_t)rep * (d + 2);
+    const int dim = tid < d ? tid : 0;
+    // requests: (m, l) of split tid, the first splits' outputs of this thread's dim
+    const bool mine = tid < nsplit;
+    const float m0 = mine ? base[tid * stride] : -INFINITY, l0 = mine ? base[tid * stride + 1] : 0.f;
+    float opre[COMB_PRE];
+#pragma unroll
+    for (int u = 0; u < COMB_PRE; u++) opre[u] = base[(u < nsplit ? u : 0) * stride + 2 + dim];
     // maxima
-    float mx = -INFINITY;
-    for (int s = tid; s < nsplit; s += 256) mx = fmaxf(mx, base[s * stride]);
+    float mx = m0;
+    for (int s = tid + 256; s < nsplit; s += 256) mx = fmaxf(mx, base[s * stride]);
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
     if (lane == 0) red[wave] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    // weights and the normaliser, summed in split order by one thread so that the result does not depend on timing
-    for (int s = tid; s < nsplit; s += 256) wgt[s] = expf(base[s * stride] - mx);
+    // weights; the normaliser is summed below in split order by every thread so that the result does not depend on timing
+    if (mine) { wgt[tid] = expf(m0 - mx); lv[tid] = l0; }
+    for (int s = tid + 256; s < nsplit; s += 256) { wgt[s] = expf(base[s * stride] - mx); lv[s] = base[s * stride + 1]; }
     __syncthreads();
-    const int dim = tid;
-    if (dim < d) {
+    {
         float l = 0.f, o = 0.f;
-        int s = 0;
-        for (; s + 4 <= nsplit; s += 4) {
-            float l4[4], o4[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                l4[u] = base[(s + u) * stride + 1];
-                o4[u] = base[(s + u) * stride + 2 + dim];
+        for (int u = 0; u < COMB_PRE; u++) {
+            if (u < nsplit) {
+                l = fmaf(lv[u], wgt[u], l);
+                o = fmaf(opre[u], wgt[u], o);
             }
+        }
+        int s = COMB_PRE;
+        for (; s + 4 <= nsplit; s += 4) {
+            float o4[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) o4[u] = base[(s + u) * stride + 2 + dim];
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                l = fmaf(l4[u], wgt[s + u], l);
+                l = fmaf(lv[s + u], wgt[s + u], l);
                 o = fmaf(o4[u], wgt[s + u], o);
             }
         }
         for (; s < nsplit; s++) {
-            l = fmaf(base[s * stride + 1], wgt[s], l);
+            l = fmaf(lv[s], wgt[s], l);
             o = fmaf(base[s * stride + 2 + dim], wgt[s], o);
         }
-        float v = o / l;
-        att[(size_t)head * d + dim] = v;
-        ov[dim] = v;
+        if (tid < d) {
+            const float v = o / l;
+            att[(size_t)head * d + tid] = v;
+            ov[tid] = v;
+        }
     }
     if (pk.xa) {
         __syncthreads();
@@ -756,7 +774,7 @@ void launch_attn_split(axq_model *m, int l, const float *qkv, int nseq, float *a
     case 128: launch_attn_partial_d<128>(m, l, qkv, nseq, st); break;
     default: launch_attn_partial_d<256>(m, l, qkv, nseq, st); break;
     }
-    const size_t comb_lds = (size_t)(m->max_splits + 8) * sizeof(float);
+    const size_t comb_lds = (size_t)(2 * m->max_splits + 8) * sizeof(float);
     attn_combine_kernel<<<dim3(c.num_attention_heads, nseq), 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
                                                                                 c.num_key_value_heads, c.head_dim, m->max_splits,
                                                                                 c.sliding_window, att, m->part_stride, pk);
