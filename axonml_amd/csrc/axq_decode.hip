@@ -1208,7 +1208,9 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     m->max_splits = (c.max_position_embeddings + ATT_CHUNK - 1) / ATT_CHUNK;
     {
         const char *knob = getenv("AXQ_ATTN_FUSED_MAX"); // development knob: 0 = always split the positions
-        m->fused_max = knob ? atoi(knob) : 384; // measured at the 7B shape: 670 against 645 tokens/s up to 224 positions, even at 384, behind from 512
+        // measured at the 7B shape: one sequence 660-680 against 642-660 tokens/s up to 224 positions, behind from 256 on;
+        // batched steps (which share the threshold and the fused kernel's LDS sizing) still gain at 150, are even around 400
+        m->fused_max = knob ? atoi(knob) : 240;
         if (m->fused_max > 32768) m->fused_max = 32768;
         m->attn_mfma = !(getenv("AXQ_ATTN_MFMA") && getenv("AXQ_ATTN_MFMA")[0] == '0');
     }

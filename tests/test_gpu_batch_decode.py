@@ -214,7 +214,7 @@ def test_one_layer_at_the_7b_shape(ctx):
 @pytest.mark.parametrize("fused_max", ["0", "25", "1000"])
 def test_batched_steps_in_both_attention_forms(ctx, monkeypatch, fused_max):
     """Short contexts: one attention workgroup per sequence and head; longer ones: the positions split over workgroups
-    and merged, for all sequences in one launch.  The switch-over (normally at 384 positions) is moved into the walk."""
+    and merged, for all sequences in one launch.  The switch-over (normally at 240 positions) is moved into the walk."""
     monkeypatch.setenv("AXQ_ATTN_FUSED_MAX", fused_max)
     c = tiny_config(max_seq_len=80)
     w = random_weights(c, 340)
