@@ -1,10 +1,12 @@
 // Plain f16 GEMMs of the large prefill shapes on the vendor's GEMM library (hipBLASLt).
 //
 // A quantised weight that meets many activation rows is expanded once per call into two f16 planes
-// (axq_gemm.hip) and multiplied with the row-scaled f16 activations by two library GEMMs that accumulate in f32
-// into the same output.  The library is opened at first use (dlopen) and is not needed to load this one: where it
+// (axq_gemm.hip), laid side by side, and multiplied with the row-scaled f16 activations (each row twice) by one
+// library GEMM that accumulates in f32.  The library is opened at first use (dlopen) and is not needed to load this one: where it
 // cannot be opened, or has no kernel for a shape, the caller stays on its own fused kernel.
 #include <dlfcn.h>
+
+#include <mutex>
 #include <hipblaslt/hipblaslt.h>
 
 #include "axq_internal.h"
@@ -36,18 +38,24 @@ bool sym(F &f, const char *name) {
     return f != nullptr;
 }
 
-bool open_api() {
-    if (g_api.tried) return g_api.ok;
+// Contexts are independent of each other and may meet here from different threads: the library is opened once.
+std::once_flag g_api_once;
+
+void open_api_once() {
     g_api.tried = true;
     g_api.lib = dlopen("libhipblaslt.so.1", RTLD_NOW | RTLD_LOCAL);
     if (!g_api.lib) g_api.lib = dlopen("libhipblaslt.so", RTLD_NOW | RTLD_LOCAL);
-    if (!g_api.lib) return false;
+    if (!g_api.lib) return;
     g_api.ok = sym(g_api.create, "hipblasLtCreate") && sym(g_api.destroy, "hipblasLtDestroy") &&
                sym(g_api.layout_create, "hipblasLtMatrixLayoutCreate") && sym(g_api.layout_destroy, "hipblasLtMatrixLayoutDestroy") &&
                sym(g_api.desc_create, "hipblasLtMatmulDescCreate") && sym(g_api.desc_destroy, "hipblasLtMatmulDescDestroy") &&
                sym(g_api.desc_set, "hipblasLtMatmulDescSetAttribute") && sym(g_api.pref_create, "hipblasLtMatmulPreferenceCreate") &&
                sym(g_api.pref_destroy, "hipblasLtMatmulPreferenceDestroy") && sym(g_api.pref_set, "hipblasLtMatmulPreferenceSetAttribute") &&
                sym(g_api.heuristic, "hipblasLtMatmulAlgoGetHeuristic") && sym(g_api.matmul, "hipblasLtMatmul");
+}
+
+bool open_api() {
+    std::call_once(g_api_once, open_api_once);
     return g_api.ok;
 }
 
@@ -55,11 +63,14 @@ constexpr size_t WORKSPACE_BYTES = 64u << 20;
 constexpr int PLAN_SLOTS = 16;
 
 // One (rows, n, k) shape: layouts and the algorithm the library's heuristic picked.
+constexpr int CANDIDATES = 8;
+
 struct LtPlan {
     int m = 0, n = 0, k = 0;
-    bool usable = false;
+    bool usable = false, tuned = false;
     hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
-    hipblasLtMatmulHeuristicResult_t heur;
+    hipblasLtMatmulHeuristicResult_t heur[CANDIDATES]; // the library's candidates, best guess first
+    int n_heur = 0, best = 0;
 };
 
 struct LtState {
@@ -67,6 +78,7 @@ struct LtState {
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatmulPreference_t pref = nullptr;
     void *workspace = nullptr;
+    hipEvent_t t0 = nullptr, t1 = nullptr; // for timing candidates (the context's own pair may be in use by the caller)
     LtPlan plans[PLAN_SLOTS];
     int n_plans = 0;
     bool failed = false;
@@ -91,7 +103,8 @@ LtState *state_of(axq_ctx *ctx) {
         g_api.desc_set(s->desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof op_n) != HIPBLAS_STATUS_SUCCESS ||
         g_api.pref_create(&s->pref) != HIPBLAS_STATUS_SUCCESS ||
         g_api.pref_set(s->pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof ws) != HIPBLAS_STATUS_SUCCESS ||
-        hipMalloc(&s->workspace, WORKSPACE_BYTES) != hipSuccess) {
+        hipMalloc(&s->workspace, WORKSPACE_BYTES) != hipSuccess || hipEventCreate(&s->t0) != hipSuccess ||
+        hipEventCreate(&s->t1) != hipSuccess) {
         (void)hipGetLastError();
         s->failed = true;
     }
@@ -115,28 +128,57 @@ LtPlan *plan_for(LtState *s, int m, int n, int k) {
     if (g_api.layout_create(&p.la, HIP_R_16F, (uint64_t)k, (uint64_t)n, k) == HIPBLAS_STATUS_SUCCESS &&
         g_api.layout_create(&p.lb, HIP_R_16F, (uint64_t)k, (uint64_t)m, k) == HIPBLAS_STATUS_SUCCESS &&
         g_api.layout_create(&p.lc, HIP_R_32F, (uint64_t)n, (uint64_t)m, n) == HIPBLAS_STATUS_SUCCESS &&
-        g_api.heuristic(s->handle, s->desc, p.la, p.lb, p.lc, p.lc, s->pref, 1, &p.heur, &found) == HIPBLAS_STATUS_SUCCESS && found > 0 &&
-        p.heur.workspaceSize <= WORKSPACE_BYTES)
-        p.usable = true;
+        g_api.heuristic(s->handle, s->desc, p.la, p.lb, p.lc, p.lc, s->pref, CANDIDATES, p.heur, &found) == HIPBLAS_STATUS_SUCCESS) {
+        for (int i = 0; i < found; i++) // keep the ones that fit the workspace, in the library's order
+            if (p.heur[i].workspaceSize <= WORKSPACE_BYTES) p.heur[p.n_heur++] = p.heur[i];
+        p.usable = p.n_heur > 0;
+    }
     return &p;
 }
 
 } // namespace
 
-// y[m, n] (f32, row-major) = x[m, k] (w1 + w2)[n, k]^T, every operand f16 in device memory.
-// Returns 1 when both GEMMs were enqueued on the context's stream, 0 when the library is not there or has no kernel
-// for the shape (nothing was enqueued), a negative status when a launch failed.
-int axq_blaslt_gemm_f16(axq_ctx *ctx, const _Float16 *w1, const _Float16 *w2, const _Float16 *x, int m, int n, int k, float *y) {
+// y[m, n] (f32, row-major) = x[m, k] w[n, k]^T, both operands f16 in device memory.
+// Returns 1 when the GEMM was enqueued on the context's stream, 0 when the library is not there or has no kernel
+// for the shape (nothing was enqueued), a negative status when the launch failed.
+int axq_blaslt_gemm_f16(axq_ctx *ctx, const _Float16 *w, const _Float16 *x, int m, int n, int k, float *y) {
     LtState *s = state_of(ctx);
     if (!s || s->failed) return 0;
     LtPlan *p = plan_for(s, m, n, k);
     if (!p->usable) return 0;
     const float one = 1.0f, zero = 0.0f;
-    hipblasStatus_t st = g_api.matmul(s->handle, s->desc, &one, w1, p->la, x, p->lb, &zero, y, p->lc, y, p->lc, &p->heur.algo, s->workspace,
-                                      WORKSPACE_BYTES, ctx->stream);
-    if (st == HIPBLAS_STATUS_SUCCESS)
-        st = g_api.matmul(s->handle, s->desc, &one, w2, p->la, x, p->lb, &one, y, p->lc, y, p->lc, &p->heur.algo, s->workspace,
-                          WORKSPACE_BYTES, ctx->stream);
+    auto run = [&](int i) {
+        return g_api.matmul(s->handle, s->desc, &one, w, p->la, x, p->lb, &zero, y, p->lc, y, p->lc, &p->heur[i].algo, s->workspace,
+                            WORKSPACE_BYTES, ctx->stream);
+    };
+    if (!p->tuned) {
+        // First call with this shape: the library's first guess is not always its fastest kernel (at 2048 x 4096 x 8192
+        // by a quarter), so every candidate runs four times on the real operands and the one with the quickest run stays.
+        p->tuned = true;
+        float best_ms = 0.f;
+        bool have = false;
+        for (int i = 0; i < p->n_heur; i++) {
+            if (run(i) != HIPBLAS_STATUS_SUCCESS) continue; // warm-up
+            float fastest = 0.f;
+            bool timed = false;
+            for (int rep = 0; rep < 3; rep++) {
+                float ms = 0.f;
+                if (hipEventRecord(s->t0, ctx->stream) != hipSuccess || run(i) != HIPBLAS_STATUS_SUCCESS ||
+                    hipEventRecord(s->t1, ctx->stream) != hipSuccess || hipEventSynchronize(s->t1) != hipSuccess ||
+                    hipEventElapsedTime(&ms, s->t0, s->t1) != hipSuccess) {
+                    (void)hipGetLastError();
+                    timed = false;
+                    break;
+                }
+                if (!timed || ms < fastest) fastest = ms;
+                timed = true;
+            }
+            if (timed && (!have || fastest < best_ms)) { have = true; best_ms = fastest; p->best = i; }
+        }
+        if (!have) p->usable = false;
+        return have ? 1 : 0; // the last candidate's run left the product in y either way
+    }
+    const hipblasStatus_t st = run(p->best);
     if (st != HIPBLAS_STATUS_SUCCESS) return axq_fail(ctx, AXQ_ERR_BLAS, "hipblasLtMatmul: status %d", (int)st);
     return 1;
 }
@@ -149,6 +191,8 @@ void axq_blaslt_release(axq_ctx *ctx) {
     if (s->desc) (void)g_api.desc_destroy(s->desc);
     if (s->handle) (void)g_api.destroy(s->handle);
     if (s->workspace) (void)hipFree(s->workspace);
+    if (s->t0) (void)hipEventDestroy(s->t0);
+    if (s->t1) (void)hipEventDestroy(s->t1);
     delete s;
     ctx->blaslt = nullptr;
 }

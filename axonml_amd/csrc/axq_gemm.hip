@@ -425,7 +425,8 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
 }
 
 // bf16 rows -> f16 rows scaled by a power of two (largest magnitude below 2^15), and the scale to undo it.
-__global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int m, int k, _Float16 *xh, float *rowscale) {
+// dup: every output row holds the scaled row twice (2k halfs), for a product with the two planes of a weight side by side.
+__global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int m, int k, _Float16 *xh, float *rowscale, int dup) {
     __shared__ float red[4];
     const int row = blockIdx.x;
     const uint16_t *xr = x + (size_t)row * k;
@@ -448,7 +449,13 @@ __global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int
     const float f = __builtin_bit_cast(float, (uint32_t)sb << 23);
     for (int i = threadIdx.x; i < k; i += blockDim.x) {
         float v = __builtin_bit_cast(float, (uint32_t)xr[i] << 16);
-        xh[(size_t)row * k + i] = (_Float16)(v * f);
+        const _Float16 hv = (_Float16)(v * f);
+        if (dup) {
+            xh[(size_t)row * 2 * k + i] = hv;
+            xh[(size_t)row * 2 * k + k + i] = hv;
+        } else {
+            xh[(size_t)row * k + i] = hv;
+        }
     }
     if (threadIdx.x == 0) rowscale[row] = 1.0f / f;
 }
@@ -679,12 +686,13 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
 
 // ---------------------------------------------------------------------------
 // Many rows: the weight expanded once per call into the two f16 planes that the kernel above builds tile by tile
-// (WS * w = wh + wl, split8_f16), for the GEMM library (axq_blaslt.hip), which multiplies both with the row-scaled f16
-// activations into the same f32 output; gemm_reduce_kernel then undoes the scales in place.
-// Thread = one 16-weight unit of the traits above; the planes are [n, k] row-major.
+// (WS * w = wh + wl, split8_f16) for the GEMM library (axq_blaslt.hip): row r of the expanded weight is [wh_r | wl_r],
+// the row-scaled f16 activations are written twice per row, [x | x], and one library GEMM over 2k puts
+// x wh^T + x wl^T into the f32 output; gemm_reduce_kernel then undoes the scales in place.
+// Thread = one 16-weight unit of the traits above.
 // ---------------------------------------------------------------------------
 template <class T>
-__global__ void __launch_bounds__(256) gemm_planes_kernel(GemmArgs a, _Float16 *wh, _Float16 *wl) {
+__global__ void __launch_bounds__(256) gemm_planes_kernel(GemmArgs a, _Float16 *wp) {
     const size_t unit = (size_t)blockIdx.x * 256 + threadIdx.x;
     const int units_per_row = a.k >> 4;
     const size_t row = unit / (size_t)units_per_row;
@@ -699,17 +707,17 @@ __global__ void __launch_bounds__(256) gemm_planes_kernel(GemmArgs a, _Float16 *
     uint4 h0, l0, h1, l1;
     split8_f16(w, sc, h0, l0);
     split8_f16(w + 8, sc, h1, l1);
-    const size_t at = row * (size_t)a.k + (size_t)kstep * BK;
-    *reinterpret_cast<uint4 *>(wh + at + k0) = h0;
-    *reinterpret_cast<uint4 *>(wh + at + k1) = h1;
-    *reinterpret_cast<uint4 *>(wl + at + k0) = l0;
-    *reinterpret_cast<uint4 *>(wl + at + k1) = l1;
+    _Float16 *wh = wp + row * 2 * (size_t)a.k + (size_t)kstep * BK, *wl = wh + a.k;
+    *reinterpret_cast<uint4 *>(wh + k0) = h0;
+    *reinterpret_cast<uint4 *>(wh + k1) = h1;
+    *reinterpret_cast<uint4 *>(wl + k0) = l0;
+    *reinterpret_cast<uint4 *>(wl + k1) = l1;
 }
 
 template <class T>
-float launch_planes(axq_ctx *ctx, const GemmArgs &a, _Float16 *wh, _Float16 *wl) {
+float launch_planes(axq_ctx *ctx, const GemmArgs &a, _Float16 *wp) {
     const size_t units = (size_t)a.n * (size_t)(a.k >> 4);
-    gemm_planes_kernel<T><<<(unsigned)((units + 255) / 256), 256, 0, ctx->stream>>>(a, wh, wl);
+    gemm_planes_kernel<T><<<(unsigned)((units + 255) / 256), 256, 0, ctx->stream>>>(a, wp);
     return T::WS;
 }
 
@@ -725,31 +733,31 @@ int lib_min_rows() {
 int gemm_bf16_on_library(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
     if (w->k % BK != 0 || w->n_rows % 4 != 0 || w->n_rows > INT32_MAX || w->k > INT32_MAX) return 0;
     const int n = (int)w->n_rows, k = (int)w->k;
-    const size_t xh_bytes = axq_align_up((size_t)m * k * 2, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
-    const size_t plane = axq_align_up((size_t)n * k * 2, 256);
+    const size_t xh_bytes = axq_align_up((size_t)m * k * 4, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
+    const size_t planes = axq_align_up((size_t)n * k * 4, 256);
     int rc;
-    if ((rc = reserve_scratch(ctx, xh_bytes + rs_bytes + 2 * plane))) return rc;
+    if ((rc = reserve_scratch(ctx, xh_bytes + rs_bytes + planes))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     _Float16 *xh = reinterpret_cast<_Float16 *>(base);
     float *rowscale = reinterpret_cast<float *>(base + xh_bytes);
-    _Float16 *wh = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes), *wl = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes + plane);
+    _Float16 *wp = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes); // [n, 2k]: the two planes of a row side by side
     GemmArgs a = {};
     a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
     a.n = n; a.k = k;
     float ws;
     switch (w->type) {
-    case AXQ_Q4_K: ws = launch_planes<GQ4K>(ctx, a, wh, wl); break;
-    case AXQ_Q4_0: ws = launch_planes<GQ4x<false>>(ctx, a, wh, wl); break;
-    case AXQ_Q4_1: ws = launch_planes<GQ4x<true>>(ctx, a, wh, wl); break;
-    case AXQ_Q5_0: ws = launch_planes<GQ5x<false>>(ctx, a, wh, wl); break;
-    case AXQ_Q5_1: ws = launch_planes<GQ5x<true>>(ctx, a, wh, wl); break;
-    case AXQ_Q8_0: ws = launch_planes<GQ80>(ctx, a, wh, wl); break;
+    case AXQ_Q4_K: ws = launch_planes<GQ4K>(ctx, a, wp); break;
+    case AXQ_Q4_0: ws = launch_planes<GQ4x<false>>(ctx, a, wp); break;
+    case AXQ_Q4_1: ws = launch_planes<GQ4x<true>>(ctx, a, wp); break;
+    case AXQ_Q5_0: ws = launch_planes<GQ5x<false>>(ctx, a, wp); break;
+    case AXQ_Q5_1: ws = launch_planes<GQ5x<true>>(ctx, a, wp); break;
+    case AXQ_Q8_0: ws = launch_planes<GQ80>(ctx, a, wp); break;
     default: return 0; // plain f16 / f32 weights stay on the fused kernel
     }
-    gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, k, xh, rowscale);
+    gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, k, xh, rowscale, 1);
     AXQ_LAUNCH_CHECK(ctx, "gemm_planes_kernel");
-    if ((rc = axq_blaslt_gemm_f16(ctx, wh, wl, xh, m, n, k, y)) <= 0) return rc;
+    if ((rc = axq_blaslt_gemm_f16(ctx, wp, xh, m, n, 2 * k, y)) <= 0) return rc;
     const size_t total4 = (size_t)m * n / 4;
     gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(y, rowscale, m, n, 1, 1.0f / ws, 1, nullptr, nullptr, y);
     AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
@@ -767,7 +775,7 @@ int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int 
     if ((rc = plan_gemm(ctx, w, m, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
-                                                   reinterpret_cast<float *>(base + p.xh_bytes));
+                                                   reinterpret_cast<float *>(base + p.xh_bytes), 0);
     return run_gemm(ctx, w, m, p, y);
 }
 
