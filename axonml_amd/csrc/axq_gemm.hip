@@ -723,9 +723,9 @@ float launch_planes(axq_ctx *ctx, const GemmArgs &a, _Float16 *wp) {
 
 // From how many rows on a bf16 call goes to the GEMM library (0: never).  Below, expanding the weight and the extra
 // pass over the output cost more than the library's faster multiplication saves (at 512 rows the kernel above wins
-// by 15 %, at 2048 the library by 19 %).
+// by 2-7 %, at 768 the library by 15-47 %, at 2048 by 20-50 %).
 int lib_min_rows() {
-    static const int v = getenv("AXQ_GEMM_LIB_MIN_ROWS") ? atoi(getenv("AXQ_GEMM_LIB_MIN_ROWS")) : 1024; // development knob
+    static const int v = getenv("AXQ_GEMM_LIB_MIN_ROWS") ? atoi(getenv("AXQ_GEMM_LIB_MIN_ROWS")) : 640; // development knob
     return v;
 }
 
