@@ -65,6 +65,7 @@ struct axq_model {
     hipGraphExec_t graph_f;         // the same with one attention workgroup per head (short contexts)
     bool graph_f_ok;
     int fused_max;                  // contexts up to this many positions take graph_f
+    int prompt_chunk;               // most prompt rows per pass through the layers
     bool attn_mfma;                 // prompt attention of many rows on the matrix pipe (development knob AXQ_ATTN_MFMA=0: off)
 };
 
@@ -891,7 +892,7 @@ int run_token(axq_model *m, int pos) {
 // of each of several sequences (a batched step).  Up to PROMPT_BATCH rows use the small-batch GEMV (one pass over the
 // weights for eight vectors), up to PROMPT_CHUNK the matrix-pipe GEMM on f32 activations once there are enough of
 // them to fill its tiles.
-constexpr int PROMPT_CHUNK = 512;
+constexpr int PROMPT_CHUNK = 2048;
 constexpr int PROMPT_GEMM_MIN = 32;
 
 // LDS of attn_prompt_kernel for queries up to position `last` (exclusive)
@@ -1098,7 +1099,7 @@ int feed_rows(axq_model *m, int seq, const int32_t *toks, int n, int pos0, int *
         Rows r;
         r.mode = ROWS_NONE; r.toks = toks + i; r.per_seq = false; r.seq = seq; r.pos0 = pos0 + i; r.split_attn = false;
         // enough rows to fill GEMM tiles (fewer where the small-batch GEMV does not apply and single rows are the alternative)
-        r.nb = left < PROMPT_CHUNK ? left : PROMPT_CHUNK;
+        r.nb = left < m->prompt_chunk ? left : m->prompt_chunk;
         if (allow >= 2 && r.nb >= (all_layers_in_small_batch_reach(m, left) ? PROMPT_GEMM_MIN : PROMPT_BATCH) &&
             rows_mode_covers(m, ROWS_GEMM, r.pos0 + r.nb, r.nb))
             r.mode = ROWS_GEMM;
@@ -1213,6 +1214,10 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
         m->fused_max = knob ? atoi(knob) : 240;
         if (m->fused_max > 32768) m->fused_max = 32768;
         m->attn_mfma = !(getenv("AXQ_ATTN_MFMA") && getenv("AXQ_ATTN_MFMA")[0] == '0');
+        const char *chunk = getenv("AXQ_PROMPT_CHUNK"); // development knob: fewer prompt rows per pass (tests cross chunk borders with it)
+        m->prompt_chunk = chunk ? atoi(chunk) : PROMPT_CHUNK;
+        if (m->prompt_chunk < PROMPT_GEMM_MIN) m->prompt_chunk = PROMPT_GEMM_MIN;
+        if (m->prompt_chunk > PROMPT_CHUNK) m->prompt_chunk = PROMPT_CHUNK;
     }
     m->n_seq = 1;
     m->seq_stride = (size_t)c.num_hidden_layers * c.num_key_value_heads * c.max_position_embeddings * c.head_dim;

@@ -138,6 +138,19 @@ def test_generate_matches_oracle_greedy_and_is_repeatable(ctx):
     (dict(max_seq_len=200, num_heads=3, num_kv_heads=1, head_dim=64, hidden_size=192), o.Q8_0, 0, 120),  # three query heads per KV head: the general kernel
 ])
 def test_prompt_fed_at_once_matches_the_oracle_token_by_token(ctx, over, qtype, n_first, n_prompt):
+    _prompt_at_once(ctx, over, qtype, n_first, n_prompt)
+
+
+@pytest.mark.parametrize("chunk,over,n_first,n_prompt", [("64", dict(max_seq_len=320), 0, 300), ("100", dict(max_seq_len=320, sliding_window=90), 21, 250),
+                                                         ("40", dict(max_seq_len=200, num_heads=8, num_kv_heads=2, head_dim=32), 0, 161)])
+def test_prompt_in_several_chunks(ctx, monkeypatch, chunk, over, n_first, n_prompt):
+    """A prompt longer than one pass takes (normally 2048 rows; the knob is read when the model is made) goes through
+    the layers in chunks: the later ones attend to the keys the earlier ones left, the last may be a single row."""
+    monkeypatch.setenv("AXQ_PROMPT_CHUNK", chunk)
+    _prompt_at_once(ctx, over, o.Q4_K, n_first, n_prompt)
+
+
+def _prompt_at_once(ctx, over, qtype, n_first, n_prompt):
     """forward_tokens (up to eight prompt tokens per pass over the weights) against the oracle's one-token steps:
     last logits and next token to the decode bar, and the KV cache against the GPU's own one-token path."""
     c = tiny_config(**over)
