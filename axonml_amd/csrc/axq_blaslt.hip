@@ -66,7 +66,7 @@ constexpr int PLAN_SLOTS = 16;
 constexpr int CANDIDATES = 8;
 
 struct LtPlan {
-    int m = 0, n = 0, k = 0;
+    int m = 0, n = 0, k = 0, ldw = 0, ldx = 0;
     bool usable = false, tuned = false;
     hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
     hipblasLtMatmulHeuristicResult_t heur[CANDIDATES]; // the library's candidates, best guess first
@@ -111,11 +111,12 @@ LtState *state_of(axq_ctx *ctx) {
     return s;
 }
 
-// In the library's column-major terms: D[n, m] = W[k, n]^T X[k, m], leading dimensions k, k and n, which is
-// y[m, n] = x[m, k] W[n, k]^T on row-major arrays.
-LtPlan *plan_for(LtState *s, int m, int n, int k) {
+// In the library's column-major terms: D[n, m] = W[k, n]^T X[k, m], leading dimensions ldw, ldx and n, which is
+// y[m, n] = x[m, k] W[n, k]^T on row-major arrays whose rows are ldx and ldw elements apart.
+LtPlan *plan_for(LtState *s, int m, int n, int k, int ldw, int ldx) {
     for (int i = 0; i < s->n_plans; i++)
-        if (s->plans[i].m == m && s->plans[i].n == n && s->plans[i].k == k) return &s->plans[i];
+        if (s->plans[i].m == m && s->plans[i].n == n && s->plans[i].k == k && s->plans[i].ldw == ldw && s->plans[i].ldx == ldx)
+            return &s->plans[i];
     if (s->n_plans == PLAN_SLOTS) { // forget the oldest
         drop_plan(s->plans[0]);
         for (int i = 1; i < PLAN_SLOTS; i++) s->plans[i - 1] = s->plans[i];
@@ -123,10 +124,10 @@ LtPlan *plan_for(LtState *s, int m, int n, int k) {
         s->n_plans--;
     }
     LtPlan &p = s->plans[s->n_plans++];
-    p.m = m; p.n = n; p.k = k;
+    p.m = m; p.n = n; p.k = k; p.ldw = ldw; p.ldx = ldx;
     int found = 0;
-    if (g_api.layout_create(&p.la, HIP_R_16F, (uint64_t)k, (uint64_t)n, k) == HIPBLAS_STATUS_SUCCESS &&
-        g_api.layout_create(&p.lb, HIP_R_16F, (uint64_t)k, (uint64_t)m, k) == HIPBLAS_STATUS_SUCCESS &&
+    if (g_api.layout_create(&p.la, HIP_R_16F, (uint64_t)k, (uint64_t)n, ldw) == HIPBLAS_STATUS_SUCCESS &&
+        g_api.layout_create(&p.lb, HIP_R_16F, (uint64_t)k, (uint64_t)m, ldx) == HIPBLAS_STATUS_SUCCESS &&
         g_api.layout_create(&p.lc, HIP_R_32F, (uint64_t)n, (uint64_t)m, n) == HIPBLAS_STATUS_SUCCESS &&
         g_api.heuristic(s->handle, s->desc, p.la, p.lb, p.lc, p.lc, s->pref, CANDIDATES, p.heur, &found) == HIPBLAS_STATUS_SUCCESS) {
         for (int i = 0; i < found; i++) // keep the ones that fit the workspace, in the library's order
@@ -138,48 +139,69 @@ LtPlan *plan_for(LtState *s, int m, int n, int k) {
 
 } // namespace
 
-// y[m, n] (f32, row-major) = x[m, k] w[n, k]^T, both operands f16 in device memory.
-// Returns 1 when the GEMM was enqueued on the context's stream, 0 when the library is not there or has no kernel
-// for the shape (nothing was enqueued), a negative status when the launch failed.
-int axq_blaslt_gemm_f16(axq_ctx *ctx, const _Float16 *w, const _Float16 *x, int m, int n, int k, float *y) {
-    LtState *s = state_of(ctx);
-    if (!s || s->failed) return 0;
-    LtPlan *p = plan_for(s, m, n, k);
-    if (!p->usable) return 0;
+namespace {
+
+// First use of a shape: the library's first guess is not always its fastest kernel (at 2048 x 4096 x 8192 by a
+// quarter), so every candidate runs four times on the real operands, overwriting y, and the one with the quickest run
+// stays.  Returns whether a candidate ran (the product is then in y).
+bool tune(axq_ctx *ctx, LtState *s, LtPlan *p, const _Float16 *w, const _Float16 *x, float *y) {
     const float one = 1.0f, zero = 0.0f;
     auto run = [&](int i) {
         return g_api.matmul(s->handle, s->desc, &one, w, p->la, x, p->lb, &zero, y, p->lc, y, p->lc, &p->heur[i].algo, s->workspace,
                             WORKSPACE_BYTES, ctx->stream);
     };
-    if (!p->tuned) {
-        // First call with this shape: the library's first guess is not always its fastest kernel (at 2048 x 4096 x 8192
-        // by a quarter), so every candidate runs four times on the real operands and the one with the quickest run stays.
-        p->tuned = true;
-        float best_ms = 0.f;
-        bool have = false;
-        for (int i = 0; i < p->n_heur; i++) {
-            if (run(i) != HIPBLAS_STATUS_SUCCESS) continue; // warm-up
-            float fastest = 0.f;
-            bool timed = false;
-            for (int rep = 0; rep < 3; rep++) {
-                float ms = 0.f;
-                if (hipEventRecord(s->t0, ctx->stream) != hipSuccess || run(i) != HIPBLAS_STATUS_SUCCESS ||
-                    hipEventRecord(s->t1, ctx->stream) != hipSuccess || hipEventSynchronize(s->t1) != hipSuccess ||
-                    hipEventElapsedTime(&ms, s->t0, s->t1) != hipSuccess) {
-                    (void)hipGetLastError();
-                    timed = false;
-                    break;
-                }
-                if (!timed || ms < fastest) fastest = ms;
-                timed = true;
+    p->tuned = true;
+    float best_ms = 0.f;
+    bool have = false;
+    for (int i = 0; i < p->n_heur; i++) {
+        if (run(i) != HIPBLAS_STATUS_SUCCESS) continue; // warm-up
+        float fastest = 0.f;
+        bool timed = false;
+        for (int rep = 0; rep < 3; rep++) {
+            float ms = 0.f;
+            if (hipEventRecord(s->t0, ctx->stream) != hipSuccess || run(i) != HIPBLAS_STATUS_SUCCESS ||
+                hipEventRecord(s->t1, ctx->stream) != hipSuccess || hipEventSynchronize(s->t1) != hipSuccess ||
+                hipEventElapsedTime(&ms, s->t0, s->t1) != hipSuccess) {
+                (void)hipGetLastError();
+                timed = false;
+                break;
             }
-            if (timed && (!have || fastest < best_ms)) { have = true; best_ms = fastest; p->best = i; }
+            if (!timed || ms < fastest) fastest = ms;
+            timed = true;
         }
-        if (!have) p->usable = false;
-        return have ? 1 : 0; // the last candidate's run left the product in y either way
+        if (timed && (!have || fastest < best_ms)) { have = true; best_ms = fastest; p->best = i; }
     }
-    const hipblasStatus_t st = run(p->best);
+    if (!have) p->usable = false;
+    return have;
+}
+
+} // namespace
+
+// y[m, n] (f32, row-major, rows n apart) = x[m, k] w[n, k]^T (+ y when `accumulate`), both operands f16 in device memory
+// with rows ldx and ldw elements apart.  Returns 1 when the GEMM was enqueued on the context's stream, 0 when the library
+// is not there or has no kernel for the shape (nothing that matters was enqueued), a negative status when the launch
+// failed.  A shape met for the first time is tuned on the way (not when accumulating, which must run exactly once:
+// axq_blaslt_tune_f16 in front of such a call does it).
+int axq_blaslt_gemm_f16(axq_ctx *ctx, const _Float16 *w, int ldw, const _Float16 *x, int ldx, int m, int n, int k, bool accumulate, float *y) {
+    LtState *s = state_of(ctx);
+    if (!s || s->failed) return 0;
+    LtPlan *p = plan_for(s, m, n, k, ldw, ldx);
+    if (!p->usable) return 0;
+    if (!p->tuned && !accumulate) return tune(ctx, s, p, w, x, y) ? 1 : 0;
+    const float one = 1.0f, zero = 0.0f;
+    const hipblasStatus_t st = g_api.matmul(s->handle, s->desc, &one, w, p->la, x, p->lb, accumulate ? &one : &zero, y, p->lc, y, p->lc,
+                                            &p->heur[p->tuned ? p->best : 0].algo, s->workspace, WORKSPACE_BYTES, ctx->stream);
     if (st != HIPBLAS_STATUS_SUCCESS) return axq_fail(ctx, AXQ_ERR_BLAS, "hipblasLtMatmul: status %d", (int)st);
+    return 1;
+}
+
+// Tunes the shape if it has not been met yet (y is overwritten then); 1 = the shape can run, 0 = it cannot.
+int axq_blaslt_tune_f16(axq_ctx *ctx, const _Float16 *w, int ldw, const _Float16 *x, int ldx, int m, int n, int k, float *y) {
+    LtState *s = state_of(ctx);
+    if (!s || s->failed) return 0;
+    LtPlan *p = plan_for(s, m, n, k, ldw, ldx);
+    if (!p->usable) return 0;
+    if (!p->tuned) return tune(ctx, s, p, w, x, y) ? 1 : 0;
     return 1;
 }
 

@@ -514,8 +514,9 @@ int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
 // f32 rows, optionally RMS-normalised on the way ((x * inv_rms) * norm_w, RMSNorm::forward, llm/src/llama.rs:158-187),
 // -> two f16 rows each under one power-of-two scale: row 2t holds the leading 11 bits of every element, row 2t + 1
 // what those leave, so that their GEMM results add up to the f32 product (the GEMM's epilogue adds them: pair mode).
+// lib: the layout for the GEMM library instead: row t of xh is [hi | hi | lo] (3k halfs) and has one scale.
 __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, const float *norm_w, float eps, int m, int k,
-                                                              _Float16 *xh, float *rowscale) {
+                                                              _Float16 *xh, float *rowscale, int lib) {
     // the row stays in registers between the passes: 16 bytes per thread and step, up to 16 steps (k <= 16384);
     // longer rows (or k not a multiple of 4) take the plain loops below
     constexpr int STEPS = 16;
@@ -590,7 +591,8 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
     int sb = 127 + 14 - (eb - 127);
     sb = sb < 1 ? 1 : (sb > 254 ? 254 : sb);
     const float f = __builtin_bit_cast(float, (uint32_t)sb << 23);
-    _Float16 *hi_row = xh + (size_t)(2 * row) * k, *lo_row = hi_row + k;
+    _Float16 *hi_row = lib ? xh + (size_t)row * 3 * k : xh + (size_t)(2 * row) * k, *lo_row = lib ? hi_row + 2 * k : hi_row + k;
+    _Float16 *hi2_row = hi_row + k; // lib only
     if (in_regs) {
 #pragma unroll
         for (int c = 0; c < STEPS; c++) {
@@ -602,6 +604,7 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
                 for (int j = 0; j < 4; j++) { h[j] = (_Float16)e[j]; l[j] = (_Float16)(e[j] - (float)h[j]); }
                 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
                 reinterpret_cast<half4 *>(hi_row)[i4] = half4{h[0], h[1], h[2], h[3]};
+                if (lib) reinterpret_cast<half4 *>(hi2_row)[i4] = half4{h[0], h[1], h[2], h[3]};
                 reinterpret_cast<half4 *>(lo_row)[i4] = half4{l[0], l[1], l[2], l[3]};
             }
         }
@@ -610,10 +613,14 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
             const float e = (norm_w ? (xr[i] * inv) * norm_w[i] : xr[i]) * f;
             const _Float16 hi = (_Float16)e;
             hi_row[i] = hi;
+            if (lib) hi2_row[i] = hi;
             lo_row[i] = (_Float16)(e - (float)hi);
         }
     }
-    if (threadIdx.x == 0) { rowscale[2 * row] = 1.0f / f; rowscale[2 * row + 1] = 1.0f / f; }
+    if (threadIdx.x == 0) {
+        if (lib) rowscale[row] = 1.0f / f;
+        else { rowscale[2 * row] = 1.0f / f; rowscale[2 * row + 1] = 1.0f / f; }
+    }
 }
 
 // The context's GEMM scratch, grown to `need` bytes (work that still uses the old one is waited for first).
@@ -729,9 +736,32 @@ int lib_min_rows() {
     return v;
 }
 
+// The weight's planes [n, 2k] at wp; returns the factor they carry (0: this weight type stays on the fused kernel).
+float expand_planes(axq_ctx *ctx, const axq_weight *w, _Float16 *wp) {
+    GemmArgs a = {};
+    a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
+    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
+    a.n = (int)w->n_rows; a.k = (int)w->k;
+    switch (w->type) {
+    case AXQ_Q4_K: return launch_planes<GQ4K>(ctx, a, wp);
+    case AXQ_Q4_0: return launch_planes<GQ4x<false>>(ctx, a, wp);
+    case AXQ_Q4_1: return launch_planes<GQ4x<true>>(ctx, a, wp);
+    case AXQ_Q5_0: return launch_planes<GQ5x<false>>(ctx, a, wp);
+    case AXQ_Q5_1: return launch_planes<GQ5x<true>>(ctx, a, wp);
+    case AXQ_Q8_0: return launch_planes<GQ80>(ctx, a, wp);
+    default: return 0.f; // plain f16 / f32 weights
+    }
+}
+
+bool library_shape(const axq_weight *w) {
+    const bool quantised = w->type == AXQ_Q4_K || w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q5_0 ||
+                           w->type == AXQ_Q5_1 || w->type == AXQ_Q8_0;
+    return quantised && w->k % BK == 0 && w->n_rows % 4 == 0 && w->n_rows <= INT32_MAX && w->k <= INT32_MAX / 4;
+}
+
 // 1 = done by the library, 0 = not (nothing that matters was enqueued), negative = error
 int gemm_bf16_on_library(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
-    if (w->k % BK != 0 || w->n_rows % 4 != 0 || w->n_rows > INT32_MAX || w->k > INT32_MAX) return 0;
+    if (!library_shape(w)) return 0;
     const int n = (int)w->n_rows, k = (int)w->k;
     const size_t xh_bytes = axq_align_up((size_t)m * k * 4, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
     const size_t planes = axq_align_up((size_t)n * k * 4, 256);
@@ -741,25 +771,48 @@ int gemm_bf16_on_library(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, i
     _Float16 *xh = reinterpret_cast<_Float16 *>(base);
     float *rowscale = reinterpret_cast<float *>(base + xh_bytes);
     _Float16 *wp = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes); // [n, 2k]: the two planes of a row side by side
-    GemmArgs a = {};
-    a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
-    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
-    a.n = n; a.k = k;
-    float ws;
-    switch (w->type) {
-    case AXQ_Q4_K: ws = launch_planes<GQ4K>(ctx, a, wp); break;
-    case AXQ_Q4_0: ws = launch_planes<GQ4x<false>>(ctx, a, wp); break;
-    case AXQ_Q4_1: ws = launch_planes<GQ4x<true>>(ctx, a, wp); break;
-    case AXQ_Q5_0: ws = launch_planes<GQ5x<false>>(ctx, a, wp); break;
-    case AXQ_Q5_1: ws = launch_planes<GQ5x<true>>(ctx, a, wp); break;
-    case AXQ_Q8_0: ws = launch_planes<GQ80>(ctx, a, wp); break;
-    default: return 0; // plain f16 / f32 weights stay on the fused kernel
-    }
+    const float ws = expand_planes(ctx, w, wp);
     gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, k, xh, rowscale, 1);
     AXQ_LAUNCH_CHECK(ctx, "gemm_planes_kernel");
-    if ((rc = axq_blaslt_gemm_f16(ctx, wp, xh, m, n, 2 * k, y)) <= 0) return rc;
+    if ((rc = axq_blaslt_gemm_f16(ctx, wp, 2 * k, xh, 2 * k, m, n, 2 * k, false, y)) <= 0) return rc;
     const size_t total4 = (size_t)m * n / 4;
     gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(y, rowscale, m, n, 1, 1.0f / ws, 1, nullptr, nullptr, y);
+    AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
+    return 1;
+}
+
+// From how many f32 rows on a call goes to the GEMM library (0: never).
+int lib_min_rows_f32() {
+    static const int v = getenv("AXQ_GEMM_LIB_MIN_ROWS_F32") ? atoi(getenv("AXQ_GEMM_LIB_MIN_ROWS_F32")) : 384; // development knob
+    return v;
+}
+
+// f32 activations on the library: x = xh + xl and WS * w = wh + wl in f16, and y = xh wh^T + xh wl^T + xl wh^T (the fourth
+// product is 2^-22 of the result).  Rows of X' are [xh | xh | xl], rows of W' [wh | wl]: one GEMM over the first 2k
+// columns of both, one over k that meets X' + 2k with W' and adds to the first.  The sums land in scratch (resid may
+// be y), gemm_reduce_kernel scales them back and adds bias and residual on the way to y.
+int gemm_f32_on_library(axq_ctx *ctx, const axq_weight *w, const float *x, int m, const float *norm_w, float eps, const float *bias,
+                        const float *resid, float *y) {
+    if (!library_shape(w)) return 0;
+    const int n = (int)w->n_rows, k = (int)w->k;
+    const size_t xh_bytes = axq_align_up((size_t)m * k * 6, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
+    const size_t planes = axq_align_up((size_t)n * k * 4, 256), sums = axq_align_up((size_t)m * n * 4, 256);
+    int rc;
+    if ((rc = reserve_scratch(ctx, xh_bytes + rs_bytes + planes + sums))) return rc;
+    uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
+    _Float16 *xh = reinterpret_cast<_Float16 *>(base);
+    float *rowscale = reinterpret_cast<float *>(base + xh_bytes);
+    _Float16 *wp = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes);
+    float *acc = reinterpret_cast<float *>(base + xh_bytes + rs_bytes + planes);
+    const float ws = expand_planes(ctx, w, wp);
+    gemm_prep_x_f32_kernel<<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, k, xh, rowscale, 1);
+    AXQ_LAUNCH_CHECK(ctx, "gemm_planes_kernel");
+    if ((rc = axq_blaslt_tune_f16(ctx, wp, 2 * k, xh, 3 * k, m, n, 2 * k, acc)) <= 0) return rc;
+    if ((rc = axq_blaslt_gemm_f16(ctx, wp, 2 * k, xh + 2 * (size_t)k, 3 * k, m, n, k, false, acc)) <= 0) return rc;
+    if ((rc = axq_blaslt_gemm_f16(ctx, wp, 2 * k, xh, 3 * k, m, n, 2 * k, true, acc)) <= 0)
+        return rc < 0 ? rc : axq_fail(ctx, AXQ_ERR_BLAS, "the GEMM library dropped a shape between two calls");
+    const size_t total4 = (size_t)m * n / 4;
+    gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(acc, rowscale, m, n, 1, 1.0f / ws, 1, bias, resid, y);
     AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
     return 1;
 }
@@ -790,9 +843,12 @@ int axq_dev_gemm_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int m, c
                      const float *resid, float *y) {
     GemmPlan p;
     int rc;
+    if (lib_min_rows_f32() > 0 && m >= lib_min_rows_f32()) {
+        if ((rc = gemm_f32_on_library(ctx, w, x, m, norm_w, eps, bias, resid, y)) != 0) return rc < 0 ? rc : AXQ_OK;
+    }
     if ((rc = plan_gemm(ctx, w, 2 * m, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     gemm_prep_x_f32_kernel<<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
-                                                       reinterpret_cast<float *>(base + p.xh_bytes));
+                                                       reinterpret_cast<float *>(base + p.xh_bytes), 0);
     return run_gemm(ctx, w, 2 * m, p, y, true, bias, resid);
 }

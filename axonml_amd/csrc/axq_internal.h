@@ -123,8 +123,10 @@ int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int
 int axq_dev_gemv_batch_chain(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
                              const float *bias, const float *resid, float *y, const axq_weight *next, const float *next_aux);
 bool axq_dev_gemv_batch_operands(axq_ctx *ctx, const axq_weight *w, uint8_t **xa, float **xsg);
-// blaslt.hip: y[m, n] = x[m, k] w[n, k]^T on the GEMM library, operands f16; 1 = enqueued, 0 = not available
-int axq_blaslt_gemm_f16(axq_ctx *ctx, const _Float16 *w, const _Float16 *x, int m, int n, int k, float *y);
+// blaslt.hip: y[m, n] = x[m, k] w[n, k]^T (+ y) on the GEMM library, operands f16 with row pitches ldx, ldw;
+// 1 = enqueued, 0 = not available
+int axq_blaslt_gemm_f16(axq_ctx *ctx, const _Float16 *w, int ldw, const _Float16 *x, int ldx, int m, int n, int k, bool accumulate, float *y);
+int axq_blaslt_tune_f16(axq_ctx *ctx, const _Float16 *w, int ldw, const _Float16 *x, int ldx, int m, int n, int k, float *y);
 void axq_blaslt_release(axq_ctx *ctx);
 // sample.hip: every pointer a device pointer; scratch = axq_sample_scratch_bytes(vocab)
 size_t axq_sample_scratch_bytes(int vocab);
