@@ -60,7 +60,9 @@ bool open_api() {
 }
 
 constexpr size_t WORKSPACE_BYTES = 64u << 20;
-constexpr int PLAN_SLOTS = 16;
+constexpr int PLAN_SLOTS = 64;
+constexpr int CHOICE_SLOTS = 256;
+constexpr int ROW_BUCKET = 128; // row counts that round up to the same multiple share a tuned choice
 
 // One (rows, n, k) shape: layouts and the algorithm the library's heuristic picked.
 constexpr int CANDIDATES = 8;
@@ -73,7 +75,15 @@ struct LtPlan {
     int n_heur = 0, best = 0;
 };
 
+// Which of the library's candidates won for a shape; kept per bucket of row counts, so that prompts of every length do
+// not each pay for a tuning run (the candidate lists of neighbouring row counts are the same in practice).
+struct LtChoice {
+    int bucket = 0, n = 0, k = 0, ldw = 0, ldx = 0, best = 0;
+};
+
 struct LtState {
+    LtChoice choices[CHOICE_SLOTS];
+    int n_choices = 0;
     hipblasLtHandle_t handle = nullptr;
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatmulPreference_t pref = nullptr;
@@ -134,6 +144,15 @@ LtPlan *plan_for(LtState *s, int m, int n, int k, int ldw, int ldx) {
             if (p.heur[i].workspaceSize <= WORKSPACE_BYTES) p.heur[p.n_heur++] = p.heur[i];
         p.usable = p.n_heur > 0;
     }
+    const int bucket = (m + ROW_BUCKET - 1) / ROW_BUCKET;
+    for (int i = 0; i < s->n_choices && p.usable; i++) {
+        const LtChoice &c = s->choices[i];
+        if (c.bucket == bucket && c.n == n && c.k == k && c.ldw == ldw && c.ldx == ldx) {
+            p.best = c.best < p.n_heur ? c.best : 0;
+            p.tuned = true;
+            break;
+        }
+    }
     return &p;
 }
 
@@ -172,6 +191,10 @@ bool tune(axq_ctx *ctx, LtState *s, LtPlan *p, const _Float16 *w, const _Float16
         if (timed && (!have || fastest < best_ms)) { have = true; best_ms = fastest; p->best = i; }
     }
     if (!have) p->usable = false;
+    if (have && s->n_choices < CHOICE_SLOTS) {
+        LtChoice &c = s->choices[s->n_choices++];
+        c.bucket = (p->m + ROW_BUCKET - 1) / ROW_BUCKET; c.n = p->n; c.k = p->k; c.ldw = p->ldw; c.ldx = p->ldx; c.best = p->best;
+    }
     return have;
 }
 
