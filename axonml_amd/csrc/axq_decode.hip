@@ -439,6 +439,8 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(const float *part, co
 // rope_append_kernel, grid (kv_heads, tokens), head_dim / 2 threads: RoPE on the new keys, keys and values
 // rounded to f16 into the cache at positions pos0 + b, exactly as the one-token kernel above writes them.
 constexpr int PROMPT_BATCH = 8;
+constexpr int MAX_SEQUENCES = 64;    // sequences side by side
+constexpr int GEMV_GROUPS_MAX = 24;  // up to here a batched step goes in groups of PROMPT_BATCH rows, beyond its linears are GEMMs
 
 __global__ void __launch_bounds__(128) rope_append_kernel(const float *qkv, int qkv_rows, int q_dim, int kv_dim,
                                                           const float *rope_cos, const float *rope_sin, uint16_t *kcache,
@@ -746,37 +748,38 @@ int copy_rows_interleaved(axq_ctx *ctx, axq_weight *dst, const axq_weight *src, 
     return AXQ_OK;
 }
 
-// Attention of the newest token of `nseq` sequences (rows of qkv, qkv_rows apart), split over the positions, and the
-// merge of the splits; results to att (rows n_heads * d apart).
+// Attention of the newest token of the `nseq` sequences from s0 on (rows of qkv, qkv_rows apart), split over the positions,
+// and the merge of the splits; results to att (rows n_heads * d apart).
 template <int D, int REP>
-void launch_attn_partial_t(axq_model *m, int l, const float *qkv, int nseq, hipStream_t st) {
+void launch_attn_partial_t(axq_model *m, int l, const float *qkv, int nseq, int s0, hipStream_t st) {
     const axq_model_config &c = m->cfg;
     const size_t kv_layer = (size_t)c.num_key_value_heads * c.max_position_embeddings * D;
     attn_partial_kernel<D, REP><<<dim3(c.num_key_value_heads, m->max_splits, nseq), 256, 0, st>>>(
-        qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer, m->vcache + (size_t)l * kv_layer, m->pos,
-        c.num_attention_heads, c.num_key_value_heads, c.max_position_embeddings, m->max_splits, c.sliding_window, m->att_part,
-        m->qkv_rows, m->seq_stride, m->part_stride);
+        qkv, m->rope_cos, m->rope_sin, m->kcache + (size_t)l * kv_layer + (size_t)s0 * m->seq_stride,
+        m->vcache + (size_t)l * kv_layer + (size_t)s0 * m->seq_stride, m->pos + s0, c.num_attention_heads, c.num_key_value_heads,
+        c.max_position_embeddings, m->max_splits, c.sliding_window, m->att_part + (size_t)s0 * m->part_stride, m->qkv_rows, m->seq_stride,
+        m->part_stride);
 }
 
 template <int D>
-void launch_attn_partial_d(axq_model *m, int l, const float *qkv, int nseq, hipStream_t st) {
+void launch_attn_partial_d(axq_model *m, int l, const float *qkv, int nseq, int s0, hipStream_t st) {
     const int rep = m->cfg.num_attention_heads / m->cfg.num_key_value_heads;
-    if (rep == 1) launch_attn_partial_t<D, 1>(m, l, qkv, nseq, st);
-    else if (rep == 2) launch_attn_partial_t<D, 2>(m, l, qkv, nseq, st);
-    else if (rep <= 4) launch_attn_partial_t<D, 4>(m, l, qkv, nseq, st);
-    else launch_attn_partial_t<D, 8>(m, l, qkv, nseq, st);
+    if (rep == 1) launch_attn_partial_t<D, 1>(m, l, qkv, nseq, s0, st);
+    else if (rep == 2) launch_attn_partial_t<D, 2>(m, l, qkv, nseq, s0, st);
+    else if (rep <= 4) launch_attn_partial_t<D, 4>(m, l, qkv, nseq, s0, st);
+    else launch_attn_partial_t<D, 8>(m, l, qkv, nseq, s0, st);
 }
 
-void launch_attn_split(axq_model *m, int l, const float *qkv, int nseq, float *att, hipStream_t st, PackOut pk = PackOut()) {
+void launch_attn_split(axq_model *m, int l, const float *qkv, int nseq, float *att, hipStream_t st, PackOut pk = PackOut(), int s0 = 0) {
     const axq_model_config &c = m->cfg;
     switch (c.head_dim) { // axq_model_create admits these four sizes only
-    case 32: launch_attn_partial_d<32>(m, l, qkv, nseq, st); break;
-    case 64: launch_attn_partial_d<64>(m, l, qkv, nseq, st); break;
-    case 128: launch_attn_partial_d<128>(m, l, qkv, nseq, st); break;
-    default: launch_attn_partial_d<256>(m, l, qkv, nseq, st); break;
+    case 32: launch_attn_partial_d<32>(m, l, qkv, nseq, s0, st); break;
+    case 64: launch_attn_partial_d<64>(m, l, qkv, nseq, s0, st); break;
+    case 128: launch_attn_partial_d<128>(m, l, qkv, nseq, s0, st); break;
+    default: launch_attn_partial_d<256>(m, l, qkv, nseq, s0, st); break;
     }
     const size_t comb_lds = (size_t)(2 * m->max_splits + 8) * sizeof(float);
-    attn_combine_kernel<<<dim3(c.num_attention_heads, nseq), 256, comb_lds, st>>>(m->att_part, m->pos, c.num_attention_heads,
+    attn_combine_kernel<<<dim3(c.num_attention_heads, nseq), 256, comb_lds, st>>>(m->att_part + (size_t)s0 * m->part_stride, m->pos + s0, c.num_attention_heads,
                                                                                 c.num_key_value_heads, c.head_dim, m->max_splits,
                                                                                 c.sliding_window, att, m->part_stride, pk);
 }
@@ -957,7 +960,7 @@ struct Rows {
     int mode;            // ROWS_GEMV or ROWS_GEMM
     const int32_t *toks; // [nb] device
     int nb;
-    bool per_seq;        // false: rows pos0.. of sequence `seq`; true: row b is the next token of sequence b (nb = n_seq)
+    bool per_seq;        // false: rows pos0.. of sequence `seq`; true: row b is the next token of sequence seq + b
     int seq, pos0;
     size_t lds;          // of the attention kernel
     bool split_attn;     // per_seq: the positions split over workgroups and merged (long contexts) instead of one workgroup per head
@@ -1040,9 +1043,10 @@ int enqueue_rows(axq_model *m, const Rows &r) {
         }
         return AXQ_OK;
     };
-    const size_t seq_off = r.per_seq ? 0 : (size_t)r.seq * m->seq_stride;
+    const size_t seq_off = (size_t)r.seq * m->seq_stride;
+    const int s0 = r.per_seq ? r.seq : 0; // per_seq: row b is sequence s0 + b
     if (r.per_seq) {
-        record_rows_kernel<<<1, nb, 0, st>>>(m->hist, c.max_position_embeddings, m->pos, r.toks);
+        record_rows_kernel<<<1, nb, 0, st>>>(m->hist + (size_t)s0 * c.max_position_embeddings, c.max_position_embeddings, m->pos + s0, r.toks);
     } else {
         int32_t *hist = m->hist + (size_t)r.seq * c.max_position_embeddings;
         for (int t0 = 0; t0 < nb; t0 += 1024) record_tokens_kernel<<<1, nb - t0 < 1024 ? nb - t0 : 1024, 0, st>>>(hist, r.pos0 + t0, r.toks + t0);
@@ -1069,8 +1073,8 @@ int enqueue_rows(axq_model *m, const Rows &r) {
             pk.even_odd = axq_dev_gemv_batch_operands(ctx, m->w_o[l], &pk.xa, &pk.xsg) ? 1 : 0;
             packed_for = m->w_o[l];
         }
-        if (r.per_seq && r.split_attn) launch_attn_split(m, l, m->pb_qkv, nb, m->pb_att, st, pk);
-        else if (!on_mfma) launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos : nullptr, seq_off, r.lds, m->pb_att, st, pk);
+        if (r.per_seq && r.split_attn) launch_attn_split(m, l, m->pb_qkv, nb, m->pb_att, st, pk, s0);
+        else if (!on_mfma) launch_attn_rows(m, l, m->pb_qkv, nb, r.pos0, r.per_seq ? m->pos + s0 : nullptr, seq_off, r.lds, m->pb_att, st, pk);
         if ((rc = lin(m->w_o[l], m->pb_att, AXQ_X_PLAIN, nullptr, m->pb_h, m->pb_h, m->w_gu[l], m->norm_ffn + (size_t)l * H))) return rc;
         if ((rc = lin(m->w_gu[l], m->pb_h, AXQ_X_RMSNORM, m->norm_ffn + (size_t)l * H, nullptr, m->pb_gu, nullptr, nullptr))) return rc;
         if ((rc = lin(m->w_down[l], m->pb_gu, AXQ_X_SWIGLU, nullptr, m->pb_h, m->pb_h, l + 1 < c.num_hidden_layers ? m->w_qkv[l + 1] : nullptr,
@@ -1078,8 +1082,9 @@ int enqueue_rows(axq_model *m, const Rows &r) {
     }
     if (r.per_seq) {
         norm_kernel<<<nb, 1024, 0, st>>>(m->pb_h, m->norm_final, H, c.rms_norm_eps, m->pb_xn);
-        if ((rc = axq_dev_gemv(ctx, m->w_head, m->pb_xn, nb, nullptr, m->logits))) return rc;
-        argmax_kernel<<<nb, 1024, 0, st>>>(m->logits, c.vocab_size, m->next, m->pos);
+        float *logits = m->logits + (size_t)s0 * c.vocab_size;
+        if ((rc = axq_dev_gemv(ctx, m->w_head, m->pb_xn, nb, nullptr, logits))) return rc;
+        argmax_kernel<<<nb, 1024, 0, st>>>(logits, c.vocab_size, m->next + s0, m->pos + s0);
     } else {
         add_i32_kernel<<<1, 1, 0, st>>>(m->pos + r.seq, nb);
     }
@@ -1141,7 +1146,26 @@ int run_batch_step(axq_model *m, int max_pos_now) {
     r.lds = prompt_attn_lds(m, r.split_attn ? 1 : m->fused_max);
     static const bool no_graph = getenv("AXQ_DECODE_GRAPH") && getenv("AXQ_DECODE_GRAPH")[0] == '0';
     int rc;
-    if (no_graph) {
+    if (m->n_seq > PROMPT_BATCH && m->n_seq <= GEMV_GROUPS_MAX && all_layers_in_small_batch_reach(m, PROMPT_BATCH)) {
+        // a few more rows than the small-batch GEMV takes: groups of eight sequences, one after the other (three passes
+        // over the weights at 2.4 ms each still beat the GEMM's 8.5-10 ms at the 7B shape); plain launches
+        rc = AXQ_OK;
+        for (int s = 0; s < m->n_seq && !rc; s += PROMPT_BATCH) {
+            Rows g = r;
+            g.seq = s; g.toks = m->tok + s;
+            g.nb = m->n_seq - s < PROMPT_BATCH ? m->n_seq - s : PROMPT_BATCH;
+            rc = enqueue_rows(m, g);
+        }
+    } else if (m->n_seq > PROMPT_BATCH) {
+        // many more: the linears are GEMMs on f32 rows (which size their scratch as they go, so no graph: a step of so
+        // many rows is long against its launches anyway)
+        r.mode = ROWS_GEMM;
+        if (!rows_mode_covers(m, ROWS_GEMM, 1, r.nb))
+            return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: more than %d sequences need linears the GEMM covers (K a multiple of 64)",
+                            PROMPT_BATCH);
+        if ((rc = reserve_prompt_rows(m, r.nb))) return rc;
+        rc = enqueue_rows(m, r);
+    } else if (no_graph) {
         rc = enqueue_rows(m, r);
     } else {
         hipGraphExec_t &exec = r.split_attn ? m->graph_b : m->graph_bf;
@@ -1239,7 +1263,7 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     TRY(dev_alloc(&m->att_part, m->part_stride));
     TRY(dev_alloc(&m->gu, (size_t)2 * I)); TRY(dev_alloc(&m->act, I)); TRY(dev_alloc(&m->logits, c.vocab_size));
     m->pb_cap = PROMPT_BATCH;
-    TRY(dev_alloc(&m->pb_h, (size_t)PROMPT_BATCH * H)); TRY(dev_alloc(&m->pb_xn, (size_t)PROMPT_BATCH * (H > I ? H : I)));
+    TRY(dev_alloc(&m->pb_h, (size_t)PROMPT_BATCH * H)); TRY(dev_alloc(&m->pb_xn, (size_t)MAX_SEQUENCES * (H > I ? H : I))); // normalised rows in front of the lm_head and of linears outside the GEMV's reach
     TRY(dev_alloc(&m->pb_qkv, (size_t)PROMPT_BATCH * m->qkv_rows)); TRY(dev_alloc(&m->pb_att, (size_t)PROMPT_BATCH * m->q_dim));
     TRY(dev_alloc(&m->pb_gu, (size_t)PROMPT_BATCH * 2 * I)); TRY(dev_alloc(&m->pb_act, (size_t)PROMPT_BATCH * I));
     TRY(dev_alloc(&m->pos, 1)); TRY(dev_alloc(&m->tok, 1)); TRY(dev_alloc(&m->next, 1)); TRY(dev_alloc(&m->gen, 1));
@@ -1438,8 +1462,9 @@ int axq_model_set_batch(axq_model *m, int n_seq) {
     if (!m) return AXQ_ERR_INVALID_ARGUMENT;
     axq_ctx *ctx = m->ctx;
     const axq_model_config &c = m->cfg;
-    if (n_seq < 1 || n_seq > PROMPT_BATCH)
-        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_set_batch: 1 to %d sequences, got %d", PROMPT_BATCH, n_seq);
+    if (n_seq < 1 || n_seq > MAX_SEQUENCES)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_model_set_batch: 1 to %d sequences, got %d", MAX_SEQUENCES, n_seq);
+
     if (n_seq > 1 && (c.vocab_size % 4 != 0 || prompt_attn_lds(m, c.max_position_embeddings) > 128 * 1024))
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH,
                         "Shape mismatch: batched steps need a vocabulary that is a multiple of 4 and at most 32768 positions "

@@ -82,7 +82,7 @@ class QuantizedLlama:
         return nxt.value, logits
 
     def set_batch(self, n_seq):
-        """Caches and positions for n_seq sequences side by side (1..8); starts all of them afresh."""
+        """Caches and positions for n_seq sequences side by side (1..64); starts all of them afresh."""
         self.ctx.check(self.ctx.lib.axq_model_set_batch(self.handle, int(n_seq)))
 
     def batch(self):

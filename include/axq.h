@@ -216,8 +216,9 @@ AXQ_API int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_
  * rounding (sums are taken in another order). */
 AXQ_API int axq_model_forward_tokens(axq_model *m, const int32_t *tokens, int n, float *logits, int32_t *next_token);
 /* Several sequences side by side (the batch dimension of forward_with_cache's input ids and of KVCache,
- * llama.rs:731-762, attention.rs:28-35): n_seq = 1..8 caches and position counters; a batched step feeds
- * one token of every sequence and reads the weights once for all of them.  Calling it discards every
+ * llama.rs:731-762, attention.rs:28-35): n_seq = 1..64 caches and position counters; a batched step feeds
+ * one token of every sequence and reads the weights once for all of them (up to eight sequences through the
+ * small-batch GEMV as a replayed graph, more through the GEMM on f32 rows, which needs K a multiple of 64).  Calling it discards every
  * cache and starts all sequences at position 0.  The one-sequence calls above keep working on sequence 0. */
 AXQ_API int axq_model_set_batch(axq_model *m, int n_seq);
 AXQ_API int axq_model_batch(const axq_model *m);

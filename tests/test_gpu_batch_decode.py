@@ -28,14 +28,16 @@ def _oracle_walk(cpu, prompt, n_new):
                                               (4, o.Q5_1, {}),  # outside the small-batch GEMV: rows go one by one
                                               (8, o.Q4_K, dict(num_heads=8, num_kv_heads=2, head_dim=32)),
                                               (3, o.Q4_1, dict(num_heads=2, num_kv_heads=1, head_dim=128)),
-                                              (4, o.Q4_K, dict(sliding_window=6)), (1, o.Q4_K, {})])
+                                              (4, o.Q4_K, dict(sliding_window=6)), (1, o.Q4_K, {}),
+                                              # more than eight: the linears of a step are GEMMs on f32 rows
+                                              (9, o.Q4_K, {}), (24, o.Q4_0, dict(num_heads=8, num_kv_heads=2, head_dim=32)), (44, o.Q5_1, {})])
 def test_generate_batch_matches_the_oracle_sequence_by_sequence(ctx, n_seq, qtype, over):
     c = tiny_config(max_seq_len=96, **over)
     w = random_weights(c, 200 + n_seq + qtype, qtype=qtype)
     cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
     gpu.set_batch(n_seq)
     rng = np.random.default_rng(n_seq)
-    lengths = [1, 2, 9, 40, 17, 3, 64, 10][:n_seq]  # ragged: one token, GEMV rows, GEMM rows
+    lengths = [[1, 2, 9, 40, 17, 3, 64, 10][i % 8] + i // 8 for i in range(n_seq)]  # ragged: one token, GEMV rows, GEMM rows
     prompts = [rng.integers(0, c["vocab_size"], size=n) for n in lengths]
     n_new = 14
     got, pre_ms, dec_ms = gpu.generate_batch(prompts, n_new)
@@ -123,7 +125,7 @@ def test_batch_errors(ctx):
     with pytest.raises(q.QuantError):
         m.set_batch(0)
     with pytest.raises(q.QuantError):
-        m.set_batch(9)
+        m.set_batch(65)
     m.set_batch(2)
     assert m.batch() == 2
     with pytest.raises(ValueError):
