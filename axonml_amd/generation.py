@@ -147,12 +147,12 @@ def beam_search_generate(model, input_ids, beam_search, max_new_tokens, batched=
     """Beam search over a `QuantizedLlama`: per step every live beam's next-token logits, then
     `expand_beams`, until `max_new_tokens` or `should_stop`.  Returns (best_sequence, beams).
 
-    batched (default: when the model can and there are 2..8 beams): every beam lives in a sequence slot of the
+    batched (default: when the model can and there are 2..64 beams): every beam lives in a sequence slot of the
     model and one batched step serves all of them; a beam that forks copies its slot (`copy_sequence`).
     Otherwise the model keeps one sequence, and a beam is brought in by rewinding the cache to the prefix it
     shares with the cached tokens and feeding the rest (`truncate`, `forward_tokens`)."""
     if batched is None:
-        batched = hasattr(model, "forward_batch") and 2 <= beam_search.num_beams <= 8
+        batched = hasattr(model, "forward_batch") and 2 <= beam_search.num_beams <= 64
     if batched:
         return _beam_search_batched(model, input_ids, beam_search, max_new_tokens)
     beams = beam_search.init_beams(input_ids)

@@ -84,7 +84,7 @@ class _OracleSequenceModel:
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("batched", [False, True])
-@pytest.mark.parametrize("num_beams,length_penalty", [(1, 1.0), (3, 1.0), (4, 0.0), (8, 1.5), (2, 1.0)])
+@pytest.mark.parametrize("num_beams,length_penalty", [(1, 1.0), (3, 1.0), (4, 0.0), (8, 1.5), (2, 1.0), (11, 1.0)])
 def test_driver_against_the_oracle(ctx, num_beams, length_penalty, batched):
     """batched: every beam in a sequence slot of the model, one batched step per search step, forks copy their slot;
     otherwise one sequence, rewound and re-fed per beam.  Both against the same bookkeeping over the CPU oracle."""
