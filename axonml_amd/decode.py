@@ -207,5 +207,14 @@ def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
     _, _, dec_bs = m.generate_batch(prompts, new_tokens)
     res["batch8_sampled_tokens_per_s"] = 8 * new_tokens / (dec_bs * 1e-3)
     log(f"  8 sequences with top-k/top-p sampling: {res['batch8_sampled_tokens_per_s']:.0f} tok/s in all")
+    # 64 sequences: the linears of a step are GEMMs on f32 rows
+    m.set_sampling(None)
+    m.set_batch(64)
+    prompts = [rng.integers(0, cfg["vocab_size"], size=prompt_len, dtype=np.int32) for _ in range(64)]
+    m.generate_batch([p[:8] for p in prompts], 4)
+    _, pre_b, dec_b = m.generate_batch(prompts, new_tokens)
+    res["batch64_tokens_per_s"] = 64 * new_tokens / (dec_b * 1e-3)
+    res["batch64_ms_per_step"] = dec_b / new_tokens
+    log(f"  64 sequences: {res['batch64_tokens_per_s']:.0f} tok/s in all ({res['batch64_ms_per_step']:.3f} ms per step)")
     m.close()
     return res
