@@ -215,7 +215,6 @@ void axq_destroy(axq_ctx *ctx) {
     (void)hipStreamDestroy(ctx->own_stream);
     (void)hipFree(ctx->xq);
     if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
-    axq_blaslt_release(ctx);
     free(ctx);
 }
 

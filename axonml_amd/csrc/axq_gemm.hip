@@ -425,8 +425,7 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
 }
 
 // bf16 rows -> f16 rows scaled by a power of two (largest magnitude below 2^15), and the scale to undo it.
-// dup: every output row holds the scaled row twice (2k halfs), for a product with the two planes of a weight side by side.
-__global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int m, int k, _Float16 *xh, float *rowscale, int dup) {
+__global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int m, int k, _Float16 *xh, float *rowscale) {
     __shared__ float red[4];
     const int row = blockIdx.x;
     const uint16_t *xr = x + (size_t)row * k;
@@ -449,13 +448,7 @@ __global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int
     const float f = __builtin_bit_cast(float, (uint32_t)sb << 23);
     for (int i = threadIdx.x; i < k; i += blockDim.x) {
         float v = __builtin_bit_cast(float, (uint32_t)xr[i] << 16);
-        const _Float16 hv = (_Float16)(v * f);
-        if (dup) {
-            xh[(size_t)row * 2 * k + i] = hv;
-            xh[(size_t)row * 2 * k + k + i] = hv;
-        } else {
-            xh[(size_t)row * k + i] = hv;
-        }
+        xh[(size_t)row * k + i] = (_Float16)(v * f);
     }
     if (threadIdx.x == 0) rowscale[row] = 1.0f / f;
 }
@@ -514,9 +507,8 @@ int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
 // f32 rows, optionally RMS-normalised on the way ((x * inv_rms) * norm_w, RMSNorm::forward, llm/src/llama.rs:158-187),
 // -> two f16 rows each under one power-of-two scale: row 2t holds the leading 11 bits of every element, row 2t + 1
 // what those leave, so that their GEMM results add up to the f32 product (the GEMM's epilogue adds them: pair mode).
-// lib: the layout for the GEMM library instead: row t of xh is [hi | hi | lo] (3k halfs) and has one scale.
 __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, const float *norm_w, float eps, int m, int k,
-                                                              _Float16 *xh, float *rowscale, int lib) {
+                                                              _Float16 *xh, float *rowscale) {
     // the row stays in registers between the passes: 16 bytes per thread and step, up to 16 steps (k <= 16384);
     // longer rows (or k not a multiple of 4) take the plain loops below
     constexpr int STEPS = 16;
@@ -591,8 +583,7 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
     int sb = 127 + 14 - (eb - 127);
     sb = sb < 1 ? 1 : (sb > 254 ? 254 : sb);
     const float f = __builtin_bit_cast(float, (uint32_t)sb << 23);
-    _Float16 *hi_row = lib ? xh + (size_t)row * 3 * k : xh + (size_t)(2 * row) * k, *lo_row = lib ? hi_row + 2 * k : hi_row + k;
-    _Float16 *hi2_row = hi_row + k; // lib only
+    _Float16 *hi_row = xh + (size_t)(2 * row) * k, *lo_row = hi_row + k;
     if (in_regs) {
 #pragma unroll
         for (int c = 0; c < STEPS; c++) {
@@ -604,7 +595,6 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
                 for (int j = 0; j < 4; j++) { h[j] = (_Float16)e[j]; l[j] = (_Float16)(e[j] - (float)h[j]); }
                 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
                 reinterpret_cast<half4 *>(hi_row)[i4] = half4{h[0], h[1], h[2], h[3]};
-                if (lib) reinterpret_cast<half4 *>(hi2_row)[i4] = half4{h[0], h[1], h[2], h[3]};
                 reinterpret_cast<half4 *>(lo_row)[i4] = half4{l[0], l[1], l[2], l[3]};
             }
         }
@@ -613,13 +603,12 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
             const float e = (norm_w ? (xr[i] * inv) * norm_w[i] : xr[i]) * f;
             const _Float16 hi = (_Float16)e;
             hi_row[i] = hi;
-            if (lib) hi2_row[i] = hi;
             lo_row[i] = (_Float16)(e - (float)hi);
         }
     }
     if (threadIdx.x == 0) {
-        if (lib) rowscale[row] = 1.0f / f;
-        else { rowscale[2 * row] = 1.0f / f; rowscale[2 * row + 1] = 1.0f / f; }
+        rowscale[2 * row] = 1.0f / f;
+        rowscale[2 * row + 1] = 1.0f / f;
     }
 }
 
@@ -691,144 +680,15 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     }
 }
 
-// ---------------------------------------------------------------------------
-// Many rows: the weight expanded once per call into the two f16 planes that the kernel above builds tile by tile
-// (WS * w = wh + wl, split8_f16) for the GEMM library (axq_blaslt.hip): row r of the expanded weight is [wh_r | wl_r],
-// the row-scaled f16 activations are written twice per row, [x | x], and one library GEMM over 2k puts
-// x wh^T + x wl^T into the f32 output; gemm_reduce_kernel then undoes the scales in place.
-// Thread = one 16-weight unit of the traits above.
-// ---------------------------------------------------------------------------
-template <class T>
-__global__ void __launch_bounds__(256) gemm_planes_kernel(GemmArgs a, _Float16 *wp) {
-    const size_t unit = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const int units_per_row = a.k >> 4;
-    const size_t row = unit / (size_t)units_per_row;
-    if (row >= (size_t)a.n) return;
-    const int in_row = (int)(unit - row * (size_t)units_per_row), kstep = in_row >> 2, u4 = in_row & 3;
-    typename T::Raw raw;
-    T::load16(a, row, kstep, u4, raw);
-    float w[16];
-    int k0, k1;
-    T::cvt16(raw, kstep, u4, w, k0, k1);
-    const float sc = T::PRESCALED ? 1.0f : T::WS;
-    uint4 h0, l0, h1, l1;
-    split8_f16(w, sc, h0, l0);
-    split8_f16(w + 8, sc, h1, l1);
-    _Float16 *wh = wp + row * 2 * (size_t)a.k + (size_t)kstep * BK, *wl = wh + a.k;
-    *reinterpret_cast<uint4 *>(wh + k0) = h0;
-    *reinterpret_cast<uint4 *>(wh + k1) = h1;
-    *reinterpret_cast<uint4 *>(wl + k0) = l0;
-    *reinterpret_cast<uint4 *>(wl + k1) = l1;
-}
-
-template <class T>
-float launch_planes(axq_ctx *ctx, const GemmArgs &a, _Float16 *wp) {
-    const size_t units = (size_t)a.n * (size_t)(a.k >> 4);
-    gemm_planes_kernel<T><<<(unsigned)((units + 255) / 256), 256, 0, ctx->stream>>>(a, wp);
-    return T::WS;
-}
-
-// From how many rows on a bf16 call goes to the GEMM library (0: never).  Below, expanding the weight and the extra
-// pass over the output cost more than the library's faster multiplication saves (at 512 rows the kernel above wins
-// by 2-7 %, at 768 the library by 15-47 %, at 2048 by 20-50 %).
-int lib_min_rows() {
-    static const int v = getenv("AXQ_GEMM_LIB_MIN_ROWS") ? atoi(getenv("AXQ_GEMM_LIB_MIN_ROWS")) : 640; // development knob
-    return v;
-}
-
-// The weight's planes [n, 2k] at wp; returns the factor they carry (0: this weight type stays on the fused kernel).
-float expand_planes(axq_ctx *ctx, const axq_weight *w, _Float16 *wp) {
-    GemmArgs a = {};
-    a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
-    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
-    a.n = (int)w->n_rows; a.k = (int)w->k;
-    switch (w->type) {
-    case AXQ_Q4_K: return launch_planes<GQ4K>(ctx, a, wp);
-    case AXQ_Q4_0: return launch_planes<GQ4x<false>>(ctx, a, wp);
-    case AXQ_Q4_1: return launch_planes<GQ4x<true>>(ctx, a, wp);
-    case AXQ_Q5_0: return launch_planes<GQ5x<false>>(ctx, a, wp);
-    case AXQ_Q5_1: return launch_planes<GQ5x<true>>(ctx, a, wp);
-    case AXQ_Q8_0: return launch_planes<GQ80>(ctx, a, wp);
-    default: return 0.f; // plain f16 / f32 weights
-    }
-}
-
-bool library_shape(const axq_weight *w) {
-    const bool quantised = w->type == AXQ_Q4_K || w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q5_0 ||
-                           w->type == AXQ_Q5_1 || w->type == AXQ_Q8_0;
-    return quantised && w->k % BK == 0 && w->n_rows % 4 == 0 && w->n_rows <= INT32_MAX && w->k <= INT32_MAX / 4;
-}
-
-// 1 = done by the library, 0 = not (nothing that matters was enqueued), negative = error
-int gemm_bf16_on_library(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
-    if (!library_shape(w)) return 0;
-    const int n = (int)w->n_rows, k = (int)w->k;
-    const size_t xh_bytes = axq_align_up((size_t)m * k * 4, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
-    const size_t planes = axq_align_up((size_t)n * k * 4, 256);
-    int rc;
-    if ((rc = reserve_scratch(ctx, xh_bytes + rs_bytes + planes))) return rc;
-    uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
-    _Float16 *xh = reinterpret_cast<_Float16 *>(base);
-    float *rowscale = reinterpret_cast<float *>(base + xh_bytes);
-    _Float16 *wp = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes); // [n, 2k]: the two planes of a row side by side
-    const float ws = expand_planes(ctx, w, wp);
-    gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, k, xh, rowscale, 1);
-    AXQ_LAUNCH_CHECK(ctx, "gemm_planes_kernel");
-    if ((rc = axq_blaslt_gemm_f16(ctx, wp, 2 * k, xh, 2 * k, m, n, 2 * k, false, y)) <= 0) return rc;
-    const size_t total4 = (size_t)m * n / 4;
-    gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(y, rowscale, m, n, 1, 1.0f / ws, 1, nullptr, nullptr, y);
-    AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
-    return 1;
-}
-
-// From how many f32 rows on a call goes to the GEMM library (0: never).
-int lib_min_rows_f32() {
-    static const int v = getenv("AXQ_GEMM_LIB_MIN_ROWS_F32") ? atoi(getenv("AXQ_GEMM_LIB_MIN_ROWS_F32")) : 384; // development knob
-    return v;
-}
-
-// f32 activations on the library: x = xh + xl and WS * w = wh + wl in f16, and y = xh wh^T + xh wl^T + xl wh^T (the fourth
-// product is 2^-22 of the result).  Rows of X' are [xh | xh | xl], rows of W' [wh | wl]: one GEMM over the first 2k
-// columns of both, one over k that meets X' + 2k with W' and adds to the first.  The sums land in scratch (resid may
-// be y), gemm_reduce_kernel scales them back and adds bias and residual on the way to y.
-int gemm_f32_on_library(axq_ctx *ctx, const axq_weight *w, const float *x, int m, const float *norm_w, float eps, const float *bias,
-                        const float *resid, float *y) {
-    if (!library_shape(w)) return 0;
-    const int n = (int)w->n_rows, k = (int)w->k;
-    const size_t xh_bytes = axq_align_up((size_t)m * k * 6, 256), rs_bytes = axq_align_up((size_t)m * 4, 256);
-    const size_t planes = axq_align_up((size_t)n * k * 4, 256), sums = axq_align_up((size_t)m * n * 4, 256);
-    int rc;
-    if ((rc = reserve_scratch(ctx, xh_bytes + rs_bytes + planes + sums))) return rc;
-    uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
-    _Float16 *xh = reinterpret_cast<_Float16 *>(base);
-    float *rowscale = reinterpret_cast<float *>(base + xh_bytes);
-    _Float16 *wp = reinterpret_cast<_Float16 *>(base + xh_bytes + rs_bytes);
-    float *acc = reinterpret_cast<float *>(base + xh_bytes + rs_bytes + planes);
-    const float ws = expand_planes(ctx, w, wp);
-    gemm_prep_x_f32_kernel<<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, k, xh, rowscale, 1);
-    AXQ_LAUNCH_CHECK(ctx, "gemm_planes_kernel");
-    if ((rc = axq_blaslt_tune_f16(ctx, wp, 2 * k, xh, 3 * k, m, n, 2 * k, acc)) <= 0) return rc;
-    if ((rc = axq_blaslt_gemm_f16(ctx, wp, 2 * k, xh + 2 * (size_t)k, 3 * k, m, n, k, false, acc)) <= 0) return rc;
-    if ((rc = axq_blaslt_gemm_f16(ctx, wp, 2 * k, xh, 3 * k, m, n, 2 * k, true, acc)) <= 0)
-        return rc < 0 ? rc : axq_fail(ctx, AXQ_ERR_BLAS, "the GEMM library dropped a shape between two calls");
-    const size_t total4 = (size_t)m * n / 4;
-    gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(acc, rowscale, m, n, 1, 1.0f / ws, 1, bias, resid, y);
-    AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
-    return 1;
-}
-
 } // namespace
 
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
     GemmPlan p;
     int rc;
-    if (lib_min_rows() > 0 && m >= lib_min_rows()) {
-        if ((rc = gemm_bf16_on_library(ctx, w, x, m, y)) != 0) return rc < 0 ? rc : AXQ_OK;
-    }
     if ((rc = plan_gemm(ctx, w, m, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
-                                                   reinterpret_cast<float *>(base + p.xh_bytes), 0);
+                                                   reinterpret_cast<float *>(base + p.xh_bytes));
     return run_gemm(ctx, w, m, p, y);
 }
 
@@ -843,12 +703,9 @@ int axq_dev_gemm_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int m, c
                      const float *resid, float *y) {
     GemmPlan p;
     int rc;
-    if (lib_min_rows_f32() > 0 && m >= lib_min_rows_f32()) {
-        if ((rc = gemm_f32_on_library(ctx, w, x, m, norm_w, eps, bias, resid, y)) != 0) return rc < 0 ? rc : AXQ_OK;
-    }
     if ((rc = plan_gemm(ctx, w, 2 * m, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     gemm_prep_x_f32_kernel<<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
-                                                       reinterpret_cast<float *>(base + p.xh_bytes), 0);
+                                                       reinterpret_cast<float *>(base + p.xh_bytes));
     return run_gemm(ctx, w, 2 * m, p, y, true, bias, resid);
 }

@@ -23,7 +23,6 @@ struct axq_ctx {
     int gemv_wgs_per_cu; // GEMV workgroups per compute unit that the rows are spread over
     void *gemm_scratch; // device scratch of the prefill GEMM (scaled f16 activations + row scales), grown on demand
     size_t gemm_scratch_bytes;
-    void *blaslt;       // state of the GEMM library route of the prefill GEMM (axq_blaslt.hip), made at first use
     char err[512];
 };
 
@@ -123,11 +122,6 @@ int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int
 int axq_dev_gemv_batch_chain(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
                              const float *bias, const float *resid, float *y, const axq_weight *next, const float *next_aux);
 bool axq_dev_gemv_batch_operands(axq_ctx *ctx, const axq_weight *w, uint8_t **xa, float **xsg);
-// blaslt.hip: y[m, n] = x[m, k] w[n, k]^T (+ y) on the GEMM library, operands f16 with row pitches ldx, ldw;
-// 1 = enqueued, 0 = not available
-int axq_blaslt_gemm_f16(axq_ctx *ctx, const _Float16 *w, int ldw, const _Float16 *x, int ldx, int m, int n, int k, bool accumulate, float *y);
-int axq_blaslt_tune_f16(axq_ctx *ctx, const _Float16 *w, int ldw, const _Float16 *x, int ldx, int m, int n, int k, float *y);
-void axq_blaslt_release(axq_ctx *ctx);
 // sample.hip: every pointer a device pointer; scratch = axq_sample_scratch_bytes(vocab)
 size_t axq_sample_scratch_bytes(int vocab);
 int axq_check_sampling_config(axq_ctx *ctx, const axq_sampling_config *cfg);

@@ -220,10 +220,17 @@ class QuantizedTensor:
         return self.data[i * bb:(i + 1) * bb]
 
 
+def _quant_type(v):
+    try:
+        return QuantType(v)
+    except ValueError:
+        raise InvalidQuantType(f"Invalid quantization type: {v}")
+
+
 def quantize_tensor(tensor, quant_type, ctx=None):
     """quantize.rs:36-54: f32 tensor -> QuantizedTensor, blocks along the flat row-major buffer."""
     ctx = ctx or default_context()
-    quant_type = QuantType(quant_type)
+    quant_type = _quant_type(quant_type)
     t = np.ascontiguousarray(tensor, dtype=np.float32)
     out = np.empty(ctx.lib.axq_packed_bytes(int(quant_type), t.size), dtype=np.uint8)
     ctx.check(ctx.lib.axq_quantize(ctx.handle, int(quant_type), t.ctypes.data, t.size, out.ctypes.data, MEM_HOST))

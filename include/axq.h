@@ -75,7 +75,7 @@ typedef enum {
     AXQ_ERR_COPY_FAILED = -22,
     AXQ_ERR_KERNEL_LAUNCH_FAILED = -23,
     AXQ_ERR_DRIVER = -24,
-    AXQ_ERR_BLAS = -25, /* BlasError: the GEMM library refused a call */
+    AXQ_ERR_BLAS = -25, /* BlasError (kept for the mirror; this library calls no BLAS) */
     /* boundary misuse (NULL handle or pointer, bad flag) */
     AXQ_ERR_INVALID_ARGUMENT = -30
 } axq_status;

@@ -162,7 +162,6 @@ def test_small_batch_reads_weights_once(ctx, qtype, batch, n, k):
 
 # ---- many vectors: f32 rows through the matrix-pipe GEMM as two f16 rows each
 @pytest.mark.parametrize("qtype", [o.Q4_K, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.F16, o.F32])
-# (from 384 rows on the quantised types go through the GEMM library: three products of f16 planes)
 @pytest.mark.parametrize("batch,n,k", [(40, 96, 512), (64, 100, 1024), (130, 33, 4096), (9, 64, 2048), (300, 257, 768), (384, 132, 512),
                                        (777, 64, 1024)])
 def test_many_vectors_go_through_the_gemm_at_f32_accuracy(ctx, qtype, batch, n, k):
