@@ -89,6 +89,7 @@ SIGNATURES = {
     "axq_weight_info": (_i, [_vp, C.POINTER(_i), C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_sz)]),
     "axq_weight_free": (None, [_vp, _vp]),
     "axq_gemv_f32": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i]),
+    "axq_gemv_f32_static": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
     "axq_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _vp, _i]),
     "axq_model_create": (_i, [_vp, C.POINTER(ModelConfig), C.POINTER(_vp)]),
     "axq_model_free": (None, [_vp]),

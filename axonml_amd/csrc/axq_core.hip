@@ -188,8 +188,14 @@ int axq_init(int device, axq_ctx **out) {
     ctx->fp8_unit_inv = 1.0f / h[0];
     {
         // one vector split, or a small batch packed plus the partial sums of its split K
-        size_t xq_bytes = axq_xq_bytes(AXQ_XQ_MAX_K), mb_bytes = (size_t)34 * AXQ_BATCH_MAX_K + (size_t)4 * 8 * AXQ_BATCH_SPLIT_ROWS * 4;
+        size_t xq_bytes = axq_xq_bytes(AXQ_XQ_MAX_K), mb_bytes = AXQ_BATCH_SCRATCH_BYTES;
         INIT_HIP(hipMalloc((void **)&ctx->xq, xq_bytes > mb_bytes ? xq_bytes : mb_bytes));
+    }
+    if (axq_gemv_static_setup(ctx) != AXQ_OK) { // this device's copy of the scratch of axq_gemv_f32_static
+        axq_fail(NULL, AXQ_ERR_DRIVER, "%s", ctx->err);
+        (void)hipFree(ctx->xq);
+        free(ctx);
+        return AXQ_ERR_DRIVER;
     }
     // A lone GEMV call splits x inside the kernel (one launch); callers that produce x on the device
     // hand over the split form instead.  AXQ_GEMV_PREP=separate forces the two-kernel form (development).

@@ -16,6 +16,8 @@
 
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "axq_internal.h"
 #include "axq_split.h"
 
@@ -430,7 +432,7 @@ __global__ void __launch_bounds__(512) mb_reduce_pack_kernel(const float *src, i
 // next_even_odd < 0: nothing follows.  Otherwise y is the input of another small-batch GEMV whose operands
 // (EVEN_ODD as given, RMSNorm with next_aux when that is not null) are prepared here, in the same scratch.
 template <class T>
-void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *aux, float eps, int next_even_odd, const float *next_aux) {
+void launch_mb(axq_ctx *ctx, MbArgs a, uint8_t *sc, const float *x, int xmode, const float *aux, float eps, int next_even_odd, const float *next_aux) {
     const dim3 pgrid((unsigned)((a.k / 8 + 255) / 256), MAX_BATCH);
     uint8_t *xa = const_cast<uint8_t *>(a.xa);
     float *xsg = const_cast<float *>(a.xsg);
@@ -462,8 +464,8 @@ void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *a
     gemv_mb_kernel<T><<<dim3(tiles, splits), 64 * S, lds, ctx->stream>>>(a);
     if (next_even_odd >= 0) {
         // y's operands for the next GEMV (k' = n_rows): the scratch layout of that call
-        uint8_t *nxa = ctx->xq;
-        float *nxsg = reinterpret_cast<float *>(ctx->xq + (size_t)32 * a.n_rows);
+        uint8_t *nxa = sc;
+        float *nxsg = reinterpret_cast<float *>(sc + (size_t)32 * a.n_rows);
         const float *src = splits > 1 ? a.ypart : a.y;
         const int nsp = splits > 1 ? (int)splits : 0;
         if (next_even_odd)
@@ -474,6 +476,31 @@ void launch_mb(axq_ctx *ctx, MbArgs a, const float *x, int xmode, const float *a
         const int total = a.n_rows * a.batch;
         mb_reduce_kernel<<<(total + 255) / 256, 256, 0, ctx->stream>>>(a.ypart, a.bias, a.resid, a.n_rows, a.batch, (int)splits, a.y);
     }
+}
+
+// One call of the small-batch GEMV with its scratch at `sc` (AXQ_BATCH_SCRATCH_BYTES bytes): 32 k bytes of A operands,
+// then 2 * (k / 32) * 8 floats of scales and sums; behind AXQ_BATCH_MAX_K's worth of those the partial sums of a split
+// K (splits only happen below AXQ_BATCH_SPLIT_ROWS rows).  Every byte that a kernel reads there is written earlier in
+// the same call, so the buffer needs no clearing between calls.
+int gemv_batch_in(axq_ctx *ctx, uint8_t *sc, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
+                  const float *bias, const float *resid, float *y, int next_even_odd, const float *next_aux) {
+    const int k = (int)w->k;
+    MbArgs a;
+    a.codes = w->codes; a.meta = w->meta;
+    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch;
+    a.xa = sc; a.xsg = reinterpret_cast<float *>(sc + (size_t)32 * k);
+    a.bias = bias; a.resid = resid; a.y = y;
+    a.ypart = w->n_rows <= AXQ_BATCH_SPLIT_ROWS ? reinterpret_cast<float *>(sc + (size_t)34 * AXQ_BATCH_MAX_K) : nullptr;
+    a.n_rows = (int)w->n_rows; a.k = k; a.batch = batch;
+    switch (w->type) {
+    case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q4_1: launch_mb<MQ4x<true>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q8_0: launch_mb<MQ80>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q4_K: launch_mb<MQ4K>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
+    }
+    AXQ_LAUNCH_CHECK(ctx, "gemv_mb_kernel");
+    return AXQ_OK;
 }
 
 } // namespace
@@ -509,31 +536,64 @@ int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int
 // xmode = AXQ_X_PACKED and no x.  The eps of a following RMSNorm is this call's eps.
 int axq_dev_gemv_batch_chain(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
                              const float *bias, const float *resid, float *y, const axq_weight *next, const float *next_aux) {
-    const int k = (int)w->k;
     int next_even_odd = -1;
     if (next) {
         if (next->k != w->n_rows || !axq_dev_gemv_batch_covers(next, batch))
             return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: the next weight does not take this one's output");
         next_even_odd = (next->type == AXQ_Q4_0 || next->type == AXQ_Q4_1) ? 1 : 0;
     }
-    // scratch (the context's x buffer): 32 k bytes of A operands, then 2 * (k / 32) * 8 floats of scales and sums
-    uint8_t *xa = ctx->xq;
-    float *xsg = reinterpret_cast<float *>(ctx->xq + (size_t)32 * k);
-    MbArgs a;
-    a.codes = w->codes; a.meta = w->meta;
-    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch;
-    a.xa = xa; a.xsg = xsg;
-    a.bias = bias; a.resid = resid; a.y = y;
-    // partial sums of a split K behind the x operands (splits only happen below AXQ_BATCH_SPLIT_ROWS rows)
-    a.ypart = w->n_rows <= AXQ_BATCH_SPLIT_ROWS ? reinterpret_cast<float *>(ctx->xq + (size_t)34 * AXQ_BATCH_MAX_K) : nullptr;
-    a.n_rows = (int)w->n_rows; a.k = k; a.batch = batch;
-    switch (w->type) {
-    case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, x, xmode, aux, eps, next_even_odd, next_aux); break;
-    case AXQ_Q4_1: launch_mb<MQ4x<true>>(ctx, a, x, xmode, aux, eps, next_even_odd, next_aux); break;
-    case AXQ_Q8_0: launch_mb<MQ80>(ctx, a, x, xmode, aux, eps, next_even_odd, next_aux); break;
-    case AXQ_Q4_K: launch_mb<MQ4K>(ctx, a, x, xmode, aux, eps, next_even_odd, next_aux); break;
-    default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
-    }
-    AXQ_LAUNCH_CHECK(ctx, "gemv_mb_kernel");
+    return gemv_batch_in(ctx, ctx->xq, w, x, xmode, aux, eps, batch, bias, resid, y, next_even_odd, next_aux);
+}
+
+// ---------------------------------------------------------------------------
+// The entry point that allocates nothing.  Its kernels are the ones above; the scratch they need (the batch's
+// operands, the partial sums of a split K) lives in a device array of this file instead of an allocation, one
+// copy per GPU, held until the process ends.  Host code never uses the array's name as an address: the set-up
+// below asks the runtime once per device where that device's copy lies and keeps the pointer.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) uint8_t scratch[AXQ_BATCH_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+uint8_t *g_scratch_ptr[MAX_DEVICES]; // per device: where `scratch` lies there (NULL: not looked up yet)
+std::mutex g_scratch_mutex;
+} // namespace
+
+// Called by axq_init with the context's device current.
+int axq_gemv_static_setup(axq_ctx *ctx) {
+    if (ctx->device < 0 || ctx->device >= MAX_DEVICES)
+        return axq_fail(ctx, AXQ_ERR_DEVICE_NOT_FOUND, "device %d: the static GEMV scratch is kept for devices 0..%d", ctx->device,
+                        MAX_DEVICES - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[ctx->device]) return AXQ_OK;
+    uint8_t *ptr = nullptr;
+    AXQ_HIP(ctx, hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)), AXQ_ERR_DRIVER);
+    if (!ptr) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipGetSymbolAddress gave no address for the static GEMV scratch");
+    // dynamic LDS beyond 64 KB has to be asked for once per kernel: here, so that the entry point itself only launches
+    AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4x<false>>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4x<true>>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<MQ80>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024), AXQ_ERR_DRIVER);
+    AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4K>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024), AXQ_ERR_DRIVER);
+    g_scratch_ptr[ctx->device] = ptr;
     return AXQ_OK;
+}
+
+int axq_gemv_f32_static(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_gemv_f32_static: NULL context");
+    if (!w || !x || !y) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_gemv_f32_static: NULL pointer");
+    if (batch < 2 || batch > MAX_BATCH)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: axq_gemv_f32_static takes 2..%d vectors per call, got %d", MAX_BATCH,
+                        batch);
+    if (w->k > AXQ_BATCH_MAX_K)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: k = %lld is beyond the static scratch (k <= %d)", (long long)w->k,
+                        AXQ_BATCH_MAX_K);
+    if (w->n_rows > INT32_MAX)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
+    if (!axq_dev_gemv_batch_covers(w, batch))
+        return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE,
+                        "axq_gemv_f32_static covers Q4_0, Q4_1, Q8_0 and Q4_K weights with k a multiple of 256 (got type %d, k = %lld)",
+                        w->type, (long long)w->k);
+    uint8_t *ptr = g_scratch_ptr[ctx->device];
+    if (!ptr) return axq_fail(ctx, AXQ_ERR_DRIVER, "the static GEMV scratch of device %d was not set up", ctx->device);
+    return gemv_batch_in(ctx, ptr, w, x, AXQ_X_PLAIN, nullptr, 0.f, batch, bias, nullptr, y, -1, nullptr);
 }

@@ -57,6 +57,8 @@ struct axq_weight {
 #define AXQ_XQ_MAX_K 65536
 #define AXQ_BATCH_MAX_K 16384 // widest weight of the small-batch GEMV: its x operands take 34 bytes per element of K
 #define AXQ_BATCH_SPLIT_ROWS 8192 // it splits K only for weights of at most this many rows: 4 splits x 8 vectors of partial sums
+// its scratch: the batch's operands (34 bytes per element of K), then the partial sums of a split K
+#define AXQ_BATCH_SCRATCH_BYTES ((size_t)34 * AXQ_BATCH_MAX_K + (size_t)4 * 8 * AXQ_BATCH_SPLIT_ROWS * 4)
 
 static inline size_t axq_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -122,6 +124,8 @@ int axq_dev_gemv_batch_ex(axq_ctx *ctx, const axq_weight *w, const float *x, int
 int axq_dev_gemv_batch_chain(axq_ctx *ctx, const axq_weight *w, const float *x, int xmode, const float *aux, float eps, int batch,
                              const float *bias, const float *resid, float *y, const axq_weight *next, const float *next_aux);
 bool axq_dev_gemv_batch_operands(axq_ctx *ctx, const axq_weight *w, uint8_t **xa, float **xsg);
+// looks up, once per device, where this device's copy of the static scratch of axq_gemv_f32_static lies (axq_init calls it)
+int axq_gemv_static_setup(axq_ctx *ctx);
 // sample.hip: every pointer a device pointer; scratch = axq_sample_scratch_bytes(vocab)
 size_t axq_sample_scratch_bytes(int vocab);
 int axq_check_sampling_config(axq_ctx *ctx, const axq_sampling_config *cfg);

@@ -168,6 +168,16 @@ AXQ_API void axq_weight_free(axq_ctx *ctx, axq_weight *w);
  * keeps f32 accuracy.  bias lives where x and y live. */
 AXQ_API int axq_gemv_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y,
                          int mem);
+/* axq_gemv_f32 for 2..8 vectors on device pointers, for callers that cannot allocate.  No counterpart in the
+ * reference: it exists for code under HIP graph capture, tight serving loops and harnesses that forbid
+ * hipMalloc.  It allocates nothing: the scratch of its kernels (the batch's matrix-pipe operands and the
+ * partial sums of a split K, 1,605,632 bytes) is a device array inside the library, one copy per GPU, held
+ * until the process ends.  Limits: Q4_0, Q4_1, Q8_0 or Q4_K weights, k a multiple of 256 up to 16384, any
+ * n_rows, batch 2..8; anything else is refused with AXQ_ERR_SHAPE_MISMATCH / AXQ_ERR_INVALID_QUANT_TYPE.
+ * x, bias (may be NULL) and y are device pointers; the launches go to the context's stream and nothing is
+ * synchronised.  Every call on a GPU shares that GPU's array (it needs no clearing: each call writes what it
+ * reads), so calls that overlap on one GPU -- from two contexts or two streams -- race; serialise them. */
+AXQ_API int axq_gemv_f32_static(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, const float *bias, float *y);
 /* y[m, n_rows] = x[m, k] * W^T, x in bf16 (raw uint16), y f32.  Prefill path. */
 AXQ_API int axq_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_bf16, int m, float *y, int mem);
 
