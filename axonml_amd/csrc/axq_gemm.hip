@@ -46,6 +46,9 @@ struct GemmArgs {
     int pair;
     const float *bias, *resid;
     int wm;                // 1: 128-row tiles, 2: 256-row tiles
+    // Q4_K kernel only: the rows' sub-block sums as f16 pairs, per split of K [hi | hi | lo | zeros] (see gemm_q4k_kernel)
+    const _Float16 *xs3;
+    int xs3_pitch;         // halfs per xs3 row
 };
 
 __device__ inline float h2f(uint32_t bits) { return __half2float(__ushort_as_half((unsigned short)bits)); }
@@ -424,8 +427,317 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
         }
 }
 
+// ---------------------------------------------------------------------------
+// Q4_K: one MFMA per product.
+//
+// A Q4_K weight is w = d * (sc * q) - dmin * m with a 4-bit code q, 6-bit sub-block scale sc and minimum m, and
+// f16 d, dmin per 256-element superblock (GGUF layout).  sc * q <= 945 is an integer of ten bits, so it is
+// EXACT in f16 -- and, as the bit pattern of an f16 subnormal, it needs no conversion at all: the integer n as
+// 16 bits is the f16 number n * 2^-24, which the matrix pipe multiplies exactly.  So the B operand of the main
+// loop is sc * q itself (two integer instructions per pair of weights), products x * (sc * q) are exact in the
+// f32 accumulator, and the superblock's d is applied to the accumulator, not to the weights:
+//   - the accumulator of an output column n holds the running sum in units of u_n, the d of the superblock
+//     being added; at a superblock boundary it is multiplied by u_n / d_next (one multiply per accumulator
+//     register per 256 k; a lane of the 32x32 MFMA output owns one column, so the factor is one number per
+//     lane).  A superblock with d = 0 contributes zeros and leaves the unit alone.
+//   - the minimum term, - sum_g dmin * m[n, g] * (sum of x over sub-block g), is a second, short GEMM over
+//     K / 32 "columns" that runs through the same pipeline after the main loop: c = dmin * m has 17 bits and
+//     goes in as two f16 (c S = ch + cl under a power-of-two S chosen per workgroup from the largest dmin it
+//     meets), the sub-block sums of x as two f16 (hi + lo, written by the x pre-pass), three products
+//     hi ch + hi cl + lo ch laid side by side along the extended K axis.
+// Against two MFMAs per product over all of K (the other block types below) this is 1 + 3/32.
+//
+// Tiling: a workgroup computes BM x 256 outputs with BM * 2 threads; every wave owns a 128 x 64 block (4 x 2 MFMA
+// tiles) and every thread also feeds: per K step of 64 it copies 64 bytes of the x tile and turns 32 codes of
+// one weight row into operands for the step after the next one's... (two LDS stages, one barrier per step;
+// the global loads of step s + 2 are in flight while step s + 1 is converted and step s multiplied).
+// x is stored by the pre-pass with elements 1 and 2 of every group of four exchanged: the codes of a dword
+// unpack to the pairs (0, 2) and (1, 3) with one mask each, and the order of k inside an MFMA is free as long
+// as both operands agree.
+// ---------------------------------------------------------------------------
+constexpr int QBN = 256; // output columns (weight rows) per workgroup
+
+// 6-bit scales and minimums of sub-blocks 2p, 2p + 1 (ggml get_scale_min_k4 order) as two bytes each
+__device__ inline void q4k_scale_min(const u32x4 &h, int p, uint32_t &scp, uint32_t &mp) {
+    const int sh = (p & 1) * 16;
+    const uint32_t ya = h[1] >> sh, za = h[2] >> sh, wa = h[3] >> sh;
+    if (p < 2) {
+        scp = ya & 0x3F3F;
+        mp = za & 0x3F3F;
+    } else {
+        scp = (wa & 0x0F0F) | ((ya >> 2) & 0x3030);
+        mp = ((wa >> 4) & 0x0F0F) | ((za >> 2) & 0x3030);
+    }
+}
+
+template <int BM>
+__global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
+    constexpr int NT = BM * 2;           // threads
+    constexpr int NW = NT / 64;          // waves: (BM / 128) x 4 blocks of 128 x 64
+    constexpr int AV = BM * 8 / NT;      // 16-byte x vectors per thread and step (= 4)
+    constexpr int BT = QBN * 2 / NT;     // (weight row, half) tasks per thread and step (1 or 2)
+    constexpr int STAGE = (BM + QBN) * LDK;
+    extern __shared__ _Float16 lds[];
+    float *wg_red = reinterpret_cast<float *>(lds + 2 * STAGE); // NW words behind the stages
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nt = (a.n + QBN - 1) / QBN, total = (int)gridDim.x;
+    int tile = blockIdx.x;
+    if (total % 8 == 0) tile = (tile & 7) * (total >> 3) + (tile >> 3); // workgroups of one XCD share x tiles
+    const int m0 = (tile / nt) * BM, n0 = (tile % nt) * QBN;
+    const int kbeg = (int)blockIdx.y * a.steps_per_split; // in steps of 64 k; a multiple of 4 (whole superblocks)
+    const int t_main = a.k / BK - kbeg < a.steps_per_split ? a.k / BK - kbeg : a.steps_per_split;
+    const int nsb = t_main >> 2;         // superblocks of this workgroup's part of K
+    const int t_min = (nsb + 1) >> 1, t_all = t_main + t_min;
+    const int last_sb = (a.k >> 8) - 1;
+
+    // ---- feeder side.  The x rows of the scratch buffer are allocated up to a multiple of BM, so row addresses need no
+    // clamp and the AV vectors of a thread lie a fixed number of rows apart.
+    struct Raw { u32x4 xa[AV]; u32x4 q[BT]; u32x4 h[BT]; };
+    const _Float16 *xrow = a.xh + (size_t)(m0 + (tid >> 3)) * a.k + (size_t)kbeg * BK + (tid & 7) * 8;
+    const _Float16 *x3row = a.xs3 + (size_t)(m0 + (tid >> 3)) * a.xs3_pitch + (size_t)(kbeg >> 2) * 32 + (tid & 7) * 8;
+    const size_t xstep = (size_t)(NT / 8) * a.k, x3step = (size_t)(NT / 8) * a.xs3_pitch; // rows between a thread's vectors
+    const uint8_t *crow[BT], *mrow[BT];
+    const int cpr = a.k >> 6; // pairs of sub-blocks (K steps) per row
+#pragma unroll
+    for (int u = 0; u < BT; u++) {
+        int gn = n0 + ((tid + u * NT) >> 1);
+        gn = gn < a.n ? gn : a.n - 1;
+        crow[u] = a.codes + (size_t)gn * a.codes_pitch;
+        mrow[u] = a.meta + (size_t)gn * a.meta_pitch;
+    }
+    const int bh = tid & 1; // which 16 bytes of a pair's 32 (NT is even: the same for every task of the thread)
+    auto fetch = [&](int step, Raw &r) {
+        if (step < t_main) {
+            const int pair = kbeg + step, slice = pair >> 6, pr = pair & 63;
+            int P = cpr - (slice << 6);
+            P = P < 64 ? P : 64;
+#pragma unroll
+            for (int i = 0; i < AV; i++) r.xa[i] = *reinterpret_cast<const u32x4 *>(xrow + i * xstep + (size_t)step * BK);
+#pragma unroll
+            for (int u = 0; u < BT; u++) {
+                r.q[u] = *reinterpret_cast<const u32x4 *>(crow[u] + (size_t)slice * 2048 + (size_t)bh * 16 * P + (size_t)pr * 16);
+                r.h[u] = *reinterpret_cast<const u32x4 *>(mrow[u] + (size_t)(pair >> 2) * 16);
+            }
+        } else if (step < t_all) {
+            // the minimum term: 64 columns = two superblocks of [hi | hi | lo | 0] x [ch | cl | ch | 0]
+            const int s2 = step - t_main;
+            int sb = (kbeg >> 2) + 2 * s2 + bh;
+            sb = sb < last_sb ? sb : last_sb;
+            // an odd count of superblocks: the second half of the last step lies beyond this part of K (or beyond the row)
+            const bool xlive = 2 * s2 + ((tid & 7) >> 2) < nsb;
+#pragma unroll
+            for (int i = 0; i < AV; i++)
+                r.xa[i] = xlive ? *reinterpret_cast<const u32x4 *>(x3row + i * x3step + (size_t)s2 * BK) : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < BT; u++) r.h[u] = *reinterpret_cast<const u32x4 *>(mrow[u] + (size_t)sb * 16);
+        }
+    };
+    uint32_t dmin_max = 0; // largest |dmin| (f16 bits) this thread has met in the main loop
+    float S = 1.0f;        // the minimum term's power-of-two factor (set one step before the main loop ends)
+    // part t (0..3) of the conversion of `r` (step `step`) into stage `st`
+    auto convert = [&](int step, const Raw &r, int st, int t) {
+        _Float16 *As = lds + st * STAGE, *Bs = As + BM * LDK;
+        {
+            const int v = tid + t * NT;
+            *reinterpret_cast<u32x4 *>(As + (v >> 3) * LDK + (v & 7) * 8) = r.xa[t];
+        }
+        if (step < t_main) {
+            const int p = (kbeg + step) & 3;
+#pragma unroll
+            for (int u = 0; u < BT; u++) {
+                const int row = (tid + u * NT) >> 1;
+                uint32_t scp, mp;
+                q4k_scale_min(r.h[u], p, scp, mp);
+                const uint32_t dd = r.h[u][0];
+                if ((dd & 0x7FFFu) == 0) scp = 0; // d = 0: the superblock adds nothing and leaves the unit alone
+                if (t == 0) {
+                    const uint32_t dm = (dd >> 16) & 0x7FFFu;
+                    dmin_max = dm > dmin_max ? dm : dmin_max;
+                }
+                const uint32_t s0 = scp & 0xFF, s1 = scp >> 8;
+                const uint32_t w = r.q[u][t];
+                // bytes 4t .. 4t+3 of the thread's 16: elements 16 bh + 4t + {0, 1, 2, 3} of both sub-blocks
+                const uint32_t la = (w & 0x000F000Fu) * s0, lb = ((w >> 8) & 0x000F000Fu) * s0;
+                const uint32_t ha = ((w >> 4) & 0x000F000Fu) * s1, hb = ((w >> 12) & 0x000F000Fu) * s1;
+                *reinterpret_cast<uint2 *>(Bs + row * LDK + bh * 16 + t * 4) = make_uint2(la, lb);
+                *reinterpret_cast<uint2 *>(Bs + row * LDK + 32 + bh * 16 + t * 4) = make_uint2(ha, hb);
+            }
+        } else {
+            const bool live = 2 * (step - t_main) + bh < nsb; // an odd count of superblocks: the last step's second half is empty
+#pragma unroll
+            for (int u = 0; u < BT; u++) {
+                const int row = (tid + u * NT) >> 1;
+                const u32x4 h = r.h[u];
+                const float dmin = live ? (-64.0f * S) * h2f(h[0] >> 16) : 0.f;
+                uint32_t o[4];
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    uint32_t scp, mp;
+                    q4k_scale_min(h, p, scp, mp);
+                    const float c0 = dmin * ubyte<0>(mp), c1 = dmin * ubyte<1>(mp); // exact: 11 x 6 bits
+                    const float h0 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, c0) & 0xFFFFE000u);
+                    const float h1 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, c1) & 0xFFFFE000u);
+                    const float v0 = t == 1 ? c0 - h0 : h0, v1 = t == 1 ? c1 - h1 : h1; // t: 0 ch, 1 cl, 2 ch, 3 nothing
+                    o[p] = t == 3 ? 0u : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(v0, v1));
+                }
+                *reinterpret_cast<u32x4 *>(Bs + row * LDK + bh * 32 + t * 8) = u32x4{o[0], o[1], o[2], o[3]};
+            }
+        }
+    };
+
+    // ---- multiplier side
+    const int wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
+    const int li = lane & 31, lk = (lane >> 5) * 8;
+    float16v acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    const uint8_t *dcol[2]; // this lane's two output columns: their superblock headers
+    float unit[2] = {1.0f, 1.0f};
+    uint32_t dnext[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        int gn = n0 + wn + j * 32 + li;
+        gn = gn < a.n ? gn : a.n - 1;
+        dcol[j] = a.meta + (size_t)gn * a.meta_pitch;
+        dnext[j] = *reinterpret_cast<const uint16_t *>(dcol[j] + (size_t)(kbeg >> 2) * 16);
+    }
+
+    Raw cur, nxt;
+    fetch(0, cur);
+    fetch(1, nxt);
+#pragma unroll
+    for (int t = 0; t < 4; t++) convert(0, cur, 0, t);
+    cur = nxt;
+    __syncthreads();
+    for (int ks = 0; ks < t_all; ks++) {
+        const _Float16 *As = lds + (ks & 1) * STAGE, *Bs = As + BM * LDK;
+        fetch(ks + 2, nxt);
+        if (ks == t_main - 1) { // every main-loop header has been seen: the factor of the minimum term
+            uint32_t mx = 0;
+            for (int w = 0; w < NW; w++) {
+                const uint32_t v = __builtin_bit_cast(uint32_t, wg_red[w]);
+                mx = v > mx ? v : mx;
+            }
+            // dmin < 2^(e + 1) -> the operands are c * 2^(8 - e) < 2^15; they meet sub-block sums stored times 1 / 64, so
+            // the accumulators then hold the result times S = 2^(2 - e).  No dmin, or inf / nan: operands c, S = 1 / 64.
+            const int e = (mx == 0 || mx >= 0x7C00u) ? 8 : (mx >= 0x400u ? (int)(mx >> 10) - 15 : -15);
+            S = __builtin_bit_cast(float, (uint32_t)(127 + 2 - e) << 23);
+        }
+        if (ks < t_main && ((kbeg + ks) & 3) == 0) {
+            // a new superblock: the accumulators change their unit to its d
+            const int sbn = ((kbeg + ks) >> 2) + 1;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const float dn = h2f(dnext[j]);
+                const float r = dn != 0.f ? unit[j] / dn : 1.0f;
+                unit[j] = dn != 0.f ? dn : unit[j];
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int q = 0; q < 16; q++) acc[i][j][q] *= r;
+                dnext[j] = *reinterpret_cast<const uint16_t *>(dcol[j] + (size_t)(sbn < last_sb ? sbn : last_sb) * 16);
+            }
+        }
+        if (ks == t_main) { // the main sum in true units, times S: the minimum term joins it
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const float f = unit[j] * 16777216.0f * S;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int q = 0; q < 16; q++) acc[i][j][q] *= f;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < BK / 16; t++) {
+            // two waves share a SIMD: while this one waits for its fragments the other one multiplies
+            half8 af[4], bf[2];
+#pragma unroll
+            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const half8 *>(As + (wm + i * 32 + li) * LDK + t * 16 + lk);
+#pragma unroll
+            for (int j = 0; j < 2; j++) bf[j] = *reinterpret_cast<const half8 *>(Bs + (wn + j * 32 + li) * LDK + t * 16 + lk);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+            if (ks + 1 < t_all) convert(ks + 1, cur, (ks + 1) & 1, t);
+        }
+        if (ks == t_main - 2) { // the last main-loop header is converted in this step
+            uint32_t mx = dmin_max;
+#pragma unroll
+            for (int s = 32; s >= 1; s >>= 1) {
+                const uint32_t o = (uint32_t)__shfl_xor((int)mx, s);
+                mx = o > mx ? o : mx;
+            }
+            if (lane == 0) wg_red[wave] = __builtin_bit_cast(float, mx);
+        }
+        cur = nxt;
+        __syncthreads();
+    }
+    // D layout: lane -> column li; register r -> row 8 * (r / 4) + 4 * (lane / 32) + r % 4
+    const float inv_s = 1.0f / S;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int gn = n0 + wn + j * 32 + li;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int gm = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (gm < a.m && gn < a.n) {
+                    if (!a.pair) {
+                        if (a.ypart) a.ypart[((size_t)blockIdx.y * a.m + gm) * a.n + gn] = acc[i][j][r] * inv_s;
+                        else a.y[(size_t)gm * a.n + gn] = acc[i][j][r] * (a.rowscale[gm] * inv_s);
+                    } else if ((r & 1) == 0) { // gm is even: this register and the next hold the two parts of row gm / 2
+                        const size_t t = (size_t)(gm >> 1);
+                        const float v = (acc[i][j][r] + acc[i][j][r + 1]) * inv_s;
+                        if (a.ypart) {
+                            a.ypart[((size_t)blockIdx.y * (a.m >> 1) + t) * a.n + gn] = v;
+                        } else {
+                            float out = v * a.rowscale[gm];
+                            if (a.bias) out += a.bias[gn];
+                            if (a.resid) out += a.resid[t * a.n + gn];
+                            a.y[t * a.n + gn] = out;
+                        }
+                    }
+                }
+            }
+        }
+}
+
+// What the Q4_K kernel wants from the x pre-pass besides the scaled f16 rows: elements 1 and 2 of every group of four
+// exchanged, and the sums of every 32 consecutive (scaled, f16) elements as f16 pairs hi + lo: 32 halfs per superblock,
+// [hi of its 8 sub-blocks | the same | lo | zeros] (NULL xs3: plain rows for the other kernels).
+struct XSums {
+    _Float16 *xs3;
+    int pitch; // halfs per row: k / 8
+};
+constexpr float XSUM_SCALE = 1.0f / 64.0f; // the sums are stored times this
+
+// The sum `s` of the caller's four elements, added over the eight threads of a 32-element group; the first of them
+// stores the pair.  g = index of the group along the row.
+__device__ inline void store_group_sum(float s, int g, int n_groups, _Float16 *row3, const XSums &xs) {
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    s += __shfl_xor(s, 4);
+    if ((threadIdx.x & 7) == 0 && g < n_groups) {
+        s *= XSUM_SCALE; // 32 elements below 2^15 each: the sum must not leave f16's range
+        const _Float16 hi = (_Float16)s, lo = (_Float16)(s - (float)hi);
+        _Float16 *base = row3 + (size_t)(g >> 3) * 32 + (g & 7);
+        base[0] = hi;
+        base[8] = hi;
+        base[16] = lo;
+        base[24] = (_Float16)0.f;
+    }
+}
+
 // bf16 rows -> f16 rows scaled by a power of two (largest magnitude below 2^15), and the scale to undo it.
-__global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int m, int k, _Float16 *xh, float *rowscale) {
+__global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int m, int k, _Float16 *xh, float *rowscale, XSums xs) {
     __shared__ float red[4];
     const int row = blockIdx.x;
     const uint16_t *xr = x + (size_t)row * k;
@@ -438,6 +750,7 @@ __global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int
 #pragma unroll
     for (int s = 32; s >= 1; s >>= 1) amax = fmaxf(amax, __shfl_xor(amax, s));
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    _Float16 *row3 = xs.xs3 ? xs.xs3 + (size_t)row * xs.pitch : nullptr;
     __syncthreads();
     amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     // amax in [2^e, 2^(e+1)) -> multiply by 2^(14 - e); inf/nan rows are passed through unscaled
@@ -446,9 +759,17 @@ __global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int
     int sb = 127 + 14 - (eb - 127);
     sb = sb < 1 ? 1 : (sb > 254 ? 254 : sb);
     const float f = __builtin_bit_cast(float, (uint32_t)sb << 23);
-    for (int i = threadIdx.x; i < k; i += blockDim.x) {
-        float v = __builtin_bit_cast(float, (uint32_t)xr[i] << 16);
-        xh[(size_t)row * k + i] = (_Float16)(v * f);
+    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+    for (int i4 = threadIdx.x; i4 < (k >> 2); i4 += blockDim.x) { // k is a multiple of 64: whole groups of eight threads
+        const uint2 raw = reinterpret_cast<const uint2 *>(xr)[i4];
+        const _Float16 h0 = (_Float16)(__builtin_bit_cast(float, raw.x << 16) * f), h1 = (_Float16)(__builtin_bit_cast(float, raw.x & 0xFFFF0000u) * f);
+        const _Float16 h2 = (_Float16)(__builtin_bit_cast(float, raw.y << 16) * f), h3 = (_Float16)(__builtin_bit_cast(float, raw.y & 0xFFFF0000u) * f);
+        if (row3) {
+            reinterpret_cast<half4 *>(xh + (size_t)row * k)[i4] = half4{h0, h2, h1, h3};
+            store_group_sum(((float)h0 + (float)h1) + ((float)h2 + (float)h3), i4 >> 3, k >> 5, row3, xs);
+        } else {
+            reinterpret_cast<half4 *>(xh + (size_t)row * k)[i4] = half4{h0, h1, h2, h3};
+        }
     }
     if (threadIdx.x == 0) rowscale[row] = 1.0f / f;
 }
@@ -508,7 +829,7 @@ int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
 // -> two f16 rows each under one power-of-two scale: row 2t holds the leading 11 bits of every element, row 2t + 1
 // what those leave, so that their GEMM results add up to the f32 product (the GEMM's epilogue adds them: pair mode).
 __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, const float *norm_w, float eps, int m, int k,
-                                                              _Float16 *xh, float *rowscale) {
+                                                              _Float16 *xh, float *rowscale, XSums xs) {
     // the row stays in registers between the passes: 16 bytes per thread and step, up to 16 steps (k <= 16384);
     // longer rows (or k not a multiple of 4) take the plain loops below
     constexpr int STEPS = 16;
@@ -584,18 +905,30 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
     sb = sb < 1 ? 1 : (sb > 254 ? 254 : sb);
     const float f = __builtin_bit_cast(float, (uint32_t)sb << 23);
     _Float16 *hi_row = xh + (size_t)(2 * row) * k, *lo_row = hi_row + k;
+    // the Q4_K kernel's extras (callers ask for them only when the row fits the registers and k is a multiple of 64)
+    _Float16 *hi3 = xs.xs3 ? xs.xs3 + (size_t)(2 * row) * xs.pitch : nullptr, *lo3 = hi3 ? hi3 + xs.pitch : nullptr;
     if (in_regs) {
 #pragma unroll
         for (int c = 0; c < STEPS; c++) {
             const int i4 = c * 256 + threadIdx.x;
-            if (i4 * 4 < k) {
+            if (c * 256 * 4 < k) { // uniform per step; with the extras k is a multiple of 32 and whole groups of eight threads are in
+                const bool live = i4 * 4 < k;
                 const float e[4] = {v[c].x * f, v[c].y * f, v[c].z * f, v[c].w * f};
                 _Float16 h[4], l[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) { h[j] = (_Float16)e[j]; l[j] = (_Float16)(e[j] - (float)h[j]); }
                 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-                reinterpret_cast<half4 *>(hi_row)[i4] = half4{h[0], h[1], h[2], h[3]};
-                reinterpret_cast<half4 *>(lo_row)[i4] = half4{l[0], l[1], l[2], l[3]};
+                if (hi3) {
+                    if (live) {
+                        reinterpret_cast<half4 *>(hi_row)[i4] = half4{h[0], h[2], h[1], h[3]};
+                        reinterpret_cast<half4 *>(lo_row)[i4] = half4{l[0], l[2], l[1], l[3]};
+                    }
+                    store_group_sum(((float)h[0] + (float)h[1]) + ((float)h[2] + (float)h[3]), live ? i4 >> 3 : k, k >> 5, hi3, xs);
+                    store_group_sum(((float)l[0] + (float)l[1]) + ((float)l[2] + (float)l[3]), live ? i4 >> 3 : k, k >> 5, lo3, xs);
+                } else if (live) {
+                    reinterpret_cast<half4 *>(hi_row)[i4] = half4{h[0], h[1], h[2], h[3]};
+                    reinterpret_cast<half4 *>(lo_row)[i4] = half4{l[0], l[1], l[2], l[3]};
+                }
             }
         }
     } else {
@@ -626,13 +959,21 @@ int reserve_scratch(axq_ctx *ctx, size_t need) {
 
 struct GemmPlan {
     int splits, steps_per_split, wm;
-    size_t xh_bytes, rs_bytes, part_bytes;
+    bool q4k;     // the one-MFMA Q4_K kernel (gemm_q4k_kernel) instead of the two-plane kernel
+    size_t xh_bytes, rs_bytes, part_bytes, xs3_bytes;
 };
+
+// Whether the one-MFMA kernel takes this weight; in_regs_only: the caller's x pre-pass produces the extras only for rows
+// that fit its registers (f32 rows).
+bool q4k_route(const axq_weight *w, bool in_regs_only) {
+    static const bool off = getenv("AXQ_GEMM_Q4K") && getenv("AXQ_GEMM_Q4K")[0] == '0'; // development knob
+    return !off && w->type == AXQ_Q4_K && w->k % 256 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
+}
 
 // Split K when the output tiles alone leave most compute units idle (short prompts): the splits' partial sums go
 // through scratch and are added in order by a second kernel.  Scratch (kept in the context, grown on demand):
-// f16 activations [m, k] | row scales [m] | partial sums of a split K | `extra` bytes for the caller.
-int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, size_t extra, GemmPlan *p) {
+// f16 activations [m, k] | row scales [m] | partial sums of a split K | sub-block sums (Q4_K) | `extra` bytes for the caller.
+int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, bool f32_rows, size_t extra, GemmPlan *p) {
     if (w->k % BK != 0)
         return axq_fail(ctx, AXQ_ERR_INVALID_BLOCK_SIZE, "Invalid block size: the prefill GEMM needs k %% 64 == 0, got %lld",
                         (long long)w->k);
@@ -641,18 +982,60 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, size_t extra, GemmPlan *
     static const int bm_knob = getenv("AXQ_GEMM_BM") ? atoi(getenv("AXQ_GEMM_BM")) : 0; // development knob: 128 or 256 for every shape
     const int bm = bm_knob ? bm_knob : (m > 128 ? 256 : 128);
     p->wm = bm / 128;
-    const long tiles = (long)((w->n_rows + BN - 1) / BN) * ((m + bm - 1) / bm);
+    p->q4k = q4k_route(w, f32_rows);
+    const int bn = p->q4k ? QBN : BN;
+    const long tiles = (long)((w->n_rows + bn - 1) / bn) * ((m + bm - 1) / bm);
     const int ksteps = (int)(w->k / BK), cus = ctx->prop.multiProcessorCount;
     int splits = (int)(cus / tiles);
     splits = splits > 8 ? 8 : splits;
     if (splits > ksteps / 4) splits = ksteps / 4;
     if (splits < 2 || w->n_rows % 4 != 0) splits = 1;
     p->steps_per_split = (ksteps + splits - 1) / splits;
+    if (p->q4k) p->steps_per_split = (p->steps_per_split + 3) & ~3; // whole superblocks per split
     p->splits = (ksteps + p->steps_per_split - 1) / p->steps_per_split;
-    p->xh_bytes = axq_align_up((size_t)m * (size_t)w->k * 2, 256);
+    // the Q4_K kernel reads whole row tiles without a clamp: its x buffers have rows up to a multiple of the tile
+    const size_t mpad = p->q4k ? (size_t)(m + bm - 1) / bm * bm : (size_t)m;
+    p->xh_bytes = axq_align_up(mpad * (size_t)w->k * 2, 256);
     p->rs_bytes = axq_align_up((size_t)m * 4, 256);
     p->part_bytes = axq_align_up(p->splits > 1 ? (size_t)p->splits * m * (size_t)w->n_rows * 4 : 0, 256);
-    return reserve_scratch(ctx, p->xh_bytes + p->rs_bytes + p->part_bytes + extra);
+    p->xs3_bytes = axq_align_up(p->q4k ? mpad * (size_t)(w->k / 8) * 2 : 0, 256);
+    return reserve_scratch(ctx, p->xh_bytes + p->rs_bytes + p->part_bytes + p->xs3_bytes + extra);
+}
+
+// What the x pre-pass has to write besides the rows (nothing for the two-plane kernel).
+XSums plan_sums(axq_ctx *ctx, const axq_weight *w, const GemmPlan &p) {
+    XSums xs = {nullptr, 0};
+    if (p.q4k) {
+        xs.xs3 = reinterpret_cast<_Float16 *>(reinterpret_cast<uint8_t *>(ctx->gemm_scratch) + p.xh_bytes + p.rs_bytes + p.part_bytes);
+        xs.pitch = (int)(w->k / 8);
+    }
+    return xs;
+}
+
+int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits) {
+    static bool attr_set = false;
+    const int bm = 128 * a.wm;
+    const unsigned tiles = (unsigned)(((a.n + QBN - 1) / QBN) * ((a.m + bm - 1) / bm));
+    const dim3 grid(tiles, (unsigned)splits);
+    const size_t lds = (size_t)2 * (bm + QBN) * LDK * sizeof(_Float16) + 64; // two stages and a word per wave
+    if (!attr_set) {
+        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_kernel<256>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * (256 + QBN) * LDK * 2 + 64)), AXQ_ERR_DRIVER);
+        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_kernel<128>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * (128 + QBN) * LDK * 2 + 64)), AXQ_ERR_DRIVER);
+        attr_set = true;
+    }
+    if (a.wm == 2) gemm_q4k_kernel<256><<<grid, 512, lds, ctx->stream>>>(a);
+    else gemm_q4k_kernel<128><<<grid, 256, lds, ctx->stream>>>(a);
+    AXQ_LAUNCH_CHECK(ctx, "gemm_q4k_kernel");
+    if (splits > 1) {
+        const int rows = a.pair ? a.m / 2 : a.m;
+        const size_t total4 = (size_t)rows * a.n / 4;
+        gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(a.ypart, a.rowscale, rows, a.n, splits, 1.0f,
+                                                                                    a.pair ? 2 : 1, a.bias, a.resid, a.y);
+        AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
+    }
+    return AXQ_OK;
 }
 
 // The GEMM proper over activations that already sit in scratch as scaled f16 rows.
@@ -667,6 +1050,9 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     a.m = m; a.n = (int)w->n_rows; a.k = (int)w->k;
     a.steps_per_split = p.steps_per_split;
     a.pair = pair ? 1 : 0; a.bias = bias; a.resid = resid; a.wm = p.wm;
+    const XSums xs = plan_sums(ctx, w, p);
+    a.xs3 = xs.xs3; a.xs3_pitch = xs.pitch;
+    if (p.q4k) return launch_gemm_q4k(ctx, a, p.splits);
     switch (w->type) {
     case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);
     case AXQ_Q4_0: return launch_gemm<GQ4x<false>>(ctx, a, p.splits);
@@ -685,10 +1071,10 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x, int m, float *y) {
     GemmPlan p;
     int rc;
-    if ((rc = plan_gemm(ctx, w, m, 0, &p))) return rc;
+    if ((rc = plan_gemm(ctx, w, m, false, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     gemm_prep_x_kernel<<<m, 256, 0, ctx->stream>>>(x, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
-                                                   reinterpret_cast<float *>(base + p.xh_bytes));
+                                                   reinterpret_cast<float *>(base + p.xh_bytes), plan_sums(ctx, w, p));
     return run_gemm(ctx, w, m, p, y);
 }
 
@@ -703,9 +1089,9 @@ int axq_dev_gemm_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int m, c
                      const float *resid, float *y) {
     GemmPlan p;
     int rc;
-    if ((rc = plan_gemm(ctx, w, 2 * m, 0, &p))) return rc;
+    if ((rc = plan_gemm(ctx, w, 2 * m, true, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
     gemm_prep_x_f32_kernel<<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
-                                                       reinterpret_cast<float *>(base + p.xh_bytes));
+                                                       reinterpret_cast<float *>(base + p.xh_bytes), plan_sums(ctx, w, p));
     return run_gemm(ctx, w, 2 * m, p, y, true, bias, resid);
 }
