@@ -20,6 +20,8 @@
 
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "axq_internal.h"
 
 namespace {
@@ -470,15 +472,35 @@ __device__ inline void q4k_scale_min(const u32x4 &h, int p, uint32_t &scp, uint3
     }
 }
 
+// A workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global load in flight, which
+// would pull the prefetched operands of later steps in front of every barrier.
+__device__ inline void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void gbl_void;
+
+// s_waitcnt vmcnt(N) lgkmcnt(0) (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4 left at 7, lgkmcnt 11:8)
+template <int N>
+__device__ inline void wait_vm_and_lds() {
+    __builtin_amdgcn_s_waitcnt(((N >> 4) << 14) | (7 << 4) | (N & 15));
+}
+
 template <int BM>
 __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
     constexpr int NT = BM * 2;           // threads
     constexpr int NW = NT / 64;          // waves: (BM / 128) x 4 blocks of 128 x 64
-    constexpr int AV = BM * 8 / NT;      // 16-byte x vectors per thread and step (= 4)
     constexpr int BT = QBN * 2 / NT;     // (weight row, half) tasks per thread and step (1 or 2)
-    constexpr int STAGE = (BM + QBN) * LDK;
+    constexpr int AROWS = BM / NW;       // x rows a wave brings in per step (= 32: four loads of eight rows)
+    // LDS (halfs): three stages of the x tile, then two of the weight tile.  A tile row is 64 halfs, unpadded, its eight
+    // 16-byte chunks stored at chunk ^ ((row / 2) & 7): x tiles are written by loads that go straight to LDS, 1 KB per
+    // wave and instruction in lane order, so padding is not to be had; the exchange keeps the fragment reads of sixteen
+    // consecutive rows, which LDS serves together, on distinct banks (64 banks of four bytes, even rows in the lower half).
+    constexpr int ASTAGE = BM * 64, BSTAGE = QBN * 64, BOFF = 3 * ASTAGE;
     extern __shared__ _Float16 lds[];
-    float *wg_red = reinterpret_cast<float *>(lds + 2 * STAGE); // NW words behind the stages
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nt = (a.n + QBN - 1) / QBN, total = (int)gridDim.x;
@@ -488,107 +510,150 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
     const int kbeg = (int)blockIdx.y * a.steps_per_split; // in steps of 64 k; a multiple of 4 (whole superblocks)
     const int t_main = a.k / BK - kbeg < a.steps_per_split ? a.k / BK - kbeg : a.steps_per_split;
     const int nsb = t_main >> 2;         // superblocks of this workgroup's part of K
-    const int t_min = (nsb + 1) >> 1, t_all = t_main + t_min;
+    const int t_min = (nsb + 1) >> 1;
     const int last_sb = (a.k >> 8) - 1;
 
-    // ---- feeder side.  The x rows of the scratch buffer are allocated up to a multiple of BM, so row addresses need no
-    // clamp and the AV vectors of a thread lie a fixed number of rows apart.
-    struct Raw { u32x4 xa[AV]; u32x4 q[BT]; u32x4 h[BT]; };
-    const _Float16 *xrow = a.xh + (size_t)(m0 + (tid >> 3)) * a.k + (size_t)kbeg * BK + (tid & 7) * 8;
-    const _Float16 *x3row = a.xs3 + (size_t)(m0 + (tid >> 3)) * a.xs3_pitch + (size_t)(kbeg >> 2) * 32 + (tid & 7) * 8;
-    const size_t xstep = (size_t)(NT / 8) * a.k, x3step = (size_t)(NT / 8) * a.xs3_pitch; // rows between a thread's vectors
-    const uint8_t *crow[BT], *mrow[BT];
+    // ---- feeder side.  Addresses are (uniform 64-bit base of the workgroup) + (32-bit offset of the thread).  The x
+    // rows of the scratch buffer are allocated up to a multiple of BM, so they need no clamp; weight rows past the end
+    // are clamped.
+    // What a thread holds of a group of four steps: main loop = one superblock: the 16 code bytes of its (row, half) for
+    // each of the four pairs (64 consecutive bytes in memory) and the superblock's header; minimum term: the headers of
+    // the four steps' superblocks (in q) -- five, or four, loads per task and group.
+    struct Raw { u32x4 q[BT][4]; u32x4 h[BT]; };
+    const uint8_t *xbase = reinterpret_cast<const uint8_t *>(a.xh + (size_t)m0 * a.k + (size_t)kbeg * BK);
+    const uint8_t *x3base = reinterpret_cast<const uint8_t *>(a.xs3 + (size_t)m0 * a.xs3_pitch + (size_t)(kbeg >> 2) * 32);
+    // a lane's part of a wave's x load: row lane / 8 of the eight, and the chunk that belongs at slot lane % 8 of that row:
+    // slot ^ ((row / 2) & 7) -- for the rows of load i that is (lane % 8) ^ (lane / 16) ^ 4 (i & 1)
+    const uint32_t xrow_l = (uint32_t)(wave * AROWS + (lane >> 3)), xchunk_l = (uint32_t)((lane & 7) ^ (lane >> 4));
+    const uint32_t xoff = (xrow_l * (uint32_t)a.k + xchunk_l * 8) * 2, x3off = (xrow_l * (uint32_t)a.xs3_pitch + xchunk_l * 8) * 2;
+    const size_t x8rows = (size_t)8 * a.k * 2, x38rows = (size_t)8 * a.xs3_pitch * 2;
+    const uint8_t *cbase = a.codes + (size_t)n0 * a.codes_pitch, *mbase = a.meta + (size_t)n0 * a.meta_pitch;
+    uint32_t coff[BT], moff[BT];
     const int cpr = a.k >> 6; // pairs of sub-blocks (K steps) per row
+    const int bh = tid & 1;   // which 16 bytes of a pair's 32 (NT is even: the same for every task of the thread)
+    int b_wr[BT];             // where the thread's operands go in a weight stage (halfs): row, and the chunk exchange
 #pragma unroll
     for (int u = 0; u < BT; u++) {
-        int gn = n0 + ((tid + u * NT) >> 1);
-        gn = gn < a.n ? gn : a.n - 1;
-        crow[u] = a.codes + (size_t)gn * a.codes_pitch;
-        mrow[u] = a.meta + (size_t)gn * a.meta_pitch;
+        const int row = (tid + u * NT) >> 1;
+        const int crow = n0 + row < a.n ? row : a.n - 1 - n0;
+        coff[u] = (uint32_t)crow * (uint32_t)a.codes_pitch;
+        moff[u] = (uint32_t)crow * (uint32_t)a.meta_pitch;
+        b_wr[u] = row * 64 + ((((row >> 1) & 7) ^ (bh * 2)) * 8);
     }
-    const int bh = tid & 1; // which 16 bytes of a pair's 32 (NT is even: the same for every task of the thread)
-    auto fetch = [&](int step, Raw &r) {
-        if (step < t_main) {
-            const int pair = kbeg + step, slice = pair >> 6, pr = pair & 63;
-            int P = cpr - (slice << 6);
-            P = P < 64 ? P : 64;
+    // x tile of main step `step` (or, MIN, of step s2 of the minimum term, clamped to the last) -> x stage `stage`
+    auto load_x = [&](auto is_min, int step, int stage) {
+        constexpr bool MIN = decltype(is_min)::value;
+        if (MIN) step = step < t_min ? step : t_min - 1;
+        const uint8_t *g = (MIN ? x3base : xbase) + (size_t)step * (BK * 2);
+        const uint32_t off = MIN ? x3off : xoff;
+        const size_t rows8 = MIN ? x38rows : x8rows;
+        _Float16 *dst = lds + stage * ASTAGE + wave * AROWS * 64;
 #pragma unroll
-            for (int i = 0; i < AV; i++) r.xa[i] = *reinterpret_cast<const u32x4 *>(xrow + i * xstep + (size_t)step * BK);
+        for (int i = 0; i < AROWS / 8; i++)
+            __builtin_amdgcn_global_load_lds((gbl_void *)(g + i * rows8 + ((i & 1) ? off ^ 64u : off)), (lds_void *)(dst + i * 8 * 64), 16, 0, 0);
+        asm volatile("" ::: "memory"); // what is requested after this stays after it: the waits in front of the barriers count on the order
+    };
+    // Main loop: the packed weights of superblock `sb` (0 .. nsb - 1, clamped) of this workgroup's part of K.
+    auto fetch_main = [&](int sb, Raw &r) {
+        sb = sb < nsb ? sb : nsb - 1;
+        const int pair = kbeg + 4 * sb, slice = pair >> 6, pr = pair & 63; // the four pairs of a superblock share a slice
+        int P = cpr - (slice << 6);
+        P = P < 64 ? P : 64;
+        const uint8_t *cb = cbase + (size_t)slice * 2048 + (size_t)pr * 16, *mb = mbase + (size_t)(pair >> 2) * 16;
+        const uint32_t hoff = (uint32_t)(bh * 16 * P);
 #pragma unroll
-            for (int u = 0; u < BT; u++) {
-                r.q[u] = *reinterpret_cast<const u32x4 *>(crow[u] + (size_t)slice * 2048 + (size_t)bh * 16 * P + (size_t)pr * 16);
-                r.h[u] = *reinterpret_cast<const u32x4 *>(mrow[u] + (size_t)(pair >> 2) * 16);
-            }
-        } else if (step < t_all) {
-            // the minimum term: 64 columns = two superblocks of [hi | hi | lo | 0] x [ch | cl | ch | 0]
-            const int s2 = step - t_main;
-            int sb = (kbeg >> 2) + 2 * s2 + bh;
-            sb = sb < last_sb ? sb : last_sb;
-            // an odd count of superblocks: the second half of the last step lies beyond this part of K (or beyond the row)
-            const bool xlive = 2 * s2 + ((tid & 7) >> 2) < nsb;
+        for (int u = 0; u < BT; u++) {
 #pragma unroll
-            for (int i = 0; i < AV; i++)
-                r.xa[i] = xlive ? *reinterpret_cast<const u32x4 *>(x3row + i * x3step + (size_t)s2 * BK) : u32x4{0, 0, 0, 0};
-#pragma unroll
-            for (int u = 0; u < BT; u++) r.h[u] = *reinterpret_cast<const u32x4 *>(mrow[u] + (size_t)sb * 16);
+            for (int j = 0; j < 4; j++) r.q[u][j] = *reinterpret_cast<const u32x4 *>(cb + j * 16 + (coff[u] + hoff));
+            r.h[u] = *reinterpret_cast<const u32x4 *>(mb + moff[u]);
         }
     };
-    uint32_t dmin_max = 0; // largest |dmin| (f16 bits) this thread has met in the main loop
-    float S = 1.0f;        // the minimum term's power-of-two factor (set one step before the main loop ends)
-    // part t (0..3) of the conversion of `r` (step `step`) into stage `st`
-    auto convert = [&](int step, const Raw &r, int st, int t) {
-        _Float16 *As = lds + st * STAGE, *Bs = As + BM * LDK;
-        {
-            const int v = tid + t * NT;
-            *reinterpret_cast<u32x4 *>(As + (v >> 3) * LDK + (v & 7) * 8) = r.xa[t];
+    // The minimum term: steps 4 grp .. 4 grp + 3 (clamped to the last step); a step = 64 columns = two superblocks of
+    // [hi | hi | lo | 0] x [ch | cl | ch | 0], of which the thread makes one
+    auto fetch_min = [&](int grp, Raw &r) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int s2 = 4 * grp + j;
+            s2 = s2 < t_min ? s2 : t_min - 1;
+            int sb = (kbeg >> 2) + 2 * s2 + bh;
+            sb = sb < last_sb ? sb : last_sb;
+#pragma unroll
+            for (int u = 0; u < BT; u++) r.q[u][j] = *reinterpret_cast<const u32x4 *>(mbase + (size_t)sb * 16 + moff[u]);
         }
-        if (step < t_main) {
-            const int p = (kbeg + step) & 3;
+    };
+    // While the minimum term is added the accumulators of a column hold the result times S, a power of two chosen from the
+    // largest |dmin| (f16 bits) the column's weight row has in this part of K: dmin < 2^(e + 1) -> the operands are
+    // c * 2^(8 - e) < 2^15; they meet sub-block sums stored times 1 / 64, so S = 2^(2 - e).  No dmin, or inf / nan:
+    // operands c, S = 1 / 64.  The feeder of a row and the lanes that own its column both work it out from the row's headers.
+    auto s_of = [](uint32_t mx) {
+        const int e = (mx == 0 || mx >= 0x7C00u) ? 8 : (mx >= 0x400u ? (int)(mx >> 10) - 15 : -15);
+        return __builtin_bit_cast(float, (uint32_t)(127 + 2 - e) << 23);
+    };
+    uint32_t dmax_r[BT];
 #pragma unroll
-            for (int u = 0; u < BT; u++) {
-                const int row = (tid + u * NT) >> 1;
+    for (int u = 0; u < BT; u++) dmax_r[u] = 0;
+    // half c1 (0, 1) of the conversion of main-loop step j (0..3) of the superblock in `r` into weight stage `stage`: bytes
+    // 8 c1 .. 8 c1 + 7 of the thread's 16, i.e. elements 16 bh + 8 c1 .. of both sub-blocks = chunk 2 bh + c1 of the row
+    // (low nibbles) and the chunk four further (high nibbles)
+    auto convert_main = [&](const Raw &r, int j, int stage, int c1) {
+        _Float16 *bs = lds + BOFF + stage * BSTAGE;
+        const int p = j; // kbeg is a multiple of 4: step j of a superblock is its pair j
+#pragma unroll
+        for (int u = 0; u < BT; u++) {
+            uint32_t scp, mp;
+            q4k_scale_min(r.h[u], p, scp, mp);
+            const uint32_t dd = r.h[u][0];
+            scp = (dd & 0x7FFFu) == 0 ? 0u : scp; // d = 0: the superblock adds nothing and leaves the unit alone
+            const uint32_t dm = (dd >> 16) & 0x7FFFu;
+            dmax_r[u] = dm > dmax_r[u] ? dm : dmax_r[u];
+            const uint32_t s0 = scp & 0xFF, s1 = scp >> 8;
+            uint32_t lo[4], hi[4];
+#pragma unroll
+            for (int d = 0; d < 2; d++) {
+                const uint32_t w = r.q[u][j][2 * c1 + d];
+                lo[2 * d] = (w & 0x000F000Fu) * s0;
+                lo[2 * d + 1] = ((w >> 8) & 0x000F000Fu) * s0;
+                hi[2 * d] = ((w >> 4) & 0x000F000Fu) * s1;
+                hi[2 * d + 1] = ((w >> 12) & 0x000F000Fu) * s1;
+            }
+            const int at = b_wr[u] ^ (c1 * 8);
+            *reinterpret_cast<u32x4 *>(bs + at) = u32x4{lo[0], lo[1], lo[2], lo[3]};
+            *reinterpret_cast<u32x4 *>(bs + (at ^ 32)) = u32x4{hi[0], hi[1], hi[2], hi[3]};
+        }
+    };
+    // part t (0..3) of step s2 of the minimum term, whose headers are q[.][j] of `r` (an odd count of superblocks: the
+    // second half of the last step gets zeros, which meet the sums of the next superblock, or the zeros that end an x row)
+    float S_r[BT];
+    auto convert_min = [&](int s2, const Raw &r, int j, int stage, int t) {
+        _Float16 *bs = lds + BOFF + stage * BSTAGE;
+        const bool live = 2 * s2 + bh < nsb;
+#pragma unroll
+        for (int u = 0; u < BT; u++) {
+            const u32x4 h = r.q[u][j];
+            const float dmin = live ? (-64.0f * S_r[u]) * h2f(h[0] >> 16) : 0.f;
+            uint32_t o[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
                 uint32_t scp, mp;
-                q4k_scale_min(r.h[u], p, scp, mp);
-                const uint32_t dd = r.h[u][0];
-                if ((dd & 0x7FFFu) == 0) scp = 0; // d = 0: the superblock adds nothing and leaves the unit alone
-                if (t == 0) {
-                    const uint32_t dm = (dd >> 16) & 0x7FFFu;
-                    dmin_max = dm > dmin_max ? dm : dmin_max;
-                }
-                const uint32_t s0 = scp & 0xFF, s1 = scp >> 8;
-                const uint32_t w = r.q[u][t];
-                // bytes 4t .. 4t+3 of the thread's 16: elements 16 bh + 4t + {0, 1, 2, 3} of both sub-blocks
-                const uint32_t la = (w & 0x000F000Fu) * s0, lb = ((w >> 8) & 0x000F000Fu) * s0;
-                const uint32_t ha = ((w >> 4) & 0x000F000Fu) * s1, hb = ((w >> 12) & 0x000F000Fu) * s1;
-                *reinterpret_cast<uint2 *>(Bs + row * LDK + bh * 16 + t * 4) = make_uint2(la, lb);
-                *reinterpret_cast<uint2 *>(Bs + row * LDK + 32 + bh * 16 + t * 4) = make_uint2(ha, hb);
+                q4k_scale_min(h, p, scp, mp);
+                const float c0 = dmin * ubyte<0>(mp), c1 = dmin * ubyte<1>(mp); // exact: 11 x 6 bits
+                const float h0 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, c0) & 0xFFFFE000u);
+                const float h1 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, c1) & 0xFFFFE000u);
+                const float v0 = t == 1 ? c0 - h0 : h0, v1 = t == 1 ? c1 - h1 : h1; // t: 0 ch, 1 cl, 2 ch, 3 nothing
+                o[p] = t == 3 ? 0u : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(v0, v1));
             }
-        } else {
-            const bool live = 2 * (step - t_main) + bh < nsb; // an odd count of superblocks: the last step's second half is empty
-#pragma unroll
-            for (int u = 0; u < BT; u++) {
-                const int row = (tid + u * NT) >> 1;
-                const u32x4 h = r.h[u];
-                const float dmin = live ? (-64.0f * S) * h2f(h[0] >> 16) : 0.f;
-                uint32_t o[4];
-#pragma unroll
-                for (int p = 0; p < 4; p++) {
-                    uint32_t scp, mp;
-                    q4k_scale_min(h, p, scp, mp);
-                    const float c0 = dmin * ubyte<0>(mp), c1 = dmin * ubyte<1>(mp); // exact: 11 x 6 bits
-                    const float h0 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, c0) & 0xFFFFE000u);
-                    const float h1 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, c1) & 0xFFFFE000u);
-                    const float v0 = t == 1 ? c0 - h0 : h0, v1 = t == 1 ? c1 - h1 : h1; // t: 0 ch, 1 cl, 2 ch, 3 nothing
-                    o[p] = t == 3 ? 0u : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(v0, v1));
-                }
-                *reinterpret_cast<u32x4 *>(Bs + row * LDK + bh * 32 + t * 8) = u32x4{o[0], o[1], o[2], o[3]};
-            }
+            // chunk 4 bh + t of the row; b_wr holds chunk 2 bh (and the exchange)
+            *reinterpret_cast<u32x4 *>(bs + (b_wr[u] ^ (((bh * 6) ^ t) * 8))) = u32x4{o[0], o[1], o[2], o[3]};
         }
     };
 
     // ---- multiplier side
     const int wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
-    const int li = lane & 31, lk = (lane >> 5) * 8;
+    const int li = lane & 31, hh = lane >> 5;
+    // fragment of sub-step t: tile row r = w + 32 i + li, chunk 2 t + hh, stored at chunk ^ ((r / 2) & 7): the address is
+    // (r * 64 + ((hh ^ (li / 2)) & 7) * 8) ^ (16 t) in halfs
+    const int sw = ((hh ^ (li >> 1)) & 7) * 8;
+    const int a_rd = (wm + li) * 64 + sw, b_rd = BOFF + (wn + li) * 64 + sw;
     float16v acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -596,96 +661,147 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-    const uint8_t *dcol[2]; // this lane's two output columns: their superblock headers
+    uint32_t doff[2]; // this lane's two output columns: their superblock headers
     float unit[2] = {1.0f, 1.0f};
-    uint32_t dnext[2];
+    uint32_t dnext[2], dmax_c[2] = {0, 0};
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        int gn = n0 + wn + j * 32 + li;
-        gn = gn < a.n ? gn : a.n - 1;
-        dcol[j] = a.meta + (size_t)gn * a.meta_pitch;
-        dnext[j] = *reinterpret_cast<const uint16_t *>(dcol[j] + (size_t)(kbeg >> 2) * 16);
+        int col = wn + j * 32 + li;
+        col = n0 + col < a.n ? col : a.n - 1 - n0;
+        doff[j] = (uint32_t)col * (uint32_t)a.meta_pitch;
+        dnext[j] = *reinterpret_cast<const uint32_t *>(mbase + (size_t)(kbeg >> 2) * 16 + doff[j]);
     }
-
-    Raw cur, nxt;
-    fetch(0, cur);
-    fetch(1, nxt);
+    // a new superblock (index sb of the row): the accumulators change their unit to its d (no branches: the loads at the end
+    // must be the same on every path, see load_x)
+    auto new_unit = [&](int sb) {
+        const int sbn = sb + 1 < last_sb ? sb + 1 : last_sb;
+        float r[2];
 #pragma unroll
-    for (int t = 0; t < 4; t++) convert(0, cur, 0, t);
-    cur = nxt;
-    __syncthreads();
-    for (int ks = 0; ks < t_all; ks++) {
-        const _Float16 *As = lds + (ks & 1) * STAGE, *Bs = As + BM * LDK;
-        fetch(ks + 2, nxt);
-        if (ks == t_main - 1) { // every main-loop header has been seen: the factor of the minimum term
-            uint32_t mx = 0;
-            for (int w = 0; w < NW; w++) {
-                const uint32_t v = __builtin_bit_cast(uint32_t, wg_red[w]);
-                mx = v > mx ? v : mx;
-            }
-            // dmin < 2^(e + 1) -> the operands are c * 2^(8 - e) < 2^15; they meet sub-block sums stored times 1 / 64, so
-            // the accumulators then hold the result times S = 2^(2 - e).  No dmin, or inf / nan: operands c, S = 1 / 64.
-            const int e = (mx == 0 || mx >= 0x7C00u) ? 8 : (mx >= 0x400u ? (int)(mx >> 10) - 15 : -15);
-            S = __builtin_bit_cast(float, (uint32_t)(127 + 2 - e) << 23);
-        }
-        if (ks < t_main && ((kbeg + ks) & 3) == 0) {
-            // a new superblock: the accumulators change their unit to its d
-            const int sbn = ((kbeg + ks) >> 2) + 1;
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const float dn = h2f(dnext[j]);
-                const float r = dn != 0.f ? unit[j] / dn : 1.0f;
-                unit[j] = dn != 0.f ? dn : unit[j];
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-#pragma unroll
-                    for (int q = 0; q < 16; q++) acc[i][j][q] *= r;
-                dnext[j] = *reinterpret_cast<const uint16_t *>(dcol[j] + (size_t)(sbn < last_sb ? sbn : last_sb) * 16);
-            }
-        }
-        if (ks == t_main) { // the main sum in true units, times S: the minimum term joins it
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const float f = unit[j] * 16777216.0f * S;
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-#pragma unroll
-                    for (int q = 0; q < 16; q++) acc[i][j][q] *= f;
-            }
+        for (int j = 0; j < 2; j++) {
+            const float dn = h2f(dnext[j] & 0xFFFFu);
+            const uint32_t dm = (dnext[j] >> 16) & 0x7FFFu;
+            dmax_c[j] = dm > dmax_c[j] ? dm : dmax_c[j];
+            const bool some = dn != 0.f;
+            const float q = unit[j] / (some ? dn : 1.0f);
+            r[j] = some ? q : 1.0f;
+            unit[j] = some ? dn : unit[j];
+            dnext[j] = *reinterpret_cast<const uint32_t *>(mbase + (size_t)sbn * 16 + doff[j]);
         }
 #pragma unroll
-        for (int t = 0; t < BK / 16; t++) {
-            // two waves share a SIMD: while this one waits for its fragments the other one multiplies
-            half8 af[4], bf[2];
-#pragma unroll
-            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const half8 *>(As + (wm + i * 32 + li) * LDK + t * 16 + lk);
-#pragma unroll
-            for (int j = 0; j < 2; j++) bf[j] = *reinterpret_cast<const half8 *>(Bs + (wn + j * 32 + li) * LDK + t * 16 + lk);
+        for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-            if (ks + 1 < t_all) convert(ks + 1, cur, (ks + 1) & 1, t);
-        }
-        if (ks == t_main - 2) { // the last main-loop header is converted in this step
-            uint32_t mx = dmin_max;
+                for (int q = 0; q < 16; q++) acc[i][j][q] *= r[j];
+    };
+    // the eight MFMAs of sub-step t (x stage at halfs `as`, weight stage PAR); the x fragments two at a time: registers
+    // are short, and while this wave waits for fragments the other wave of its SIMD multiplies
+    auto multiply = [&](int as, int par, int t) {
+        half8 bf[2];
 #pragma unroll
-            for (int s = 32; s >= 1; s >>= 1) {
-                const uint32_t o = (uint32_t)__shfl_xor((int)mx, s);
-                mx = o > mx ? o : mx;
+        for (int j = 0; j < 2; j++) bf[j] = *reinterpret_cast<const half8 *>(lds + par * BSTAGE + (b_rd ^ (t * 16)) + j * 32 * 64);
+#pragma unroll
+        for (int ih = 0; ih < 2; ih++) {
+            half8 af[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) af[i] = *reinterpret_cast<const half8 *>(lds + as + (a_rd ^ (t * 16)) + (2 * ih + i) * 32 * 64);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[2 * ih + i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[2 * ih + i][j], 0, 0, 0);
+        }
+    };
+    // The steps of the main loop and of the minimum term are numbered through, g = 0 .. t_main + t_min - 1, and taken in
+    // groups of four (a superblock of the main loop; four steps of the minimum term).  Step g multiplies x stage g % 3 with
+    // weight stage g & 1, brings the x tile of step g + 2 into its stage and converts the packed weights of step g + 1
+    // into the other weight stage; the first step of a group also requests the packed weights of the next group.  Every
+    // path through a step issues the same loads in the same order, so that the wait in front of its barrier (for the
+    // x tile of step g + 1, requested a step ago) can leave the younger requests in flight.
+    Raw cur, nxt; // this group's packed weights, the next group's
+    const int sb0 = kbeg >> 2;
+    int g3 = 0;   // g % 3
+    // One group.  KG, KN, KF: kind (0 main, 1 minimum term) of this group, the next one, and the one after (whose x tiles
+    // this one does not touch); grp: index of the group among those of its kind.
+    auto group = [&](auto kg, auto kn, int grp) {
+        constexpr bool KG = decltype(kg)::value, KN = decltype(kn)::value;
+        constexpr int F = KN ? 4 * BT : 5 * BT; // loads of the weight request
+        if (!KG) new_unit(sb0 + grp);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (KG && 4 * grp + i >= t_min) break; // the minimum term's last group may be short (the same for every wave)
+            const int as = g3 * ASTAGE, xs = (g3 == 0 ? 2 : g3 - 1); // x stages g % 3 and (g + 2) % 3
+            // x tile of step g + 2: of this group (i < 2) or the next
+            if (i < 2) load_x(kg, 4 * grp + i + 2, xs);
+            else load_x(kn, (KG == KN ? 4 * grp + 4 : 0) + i - 2, xs);
+            if (i == 0) {
+                if (KN) fetch_min(KG ? grp + 1 : 0, nxt);
+                else fetch_main(grp + 1, nxt);
             }
-            if (lane == 0) wg_red[wave] = __builtin_bit_cast(float, mx);
+#pragma unroll
+            for (int t = 0; t < BK / 16; t++) {
+                multiply(as, i & 1, t);
+                // step g + 1: of this group (i < 3) or the first of the next
+                if (i < 3) {
+                    if (KG) {
+                        if (4 * grp + i + 1 < t_min) convert_min(4 * grp + i + 1, cur, i + 1, (i + 1) & 1, t);
+                    } else if (t & 1) {
+                        convert_main(cur, i + 1, (i + 1) & 1, t >> 1);
+                    }
+                } else {
+                    if (KN) {
+                        const int s2 = KG ? 4 * grp + 4 : 0;
+                        if (s2 < t_min) convert_min(s2, nxt, 0, 0, t);
+                    } else if (t & 1) {
+                        convert_main(nxt, 0, 0, t >> 1);
+                    }
+                }
+            }
+            // younger than the x tile of step g + 1: see the order of the loads above
+            if (i == 0) wait_vm_and_lds<(KG ? 0 : 2) + 4 + F>();
+            else if (i == 1) wait_vm_and_lds<F + 4>();
+            else wait_vm_and_lds<4>();
+            lds_barrier();
+            g3 = g3 == 2 ? 0 : g3 + 1;
+            if (i == 2 && !KG && KN) {
+#pragma unroll
+                for (int u = 0; u < BT; u++) S_r[u] = s_of(dmax_r[u]); // every header of the thread's rows has been looked at
+            }
         }
         cur = nxt;
-        __syncthreads();
+    };
+    using MAIN = std::false_type;
+    using MIN = std::true_type;
+
+    load_x(MAIN{}, 0, 0);
+    load_x(MAIN{}, 1, 1);
+    fetch_main(0, cur);
+    convert_main(cur, 0, 0, 0);
+    convert_main(cur, 0, 0, 1);
+    wait_vm_and_lds<0>();
+    lds_barrier();
+    for (int sb = 0; sb < nsb - 1; sb++) group(MAIN{}, MAIN{}, sb); // every superblock but the last
+    group(MAIN{}, MIN{}, nsb - 1); // the last: what it requests and prepares beyond itself belongs to the minimum term
+    // the main sum in true units, times S: the minimum term joins it
+    float S_c[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        S_c[j] = s_of(dmax_c[j]);
+        const float f = unit[j] * 16777216.0f * S_c[j];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) acc[i][j][q] *= f;
     }
+    for (int grp = 0; 4 * grp < t_min; grp++) group(MIN{}, MIN{}, grp);
+    wait_vm_and_lds<0>(); // nothing of this workgroup may still be on its way into LDS when it ends
     // D layout: lane -> column li; register r -> row 8 * (r / 4) + 4 * (lane / 32) + r % 4
-    const float inv_s = 1.0f / S;
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int gn = n0 + wn + j * 32 + li;
+            const float inv_s = 1.0f / S_c[j];
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int gm = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
@@ -715,9 +831,11 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
 // [hi of its 8 sub-blocks | the same | lo | zeros] (NULL xs3: plain rows for the other kernels).
 struct XSums {
     _Float16 *xs3;
-    int pitch; // halfs per row: k / 8
+    int pitch; // halfs per row: 32 per superblock and 32 or 64 zeros, see xs3_pitch
 };
 constexpr float XSUM_SCALE = 1.0f / 64.0f; // the sums are stored times this
+// one or two superblocks of zeros end a row: the last step of the minimum term may look one superblock past the end
+__host__ __device__ inline int xs3_pitch(int64_t k) { return (int)(((k >> 8) + 2) & ~(int64_t)1) * 32; }
 
 // The sum `s` of the caller's four elements, added over the eight threads of a 32-element group; the first of them
 // stores the pair.  g = index of the group along the row.
@@ -771,6 +889,7 @@ __global__ void __launch_bounds__(256) gemm_prep_x_kernel(const uint16_t *x, int
             reinterpret_cast<half4 *>(xh + (size_t)row * k)[i4] = half4{h0, h1, h2, h3};
         }
     }
+    if (row3 && (int)threadIdx.x < xs.pitch - (k >> 8) * 32) row3[(size_t)(k >> 8) * 32 + threadIdx.x] = (_Float16)0.f; // the zeros that end a row
     if (threadIdx.x == 0) rowscale[row] = 1.0f / f;
 }
 
@@ -939,6 +1058,10 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
             lo_row[i] = (_Float16)(e - (float)hi);
         }
     }
+    if (hi3 && (int)threadIdx.x < xs.pitch - (k >> 8) * 32) { // the zeros that end a row
+        hi3[(size_t)(k >> 8) * 32 + threadIdx.x] = (_Float16)0.f;
+        lo3[(size_t)(k >> 8) * 32 + threadIdx.x] = (_Float16)0.f;
+    }
     if (threadIdx.x == 0) {
         rowscale[2 * row] = 1.0f / f;
         rowscale[2 * row + 1] = 1.0f / f;
@@ -998,7 +1121,7 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, bool f32_rows, size_t ex
     p->xh_bytes = axq_align_up(mpad * (size_t)w->k * 2, 256);
     p->rs_bytes = axq_align_up((size_t)m * 4, 256);
     p->part_bytes = axq_align_up(p->splits > 1 ? (size_t)p->splits * m * (size_t)w->n_rows * 4 : 0, 256);
-    p->xs3_bytes = axq_align_up(p->q4k ? mpad * (size_t)(w->k / 8) * 2 : 0, 256);
+    p->xs3_bytes = axq_align_up(p->q4k ? mpad * (size_t)xs3_pitch(w->k) * 2 : 0, 256);
     return reserve_scratch(ctx, p->xh_bytes + p->rs_bytes + p->part_bytes + p->xs3_bytes + extra);
 }
 
@@ -1007,7 +1130,7 @@ XSums plan_sums(axq_ctx *ctx, const axq_weight *w, const GemmPlan &p) {
     XSums xs = {nullptr, 0};
     if (p.q4k) {
         xs.xs3 = reinterpret_cast<_Float16 *>(reinterpret_cast<uint8_t *>(ctx->gemm_scratch) + p.xh_bytes + p.rs_bytes + p.part_bytes);
-        xs.pitch = (int)(w->k / 8);
+        xs.pitch = xs3_pitch(w->k);
     }
     return xs;
 }
@@ -1017,12 +1140,12 @@ int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits) {
     const int bm = 128 * a.wm;
     const unsigned tiles = (unsigned)(((a.n + QBN - 1) / QBN) * ((a.m + bm - 1) / bm));
     const dim3 grid(tiles, (unsigned)splits);
-    const size_t lds = (size_t)2 * (bm + QBN) * LDK * sizeof(_Float16) + 64; // two stages and a word per wave
+    const size_t lds = (size_t)(3 * bm * 64 + 2 * QBN * 64) * sizeof(_Float16); // three x stages, two weight stages
     if (!attr_set) {
         AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_kernel<256>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * (256 + QBN) * LDK * 2 + 64)), AXQ_ERR_DRIVER);
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)((3 * 256 * 64 + 2 * QBN * 64) * 2)), AXQ_ERR_DRIVER);
         AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_kernel<128>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * (128 + QBN) * LDK * 2 + 64)), AXQ_ERR_DRIVER);
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)((3 * 128 * 64 + 2 * QBN * 64) * 2)), AXQ_ERR_DRIVER);
         attr_set = true;
     }
     if (a.wm == 2) gemm_q4k_kernel<256><<<grid, 512, lds, ctx->stream>>>(a);
