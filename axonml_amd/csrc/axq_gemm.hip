@@ -478,6 +478,7 @@ __device__ inline void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0); // nothing moves across: what follows may count on the waits in front of the barrier
 }
 
 typedef __attribute__((address_space(3))) void lds_void;

@@ -30,6 +30,8 @@
 // kept in flight and refilled as soon as a step has been consumed.
 #include <hip/hip_fp16.h>
 
+#include <stdlib.h>
+
 #include "axq_internal.h"
 #include "axq_split.h"
 
@@ -81,9 +83,15 @@ struct XOp {
 struct Bases { const uint8_t *codes, *meta, *qh; };  // planes at the workgroup's first row
 struct RowOff { uint32_t c, m, h; };                 // (row - first row) * pitch, per plane
 struct LaneOff { uint32_t c[2], m[2], h[2]; };       // the lane's byte offsets inside a row, per plane
-__device__ inline uint4 ld16(const uint8_t *base, uint32_t off) { return *reinterpret_cast<const uint4 *>(base + off); }
-__device__ inline uint32_t ld4(const uint8_t *base, uint32_t off) { return *reinterpret_cast<const uint32_t *>(base + off); }
-__device__ inline uint32_t ld2(const uint8_t *base, uint32_t off) { return *reinterpret_cast<const uint16_t *>(base + off); }
+// Weights are read once per call: non-temporal loads keep them from displacing x and the other kernels' operands in
+// the caches, and stream measurably faster (a pure read of 33 MB: 6.2 against 6.75 us per launch).
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ inline uint4 ld16(const uint8_t *base, uint32_t off) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(base + off));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ inline uint32_t ld4(const uint8_t *base, uint32_t off) { return __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(base + off)); }
+__device__ inline uint32_t ld2(const uint8_t *base, uint32_t off) { return __builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(base + off)); }
 
 // ---------------------------------------------------------------------------
 // Per-type traits.  A lane covers 64 weights of one row per pass = two
@@ -531,6 +539,175 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same kernel with x staged per wave.  Timestamps of the kernel above showed its critical path: x requested
+// 0.4 us after entry, split by all waves together, two workgroup barriers (every wave waits for the one that was held
+// up longest issuing its first weight requests) -- first fold 3.5 us after entry, then seven folds at the vector
+// ALU's pace, 0.5 us each: latency and ALU in series, with the memory stream idling beside them.  Here a wave needs
+// nobody: it fetches and splits the 1024 elements of x of its own K slice (the G row groups of a workgroup repeat
+// that work, which costs less than the barriers did), keeps the split form in an LDS region of its own, and starts
+// folding as soon as its own x and its first weights have arrived.  A fused RMSNorm needs the whole vector's sum
+// of squares, but only as one factor on the result: y = inv_rms * sum_k W[n, k] (x[k] w[k]), so the waves split
+// x[k] w[k] and leave their slices' sums of squares in LDS for the final reduction.
+// ---------------------------------------------------------------------------
+template <class T, int NB>
+__global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(DpArgs a) {
+    extern __shared__ uint4 lds_raw[];
+    constexpr int SLICE_K = 1024, REGION16 = (4 * SLICE_K + (SLICE_K / 32) * 16) / 16; // a wave's split x, in 16-byte units
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g_idx = wave / a.S, slice = wave - g_idx * a.S;
+    const int blk = lane >> 2, j = lane & 3;
+    const int c = (slice << 4) + blk; // this lane's 64-weight chunk of the row
+    const int nwaves = a.G * a.S;
+    const int k0 = slice * SLICE_K;
+    const int klen = a.k - k0 < SLICE_K ? a.k - k0 : SLICE_K; // a multiple of 64
+
+    // 1. x first: this wave's slice, two 8-element tasks per lane (and the norm weights of a fused RMSNorm)
+    const bool live0 = lane * 8 < klen, live1 = (lane + 64) * 8 < klen; // whole quads of lanes
+    const float *xs = a.x + k0 + (live0 ? lane * 8 : (lane & 3) * 8);
+    const float *xs1 = a.x + k0 + (live1 ? (lane + 64) * 8 : (lane & 3) * 8);
+    const uint4 x0 = reinterpret_cast<const uint4 *>(xs)[0], x1 = reinterpret_cast<const uint4 *>(xs)[1];
+    const uint4 x2 = reinterpret_cast<const uint4 *>(xs1)[0], x3 = reinterpret_cast<const uint4 *>(xs1)[1];
+    uint4 e0 = {0, 0, 0, 0}, e1 = e0, e2 = e0, e3 = e0;
+    if (a.mode == AXQ_X_RMSNORM) {
+        const float *es = a.aux + (xs - a.x), *es1 = a.aux + (xs1 - a.x);
+        e0 = reinterpret_cast<const uint4 *>(es)[0]; e1 = reinterpret_cast<const uint4 *>(es)[1];
+        e2 = reinterpret_cast<const uint4 *>(es1)[0]; e3 = reinterpret_cast<const uint4 *>(es1)[1];
+    }
+    // 2. the ring: rows past the group's end re-read its first step (cache hits, no HBM traffic)
+    uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw + wave * REGION16);
+    uint4 *wgrp = reinterpret_cast<uint4 *>(wplanes + 4 * SLICE_K);
+    float *wsum = reinterpret_cast<float *>(lds_raw + nwaves * REGION16); // one float per wave (64 bytes kept)
+    float *red = wsum + 16;
+    const int rows_per_group = a.steps * 4;
+    const int last = a.n_rows - 1;
+    const int red_stride = 4 * a.S; // partial sums per output row in the LDS reduction buffer
+    float *red_lane = red + (g_idx * rows_per_group + j) * red_stride + slice * 4 + (lane >> 4);
+    typename T::Raw buf[NB];
+    LaneOff lo;
+    T::lane_offsets(a, c, lo);
+    const int wg_row0 = blockIdx.x * a.G * rows_per_group;
+    const Bases bases = {a.codes + (size_t)wg_row0 * a.codes_pitch, a.meta + (size_t)wg_row0 * a.meta_pitch,
+                         a.qh + (size_t)wg_row0 * a.qh_pitch};
+    const uint32_t cp = (uint32_t)a.codes_pitch, mp = (uint32_t)a.meta_pitch, qp = (uint32_t)a.qh_pitch;
+    const int rl0 = g_idx * rows_per_group + j, rl_last = last - wg_row0; // rows relative to the workgroup's first
+    auto request = [&](int step, int b) {
+        int rl = rl0 + 4 * (step < a.steps ? step : 0);
+        rl = rl < rl_last ? rl : rl_last;
+        const RowOff ro = {(uint32_t)rl * cp, (uint32_t)rl * mp, (uint32_t)rl * qp};
+        T::load(bases, ro, lo, buf[b]);
+    };
+    constexpr int NB0 = NB < 2 ? NB : 2; // steps requested before x is split: enough to start the stream, few enough that
+                                         // the wave is not held up issuing them when its x arrives
+#pragma unroll
+    for (int b = 0; b < NB0; b++) request(b, b);
+    // 3. x -> split form in the wave's own LDS region -> this lane's A operands
+    {
+        auto unpack = [](const uint4 &lo4, const uint4 &hi4, float (&v)[8]) {
+            v[0] = __builtin_bit_cast(float, lo4.x); v[1] = __builtin_bit_cast(float, lo4.y);
+            v[2] = __builtin_bit_cast(float, lo4.z); v[3] = __builtin_bit_cast(float, lo4.w);
+            v[4] = __builtin_bit_cast(float, hi4.x); v[5] = __builtin_bit_cast(float, hi4.y);
+            v[6] = __builtin_bit_cast(float, hi4.z); v[7] = __builtin_bit_cast(float, hi4.w);
+        };
+        float xv[2][8], ev[2][8];
+        unpack(x0, x1, xv[0]);
+        unpack(x2, x3, xv[1]);
+        if (a.mode == AXQ_X_RMSNORM) {
+            // RMSNorm::forward (llm/src/llama.rs:158-187): (x / rms) * w; the 1 / rms is applied to the result
+            unpack(e0, e1, ev[0]);
+            unpack(e2, e3, ev[1]);
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                if (live0) ss = fmaf(xv[0][i], xv[0][i], ss);
+                if (live1) ss = fmaf(xv[1][i], xv[1][i], ss);
+            }
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+            if (lane == 0) wsum[wave] = ss; // read after the final barrier (group 0's waves cover K once)
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                xv[0][i] *= ev[0][i];
+                xv[1][i] *= ev[1][i];
+            }
+        }
+        if (!live0) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) xv[0][i] = 0.f;
+        }
+        if (!live1) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) xv[1][i] = 0.f;
+        }
+        axq_split8(xv[0], lane, live0, wplanes, wgrp, SLICE_K);
+        axq_split8(xv[1], lane + 64, live1, wplanes, wgrp, SLICE_K);
+    }
+    XOp xo;
+    fetch_xop<T>(wplanes, wgrp, SLICE_K, klen, j, blk, xo); // same wave: LDS serves its stores and loads in order
+#pragma unroll
+    for (int b = NB0; b < NB; b++) request(b, b);
+
+    // 4. fold the steps through the ring
+    const bool writer = (blk & 3) == 3;
+    const int red_step = 4 * red_stride;
+    auto fold = [&](int b, int step) {
+        float tot = sum_within_row(T::dot(buf[b], xo, c));
+        if (writer) red_lane[step * red_step] = tot;
+    };
+    const int rounds = (a.steps + NB - 1) / NB;
+    int step = 0;
+    for (int round = 0; round < rounds - 1; round++, step += NB) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            fold(b, step + b);
+            request(step + NB + b, b);
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+        if (step + b < a.steps) fold(b, step + b); // the last round may be short: its spare slots hold re-reads
+
+    // partial sums -> y, in a fixed order
+    __syncthreads();
+    const int nthreads = 64 * nwaves;
+    const int wg_rows = a.G * rows_per_group;
+    float inv = 1.0f;
+    if (a.mode == AXQ_X_RMSNORM) {
+        float tot = 0.f;
+        for (int s = 0; s < a.S; s++) tot += wsum[s];
+        inv = 1.0f / sqrtf(tot / (float)a.k + a.eps);
+    }
+    auto row_total = [&](int t) { // slice by slice, the four DPP rows of each in order
+        const float4 *pr = reinterpret_cast<const float4 *>(red + (size_t)t * red_stride);
+        float tot = 0.f;
+        for (int s = 0; s < a.S; s++) {
+            float4 v = pr[s];
+            tot += (v.x + v.y) + (v.z + v.w);
+        }
+        return tot * inv;
+    };
+    if (a.ymode == AXQ_Y_SWIGLU) {
+        // rows 8b..8b+3 are gate rows, 8b+4..8b+7 the up rows of the same outputs (wg_rows is a multiple of 8)
+        for (int t = tid; t < (wg_rows >> 1); t += nthreads) {
+            const int lg = ((t >> 2) << 3) + (t & 3);
+            const int row = blockIdx.x * wg_rows + lg;
+            if (row + 4 < a.n_rows) {
+                const float g = row_total(lg), u = row_total(lg + 4);
+                a.y[(blockIdx.x * wg_rows >> 1) + t] = (g * (1.0f / (1.0f + expf(-g)))) * u;
+            }
+        }
+        return;
+    }
+    for (int t = tid; t < wg_rows; t += nthreads) {
+        int row = blockIdx.x * wg_rows + t;
+        if (row < a.n_rows) {
+            const float tot = row_total(t);
+            a.y[row] = a.bias ? tot + a.bias[row] : tot;
+        }
+    }
+}
+
 __global__ void __launch_bounds__(256) prep_x_kernel(const float *x, int k, uint8_t *xq) {
     const int kpad = (k + 15) & ~15;
     stage_x(x, k, xq, reinterpret_cast<uint4 *>(xq + (size_t)4 * kpad), (int)(blockIdx.x * blockDim.x + threadIdx.x),
@@ -540,6 +717,21 @@ __global__ void __launch_bounds__(256) prep_x_kernel(const float *x, int k, uint
 template <class T, int NB, bool PRE>
 void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
     static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
+    static const bool shared_x = getenv("AXQ_GEMV_SHARED_X") && getenv("AXQ_GEMV_SHARED_X")[0] == '1'; // development knob: the kernel that splits x once per workgroup
+    if (!PRE && !shared_x) {
+        // x arrives raw: every wave stages its own slice
+        const size_t lds_w = (size_t)(block / 64) * (4 * 1024 + 32 * 16) + 64 + (size_t)a.G * a.steps * 4 * a.S * 4 * sizeof(float);
+        static bool big_lds_allowed_w = false;
+        if (lds_w > 64 * 1024 && !big_lds_allowed_w) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      160 * 1024);
+            big_lds_allowed_w = true;
+        }
+        if (lds_w <= 160 * 1024) {
+            gemv_dpw_kernel<T, NB><<<grid, block, lds_w, ctx->stream>>>(a);
+            return;
+        }
+    }
     if (lds > 64 * 1024 && !big_lds_allowed) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
