@@ -32,7 +32,9 @@ def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(
                     ctx.check(lib.axq_gemm_bf16(ctx.handle, h, xd, m, yd, MEM_DEVICE))
                 t = ctx.timer_stop() / iters
                 flops = 2.0 * m * n * k
-                r = {"type": str(qt), "m": m, "n": n, "k": k, "ms": t, "tflops": flops / (t * 1e-3) / 1e12}
+                r = {"type": str(qt), "m": m, "n": n, "k": k, "ms": t, "tflops": flops / (t * 1e-3) / 1e12,
+                     "route": "hand-written MFMA GEMM, scaled codes as f16, one product per weight" if qt == QuantType.Q4_K
+                     else "hand-written MFMA GEMM, weights dequantised to two f16 terms, two products per weight"}
                 r["frac_of_mfma_f16_peak"] = r["tflops"] / MFMA_F16_PEAK_TFLOPS
                 out.append(r)
                 log(f"  prefill {r['type']} M={m} N={n}: {t * 1e3:.1f} us, {r['tflops']:.1f} TFLOP/s")

@@ -52,15 +52,46 @@ def make_ring(ctx, qtype, n, k, copies, outlier_p, seed0=1234):
     return ws
 
 
+INTERNAL_WARMUP = 200  # untimed launches before any timed one, whatever --warmup says (clocks and caches settle)
+MIN_PER_REPEAT = 200   # launches between one pair of events, at least
+REPEATS = 25           # timed repeats, each between its own pair of events; the median repeat is reported
+
+
+def time_ring(ctx, launch, ring_len, steps, warmup):
+    """launch(first, count) enqueues `count` launches that walk the ring from position `first`.  Returns (median ms
+    per launch, per-repeat ms per launch, launches per repeat, untimed launches).  The timed launches are split into
+    REPEATS event-bracketed repeats of steps // REPEATS launches, and of MIN_PER_REPEAT at least: the queue is empty
+    when a repeat starts, and the 20 us or so until launches overlap again would otherwise weigh on a short repeat as
+    if it were the kernel's time.  The ring position runs on across repeats, so no repeat starts on a copy the caches
+    still hold."""
+    untimed = max(INTERNAL_WARMUP, warmup)
+    per = max(MIN_PER_REPEAT, steps // REPEATS)
+    pos = 0
+    launch(pos, untimed)
+    pos += untimed
+    ctx.synchronize()
+    times = []
+    for _ in range(REPEATS):
+        ctx.timer_start()
+        launch(pos % ring_len, per)
+        times.append(ctx.timer_stop() / per)
+        pos += per
+    return float(np.median(times)), times, per, untimed
+
+
 def time_gemv(ctx, ws, x_dev, y_dev, batch, steps, warmup):
     lib = ctx.lib
     arr = (C.c_void_p * len(ws))(*[w.value for w in ws])
-    ctx.check(lib.axq_bench_gemv_ring(ctx.handle, arr, len(ws), x_dev, batch, y_dev, warmup))
-    ctx.synchronize()
-    ctx.timer_start()
-    ctx.check(lib.axq_bench_gemv_ring(ctx.handle, arr, len(ws), x_dev, batch, y_dev, steps))
-    ms = ctx.timer_stop()
-    return ms / steps
+    return time_ring(ctx, lambda first, n: ctx.check(lib.axq_bench_gemv_ring(ctx.handle, arr, len(ws), first, x_dev, batch, y_dev, n)),
+                     len(ws), steps, warmup)
+
+
+def time_read(ctx, ws, sink_dev, steps, warmup):
+    """The same ring under a kernel that only reads each weight's device image, on the GEMV's grid."""
+    lib = ctx.lib
+    arr = (C.c_void_p * len(ws))(*[w.value for w in ws])
+    return time_ring(ctx, lambda first, n: ctx.check(lib.axq_bench_read_ring(ctx.handle, arr, len(ws), first, sink_dev, n)),
+                     len(ws), steps, warmup)
 
 
 def gemv_case(ctx, qtype, n, k, batch, steps, warmup, outlier_p=0.0, ring=True):
@@ -74,9 +105,10 @@ def gemv_case(ctx, qtype, n, k, batch, steps, warmup, outlier_p=0.0, ring=True):
     x = rng.standard_normal((batch, k)).astype(np.float32)
     x_dev = ctx.to_device(x)
     y_dev = ctx.malloc(batch * n * 4)
-    ms = time_gemv(ctx, ws, x_dev, y_dev, batch, steps, warmup)
+    ms, times, per, untimed = time_gemv(ctx, ws, x_dev, y_dev, batch, steps, warmup)
     algo_bytes = wbytes + 4 * batch * (n + k)
     res = {"type": str(q.QuantType(qtype)), "n": n, "k": k, "batch": batch, "us_per_step": ms * 1e3,
+           "us_per_step_min_max": [min(times) * 1e3, max(times) * 1e3], "launches_per_repeat": per, "untimed_launches": untimed,
            "algorithmic_bytes": algo_bytes, "gbps": algo_bytes / (ms * 1e-3) / 1e9, "ring_copies": copies}
     res["frac_of_hbm_peak"] = res["gbps"] / HBM_PEAK_GBPS
     return res, ws, x, x_dev, y_dev
@@ -261,6 +293,7 @@ def main():
     from axonml_amd import quant as q
 
     ctx = q.default_context()
+    lib = ctx.lib
     info = ctx.device_info()
     log(f"device: {info.name.decode()} {info.arch.decode()} CUs={info.compute_units}")
     T = q.QuantType
@@ -275,8 +308,15 @@ def main():
     log(f"headline: {head['us_per_step']:.2f} us/step, {head['gbps']:.0f} GB/s, max rel err vs oracle {err:.2e}")
     if err > 1e-3:
         sys.exit(f"bench.py: GPU result differs from the oracle (max rel err {err:.3e} > 1e-3)")
+    # the read ceiling of the same run: the same ring, the same grid, a kernel that only reads
+    sink = ctx.malloc(256)
+    ms_read, _, _, _ = time_read(ctx, ws, sink, args.steps, args.warmup)
+    ctx.free(sink)
+    read_gbps = lib.axq_packed_bytes(int(T.Q4_K), N_HEAD * K_HEAD) / (ms_read * 1e-3) / 1e9
+    log(f"read-only kernel over the same ring: {ms_read * 1e3:.2f} us/launch, {read_gbps:.0f} GB/s; "
+        f"the GEMV runs at {head['gbps'] / read_gbps:.2f} of it")
     # cache-resident figure, labelled as such
-    ms_hot = time_gemv(ctx, ws[:1], x_dev, y_dev, 1, args.steps, args.warmup)
+    ms_hot = time_gemv(ctx, ws[:1], x_dev, y_dev, 1, args.steps, args.warmup)[0]
     free_case(ctx, ws, x_dev, y_dev)
 
     cpu = None
@@ -284,7 +324,12 @@ def main():
         cpu = cpu_baseline(packed, T.Q4_K, N_HEAD, K_HEAD, x)
         log(f"cpu baseline: {cpu['ms_per_step']:.1f} ms/step on {cpu['cores']} threads")
 
-    extra = {"headline_cache_resident_us": ms_hot * 1e3,
+    extra = {"read_ceiling_gbps": read_gbps, "read_ceiling_us": ms_read * 1e3,
+             "read_ceiling_note": "same run, same ring of weight copies, one 512-thread workgroup per compute unit reading each "
+                                  "copy's packed image with non-temporal 16-byte loads and keeping nothing",
+             "frac_of_read_ceiling": head["gbps"] / read_gbps,
+             "headline_us_per_step_min_max_over_repeats": head["us_per_step_min_max"],
+             "headline_cache_resident_us": ms_hot * 1e3,
              "headline_cache_resident_gbps": head["algorithmic_bytes"] / (ms_hot * 1e-3) / 1e9,
              "max_rel_err_vs_oracle": err}
     if not args.no_extras:
@@ -294,7 +339,7 @@ def main():
                  (T.Q4_1, 4096, 11008, 8, 0.0)]
         gem = []
         for qt, n, k, b, op in cases:
-            r, ws2, _, xd, yd = gemv_case(ctx, qt, n, k, b, max(200, args.steps // 4), 50, outlier_p=op)
+            r, ws2, _, xd, yd = gemv_case(ctx, qt, n, k, b, args.steps, 50, outlier_p=op)
             free_case(ctx, ws2, xd, yd)
             gem.append(r)
             log(f"  {r['type']} [{n},{k}] b={b}: {r['us_per_step']:.2f} us, {r['gbps']:.0f} GB/s")
@@ -337,14 +382,24 @@ def main():
         "data": "synthetic",
         "config": {"workload": "Q4_K GEMV 14336x4096, batch 1 (BASELINE config 3)", "quant_type": "Q4_K",
                    "n_rows": N_HEAD, "k": K_HEAD, "batch": 1, "ring_copies": head["ring_copies"],
+                   "repeats": REPEATS, "launches_per_repeat": head["launches_per_repeat"],
+                   "internal_warmup": head["untimed_launches"],
+                   "timing": "median over `repeats` event-bracketed repeats of `launches_per_repeat` = max(200, steps / repeats) "
+                             "back-to-back launches each, after `internal_warmup` untimed launches",
                    "algorithmic_bytes_per_step": head["algorithmic_bytes"],
                    "inputs": "W~N(0,0.02) with 1% at +-0.5, x~N(0,1), generated and quantised on the device"},
         "roofline": {"bound": "hbm", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": head["gbps"] / HBM_PEAK_GBPS, "traffic": measured_traffic()},
+                     "frac": head["gbps"] / HBM_PEAK_GBPS, "traffic": measured_traffic(),
+                     "traffic_source": "profiles/gemv_q4k_14336x4096_hbm_counters.txt (profiler counter runs of this "
+                                       "kernel), not measured in this run"},
         "cpu_baseline": cpu,
         "extra": extra,
     }
     print(json.dumps(out), flush=True)
+    # Leave at once: the context's teardown and the host thread pool's have nothing left to do for the caller, and
+    # a process that lingers after its one line of output looks like a stray to whoever launched it.
+    sys.stderr.flush()
+    os._exit(0)
 
 
 if __name__ == "__main__":

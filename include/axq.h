@@ -287,10 +287,16 @@ AXQ_API int axq_model_set_sampling(axq_model *m, const axq_sampling_config *cfg,
 AXQ_API int axq_fill_normal_f32(axq_ctx *ctx, float *dst_dev, size_t n, float mean, float std, float outlier_p,
                                 float outlier_mag, uint64_t seed);
 
-/* Enqueues `iters` GEMV launches back to back from C, launch i using weights[i % n_weights] (a ring
+/* Enqueues `iters` GEMV launches back to back from C, launch i using weights[(first + i) % n_weights] (a ring
  * of copies larger than the last-level cache keeps every launch streaming from HBM).  Device pointers. */
-AXQ_API int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, const float *x_dev,
-                                int batch, float *y_dev, int iters);
+AXQ_API int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
+                                const float *x_dev, int batch, float *y_dev, int iters);
+
+/* The same ring walked by a kernel that only reads each weight's device image (one 512-thread workgroup per
+ * compute unit, non-temporal 16-byte loads): the rate the memory system gives a launch of that size, to set
+ * beside the GEMV's.  sink_dev: four writable device bytes. */
+AXQ_API int axq_bench_read_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
+                                uint32_t *sink_dev, int iters);
 
 /* Enqueues `iters` launches of a plain copy kernel (reads `bytes`, writes `bytes`; both pointers and the
  * size multiples of 16).  A kernel of known traffic against which profiler memory counters are scaled. */
