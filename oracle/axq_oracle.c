@@ -41,7 +41,10 @@
  *     aliases Q4_0, quantize.rs:47-50; Q4_K does not exist).  Byte layouts
  *     follow the public GGUF block spec and are pinned by hand-built blocks;
  *     the QUANTISER rules are this build's own ("parity unpinned": nothing in
- *     the reference can confirm them).
+ *     the reference can confirm them).  What the rules say is pinned by
+ *     known-answer blocks worked by hand (half-way values, a whole Q4_K
+ *     superblock with power-of-two spans, the 6-bit rounding of scale and
+ *     minimum) and by the error bound the rule implies from the stored fields.
  *
  * Build: see oracle/Makefile (gcc, -O2 -ffp-contract=off, no fast-math).
  */

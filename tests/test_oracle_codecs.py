@@ -318,21 +318,147 @@ def test_q4_k_six_bit_fields_roundtrip_all_values():
         assert got == want, (base, got, want)
 
 
+# --------------------------------------------------------------------------- quantiser rules of the GGUF-only types, by hand
+def _pack_q5(codes):
+    """32 five-bit codes -> (qh, qs) in the GGUF order: element j < 16 in the low nibble of qs[j] and bit j of qh,
+    element j + 16 in the high nibble of qs[j] and bit j + 16."""
+    qh = sum(((c >> 4) & 1) << e for e, c in enumerate(codes))
+    qs = [(codes[j] & 15) | ((codes[j + 16] & 15) << 4) for j in range(16)]
+    return [qh & 255, (qh >> 8) & 255, (qh >> 16) & 255, qh >> 24], qs
+
+
+def test_q5_0_known_block_with_half_way_values():
+    # max |x| = 15 -> scale 1.0; q = round half away from zero, stored code = q + 16
+    x = np.zeros(32, np.float32)
+    x[:16] = [-15, 2.5, -2.5, 14.5, -14.5, 0, 1, -1, 0.49, -0.49, 7, -8, 0.5, -0.5, 15, 3]
+    x[16], x[31] = 0.5, -0.5
+    codes = [1, 19, 13, 31, 1, 16, 17, 15, 16, 16, 23, 8, 17, 15, 31, 19] + [17] + [16] * 14 + [15]
+    qh, qs = _pack_q5(codes)
+    assert qh == [0x6A, 0xD7, 0xFF, 0x7F]  # worked by hand from the bit 4 of each code
+    assert o.quantize(o.Q5_0, x).tolist() == [0x00, 0x3C] + qh + qs
+    # scale = max_abs / 15 is not a power of two in general: 7.5 / 15 = 0.5, -7.5 -> -15 -> code 1, 0.25 -> 0.5 -> 1 -> code 17
+    y = np.zeros(32, np.float32)
+    y[0], y[1], y[2] = -7.5, 0.25, -0.25
+    qh, qs = _pack_q5([1, 17, 15] + [16] * 29)
+    assert o.quantize(o.Q5_0, y).tolist() == [0x00, 0x38] + qh + qs
+    # zero block: scale 1.0, every code 16
+    qh, qs = _pack_q5([16] * 32)
+    assert o.quantize(o.Q5_0, np.zeros(32, np.float32)).tolist() == [0x00, 0x3C] + qh + qs
+
+
+def test_q5_1_known_block_with_half_way_values():
+    # min -2, max 29 -> scale 31 / 31 = 1.0; code = round half away ((x - min) / scale)
+    x = np.full(32, -2.0, np.float32)
+    x[1], x[2], x[3], x[4], x[5], x[20], x[31] = 29, 0.5, -1.5, 27.5, -1.51, 13.49, 14.0
+    codes = [0, 31, 3, 1, 30, 0] + [0] * 14 + [15] + [0] * 10 + [16]
+    qh, qs = _pack_q5(codes)
+    assert o.quantize(o.Q5_1, x).tolist() == [0x00, 0x3C, 0x00, 0xC0] + qh + qs
+    # constant block: scale 1.0, min = the value, codes 0
+    qh, qs = _pack_q5([0] * 32)
+    assert o.quantize(o.Q5_1, np.full(32, 0.75, np.float32)).tolist() == [0x00, 0x3C, 0x00, 0x3A] + qh + qs
+    # a span that is not a power of two: min 1, max 16.5 -> scale 0.5 (15.5 / 31), 1.25 -> 0.5 -> code 1, 1.24 -> code 0
+    z = np.full(32, 1.0, np.float32)
+    z[1], z[2], z[3] = 16.5, 1.25, 1.24
+    qh, qs = _pack_q5([0, 31, 1, 0] + [0] * 28)
+    assert o.quantize(o.Q5_1, z).tolist() == [0x00, 0x38, 0x00, 0x3C] + qh + qs
+
+
+def _pack_q4k_codes(q):
+    """256 four-bit codes -> qs[128]: pair p holds sub-block 2p in the low nibbles and 2p + 1 in the high."""
+    return [q[64 * p + l] | (q[64 * p + 32 + l] << 4) for p in range(4) for l in range(32)]
+
+
+def test_q4_k_known_superblock_worked_by_hand():
+    """Sub-block s spans [-lm_s / 32, -lm_s / 32 + 15 ls_s / 64]: every quantity of the rule is an integer over a power
+    of two.  max scale = 63/64 -> d = 1/64 (f16 0x2400), max min = 63/32 -> dmin = 1/32 (f16 0x2800), the 6-bit
+    fields come back as the ls, lm chosen, and every code as placed (half-way values round away from zero)."""
+    ls = [63, 1, 2, 32, 33, 47, 16, 0]  # sub-block 7 is constant: scale 0, codes 0
+    lm = [63, 0, 5, 31, 32, 48, 17, 9]  # sub-block 1 has no negative value: min 0
+    q = [[(7 * i + s) % 16 for i in range(32)] for s in range(8)]  # every code 0..15 twice per sub-block
+    q[7] = [0] * 32
+    x = np.zeros(256, np.float32)
+    for s in range(8):
+        for i in range(32):
+            x[32 * s + i] = ls[s] / 64 * q[s][i] - lm[s] / 32
+    # half-way values inside the range of sub-block 3 (step 1/2, offset 31/32): 6.5 steps -> 7, 13.5 steps -> 14
+    x[96 + 5], x[96 + 6] = 0.5 * 6.5 - 31 / 32, 0.5 * 13.5 - 31 / 32
+    q[3][5], q[3][6] = 7, 14
+    scales = [191, 129, 66, 32, 191, 192, 69, 31, 1, 15, 16, 144]  # packed by hand from ls, lm (get_scale_min_k4 order)
+    want = [0x00, 0x24, 0x00, 0x28] + scales + _pack_q4k_codes([c for sub in q for c in sub])
+    got = o.quantize(o.Q4_K, x)
+    assert got.tolist() == want
+    y = o.dequantize(o.Q4_K, got, 256)
+    keep = np.ones(256, bool)
+    keep[[96 + 5, 96 + 6]] = False
+    assert np.array_equal(y[keep], x[keep])  # everything but the two half-way values is a grid point
+    assert y[96 + 5] == 0.5 * 7 - 31 / 32 and y[96 + 6] == 0.5 * 14 - 31 / 32
+
+
+def test_q4_k_six_bit_rounding_is_to_nearest_half_away():
+    # two sub-blocks with spans 15 and 7.5 -> scales 1 and 0.5 -> ls = 63 and round(31.5) = 32; mins 4 and 2.03 -> lm = 63 and
+    # round(31.97) = 32; d = f16(1/63) = 0x2410 (2^-6 * (1 + 16/1024)), dmin = f16(4/63) = 0x2C10
+    x = np.zeros(256, np.float32)
+    x[0], x[1] = -4.0, 11.0
+    x[32], x[33] = -2.03, np.float32(7.5) + np.float32(-2.03)
+    p = o.quantize(o.Q4_K, x)
+    assert p[:4].tolist() == [0x10, 0x24, 0x10, 0x2C]
+    assert (p[4] & 63, p[5] & 63, p[8] & 63, p[9] & 63) == (63, 32, 63, 32)
+    # codes with the stored d, dmin: sd = d * 63, sm = dmin * 63 for sub-block 0
+    d, dmin = np.float32(0.015869140625), np.float32(0.0634765625)
+    sd0, sm0 = float(d) * 63, float(dmin) * 63
+    assert (p[16] & 15, p[17] & 15) == (int(np.floor((-4.0 + sm0) / sd0 + 0.5)), min(15, int(np.floor((11.0 + sm0) / sd0 + 0.5))))
+
+
 # --------------------------------------------------------------------------- invariants, all types
-@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K])
+@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1])
 def test_roundtrip_error_bound(qtype):
     rng = np.random.default_rng(11)
     n = 4096
     x = (rng.standard_normal(n) * 0.02).astype(np.float32)
     y = o.dequantize(qtype, o.quantize(qtype, x), n)
-    bs = {o.Q4_K: 32}.get(qtype, 32)
-    xb, yb = x.reshape(-1, bs), y.reshape(-1, bs)
-    levels = {o.Q8_0: 127 * 2, o.Q4_0: 14, o.Q4_1: 15, o.Q5_0: 30, o.Q5_1: 31, o.Q4_K: 15}[qtype]
-    span = xb.max(1) - np.minimum(xb.min(1), 0) if qtype == o.Q4_K else (
-        2 * np.abs(xb).max(1) if qtype in (o.Q8_0, o.Q4_0, o.Q5_0) else xb.max(1) - xb.min(1))
+    xb, yb = x.reshape(-1, 32), y.reshape(-1, 32)
+    levels = {o.Q8_0: 127 * 2, o.Q4_0: 14, o.Q4_1: 15, o.Q5_0: 30, o.Q5_1: 31}[qtype]
+    span = 2 * np.abs(xb).max(1) if qtype in (o.Q8_0, o.Q4_0, o.Q5_0) else xb.max(1) - xb.min(1)
     step = span / levels
-    slack = 1.6 if qtype == o.Q4_K else 0.51  # Q4_K re-quantises its scale and min to 6 bits
-    assert (np.abs(xb - yb).max(1) <= step * slack + np.abs(xb).max(1) * 2 ** -9).all()
+    # half a step, plus the f16 rounding of the scale (and of the minimum) carried over the block's range
+    assert (np.abs(xb - yb).max(1) <= step * 0.5 + np.abs(xb).max(1) * 2 ** -9).all()
+
+
+def _q4k_fields(p):
+    """(d, dmin, ls[8], lm[8]) of one 144-byte superblock, per the GGUF spec."""
+    d, dmin = (float(v) for v in p[0:4].view(np.float16))
+    sc = p[4:16].astype(np.int32)
+    ls = [(sc[j] & 63) if j < 4 else ((sc[j + 4] & 0xF) | ((sc[j - 4] >> 6) << 4)) for j in range(8)]
+    lm = [(sc[j + 4] & 63) if j < 4 else ((sc[j + 4] >> 4) | ((sc[j] >> 6) << 4)) for j in range(8)]
+    return d, dmin, ls, lm
+
+
+def test_q4_k_roundtrip_error_is_what_the_rule_implies():
+    """From the stored fields: a value inside the code range is off by at most half a step sd; one pushed outside it by the
+    6-bit rounding of the scale and the minimum is off by exactly how far outside it lies.  The stored 6-bit fields are the
+    nearest ones: |sd - scale| <= d / 2 and |sm - min| <= dmin / 2, up to the f16 rounding of d and dmin."""
+    rng = np.random.default_rng(12)
+    n = 256 * 64
+    x = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    x[rng.random(n) < 0.01] = 0.5
+    x[256 * 5:256 * 5 + 64] = np.abs(x[256 * 5:256 * 5 + 64])  # two sub-blocks without a negative value
+    packed = o.quantize(o.Q4_K, x)
+    y = o.dequantize(o.Q4_K, packed, n)
+    for b, p in enumerate(packed.reshape(-1, 144)):
+        d, dmin, ls, lm = _q4k_fields(p)
+        xs = x[256 * b:256 * b + 256].astype(np.float64).reshape(8, 32)
+        ys = y[256 * b:256 * b + 256].astype(np.float64).reshape(8, 32)
+        mins = np.maximum(0.0, -xs.min(1))
+        scales = (xs.max(1) + mins) / 15
+        assert abs(d - scales.max() / 63) <= scales.max() / 63 * 2 ** -11 and abs(dmin - mins.max() / 63) <= mins.max() / 63 * 2 ** -11
+        for s in range(8):
+            sd, sm = d * ls[s], dmin * lm[s]
+            assert abs(sd - scales[s]) <= d * 0.5 + scales[s] * 2 ** -10, (b, s)
+            assert abs(sm - mins[s]) <= dmin * 0.5 + mins[s] * 2 ** -10, (b, s)
+            below = max(0.0, mins[s] - sm)                 # how far the smallest value lies under code 0
+            above = max(0.0, xs[s].max() + sm - 15 * sd)   # ... and the largest above code 15
+            bound = max(sd * 0.5, below, above) + 1e-6 * np.abs(xs[s]).max()
+            assert np.abs(xs[s] - ys[s]).max() <= bound, (b, s)
 
 
 def test_q8_0_requantising_dequantised_values_is_idempotent():
