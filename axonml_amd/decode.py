@@ -10,7 +10,7 @@ import numpy as np
 
 from . import _lib
 from ._lib import MEM_HOST
-from .quant import DeviceWeight, QuantType, default_context
+from .quant import DeviceWeight, QuantType, ShapeMismatch, default_context
 
 LINEARS = {"q": 0, "k": 1, "v": 2, "o": 3, "gate": 4, "up": 5, "down": 6}
 
@@ -33,18 +33,24 @@ class QuantizedLlama:
     # ---- weights
     def set_embedding_f16(self, table_bits):
         t = np.ascontiguousarray(table_bits, dtype=np.uint16)
-        assert t.size == self.cfg.vocab_size * self.cfg.hidden_size
+        if t.size != self.cfg.vocab_size * self.cfg.hidden_size:
+            raise ShapeMismatch(f"Shape mismatch: embedding table of {t.size} elements, expected vocab_size * hidden_size = "
+                                f"{self.cfg.vocab_size} * {self.cfg.hidden_size}")
         self.ctx.check(self.ctx.lib.axq_model_set_embedding_f16(self.handle, t.ctypes.data, MEM_HOST))
 
     def set_norm(self, layer, which, w):
         w = np.ascontiguousarray(w, dtype=np.float32)
+        if w.size != self.cfg.hidden_size:  # the library copies hidden_size floats from this pointer
+            raise ShapeMismatch(f"Shape mismatch: norm weight of {w.size} elements, expected hidden_size = {self.cfg.hidden_size}")
         self.ctx.check(self.ctx.lib.axq_model_set_norm(self.handle, layer, which, w.ctypes.data, MEM_HOST))
 
     def set_linear(self, layer, name, weight):
         """weight: QuantizedTensor or DeviceWeight of the linear's [out, in] shape; layer -1 = lm_head."""
+        if name not in LINEARS:
+            raise KeyError(f"unknown linear {name!r}: one of {sorted(LINEARS)}")
         dw = weight if isinstance(weight, DeviceWeight) else DeviceWeight.upload(weight, self.ctx)
         try:
-            self.ctx.check(self.ctx.lib.axq_model_set_linear(self.handle, layer, LINEARS.get(name, 0), dw.handle))
+            self.ctx.check(self.ctx.lib.axq_model_set_linear(self.handle, layer, LINEARS[name], dw.handle))
         finally:
             if dw is not weight:
                 dw.free()

@@ -245,6 +245,12 @@ def test_error_paths(ctx):
                            rms_norm_eps=1e-5, rope_theta=1e4)
     with pytest.raises(q.InvalidData):  # weights not set
         fresh.forward(1)
+    with pytest.raises(q.ShapeMismatch):  # a norm weight that is not hidden_size long
+        fresh.set_norm(0, 0, np.ones(255, np.float32))
+    with pytest.raises(q.ShapeMismatch):  # an embedding table of the wrong size
+        fresh.set_embedding_f16(np.zeros(64 * 255, np.uint16))
+    with pytest.raises(KeyError):  # a projection name that does not exist must not land on q_proj
+        fresh.set_linear(0, "q_proj", q.quantize_tensor(np.zeros((256, 256), np.float32), q.QuantType.Q4_K, ctx))
     for _ in range(c["max_seq_len"]):
         m.forward(1, want_logits=False)
     with pytest.raises(q.Overflow):  # cache full
