@@ -2,6 +2,8 @@
 // device kernels of axq_codec.hip).
 #include <stdlib.h>
 
+#include <stdio.h>
+#include <stdlib.h>
 #include "axq_internal.h"
 
 namespace {

@@ -162,9 +162,9 @@ class QuantizedLlama:
             pass
 
 
-def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
+def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128, one_sequence_only=False):
     """Decode benchmark: Mistral-7B shape, random init, all linears Q4_K, f16 KV cache; greedy, sampled, and several
-    sequences side by side."""
+    sequences side by side (one_sequence_only: the greedy single-sequence run alone, for kernel profiles)."""
     cfg = mistral_7b_config(prompt_len + new_tokens)
     m = QuantizedLlama(ctx, **cfg)
     m.random_init(QuantType.Q4_K, 0.02, 1)
@@ -185,6 +185,9 @@ def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128):
            "frac_of_hbm_peak": bytes_per_token * tok_s / 8e12, "distinct_generated_ids": int(len(set(out.tolist())))}
     log(f"  decode 7B-shape: {tok_s:.1f} tok/s ({res['ms_per_token']:.3f} ms/token, {res['gbps']:.0f} GB/s), "
         f"prefill {res['prefill_tokens_per_s']:.0f} tok/s")
+    if one_sequence_only:
+        m.close()
+        return res
     # the same with the sampler in the loop (temperature 0.8, top-k 40, top-p 0.9, repetition penalty 1.1)
     from .generation import GenerationConfig
 
