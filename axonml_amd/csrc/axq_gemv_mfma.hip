@@ -104,6 +104,12 @@ struct DQ4K {
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 8; // w = d*sc*(q - 8) + (8*d*sc - dmin*m)
     static constexpr int BIG_NB = 4; // row steps a lane can hold within 128 registers
+    static constexpr bool ROUND_META = true; // the kernels that stage x per wave fetch the headers once per round of steps
+    __device__ static void load_codes(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+        r.q0 = ld16(b.codes, ro.c + o.c[0]);
+        r.q1 = ld16(b.codes, ro.c + o.c[1]);
+    }
+    __device__ static void set_header(Raw &r, const uint4 &h) { r.h = h; }
     __device__ static int group_k(int c, int g) { return c * 64 + g * 32; }
     __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
         // the code plane interleaves, per 64-pair slice, the first 16 bytes of every pair, then the second 16
@@ -171,6 +177,9 @@ struct DQ4x {
     static constexpr bool PERM_A = true; // dword w of a block: low nibbles = elements 8w+{0,2,4,6}, high = 8w+{1,3,5,7}
     static constexpr int CENTRE = 8;
     static constexpr int BIG_NB = 4;
+    static constexpr bool ROUND_META = false;
+    __device__ static void load_codes(const Bases &, const RowOff &, const LaneOff &, Raw &) {}
+    __device__ static void set_header(Raw &, const uint4 &) {}
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
     __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
@@ -217,6 +226,9 @@ struct DQ5x {
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 16;
     static constexpr int BIG_NB = 4;
+    static constexpr bool ROUND_META = false;
+    __device__ static void load_codes(const Bases &, const RowOff &, const LaneOff &, Raw &) {}
+    __device__ static void set_header(Raw &, const uint4 &) {}
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
     __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
@@ -267,6 +279,9 @@ struct DQ80 {
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 0;
     static constexpr int BIG_NB = 3;
+    static constexpr bool ROUND_META = false;
+    __device__ static void load_codes(const Bases &, const RowOff &, const LaneOff &, Raw &) {}
+    __device__ static void set_header(Raw &, const uint4 &) {}
     // 16-byte vector v (0..3) of chunk c: vector index along the row; block = vector / 2
     __device__ static int vec_index(int c, int v) { return ((c >> 4) << 6) + (v >> 1) * 32 + (c & 15) * 2 + (v & 1); }
     __device__ static int group_k(int c, int g) { return vec_index(c, 2 * g) * 16; }
@@ -786,6 +801,10 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     const int red_stride = 4 * a.S; // partial sums per output row in the LDS reduction buffer
     float *red_lane = red + (g_idx * rows_per_group + j) * red_stride + slice * 4 + (lane >> 4);
     typename T::Raw buf[NB];
+    // T::ROUND_META (see gemv_q4k_kernel): one header load per round of NB <= 4 steps, parked in an LDS patch of the wave
+    constexpr bool ROUNDS = T::ROUND_META && NB <= 4;
+    uint4 hm = {0, 0, 0, 0};
+    uint4 *wmeta = reinterpret_cast<uint4 *>(red + a.G * rows_per_group * red_stride) + wave * 64;
     LaneOff lo;
     T::lane_offsets(a, c, lo);
     const int wg_row0 = blockIdx.x * a.G * rows_per_group;
@@ -793,11 +812,24 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
                          a.qh + (size_t)wg_row0 * a.qh_pitch};
     const uint32_t cp = (uint32_t)a.codes_pitch, mp = (uint32_t)a.meta_pitch, qp = (uint32_t)a.qh_pitch;
     const int rl0 = g_idx * rows_per_group + j, rl_last = last - wg_row0; // rows relative to the workgroup's first
+    const int nsb = a.k >> 8;
+    const uint32_t moff = (uint32_t)(slice * 4 + (lane & 3) < nsb ? slice * 4 + (lane & 3) : nsb - 1) * 16;
+    const int mrl0 = g_idx * rows_per_group + (lane >> 2);
     auto request = [&](int step, int b) {
-        int rl = rl0 + 4 * (step < a.steps ? step : 0);
+        const int s = step < a.steps ? step : 0;
+        int rl = rl0 + 4 * s;
         rl = rl < rl_last ? rl : rl_last;
         const RowOff ro = {(uint32_t)rl * cp, (uint32_t)rl * mp, (uint32_t)rl * qp};
-        T::load(bases, ro, lo, buf[b]);
+        if constexpr (ROUNDS) {
+            if (b == 0) { // rows past the group's steps: read, not used
+                int rlm = mrl0 + 4 * s;
+                rlm = rlm < rl_last ? rlm : rl_last;
+                hm = ld16(bases.meta, (uint32_t)rlm * mp + moff);
+            }
+            T::load_codes(bases, ro, lo, buf[b]);
+        } else {
+            T::load(bases, ro, lo, buf[b]);
+        }
     };
     constexpr int NB0 = NB < 2 ? NB : 2; // steps requested before x is split: enough to start the stream, few enough that
                                          // the wave is not held up issuing them when its x arrives
@@ -852,7 +884,12 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     // 4. fold the steps through the ring
     const bool writer = (blk & 3) == 3;
     const int red_step = 4 * red_stride;
+    const int hidx = j * 4 + (blk >> 2);
     auto fold = [&](int b, int step) {
+        if constexpr (ROUNDS) {
+            if (b == 0) wmeta[lane] = hm; // the wave's own patch: LDS serves a wave's stores and loads in order
+            T::set_header(buf[b], wmeta[b * 16 + hidx]);
+        }
         float tot = sum_within_row(T::dot(buf[b], xo, c));
         if (writer) red_lane[step * red_step] = tot;
     };
@@ -921,7 +958,8 @@ void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, si
     static const bool shared_x = getenv("AXQ_GEMV_SHARED_X") && getenv("AXQ_GEMV_SHARED_X")[0] == '1'; // development knob: the kernel that splits x once per workgroup
     if (!PRE && !shared_x) {
         // x arrives raw: every wave stages its own slice
-        const size_t lds_w = (size_t)(block / 64) * (4 * 1024 + 32 * 16) + 64 + (size_t)a.G * a.steps * 4 * a.S * 4 * sizeof(float);
+        const size_t lds_w = (size_t)(block / 64) * (4 * 1024 + 32 * 16 + (T::ROUND_META ? 1024 : 0)) + 64 +
+                             (size_t)a.G * a.steps * 4 * a.S * 4 * sizeof(float);
         static bool big_lds_allowed_w = false;
         if (lds_w > 64 * 1024 && !big_lds_allowed_w) {
             (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1006,6 +1044,7 @@ bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t 
     int nb = block > 512 ? T::BIG_NB : 8;
     if (nb > ctx->gemv_max_nb) nb = ctx->gemv_max_nb;
     if (nb > steps) nb = steps;
+    if (T::ROUND_META && !xq && nb > 4) nb = 4; // a round of the per-wave staging kernel is at most four steps
     const unsigned grid = (unsigned)((rowsteps + steps * a.G - 1) / (steps * a.G));
     size_t lds = (size_t)a.G * steps * 4 * a.S * 4 * sizeof(float);
     lds += axq_split_bytes(a.k) + 16 + 64;
