@@ -9,7 +9,9 @@ from .quant import QuantType, f32_to_bf16_bits
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16, published
 
 
-def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(QuantType.Q4_K, QuantType.Q5_1), iters=20):
+def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(QuantType.Q4_K, QuantType.Q5_1), iters=20,
+          f32_rows=True):
+    """Times axq_gemm_bf16 (and, with f32_rows, the same product from f32 rows through axq_gemv_f32) per shape and type."""
     lib = ctx.lib
     rng = np.random.default_rng(0)
     out = []
@@ -39,6 +41,9 @@ def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(
                 out.append(r)
                 log(f"  prefill {r['type']} M={m} N={n}: {t * 1e3:.1f} us, {r['tflops']:.1f} TFLOP/s")
                 ctx.free(xd)
+                if not f32_rows:
+                    ctx.free(yd)
+                    continue
                 # the same product from f32 rows (axq_gemv_f32 sends 40 rows or more through the GEMM as two f16 rows each)
                 xf = ctx.to_device(rng.standard_normal((m, k)).astype(np.float32))
                 for _ in range(3):
