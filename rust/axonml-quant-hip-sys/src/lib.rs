@@ -2,7 +2,7 @@
 //!
 //! NOT COMPILED in this repository's build or tests: the image this library is built in has no Rust toolchain.
 //! The declarations restate `include/axq.h` by hand; `tests/test_abi.py` checks that the shared library exports every
-//! symbol the header declares.  The safe layer that `axonml-quant` would put on top is sketched in INTEGRATION.md.
+//! symbol the header declares.  A safe layer (context, device weight, quantized_matmul) belongs in `axonml-quant` itself.
 #![allow(non_camel_case_types)]
 use std::os::raw::{c_char, c_int, c_void};
 
