@@ -104,12 +104,17 @@ struct DQ4K {
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 8; // w = d*sc*(q - 8) + (8*d*sc - dmin*m)
     static constexpr int BIG_NB = 4; // row steps a lane can hold within 128 registers
-    static constexpr bool ROUND_META = true; // the kernels that stage x per wave fetch the headers once per round of steps
+    // The kernel that stages x per wave fetches the scale records once per round of up to four row steps (see
+    // gemv_q4k_kernel): META_SLICE_BYTES of the meta plane per row and 1024-wide K slice, parked in LDS; set_meta picks
+    // the lane's own out of its row's.
+    static constexpr bool ROUND_META = true;
+    static constexpr int META_SLICE_BYTES = 64; // four superblock headers
+    __host__ __device__ static int meta_row_bytes(int k) { return (k >> 8) * 16; }
     __device__ static void load_codes(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
         r.q0 = ld16(b.codes, ro.c + o.c[0]);
         r.q1 = ld16(b.codes, ro.c + o.c[1]);
     }
-    __device__ static void set_header(Raw &r, const uint4 &h) { r.h = h; }
+    __device__ static void set_meta(Raw &r, const uint8_t *row, int blk, int) { r.h = *reinterpret_cast<const uint4 *>(row + (blk >> 2) * 16); }
     __device__ static int group_k(int c, int g) { return c * 64 + g * 32; }
     __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
         // the code plane interleaves, per 64-pair slice, the first 16 bytes of every pair, then the second 16
@@ -177,9 +182,20 @@ struct DQ4x {
     static constexpr bool PERM_A = true; // dword w of a block: low nibbles = elements 8w+{0,2,4,6}, high = 8w+{1,3,5,7}
     static constexpr int CENTRE = 8;
     static constexpr int BIG_NB = 4;
-    static constexpr bool ROUND_META = false;
-    __device__ static void load_codes(const Bases &, const RowOff &, const LaneOff &, Raw &) {}
-    __device__ static void set_header(Raw &, const uint4 &) {}
+    static constexpr bool ROUND_META = true;
+    static constexpr int META_SLICE_BYTES = WITH_MIN ? 128 : 64; // 32 blocks' scales (and minimums)
+    __host__ __device__ static int meta_row_bytes(int k) { return (k >> 5) * (WITH_MIN ? 4 : 2); }
+    __device__ static void load_codes(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+        r.q[0] = ld16(b.codes, ro.c + o.c[0]);
+        r.q[1] = ld16(b.codes, ro.c + o.c[1]);
+    }
+    __device__ static void set_meta(Raw &r, const uint8_t *row, int, int c) {
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const int b = g * 16 + (c & 15); // the block inside the slice
+            r.m[g] = WITH_MIN ? *reinterpret_cast<const uint32_t *>(row + b * 4) : *reinterpret_cast<const uint16_t *>(row + b * 2);
+        }
+    }
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
     __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
@@ -226,9 +242,23 @@ struct DQ5x {
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 16;
     static constexpr int BIG_NB = 4;
-    static constexpr bool ROUND_META = false;
-    __device__ static void load_codes(const Bases &, const RowOff &, const LaneOff &, Raw &) {}
-    __device__ static void set_header(Raw &, const uint4 &) {}
+    static constexpr bool ROUND_META = true;
+    static constexpr int META_SLICE_BYTES = WITH_MIN ? 128 : 64;
+    __host__ __device__ static int meta_row_bytes(int k) { return (k >> 5) * (WITH_MIN ? 4 : 2); }
+    __device__ static void load_codes(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            r.q[g] = ld16(b.codes, ro.c + o.c[g]);
+            r.qh[g] = ld4(b.qh, ro.h + o.h[g]);
+        }
+    }
+    __device__ static void set_meta(Raw &r, const uint8_t *row, int, int c) {
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const int b = g * 16 + (c & 15);
+            r.m[g] = WITH_MIN ? *reinterpret_cast<const uint32_t *>(row + b * 4) : *reinterpret_cast<const uint16_t *>(row + b * 2);
+        }
+    }
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
     __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
@@ -279,9 +309,20 @@ struct DQ80 {
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 0;
     static constexpr int BIG_NB = 3;
-    static constexpr bool ROUND_META = false;
-    __device__ static void load_codes(const Bases &, const RowOff &, const LaneOff &, Raw &) {}
-    __device__ static void set_header(Raw &, const uint4 &) {}
+    static constexpr bool ROUND_META = true;
+    static constexpr int META_SLICE_BYTES = 64;
+    __host__ __device__ static int meta_row_bytes(int k) { return (k >> 5) * 2; }
+    __device__ static void load_codes(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            r.q[2 * g] = ld16(b.codes, ro.c + o.c[g]);
+            r.q[2 * g + 1] = ld16(b.codes, ro.c + o.c[g] + 16);
+        }
+    }
+    __device__ static void set_meta(Raw &r, const uint8_t *row, int, int c) {
+#pragma unroll
+        for (int g = 0; g < 2; g++) r.m[g] = *reinterpret_cast<const uint16_t *>(row + (g * 16 + (c & 15)) * 2);
+    }
     // 16-byte vector v (0..3) of chunk c: vector index along the row; block = vector / 2
     __device__ static int vec_index(int c, int v) { return ((c >> 4) << 6) + (v >> 1) * 32 + (c & 15) * 2 + (v & 1); }
     __device__ static int group_k(int c, int g) { return vec_index(c, 2 * g) * 16; }
@@ -803,8 +844,9 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     typename T::Raw buf[NB];
     // T::ROUND_META (see gemv_q4k_kernel): one header load per round of NB <= 4 steps, parked in an LDS patch of the wave
     constexpr bool ROUNDS = T::ROUND_META && NB <= 4;
-    uint4 hm = {0, 0, 0, 0};
-    uint4 *wmeta = reinterpret_cast<uint4 *>(red + a.G * rows_per_group * red_stride) + wave * 64;
+    constexpr int MSB = T::META_SLICE_BYTES, NM = MSB / 64, CPR = MSB / 16; // loads per round, 16-byte chunks per row
+    uint4 hm[NM];
+    uint4 *wmeta = reinterpret_cast<uint4 *>(red + a.G * rows_per_group * red_stride) + wave * 64 * NM;
     LaneOff lo;
     T::lane_offsets(a, c, lo);
     const int wg_row0 = blockIdx.x * a.G * rows_per_group;
@@ -812,9 +854,19 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
                          a.qh + (size_t)wg_row0 * a.qh_pitch};
     const uint32_t cp = (uint32_t)a.codes_pitch, mp = (uint32_t)a.meta_pitch, qp = (uint32_t)a.qh_pitch;
     const int rl0 = g_idx * rows_per_group + j, rl_last = last - wg_row0; // rows relative to the workgroup's first
-    const int nsb = a.k >> 8;
-    const uint32_t moff = (uint32_t)(slice * 4 + (lane & 3) < nsb ? slice * 4 + (lane & 3) : nsb - 1) * 16;
-    const int mrl0 = g_idx * rows_per_group + (lane >> 2);
+    // header loads of a round: 64 * NM lanes = (row of the round's 16, 16-byte chunk of the slice's MSB bytes); chunks past the
+    // row's end (a last slice that is not whole) are moved back inside it: they serve lanes whose x is zero
+    uint32_t moff[NM];
+    int mrl0[NM];
+    {
+        const int row_bytes = T::meta_row_bytes(a.k);
+#pragma unroll
+        for (int i = 0; i < NM; i++) {
+            const int flat = i * 64 + lane, off = slice * MSB + (flat % CPR) * 16;
+            moff[i] = (uint32_t)(off + 16 <= row_bytes ? off : row_bytes - 16);
+            mrl0[i] = g_idx * rows_per_group + flat / CPR;
+        }
+    }
     auto request = [&](int step, int b) {
         const int s = step < a.steps ? step : 0;
         int rl = rl0 + 4 * s;
@@ -822,9 +874,12 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
         const RowOff ro = {(uint32_t)rl * cp, (uint32_t)rl * mp, (uint32_t)rl * qp};
         if constexpr (ROUNDS) {
             if (b == 0) { // rows past the group's steps: read, not used
-                int rlm = mrl0 + 4 * s;
-                rlm = rlm < rl_last ? rlm : rl_last;
-                hm = ld16(bases.meta, (uint32_t)rlm * mp + moff);
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    int rlm = mrl0[i] + 4 * s;
+                    rlm = rlm < rl_last ? rlm : rl_last;
+                    hm[i] = ld16(bases.meta, (uint32_t)rlm * mp + moff[i]);
+                }
             }
             T::load_codes(bases, ro, lo, buf[b]);
         } else {
@@ -884,11 +939,13 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     // 4. fold the steps through the ring
     const bool writer = (blk & 3) == 3;
     const int red_step = 4 * red_stride;
-    const int hidx = j * 4 + (blk >> 2);
     auto fold = [&](int b, int step) {
         if constexpr (ROUNDS) {
-            if (b == 0) wmeta[lane] = hm; // the wave's own patch: LDS serves a wave's stores and loads in order
-            T::set_header(buf[b], wmeta[b * 16 + hidx]);
+            if (b == 0) { // the wave's own patch: LDS serves a wave's stores and loads in order
+#pragma unroll
+                for (int i = 0; i < NM; i++) wmeta[i * 64 + lane] = hm[i];
+            }
+            T::set_meta(buf[b], reinterpret_cast<const uint8_t *>(wmeta) + (b * 4 + j) * MSB, blk, c);
         }
         float tot = sum_within_row(T::dot(buf[b], xo, c));
         if (writer) red_lane[step * red_step] = tot;
@@ -956,9 +1013,11 @@ template <class T, int NB, bool PRE>
 void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
     static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
     static const bool shared_x = getenv("AXQ_GEMV_SHARED_X") && getenv("AXQ_GEMV_SHARED_X")[0] == '1'; // development knob: the kernel that splits x once per workgroup
-    if (!PRE && !shared_x) {
+    // the per-round scale loads are 16 bytes wide: the rows of the meta plane have to be whole 16-byte pieces
+    const bool rounds_ok = !T::ROUND_META || NB > 4 || (T::meta_row_bytes(a.k) % 16 == 0 && a.meta_pitch % 16 == 0 && T::meta_row_bytes(a.k) >= 16);
+    if (!PRE && !shared_x && rounds_ok) {
         // x arrives raw: every wave stages its own slice
-        const size_t lds_w = (size_t)(block / 64) * (4 * 1024 + 32 * 16 + (T::ROUND_META ? 1024 : 0)) + 64 +
+        const size_t lds_w = (size_t)(block / 64) * (4 * 1024 + 32 * 16 + (T::ROUND_META ? 16 * T::META_SLICE_BYTES : 0)) + 64 +
                              (size_t)a.G * a.steps * 4 * a.S * 4 * sizeof(float);
         static bool big_lds_allowed_w = false;
         if (lds_w > 64 * 1024 && !big_lds_allowed_w) {
