@@ -276,12 +276,9 @@ size_t flash_lds_bytes() {
 template <int D, int REP>
 int launch_flash(axq_ctx *ctx, const FlashArgs &a) {
     const size_t lds = flash_lds_bytes<D, REP>();
-    static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
-    if (lds > 48 * 1024 && !big_lds_allowed) {
-        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_flash_kernel<D, REP>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds), AXQ_ERR_DRIVER);
-        big_lds_allowed = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    int rc;
+    if (lds > 48 * 1024 && (rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(&attn_flash_kernel<D, REP>), lds_allowed, lds))) return rc;
     const int tq = VQ / REP;
     attn_flash_kernel<D, REP><<<dim3(a.n_kv, (a.T + tq - 1) / tq), 256, lds, ctx->stream>>>(a);
     AXQ_LAUNCH_CHECK(ctx, "attn_flash_kernel");

@@ -970,12 +970,9 @@ template <int D, bool APPEND>
 void launch_attn_rows_t(axq_model *m, int l, const float *qkv, int nb, int pos0, const int32_t *pos_arr, size_t cache_off, size_t lds,
                         float *att, hipStream_t st, PackOut pk) {
     const axq_model_config &c = m->cfg;
-    static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
-    if (lds > 48 * 1024 && !big_lds_allowed) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prompt_kernel<D, APPEND>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  128 * 1024);
-        big_lds_allowed = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (lds > 48 * 1024) (void)axq_allow_lds(m->ctx, reinterpret_cast<const void *>(&attn_prompt_kernel<D, APPEND>), lds_allowed, 128 * 1024); // a
+    // refusal is the context's error now, and the launch below fails with it
     const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * D + cache_off;
     attn_prompt_kernel<D, APPEND><<<dim3(c.num_attention_heads, nb), 1024, lds, st>>>(
         qkv, m->qkv_rows, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, pos0, pos_arr, m->seq_stride, c.num_attention_heads,

@@ -270,6 +270,15 @@ __device__ inline void split8_f16(const float *w, float scale, uint4 &hi, uint4 
     lo = make_uint4(l[0], l[1], l[2], l[3]);
 }
 
+// A workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global load in flight, which
+// would pull the prefetched operands of later steps in front of every barrier.
+__device__ inline void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0); // nothing moves across: what follows may count on the waits in front of the barrier
+}
+
 // WM = 1 or 2: the workgroup computes (128 * WM) x 128 outputs with 4 * WM waves of two kinds.
 //   - 2 * WM "multiplier" waves each own a 128 x 64 block (4 x 2 MFMA tiles, 128 accumulator registers) and
 //     do nothing but read the current LDS stage and issue MFMAs;
@@ -355,7 +364,8 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
                     *reinterpret_cast<uint4 *>(Bl + row * LDK + k1[u]) = l1;
                 }
             }
-            __syncthreads(); // barrier ks: stage ks & 1 is complete, stage (ks + 1) & 1 has been read
+            lds_barrier(); // barrier ks: stage ks & 1 is complete, stage (ks + 1) & 1 has been read; the loads of step
+                           // ks + 1 stay in flight across it
         }
         return;
     }
@@ -472,14 +482,6 @@ __device__ inline void q4k_scale_min(const u32x4 &h, int p, uint32_t &scp, uint3
     }
 }
 
-// A workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global load in flight, which
-// would pull the prefetched operands of later steps in front of every barrier.
-__device__ inline void lds_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0); // nothing moves across: what follows may count on the waits in front of the barrier
-}
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
@@ -920,17 +922,15 @@ __global__ void __launch_bounds__(256) gemm_reduce_kernel(const float *ypart, co
 
 template <class T>
 int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
-    static bool attr_set = false;
+    static std::atomic<uint64_t> lds_allowed[2]; // per kernel: a bit per device
     const int wm = a.wm, bm = 128 * wm;
     const unsigned tiles = (unsigned)(((a.n + BN - 1) / BN) * ((a.m + bm - 1) / bm));
     const dim3 grid(tiles, (unsigned)splits);
     const size_t lds = (size_t)2 * (bm + 2 * BN) * LDK * sizeof(_Float16); // two stages
-    if (!attr_set) {
-        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, 2>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * (256 + 2 * BN) * LDK * 2)), AXQ_ERR_DRIVER);
-        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, 1>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * (128 + 2 * BN) * LDK * 2)), AXQ_ERR_DRIVER);
-        attr_set = true;
+    {
+        int rc;
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_kernel<T, 2>), lds_allowed[1], 2 * (256 + 2 * BN) * LDK * 2))) return rc;
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_kernel<T, 1>), lds_allowed[0], 2 * (128 + 2 * BN) * LDK * 2))) return rc;
     }
     if (wm == 2) gemm_kernel<T, 2><<<grid, 512, lds, ctx->stream>>>(a);
     else gemm_kernel<T, 1><<<grid, 256, lds, ctx->stream>>>(a);
@@ -1137,17 +1137,15 @@ XSums plan_sums(axq_ctx *ctx, const axq_weight *w, const GemmPlan &p) {
 }
 
 int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits) {
-    static bool attr_set = false;
+    static std::atomic<uint64_t> lds_allowed[2]; // per kernel: a bit per device
     const int bm = 128 * a.wm;
     const unsigned tiles = (unsigned)(((a.n + QBN - 1) / QBN) * ((a.m + bm - 1) / bm));
     const dim3 grid(tiles, (unsigned)splits);
     const size_t lds = (size_t)(3 * bm * 64 + 2 * QBN * 64) * sizeof(_Float16); // three x stages, two weight stages
-    if (!attr_set) {
-        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_kernel<256>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)((3 * 256 * 64 + 2 * QBN * 64) * 2)), AXQ_ERR_DRIVER);
-        AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_kernel<128>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)((3 * 128 * 64 + 2 * QBN * 64) * 2)), AXQ_ERR_DRIVER);
-        attr_set = true;
+    {
+        int rc;
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<256>), lds_allowed[1], (3 * 256 * 64 + 2 * QBN * 64) * 2))) return rc;
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<128>), lds_allowed[0], (3 * 128 * 64 + 2 * QBN * 64) * 2))) return rc;
     }
     if (a.wm == 2) gemm_q4k_kernel<256><<<grid, 512, lds, ctx->stream>>>(a);
     else gemm_q4k_kernel<128><<<grid, 256, lds, ctx->stream>>>(a);

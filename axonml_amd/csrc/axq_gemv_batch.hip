@@ -456,11 +456,9 @@ void launch_mb(axq_ctx *ctx, MbArgs a, uint8_t *sc, const float *x, int xmode, c
     static const unsigned smax = getenv("AXQ_BATCH_WAVES") ? (unsigned)atoi(getenv("AXQ_BATCH_WAVES")) : 8; // development knob (1..8)
     const unsigned S = (unsigned)a.chunks_per_split < smax ? (unsigned)a.chunks_per_split : smax;
     const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float) + (size_t)S * 32 * T::NP * 16;
-    static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
-    if (lds > 64 * 1024 && !big_lds_allowed) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        big_lds_allowed = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (lds > 64 * 1024) (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_mb_kernel<T>), lds_allowed, 160 * 1024); // a refusal is
+    // the context's error now, and the launch below fails with it
     gemv_mb_kernel<T><<<dim3(tiles, splits), 64 * S, lds, ctx->stream>>>(a);
     if (next_even_odd >= 0) {
         // y's operands for the next GEMV (k' = n_rows): the scratch layout of that call

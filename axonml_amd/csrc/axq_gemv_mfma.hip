@@ -1011,7 +1011,8 @@ __global__ void __launch_bounds__(256) prep_x_kernel(const float *x, int k, uint
 
 template <class T, int NB, bool PRE>
 void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
-    static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once per kernel
+    static std::atomic<uint64_t> lds_allowed{0}, lds_allowed_w{0}; // dynamic LDS beyond 64 KB is asked for per kernel and device; a
+    // refusal is the context's error, and the launch that follows fails with it
     static const bool shared_x = getenv("AXQ_GEMV_SHARED_X") && getenv("AXQ_GEMV_SHARED_X")[0] == '1'; // development knob: the kernel that splits x once per workgroup
     // the per-round scale loads are 16 bytes wide: the rows of the meta plane have to be whole 16-byte pieces
     const bool rounds_ok = !T::ROUND_META || NB > 4 || (T::meta_row_bytes(a.k) % 16 == 0 && a.meta_pitch % 16 == 0 && T::meta_row_bytes(a.k) >= 16);
@@ -1019,22 +1020,14 @@ void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, si
         // x arrives raw: every wave stages its own slice
         const size_t lds_w = (size_t)(block / 64) * (4 * 1024 + 32 * 16 + (T::ROUND_META ? 16 * T::META_SLICE_BYTES : 0)) + 64 +
                              (size_t)a.G * a.steps * 4 * a.S * 4 * sizeof(float);
-        static bool big_lds_allowed_w = false;
-        if (lds_w > 64 * 1024 && !big_lds_allowed_w) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      160 * 1024);
-            big_lds_allowed_w = true;
-        }
+        if (lds_w > 64 * 1024 && lds_w <= 160 * 1024)
+            (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), lds_allowed_w, 160 * 1024);
         if (lds_w <= 160 * 1024) {
             gemv_dpw_kernel<T, NB><<<grid, block, lds_w, ctx->stream>>>(a);
             return;
         }
     }
-    if (lds > 64 * 1024 && !big_lds_allowed) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        big_lds_allowed = true;
-    }
+    if (lds > 64 * 1024) (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE>), lds_allowed, 160 * 1024);
     gemv_dp_kernel<T, NB, PRE><<<grid, block, lds, ctx->stream>>>(a);
 }
 
@@ -1058,7 +1051,7 @@ bool launch_q4k_rounds(axq_ctx *, const DpArgs &, unsigned, unsigned, size_t) { 
 template <>
 bool launch_q4k_rounds<DQ4K>(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
     static const bool off = getenv("AXQ_GEMV_Q4K_ROUNDS") && getenv("AXQ_GEMV_Q4K_ROUNDS")[0] == '0'; // development knob
-    static bool big_lds_allowed = false;
+    static std::atomic<uint64_t> lds_allowed[2];
     if (off) return false;
     // measured inside the 7B-shape decode: a gain from three steps per group on (qkv 6.6 -> 6.0 us, gate/up 15.4 -> 14.8 us);
     // with two steps (o projection) or one group of 14 waves over a long K (down projection, two split tasks per thread)
@@ -1066,10 +1059,9 @@ bool launch_q4k_rounds<DQ4K>(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsig
     if (a.G < 2 || a.steps < 3) return false;
     lds += (size_t)(block / 64) * 1024;
     if (lds > 160 * 1024) return false;
-    if (lds > 64 * 1024 && !big_lds_allowed) {
-        for (const void *f : {reinterpret_cast<const void *>(&gemv_q4k_kernel<3>), reinterpret_cast<const void *>(&gemv_q4k_kernel<4>)})
-            (void)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        big_lds_allowed = true;
+    if (lds > 64 * 1024) {
+        (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_q4k_kernel<3>), lds_allowed[0], 160 * 1024);
+        (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_q4k_kernel<4>), lds_allowed[1], 160 * 1024);
     }
     if (a.steps == 3) gemv_q4k_kernel<3><<<grid, block, lds, ctx->stream>>>(a);
     else gemv_q4k_kernel<4><<<grid, block, lds, ctx->stream>>>(a);

@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "../../include/axq.h"
 
 // ---------------------------------------------------------------------------
@@ -90,6 +92,18 @@ int axq_fail(axq_ctx *ctx, int code, const char *fmt, ...);
         if (e_ != hipSuccess)                                                                 \
             return axq_fail((ctx), AXQ_ERR_KERNEL_LAUNCH_FAILED, "%s: %s", (what), hipGetErrorString(e_)); \
     } while (0)
+
+// Dynamic LDS beyond the default limit has to be asked for once per kernel AND device.  `done` holds a bit per device (a
+// static of the call site, so one per kernel instantiation); asking twice is harmless, hence so is the race of two first
+// callers.  A refusal is recorded as the context's error and returned; the launch that follows would fail too.
+static inline int axq_allow_lds(axq_ctx *ctx, const void *kernel, std::atomic<uint64_t> &done, size_t bytes) {
+    const uint64_t bit = 1ull << (ctx->device & 63);
+    if (done.load(std::memory_order_acquire) & bit) return AXQ_OK;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipFuncSetAttribute(max dynamic LDS %zu): %s", bytes, hipGetErrorString(e));
+    done.fetch_or(bit, std::memory_order_release);
+    return AXQ_OK;
+}
 
 // Cross-TU entry points -----------------------------------------------------
 // codec.hip

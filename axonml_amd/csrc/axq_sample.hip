@@ -460,11 +460,10 @@ int axq_dev_sample_rows(axq_ctx *ctx, int rows, const float *logits, size_t logi
     a.u = u; a.counter_dev = counter_dev; a.seed = seed;
     a.out = out; a.filtered_out = filtered_out;
     a.logits_stride = logits_stride; a.hist_stride = hist_stride; a.work_stride = 2 * padded_words(vocab); a.seed_stride = seed_stride;
-    static bool big_lds_allowed = false; // dynamic LDS beyond 64 KB has to be asked for once
-    if (!big_lds_allowed) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&sample_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)(padded_words(LDS_VOCAB) * 4));
-        big_lds_allowed = true;
+    static std::atomic<uint64_t> lds_allowed{0};
+    {
+        int rc;
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(&sample_kernel<true>), lds_allowed, padded_words(LDS_VOCAB) * 4))) return rc;
     }
     if (vocab <= LDS_VOCAB) sample_kernel<true><<<rows, ST, padded_words(vocab) * 4, ctx->stream>>>(a);
     else sample_kernel<false><<<rows, ST, 0, ctx->stream>>>(a);
