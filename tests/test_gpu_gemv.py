@@ -65,6 +65,23 @@ def test_config_q4_k_headline(ctx, n, k):
     _check(ctx, o.Q4_K, n, k, 1, seed=3, outlier_p=0.01)
 
 
+@pytest.mark.parametrize("qtype,n,k", [
+    (o.Q4_K, 7001, 2304),   # per-round headers, K slices 1024 + 1024 + 256, rows that do not fill the last workgroup
+    (o.Q4_K, 9000, 1280),   # four row groups of three steps: the three-deep ring
+    (o.Q4_K, 40000, 1024),  # one slice, eight row groups, two rounds of steps
+    (o.Q4_K, 3000, 6144),   # six slices, one row group: per-wave staging, headers per round
+    (o.Q4_0, 6000, 320),    # 20 bytes of scales per row: no 16-byte scale loads, the kernel without rounds
+    (o.Q4_0, 6000, 1280),   # scales per round, last slice a quarter full
+    (o.Q4_1, 5000, 2304),   # two scale loads per round
+    (o.Q5_0, 5000, 1536),
+    (o.Q5_1, 5000, 1088),   # 136 bytes of scale records per row: the kernel without rounds
+    (o.Q8_0, 5000, 2560),
+])
+def test_gemv_scale_records_per_round(ctx, qtype, n, k):
+    """Shapes that take the one-vector kernels through several rounds of row steps, partial K slices and ragged row counts."""
+    _check(ctx, qtype, n, k, 1, seed=n + k)
+
+
 @pytest.mark.parametrize("qtype", ALL)
 def test_one_hot_activation_selects_dequantised_column(ctx, qtype):
     # exactness of the in-register unpack: y = W[:, col] up to the scale factorisation's rounding
