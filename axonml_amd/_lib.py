@@ -94,6 +94,7 @@ SIGNATURES = {
     "axq_model_create": (_i, [_vp, C.POINTER(ModelConfig), C.POINTER(_vp)]),
     "axq_model_free": (None, [_vp]),
     "axq_model_set_embedding_f16": (_i, [_vp, _vp, _i]),
+    "axq_model_set_embedding_f32": (_i, [_vp, _vp, _i]),
     "axq_model_set_norm": (_i, [_vp, _i, _i, _vp, _i]),
     "axq_model_set_linear": (_i, [_vp, _i, _i, _vp]),
     "axq_model_random_init": (_i, [_vp, _i, C.c_float, C.c_uint64]),

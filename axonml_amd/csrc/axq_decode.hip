@@ -29,7 +29,8 @@ struct axq_model {
     axq_model_config cfg;
     int qkv_rows, q_dim, kv_dim;
     // weights
-    uint16_t *emb;                  // f16 [vocab, hidden]
+    uint16_t *emb;                  // f16 [vocab, hidden], or
+    float *emb32 = nullptr;         // f32 [vocab, hidden] as the reference keeps it (one of the two is set)
     float *norm_attn, *norm_ffn;    // [layers, hidden]
     float *norm_final;              // [hidden]
     std::vector<axq_weight *> w_qkv, w_o, w_gu, w_down;
@@ -84,10 +85,17 @@ __device__ inline float block_sum(float v, float *scratch) {
 }
 
 // h = embedding[tok] widened to f32 (Embedding::lookup, nn/src/layers/embedding.rs:103-146); grid.y = tokens.
-__global__ void __launch_bounds__(256) embed_kernel(const uint16_t *emb, const int32_t *tok, float *h, int hidden) {
+__global__ void __launch_bounds__(256) embed_kernel(const uint16_t *emb, const float *emb32, const int32_t *tok, float *h, int hidden) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (hidden >> 3)) return;
     h += (size_t)blockIdx.y * hidden;
+    if (emb32) { // an f32 table: the row as it is
+        const float4 *src = reinterpret_cast<const float4 *>(emb32 + (size_t)tok[blockIdx.y] * hidden + (size_t)t * 8);
+        float4 *dst = reinterpret_cast<float4 *>(h + (size_t)t * 8);
+        dst[0] = src[0];
+        dst[1] = src[1];
+        return;
+    }
     const uint4 raw = *reinterpret_cast<const uint4 *>(emb + (size_t)tok[blockIdx.y] * hidden + (size_t)t * 8);
     const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
     float v[8];
@@ -823,7 +831,7 @@ int enqueue_step(axq_model *m, bool short_ctx) {
     hipStream_t st = ctx->stream;
     const int H = c.hidden_size;
     int rc;
-    embed_kernel<<<(H / 8 + 255) / 256, 256, 0, st>>>(m->emb, m->tok, m->h, H);
+    embed_kernel<<<(H / 8 + 255) / 256, 256, 0, st>>>(m->emb, m->emb32, m->tok, m->h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
         if ((rc = linear(m, m->w_qkv[l], m->h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, AXQ_Y_PLAIN, m->xn, nullptr, m->qkv)))
             return rc;
@@ -845,7 +853,7 @@ int enqueue_step(axq_model *m, bool short_ctx) {
 }
 
 int check_ready(axq_model *m) {
-    if (!m->emb || !m->head_set) return axq_fail(m->ctx, AXQ_ERR_INVALID_DATA, "Invalid quantized data: embedding or lm_head not set");
+    if ((!m->emb && !m->emb32) || !m->head_set) return axq_fail(m->ctx, AXQ_ERR_INVALID_DATA, "Invalid quantized data: embedding or lm_head not set");
     for (int l = 0; l < m->cfg.num_hidden_layers; l++)
         if (m->set_mask[l] != (1u << AXQ_LIN_COUNT) - 1)
             return axq_fail(m->ctx, AXQ_ERR_INVALID_DATA, "Invalid quantized data: layer %d has unset linears (mask %#x)", l,
@@ -1048,7 +1056,7 @@ int enqueue_rows(axq_model *m, const Rows &r) {
         int32_t *hist = m->hist + (size_t)r.seq * c.max_position_embeddings;
         for (int t0 = 0; t0 < nb; t0 += 1024) record_tokens_kernel<<<1, nb - t0 < 1024 ? nb - t0 : 1024, 0, st>>>(hist, r.pos0 + t0, r.toks + t0);
     }
-    embed_kernel<<<dim3((H / 8 + 255) / 256, nb), 256, 0, st>>>(m->emb, r.toks, m->pb_h, H);
+    embed_kernel<<<dim3((H / 8 + 255) / 256, nb), 256, 0, st>>>(m->emb, m->emb32, r.toks, m->pb_h, H);
     for (int l = 0; l < c.num_hidden_layers; l++) {
         const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * d + seq_off;
         if ((rc = lin(m->w_qkv[l], m->pb_h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv, nullptr, nullptr))) return rc;
@@ -1195,6 +1203,15 @@ int run_batch_step(axq_model *m, int max_pos_now) {
 template <class T>
 hipError_t dev_alloc(T **p, size_t count) { return hipMalloc((void **)p, (count ? count : 1) * sizeof(T)); }
 
+// The captured steps hold device addresses: whoever replaces a buffer they read drops them; the next step captures anew.
+void invalidate_graphs(axq_model *m) {
+    if (m->graph_ok) (void)hipGraphExecDestroy(m->graph);
+    if (m->graph_f_ok) (void)hipGraphExecDestroy(m->graph_f);
+    if (m->graph_b_ok) (void)hipGraphExecDestroy(m->graph_b);
+    if (m->graph_bf_ok) (void)hipGraphExecDestroy(m->graph_bf);
+    m->graph_ok = m->graph_f_ok = m->graph_b_ok = m->graph_bf_ok = false;
+}
+
 } // namespace
 
 extern "C" {
@@ -1322,7 +1339,7 @@ void axq_model_free(axq_model *m) {
     for (auto *w : m->w_gu) axq_weight_free(ctx, w);
     for (auto *w : m->w_down) axq_weight_free(ctx, w);
     axq_weight_free(ctx, m->w_head);
-    void *bufs[] = {m->emb, m->norm_attn, m->norm_ffn, m->norm_final, m->rope_cos, m->rope_sin, m->kcache, m->vcache, m->h,
+    void *bufs[] = {m->emb, m->emb32, m->norm_attn, m->norm_ffn, m->norm_final, m->rope_cos, m->rope_sin, m->kcache, m->vcache, m->h,
                     m->xn, m->qkv, m->att, m->att_part, m->gu, m->act, m->logits, m->pos, m->tok,
                     m->next, m->gen, m->prompt, m->out, m->hist, m->sample_scratch, m->pb_h, m->pb_xn, m->pb_qkv, m->pb_att,
                     m->pb_gu, m->pb_act};
@@ -1335,8 +1352,23 @@ int axq_model_set_embedding_f16(axq_model *m, const uint16_t *table, int mem) {
     if (!m || !table) return AXQ_ERR_INVALID_ARGUMENT;
     axq_ctx *ctx = m->ctx;
     size_t n = (size_t)m->cfg.vocab_size * m->cfg.hidden_size;
-    if (!m->emb) AXQ_HIP(ctx, dev_alloc(&m->emb, n), AXQ_ERR_ALLOCATION_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    if (m->emb32) { (void)hipFree(m->emb32); m->emb32 = nullptr; invalidate_graphs(m); } // the graphs hold the table's address
+    if (!m->emb) { AXQ_HIP(ctx, dev_alloc(&m->emb, n), AXQ_ERR_ALLOCATION_FAILED); invalidate_graphs(m); }
     AXQ_HIP(ctx, hipMemcpyAsync(m->emb, table, n * 2, mem == AXQ_MEM_DEVICE ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
+                                ctx->stream), AXQ_ERR_COPY_FAILED);
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+
+int axq_model_set_embedding_f32(axq_model *m, const float *table, int mem) {
+    if (!m || !table) return AXQ_ERR_INVALID_ARGUMENT;
+    axq_ctx *ctx = m->ctx;
+    size_t n = (size_t)m->cfg.vocab_size * m->cfg.hidden_size;
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    if (m->emb) { (void)hipFree(m->emb); m->emb = nullptr; invalidate_graphs(m); }
+    if (!m->emb32) { AXQ_HIP(ctx, dev_alloc(&m->emb32, n), AXQ_ERR_ALLOCATION_FAILED); invalidate_graphs(m); }
+    AXQ_HIP(ctx, hipMemcpyAsync(m->emb32, table, n * 4, mem == AXQ_MEM_DEVICE ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
                                 ctx->stream), AXQ_ERR_COPY_FAILED);
     AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
     return AXQ_OK;
@@ -1424,7 +1456,11 @@ int axq_model_random_init(axq_model *m, int type, float std, uint64_t seed) {
     if (!rc) {
         size_t n = (size_t)c.vocab_size * c.hidden_size;
         rc = axq_fill_normal_f32(ctx, tmp, n, 0.0f, std, 0.0f, 0.0f, ++s);
-        if (!rc && !m->emb && dev_alloc(&m->emb, n) != hipSuccess) rc = axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "embedding");
+        if (!rc && m->emb32) { (void)hipFree(m->emb32); m->emb32 = nullptr; invalidate_graphs(m); }
+        if (!rc && !m->emb) {
+            if (dev_alloc(&m->emb, n) != hipSuccess) rc = axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "embedding");
+            invalidate_graphs(m);
+        }
         if (!rc) f32_to_f16_kernel<<<(unsigned)((n + 255) / 256), 256, 0, ctx->stream>>>(tmp, n, m->emb);
     }
     (void)hipStreamSynchronize(ctx->stream);

@@ -38,6 +38,14 @@ class QuantizedLlama:
                                 f"{self.cfg.vocab_size} * {self.cfg.hidden_size}")
         self.ctx.check(self.ctx.lib.axq_model_set_embedding_f16(self.handle, t.ctypes.data, MEM_HOST))
 
+    def set_embedding_f32(self, table):
+        """The embedding table in f32, as the reference keeps it (embedding.rs:103-146)."""
+        t = np.ascontiguousarray(table, dtype=np.float32)
+        if t.size != self.cfg.vocab_size * self.cfg.hidden_size:
+            raise ShapeMismatch(f"Shape mismatch: embedding table of {t.size} elements, expected vocab_size * hidden_size = "
+                                f"{self.cfg.vocab_size} * {self.cfg.hidden_size}")
+        self.ctx.check(self.ctx.lib.axq_model_set_embedding_f32(self.handle, t.ctypes.data, MEM_HOST))
+
     def set_norm(self, layer, which, w):
         w = np.ascontiguousarray(w, dtype=np.float32)
         if w.size != self.cfg.hidden_size:  # the library copies hidden_size floats from this pointer

@@ -344,7 +344,9 @@ def load_llama(path, ctx=None, max_position_embeddings=None, permuted_qk=True):
         cfg["vocab_size"] = int(r.metadata.get("llama.vocab_size", emb_info.shape[0]))
         model = QuantizedLlama(ctx, **cfg)
         emb = load_f32(r, "token_embd.weight", ctx)
-        model.set_embedding_f16(emb.astype(np.float16).view(np.uint16))
+        from .hf_loader import set_embedding
+
+        set_embedding(model, emb)
 
         def linear(layer, which, name, heads=None):
             qt = load_quantized_tensor(r, name, ctx)

@@ -162,6 +162,18 @@ _PROJ = {"q": "self_attn.q_proj", "k": "self_attn.k_proj", "v": "self_attn.v_pro
          "gate": "mlp.gate_proj", "up": "mlp.up_proj", "down": "mlp.down_proj"}
 
 
+def set_embedding(model, emb):
+    """The embedding table as the reference holds it, f32 (embedding.rs:103-146).  A table whose values all fit f16 exactly
+    (an F16 checkpoint) goes to the device as f16: the same rows come out, at half the memory."""
+    emb = np.ascontiguousarray(emb, dtype=np.float32)
+    with np.errstate(over="ignore"):
+        half = emb.astype(np.float16)
+    if np.array_equal(half.astype(np.float32), emb):
+        model.set_embedding_f16(half.view(np.uint16))
+    else:
+        model.set_embedding_f32(emb)
+
+
 def load_llama(path, quant_type=QuantType.Q4_K, ctx=None, max_position_embeddings=None):
     """Directory -> QuantizedLlama: every linear quantised to `quant_type` on the device as it is read."""
     from .decode import QuantizedLlama
@@ -179,7 +191,7 @@ def load_llama(path, quant_type=QuantType.Q4_K, ctx=None, max_position_embedding
 
     model = QuantizedLlama(ctx, **cfg)
     emb = get("model.embed_tokens.weight", "embed_tokens.weight")
-    model.set_embedding_f16(emb.astype(np.float16).view(np.uint16))
+    set_embedding(model, emb)
 
     def linear(layer, which, w):
         dw = DeviceWeight.quantize(w, quant_type, ctx)

@@ -201,6 +201,9 @@ AXQ_API int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_mode
 AXQ_API void axq_model_free(axq_model *m);
 /* f16 table [vocab, hidden] (Embedding::lookup, nn/src/layers/embedding.rs:103-146). */
 AXQ_API int axq_model_set_embedding_f16(axq_model *m, const uint16_t *table, int mem);
+/* The same table in f32, as the reference keeps it (embedding.rs:103-146: lookup copies f32 rows); replaces an f16 table
+ * and the other way round. */
+AXQ_API int axq_model_set_embedding_f32(axq_model *m, const float *table, int mem);
 /* layer -1 = final norm; which 0 = attention norm, 1 = ffn norm.  f32[hidden]. */
 AXQ_API int axq_model_set_norm(axq_model *m, int layer, int which, const float *w, int mem);
 /* layer -1 = lm_head.  The model copies the weight's blocks; the caller may free `w`. */

@@ -59,6 +59,7 @@ def lib():
         L.axo_model_create.restype, L.axo_model_create.argtypes = vp, [C.POINTER(ModelConfig)]
         L.axo_model_free.restype, L.axo_model_free.argtypes = None, [vp]
         L.axo_model_set_embedding_f16.restype, L.axo_model_set_embedding_f16.argtypes = i, [vp, vp]
+        L.axo_model_set_embedding_f32.restype, L.axo_model_set_embedding_f32.argtypes = i, [vp, vp]
         L.axo_model_set_norm.restype, L.axo_model_set_norm.argtypes = i, [vp, i, i, vp]
         L.axo_model_set_linear.restype, L.axo_model_set_linear.argtypes = i, [vp, i, i, i, vp]
         L.axo_model_forward.restype, L.axo_model_forward.argtypes = i, [vp, i, i, vp]
@@ -143,6 +144,10 @@ class DecodeModel:
     def set_embedding_f16(self, table_bits):
         t = np.ascontiguousarray(table_bits, dtype=np.uint16)
         lib().axo_model_set_embedding_f16(self.h, t.ctypes.data)
+
+    def set_embedding_f32(self, table):
+        t = np.ascontiguousarray(table, dtype=np.float32)
+        lib().axo_model_set_embedding_f32(self.h, t.ctypes.data)
 
     def set_norm(self, layer, which, w):
         w = np.ascontiguousarray(w, dtype=np.float32)

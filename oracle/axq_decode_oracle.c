@@ -61,7 +61,8 @@ typedef struct {
 
 typedef struct axo_model {
     axo_model_config cfg;
-    uint16_t *emb; /* f16 [vocab, hidden] */
+    uint16_t *emb; /* f16 [vocab, hidden], or */
+    float *emb32;  /* f32 [vocab, hidden] (embedding.rs:103-146 keeps f32): one of the two is set */
     float *final_norm;
     float *head; /* f32 [vocab, hidden] */
     axo_layer *layers;
@@ -112,7 +113,7 @@ AXO_API void axo_model_free(axo_model *m) {
         free(m->layers[l].norm[0]); free(m->layers[l].norm[1]);
         free(m->layers[l].kc); free(m->layers[l].vc);
     }
-    free(m->layers); free(m->emb); free(m->final_norm); free(m->head);
+    free(m->layers); free(m->emb); free(m->emb32); free(m->final_norm); free(m->head);
     free(m->h); free(m->xn); free(m->q); free(m->k); free(m->v); free(m->att); free(m->o);
     free(m->g); free(m->u); free(m->scores);
     free(m);
@@ -121,9 +122,23 @@ AXO_API void axo_model_free(axo_model *m) {
 AXO_API int axo_model_set_embedding_f16(axo_model *m, const uint16_t *table) {
     size_t n = (size_t)m->cfg.vocab_size * m->cfg.hidden_size;
     free(m->emb);
+    free(m->emb32);
+    m->emb32 = NULL;
     m->emb = (uint16_t *)malloc(n * 2);
     if (!m->emb) return -1;
     memcpy(m->emb, table, n * 2);
+    return 0;
+}
+
+/* Embedding::lookup on the f32 weight (nn/src/layers/embedding.rs:103-146): the row is copied as it is. */
+AXO_API int axo_model_set_embedding_f32(axo_model *m, const float *table) {
+    size_t n = (size_t)m->cfg.vocab_size * m->cfg.hidden_size;
+    free(m->emb);
+    free(m->emb32);
+    m->emb = NULL;
+    m->emb32 = (float *)malloc(n * 4);
+    if (!m->emb32) return -1;
+    memcpy(m->emb32, table, n * 4);
     return 0;
 }
 
@@ -193,7 +208,8 @@ AXO_API int axo_model_forward(axo_model *m, int token, int pos, float *logits) {
     size_t qd = (size_t)nh * d, kd = (size_t)nkv * d;
     int group = nh / nkv;
     if (token < 0 || token >= c->vocab_size || pos < 0 || pos >= c->max_seq_len) return -1;
-    for (size_t i = 0; i < H; i++) m->h[i] = axo_f16_to_f32(m->emb[(size_t)token * H + i]);
+    if (m->emb32) memcpy(m->h, m->emb32 + (size_t)token * H, H * sizeof(float));
+    else for (size_t i = 0; i < H; i++) m->h[i] = axo_f16_to_f32(m->emb[(size_t)token * H + i]);
     float scale = 1.0f / sqrtf((float)d);
     for (int l = 0; l < c->num_layers; l++) {
         axo_layer *L = &m->layers[l];

@@ -52,6 +52,7 @@ extern "C" {
     pub fn axq_model_create(ctx: *mut axq_ctx, cfg: *const axq_model_config, out: *mut *mut axq_model) -> c_int;
     pub fn axq_model_free(m: *mut axq_model);
     pub fn axq_model_set_embedding_f16(m: *mut axq_model, table: *const u16, mem: c_int) -> c_int;
+    pub fn axq_model_set_embedding_f32(m: *mut axq_model, table: *const f32, mem: c_int) -> c_int;
     pub fn axq_model_set_norm(m: *mut axq_model, layer: c_int, which: c_int, w: *const f32, mem: c_int) -> c_int;
     pub fn axq_model_set_linear(m: *mut axq_model, layer: c_int, which: c_int, w: *const axq_weight) -> c_int;
     pub fn axq_model_reset(m: *mut axq_model) -> c_int;

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 import oracle as o
+from axonml_amd import quant as q
 from tests.decode_common import load_gpu, load_oracle, random_weights, tiny_config
 from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err
 
@@ -115,6 +116,50 @@ def test_generate_matches_oracle_greedy_and_is_repeatable(ctx):
     again, _, _ = gpu.generate(prompt, 128)
     assert again.tolist() == want  # graph replays are deterministic and the reset clears the position
     gpu.close()
+
+
+def test_f32_embedding_table_as_the_reference_keeps_it(ctx):
+    """Embedding::lookup copies f32 rows (nn/src/layers/embedding.rs:103-146).  A table whose values do not fit f16 goes in
+    as f32 on both sides; it replaces the f16 table after the step graph has been captured, and the f16 one comes back."""
+    c = tiny_config(max_seq_len=64)
+    w = random_weights(c, 77)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    rng = np.random.default_rng(5)
+    prompt = rng.integers(0, c["vocab_size"], size=9)
+
+    def walk(n):
+        want = []
+        for pos, t in enumerate(prompt):
+            tok, _ = cpu.forward(int(t), pos)
+        for i in range(n):
+            want.append(tok)
+            tok, _ = cpu.forward(tok, len(prompt) + i)
+        return want
+
+    got, _, _ = gpu.generate(prompt, 12)  # captures the step graph over the f16 table
+    assert got.tolist() == walk(12)
+    table = (rng.standard_normal((c["vocab_size"], c["hidden_size"])) * 0.7).astype(np.float32)
+    assert not np.array_equal(table.astype(np.float16).astype(np.float32), table)
+    gpu.set_embedding_f32(table)
+    cpu.set_embedding_f32(table)
+    gpu.reset()
+    got32, _, _ = gpu.generate(prompt, 12)
+    want32 = walk(12)
+    assert got32.tolist() == want32 and want32 != got.tolist()
+    gpu.reset()
+    g_next, g_logits = gpu.forward_tokens(prompt)
+    for pos, t in enumerate(prompt):
+        c_next, c_logits = cpu.forward(int(t), pos)
+    assert g_next == c_next and max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL
+    gpu.set_embedding_f16(w["emb"])
+    cpu.set_embedding_f16(w["emb"])
+    gpu.reset()
+    back, _, _ = gpu.generate(prompt, 12)
+    assert back.tolist() == got.tolist()
+    with pytest.raises(q.ShapeMismatch):
+        gpu.set_embedding_f32(table[:-1])
+    gpu.close()
+    cpu.close()
 
 
 @pytest.mark.parametrize("over,qtype,n_first,n_prompt", [

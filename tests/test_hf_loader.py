@@ -117,7 +117,8 @@ def _tiny_checkpoint(tmp_path, c, seed, sharded, tied, prefix="model."):
         files[shard if sharded else 0][name] = (dtype, arr.shape, raw)
         seen[name] = back
 
-    put(f"{prefix}embed_tokens.weight", rng.standard_normal((c["vocab_size"], c["hidden_size"])) * 0.7, "F16", 0)
+    # tied checkpoints carry an F32 table whose values do not fit f16 (the loader must keep them), the others an F16 table
+    put(f"{prefix}embed_tokens.weight", rng.standard_normal((c["vocab_size"], c["hidden_size"])) * 0.7, "F32" if tied else "F16", 0)
     stems = {"q": "self_attn.q_proj", "k": "self_attn.k_proj", "v": "self_attn.v_proj", "o": "self_attn.o_proj",
              "gate": "mlp.gate_proj", "up": "mlp.up_proj", "down": "mlp.down_proj"}
     for i in range(c["num_layers"]):
@@ -161,7 +162,9 @@ def test_llama_quantised_on_load_decodes_like_the_oracle(ctx, tmp_path, qtype, s
                         num_layers=c["num_layers"], num_heads=c["num_heads"], num_kv_heads=c["num_kv_heads"], head_dim=c["head_dim"],
                         max_seq_len=c["max_seq_len"], rms_norm_eps=c["rms_norm_eps"], rope_theta=c["rope_theta"])
     emb = seen[f"{prefix}embed_tokens.weight"]
-    cpu.set_embedding_f16(emb.astype(np.float16).view(np.uint16))
+    cpu.set_embedding_f32(emb)  # the reference's table is f32 (embedding.rs:103-146)
+    if tied:
+        assert not np.array_equal(emb.astype(np.float16).astype(np.float32), emb)
     for i in range(c["num_layers"]):
         cpu.set_norm(i, 0, seen[f"{prefix}layers.{i}.input_layernorm.weight"])
         cpu.set_norm(i, 1, seen[f"{prefix}layers.{i}.post_attention_layernorm.weight"])
