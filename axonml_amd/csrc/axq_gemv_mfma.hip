@@ -105,7 +105,7 @@ struct DQ4K {
     static constexpr int CENTRE = 8; // w = d*sc*(q - 8) + (8*d*sc - dmin*m)
     static constexpr int BIG_NB = 4; // row steps a lane can hold within 128 registers
     // The kernel that stages x per wave fetches the scale records once per round of up to four row steps (see
-    // gemv_q4k_kernel): META_SLICE_BYTES of the meta plane per row and 1024-wide K slice, parked in LDS; set_meta picks
+    // gemv_dp_kernel's RND): META_SLICE_BYTES of the meta plane per row and 1024-wide K slice, parked in LDS; set_meta picks
     // the lane's own out of its row's.
     static constexpr bool ROUND_META = true;
     static constexpr int META_SLICE_BYTES = 64; // four superblock headers
@@ -430,8 +430,21 @@ __device__ inline void lds_only_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <class T, int NB, bool PRE>
+// ---------------------------------------------------------------------------
+// RND: the scale records fetched once per round of up to four row steps (Q4_K from a raw x takes this route).
+//
+// A compute unit keeps about 64 vector memory instructions in flight, whatever they fetch (a wave that finds them
+// taken waits at its next load and does nothing else), and the stream runs at (bytes in flight) / latency.  A Q4_K
+// header load has four lanes on each 16 bytes and so fetches 256 bytes where a code load fetches 1024: one in three
+// places in flight was spent on one ninth of the bytes.  With RND one load per round fetches the headers of all its
+// 16 rows (lane = row and superblock), the wave parks them in an LDS patch of its own, and every fold reads its
+// header from there: nine loads of 1 KB per round instead of twelve.  The ring is then four steps deep: 8 waves x 4
+// steps x 2 loads fill the compute unit's 64 places, and no refill waits.
+// ---------------------------------------------------------------------------
+template <class T, int NB, bool PRE, bool RND>
 __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(DpArgs a) {
+    static_assert(!RND || (!PRE && T::ROUND_META && NB <= 4), "per-round scale records: a raw x, a type that has them, at most four steps per round");
+    constexpr int MSB = T::META_SLICE_BYTES, NM = MSB / 64, CPR = MSB / 16; // scale loads per round, 16-byte chunks per row
     extern __shared__ uint4 lds_raw[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -451,37 +464,40 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     const int red_stride = 4 * a.S; // partial sums per output row in the LDS reduction buffer
     float *red_lane = red + (g_idx * rows_per_group + j) * red_stride + slice * 4 + (lane >> 4);
     const int nthreads = (int)blockDim.x;
+    // this wave's patch of scale records: 64 * NM x 16 bytes behind the reduction buffer
+    uint4 *wmeta = lds_raw + n16 + 1 + 4 + (a.G * rows_per_group * red_stride) / 4 + wave * 64 * NM;
 
     // 1. x first.  The compute unit's memory pipeline is one queue for all its waves, so the barrier makes
-    //    sure that no wave's x request stands behind another wave's weight requests.  A thread fetches at
-    //    most two 8-element split tasks of raw x (K <= 16 per thread by construction of the launch), or at
-    //    most five 16-byte pieces of an x that arrives already split.
-    uint4 x0, x1, x2, x3, x4 = {0, 0, 0, 0};
-    uint4 e0 = {0, 0, 0, 0}, e1 = e0, e2 = e0, e3 = e0; // second operand of a fused prologue
+    //    sure that no wave's x request stands behind another wave's weight requests.  A thread fetches one
+    //    8-element split task of raw x, and a second one where K exceeds eight elements per thread (K <= 16 per thread by
+    //    construction of the launch): a load nobody needs would still take a place in the pipeline.  Of an x that arrives
+    //    already split it fetches at most five 16-byte pieces.
+    const uint4 zero4 = {0, 0, 0, 0};
+    uint4 x0, x1, x2 = zero4, x3 = zero4, x4 = zero4;
+    uint4 e0 = zero4, e1 = zero4, e2 = zero4, e3 = zero4; // second operand of a fused prologue
     const int ntask = a.k >> 3; // K is a multiple of 64 here: whole quads of tasks
+    const bool second = nthreads < ntask;
     if (PRE) {
         const uint4 *src = reinterpret_cast<const uint4 *>(a.xq);
         auto piece = [&](int u) { int i = tid + u * nthreads; return src[i < n16 ? i : 0]; };
         x0 = piece(0); x1 = piece(1); x2 = piece(2); x3 = piece(3); x4 = piece(4);
     } else {
-        auto half = [&](int u, int h) {
+        auto half = [&](const float *src, int u, int h) {
             int t = tid + u * nthreads;
             t = t < ntask ? t : (t & 3);
-            return reinterpret_cast<const uint4 *>(a.x + (size_t)t * 8)[h];
+            return reinterpret_cast<const uint4 *>(src + (size_t)t * 8)[h];
         };
-        x0 = half(0, 0); x1 = half(0, 1); x2 = half(1, 0); x3 = half(1, 1);
+        x0 = half(a.x, 0, 0); x1 = half(a.x, 0, 1);
+        if (second) { x2 = half(a.x, 1, 0); x3 = half(a.x, 1, 1); }
         if (a.mode != AXQ_X_PLAIN) {
-            auto half2 = [&](int u, int h) {
-                int t = tid + u * nthreads;
-                t = t < ntask ? t : (t & 3);
-                return reinterpret_cast<const uint4 *>(a.aux + (size_t)t * 8)[h];
-            };
-            e0 = half2(0, 0); e1 = half2(0, 1); e2 = half2(1, 0); e3 = half2(1, 1);
+            e0 = half(a.aux, 0, 0); e1 = half(a.aux, 0, 1);
+            if (second) { e2 = half(a.aux, 1, 0); e3 = half(a.aux, 1, 1); }
         }
     }
     __builtin_amdgcn_s_barrier();
     // 2. the ring: rows past the group's end re-read its first step (cache hits, no HBM traffic)
     typename T::Raw buf[NB];
+    uint4 hm[NM];
     LaneOff lo;
     T::lane_offsets(a, c, lo);
     const int wg_row0 = blockIdx.x * a.G * rows_per_group;
@@ -489,14 +505,42 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
                          a.qh + (size_t)wg_row0 * a.qh_pitch};
     const uint32_t cp = (uint32_t)a.codes_pitch, mp = (uint32_t)a.meta_pitch, qp = (uint32_t)a.qh_pitch;
     const int rl0 = g_idx * rows_per_group + j, rl_last = last - wg_row0; // rows relative to the workgroup's first
+    // scale loads of a round (RND): 64 * NM lanes = (row of the round's 16, 16-byte chunk of the slice's MSB bytes); chunks past
+    // the row's end (a last slice that is not whole) are moved back inside it: they serve lanes whose x is zero
+    uint32_t moff[NM];
+    int mrl0[NM];
+    {
+        const int row_bytes = T::meta_row_bytes(a.k);
+#pragma unroll
+        for (int i = 0; i < NM; i++) {
+            const int flat = i * 64 + lane, off = slice * MSB + (flat % CPR) * 16;
+            moff[i] = (uint32_t)(off + 16 <= row_bytes ? off : row_bytes - 16);
+            mrl0[i] = g_idx * rows_per_group + flat / CPR;
+        }
+    }
     auto request = [&](int step, int b) {
-        int rl = rl0 + 4 * (step < a.steps ? step : 0);
+        const int s = step < a.steps ? step : 0;
+        int rl = rl0 + 4 * s;
         rl = rl < rl_last ? rl : rl_last;
         const RowOff ro = {(uint32_t)rl * cp, (uint32_t)rl * mp, (uint32_t)rl * qp};
-        T::load(bases, ro, lo, buf[b]);
+        if constexpr (RND) {
+            if (b == 0) { // rows past the group's steps belong to the next group or repeat the matrix's last row: read, not used
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    int rlm = mrl0[i] + 4 * s;
+                    rlm = rlm < rl_last ? rlm : rl_last;
+                    hm[i] = ld16(bases.meta, (uint32_t)rlm * mp + moff[i]);
+                }
+            }
+            T::load_codes(bases, ro, lo, buf[b]);
+        } else {
+            T::load(bases, ro, lo, buf[b]);
+        }
     };
-    constexpr int NB0 = NB < 2 ? NB : 2; // steps requested before x is staged: enough to start the stream,
-                                         // few enough that no wave is still blocked issuing them at the barrier
+    // steps requested before x is staged: enough to start the stream, few enough that no wave is still held up issuing them
+    // when the others want to pass the barrier.  With per-round records three: x (two loads) and the record load make nine
+    // places per wave, a few more than the compute unit holds -- x comes back first and makes room.
+    constexpr int NB0 = NB < (RND ? 3 : 2) ? NB : (RND ? 3 : 2);
 #pragma unroll
     for (int b = 0; b < NB0; b++) request(b, b);
     // 3. x -> LDS in split form -> this lane's A operands, while the weights are on their way
@@ -547,6 +591,13 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     const bool writer = (blk & 3) == 3;
     const int red_step = 4 * red_stride;
     auto fold = [&](int b, int step) {
+        if constexpr (RND) {
+            if (b == 0) { // the wave's own patch: LDS serves a wave's stores and loads in order
+#pragma unroll
+                for (int i = 0; i < NM; i++) wmeta[i * 64 + lane] = hm[i];
+            }
+            T::set_meta(buf[b], reinterpret_cast<const uint8_t *>(wmeta) + (b * 4 + j) * MSB, blk, c);
+        }
         float tot = sum_within_row(T::dot(buf[b], xo, c));
         if (writer) red_lane[step * red_step] = tot;
     };
@@ -568,199 +619,6 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     const int wg_rows = a.G * rows_per_group;
     float inv = 1.0f;
     if (!PRE && a.mode == AXQ_X_RMSNORM) {
-        const float *wsum = reinterpret_cast<const float *>(lds_raw + n16 + 1);
-        float tot = 0.f;
-        for (int i = 0; i < (nthreads >> 6); i++) tot += wsum[i];
-        inv = 1.0f / sqrtf(tot / (float)a.k + a.eps);
-    }
-    auto row_total = [&](int t) { // slice by slice, the four DPP rows of each in order
-        const float4 *pr = reinterpret_cast<const float4 *>(red + (size_t)t * red_stride);
-        float tot = 0.f;
-        for (int s = 0; s < a.S; s++) {
-            float4 v = pr[s];
-            tot += (v.x + v.y) + (v.z + v.w);
-        }
-        return tot * inv;
-    };
-    if (a.ymode == AXQ_Y_SWIGLU) {
-        // rows 8b..8b+3 are gate rows, 8b+4..8b+7 the up rows of the same outputs (wg_rows is a multiple of 8)
-        for (int t = tid; t < (wg_rows >> 1); t += nthreads) {
-            const int lg = ((t >> 2) << 3) + (t & 3);
-            const int row = blockIdx.x * wg_rows + lg;
-            if (row + 4 < a.n_rows) {
-                const float g = row_total(lg), u = row_total(lg + 4);
-                a.y[(blockIdx.x * wg_rows >> 1) + t] = (g * (1.0f / (1.0f + expf(-g)))) * u;
-            }
-        }
-        return;
-    }
-    for (int t = tid; t < wg_rows; t += nthreads) {
-        int row = blockIdx.x * wg_rows + t;
-        if (row < a.n_rows) {
-            const float tot = row_total(t);
-            a.y[row] = a.bias ? tot + a.bias[row] : tot;
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Q4_K from a raw x: the kernel above with the superblock headers fetched once per round of four row steps.
-//
-// A compute unit keeps about 64 vector memory instructions in flight, whatever they fetch (a wave that finds them
-// taken waits at its next load and does nothing else), and the stream runs at (bytes in flight) / latency.  A
-// header load has four lanes on each 16 bytes and so fetches 256 bytes where a code load fetches 1024: one in three
-// places in flight was spent on one ninth of the bytes.  Here one load per round fetches the headers of all its
-// 16 rows (lane = row and superblock), the wave parks them in an LDS patch of its own, and every fold reads its
-// header from there: nine loads of 1 KB per round instead of twelve.  The ring is four steps deep: 8 waves x 4 steps
-// x 2 loads fill the compute unit's 64 places, and no refill waits.
-// ---------------------------------------------------------------------------
-template <int NB> // ring depth: 4, or 3 for a group of three steps
-__global__ void __launch_bounds__(1024) gemv_q4k_kernel(DpArgs a) {
-    using T = DQ4K;
-    extern __shared__ uint4 lds_raw[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int g_idx = wave / a.S, slice = wave - g_idx * a.S;
-    const int blk = lane >> 2, j = lane & 3;
-    const int c = (slice << 4) + blk; // this lane's 64-weight chunk of the row
-
-    // LDS: the split form of x (limb planes, then group records), then the reduction buffer
-    uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw);
-    const int kpad = (a.k + 15) & ~15;
-    uint4 *wgrp = reinterpret_cast<uint4 *>(wplanes + (size_t)4 * kpad);
-    const int n16 = (int)(axq_split_bytes(a.k) >> 4);
-    // one spare 16-byte slot takes the surplus stores of step 3, 64 bytes hold per-wave sums of a fused RMSNorm
-    float *red = reinterpret_cast<float *>(lds_raw + n16 + 1 + 4);
-    const int rows_per_group = a.steps * 4;
-    const int last = a.n_rows - 1;
-    const int red_stride = 4 * a.S; // partial sums per output row in the LDS reduction buffer
-    float *red_lane = red + (g_idx * rows_per_group + j) * red_stride + slice * 4 + (lane >> 4);
-    const int nthreads = (int)blockDim.x;
-    // this wave's header patch: 64 x 16 bytes behind the reduction buffer
-    uint4 *wmeta = lds_raw + n16 + 1 + 4 + (a.G * rows_per_group * red_stride) / 4 + wave * 64;
-
-    // 1. x first.  The compute unit's memory pipeline is one queue for all its waves, so the barrier makes
-    //    sure that no wave's x request stands behind another wave's weight requests.  A thread fetches one
-    //    8-element split task of x, and a second one where K exceeds eight elements per thread (K <= 16 per thread by
-    //    construction of the launch): a load nobody needs would still take a place in the pipeline.
-    const uint4 zero4 = {0, 0, 0, 0};
-    uint4 x0, x1, x2 = zero4, x3 = zero4;
-    uint4 e0 = zero4, e1 = zero4, e2 = zero4, e3 = zero4; // second operand of a fused prologue
-    const int ntask = a.k >> 3; // K is a multiple of 64 here: whole quads of tasks
-    const bool second = nthreads < ntask;
-    {
-        auto half = [&](const float *src, int u, int h) {
-            int t = tid + u * nthreads;
-            t = t < ntask ? t : (t & 3);
-            return reinterpret_cast<const uint4 *>(src + (size_t)t * 8)[h];
-        };
-        x0 = half(a.x, 0, 0); x1 = half(a.x, 0, 1);
-        if (second) { x2 = half(a.x, 1, 0); x3 = half(a.x, 1, 1); }
-        if (a.mode != AXQ_X_PLAIN) {
-            e0 = half(a.aux, 0, 0); e1 = half(a.aux, 0, 1);
-            if (second) { e2 = half(a.aux, 1, 0); e3 = half(a.aux, 1, 1); }
-        }
-    }
-    __builtin_amdgcn_s_barrier();
-    // 2. the ring: rows past the group's end re-read its first step (cache hits, no HBM traffic)
-    uint4 q0[NB], q1[NB], hm;
-    LaneOff lo;
-    T::lane_offsets(a, c, lo);
-    const int wg_row0 = blockIdx.x * a.G * rows_per_group;
-    const Bases bases = {a.codes + (size_t)wg_row0 * a.codes_pitch, a.meta + (size_t)wg_row0 * a.meta_pitch,
-                         a.qh + (size_t)wg_row0 * a.qh_pitch};
-    const uint32_t cp = (uint32_t)a.codes_pitch, mp = (uint32_t)a.meta_pitch, qp = (uint32_t)a.qh_pitch;
-    const int rl0 = g_idx * rows_per_group + j, rl_last = last - wg_row0; // rows relative to the workgroup's first
-    // header load of a round: lane = (row of the round's 16, superblock of the wave's four)
-    const int nsb = a.k >> 8;
-    const int msb = slice * 4 + (lane & 3) < nsb ? slice * 4 + (lane & 3) : nsb - 1;
-    const uint32_t moff = (uint32_t)msb * 16;
-    const int mrl0 = g_idx * rows_per_group + (lane >> 2);
-    auto request = [&](int step, int b) {
-        const int s = step < a.steps ? step : 0;
-        if (b == 0) { // rows past the group's steps belong to the next group or repeat the matrix's last row: read, not used
-            int rlm = mrl0 + 4 * s;
-            rlm = rlm < rl_last ? rlm : rl_last;
-            hm = ld16(bases.meta, (uint32_t)rlm * mp + moff);
-        }
-        int rl = rl0 + 4 * s;
-        rl = rl < rl_last ? rl : rl_last;
-        q0[b] = ld16(bases.codes, (uint32_t)rl * cp + lo.c[0]);
-        q1[b] = ld16(bases.codes, (uint32_t)rl * cp + lo.c[1]);
-    };
-    constexpr int NB0 = NB < 3 ? NB : 3; // steps requested before x is staged: with the two loads of x and the header load, nine places
-                           // per wave, a few more than the compute unit holds -- x comes back first and makes room
-#pragma unroll
-    for (int b = 0; b < NB0; b++) request(b, b);
-    // 3. x -> LDS in split form -> this lane's A operands, while the weights are on their way
-    {
-        auto unpack = [](const uint4 &lo, const uint4 &hi, float (&v)[8]) {
-            v[0] = __builtin_bit_cast(float, lo.x); v[1] = __builtin_bit_cast(float, lo.y);
-            v[2] = __builtin_bit_cast(float, lo.z); v[3] = __builtin_bit_cast(float, lo.w);
-            v[4] = __builtin_bit_cast(float, hi.x); v[5] = __builtin_bit_cast(float, hi.y);
-            v[6] = __builtin_bit_cast(float, hi.z); v[7] = __builtin_bit_cast(float, hi.w);
-        };
-        float xv[2][8], ev[2][8];
-        unpack(x0, x1, xv[0]);
-        unpack(x2, x3, xv[1]);
-        const bool live0 = tid < ntask, live1 = tid + nthreads < ntask; // whole quads of lanes: K is a multiple of 64
-        if (a.mode == AXQ_X_RMSNORM) {
-            // RMSNorm::forward (llm/src/llama.rs:158-187) of the whole vector, by every workgroup for itself
-            unpack(e0, e1, ev[0]);
-            unpack(e2, e3, ev[1]);
-            float ss = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                if (live0) ss = fmaf(xv[0][i], xv[0][i], ss);
-                if (live1) ss = fmaf(xv[1][i], xv[1][i], ss);
-            }
-#pragma unroll
-            for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
-            float *wsum = reinterpret_cast<float *>(lds_raw + n16 + 1); // 16 floats kept for this between x and `red`
-            if (lane == 0) wsum[wave] = ss; // read after the final barrier: 1 / rms is a factor on the result
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                xv[0][i] *= ev[0][i];
-                xv[1][i] *= ev[1][i];
-            }
-        }
-        if (live0) axq_split8(xv[0], tid, true, wplanes, wgrp, kpad);
-        if (live1) axq_split8(xv[1], tid + nthreads, true, wplanes, wgrp, kpad);
-    }
-    lds_only_barrier(); // not __syncthreads(): that would also wait for the weights in flight
-    XOp xo;
-    fetch_xop<T>(wplanes, wgrp, kpad, a.k, j, c, xo);
-#pragma unroll
-    for (int b = NB0; b < NB; b++) request(b, b);
-
-    // 4. fold the steps through the ring
-    const bool writer = (blk & 3) == 3;
-    const int red_step = 4 * red_stride;
-    const int hidx = j * 4 + (blk >> 2);
-    auto fold = [&](int b, int step) {
-        if (b == 0) wmeta[lane] = hm; // the wave's own patch: LDS serves a wave's stores and loads in order
-        const DQ4K::Raw r = {q0[b], q1[b], wmeta[b * 16 + hidx]};
-        float tot = sum_within_row(T::dot(r, xo, c));
-        if (writer) red_lane[step * red_step] = tot;
-    };
-    const int rounds = (a.steps + NB - 1) / NB;
-    int step = 0;
-    for (int round = 0; round < rounds - 1; round++, step += NB) {
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            fold(b, step + b);
-            request(step + NB + b, b);
-        }
-    }
-#pragma unroll
-    for (int b = 0; b < NB; b++)
-        if (step + b < a.steps) fold(b, step + b); // the last round may be short: its spare slots hold re-reads
-
-    // partial sums -> y, in a fixed order
-    __syncthreads();
-    const int wg_rows = a.G * rows_per_group;
-    float inv = 1.0f;
-    if (a.mode == AXQ_X_RMSNORM) {
         const float *wsum = reinterpret_cast<const float *>(lds_raw + n16 + 1);
         float tot = 0.f;
         for (int i = 0; i < (nthreads >> 6); i++) tot += wsum[i];
@@ -842,7 +700,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     const int red_stride = 4 * a.S; // partial sums per output row in the LDS reduction buffer
     float *red_lane = red + (g_idx * rows_per_group + j) * red_stride + slice * 4 + (lane >> 4);
     typename T::Raw buf[NB];
-    // T::ROUND_META (see gemv_q4k_kernel): one header load per round of NB <= 4 steps, parked in an LDS patch of the wave
+    // T::ROUND_META (see gemv_dp_kernel's RND): one load of scale records per round of NB <= 4 steps, parked in an LDS patch of the wave
     constexpr bool ROUNDS = T::ROUND_META && NB <= 4;
     constexpr int MSB = T::META_SLICE_BYTES, NM = MSB / 64, CPR = MSB / 16; // loads per round, 16-byte chunks per row
     uint4 hm[NM];
@@ -1027,8 +885,8 @@ void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, si
             return;
         }
     }
-    if (lds > 64 * 1024) (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE>), lds_allowed, 160 * 1024);
-    gemv_dp_kernel<T, NB, PRE><<<grid, block, lds, ctx->stream>>>(a);
+    if (lds > 64 * 1024) (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE, false>), lds_allowed, 160 * 1024);
+    gemv_dp_kernel<T, NB, PRE, false><<<grid, block, lds, ctx->stream>>>(a);
 }
 
 template <class T, bool PRE>
@@ -1057,14 +915,14 @@ bool launch_q4k_rounds<DQ4K>(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsig
     // with two steps (o projection) or one group of 14 waves over a long K (down projection, two split tasks per thread)
     // the kernel with per-wave staging and no barrier is ahead
     if (a.G < 2 || a.steps < 3) return false;
-    lds += (size_t)(block / 64) * 1024;
+    lds += (size_t)(block / 64) * 16 * DQ4K::META_SLICE_BYTES; // the waves' patches of scale records
     if (lds > 160 * 1024) return false;
     if (lds > 64 * 1024) {
-        (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_q4k_kernel<3>), lds_allowed[0], 160 * 1024);
-        (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_q4k_kernel<4>), lds_allowed[1], 160 * 1024);
+        (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<DQ4K, 3, false, true>), lds_allowed[0], 160 * 1024);
+        (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<DQ4K, 4, false, true>), lds_allowed[1], 160 * 1024);
     }
-    if (a.steps == 3) gemv_q4k_kernel<3><<<grid, block, lds, ctx->stream>>>(a);
-    else gemv_q4k_kernel<4><<<grid, block, lds, ctx->stream>>>(a);
+    if (a.steps == 3) gemv_dp_kernel<DQ4K, 3, false, true><<<grid, block, lds, ctx->stream>>>(a);
+    else gemv_dp_kernel<DQ4K, 4, false, true><<<grid, block, lds, ctx->stream>>>(a);
     return true;
 }
 
