@@ -459,8 +459,8 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
 //     hi ch + hi cl + lo ch laid side by side along the extended K axis.
 // Against two MFMAs per product over all of K (the other block types below) this is 1 + 3/32.
 //
-// Tiling: a workgroup computes BM x 256 outputs with BM * 2 threads; every wave owns a 128 x 64 block (4 x 2 MFMA
-// tiles) and every thread also feeds: per K step of 64 it copies 64 bytes of the x tile and turns 32 codes of
+// Tiling: a workgroup computes BM x 256 outputs with eight waves, each a block of 128 x 64 (BM = 256: 4 x 2 MFMA
+// tiles) or 64 x 64 (BM = 128), and every thread also feeds: per K step of 64 it copies 64 bytes of the x tile and turns 32 codes of
 // one weight row into operands for the step after the next one's... (two LDS stages, one barrier per step;
 // the global loads of step s + 2 are in flight while step s + 1 is converted and step s multiplied).
 // x is stored by the pre-pass with elements 1 and 2 of every group of four exchanged: the codes of a dword
@@ -492,12 +492,15 @@ __device__ inline void wait_vm_and_lds() {
     __builtin_amdgcn_s_waitcnt(((N >> 4) << 14) | (7 << 4) | (N & 15));
 }
 
-template <int BM>
-__global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
-    constexpr int NT = BM * 2;           // threads
-    constexpr int NW = NT / 64;          // waves: (BM / 128) x 4 blocks of 128 x 64
+template <int BM, int NT>
+__global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
+    constexpr int NW = NT / 64;          // waves: NW / 4 rows of four, each wave a block of WROWS x 64
+    constexpr int WROWS = BM / (NW / 4); // 128 or 64
+    constexpr int MI = WROWS / 32;       // MFMA tiles of a wave along M
     constexpr int BT = QBN * 2 / NT;     // (weight row, half) tasks per thread and step (1 or 2)
-    constexpr int AROWS = BM / NW;       // x rows a wave brings in per step (= 32: four loads of eight rows)
+    constexpr int AROWS = BM / NW;       // x rows a wave brings in per step: XL loads of eight rows
+    constexpr int XL = AROWS / 8;
+    static_assert(AROWS % 16 == 0 && MI % 2 == 0 && BT >= 1, "tile shape");
     // LDS (halfs): three stages of the x tile, then two of the weight tile.  A tile row is 64 halfs, unpadded, its eight
     // 16-byte chunks stored at chunk ^ ((row / 2) & 7): x tiles are written by loads that go straight to LDS, 1 KB per
     // wave and instruction in lane order, so padding is not to be had; the exchange keeps the fragment reads of sixteen
@@ -651,15 +654,15 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
     };
 
     // ---- multiplier side
-    const int wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
+    const int wm = (wave >> 2) * WROWS, wn = (wave & 3) * 64;
     const int li = lane & 31, hh = lane >> 5;
     // fragment of sub-step t: tile row r = w + 32 i + li, chunk 2 t + hh, stored at chunk ^ ((r / 2) & 7): the address is
     // (r * 64 + ((hh ^ (li / 2)) & 7) * 8) ^ (16 t) in halfs
     const int sw = ((hh ^ (li >> 1)) & 7) * 8;
     const int a_rd = (wm + li) * 64 + sw, b_rd = BOFF + (wn + li) * 64 + sw;
-    float16v acc[4][2];
+    float16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -693,7 +696,7 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int q = 0; q < 16; q++) acc[i][j][q] *= r[j];
     };
@@ -704,7 +707,7 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < 2; j++) bf[j] = *reinterpret_cast<const half8 *>(lds + par * BSTAGE + (b_rd ^ (t * 16)) + j * 32 * 64);
 #pragma unroll
-        for (int ih = 0; ih < 2; ih++) {
+        for (int ih = 0; ih < MI / 2; ih++) {
             half8 af[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) af[i] = *reinterpret_cast<const half8 *>(lds + as + (a_rd ^ (t * 16)) + (2 * ih + i) * 32 * 64);
@@ -761,9 +764,9 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
                 }
             }
             // younger than the x tile of step g + 1: see the order of the loads above
-            if (i == 0) wait_vm_and_lds<(KG ? 0 : 2) + 4 + F>();
-            else if (i == 1) wait_vm_and_lds<F + 4>();
-            else wait_vm_and_lds<4>();
+            if (i == 0) wait_vm_and_lds<(KG ? 0 : 2) + XL + F>();
+            else if (i == 1) wait_vm_and_lds<F + XL>();
+            else wait_vm_and_lds<XL>();
             lds_barrier();
             g3 = g3 == 2 ? 0 : g3 + 1;
             if (i == 2 && !KG && KN) {
@@ -792,7 +795,7 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
         S_c[j] = s_of(dmax_c[j]);
         const float f = unit[j] * 16777216.0f * S_c[j];
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < MI; i++)
 #pragma unroll
             for (int q = 0; q < 16; q++) acc[i][j][q] *= f;
     }
@@ -800,7 +803,7 @@ __global__ void __launch_bounds__(BM * 2) gemm_q4k_kernel(GemmArgs a) {
     wait_vm_and_lds<0>(); // nothing of this workgroup may still be on its way into LDS when it ends
     // D layout: lane -> column li; register r -> row 8 * (r / 4) + 4 * (lane / 32) + r % 4
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int gn = n0 + wn + j * 32 + li;
@@ -1103,10 +1106,13 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, bool f32_rows, size_t ex
                         (long long)w->k);
     if (w->n_rows > INT32_MAX || w->k > INT32_MAX)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
+    // rows of a workgroup's tile: the Q4_K kernel's 128-row tile keeps eight waves (64 x 64 each), so it also serves
+    // 129..256 rows, where the 256-row tile would leave half the compute units idle
+    const bool route_q4k = q4k_route(w, f32_rows);
     static const int bm_knob = getenv("AXQ_GEMM_BM") ? atoi(getenv("AXQ_GEMM_BM")) : 0; // development knob: 128 or 256 for every shape
-    const int bm = bm_knob ? bm_knob : (m > 128 ? 256 : 128);
+    const int bm = bm_knob ? bm_knob : (m > (route_q4k ? 256 : 128) ? 256 : 128);
     p->wm = bm / 128;
-    p->q4k = q4k_route(w, f32_rows);
+    p->q4k = route_q4k;
     const int bn = p->q4k ? QBN : BN;
     const long tiles = (long)((w->n_rows + bn - 1) / bn) * ((m + bm - 1) / bm);
     const int ksteps = (int)(w->k / BK), cus = ctx->prop.multiProcessorCount;
@@ -1144,11 +1150,11 @@ int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits) {
     const size_t lds = (size_t)(3 * bm * 64 + 2 * QBN * 64) * sizeof(_Float16); // three x stages, two weight stages
     {
         int rc;
-        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<256>), lds_allowed[1], (3 * 256 * 64 + 2 * QBN * 64) * 2))) return rc;
-        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<128>), lds_allowed[0], (3 * 128 * 64 + 2 * QBN * 64) * 2))) return rc;
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<256, 512>), lds_allowed[1], (3 * 256 * 64 + 2 * QBN * 64) * 2))) return rc;
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<128, 512>), lds_allowed[0], (3 * 128 * 64 + 2 * QBN * 64) * 2))) return rc;
     }
-    if (a.wm == 2) gemm_q4k_kernel<256><<<grid, 512, lds, ctx->stream>>>(a);
-    else gemm_q4k_kernel<128><<<grid, 256, lds, ctx->stream>>>(a);
+    if (a.wm == 2) gemm_q4k_kernel<256, 512><<<grid, 512, lds, ctx->stream>>>(a);
+    else gemm_q4k_kernel<128, 512><<<grid, 512, lds, ctx->stream>>>(a);
     AXQ_LAUNCH_CHECK(ctx, "gemm_q4k_kernel");
     if (splits > 1) {
         const int rows = a.pair ? a.m / 2 : a.m;

@@ -43,7 +43,7 @@ def test_config_prefill_k4096(ctx, qtype, m):
 
 
 @pytest.mark.parametrize("qtype", [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K])
-@pytest.mark.parametrize("m,n,k", [(640, 136, 512), (1100, 520, 1024)])
+@pytest.mark.parametrize("m,n,k", [(250, 300, 1024), (640, 136, 512), (1100, 520, 1024)])
 def test_many_rows(ctx, qtype, m, n, k):
     """Several row tiles per column tile, ragged in both directions."""
     _check(ctx, qtype, m, n, k, seed=m + qtype)
