@@ -279,18 +279,19 @@ __device__ inline void lds_barrier() {
     __builtin_amdgcn_sched_barrier(0); // nothing moves across: what follows may count on the waits in front of the barrier
 }
 
-// WM = 1 or 2: the workgroup computes (128 * WM) x 128 outputs with 4 * WM waves of two kinds.
-//   - 2 * WM "multiplier" waves each own a 128 x 64 block (4 x 2 MFMA tiles, 128 accumulator registers) and
-//     do nothing but read the current LDS stage and issue MFMAs;
-//   - 2 * WM "feeder" waves fetch the x tile and the packed weights of the step after next, convert the
+// WM = 1 or 2: the workgroup computes (128 * WM) x 128 outputs with eight waves of two kinds.
+//   - four "multiplier" waves each own a (64 * WM) x 64 block (2 WM x 2 MFMA tiles) and do nothing but read the
+//     current LDS stage and issue MFMAs;
+//   - four "feeder" waves fetch the x tile and the packed weights of the step after next, convert the
 //     next step's weights (dequantise, split into two f16) and write the other LDS stage.
-// Waves are dealt to the four SIMDs in turn, so with WM = 2 every SIMD holds one wave of each kind and its
-// vector ALU converts while its matrix pipe multiplies; one barrier per K step hands the stages over.
+// Waves are dealt to the four SIMDs in turn, so every SIMD holds one wave of each kind and its vector ALU converts
+// while its matrix pipe multiplies; one barrier per K step hands the stages over.
 template <class T, int WM>
-__global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
-    constexpr int BM = 128 * WM, NTF = 128 * WM; // rows of x per tile; feeder threads
-    constexpr int XV = BM * 8 / NTF;             // 16-byte x vectors per feeder thread and K step (= 8)
-    constexpr int UNITS = BN * 4 / NTF;          // 16-weight units per feeder thread and K step (2 or 4)
+__global__ void __launch_bounds__(512) gemm_kernel(GemmArgs a) {
+    constexpr int BM = 128 * WM, NTF = 256;      // rows of x per tile; feeder threads
+    constexpr int MI = 2 * WM;                   // MFMA tiles of a multiplier wave along M
+    constexpr int XV = BM * 8 / NTF;             // 16-byte x vectors per feeder thread and K step (4 or 8)
+    constexpr int UNITS = BN * 4 / NTF;          // 16-weight units per feeder thread and K step (= 2)
     constexpr int STAGE = (BM + 2 * BN) * LDK;   // halfs per LDS stage
     extern __shared__ _Float16 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -370,11 +371,11 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
         return;
     }
 
-    const int wm = (wave >> 1) * 128, wn = (wave & 1) * 64; // this wave's block inside the tile
+    const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 64; // this wave's block inside the tile
     const int li = lane & 31, lk = (lane >> 5) * 8;
-    float16v acc[4][2];
+    float16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -383,10 +384,10 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
     for (int ks = 0; ks < ksteps; ks++) {
         const _Float16 *As = lds + (ks & 1) * STAGE, *Bh = As + BM * LDK, *Bl = Bh + BN * LDK;
         // fragments of sub-step kk + 1 are read from LDS while the sixteen MFMAs of sub-step kk run
-        half8 af[2][4], bh[2][2], bl[2][2];
+        half8 af[2][MI], bh[2][2], bl[2][2];
         auto read_frags = [&](int kk, int slot) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) af[slot][i] = *reinterpret_cast<const half8 *>(As + (wm + i * 32 + li) * LDK + kk + lk);
+            for (int i = 0; i < MI; i++) af[slot][i] = *reinterpret_cast<const half8 *>(As + (wm + i * 32 + li) * LDK + kk + lk);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 bh[slot][j] = *reinterpret_cast<const half8 *>(Bh + (wn + j * 32 + li) * LDK + kk + lk);
@@ -399,7 +400,7 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
             if (t + 1 < BK / 16) read_frags((t + 1) * 16, (t + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t & 1][i], bl[t & 1][j], acc[i][j], 0, 0, 0);
@@ -411,7 +412,7 @@ __global__ void __launch_bounds__(256 * WM) gemm_kernel(GemmArgs a) {
     }
     // D layout: lane -> column li; register r -> row 8 * (r / 4) + 4 * (lane / 32) + r % 4
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int gn = n0 + wn + j * 32 + li;
@@ -936,7 +937,7 @@ int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
         if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_kernel<T, 1>), lds_allowed[0], 2 * (128 + 2 * BN) * LDK * 2))) return rc;
     }
     if (wm == 2) gemm_kernel<T, 2><<<grid, 512, lds, ctx->stream>>>(a);
-    else gemm_kernel<T, 1><<<grid, 256, lds, ctx->stream>>>(a);
+    else gemm_kernel<T, 1><<<grid, 512, lds, ctx->stream>>>(a);
     AXQ_LAUNCH_CHECK(ctx, "gemm_kernel");
     if (splits > 1) {
         const int rows = a.pair ? a.m / 2 : a.m;
