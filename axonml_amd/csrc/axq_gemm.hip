@@ -124,7 +124,7 @@ struct GQ4K {
 
 template <bool WITH_MIN>
 struct GQ4x { // reference nibble order: byte i = elements 2i (low), 2i+1 (high)
-    static constexpr bool PRESCALED = false;
+    static constexpr bool PRESCALED = true;
     static constexpr float WS = WSCALE;
     struct Raw { uint2 q; uint32_t m; };
     __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
@@ -136,17 +136,17 @@ struct GQ4x { // reference nibble order: byte i = elements 2i (low), 2i+1 (high)
     }
     __device__ static void cvt16(const Raw &r, int, int u4, float (&w)[16], int &k0, int &k1) {
         const int part = u4 & 1;
-        const float scale = h2f(r.m & 0xFFFF), mn = WITH_MIN ? h2f(r.m >> 16) : 0.f;
+        // (nib - 8) * d = nib * d - 8 d exactly; with a minimum one rounding (fma) where the f32 reference has two: far
+        // below what f16 pairs resolve.  Four codes per mask, one conversion per code straight from its byte.
+        const float scale = WSCALE * h2f(r.m & 0xFFFF), mn = WITH_MIN ? WSCALE * h2f(r.m >> 16) : -8.0f * scale;
         const uint32_t qq[2] = {r.q.x, r.q.y};
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            uint32_t nib = (qq[i >> 3] >> (4 * (i & 7))) & 0xF;
-            if (WITH_MIN) {
-                float t = (float)nib * scale;
-                w[i] = t + mn;
-            } else {
-                w[i] = (float)((int)nib - 8) * scale;
-            }
+        for (int j = 0; j < 2; j++) {
+            const uint32_t lo = qq[j] & 0x0F0F0F0Fu, hi = (qq[j] >> 4) & 0x0F0F0F0Fu;
+            w[8 * j + 0] = fmaf(ubyte<0>(lo), scale, mn); w[8 * j + 1] = fmaf(ubyte<0>(hi), scale, mn);
+            w[8 * j + 2] = fmaf(ubyte<1>(lo), scale, mn); w[8 * j + 3] = fmaf(ubyte<1>(hi), scale, mn);
+            w[8 * j + 4] = fmaf(ubyte<2>(lo), scale, mn); w[8 * j + 5] = fmaf(ubyte<2>(hi), scale, mn);
+            w[8 * j + 6] = fmaf(ubyte<3>(lo), scale, mn); w[8 * j + 7] = fmaf(ubyte<3>(hi), scale, mn);
         }
         k0 = (u4 >> 1) * 32 + part * 16;
         k1 = k0 + 8;
@@ -155,7 +155,7 @@ struct GQ4x { // reference nibble order: byte i = elements 2i (low), 2i+1 (high)
 
 template <bool WITH_MIN>
 struct GQ5x { // byte j = elements j (low nibble) and j + 16 (high); qh bit e = bit 4 of element e
-    static constexpr bool PRESCALED = false;
+    static constexpr bool PRESCALED = true;
     static constexpr float WS = WSCALE;
     struct Raw { uint2 q; uint32_t qh, m; };
     __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
@@ -169,22 +169,20 @@ struct GQ5x { // byte j = elements j (low nibble) and j + 16 (high); qh bit e = 
     __device__ static void cvt16(const Raw &r, int, int u4, float (&w)[16], int &k0, int &k1) {
         const int part = u4 & 1;
         const uint32_t qh = r.qh;
-        const float d = h2f(r.m & 0xFFFF), mn = WITH_MIN ? h2f(r.m >> 16) : 0.f;
+        // (u - 16) * d = u * d - 16 d exactly; with a minimum one rounding (fma) where the f32 reference has two.
+        const float d = WSCALE * h2f(r.m & 0xFFFF), mn = WITH_MIN ? WSCALE * h2f(r.m >> 16) : -16.0f * d;
         const uint32_t qq[2] = {r.q.x, r.q.y};
+        // four bits of qh -> bit 4 of four bytes: the copies of the multiplication lie 7 bits apart and do not meet
+        auto fifth = [](uint32_t four) { return ((four * 0x00204081u) & 0x01010101u) << 4; };
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int e = part * 8 + i;
-            uint32_t byte = (qq[i >> 2] >> (8 * (i & 3))) & 0xFF;
-            int u0 = (int)((byte & 0xF) | (((qh >> e) & 1u) << 4));
-            int u1 = (int)((byte >> 4) | (((qh >> (e + 16)) & 1u) << 4));
-            if (WITH_MIN) {
-                float t0 = (float)u0 * d, t1 = (float)u1 * d;
-                w[i] = t0 + mn;
-                w[8 + i] = t1 + mn;
-            } else {
-                w[i] = (float)(u0 - 16) * d;
-                w[8 + i] = (float)(u1 - 16) * d;
-            }
+        for (int j = 0; j < 2; j++) {
+            const int e = part * 8 + 4 * j;
+            const uint32_t lo = (qq[j] & 0x0F0F0F0Fu) | fifth((qh >> e) & 0xFu);
+            const uint32_t hi = ((qq[j] >> 4) & 0x0F0F0F0Fu) | fifth((qh >> (e + 16)) & 0xFu);
+            w[4 * j + 0] = fmaf(ubyte<0>(lo), d, mn); w[4 * j + 1] = fmaf(ubyte<1>(lo), d, mn);
+            w[4 * j + 2] = fmaf(ubyte<2>(lo), d, mn); w[4 * j + 3] = fmaf(ubyte<3>(lo), d, mn);
+            w[8 + 4 * j + 0] = fmaf(ubyte<0>(hi), d, mn); w[8 + 4 * j + 1] = fmaf(ubyte<1>(hi), d, mn);
+            w[8 + 4 * j + 2] = fmaf(ubyte<2>(hi), d, mn); w[8 + 4 * j + 3] = fmaf(ubyte<3>(hi), d, mn);
         }
         k0 = (u4 >> 1) * 32 + part * 8;
         k1 = k0 + 16;
@@ -192,7 +190,7 @@ struct GQ5x { // byte j = elements j (low nibble) and j + 16 (high); qh bit e = 
 };
 
 struct GQ80 {
-    static constexpr bool PRESCALED = false;
+    static constexpr bool PRESCALED = true;
     static constexpr float WS = WSCALE;
     struct Raw { uint4 q; uint32_t m; };
     __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
@@ -202,10 +200,14 @@ struct GQ80 {
     }
     __device__ static void cvt16(const Raw &r, int, int u4, float (&w)[16], int &k0, int &k1) {
         const int part = u4 & 1;
-        const float scale = h2f(r.m);
-        const uint32_t qq[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        // q * d = (q + 128) * d - 128 d exactly: the codes as unsigned bytes, one conversion each
+        const float scale = WSCALE * h2f(r.m), off = -128.0f * scale;
+        const uint32_t qq[4] = {r.q.x ^ 0x80808080u, r.q.y ^ 0x80808080u, r.q.z ^ 0x80808080u, r.q.w ^ 0x80808080u};
 #pragma unroll
-        for (int i = 0; i < 16; i++) w[i] = (float)(signed char)((qq[i >> 2] >> (8 * (i & 3))) & 0xFF) * scale;
+        for (int j = 0; j < 4; j++) {
+            w[4 * j + 0] = fmaf(ubyte<0>(qq[j]), scale, off); w[4 * j + 1] = fmaf(ubyte<1>(qq[j]), scale, off);
+            w[4 * j + 2] = fmaf(ubyte<2>(qq[j]), scale, off); w[4 * j + 3] = fmaf(ubyte<3>(qq[j]), scale, off);
+        }
         k0 = (u4 >> 1) * 32 + part * 16;
         k1 = k0 + 8;
     }
