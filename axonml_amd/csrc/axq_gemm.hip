@@ -835,6 +835,296 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
         }
 }
 
+// ---------------------------------------------------------------------------
+// Q5_0 / Q5_1: one MFMA per product, the block's scale applied by the vector ALU.
+//
+// w = d * (q - 16) (Q5_0) or d * q + m (Q5_1) with a five-bit code q and f16 d (and m) per block of 32.  The B operand
+// is the centred code q - 16 itself, an integer that f16 holds exactly: the two MFMAs of a block (32 k) start from
+// zero, so their result is the block's sum of (q - 16) * x, exact in f32 to within the accumulation, and every lane
+// then adds it, times the d of its column and block, into its accumulators (a lane of the 32 x 32 MFMA output owns
+// one column): sixteen v_fma per tile and block where gemm_kernel pays a second MFMA per product and about ten
+// vector-ALU instructions per weight for the dequantisation and the high/low split.  Converting costs two instructions
+// per pair of weights: the code pairs come out of the packed nibbles two at a time with one mask each, the fifth bits
+// out of qh four at a time with one multiplication, 0x6400 | q is the f16 number 1024 + q, and one packed subtraction
+// of 1040 centres it.  x is stored with elements 1 and 2 of every four exchanged, as for the Q4_K kernel, which is the
+// order the masks produce.
+// Q5_1 goes in as d * (q - 16) + (m + 16 d): the first sum is then as well conditioned as the weights themselves (with
+// q as it is, 0..31, two sums three times the size of the result would cancel in f32).  The second,
+// sum_b (m + 16 d)[n, b] * (sum of x over block b), goes through the matrix pipe too, two MFMAs per tile and
+// superblock of 256 k: A = the eight block sums of the row as f16 pairs (hi for k 0..7, lo for k 8..15, written by the
+// x pre-pass for the Q4_K kernel's minimum term, times 1 / 64), B = the eight m of the column, twice, and then the
+// eight 16 d, both times 256; the main term's scales are d * 256 / 64 to match.
+//
+// The pipeline is the Q4_K kernel's: 256 x 128 outputs per workgroup of eight waves (64 x 64 each), x tiles straight
+// from memory into three LDS stages, two weight stages, one barrier per K step that waits for LDS only, explicit
+// counts of the loads issued since.  A thread converts half a block (16 weights of one row) per step.  The scale
+// records of the tile's columns lie in LDS too, a superblock of them at a time.
+// ---------------------------------------------------------------------------
+constexpr int PBN = 128; // output columns (weight rows) per workgroup
+constexpr float XSUM_SCALE = 1.0f / 64.0f; // the x pre-pass stores the block sums times this
+
+template <bool WITH_MIN>
+__global__ void __launch_bounds__(512) gemm_q5_kernel(GemmArgs a) {
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    constexpr int BM = 256, NW = 8, AROWS = BM / NW, XL = AROWS / 8;
+    constexpr int ASTAGE = BM * 64, BSTAGE = PBN * 64, BOFF = 3 * ASTAGE; // halfs
+    constexpr int F = 2;                   // loads of a weight request: codes, fifth bits
+    constexpr int ML = 1;                  // per superblock: this wave's kilobyte of scale records
+    constexpr float OFF = 1040.0f;         // 0x6400 | q is 1024 + q; the codes go in centred, q - 16 (Q5_0's own form)
+    constexpr float ASCALE = WSCALE * XSUM_SCALE; // the accumulators hold the result times this
+    extern __shared__ _Float16 lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nt = (a.n + PBN - 1) / PBN, total = (int)gridDim.x;
+    int tile = blockIdx.x;
+    if (total % 8 == 0) tile = (tile & 7) * (total >> 3) + (tile >> 3); // workgroups of one XCD share x tiles
+    const int m0 = (tile / nt) * BM, n0 = (tile % nt) * PBN;
+    const int kbeg = (int)blockIdx.y * a.steps_per_split; // in steps of 64 k; a multiple of 4 (whole superblocks)
+    const int T = a.k / BK - kbeg < a.steps_per_split ? a.k / BK - kbeg : a.steps_per_split; // a multiple of 4
+
+    // ---- x tiles (rows of the scratch buffer are allocated up to a multiple of BM: no clamp)
+    const uint8_t *xbase = reinterpret_cast<const uint8_t *>(a.xh + (size_t)m0 * a.k + (size_t)kbeg * BK);
+    const uint32_t xrow_l = (uint32_t)(wave * AROWS + (lane >> 3)), xchunk_l = (uint32_t)((lane & 7) ^ (lane >> 4));
+    const uint32_t xoff = (xrow_l * (uint32_t)a.k + xchunk_l * 8) * 2;
+    const size_t x8rows = (size_t)8 * a.k * 2;
+    auto load_x = [&](int step, int stage) {
+        step = step < T ? step : T - 1;
+        const uint8_t *g = xbase + (size_t)step * (BK * 2);
+        _Float16 *dst = lds + stage * ASTAGE + wave * AROWS * 64;
+#pragma unroll
+        for (int i = 0; i < XL; i++)
+            __builtin_amdgcn_global_load_lds((gbl_void *)(g + i * x8rows + ((i & 1) ? xoff ^ 64u : xoff)), (lds_void *)(dst + i * 8 * 64), 16, 0, 0);
+        asm volatile("" ::: "memory"); // what is requested after this stays after it: the waits in front of the barriers count on the order
+    };
+
+    // ---- weights: this thread's half block (16 weights) of every step
+    const int wrow = tid & 127, bis = tid >> 8, half = (tid >> 7) & 1; // row of the tile; which of the step's two blocks; which half of it
+    const int crow = n0 + wrow < a.n ? n0 + wrow : a.n - 1;
+    const uint8_t *cp = a.codes + (size_t)crow * a.codes_pitch, *qp = a.qh + (size_t)crow * a.qh_pitch;
+    struct Raw { u32x4 q; uint32_t qh; };
+    auto fetch = [&](int step, Raw &r) { // the thread's block of a step (both halves fetch all of it: the nibbles interleave)
+        step = step < T ? step : T - 1;
+        const size_t blk = (size_t)(kbeg + step) * 2 + bis;
+        r.q = *reinterpret_cast<const u32x4 *>(cp + blk * 16);
+        r.qh = *reinterpret_cast<const uint32_t *>(qp + blk * 4);
+        asm volatile("" ::: "memory");
+    };
+    const int b_wr = wrow * 64; // the thread's row in a weight plane; chunk ch of it lies at (ch ^ ((wrow / 2) & 7)) * 8
+    const int b_sw = (wrow >> 1) & 7;
+    // chunk 2 half + cc (cc = 0, 1: eight weights) of the block in `r` -> weight stage `stage`: the low nibbles of a block
+    // are its elements 0..15, the high nibbles 16..31
+    auto convert = [&](const Raw &r, int cc, int stage) {
+        const uint32_t d0 = cc ? r.q[2] : r.q[0], d1 = cc ? r.q[3] : r.q[1];
+        const int sh = half * 4, c = 2 * half + cc;
+        uint32_t pr[4] = {(d0 >> sh) & 0x000F000Fu, (d0 >> (sh + 8)) & 0x000F000Fu, (d1 >> sh) & 0x000F000Fu, (d1 >> (sh + 8)) & 0x000F000Fu};
+        // bits b0..b3 of `four` times (2^4 + 2^18): b0 lands on bit 4 and b2 on bit 20 (of the pair e, e + 2), nothing else does
+        const uint32_t eight = (r.qh >> (8 * c)) & 0xFFu;
+        pr[0] |= ((eight & 0xFu) * 0x40010u) & 0x00100010u;
+        pr[1] |= (((eight >> 1) & 0x7u) * 0x40010u) & 0x00100010u;
+        pr[2] |= ((eight >> 4) * 0x40010u) & 0x00100010u;
+        pr[3] |= ((eight >> 5) * 0x40010u) & 0x00100010u;
+        const half2v off2 = {(_Float16)OFF, (_Float16)OFF};
+        uint32_t oh[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t bits = pr[i] | 0x64006400u;
+            const half2v qf = __builtin_bit_cast(half2v, bits) - off2; // exact: integers below 2048
+            oh[i] = __builtin_bit_cast(uint32_t, qf);
+        }
+        _Float16 *bs = lds + BOFF + stage * BSTAGE + b_wr + (((4 * bis + c) ^ b_sw) * 8);
+        *reinterpret_cast<u32x4 *>(bs) = u32x4{oh[0], oh[1], oh[2], oh[3]};
+    };
+
+    // ---- multiplier side
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int li = lane & 31, hh = lane >> 5;
+    const int sw = ((hh ^ (li >> 1)) & 7) * 8;
+    const int a_rd = (wm + li) * 64 + sw, b_rd = BOFF + (wn + li) * 64 + sw;
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    // The scale records of the tile's 128 columns, eight blocks of a superblock each ((d, m) pairs for Q5_1: 32 bytes;
+    // d alone for Q5_0: 16 bytes), lie in LDS behind the weight stages, two superblocks of them: every wave brings in a
+    // kilobyte of the next superblock's at the first step of a superblock (the same kilobyte twice or four times over:
+    // one request per wave keeps the waves' counts of loads equal).
+    constexpr int RV = WITH_MIN ? 2 : 1;      // 16-byte vectors per column and superblock
+    constexpr int RECB = PBN * 16 * RV;       // bytes of one superblock's records
+    uint8_t *rec_lds = reinterpret_cast<uint8_t *>(lds + BOFF + 2 * BSTAGE);
+    const int nsb = T >> 2;
+    const int rc0 = WITH_MIN ? (wave & 3) * 32 : (wave & 1) * 64; // first column of this wave's kilobyte
+    int rcol = n0 + rc0 + (WITH_MIN ? lane >> 1 : lane);
+    rcol = rcol < a.n ? rcol : a.n - 1;
+    const uint8_t *rsrc = a.meta + (size_t)rcol * a.meta_pitch + (size_t)(kbeg >> 2) * (16 * RV) + (WITH_MIN ? (lane & 1) * 16 : 0);
+    auto fetch_records = [&](int sb) {
+        sb = sb < nsb ? sb : nsb - 1;
+        __builtin_amdgcn_global_load_lds((gbl_void *)(rsrc + (size_t)sb * (16 * RV)), (lds_void *)(rec_lds + (sb & 1) * RECB + rc0 * 16 * RV), 16, 0, 0);
+        asm volatile("" ::: "memory");
+    };
+    u32x4 mx[2];
+    const uint8_t *x3p = reinterpret_cast<const uint8_t *>(a.xs3 + (size_t)(m0 + wm + li) * a.xs3_pitch + (size_t)(kbeg >> 2) * 32 + hh * 16);
+    auto fetch_sums = [&](int sb) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) mx[i] = *reinterpret_cast<const u32x4 *>(x3p + ((size_t)i * 32 * a.xs3_pitch + (size_t)sb * 32) * 2);
+    };
+    // d of block bq (0..7) of superblock sb, column j of this lane, times WSCALE
+    const uint8_t *rlane = rec_lds + (wn + li) * 16 * RV;
+    auto scale_of = [&](int sb, int j, int bq) {
+        const uint16_t w = *reinterpret_cast<const uint16_t *>(rlane + (sb & 1) * RECB + j * 32 * 16 * RV + bq * (WITH_MIN ? 4 : 2));
+        return ASCALE * h2f(w);
+    };
+    // One block of 32 k = two sub-steps t0 = 2 hb, t0 + 1 of the step: its sum over k, then times the block's d into the
+    // accumulators.  bq: the block's number in the superblock.
+    auto multiply_block = [&](int as, int par, int hb, int sb, int bq) {
+        const float16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const int t0 = 2 * hb, t1 = 2 * hb + 1;
+        const float df[2] = {scale_of(sb, 0, bq), scale_of(sb, 1, bq)};
+        half8 b0[2], b1[2]; // the block's weight fragments serve both row tiles
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            b0[j] = *reinterpret_cast<const half8 *>(lds + par * BSTAGE + (b_rd ^ (t0 * 16)) + j * 32 * 64);
+            b1[j] = *reinterpret_cast<const half8 *>(lds + par * BSTAGE + (b_rd ^ (t1 * 16)) + j * 32 * 64);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) { // one row tile's two sums at a time: registers
+            const half8 a0 = *reinterpret_cast<const half8 *>(lds + as + (a_rd ^ (t0 * 16)) + i * 32 * 64);
+            const half8 a1 = *reinterpret_cast<const half8 *>(lds + as + (a_rd ^ (t1 * 16)) + i * 32 * 64);
+            float16v S[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++) S[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b0[j], zero, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 2; j++) S[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1[j], S[j], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(S[j][r], df[j], acc[i][j][r]);
+        }
+    };
+    auto multiply_min = [&](int sb) {
+        const half2v ws2 = {(_Float16)WSCALE, (_Float16)WSCALE}, wd2 = {(_Float16)(16.0f * WSCALE), (_Float16)(16.0f * WSCALE)};
+        half8 bm[2], bd[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            uint32_t om[4], od[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) { // blocks 2 q, 2 q + 1: the (d, m) records' upper halves are the minimums
+                // (read as a plain vector: a read through HIP's uint2 made the compiler wait for every load in flight)
+                typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                const u32x2 r2 = *reinterpret_cast<const u32x2 *>(rlane + (sb & 1) * RECB + j * 32 * 16 * RV + q * 8);
+                const uint32_t r0 = r2[0], r1 = r2[1];
+                const uint32_t ms = (r0 >> 16) | (r1 & 0xFFFF0000u), dsc = (r0 & 0xFFFFu) | (r1 << 16);
+                const half2v vm = __builtin_bit_cast(half2v, ms) * ws2, vd = __builtin_bit_cast(half2v, dsc) * wd2;
+                om[q] = __builtin_bit_cast(uint32_t, vm);
+                od[q] = __builtin_bit_cast(uint32_t, vd);
+            }
+            bm[j] = __builtin_bit_cast(half8, u32x4{om[0], om[1], om[2], om[3]});
+            bd[j] = __builtin_bit_cast(half8, u32x4{od[0], od[1], od[2], od[3]});
+        }
+        // the block sums are stored times XSUM_SCALE and these operands times WSCALE: the accumulators hold the result times
+        // WSCALE * XSUM_SCALE, and the main term scales its sums to match (scale_of)
+        // (added by the vector ALU like the main term: accumulators that the matrix pipe also wrote would be kept twice)
+        const float16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            float16v S[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++) S[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bm[j], zero, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 2; j++) S[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bd[j], S[j], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] += S[j][r];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // Steps g = 0 .. T - 1 in groups of four (a superblock).  Step g multiplies x stage g % 3 with weight stage g & 1,
+    // brings the x tile of step g + 2 into its stage, converts the weights of step g + 1 into the other weight stage
+    // and requests those of step g + 3; the first step of a group also requests the scale records of the next
+    // superblock, the third this one's block sums.  Every wave issues the same loads in the same order, so that the
+    // wait in front of a barrier (for the x tile of step g + 1, requested a step ago) can leave the younger requests in
+    // flight.
+    Raw buf[4]; // the blocks of steps g .. g + 3, at g % 4 ..
+    load_x(0, 0);
+    load_x(1, 1);
+    fetch(0, buf[0]);
+    fetch(1, buf[1]);
+    fetch(2, buf[2]);
+    fetch_records(0);
+    convert(buf[0], 0, 0);
+    convert(buf[0], 1, 0);
+    wait_vm_and_lds<0>();
+    lds_barrier();
+    int g3 = 0;
+    for (int sb = 0; sb < nsb; sb++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int g = 4 * sb + i;
+            const int as = g3 * ASTAGE, xs = (g3 == 0 ? 2 : g3 - 1);
+            // the order of the requests: the weight blocks first, so that the wait at the end of the next step, which
+            // lets that step's x tile and what follows it stay out, covers them
+            if (WITH_MIN && i == 2) { // this superblock's block sums, for the end of the next step: ahead of the step's other
+                fetch_sums(sb);       // requests, so that the wait at its end covers them
+                asm volatile("" ::: "memory");
+            }
+            fetch(g + 3, buf[(i + 3) & 3]);
+            load_x(g + 2, xs);
+            if (i == 0) fetch_records(sb + 1);
+            // (past the last step the conversion writes a stage that nobody reads)
+#pragma unroll
+            for (int hb = 0; hb < 2; hb++) {
+                multiply_block(as, i & 1, hb, sb, 2 * i + hb);
+                convert(buf[(i + 1) & 3], hb, (i + 1) & 1);
+            }
+            if (WITH_MIN && i == 3) multiply_min(sb);
+            // younger than the x tile of step g + 1 (requested a step ago): what followed it in that step, and this step's
+            if (i == 0) wait_vm_and_lds<F + XL + ML>();
+            else if (i == 1) wait_vm_and_lds<ML + F + XL>();
+            else wait_vm_and_lds<F + XL>();
+            lds_barrier();
+            g3 = g3 == 2 ? 0 : g3 + 1;
+        }
+    }
+    wait_vm_and_lds<0>(); // nothing of this workgroup may still be on its way into LDS when it ends
+    // D layout: lane -> column li; register r -> row 8 * (r / 4) + 4 * (lane / 32) + r % 4
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int gn = n0 + wn + j * 32 + li;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int gm = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (gm < a.m && gn < a.n) {
+                    if (!a.pair) {
+                        if (a.ypart) a.ypart[((size_t)blockIdx.y * a.m + gm) * a.n + gn] = acc[i][j][r];
+                        else a.y[(size_t)gm * a.n + gn] = acc[i][j][r] * (a.rowscale[gm] * (1.0f / ASCALE));
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) { // pair mode: an even row and the next hold the two parts of activation row gm / 2
+                const int gm = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (a.pair && gm < a.m && gn < a.n) {
+                    const size_t t = (size_t)(gm >> 1);
+                    const float v = acc[i][j][r] + acc[i][j][r + 1];
+                    if (a.ypart) {
+                        a.ypart[((size_t)blockIdx.y * (a.m >> 1) + t) * a.n + gn] = v;
+                    } else {
+                        float out = v * (a.rowscale[gm] * (1.0f / ASCALE));
+                        if (a.bias) out += a.bias[gn];
+                        if (a.resid) out += a.resid[t * a.n + gn];
+                        a.y[t * a.n + gn] = out;
+                    }
+                }
+            }
+        }
+}
+
 // What the Q4_K kernel wants from the x pre-pass besides the scaled f16 rows: elements 1 and 2 of every group of four
 // exchanged, and the sums of every 32 consecutive (scaled, f16) elements as f16 pairs hi + lo: 32 halfs per superblock,
 // [hi of its 8 sub-blocks | the same | lo | zeros] (NULL xs3: plain rows for the other kernels).
@@ -842,7 +1132,6 @@ struct XSums {
     _Float16 *xs3;
     int pitch; // halfs per row: 32 per superblock and 32 or 64 zeros, see xs3_pitch
 };
-constexpr float XSUM_SCALE = 1.0f / 64.0f; // the sums are stored times this
 // one or two superblocks of zeros end a row: the last step of the minimum term may look one superblock past the end
 __host__ __device__ inline int xs3_pitch(int64_t k) { return (int)(((k >> 8) + 2) & ~(int64_t)1) * 32; }
 
@@ -1090,6 +1379,7 @@ int reserve_scratch(axq_ctx *ctx, size_t need) {
 struct GemmPlan {
     int splits, steps_per_split, wm;
     bool q4k;     // the one-MFMA Q4_K kernel (gemm_q4k_kernel) instead of the two-plane kernel
+    bool q5;      // the one-MFMA Q5_0 / Q5_1 kernel (gemm_q5_kernel)
     size_t xh_bytes, rs_bytes, part_bytes, xs3_bytes;
 };
 
@@ -1098,6 +1388,13 @@ struct GemmPlan {
 bool q4k_route(const axq_weight *w, bool in_regs_only) {
     static const bool off = getenv("AXQ_GEMM_Q4K") && getenv("AXQ_GEMM_Q4K")[0] == '0'; // development knob
     return !off && w->type == AXQ_Q4_K && w->k % 256 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
+}
+
+// Whether gemm_q5_kernel takes this call (256-row tiles only: fewer rows stay on the two-plane kernel).
+bool q5_route(const axq_weight *w, int m, bool in_regs_only) {
+    static const bool off = getenv("AXQ_GEMM_Q5") && getenv("AXQ_GEMM_Q5")[0] == '0'; // development knob
+    return !off && (w->type == AXQ_Q5_0 || w->type == AXQ_Q5_1) && w->k % 256 == 0 && m > 128 && w->meta_pitch % 16 == 0 &&
+           (!in_regs_only || w->k <= 16 * 256 * 4);
 }
 
 // Split K when the output tiles alone leave most compute units idle (short prompts): the splits' partial sums go
@@ -1116,6 +1413,7 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, bool f32_rows, size_t ex
     const int bm = bm_knob ? bm_knob : (m > (route_q4k ? 256 : 128) ? 256 : 128);
     p->wm = bm / 128;
     p->q4k = route_q4k;
+    p->q5 = bm == 256 && q5_route(w, m, f32_rows);
     const int bn = p->q4k ? QBN : BN;
     const long tiles = (long)((w->n_rows + bn - 1) / bn) * ((m + bm - 1) / bm);
     const int ksteps = (int)(w->k / BK), cus = ctx->prop.multiProcessorCount;
@@ -1124,21 +1422,21 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, bool f32_rows, size_t ex
     if (splits > ksteps / 4) splits = ksteps / 4;
     if (splits < 2 || w->n_rows % 4 != 0) splits = 1;
     p->steps_per_split = (ksteps + splits - 1) / splits;
-    if (p->q4k) p->steps_per_split = (p->steps_per_split + 3) & ~3; // whole superblocks per split
+    if (p->q4k || p->q5) p->steps_per_split = (p->steps_per_split + 3) & ~3; // whole superblocks per split
     p->splits = (ksteps + p->steps_per_split - 1) / p->steps_per_split;
     // the Q4_K kernel reads whole row tiles without a clamp: its x buffers have rows up to a multiple of the tile
-    const size_t mpad = p->q4k ? (size_t)(m + bm - 1) / bm * bm : (size_t)m;
+    const size_t mpad = (p->q4k || p->q5) ? (size_t)(m + bm - 1) / bm * bm : (size_t)m;
     p->xh_bytes = axq_align_up(mpad * (size_t)w->k * 2, 256);
     p->rs_bytes = axq_align_up((size_t)m * 4, 256);
     p->part_bytes = axq_align_up(p->splits > 1 ? (size_t)p->splits * m * (size_t)w->n_rows * 4 : 0, 256);
-    p->xs3_bytes = axq_align_up(p->q4k ? mpad * (size_t)xs3_pitch(w->k) * 2 : 0, 256);
+    p->xs3_bytes = axq_align_up((p->q4k || p->q5) ? mpad * (size_t)xs3_pitch(w->k) * 2 : 0, 256);
     return reserve_scratch(ctx, p->xh_bytes + p->rs_bytes + p->part_bytes + p->xs3_bytes + extra);
 }
 
 // What the x pre-pass has to write besides the rows (nothing for the two-plane kernel).
 XSums plan_sums(axq_ctx *ctx, const axq_weight *w, const GemmPlan &p) {
     XSums xs = {nullptr, 0};
-    if (p.q4k) {
+    if (p.q4k || p.q5) {
         xs.xs3 = reinterpret_cast<_Float16 *>(reinterpret_cast<uint8_t *>(ctx->gemm_scratch) + p.xh_bytes + p.rs_bytes + p.part_bytes);
         xs.pitch = xs3_pitch(w->k);
     }
@@ -1169,6 +1467,27 @@ int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits) {
     return AXQ_OK;
 }
 
+int launch_gemm_q5(axq_ctx *ctx, GemmArgs a, int splits, bool with_min) {
+    static std::atomic<uint64_t> lds_allowed[2]; // per kernel: a bit per device
+    const unsigned tiles = (unsigned)(((a.n + PBN - 1) / PBN) * ((a.m + 255) / 256));
+    const dim3 grid(tiles, (unsigned)splits);
+    const size_t lds = (size_t)(3 * 256 * 64 + 2 * PBN * 64) * sizeof(_Float16) + 2 * PBN * 32; // three x stages, two weight stages, scale records
+    int rc;
+    if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q5_kernel<true>), lds_allowed[1], (int)lds))) return rc;
+    if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q5_kernel<false>), lds_allowed[0], (int)lds))) return rc;
+    if (with_min) gemm_q5_kernel<true><<<grid, 512, lds, ctx->stream>>>(a);
+    else gemm_q5_kernel<false><<<grid, 512, lds, ctx->stream>>>(a);
+    AXQ_LAUNCH_CHECK(ctx, "gemm_q5_kernel");
+    if (splits > 1) {
+        const int rows = a.pair ? a.m / 2 : a.m;
+        const size_t total4 = (size_t)rows * a.n / 4;
+        gemm_reduce_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, ctx->stream>>>(a.ypart, a.rowscale, rows, a.n, splits,
+                                                                                    1.0f / (WSCALE * XSUM_SCALE), a.pair ? 2 : 1, a.bias, a.resid, a.y);
+        AXQ_LAUNCH_CHECK(ctx, "gemm_reduce_kernel");
+    }
+    return AXQ_OK;
+}
+
 // The GEMM proper over activations that already sit in scratch as scaled f16 rows.
 int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float *y, bool pair = false, const float *bias = nullptr,
              const float *resid = nullptr) {
@@ -1184,6 +1503,7 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     const XSums xs = plan_sums(ctx, w, p);
     a.xs3 = xs.xs3; a.xs3_pitch = xs.pitch;
     if (p.q4k) return launch_gemm_q4k(ctx, a, p.splits);
+    if (p.q5) return launch_gemm_q5(ctx, a, p.splits, w->type == AXQ_Q5_1);
     switch (w->type) {
     case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);
     case AXQ_Q4_0: return launch_gemm<GQ4x<false>>(ctx, a, p.splits);
