@@ -836,7 +836,7 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// Q5_0 / Q5_1: one MFMA per product, the block's scale applied by the vector ALU.
+// Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q8_0 (blocks of 32): one MFMA per product, the block's scale applied by the vector ALU.
 //
 // w = d * (q - 16) (Q5_0) or d * q + m (Q5_1) with a five-bit code q and f16 d (and m) per block of 32.  The B operand
 // is the centred code q - 16 itself, an integer that f16 holds exactly: the two MFMAs of a block (32 k) start from
@@ -863,14 +863,15 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 constexpr int PBN = 128; // output columns (weight rows) per workgroup
 constexpr float XSUM_SCALE = 1.0f / 64.0f; // the x pre-pass stores the block sums times this
 
-template <bool WITH_MIN>
-__global__ void __launch_bounds__(512) gemm_q5_kernel(GemmArgs a) {
+template <int BITS, bool WITH_MIN>
+__global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
     typedef _Float16 half2v __attribute__((ext_vector_type(2)));
     constexpr int BM = 256, NW = 8, AROWS = BM / NW, XL = AROWS / 8;
     constexpr int ASTAGE = BM * 64, BSTAGE = PBN * 64, BOFF = 3 * ASTAGE; // halfs
-    constexpr int F = 2;                   // loads of a weight request: codes, fifth bits
+    constexpr int F = BITS == 5 ? 2 : 1;   // loads of a weight request: codes (and fifth bits)
+    constexpr int CENTER = BITS == 5 ? 16 : BITS == 4 ? 8 : 128; // the codes go in centred (Q5_0's, Q4_0's and Q8_0's own form)
     constexpr int ML = 1;                  // per superblock: this wave's kilobyte of scale records
-    constexpr float OFF = 1040.0f;         // 0x6400 | q is 1024 + q; the codes go in centred, q - 16 (Q5_0's own form)
+    constexpr float OFF = 1024.0f + CENTER; // 0x6400 | q is 1024 + q
     constexpr float ASCALE = WSCALE * XSUM_SCALE; // the accumulators hold the result times this
     extern __shared__ _Float16 lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -900,29 +901,45 @@ __global__ void __launch_bounds__(512) gemm_q5_kernel(GemmArgs a) {
     // ---- weights: this thread's half block (16 weights) of every step
     const int wrow = tid & 127, bis = tid >> 8, half = (tid >> 7) & 1; // row of the tile; which of the step's two blocks; which half of it
     const int crow = n0 + wrow < a.n ? n0 + wrow : a.n - 1;
-    const uint8_t *cp = a.codes + (size_t)crow * a.codes_pitch, *qp = a.qh + (size_t)crow * a.qh_pitch;
+    const uint8_t *cp = a.codes + (size_t)crow * a.codes_pitch, *qp = BITS == 5 ? a.qh + (size_t)crow * a.qh_pitch : nullptr;
     struct Raw { u32x4 q; uint32_t qh; };
-    auto fetch = [&](int step, Raw &r) { // the thread's block of a step (both halves fetch all of it: the nibbles interleave)
+    // the thread's block of a step: 16 bytes of nibbles (Q5: both halves fetch all of them, they interleave), or its own
+    // 16 of the block's 32 bytes (Q8_0)
+    auto fetch = [&](int step, Raw &r) {
         step = step < T ? step : T - 1;
         const size_t blk = (size_t)(kbeg + step) * 2 + bis;
-        r.q = *reinterpret_cast<const u32x4 *>(cp + blk * 16);
-        r.qh = *reinterpret_cast<const uint32_t *>(qp + blk * 4);
+        r.q = *reinterpret_cast<const u32x4 *>(BITS == 8 ? cp + blk * 32 + half * 16 : cp + blk * 16);
+        if (BITS == 5) r.qh = *reinterpret_cast<const uint32_t *>(qp + blk * 4);
         asm volatile("" ::: "memory");
     };
     const int b_wr = wrow * 64; // the thread's row in a weight plane; chunk ch of it lies at (ch ^ ((wrow / 2) & 7)) * 8
     const int b_sw = (wrow >> 1) & 7;
-    // chunk 2 half + cc (cc = 0, 1: eight weights) of the block in `r` -> weight stage `stage`: the low nibbles of a block
-    // are its elements 0..15, the high nibbles 16..31
+    // chunk c = 2 half + cc (cc = 0, 1: elements 8 c .. 8 c + 7) of the block in `r` -> weight stage `stage`, as pairs of
+    // codes in the two halves of a dword, in the order [e0, e2, e1, e3, e4, e6, e5, e7]
     auto convert = [&](const Raw &r, int cc, int stage) {
-        const uint32_t d0 = cc ? r.q[2] : r.q[0], d1 = cc ? r.q[3] : r.q[1];
-        const int sh = half * 4, c = 2 * half + cc;
-        uint32_t pr[4] = {(d0 >> sh) & 0x000F000Fu, (d0 >> (sh + 8)) & 0x000F000Fu, (d1 >> sh) & 0x000F000Fu, (d1 >> (sh + 8)) & 0x000F000Fu};
-        // bits b0..b3 of `four` times (2^4 + 2^18): b0 lands on bit 4 and b2 on bit 20 (of the pair e, e + 2), nothing else does
-        const uint32_t eight = (r.qh >> (8 * c)) & 0xFFu;
-        pr[0] |= ((eight & 0xFu) * 0x40010u) & 0x00100010u;
-        pr[1] |= (((eight >> 1) & 0x7u) * 0x40010u) & 0x00100010u;
-        pr[2] |= ((eight >> 4) * 0x40010u) & 0x00100010u;
-        pr[3] |= ((eight >> 5) * 0x40010u) & 0x00100010u;
+        const int c = 2 * half + cc;
+        uint32_t pr[4];
+        if (BITS == 5) { // GGUF: byte j = elements j (low nibble) and j + 16 (high); qh bit e = bit 4 of element e
+            const uint32_t d0 = cc ? r.q[2] : r.q[0], d1 = cc ? r.q[3] : r.q[1];
+            const int sh = half * 4;
+            pr[0] = (d0 >> sh) & 0x000F000Fu; pr[1] = (d0 >> (sh + 8)) & 0x000F000Fu;
+            pr[2] = (d1 >> sh) & 0x000F000Fu; pr[3] = (d1 >> (sh + 8)) & 0x000F000Fu;
+            // bits b0..b3 of `four` times (2^4 + 2^18): b0 lands on bit 4 and b2 on bit 20 (of the pair e, e + 2), nothing else does
+            const uint32_t eight = (r.qh >> (8 * c)) & 0xFFu;
+            pr[0] |= ((eight & 0xFu) * 0x40010u) & 0x00100010u;
+            pr[1] |= (((eight >> 1) & 0x7u) * 0x40010u) & 0x00100010u;
+            pr[2] |= ((eight >> 4) * 0x40010u) & 0x00100010u;
+            pr[3] |= ((eight >> 5) * 0x40010u) & 0x00100010u;
+        } else if (BITS == 4) { // reference nibble order: byte i = elements 2 i (low), 2 i + 1 (high): dword c is the chunk
+            const uint32_t w = half ? (cc ? r.q[3] : r.q[2]) : (cc ? r.q[1] : r.q[0]);
+            const uint32_t p4 = __builtin_amdgcn_perm(w, w, 0x03010200u); // bytes 0, 2, 1, 3: a half dword = two neighbours
+            pr[0] = p4 & 0x000F000Fu; pr[1] = (p4 >> 4) & 0x000F000Fu;
+            pr[2] = (p4 >> 8) & 0x000F000Fu; pr[3] = (p4 >> 12) & 0x000F000Fu;
+        } else { // signed bytes in element order, as unsigned ones (+ 128)
+            const uint32_t x0 = (cc ? r.q[2] : r.q[0]) ^ 0x80808080u, x1 = (cc ? r.q[3] : r.q[1]) ^ 0x80808080u;
+            pr[0] = x0 & 0x00FF00FFu; pr[1] = (x0 >> 8) & 0x00FF00FFu;
+            pr[2] = x1 & 0x00FF00FFu; pr[3] = (x1 >> 8) & 0x00FF00FFu;
+        }
         const half2v off2 = {(_Float16)OFF, (_Float16)OFF};
         uint32_t oh[4];
 #pragma unroll
@@ -1004,7 +1021,7 @@ __global__ void __launch_bounds__(512) gemm_q5_kernel(GemmArgs a) {
         }
     };
     auto multiply_min = [&](int sb) {
-        const half2v ws2 = {(_Float16)WSCALE, (_Float16)WSCALE}, wd2 = {(_Float16)(16.0f * WSCALE), (_Float16)(16.0f * WSCALE)};
+        const half2v ws2 = {(_Float16)WSCALE, (_Float16)WSCALE}, wd2 = {(_Float16)(CENTER * WSCALE), (_Float16)(CENTER * WSCALE)};
         half8 bm[2], bd[2];
 #pragma unroll
         for (int j = 0; j < 2; j++) {
@@ -1379,7 +1396,7 @@ int reserve_scratch(axq_ctx *ctx, size_t need) {
 struct GemmPlan {
     int splits, steps_per_split, wm;
     bool q4k;     // the one-MFMA Q4_K kernel (gemm_q4k_kernel) instead of the two-plane kernel
-    bool q5;      // the one-MFMA Q5_0 / Q5_1 kernel (gemm_q5_kernel)
+    bool q5;      // the one-MFMA kernel of the types with blocks of 32 (gemm_blk32_kernel)
     size_t xh_bytes, rs_bytes, part_bytes, xs3_bytes;
 };
 
@@ -1390,11 +1407,11 @@ bool q4k_route(const axq_weight *w, bool in_regs_only) {
     return !off && w->type == AXQ_Q4_K && w->k % 256 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
 }
 
-// Whether gemm_q5_kernel takes this call (256-row tiles only: fewer rows stay on the two-plane kernel).
+// Whether gemm_blk32_kernel takes this call (256-row tiles only: fewer rows stay on the two-plane kernel).
 bool q5_route(const axq_weight *w, int m, bool in_regs_only) {
-    static const bool off = getenv("AXQ_GEMM_Q5") && getenv("AXQ_GEMM_Q5")[0] == '0'; // development knob
-    return !off && (w->type == AXQ_Q5_0 || w->type == AXQ_Q5_1) && w->k % 256 == 0 && m > 128 && w->meta_pitch % 16 == 0 &&
-           (!in_regs_only || w->k <= 16 * 256 * 4);
+    static const bool off = getenv("AXQ_GEMM_BLK32") && getenv("AXQ_GEMM_BLK32")[0] == '0'; // development knob
+    const bool type_ok = w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q5_0 || w->type == AXQ_Q5_1 || w->type == AXQ_Q8_0;
+    return !off && type_ok && w->k % 256 == 0 && m > 128 && w->meta_pitch % 16 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
 }
 
 // Split K when the output tiles alone leave most compute units idle (short prompts): the splits' partial sums go
@@ -1467,17 +1484,29 @@ int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits) {
     return AXQ_OK;
 }
 
-int launch_gemm_q5(axq_ctx *ctx, GemmArgs a, int splits, bool with_min) {
-    static std::atomic<uint64_t> lds_allowed[2]; // per kernel: a bit per device
+template <int BITS, bool WITH_MIN>
+int launch_blk32(axq_ctx *ctx, const GemmArgs &a, dim3 grid, size_t lds) {
+    static std::atomic<uint64_t> lds_allowed{0}; // a bit per device
+    int rc;
+    if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_blk32_kernel<BITS, WITH_MIN>), lds_allowed, lds))) return rc;
+    gemm_blk32_kernel<BITS, WITH_MIN><<<grid, 512, lds, ctx->stream>>>(a);
+    return AXQ_OK;
+}
+
+int launch_gemm_q5(axq_ctx *ctx, GemmArgs a, int splits, int type) {
     const unsigned tiles = (unsigned)(((a.n + PBN - 1) / PBN) * ((a.m + 255) / 256));
     const dim3 grid(tiles, (unsigned)splits);
     const size_t lds = (size_t)(3 * 256 * 64 + 2 * PBN * 64) * sizeof(_Float16) + 2 * PBN * 32; // three x stages, two weight stages, scale records
     int rc;
-    if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q5_kernel<true>), lds_allowed[1], (int)lds))) return rc;
-    if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q5_kernel<false>), lds_allowed[0], (int)lds))) return rc;
-    if (with_min) gemm_q5_kernel<true><<<grid, 512, lds, ctx->stream>>>(a);
-    else gemm_q5_kernel<false><<<grid, 512, lds, ctx->stream>>>(a);
-    AXQ_LAUNCH_CHECK(ctx, "gemm_q5_kernel");
+    switch (type) {
+    case AXQ_Q4_0: rc = launch_blk32<4, false>(ctx, a, grid, lds); break;
+    case AXQ_Q4_1: rc = launch_blk32<4, true>(ctx, a, grid, lds); break;
+    case AXQ_Q5_0: rc = launch_blk32<5, false>(ctx, a, grid, lds); break;
+    case AXQ_Q5_1: rc = launch_blk32<5, true>(ctx, a, grid, lds); break;
+    default: rc = launch_blk32<8, false>(ctx, a, grid, lds); break;
+    }
+    if (rc) return rc;
+    AXQ_LAUNCH_CHECK(ctx, "gemm_blk32_kernel");
     if (splits > 1) {
         const int rows = a.pair ? a.m / 2 : a.m;
         const size_t total4 = (size_t)rows * a.n / 4;
@@ -1503,7 +1532,7 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     const XSums xs = plan_sums(ctx, w, p);
     a.xs3 = xs.xs3; a.xs3_pitch = xs.pitch;
     if (p.q4k) return launch_gemm_q4k(ctx, a, p.splits);
-    if (p.q5) return launch_gemm_q5(ctx, a, p.splits, w->type == AXQ_Q5_1);
+    if (p.q5) return launch_gemm_q5(ctx, a, p.splits, w->type);
     switch (w->type) {
     case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);
     case AXQ_Q4_0: return launch_gemm<GQ4x<false>>(ctx, a, p.splits);
