@@ -863,10 +863,11 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 constexpr int PBN = 128; // output columns (weight rows) per workgroup
 constexpr float XSUM_SCALE = 1.0f / 64.0f; // the x pre-pass stores the block sums times this
 
-template <int BITS, bool WITH_MIN>
+template <int BITS, bool WITH_MIN, int BM>
 __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
     typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-    constexpr int BM = 256, NW = 8, AROWS = BM / NW, XL = AROWS / 8;
+    constexpr int NW = 8, AROWS = BM / NW, XL = AROWS / 8; // BM = 256 or 128 rows of x per workgroup
+    constexpr int MI = BM / 128;                           // MFMA tiles of a wave along M: the waves lie 4 x 2, (32 MI) x 64 each
     constexpr int ASTAGE = BM * 64, BSTAGE = PBN * 64, BOFF = 3 * ASTAGE; // halfs
     constexpr int F = BITS == 5 ? 2 : 1;   // loads of a weight request: codes (and fifth bits)
     constexpr int CENTER = BITS == 5 ? 16 : BITS == 4 ? 8 : 128; // the codes go in centred (Q5_0's, Q4_0's and Q8_0's own form)
@@ -953,13 +954,13 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
     };
 
     // ---- multiplier side
-    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 64;
     const int li = lane & 31, hh = lane >> 5;
     const int sw = ((hh ^ (li >> 1)) & 7) * 8;
     const int a_rd = (wm + li) * 64 + sw, b_rd = BOFF + (wn + li) * 64 + sw;
-    float16v acc[2][2];
+    float16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -981,11 +982,11 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
         __builtin_amdgcn_global_load_lds((gbl_void *)(rsrc + (size_t)sb * (16 * RV)), (lds_void *)(rec_lds + (sb & 1) * RECB + rc0 * 16 * RV), 16, 0, 0);
         asm volatile("" ::: "memory");
     };
-    u32x4 mx[2];
+    u32x4 mx[MI];
     const uint8_t *x3p = reinterpret_cast<const uint8_t *>(a.xs3 + (size_t)(m0 + wm + li) * a.xs3_pitch + (size_t)(kbeg >> 2) * 32 + hh * 16);
     auto fetch_sums = [&](int sb) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) mx[i] = *reinterpret_cast<const u32x4 *>(x3p + ((size_t)i * 32 * a.xs3_pitch + (size_t)sb * 32) * 2);
+        for (int i = 0; i < MI; i++) mx[i] = *reinterpret_cast<const u32x4 *>(x3p + ((size_t)i * 32 * a.xs3_pitch + (size_t)sb * 32) * 2);
     };
     // d of block bq (0..7) of superblock sb, column j of this lane, times WSCALE
     const uint8_t *rlane = rec_lds + (wn + li) * 16 * RV;
@@ -1006,7 +1007,7 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
             b1[j] = *reinterpret_cast<const half8 *>(lds + par * BSTAGE + (b_rd ^ (t1 * 16)) + j * 32 * 64);
         }
 #pragma unroll
-        for (int i = 0; i < 2; i++) { // one row tile's two sums at a time: registers
+        for (int i = 0; i < MI; i++) { // one row tile's two sums at a time: registers
             const half8 a0 = *reinterpret_cast<const half8 *>(lds + as + (a_rd ^ (t0 * 16)) + i * 32 * 64);
             const half8 a1 = *reinterpret_cast<const half8 *>(lds + as + (a_rd ^ (t1 * 16)) + i * 32 * 64);
             float16v S[2];
@@ -1045,7 +1046,7 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
         // (added by the vector ALU like the main term: accumulators that the matrix pipe also wrote would be kept twice)
         const float16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < MI; i++) {
             float16v S[2];
 #pragma unroll
             for (int j = 0; j < 2; j++) S[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bm[j], zero, 0, 0, 0);
@@ -1109,7 +1110,7 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
     wait_vm_and_lds<0>(); // nothing of this workgroup may still be on its way into LDS when it ends
     // D layout: lane -> column li; register r -> row 8 * (r / 4) + 4 * (lane / 32) + r % 4
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int gn = n0 + wn + j * 32 + li;
@@ -1407,11 +1408,12 @@ bool q4k_route(const axq_weight *w, bool in_regs_only) {
     return !off && w->type == AXQ_Q4_K && w->k % 256 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
 }
 
-// Whether gemm_blk32_kernel takes this call (256-row tiles only: fewer rows stay on the two-plane kernel).
+// Whether gemm_blk32_kernel takes this call.
 bool q5_route(const axq_weight *w, int m, bool in_regs_only) {
     static const bool off = getenv("AXQ_GEMM_BLK32") && getenv("AXQ_GEMM_BLK32")[0] == '0'; // development knob
     const bool type_ok = w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q5_0 || w->type == AXQ_Q5_1 || w->type == AXQ_Q8_0;
-    return !off && type_ok && w->k % 256 == 0 && m > 128 && w->meta_pitch % 16 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
+    static const int min_rows = getenv("AXQ_GEMM_BLK32_MIN_ROWS") ? atoi(getenv("AXQ_GEMM_BLK32_MIN_ROWS")) : 1; // development knob
+    return !off && type_ok && w->k % 256 == 0 && m >= min_rows && w->meta_pitch % 16 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
 }
 
 // Split K when the output tiles alone leave most compute units idle (short prompts): the splits' partial sums go
@@ -1430,7 +1432,7 @@ int plan_gemm(axq_ctx *ctx, const axq_weight *w, int m, bool f32_rows, size_t ex
     const int bm = bm_knob ? bm_knob : (m > (route_q4k ? 256 : 128) ? 256 : 128);
     p->wm = bm / 128;
     p->q4k = route_q4k;
-    p->q5 = bm == 256 && q5_route(w, m, f32_rows);
+    p->q5 = q5_route(w, m, f32_rows);
     const int bn = p->q4k ? QBN : BN;
     const long tiles = (long)((w->n_rows + bn - 1) / bn) * ((m + bm - 1) / bm);
     const int ksteps = (int)(w->k / BK), cus = ctx->prop.multiProcessorCount;
@@ -1486,17 +1488,23 @@ int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits) {
 
 template <int BITS, bool WITH_MIN>
 int launch_blk32(axq_ctx *ctx, const GemmArgs &a, dim3 grid, size_t lds) {
-    static std::atomic<uint64_t> lds_allowed{0}; // a bit per device
+    static std::atomic<uint64_t> lds_allowed[2]; // per kernel: a bit per device
     int rc;
-    if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_blk32_kernel<BITS, WITH_MIN>), lds_allowed, lds))) return rc;
-    gemm_blk32_kernel<BITS, WITH_MIN><<<grid, 512, lds, ctx->stream>>>(a);
+    if (a.wm == 2) {
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_blk32_kernel<BITS, WITH_MIN, 256>), lds_allowed[1], lds))) return rc;
+        gemm_blk32_kernel<BITS, WITH_MIN, 256><<<grid, 512, lds, ctx->stream>>>(a);
+    } else {
+        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_blk32_kernel<BITS, WITH_MIN, 128>), lds_allowed[0], lds))) return rc;
+        gemm_blk32_kernel<BITS, WITH_MIN, 128><<<grid, 512, lds, ctx->stream>>>(a);
+    }
     return AXQ_OK;
 }
 
 int launch_gemm_q5(axq_ctx *ctx, GemmArgs a, int splits, int type) {
-    const unsigned tiles = (unsigned)(((a.n + PBN - 1) / PBN) * ((a.m + 255) / 256));
+    const int bm = 128 * a.wm;
+    const unsigned tiles = (unsigned)(((a.n + PBN - 1) / PBN) * ((a.m + bm - 1) / bm));
     const dim3 grid(tiles, (unsigned)splits);
-    const size_t lds = (size_t)(3 * 256 * 64 + 2 * PBN * 64) * sizeof(_Float16) + 2 * PBN * 32; // three x stages, two weight stages, scale records
+    const size_t lds = (size_t)(3 * bm * 64 + 2 * PBN * 64) * sizeof(_Float16) + 2 * PBN * 32; // three x stages, two weight stages, scale records
     int rc;
     switch (type) {
     case AXQ_Q4_0: rc = launch_blk32<4, false>(ctx, a, grid, lds); break;
