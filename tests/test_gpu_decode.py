@@ -218,7 +218,11 @@ def _prompt_at_once(ctx, over, qtype, n_first, n_prompt):
             a, b = one.kv(layer, which)[:, :n], gpu.kv(layer, which)[:, :n]
             af, bf = a.view(np.float16).astype(np.float64), b.view(np.float16).astype(np.float64)
             ulp = np.maximum(np.abs(af) * 2.0 ** -10, 5e-5 * np.abs(af).max())  # as in the cache test above
-            bad = np.argwhere(np.abs(af - bf) > ulp)
+            # The first layer's cache sees the same inputs on both paths: f32 noise flips an f16 rounding at most.  Every
+            # flipped rounding then reaches the layers above as a difference of 1e-4 of the hidden state, and the two
+            # paths (GEMV on integer limbs, GEMM on f16 pairs) round differently, so the allowance grows by one unit per
+            # layer; the logits at the end are held to the decode bar against the oracle above.
+            bad = np.argwhere(np.abs(af - bf) > (1 + layer) * ulp)
             assert bad.size == 0, (layer, which, bad[0])
     # the two paths go on alike: a few more steps, one token at a time
     tok = c_next
