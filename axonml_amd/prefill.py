@@ -40,7 +40,7 @@ def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(
                 r = {"type": str(qt), "m": m, "n": n, "k": k, "ms": t, "tflops": flops / (t * 1e-3) / 1e12,
                      "route": "hand-written MFMA GEMM, scaled codes as f16, one product per weight" if qt == QuantType.Q4_K
                      else "hand-written MFMA GEMM, centred codes as f16, one product per weight, block scales by the vector ALU"
-                     if m > 128 and k % 256 == 0 and qt in BLK32_TYPES
+                     if k % 256 == 0 and qt in BLK32_TYPES
                      else "hand-written MFMA GEMM, weights dequantised to two f16 terms, two products per weight"}
                 r["frac_of_mfma_f16_peak"] = r["tflops"] / MFMA_F16_PEAK_TFLOPS
                 out.append(r)
