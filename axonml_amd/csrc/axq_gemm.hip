@@ -838,27 +838,28 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 // ---------------------------------------------------------------------------
 // Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q8_0 (blocks of 32): one MFMA per product, the block's scale applied by the vector ALU.
 //
-// w = d * (q - 16) (Q5_0) or d * q + m (Q5_1) with a five-bit code q and f16 d (and m) per block of 32.  The B operand
-// is the centred code q - 16 itself, an integer that f16 holds exactly: the two MFMAs of a block (32 k) start from
-// zero, so their result is the block's sum of (q - 16) * x, exact in f32 to within the accumulation, and every lane
-// then adds it, times the d of its column and block, into its accumulators (a lane of the 32 x 32 MFMA output owns
-// one column): sixteen v_fma per tile and block where gemm_kernel pays a second MFMA per product and about ten
-// vector-ALU instructions per weight for the dequantisation and the high/low split.  Converting costs two instructions
-// per pair of weights: the code pairs come out of the packed nibbles two at a time with one mask each, the fifth bits
-// out of qh four at a time with one multiplication, 0x6400 | q is the f16 number 1024 + q, and one packed subtraction
-// of 1040 centres it.  x is stored with elements 1 and 2 of every four exchanged, as for the Q4_K kernel, which is the
-// order the masks produce.
-// Q5_1 goes in as d * (q - 16) + (m + 16 d): the first sum is then as well conditioned as the weights themselves (with
-// q as it is, 0..31, two sums three times the size of the result would cancel in f32).  The second,
-// sum_b (m + 16 d)[n, b] * (sum of x over block b), goes through the matrix pipe too, two MFMAs per tile and
+// w = d * (q - c) (Q4_0: c = 8, Q5_0: 16, Q8_0: the code is a signed byte) or d * q + m (Q4_1, Q5_1) with f16 d (and
+// m) per block of 32.  The B operand is the centred code q - c itself, an integer that f16 holds exactly: the two
+// MFMAs of a block (32 k) start from zero, so their result is the block's sum of (q - c) * x, exact in f32 to within
+// the accumulation, and every lane then adds it, times the d of its column and block, into its accumulators (a lane of
+// the 32 x 32 MFMA output owns one column): sixteen v_fma per tile and block where gemm_kernel pays a second MFMA per
+// product and about ten vector-ALU instructions per weight for the dequantisation and the high/low split.  Converting
+// costs two instructions per pair of weights: the code pairs come out of the packed nibbles two at a time with one mask
+// each (Q4: after one byte permutation, its neighbours share a byte; Q8_0: bytes 0, 2 and 1, 3 of a dword), Q5's fifth
+// bits out of qh four at a time with one multiplication, 0x6400 | q is the f16 number 1024 + q, and one packed
+// subtraction of 1024 + c centres it.  x is stored with elements 1 and 2 of every four exchanged, as for the Q4_K
+// kernel, which is the order the masks produce.
+// The types with a minimum go in as d * (q - c) + (m + c d): the first sum is then as well conditioned as the weights
+// themselves (with q as it is, two sums three times the size of the result would cancel in f32).  The second,
+// sum_b (m + c d)[n, b] * (sum of x over block b), goes through the matrix pipe too, two MFMAs per tile and
 // superblock of 256 k: A = the eight block sums of the row as f16 pairs (hi for k 0..7, lo for k 8..15, written by the
 // x pre-pass for the Q4_K kernel's minimum term, times 1 / 64), B = the eight m of the column, twice, and then the
-// eight 16 d, both times 256; the main term's scales are d * 256 / 64 to match.
+// eight c d, both times 256; the main term's scales are d * 256 / 64 to match.
 //
-// The pipeline is the Q4_K kernel's: 256 x 128 outputs per workgroup of eight waves (64 x 64 each), x tiles straight
-// from memory into three LDS stages, two weight stages, one barrier per K step that waits for LDS only, explicit
-// counts of the loads issued since.  A thread converts half a block (16 weights of one row) per step.  The scale
-// records of the tile's columns lie in LDS too, a superblock of them at a time.
+// The pipeline is the Q4_K kernel's: BM x 128 outputs per workgroup of eight waves (BM = 256: 64 x 64 each; 128: 32 x 64),
+// x tiles straight from memory into three LDS stages, two weight stages, one barrier per K step that waits for LDS only,
+// explicit counts of the loads issued since.  A thread converts half a block (16 weights of one row) per step.  The
+// scale records of the tile's columns lie in LDS too, a superblock of them at a time.
 // ---------------------------------------------------------------------------
 constexpr int PBN = 128; // output columns (weight rows) per workgroup
 constexpr float XSUM_SCALE = 1.0f / 64.0f; // the x pre-pass stores the block sums times this
