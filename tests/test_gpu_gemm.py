@@ -49,6 +49,14 @@ def test_many_rows(ctx, qtype, m, n, k):
     _check(ctx, qtype, m, n, k, seed=m + qtype)
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q5_1, o.Q8_0])
+@pytest.mark.parametrize("m", [40, 160])
+def test_llama_ffn_width_with_an_odd_count_of_superblocks(ctx, qtype, m):
+    """K = 11008 (the 7B LLaMA feed-forward width, 43 superblocks of 256): the block-of-32 kernel's two record buffers and
+    its split of K over workgroups at an odd count, on both of its row tiles."""
+    _check(ctx, qtype, m, 96, 11008, seed=m + qtype)
+
+
 @pytest.mark.parametrize("xscale", [1e-30, 1e30])
 def test_many_rows_of_extreme_magnitude(ctx, xscale):
     _check(ctx, o.Q4_K, 1030, 128, 512, seed=11, xscale=xscale)
