@@ -57,6 +57,14 @@ def test_llama_ffn_width_with_an_odd_count_of_superblocks(ctx, qtype, m):
     _check(ctx, qtype, m, 96, 11008, seed=m + qtype)
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0])
+@pytest.mark.parametrize("m,n,k", [(1, 1, 256), (127, 31, 768), (129, 129, 256), (257, 255, 512), (300, 130, 2304), (513, 4, 1280)])
+def test_ragged_tiles_of_the_block_of_32_kernel(ctx, qtype, m, n, k):
+    """Row and column counts on both sides of its tile edges (128 and 256 rows, 128 columns, 32 and 64 per wave), one
+    superblock and an odd count of them, every type it takes."""
+    _check(ctx, qtype, m, n, k, seed=m * 3 + n + k + qtype)
+
+
 @pytest.mark.parametrize("xscale", [1e-30, 1e30])
 def test_many_rows_of_extreme_magnitude(ctx, xscale):
     _check(ctx, o.Q4_K, 1030, 128, 512, seed=11, xscale=xscale)
