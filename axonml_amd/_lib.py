@@ -115,6 +115,8 @@ SIGNATURES = {
     "axq_fill_normal_f32": (_i, [_vp, _vp, _sz, C.c_float, C.c_float, C.c_float, C.c_float, C.c_uint64]),
     "axq_bench_gemv_ring": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i, _vp, _i]),
     "axq_bench_read_ring": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i]),
+    "axq_bench_read_ring_ex": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i]),
+    "axq_bench_gemv_ring_streams": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i, _vp, _i, _i]),
     "axq_bench_copy": (_i, [_vp, _vp, _vp, _sz, _i]),
     "axq_sample_token": (_i, [_vp, _vp, _i, _vp, _i, C.POINTER(SamplingConfig), C.c_float, C.POINTER(C.c_int32), _vp, _i]),
     "axq_model_set_sampling": (_i, [_vp, C.POINTER(SamplingConfig), C.c_uint64]),

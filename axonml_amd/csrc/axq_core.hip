@@ -152,12 +152,20 @@ int axq_init(int device, axq_ctx **out) {
     axq_ctx *ctx = (axq_ctx *)calloc(1, sizeof(axq_ctx));
     if (!ctx) return axq_fail(NULL, AXQ_ERR_ALLOCATION_FAILED, "out of host memory");
     ctx->device = device;
+    // one way out of a failed set-up: whatever exists by then is released, with the device still current
+    auto undo = [&]() {
+        if (ctx->xq) (void)hipFree(ctx->xq);
+        if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+        if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+        if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
+        free(ctx);
+    };
 #define INIT_HIP(call)                                                                         \
     do {                                                                                       \
         hipError_t e_ = (call);                                                                \
         if (e_ != hipSuccess) {                                                                \
             axq_fail(NULL, AXQ_ERR_DRIVER, "%s: %s", #call, hipGetErrorString(e_));            \
-            free(ctx);                                                                         \
+            undo();                                                                            \
             return AXQ_ERR_DRIVER;                                                             \
         }                                                                                      \
     } while (0)
@@ -166,7 +174,7 @@ int axq_init(int device, axq_ctx **out) {
     if (strncmp(ctx->prop.gcnArchName, "gfx950", 6) != 0) {
         axq_fail(NULL, AXQ_ERR_DEVICE_NOT_FOUND, "device %d is %s; this library is built for gfx950 only", device,
                  ctx->prop.gcnArchName);
-        free(ctx);
+        undo();
         return AXQ_ERR_DEVICE_NOT_FOUND;
     }
     INIT_HIP(hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking));
@@ -177,12 +185,13 @@ int axq_init(int device, axq_ctx **out) {
     INIT_HIP(hipMalloc((void **)&probe, 2 * sizeof(float)));
     axq_probe_fp8_kernel<<<1, 1, 0, ctx->stream>>>(probe);
     float h[2] = {0, 0};
-    INIT_HIP(hipMemcpyAsync(h, probe, sizeof h, hipMemcpyDeviceToHost, ctx->stream));
-    INIT_HIP(hipStreamSynchronize(ctx->stream));
-    INIT_HIP(hipFree(probe));
+    hipError_t pe = hipMemcpyAsync(h, probe, sizeof h, hipMemcpyDeviceToHost, ctx->stream);
+    if (pe == hipSuccess) pe = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(probe);
+    INIT_HIP(pe);
     if (!(h[0] > 0.0f) || h[1] != 15.0f * h[0]) {
         axq_fail(NULL, AXQ_ERR_DRIVER, "fp8 probe: byte 0x01 -> %g, 0x0F -> %g (not linear)", h[0], h[1]);
-        free(ctx);
+        undo();
         return AXQ_ERR_DRIVER;
     }
     ctx->fp8_unit_inv = 1.0f / h[0];
@@ -191,12 +200,10 @@ int axq_init(int device, axq_ctx **out) {
         size_t xq_bytes = axq_xq_bytes(AXQ_XQ_MAX_K), mb_bytes = AXQ_BATCH_SCRATCH_BYTES;
         INIT_HIP(hipMalloc((void **)&ctx->xq, xq_bytes > mb_bytes ? xq_bytes : mb_bytes));
     }
-    if (axq_gemv_static_setup(ctx) != AXQ_OK) { // this device's copy of the scratch of axq_gemv_f32_static
-        axq_fail(NULL, AXQ_ERR_DRIVER, "%s", ctx->err);
-        (void)hipFree(ctx->xq);
-        free(ctx);
-        return AXQ_ERR_DRIVER;
-    }
+    // this device's copy of the scratch of axq_gemv_f32_static; a device the table has no place for (or a failed
+    // look-up) leaves that one entry point refusing its calls, the rest of the library works
+    (void)axq_gemv_static_setup(ctx);
+    ctx->err[0] = 0;
     // A lone GEMV call splits x inside the kernel (one launch); callers that produce x on the device
     // hand over the split form instead.  AXQ_GEMV_PREP=separate forces the two-kernel form (development).
     const char *prep = getenv("AXQ_GEMV_PREP");
@@ -219,6 +226,11 @@ void axq_destroy(axq_ctx *ctx) {
     (void)hipEventDestroy(ctx->ev_start);
     (void)hipEventDestroy(ctx->ev_stop);
     (void)hipStreamDestroy(ctx->own_stream);
+    for (int i = 0; i < AXQ_AUX_STREAMS; i++) {
+        if (ctx->aux_stream[i]) (void)hipStreamDestroy(ctx->aux_stream[i]);
+        if (ctx->aux_event[i]) (void)hipEventDestroy(ctx->aux_event[i]);
+    }
+    if (ctx->aux_fork) (void)hipEventDestroy(ctx->aux_fork);
     (void)hipFree(ctx->xq);
     if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
     free(ctx);

@@ -1294,11 +1294,18 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     if (nn) fill_f32_kernel<<<(unsigned)((nn + 255) / 256), 256, 0, ctx->stream>>>(m->norm_attn, nn, 1.0f);
     if (nn) fill_f32_kernel<<<(unsigned)((nn + 255) / 256), 256, 0, ctx->stream>>>(m->norm_ffn, nn, 1.0f);
     fill_f32_kernel<<<(H + 255) / 256, 256, 0, ctx->stream>>>(m->norm_final, H, 1.0f);
-    (void)hipMemsetAsync(m->kcache, 0, kv * 2, ctx->stream);
-    (void)hipMemsetAsync(m->vcache, 0, kv * 2, ctx->stream);
-    (void)hipMemsetAsync(m->pos, 0, 4, ctx->stream);
-    (void)hipMemsetAsync(m->gen, 0, 4, ctx->stream);
-    (void)hipMemsetAsync(m->tok, 0, 4, ctx->stream);
+    {
+        hipError_t e = hipMemsetAsync(m->kcache, 0, kv * 2, ctx->stream);
+        if (e == hipSuccess) e = hipMemsetAsync(m->vcache, 0, kv * 2, ctx->stream);
+        if (e == hipSuccess) e = hipMemsetAsync(m->pos, 0, 4, ctx->stream);
+        if (e == hipSuccess) e = hipMemsetAsync(m->gen, 0, 4, ctx->stream);
+        if (e == hipSuccess) e = hipMemsetAsync(m->tok, 0, 4, ctx->stream);
+        if (e != hipSuccess) {
+            const int st = axq_fail(ctx, AXQ_ERR_DRIVER, "axq_model_create: clearing the cache and the counters: %s", hipGetErrorString(e));
+            axq_model_free(m);
+            return st;
+        }
+    }
     // RotaryEmbedding::new (llama.rs:223-252): inv_freq_i = 1 / theta^(2i/d), tables of cos/sin(pos * inv_freq_i)
     {
         const int half = c.head_dim / 2;

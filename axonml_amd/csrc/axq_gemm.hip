@@ -1023,7 +1023,9 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
         }
     };
     auto multiply_min = [&](int sb) {
-        const half2v ws2 = {(_Float16)WSCALE, (_Float16)WSCALE}, wd2 = {(_Float16)(CENTER * WSCALE), (_Float16)(CENTER * WSCALE)};
+        // The operands are the stored f16 numbers themselves, m and d: any f16 a block can hold goes through exactly (m times
+        // a power of two, or 16 d, would overflow f16 for minimums from 256 and scales from 16 on).  The powers of two --
+        // WSCALE for both, the code centre for the d sum -- are applied in f32 when the sums are added.
         half8 bm[2], bd[2];
 #pragma unroll
         for (int j = 0; j < 2; j++) {
@@ -1034,29 +1036,25 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
                 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
                 const u32x2 r2 = *reinterpret_cast<const u32x2 *>(rlane + (sb & 1) * RECB + j * 32 * 16 * RV + q * 8);
                 const uint32_t r0 = r2[0], r1 = r2[1];
-                const uint32_t ms = (r0 >> 16) | (r1 & 0xFFFF0000u), dsc = (r0 & 0xFFFFu) | (r1 << 16);
-                const half2v vm = __builtin_bit_cast(half2v, ms) * ws2, vd = __builtin_bit_cast(half2v, dsc) * wd2;
-                om[q] = __builtin_bit_cast(uint32_t, vm);
-                od[q] = __builtin_bit_cast(uint32_t, vd);
+                om[q] = (r0 >> 16) | (r1 & 0xFFFF0000u);
+                od[q] = (r0 & 0xFFFFu) | (r1 << 16);
             }
             bm[j] = __builtin_bit_cast(half8, u32x4{om[0], om[1], om[2], om[3]});
             bd[j] = __builtin_bit_cast(half8, u32x4{od[0], od[1], od[2], od[3]});
         }
-        // the block sums are stored times XSUM_SCALE and these operands times WSCALE: the accumulators hold the result times
-        // WSCALE * XSUM_SCALE, and the main term scales its sums to match (scale_of)
+        // the block sums are stored times XSUM_SCALE: with the factors below the accumulators receive the term times
+        // WSCALE * XSUM_SCALE, which is what the main term scales its sums to (scale_of)
         // (added by the vector ALU like the main term: accumulators that the matrix pipe also wrote would be kept twice)
         const float16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < MI; i++) {
-            float16v S[2];
 #pragma unroll
-            for (int j = 0; j < 2; j++) S[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bm[j], zero, 0, 0, 0);
+            for (int j = 0; j < 2; j++) {
+                const float16v Sm = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bm[j], zero, 0, 0, 0);
+                const float16v Sd = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bd[j], zero, 0, 0, 0);
 #pragma unroll
-            for (int j = 0; j < 2; j++) S[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bd[j], S[j], 0, 0, 0);
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) acc[i][j][r] += S[j][r];
+                for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(Sd[r], CENTER * WSCALE, fmaf(Sm[r], WSCALE, acc[i][j][r]));
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
     };

@@ -431,8 +431,19 @@ __global__ void __launch_bounds__(512) mb_reduce_pack_kernel(const float *src, i
 
 // next_even_odd < 0: nothing follows.  Otherwise y is the input of another small-batch GEMV whose operands
 // (EVEN_ODD as given, RMSNorm with next_aux when that is not null) are prepared here, in the same scratch.
+// Dynamic LDS beyond 64 KB is asked for once per kernel and device; bit d = device d has been asked (axq_allow_lds).
 template <class T>
-void launch_mb(axq_ctx *ctx, MbArgs a, uint8_t *sc, const float *x, int xmode, const float *aux, float eps, int next_even_odd, const float *next_aux) {
+std::atomic<uint64_t> &mb_lds_mask() {
+    static std::atomic<uint64_t> mask{0};
+    return mask;
+}
+unsigned mb_max_waves() {
+    static const unsigned smax = getenv("AXQ_BATCH_WAVES") ? (unsigned)atoi(getenv("AXQ_BATCH_WAVES")) : 8; // development knob (1..8)
+    return smax < 1 ? 1 : (smax > 8 ? 8 : smax);
+}
+
+template <class T>
+int launch_mb(axq_ctx *ctx, MbArgs a, uint8_t *sc, const float *x, int xmode, const float *aux, float eps, int next_even_odd, const float *next_aux) {
     const dim3 pgrid((unsigned)((a.k / 8 + 255) / 256), MAX_BATCH);
     uint8_t *xa = const_cast<uint8_t *>(a.xa);
     float *xsg = const_cast<float *>(a.xsg);
@@ -453,12 +464,13 @@ void launch_mb(axq_ctx *ctx, MbArgs a, uint8_t *sc, const float *x, int xmode, c
     a.chunks_per_split = (int)((chunks + splits - 1) / splits);
     splits = (chunks + a.chunks_per_split - 1) / a.chunks_per_split;
     if (splits < 2) a.ypart = nullptr;
-    static const unsigned smax = getenv("AXQ_BATCH_WAVES") ? (unsigned)atoi(getenv("AXQ_BATCH_WAVES")) : 8; // development knob (1..8)
+    const unsigned smax = mb_max_waves();
     const unsigned S = (unsigned)a.chunks_per_split < smax ? (unsigned)a.chunks_per_split : smax;
     const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float) + (size_t)S * 32 * T::NP * 16;
-    static std::atomic<uint64_t> lds_allowed{0};
-    if (lds > 64 * 1024) (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_mb_kernel<T>), lds_allowed, 160 * 1024); // a refusal is
-    // the context's error now, and the launch below fails with it
+    if (lds > 64 * 1024) {
+        const int st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_mb_kernel<T>), mb_lds_mask<T>(), 160 * 1024);
+        if (st != AXQ_OK) return st; // the refusal is the call's error: nothing is launched into it
+    }
     gemv_mb_kernel<T><<<dim3(tiles, splits), 64 * S, lds, ctx->stream>>>(a);
     if (next_even_odd >= 0) {
         // y's operands for the next GEMV (k' = n_rows): the scratch layout of that call
@@ -474,6 +486,7 @@ void launch_mb(axq_ctx *ctx, MbArgs a, uint8_t *sc, const float *x, int xmode, c
         const int total = a.n_rows * a.batch;
         mb_reduce_kernel<<<(total + 255) / 256, 256, 0, ctx->stream>>>(a.ypart, a.bias, a.resid, a.n_rows, a.batch, (int)splits, a.y);
     }
+    return AXQ_OK;
 }
 
 // One call of the small-batch GEMV with its scratch at `sc` (AXQ_BATCH_SCRATCH_BYTES bytes): 32 k bytes of A operands,
@@ -490,13 +503,15 @@ int gemv_batch_in(axq_ctx *ctx, uint8_t *sc, const axq_weight *w, const float *x
     a.bias = bias; a.resid = resid; a.y = y;
     a.ypart = w->n_rows <= AXQ_BATCH_SPLIT_ROWS ? reinterpret_cast<float *>(sc + (size_t)34 * AXQ_BATCH_MAX_K) : nullptr;
     a.n_rows = (int)w->n_rows; a.k = k; a.batch = batch;
+    int st;
     switch (w->type) {
-    case AXQ_Q4_0: launch_mb<MQ4x<false>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
-    case AXQ_Q4_1: launch_mb<MQ4x<true>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
-    case AXQ_Q8_0: launch_mb<MQ80>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
-    case AXQ_Q4_K: launch_mb<MQ4K>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q4_0: st = launch_mb<MQ4x<false>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q4_1: st = launch_mb<MQ4x<true>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q8_0: st = launch_mb<MQ80>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q4_K: st = launch_mb<MQ4K>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
     default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
     }
+    if (st != AXQ_OK) return st;
     AXQ_LAUNCH_CHECK(ctx, "gemv_mb_kernel");
     return AXQ_OK;
 }
@@ -567,11 +582,14 @@ int axq_gemv_static_setup(axq_ctx *ctx) {
     uint8_t *ptr = nullptr;
     AXQ_HIP(ctx, hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)), AXQ_ERR_DRIVER);
     if (!ptr) return axq_fail(ctx, AXQ_ERR_DRIVER, "hipGetSymbolAddress gave no address for the static GEMV scratch");
-    // dynamic LDS beyond 64 KB has to be asked for once per kernel: here, so that the entry point itself only launches
-    AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4x<false>>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024), AXQ_ERR_DRIVER);
-    AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4x<true>>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024), AXQ_ERR_DRIVER);
-    AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<MQ80>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024), AXQ_ERR_DRIVER);
-    AXQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4K>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024), AXQ_ERR_DRIVER);
+    // Dynamic LDS beyond 64 KB has to be asked for once per kernel and device, and the development knob is read once: both
+    // here, through the very masks the launch code consults, so that the entry point itself only launches.
+    int st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4x<false>>), mb_lds_mask<MQ4x<false>>(), 160 * 1024);
+    if (st == AXQ_OK) st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4x<true>>), mb_lds_mask<MQ4x<true>>(), 160 * 1024);
+    if (st == AXQ_OK) st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_mb_kernel<MQ80>), mb_lds_mask<MQ80>(), 160 * 1024);
+    if (st == AXQ_OK) st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_mb_kernel<MQ4K>), mb_lds_mask<MQ4K>(), 160 * 1024);
+    if (st != AXQ_OK) return st;
+    (void)mb_max_waves();
     g_scratch_ptr[ctx->device] = ptr;
     return AXQ_OK;
 }
@@ -587,11 +605,12 @@ int axq_gemv_f32_static(axq_ctx *ctx, const axq_weight *w, const float *x, int b
                         AXQ_BATCH_MAX_K);
     if (w->n_rows > INT32_MAX)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: weight dimensions exceed 2^31");
+    if (w->k % 256 != 0)
+        return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: axq_gemv_f32_static takes k a multiple of 256, got %lld", (long long)w->k);
     if (!axq_dev_gemv_batch_covers(w, batch))
-        return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE,
-                        "axq_gemv_f32_static covers Q4_0, Q4_1, Q8_0 and Q4_K weights with k a multiple of 256 (got type %d, k = %lld)",
-                        w->type, (long long)w->k);
-    uint8_t *ptr = g_scratch_ptr[ctx->device];
-    if (!ptr) return axq_fail(ctx, AXQ_ERR_DRIVER, "the static GEMV scratch of device %d was not set up", ctx->device);
+        return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "axq_gemv_f32_static covers Q4_0, Q4_1, Q8_0 and Q4_K weights (got type %d)", w->type);
+    uint8_t *ptr = (ctx->device >= 0 && ctx->device < MAX_DEVICES) ? g_scratch_ptr[ctx->device] : nullptr;
+    if (!ptr) return axq_fail(ctx, AXQ_ERR_DRIVER, "the static GEMV scratch of device %d was not set up (devices 0..%d have one)", ctx->device, MAX_DEVICES - 1);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
     return gemv_batch_in(ctx, ptr, w, x, AXQ_X_PLAIN, nullptr, 0.f, batch, bias, nullptr, y, -1, nullptr);
 }

@@ -867,10 +867,11 @@ __global__ void __launch_bounds__(256) prep_x_kernel(const float *x, int k, uint
             (int)(gridDim.x * blockDim.x));
 }
 
+// The launchers return AXQ_OK or the status of a refused request for dynamic LDS (nothing is launched then).
 template <class T, int NB, bool PRE>
-void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
-    static std::atomic<uint64_t> lds_allowed{0}, lds_allowed_w{0}; // dynamic LDS beyond 64 KB is asked for per kernel and device; a
-    // refusal is the context's error, and the launch that follows fails with it
+int launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
+    static std::atomic<uint64_t> lds_allowed{0}, lds_allowed_w{0}; // dynamic LDS beyond 64 KB is asked for per kernel and device
+    int st;
     static const bool shared_x = getenv("AXQ_GEMV_SHARED_X") && getenv("AXQ_GEMV_SHARED_X")[0] == '1'; // development knob: the kernel that splits x once per workgroup
     // the per-round scale loads are 16 bytes wide: the rows of the meta plane have to be whole 16-byte pieces
     const bool rounds_ok = !T::ROUND_META || NB > 4 || (T::meta_row_bytes(a.k) % 16 == 0 && a.meta_pitch % 16 == 0 && T::meta_row_bytes(a.k) >= 16);
@@ -878,58 +879,63 @@ void launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, si
         // x arrives raw: every wave stages its own slice
         const size_t lds_w = (size_t)(block / 64) * (4 * 1024 + 32 * 16 + (T::ROUND_META ? 16 * T::META_SLICE_BYTES : 0)) + 64 +
                              (size_t)a.G * a.steps * 4 * a.S * 4 * sizeof(float);
-        if (lds_w > 64 * 1024 && lds_w <= 160 * 1024)
-            (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), lds_allowed_w, 160 * 1024);
+        if (lds_w > 64 * 1024 && lds_w <= 160 * 1024 &&
+            (st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), lds_allowed_w, 160 * 1024)) != AXQ_OK)
+            return st;
         if (lds_w <= 160 * 1024) {
             gemv_dpw_kernel<T, NB><<<grid, block, lds_w, ctx->stream>>>(a);
-            return;
+            return AXQ_OK;
         }
     }
-    if (lds > 64 * 1024) (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE, false>), lds_allowed, 160 * 1024);
+    if (lds > 64 * 1024 && (st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE, false>), lds_allowed, 160 * 1024)) != AXQ_OK)
+        return st;
     gemv_dp_kernel<T, NB, PRE, false><<<grid, block, lds, ctx->stream>>>(a);
+    return AXQ_OK;
 }
 
 template <class T, bool PRE>
-void launch_nb(axq_ctx *ctx, const DpArgs &a, int nb, unsigned grid, unsigned block, size_t lds) {
+int launch_nb(axq_ctx *ctx, const DpArgs &a, int nb, unsigned grid, unsigned block, size_t lds) {
     switch (nb) {
-    case 1: launch_one<T, 1, PRE>(ctx, a, grid, block, lds); break;
-    case 2: launch_one<T, 2, PRE>(ctx, a, grid, block, lds); break;
-    case 3: launch_one<T, 3, PRE>(ctx, a, grid, block, lds); break;
-    case 4: launch_one<T, 4, PRE>(ctx, a, grid, block, lds); break;
-    case 5: launch_one<T, 5, PRE>(ctx, a, grid, block, lds); break;
-    case 6: launch_one<T, 6, PRE>(ctx, a, grid, block, lds); break;
-    case 7: launch_one<T, 7, PRE>(ctx, a, grid, block, lds); break;
-    default: launch_one<T, 8, PRE>(ctx, a, grid, block, lds); break;
+    case 1: return launch_one<T, 1, PRE>(ctx, a, grid, block, lds);
+    case 2: return launch_one<T, 2, PRE>(ctx, a, grid, block, lds);
+    case 3: return launch_one<T, 3, PRE>(ctx, a, grid, block, lds);
+    case 4: return launch_one<T, 4, PRE>(ctx, a, grid, block, lds);
+    case 5: return launch_one<T, 5, PRE>(ctx, a, grid, block, lds);
+    case 6: return launch_one<T, 6, PRE>(ctx, a, grid, block, lds);
+    case 7: return launch_one<T, 7, PRE>(ctx, a, grid, block, lds);
+    default: return launch_one<T, 8, PRE>(ctx, a, grid, block, lds);
     }
 }
 
-// Q4_K with a raw x: the kernel with one header load per round.
+// Q4_K with a raw x: the kernel with one header load per round.  1 = launched, 0 = not this kernel's case, < 0 = status.
 template <class T>
-bool launch_q4k_rounds(axq_ctx *, const DpArgs &, unsigned, unsigned, size_t) { return false; }
+int launch_q4k_rounds(axq_ctx *, const DpArgs &, unsigned, unsigned, size_t) { return 0; }
 template <>
-bool launch_q4k_rounds<DQ4K>(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
+int launch_q4k_rounds<DQ4K>(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, size_t lds) {
     static const bool off = getenv("AXQ_GEMV_Q4K_ROUNDS") && getenv("AXQ_GEMV_Q4K_ROUNDS")[0] == '0'; // development knob
     static std::atomic<uint64_t> lds_allowed[2];
-    if (off) return false;
+    if (off) return 0;
     // measured inside the 7B-shape decode: a gain from three steps per group on (qkv 6.6 -> 6.0 us, gate/up 15.4 -> 14.8 us);
     // with two steps (o projection) or one group of 14 waves over a long K (down projection, two split tasks per thread)
     // the kernel with per-wave staging and no barrier is ahead
-    if (a.G < 2 || a.steps < 3) return false;
+    if (a.G < 2 || a.steps < 3) return 0;
     lds += (size_t)(block / 64) * 16 * DQ4K::META_SLICE_BYTES; // the waves' patches of scale records
-    if (lds > 160 * 1024) return false;
+    if (lds > 160 * 1024) return 0;
     if (lds > 64 * 1024) {
-        (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<DQ4K, 3, false, true>), lds_allowed[0], 160 * 1024);
-        (void)axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<DQ4K, 4, false, true>), lds_allowed[1], 160 * 1024);
+        int st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<DQ4K, 3, false, true>), lds_allowed[0], 160 * 1024);
+        if (st == AXQ_OK) st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<DQ4K, 4, false, true>), lds_allowed[1], 160 * 1024);
+        if (st != AXQ_OK) return st;
     }
     if (a.steps == 3) gemv_dp_kernel<DQ4K, 3, false, true><<<grid, block, lds, ctx->stream>>>(a);
     else gemv_dp_kernel<DQ4K, 4, false, true><<<grid, block, lds, ctx->stream>>>(a);
-    return true;
+    return 1;
 }
 
+// 1 = launched, 0 = the shape is not this kernel's, < 0 = status
 template <class T>
-bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux, float eps,
-               int ymode, const float *bias, float *y) {
-    if (w->k % 64 != 0 || w->k > 16384) return false;
+int launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux, float eps,
+              int ymode, const float *bias, float *y) {
+    if (w->k % 64 != 0 || w->k > 16384) return 0;
     DpArgs a;
     a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
     a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
@@ -957,11 +963,13 @@ bool launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t 
     const unsigned grid = (unsigned)((rowsteps + steps * a.G - 1) / (steps * a.G));
     size_t lds = (size_t)a.G * steps * 4 * a.S * 4 * sizeof(float);
     lds += axq_split_bytes(a.k) + 16 + 64;
-    if (lds > 160 * 1024) return false;
-    if (!xq && launch_q4k_rounds<T>(ctx, a, grid, block, lds)) return true;
-    if (xq) launch_nb<T, true>(ctx, a, nb, grid, block, lds);
-    else launch_nb<T, false>(ctx, a, nb, grid, block, lds);
-    return true;
+    if (lds > 160 * 1024) return 0;
+    if (!xq) {
+        const int r = launch_q4k_rounds<T>(ctx, a, grid, block, lds);
+        if (r != 0) return r;
+    }
+    const int st = xq ? launch_nb<T, true>(ctx, a, nb, grid, block, lds) : launch_nb<T, false>(ctx, a, nb, grid, block, lds);
+    return st == AXQ_OK ? 1 : st;
 }
 
 } // namespace
@@ -983,7 +991,7 @@ int axq_dev_prep_x(axq_ctx *ctx, const float *x, int64_t k, uint8_t *xq) {
 // applying the prologue `mode` (axq_internal.h) with its second operand `aux`.
 int axq_dev_gemv_dp_ex(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux,
                        float eps, int ymode, const float *bias, float *y) {
-    bool ok;
+    int ok;
     if (xq && mode != AXQ_X_PLAIN) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "a fused prologue needs the raw x");
     if (ymode == AXQ_Y_SWIGLU && (w->n_rows % 8 != 0 || bias))
         return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "the SwiGLU epilogue needs whole groups of 8 rows and no bias");
@@ -996,7 +1004,7 @@ int axq_dev_gemv_dp_ex(axq_ctx *ctx, const axq_weight *w, const float *x, const 
     case AXQ_Q8_0: ok = launch_dp<DQ80>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
     default: return 0;
     }
-    if (!ok) return 0;
+    if (ok <= 0) return ok;
     AXQ_LAUNCH_CHECK(ctx, "gemv_dp_kernel");
     return 1;
 }

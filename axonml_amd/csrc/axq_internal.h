@@ -25,8 +25,14 @@ struct axq_ctx {
     int gemv_wgs_per_cu; // GEMV workgroups per compute unit that the rows are spread over
     void *gemm_scratch; // device scratch of the prefill GEMM (scaled f16 activations + row scales), grown on demand
     size_t gemm_scratch_bytes;
+    hipStream_t aux_stream[4]; // benchmarks only: launches that may overlap (created on first use, default priority)
+    hipEvent_t aux_event[4], aux_fork;
     char err[512];
 };
+#define AXQ_AUX_STREAMS 4
+int axq_aux_streams(axq_ctx *ctx, int n);
+int axq_aux_fork(axq_ctx *ctx, int n);
+int axq_aux_join(axq_ctx *ctx, int n);
 
 // ---------------------------------------------------------------------------
 // Device-resident weight: "planar" layout, one allocation.

@@ -99,24 +99,93 @@ __global__ void axq_copy16_kernel(uint4 *__restrict__ dst, const uint4 *__restri
 }
 
 // Reads `n16*16` bytes and keeps nothing: what the memory system gives a launch that only streams a weight.  Each
-// workgroup takes one contiguous share, sixteen 16-byte non-temporal loads per lane in flight; indices past the
-// end re-read the last element.
+// workgroup takes one contiguous share and keeps U 16-byte loads per lane in flight (non-temporal when NT); a lane whose
+// index lies past the workgroup's share re-reads the share's last element (a cache hit), so that the bytes fetched
+// from memory are the image's own and no more.
 typedef uint32_t axq_u32x4 __attribute__((ext_vector_type(4)));
-__global__ void __launch_bounds__(512) axq_read16_kernel(const axq_u32x4 *__restrict__ src, size_t n16, uint32_t *sink) {
+template <int U, bool NT, int TPB>
+__global__ void __launch_bounds__(TPB) axq_read_kernel(const axq_u32x4 *__restrict__ src, size_t n16, uint32_t *sink) {
     const size_t share = (n16 + gridDim.x - 1) / gridDim.x;
     const size_t lo = (size_t)blockIdx.x * share, hi = lo + share < n16 ? lo + share : n16;
     uint32_t acc = 0;
-    for (size_t i = lo + threadIdx.x; i < hi; i += 16 * 512) {
-        axq_u32x4 v[16];
+    for (size_t i = lo + threadIdx.x; i < hi; i += (size_t)U * TPB) {
+        axq_u32x4 v[U];
 #pragma unroll
-        for (int u = 0; u < 16; u++) {
-            size_t j = i + (size_t)u * 512;
-            v[u] = __builtin_nontemporal_load(src + (j < n16 ? j : n16 - 1));
+        for (int u = 0; u < U; u++) {
+            size_t j = i + (size_t)u * TPB;
+            j = j < hi ? j : hi - 1;
+            v[u] = NT ? __builtin_nontemporal_load(src + j) : src[j];
         }
 #pragma unroll
-        for (int u = 0; u < 16; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+        for (int u = 0; u < U; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
     }
     if (acc == 0x9E3779B9u) sink[0] = acc; // keeps the loads alive; a match writes four bytes of no consequence
+}
+
+// The same bytes in the order the one-vector GEMV asks for them: a workgroup of eight waves owns `rows` consecutive rows of
+// the code plane (pitch bytes each, 2048 of them used), wave (g, s) walks the 4-row steps of half g and reads, per step,
+// two pieces of 256 bytes of each of the step's four rows (lane = (16-byte chunk, row)), NB steps in flight.
+template <int NB>
+__global__ void __launch_bounds__(512) axq_read_rows_kernel(const uint8_t *__restrict__ codes, size_t pitch, int n_rows, int rows_per_wg, uint32_t *sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = wave >> 2, s = wave & 3;
+    const int blk = lane >> 2, j = lane & 3;
+    const int half_rows = rows_per_wg / 2, steps = half_rows / 4;
+    const int row0 = blockIdx.x * rows_per_wg + g * half_rows + j;
+    uint32_t acc = 0;
+    for (int st = 0; st < steps; st += NB) {
+        axq_u32x4 v[NB][2];
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            int row = row0 + 4 * (st + b < steps ? st + b : 0);
+            row = row < n_rows ? row : n_rows - 1;
+            const uint8_t *p = codes + (size_t)row * pitch + s * 256 + blk * 16;
+            v[b][0] = __builtin_nontemporal_load(reinterpret_cast<const axq_u32x4 *>(p));
+            v[b][1] = __builtin_nontemporal_load(reinterpret_cast<const axq_u32x4 *>(p + 1024));
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) acc ^= v[b][0].x ^ v[b][0].w ^ v[b][1].y ^ v[b][1].z;
+    }
+    if (acc == 0x9E3779B9u) sink[0] = acc;
+}
+
+template <int U, bool NT>
+static void launch_read(int threads, unsigned grid, hipStream_t st, const axq_u32x4 *src, size_t n16, uint32_t *sink) {
+    if (threads == 256) axq_read_kernel<U, NT, 256><<<grid, 256, 0, st>>>(src, n16, sink);
+    else if (threads == 512) axq_read_kernel<U, NT, 512><<<grid, 512, 0, st>>>(src, n16, sink);
+    else axq_read_kernel<(U > 16 ? 16 : U), NT, 1024><<<grid, 1024, 0, st>>>(src, n16, sink); // 1024 threads: 128 registers each
+}
+template <bool NT>
+static void launch_read_u(int in_flight, int threads, unsigned grid, hipStream_t st, const axq_u32x4 *src, size_t n16, uint32_t *sink) {
+    if (in_flight <= 4) launch_read<4, NT>(threads, grid, st, src, n16, sink);
+    else if (in_flight <= 8) launch_read<8, NT>(threads, grid, st, src, n16, sink);
+    else if (in_flight <= 16) launch_read<16, NT>(threads, grid, st, src, n16, sink);
+    else launch_read<32, NT>(threads, grid, st, src, n16, sink);
+}
+
+// Streams beside the context's own, for launches that may overlap (benchmarks only; default priority).  The first use
+// creates them; axq_destroy releases them.
+int axq_aux_streams(axq_ctx *ctx, int n) {
+    if (n > AXQ_AUX_STREAMS) n = AXQ_AUX_STREAMS;
+    for (int i = 0; i < n; i++) {
+        if (!ctx->aux_stream[i]) AXQ_HIP(ctx, hipStreamCreateWithFlags(&ctx->aux_stream[i], hipStreamNonBlocking), AXQ_ERR_DRIVER);
+        if (!ctx->aux_event[i]) AXQ_HIP(ctx, hipEventCreateWithFlags(&ctx->aux_event[i], hipEventDisableTiming), AXQ_ERR_DRIVER);
+    }
+    if (!ctx->aux_fork) AXQ_HIP(ctx, hipEventCreateWithFlags(&ctx->aux_fork, hipEventDisableTiming), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+// Everything enqueued on the context's stream so far happens before what the first n side streams get next ...
+int axq_aux_fork(axq_ctx *ctx, int n) {
+    AXQ_HIP(ctx, hipEventRecord(ctx->aux_fork, ctx->stream), AXQ_ERR_DRIVER);
+    for (int i = 0; i < n; i++) AXQ_HIP(ctx, hipStreamWaitEvent(ctx->aux_stream[i], ctx->aux_fork, 0), AXQ_ERR_DRIVER);
+    return AXQ_OK;
+}
+// ... and what they have been given happens before whatever the context's stream gets next.
+int axq_aux_join(axq_ctx *ctx, int n) {
+    for (int i = 0; i < n; i++) {
+        AXQ_HIP(ctx, hipEventRecord(ctx->aux_event[i], ctx->aux_stream[i]), AXQ_ERR_DRIVER);
+        AXQ_HIP(ctx, hipStreamWaitEvent(ctx->stream, ctx->aux_event[i], 0), AXQ_ERR_DRIVER);
+    }
+    return AXQ_OK;
 }
 
 extern "C" {
@@ -321,21 +390,70 @@ int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_we
     return AXQ_OK;
 }
 
+int axq_bench_gemv_ring_streams(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first, const float *x_dev,
+                                int batch, float *y_dev, int iters, int streams) {
+    if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_gemv_ring_streams: NULL context");
+    if (!weights || n_weights <= 0 || first < 0 || !x_dev || !y_dev || batch != 1 || streams < 1 || streams > AXQ_AUX_STREAMS)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_gemv_ring_streams: bad argument (one vector per launch, 1..%d streams)", AXQ_AUX_STREAMS);
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    int rc;
+    if ((rc = axq_aux_streams(ctx, streams)) || (rc = axq_aux_fork(ctx, streams))) return rc;
+    hipStream_t own = ctx->stream;
+    for (int i = 0; i < iters && rc == AXQ_OK; i++) {
+        const axq_weight *w = weights[(first + i) % n_weights];
+        if (!w) { rc = axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_gemv_ring_streams: NULL weight"); break; }
+        ctx->stream = ctx->aux_stream[i % streams]; // the one-vector GEMV keeps no scratch outside its own launch
+        rc = axq_dev_gemv(ctx, w, x_dev, 1, NULL, y_dev);
+    }
+    ctx->stream = own;
+    if (rc) return rc;
+    return axq_aux_join(ctx, streams);
+}
+
 int axq_bench_read_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first, uint32_t *sink_dev,
                         int iters) {
+    return axq_bench_read_ring_ex(ctx, weights, n_weights, first, sink_dev, iters, 1, 512, 16, 1, 0, 1);
+}
+
+int axq_bench_read_ring_ex(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first, uint32_t *sink_dev,
+                           int iters, int wgs_per_cu, int threads, int in_flight, int nontemporal, int pattern, int streams) {
     if (!ctx) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring: NULL context");
     if (!weights || n_weights <= 0 || first < 0 || !sink_dev)
         return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring: bad argument");
+    if (wgs_per_cu < 1 || wgs_per_cu > 8 || (threads != 256 && threads != 512 && threads != 1024) || in_flight < 1 || in_flight > 32 ||
+        streams < 1 || streams > AXQ_AUX_STREAMS || pattern < 0 || pattern > 1)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring_ex: 1..8 workgroups per compute unit, 256/512/1024 threads, 1..32 "
+                                                       "loads in flight, 1..%d streams, pattern 0 or 1", AXQ_AUX_STREAMS);
     AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
-    const unsigned grid = (unsigned)ctx->prop.multiProcessorCount; // one 512-thread workgroup per compute unit, as the GEMV
+    int rc;
+    if (streams > 1) {
+        if ((rc = axq_aux_streams(ctx, streams))) return rc;
+        if ((rc = axq_aux_fork(ctx, streams))) return rc;
+    }
+    const unsigned grid = (unsigned)(ctx->prop.multiProcessorCount * wgs_per_cu);
     for (int i = 0; i < iters; i++) {
         const axq_weight *w = weights[(first + i) % n_weights];
         if (!w) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring: NULL weight");
-        const size_t n16 = w->alloc_bytes / 16;
-        if (n16 == 0) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring: empty weight");
-        axq_read16_kernel<<<grid, 512, 0, ctx->stream>>>((const axq_u32x4 *)w->base, n16, sink_dev);
+        hipStream_t st = streams > 1 ? ctx->aux_stream[i % streams] : ctx->stream;
+        if (pattern == 1) {
+            // the code plane of a Q4_K weight with k = 4096, rows in the one-vector GEMV's order
+            if (w->type != AXQ_Q4_K || w->k != 4096)
+                return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring_ex: the row pattern reads Q4_K weights with k = 4096");
+            int rows_per_wg = (int)((w->n_rows + grid - 1) / grid);
+            rows_per_wg = (rows_per_wg + 7) / 8 * 8;
+            const unsigned g2 = (unsigned)((w->n_rows + rows_per_wg - 1) / rows_per_wg);
+            if (in_flight <= 4) axq_read_rows_kernel<2><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev);
+            else if (in_flight <= 8) axq_read_rows_kernel<4><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev);
+            else axq_read_rows_kernel<7><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev);
+        } else {
+            const size_t n16 = w->alloc_bytes / 16;
+            if (n16 == 0) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring: empty weight");
+            if (nontemporal) launch_read_u<true>(in_flight, threads, grid, st, (const axq_u32x4 *)w->base, n16, sink_dev);
+            else launch_read_u<false>(in_flight, threads, grid, st, (const axq_u32x4 *)w->base, n16, sink_dev);
+        }
         AXQ_LAUNCH_CHECK(ctx, "axq_bench_read_ring");
     }
+    if (streams > 1 && (rc = axq_aux_join(ctx, streams))) return rc;
     return AXQ_OK;
 }
 

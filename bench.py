@@ -36,7 +36,10 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def make_ring(ctx, qtype, n, k, copies, outlier_p, seed0=1234):
+RING_SEED0 = 1234  # copy i of a ring is drawn with seed RING_SEED0 + i
+
+
+def make_ring(ctx, qtype, n, k, copies, outlier_p, seed0=RING_SEED0):
     """`copies` device-resident weights, generated and quantised on the device."""
     from axonml_amd._lib import MEM_DEVICE
 
@@ -137,6 +140,20 @@ def check_against_oracle(ctx, w_handle, qtype, n, k, x, y_dev):
     want = o.matmul_ref(int(qtype), packed, x, n, k)
     denom = np.maximum(np.abs(want), 1e-2 * np.abs(want).max())
     return float((np.abs(got - want) / denom).max()), packed
+
+
+def codes_bit_exact(ctx, packed, qtype, n, k, outlier_p, seed):
+    """The other half of the same-run gate (quantize.rs:82-205 restated on the device): the f32 weight the device drew
+    for ring copy 0 comes back to the host, the oracle quantises it there, and every packed byte -- codes and f16
+    scales -- has to equal what the device quantiser left in the weight the benchmark multiplies with."""
+    import oracle as o
+
+    f = ctx.malloc(n * k * 4)
+    ctx.check(ctx.lib.axq_fill_normal_f32(ctx.handle, f, n * k, 0.0, 0.02, outlier_p, 0.5, seed))
+    w = ctx.to_host(f, (n * k,), np.float32)
+    ctx.free(f)
+    want = o.quantize(int(qtype), w)
+    return bool(want.size == packed.size and np.array_equal(want, packed))
 
 
 def cpu_baseline(packed, qtype, n, k, x, budget_s=12.0):
@@ -311,6 +328,10 @@ def main():
     log(f"headline: {head['us_per_step']:.2f} us/step, {head['gbps']:.0f} GB/s, max rel err vs oracle {err:.2e}")
     if err > 1e-3:
         sys.exit(f"bench.py: GPU result differs from the oracle (max rel err {err:.3e} > 1e-3)")
+    exact = codes_bit_exact(ctx, packed, T.Q4_K, N_HEAD, K_HEAD, 0.01, RING_SEED0)
+    log(f"headline weight: device-quantised codes and scales {'equal' if exact else 'DIFFER FROM'} the oracle's, byte for byte")
+    if not exact:
+        sys.exit("bench.py: the device quantiser's packed bytes differ from the oracle's on the headline weight")
     # the read ceiling of the same run: the same ring, the same grid, a kernel that only reads
     sink = ctx.malloc(256)
     ms_read, _, _, _ = time_read(ctx, ws, sink, args.steps, args.warmup)
@@ -335,6 +356,9 @@ def main():
              "headline_cache_resident_us": ms_hot * 1e3 if ms_hot else None,
              "headline_cache_resident_gbps": head["algorithmic_bytes"] / (ms_hot * 1e-3) / 1e9 if ms_hot else None,
              "max_rel_err_vs_oracle": err}
+    gate = {"codes_bit_exact": exact, "max_rel_err_vs_oracle": err, "tolerance": 1e-3,
+            "what": "ring copy 0 of the headline weight: the f32 the device drew, quantised by the oracle on the host, equals the "
+                    "device quantiser's packed image byte for byte; the GEMV on it against the oracle's dequantise -> f32 sgemm"}
     if not args.no_extras:
         cases = [(T.Q4_K, 4096, 14336, 1, 0.01), (T.Q8_0, 4096, 4096, 1, 0.0), (T.Q4_0, 11008, 4096, 1, 0.0),
                  (T.Q4_0, 4096, 11008, 1, 0.0), (T.Q4_1, 11008, 4096, 1, 0.0), (T.Q4_1, 4096, 11008, 1, 0.0),
@@ -396,6 +420,8 @@ def main():
                      "traffic_source": "profiles/gemv_q4k_14336x4096_hbm_counters.txt (profiler counter runs of this "
                                        "kernel), not measured in this run"},
         "cpu_baseline": cpu,
+        "codes_bit_exact": exact,
+        "correctness_gate": gate,
         "extra": extra,
     }
     print(json.dumps(out), flush=True)

@@ -301,6 +301,23 @@ AXQ_API int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, 
 AXQ_API int axq_bench_read_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
                                 uint32_t *sink_dev, int iters);
 
+/* The read-only kernel with its parameters open, for the table of what the memory system gives a launch of this size:
+ * wgs_per_cu workgroups per compute unit (1..8) of `threads` (256, 512, 1024), each lane keeping `in_flight` 16-byte loads
+ * in flight (4, 8, 16, 32; 16 at most with 1024 threads), non-temporal or plain loads; pattern 0 reads each weight's
+ * device image as contiguous shares, pattern 1 reads the code plane of a Q4_K weight with k = 4096 row step by row step,
+ * as the one-vector GEMV does (in_flight = 4, 8 or 14: two loads per step); streams > 1 spreads the launches over that
+ * many streams so that consecutive launches may overlap (the context's stream waits for all of them at the end).
+ * axq_bench_read_ring is (1, 512, 16, 1, 0, 1). */
+AXQ_API int axq_bench_read_ring_ex(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
+                                   uint32_t *sink_dev, int iters, int wgs_per_cu, int threads, int in_flight,
+                                   int nontemporal, int pattern, int streams);
+
+/* axq_bench_gemv_ring with the launches spread over `streams` streams (1..4): GEMVs that do not depend on each other
+ * (every launch of the ring reads the same x and overwrites the same y) may then overlap.  A figure beside the
+ * single-stream one, which is the one reported. */
+AXQ_API int axq_bench_gemv_ring_streams(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
+                                        const float *x_dev, int batch, float *y_dev, int iters, int streams);
+
 /* Enqueues `iters` launches of a plain copy kernel (reads `bytes`, writes `bytes`; both pointers and the
  * size multiples of 16).  A kernel of known traffic against which profiler memory counters are scaled. */
 AXQ_API int axq_bench_copy(axq_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes, int iters);

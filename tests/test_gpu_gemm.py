@@ -65,6 +65,27 @@ def test_ragged_tiles_of_the_block_of_32_kernel(ctx, qtype, m, n, k):
     _check(ctx, qtype, m, n, k, seed=m * 3 + n + k + qtype)
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_1, o.Q5_1, o.Q4_0, o.Q5_0, o.Q8_0, o.Q4_K])
+@pytest.mark.parametrize("m", [48, 300])
+def test_large_weights_block_minimums_beyond_256_and_scales_beyond_32(ctx, qtype, m):
+    """Weights around 300 with a spread of 100: block minimums of magnitude 256 and more, block scales of 16 to 40.  The
+    reference's dequantise -> f32 sgemm is finite there, so the GEMM has to be (operands formed as minimum x 256 or
+    16 d x 256 in f16 would overflow)."""
+    rng = np.random.default_rng(300 + qtype + m)
+    n, k = 160, 1024
+    w = (gen_weight(rng, n, k) * 5000.0 + 300.0).astype(np.float32)
+    xb = q.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    x = q.bf16_bits_to_f32(xb)
+    wq = o.quantize(qtype, w)
+    deq = o.dequantize(qtype, wq, n * k)
+    assert np.abs(deq).max() > 500
+    want = o.matmul_ref(qtype, wq, x, n, k)
+    got = q.quantized_matmul_bf16(xb, q.QuantizedTensor([n, k], qtype, wq), ctx)
+    assert np.isfinite(got).all()
+    assert max_rel_err(got, want) <= MATMUL_RTOL
+    assert max_rel_err(got, o.matmul_f64(deq.reshape(n, k), x), STRICT_FLOOR) <= MATMUL_RTOL
+
+
 @pytest.mark.parametrize("xscale", [1e-30, 1e30])
 def test_many_rows_of_extreme_magnitude(ctx, xscale):
     _check(ctx, o.Q4_K, 1030, 128, 512, seed=11, xscale=xscale)
