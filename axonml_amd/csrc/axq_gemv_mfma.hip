@@ -116,9 +116,9 @@ struct DQ4K {
     }
     __device__ static void set_meta(Raw &r, const uint8_t *row, int blk, int) { r.h = *reinterpret_cast<const uint4 *>(row + (blk >> 2) * 16); }
     __device__ static int group_k(int c, int g) { return c * 64 + g * 32; }
-    __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
+    __device__ static void lane_offsets(int k, int c, LaneOff &o) {
         // the code plane interleaves, per 64-pair slice, the first 16 bytes of every pair, then the second 16
-        const int cpr = a.k >> 6;
+        const int cpr = k >> 6;
         c = c < cpr ? c : cpr - 1; // lanes past the end of the row re-read its last chunk against x = 0
         int slice = c >> 6, pr = c & 63;
         int P = cpr - (slice << 6);
@@ -198,8 +198,8 @@ struct DQ4x {
     }
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
-    __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
-        const int nblk = a.k >> 5;
+    __device__ static void lane_offsets(int k, int c, LaneOff &o) {
+        const int nblk = k >> 5;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             int b = blk_index(c, g);
@@ -261,8 +261,8 @@ struct DQ5x {
     }
     __device__ static int blk_index(int c, int g) { return ((c >> 4) << 5) + g * 16 + (c & 15); }
     __device__ static int group_k(int c, int g) { return blk_index(c, g) * 32; }
-    __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
-        const int nblk = a.k >> 5;
+    __device__ static void lane_offsets(int k, int c, LaneOff &o) {
+        const int nblk = k >> 5;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             int b = blk_index(c, g);
@@ -326,8 +326,8 @@ struct DQ80 {
     // 16-byte vector v (0..3) of chunk c: vector index along the row; block = vector / 2
     __device__ static int vec_index(int c, int v) { return ((c >> 4) << 6) + (v >> 1) * 32 + (c & 15) * 2 + (v & 1); }
     __device__ static int group_k(int c, int g) { return vec_index(c, 2 * g) * 16; }
-    __device__ static void lane_offsets(const DpArgs &a, int c, LaneOff &o) {
-        const int nvec = a.k >> 4;
+    __device__ static void lane_offsets(int k, int c, LaneOff &o) {
+        const int nvec = k >> 4;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             int v0 = vec_index(c, 2 * g);
@@ -499,7 +499,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
     typename T::Raw buf[NB];
     uint4 hm[NM];
     LaneOff lo;
-    T::lane_offsets(a, c, lo);
+    T::lane_offsets(a.k, c, lo);
     const int wg_row0 = blockIdx.x * a.G * rows_per_group;
     const Bases bases = {a.codes + (size_t)wg_row0 * a.codes_pitch, a.meta + (size_t)wg_row0 * a.meta_pitch,
                          a.qh + (size_t)wg_row0 * a.qh_pitch};
@@ -706,7 +706,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     uint4 hm[NM];
     uint4 *wmeta = reinterpret_cast<uint4 *>(red + a.G * rows_per_group * red_stride) + wave * 64 * NM;
     LaneOff lo;
-    T::lane_offsets(a, c, lo);
+    T::lane_offsets(a.k, c, lo);
     const int wg_row0 = blockIdx.x * a.G * rows_per_group;
     const Bases bases = {a.codes + (size_t)wg_row0 * a.codes_pitch, a.meta + (size_t)wg_row0 * a.meta_pitch,
                          a.qh + (size_t)wg_row0 * a.qh_pitch};
@@ -861,6 +861,254 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     }
 }
 
+#ifdef AXQ_STAMPS
+// Development builds only (-DAXQ_STAMPS): every wave keeps wall-clock stamps (100 MHz) of its progress in LDS (the last
+// 4 KB of the 160) and copies them out when it ends, into a buffer the host has set with axq_debug_set_stamps:
+// [launch % 4][workgroup][wave (16)][slot (16)].
+__device__ unsigned long long *axq_stamps;
+__device__ unsigned int axq_stamp_launch;
+#define STAMP_INIT() unsigned long long *st_lds_ = reinterpret_cast<unsigned long long *>(reinterpret_cast<uint8_t *>(lds_raw) + 156 * 1024) + wave * 16; \
+                     if (lane < 16) st_lds_[lane] = 0
+#define STAMP(slot) do { if (lane == 0) st_lds_[slot] = wall_clock64(); } while (0)
+#define STAMP_END() do { unsigned long long *g_ = axq_stamps; if (g_ && lane < 16) { \
+                         g_[((((size_t)(*(volatile unsigned int *)&axq_stamp_launch & 3) * gridDim.x + blockIdx.x) * 16 + wave) * 16) + lane] = st_lds_[lane]; } \
+                         __syncthreads(); if (g_ && blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&axq_stamp_launch, 1u); } while (0)
+#else
+#define STAMP_INIT() do {} while (0)
+#define STAMP(slot) do {} while (0)
+#define STAMP_END() do {} while (0)
+#endif
+
+// ---------------------------------------------------------------------------
+// The kernel with waves of two kinds.  Whoever splits x cannot request weights meanwhile, and whoever stands at a
+// weight request (the compute unit's places for loads in flight taken) cannot split: in the kernels above x is split by
+// the waves that also own the weights, and the memory pipeline drains while they do it.  Here a workgroup is NS
+// "split" waves, which own no weights (they fetch x, split it -- two tasks per lane at K = 4096 -- and stage it in LDS),
+// beside the G x S weight waves, which start requesting at once, three row steps and the round's scale records, and
+// meet the split waves at one LDS-only barrier; from there on the ring runs as in gemv_dp_kernel with per-round
+// records.  The split waves are the workgroup's first, so their requests for x stand in front of the weights'.  The
+// workgroup's row steps are dealt to its G row groups in turn (group g takes steps g, g + G, ...).
+//
+// Scalar arguments instead of a struct passed by value: the first fourteen dwords are preloaded into scalar
+// registers when the wave starts (the file is compiled with -amdgpu-kernarg-preload-count), so the pointers the first
+// loads need are there without a trip to memory.
+// ---------------------------------------------------------------------------
+template <class T, int NB, int NB0, int NS>
+__global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__ x, const uint8_t *__restrict__ codes,
+                                                               const uint8_t *__restrict__ meta, uint32_t cp, uint32_t mp, int n_rows, int k,
+                                                               int steps, int flags, float eps, float *__restrict__ y,
+                                                               const float *__restrict__ bias, const float *__restrict__ aux,
+                                                               const uint8_t *__restrict__ qhp, uint32_t qp) {
+    static_assert(T::ROUND_META && NB <= 8 && NB0 <= NB && NB0 >= 1, "per-round scale records; a ring of at most eight steps");
+    // scale records of a round of NB steps: 4 NB rows x CPR 16-byte chunks of this wave's K slice, in NM loads of 64 lanes
+    constexpr int MSB = T::META_SLICE_BYTES, CPR = MSB / 16, NM = (4 * NB * CPR + 63) / 64;
+    constexpr int NST = 64 * NS, MAXT = 4;                                   // split threads; tasks of eight elements each of them takes at most
+    extern __shared__ uint4 lds_raw[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int mode = flags & 0xFF, ymode = (flags >> 8) & 0xFF, G = (flags >> 16) & 0xFF;
+    STAMP_INIT();
+    STAMP(0);
+    const int S = (k + 1023) >> 10;
+    // LDS: the split form of x (limb planes, then group records), a spare slot, per-wave sums of a fused RMSNorm, the
+    // reduction buffer, the weight waves' patches of scale records
+    uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw);
+    const int kpad = (k + 15) & ~15;
+    uint4 *wgrp = reinterpret_cast<uint4 *>(wplanes + (size_t)4 * kpad);
+    const int n16 = (int)(axq_split_bytes(k) >> 4);
+    float *wsum = reinterpret_cast<float *>(lds_raw + n16 + 1);
+    float *red = reinterpret_cast<float *>(lds_raw + n16 + 1 + 4);
+    // `steps` 4-row steps per workgroup, dealt to its G row groups in turn: group g takes steps g, g + G, g + 2 G, ...
+    const int wg_rows = steps * 4;
+    const int red_stride = 4 * S; // partial sums per output row in the LDS reduction buffer
+
+    if (wave < NS) {
+        // ---- split waves: x (times the norm weights of a fused RMSNorm) -> split form in LDS
+        const int ntask = k >> 3; // K is a multiple of 64: whole quads of tasks
+        uint4 xa[MAXT], xb[MAXT], ea[MAXT], eb[MAXT];
+#pragma unroll
+        for (int u = 0; u < MAXT; u++) {
+            if (u * NST < ntask) {
+                int t = tid + u * NST;
+                t = t < ntask ? t : (t & 3);
+                const uint4 *px = reinterpret_cast<const uint4 *>(x + (size_t)t * 8);
+                xa[u] = px[0]; xb[u] = px[1];
+                if (mode == AXQ_X_RMSNORM) {
+                    const uint4 *pe = reinterpret_cast<const uint4 *>(aux + (size_t)t * 8);
+                    ea[u] = pe[0]; eb[u] = pe[1];
+                }
+            }
+        }
+        STAMP(1);
+        auto unpack = [](const uint4 &lo, const uint4 &hi, float (&v)[8]) {
+            v[0] = __builtin_bit_cast(float, lo.x); v[1] = __builtin_bit_cast(float, lo.y);
+            v[2] = __builtin_bit_cast(float, lo.z); v[3] = __builtin_bit_cast(float, lo.w);
+            v[4] = __builtin_bit_cast(float, hi.x); v[5] = __builtin_bit_cast(float, hi.y);
+            v[6] = __builtin_bit_cast(float, hi.z); v[7] = __builtin_bit_cast(float, hi.w);
+        };
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < MAXT; u++) {
+            if (u * NST < ntask) {
+                const int t = tid + u * NST;
+                const bool live = t < ntask;
+                float xv[8];
+                unpack(xa[u], xb[u], xv);
+                if (mode == AXQ_X_RMSNORM) {
+                    // RMSNorm::forward (llm/src/llama.rs:158-187); the 1 / rms is one factor on the result
+                    float ev[8];
+                    unpack(ea[u], eb[u], ev);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        if (live) ss = fmaf(xv[i], xv[i], ss);
+                        xv[i] *= ev[i];
+                    }
+                }
+                if (live) axq_split8(xv, t, true, wplanes, wgrp, kpad);
+            }
+        }
+        if (mode == AXQ_X_RMSNORM) {
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+            if (lane == 0) wsum[wave] = ss;
+        }
+        STAMP(2);
+        lds_only_barrier(); // x is staged
+        STAMP(3);
+    } else {
+        // ---- weight waves
+        const int ww = wave - NS;
+        const int g_idx = ww / S, slice = ww - g_idx * S;
+        const int blk = lane >> 2, j = lane & 3;
+        const int c = (slice << 4) + blk; // this lane's 64-weight chunk of the row
+        const int my_steps = (steps - g_idx + G - 1) / G; // this group's share
+        float *red_lane = red + (4 * g_idx + j) * red_stride + slice * 4 + (lane >> 4);
+        uint4 *wmeta = lds_raw + n16 + 1 + 4 + (wg_rows * red_stride) / 4 + ww * 64 * NM;
+        typename T::Raw buf[NB];
+        uint4 hm[NM];
+        LaneOff lo;
+        T::lane_offsets(k, c, lo);
+        const int wg_row0 = blockIdx.x * wg_rows;
+        const Bases bases = {codes + (size_t)wg_row0 * cp, meta + (size_t)wg_row0 * mp, qhp + (size_t)wg_row0 * qp};
+        const int rl0 = 4 * g_idx + j, rl_last = n_rows - 1 - wg_row0; // rows relative to the workgroup's first
+        const int gstride = 4 * G;                                            // rows from one of the group's steps to its next
+        uint32_t moff[NM];
+        int mrl0[NM], mst[NM];
+        {
+            const int row_bytes = T::meta_row_bytes(k);
+#pragma unroll
+            for (int i = 0; i < NM; i++) {
+                const int flat = i * 64 + lane, off = slice * MSB + (flat % CPR) * 16;
+                const int r = flat / CPR < 4 * NB ? flat / CPR : 4 * NB - 1; // lanes beyond the round's rows repeat its last
+                moff[i] = (uint32_t)(off + 16 <= row_bytes ? off : row_bytes - 16);
+                mrl0[i] = 4 * g_idx + (r & 3); // row r of the round: row r % 4 of its step r / 4
+                mst[i] = r >> 2;
+            }
+        }
+        auto request = [&](int step, int b) {
+            const int s = step < my_steps ? step : 0;
+            int rl = rl0 + gstride * s;
+            rl = rl < rl_last ? rl : rl_last;
+            const RowOff ro = {(uint32_t)rl * cp, (uint32_t)rl * mp, (uint32_t)rl * qp};
+            if (b == 0) { // rows past the group's steps belong to the next group or repeat the matrix's last row: read, not used
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    int sm = s + mst[i];
+                    sm = sm < my_steps ? sm : 0;
+                    int rlm = mrl0[i] + gstride * sm;
+                    rlm = rlm < rl_last ? rlm : rl_last;
+                    hm[i] = ld16(bases.meta, (uint32_t)rlm * mp + moff[i]);
+                }
+            }
+            T::load_codes(bases, ro, lo, buf[b]);
+        };
+        // three steps before x is staged (with the round's records and the split waves' x a few more loads than the compute
+        // unit holds in flight: x returns first and makes room), the ring's last after the barrier
+#pragma unroll
+        for (int b = 0; b < NB0; b++) request(b, b);
+        STAMP(1);
+        lds_only_barrier(); // x is staged
+        STAMP(3);
+        XOp xo;
+        fetch_xop<T>(wplanes, wgrp, kpad, k, j, c, xo);
+#pragma unroll
+        for (int b = NB0; b < NB; b++) request(b, b);
+        STAMP(4);
+        const bool writer = (blk & 3) == 3;
+        const int red_step = gstride * red_stride;
+        auto fold = [&](int b, int step) {
+            if (b == 0) { // the wave's own patch: LDS serves a wave's stores and loads in order
+#pragma unroll
+                for (int i = 0; i < NM; i++) wmeta[i * 64 + lane] = hm[i];
+            }
+            T::set_meta(buf[b], reinterpret_cast<const uint8_t *>(wmeta) + (b * 4 + j) * MSB, blk, c);
+#ifdef AXQ_TIMING_NOFOLD // timing builds only (results not valid): the loads are waited for and nothing is computed
+            float tot = __builtin_bit_cast(float, reinterpret_cast<const uint32_t *>(&buf[b])[0] ^ reinterpret_cast<const uint32_t *>(&buf[b])[7]) + xo.sg[0];
+#else
+            float tot = sum_within_row(T::dot(buf[b], xo, c));
+#endif
+            if (writer) red_lane[step * red_step] = tot;
+            STAMP(5 + (step < 8 ? step : 8));
+        };
+        const int rounds = (my_steps + NB - 1) / NB;
+        int step = 0;
+        for (int round = 0; round < rounds - 1; round++, step += NB) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                fold(b, step + b);
+                request(step + NB + b, b); // steps past the end re-read the first (cache hits): every wave's count of loads stays the same
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+            if (step + b < my_steps) fold(b, step + b);
+    }
+
+    // partial sums -> y, in a fixed order, by every thread of the workgroup
+    __syncthreads();
+    STAMP(14);
+    const int nthreads = (int)blockDim.x;
+    float inv = 1.0f;
+    if (mode == AXQ_X_RMSNORM) {
+        float tot = 0.f;
+#pragma unroll
+        for (int i = 0; i < NS; i++) tot += wsum[i];
+        inv = 1.0f / sqrtf(tot / (float)k + eps);
+    }
+    auto row_total = [&](int t) { // slice by slice, the four DPP rows of each in order
+        const float4 *pr = reinterpret_cast<const float4 *>(red + (size_t)t * red_stride);
+        float tot = 0.f;
+        for (int s2 = 0; s2 < S; s2++) {
+            float4 v = pr[s2];
+            tot += (v.x + v.y) + (v.z + v.w);
+        }
+        return tot * inv;
+    };
+    if (ymode == AXQ_Y_SWIGLU) {
+        // rows 8b..8b+3 are gate rows, 8b+4..8b+7 the up rows of the same outputs (wg_rows is a multiple of 8)
+        for (int t = tid; t < (wg_rows >> 1); t += nthreads) {
+            const int lg = ((t >> 2) << 3) + (t & 3);
+            const int row = blockIdx.x * wg_rows + lg;
+            if (row + 4 < n_rows) {
+                const float g = row_total(lg), u = row_total(lg + 4);
+                y[(blockIdx.x * wg_rows >> 1) + t] = (g * (1.0f / (1.0f + expf(-g)))) * u;
+            }
+        }
+        STAMP(15);
+        STAMP_END();
+        return;
+    }
+    for (int t = tid; t < wg_rows; t += nthreads) {
+        int row = blockIdx.x * wg_rows + t;
+        if (row < n_rows) {
+            const float tot = row_total(t);
+            y[row] = bias ? tot + bias[row] : tot;
+        }
+    }
+    STAMP(15);
+    STAMP_END();
+}
+
 __global__ void __launch_bounds__(256) prep_x_kernel(const float *x, int k, uint8_t *xq) {
     const int kpad = (k + 15) & ~15;
     stage_x(x, k, xq, reinterpret_cast<uint4 *>(xq + (size_t)4 * kpad), (int)(blockIdx.x * blockDim.x + threadIdx.x),
@@ -931,6 +1179,50 @@ int launch_q4k_rounds<DQ4K>(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsign
     return 1;
 }
 
+// The kernel with split waves: a raw x, K within eight 1024-wide slices and four tasks per split thread.  The row steps
+// are dealt to workgroups (one per compute unit) and, inside a workgroup, to G row groups in turn.
+template <class T>
+int launch_sw(axq_ctx *ctx, const DpArgs &a) {
+    constexpr int NS = 4; // split waves: two tasks per lane at K = 4096 (8 measured slower, 2 much slower)
+    static std::atomic<uint64_t> lds_allowed[8];
+    const int S = a.S;
+    if (S > 8 || (a.k >> 3) > 4 * 64 * NS) return 0;
+    // the per-round scale loads are 16 bytes wide: the rows of the meta plane have to be whole 16-byte pieces
+    if (T::meta_row_bytes(a.k) % 16 != 0 || a.meta_pitch % 16 != 0 || T::meta_row_bytes(a.k) < 16) return 0;
+    int G = 8 / S; // eight weight waves (twelve, three per SIMD, measured slower: 8.7 against 8.1 us at 14336 x 4096)
+    const int rowsteps = (a.n_rows + 3) / 4;
+    const int cus = ctx->prop.multiProcessorCount * ctx->gemv_wgs_per_cu;
+    int steps = (rowsteps + cus - 1) / cus;
+    if (a.ymode == AXQ_Y_SWIGLU && (steps & 1)) steps++; // a workgroup must hold whole gate/up groups of 8 rows
+    if (steps < G) G = steps;
+    const unsigned grid = (unsigned)((rowsteps + steps - 1) / steps);
+    const int per_group = (steps + G - 1) / G;
+    const int nb = per_group < 4 ? per_group : 4; // ring depth: deeper rings measured slower (a wave that stands at its requests folds nothing)
+    const int cpr = T::META_SLICE_BYTES / 16, nm = (4 * nb * cpr + 63) / 64;
+    size_t lds = axq_split_bytes(a.k) + 16 + 64 + (size_t)steps * 4 * 4 * S * sizeof(float) + (size_t)(S * G) * nm * 1024;
+    if (lds > 160 * 1024) return 0;
+    const unsigned block = (unsigned)(64 * (S * G + NS));
+    const int flags = a.mode | (a.ymode << 8) | (G << 16);
+    auto go = [&](auto kern, std::atomic<uint64_t> &mask) -> int {
+#ifdef AXQ_STAMPS
+        lds = 160 * 1024; // the stamps live in the last 4 KB
+#endif
+        if (lds > 64 * 1024) {
+            const int st = axq_allow_lds(ctx, reinterpret_cast<const void *>(kern), mask, 160 * 1024);
+            if (st != AXQ_OK) return st;
+        }
+        kern<<<grid, block, lds, ctx->stream>>>(a.x, a.codes, a.meta, (uint32_t)a.codes_pitch, (uint32_t)a.meta_pitch, a.n_rows, a.k, steps, flags,
+                                                a.eps, a.y, a.bias, a.aux, a.qh, (uint32_t)a.qh_pitch);
+        return 1;
+    };
+    switch (nb) {
+    case 1: return go(&gemv_sw_kernel<T, 1, 1, NS>, lds_allowed[1]);
+    case 2: return go(&gemv_sw_kernel<T, 2, 2, NS>, lds_allowed[2]);
+    case 3: return go(&gemv_sw_kernel<T, 3, 3, NS>, lds_allowed[3]);
+    default: return go(&gemv_sw_kernel<T, 4, 3, NS>, lds_allowed[4]);
+    }
+}
+
 // 1 = launched, 0 = the shape is not this kernel's, < 0 = status
 template <class T>
 int launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux, float eps,
@@ -964,6 +1256,11 @@ int launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *
     size_t lds = (size_t)a.G * steps * 4 * a.S * 4 * sizeof(float);
     lds += axq_split_bytes(a.k) + 16 + 64;
     if (lds > 160 * 1024) return 0;
+    static const bool sw_off = getenv("AXQ_GEMV_SW") && getenv("AXQ_GEMV_SW")[0] == '0'; // development knob: no split waves
+    if (!xq && !sw_off) {
+        const int r = launch_sw<T>(ctx, a);
+        if (r != 0) return r;
+    }
     if (!xq) {
         const int r = launch_q4k_rounds<T>(ctx, a, grid, block, lds);
         if (r != 0) return r;
@@ -1021,3 +1318,12 @@ bool axq_dev_gemv_dp_covers(const axq_weight *w) {
     default: return false;
     }
 }
+
+#ifdef AXQ_STAMPS
+extern "C" __attribute__((visibility("default"))) int axq_debug_set_stamps(void *buf) {
+    unsigned int zero = 0;
+    if (hipMemcpyToSymbol(HIP_SYMBOL(axq_stamps), &buf, sizeof buf) != hipSuccess) return -1;
+    if (hipMemcpyToSymbol(HIP_SYMBOL(axq_stamp_launch), &zero, sizeof zero) != hipSuccess) return -1;
+    return 0;
+}
+#endif
