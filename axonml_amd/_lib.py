@@ -117,6 +117,10 @@ SIGNATURES = {
     "axq_bench_read_ring": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i]),
     "axq_bench_read_ring_ex": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i]),
     "axq_bench_gemv_ring_streams": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i, _vp, _i, _i]),
+    "axq_bench_graph_create": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i, _vp, _i, C.POINTER(_vp)]),
+    "axq_bench_graph_create_read": (_i, [_vp, C.POINTER(_vp), _i, _i, _vp, _i, C.POINTER(_vp)]),
+    "axq_bench_graph_launch": (_i, [_vp, _vp, _i]),
+    "axq_bench_graph_destroy": (None, [_vp, _vp]),
     "axq_bench_copy": (_i, [_vp, _vp, _vp, _sz, _i]),
     "axq_sample_token": (_i, [_vp, _vp, _i, _vp, _i, C.POINTER(SamplingConfig), C.c_float, C.POINTER(C.c_int32), _vp, _i]),
     "axq_model_set_sampling": (_i, [_vp, C.POINTER(SamplingConfig), C.c_uint64]),

@@ -53,6 +53,17 @@ struct DpArgs {
     float eps;
     int ymode;     // AXQ_Y_PLAIN or AXQ_Y_SWIGLU
 };
+// The kernels take these fields as scalar arguments, the ones the first loads need in front: the first fourteen dwords
+// are preloaded into scalar registers when a wave starts (-amdgpu-kernarg-preload-count), a struct passed by value is not.
+// shape = S | G << 8 | steps << 16, flags = mode | ymode << 8.
+#define DP_KERNEL_PARAMS const float *p_x, const uint8_t *p_codes, const uint8_t *p_meta, uint32_t p_cp, uint32_t p_mp, int p_n_rows, int p_k, \
+                         int p_shape, int p_flags, float p_eps, float *p_y, const float *p_bias, const float *p_aux, const uint8_t *p_qh, uint32_t p_qp, \
+                         const uint8_t *p_xq
+#define DP_KERNEL_ARGS DpArgs{p_codes, p_meta, p_qh, p_cp, p_mp, p_qp, p_x, p_bias, p_xq, p_y, p_n_rows, p_k, p_shape & 0xFF, (p_shape >> 8) & 0xFF, 1, \
+                              p_shape >> 16, p_flags & 0xFF, p_aux, p_eps, (p_flags >> 8) & 0xFF}
+#define DP_LAUNCH_ARGS(a) (a).x, (a).codes, (a).meta, (uint32_t)(a).codes_pitch, (uint32_t)(a).meta_pitch, (a).n_rows, (a).k, \
+                          ((a).S | ((a).G << 8) | ((a).steps << 16)), ((a).mode | ((a).ymode << 8)), (a).eps, (a).y, (a).bias, (a).aux, (a).qh, \
+                          (uint32_t)(a).qh_pitch, (a).xq
 
 __device__ inline float f16lo(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v & 0xFFFF))); }
 __device__ inline float f16hi(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v >> 16))); }
@@ -442,7 +453,8 @@ __device__ inline void lds_only_barrier() {
 // steps x 2 loads fill the compute unit's 64 places, and no refill waits.
 // ---------------------------------------------------------------------------
 template <class T, int NB, bool PRE, bool RND>
-__global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(DpArgs a) {
+__global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(DP_KERNEL_PARAMS) {
+    const DpArgs a = DP_KERNEL_ARGS;
     static_assert(!RND || (!PRE && T::ROUND_META && NB <= 4), "per-round scale records: a raw x, a type that has them, at most four steps per round");
     constexpr int MSB = T::META_SLICE_BYTES, NM = MSB / 64, CPR = MSB / 16; // scale loads per round, 16-byte chunks per row
     extern __shared__ uint4 lds_raw[];
@@ -666,7 +678,8 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(Dp
 // x[k] w[k] and leave their slices' sums of squares in LDS for the final reduction.
 // ---------------------------------------------------------------------------
 template <class T, int NB>
-__global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(DpArgs a) {
+__global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(DP_KERNEL_PARAMS) {
+    const DpArgs a = DP_KERNEL_ARGS;
     extern __shared__ uint4 lds_raw[];
     constexpr int SLICE_K = 1024, REGION16 = (4 * SLICE_K + (SLICE_K / 32) * 16) / 16; // a wave's split x, in 16-byte units
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1131,13 +1144,13 @@ int launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, siz
             (st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), lds_allowed_w, 160 * 1024)) != AXQ_OK)
             return st;
         if (lds_w <= 160 * 1024) {
-            gemv_dpw_kernel<T, NB><<<grid, block, lds_w, ctx->stream>>>(a);
+            gemv_dpw_kernel<T, NB><<<grid, block, lds_w, ctx->stream>>>(DP_LAUNCH_ARGS(a));
             return AXQ_OK;
         }
     }
     if (lds > 64 * 1024 && (st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<T, NB, PRE, false>), lds_allowed, 160 * 1024)) != AXQ_OK)
         return st;
-    gemv_dp_kernel<T, NB, PRE, false><<<grid, block, lds, ctx->stream>>>(a);
+    gemv_dp_kernel<T, NB, PRE, false><<<grid, block, lds, ctx->stream>>>(DP_LAUNCH_ARGS(a));
     return AXQ_OK;
 }
 
@@ -1174,8 +1187,8 @@ int launch_q4k_rounds<DQ4K>(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsign
         if (st == AXQ_OK) st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dp_kernel<DQ4K, 4, false, true>), lds_allowed[1], 160 * 1024);
         if (st != AXQ_OK) return st;
     }
-    if (a.steps == 3) gemv_dp_kernel<DQ4K, 3, false, true><<<grid, block, lds, ctx->stream>>>(a);
-    else gemv_dp_kernel<DQ4K, 4, false, true><<<grid, block, lds, ctx->stream>>>(a);
+    if (a.steps == 3) gemv_dp_kernel<DQ4K, 3, false, true><<<grid, block, lds, ctx->stream>>>(DP_LAUNCH_ARGS(a));
+    else gemv_dp_kernel<DQ4K, 4, false, true><<<grid, block, lds, ctx->stream>>>(DP_LAUNCH_ARGS(a));
     return 1;
 }
 

@@ -4,6 +4,8 @@
 
 #include <stdio.h>
 #include <stdlib.h>
+#include <new>
+
 #include "axq_internal.h"
 
 namespace {
@@ -388,6 +390,99 @@ int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_we
         if (rc) return rc;
     }
     return AXQ_OK;
+}
+
+// A recorded ring: `iters` GEMV launches captured once into a graph and replayed as one submission (what a decode loop
+// does with its step).  The capture runs on the context's stream; nothing executes until the replay.
+struct axq_bench_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    int launches;
+};
+
+int axq_bench_graph_create(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first, const float *x_dev, int batch,
+                           float *y_dev, int iters, axq_bench_graph **out) {
+    if (!ctx || !out) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_graph_create: NULL argument");
+    *out = nullptr;
+    if (!weights || n_weights <= 0 || first < 0 || !x_dev || !y_dev || batch <= 0 || iters <= 0)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_graph_create: bad argument");
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    // every kernel the ring uses has run once before the capture (attributes are set on first use, outside any capture)
+    int rc = axq_dev_gemv(ctx, weights[first % n_weights], x_dev, batch, NULL, y_dev);
+    if (rc) return rc;
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    axq_bench_graph *g = new (std::nothrow) axq_bench_graph{nullptr, nullptr, iters};
+    if (!g) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "out of host memory");
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) {
+        delete g;
+        return axq_fail(ctx, AXQ_ERR_DRIVER, "hipStreamBeginCapture: %s", hipGetErrorString(e));
+    }
+    for (int i = 0; i < iters && rc == AXQ_OK; i++) {
+        const axq_weight *w = weights[(first + i) % n_weights];
+        rc = w ? axq_dev_gemv(ctx, w, x_dev, batch, NULL, y_dev) : axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_graph_create: NULL weight");
+    }
+    e = hipStreamEndCapture(ctx->stream, &g->graph);
+    if (rc == AXQ_OK && e != hipSuccess) rc = axq_fail(ctx, AXQ_ERR_DRIVER, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    if (rc == AXQ_OK) {
+        e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+        if (e != hipSuccess) rc = axq_fail(ctx, AXQ_ERR_DRIVER, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    }
+    if (rc != AXQ_OK) {
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        delete g;
+        return rc;
+    }
+    *out = g;
+    return AXQ_OK;
+}
+
+// The read-only kernel's ring (axq_bench_read_ring) recorded the same way.
+int axq_bench_graph_create_read(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first, uint32_t *sink_dev, int iters,
+                                axq_bench_graph **out) {
+    if (!ctx || !out) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_graph_create_read: NULL argument");
+    *out = nullptr;
+    if (!weights || n_weights <= 0 || first < 0 || !sink_dev || iters <= 0)
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_graph_create_read: bad argument");
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    int rc = axq_bench_read_ring(ctx, weights, n_weights, first, sink_dev, 1);
+    if (rc) return rc;
+    AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+    axq_bench_graph *g = new (std::nothrow) axq_bench_graph{nullptr, nullptr, iters};
+    if (!g) return axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "out of host memory");
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) {
+        delete g;
+        return axq_fail(ctx, AXQ_ERR_DRIVER, "hipStreamBeginCapture: %s", hipGetErrorString(e));
+    }
+    rc = axq_bench_read_ring(ctx, weights, n_weights, first, sink_dev, iters);
+    e = hipStreamEndCapture(ctx->stream, &g->graph);
+    if (rc == AXQ_OK && e != hipSuccess) rc = axq_fail(ctx, AXQ_ERR_DRIVER, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    if (rc == AXQ_OK) {
+        e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+        if (e != hipSuccess) rc = axq_fail(ctx, AXQ_ERR_DRIVER, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    }
+    if (rc != AXQ_OK) {
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        delete g;
+        return rc;
+    }
+    *out = g;
+    return AXQ_OK;
+}
+
+int axq_bench_graph_launch(axq_ctx *ctx, axq_bench_graph *g, int times) {
+    if (!ctx || !g) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_graph_launch: NULL argument");
+    for (int i = 0; i < times; i++) AXQ_HIP(ctx, hipGraphLaunch(g->exec, ctx->stream), AXQ_ERR_KERNEL_LAUNCH_FAILED);
+    return AXQ_OK;
+}
+
+void axq_bench_graph_destroy(axq_ctx *ctx, axq_bench_graph *g) {
+    if (!g) return;
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
 }
 
 int axq_bench_gemv_ring_streams(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first, const float *x_dev,

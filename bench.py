@@ -89,6 +89,32 @@ def time_gemv(ctx, ws, x_dev, y_dev, batch, steps, warmup):
                      len(ws), steps, warmup)
 
 
+def time_graph(ctx, ws, x_dev, y_dev, batch, warmup_replays=2, read_sink=None):
+    """The ring recorded once as a HIP graph (a whole number of trips round the ring, MIN_PER_REPEAT launches at least) and
+    replayed REPEATS times, each replay between its own pair of events: the same dependent launches as time_gemv's, handed
+    to the GPU in one submission, the way a decode loop replays its step.  Returns (median ms per launch, per-replay ms
+    per launch, launches per replay)."""
+    lib = ctx.lib
+    arr = (C.c_void_p * len(ws))(*[w.value for w in ws])
+    per = len(ws) * -(-MIN_PER_REPEAT // len(ws))
+    g = C.c_void_p()
+    if read_sink is not None:  # the read-only kernel's launches instead of the GEMV's
+        ctx.check(lib.axq_bench_graph_create_read(ctx.handle, arr, len(ws), 0, read_sink, per, C.byref(g)))
+    else:
+        ctx.check(lib.axq_bench_graph_create(ctx.handle, arr, len(ws), 0, x_dev, batch, y_dev, per, C.byref(g)))
+    try:
+        ctx.check(lib.axq_bench_graph_launch(ctx.handle, g, warmup_replays))
+        ctx.synchronize()
+        times = []
+        for _ in range(REPEATS):
+            ctx.timer_start()
+            ctx.check(lib.axq_bench_graph_launch(ctx.handle, g, 1))
+            times.append(ctx.timer_stop() / per)
+    finally:
+        lib.axq_bench_graph_destroy(ctx.handle, g)
+    return float(np.median(times)), times, per
+
+
 def time_read(ctx, ws, sink_dev, steps, warmup):
     """The same ring under a kernel that only reads each weight's device image, on the GEMV's grid."""
     lib = ctx.lib
@@ -97,7 +123,7 @@ def time_read(ctx, ws, sink_dev, steps, warmup):
                      len(ws), steps, warmup)
 
 
-def gemv_case(ctx, qtype, n, k, batch, steps, warmup, outlier_p=0.0, ring=True):
+def gemv_case(ctx, qtype, n, k, batch, steps, warmup, outlier_p=0.0, ring=True, graph=True):
     from axonml_amd import quant as q
 
     lib = ctx.lib
@@ -108,10 +134,16 @@ def gemv_case(ctx, qtype, n, k, batch, steps, warmup, outlier_p=0.0, ring=True):
     x = rng.standard_normal((batch, k)).astype(np.float32)
     x_dev = ctx.to_device(x)
     y_dev = ctx.malloc(batch * n * 4)
-    ms, times, per, untimed = time_gemv(ctx, ws, x_dev, y_dev, batch, steps, warmup)
+    ms_s, times_s, per_s, untimed = time_gemv(ctx, ws, x_dev, y_dev, batch, steps, warmup)
+    ms_g, times_g, per_g = time_graph(ctx, ws, x_dev, y_dev, batch) if graph and copies > 1 else (None, None, None)
+    # the figure of the case: the recorded graph when it is the faster way to hand over the same launches
+    use_graph = ms_g is not None and ms_g < ms_s
+    ms, times, per = (ms_g, times_g, per_g) if use_graph else (ms_s, times_s, per_s)
     algo_bytes = wbytes + 4 * batch * (n + k)
     res = {"type": str(q.QuantType(qtype)), "n": n, "k": k, "batch": batch, "us_per_step": ms * 1e3,
            "us_per_step_min_max": [min(times) * 1e3, max(times) * 1e3], "launches_per_repeat": per, "untimed_launches": untimed,
+           "submission": "hipGraph replay" if use_graph else "stream launches",
+           "us_per_step_stream_launches": ms_s * 1e3, "us_per_step_graph_replay": ms_g * 1e3 if ms_g is not None else None,
            "algorithmic_bytes": algo_bytes, "gbps": algo_bytes / (ms * 1e-3) / 1e9, "ring_copies": copies}
     res["frac_of_hbm_peak"] = res["gbps"] / HBM_PEAK_GBPS
     return res, ws, x, x_dev, y_dev
@@ -303,6 +335,7 @@ def main():
     ap.add_argument("--ring-only", action="store_true",
                     help="for kernel-trace profiles: skip the cache-resident leg, so that every launch of the GEMV kernel "
                          "but the one oracle check streams a ring copy from HBM")
+    ap.add_argument("--profile-graph", action="store_true", help="for kernel-trace profiles: one more pass of graph replays of the headline ring")
     ap.add_argument("--counter-probe", action="store_true",
                     help="for profiler counter runs: a few launches of a 256 MiB plain copy kernel, then the "
                          "headline GEMV ring; no oracle, no CPU leg, no JSON line")
@@ -334,13 +367,25 @@ def main():
         sys.exit("bench.py: the device quantiser's packed bytes differ from the oracle's on the headline weight")
     # the read ceiling of the same run: the same ring, the same grid, a kernel that only reads
     sink = ctx.malloc(256)
-    ms_read, _, _, _ = time_read(ctx, ws, sink, args.steps, args.warmup)
+    ms_read_s, _, _, _ = time_read(ctx, ws, sink, args.steps, args.warmup)
+    ms_read_g, _, _ = time_graph(ctx, ws, None, None, 1, read_sink=sink)
+    ms_read = min(ms_read_s, ms_read_g)  # the ceiling is whichever way of handing over the launches is faster, as for the GEMV
+    # launches that do not wait for each other: the same ring spread over three streams (a figure beside the reported one)
+    arr = (C.c_void_p * len(ws))(*[w.value for w in ws])
+    ms_streams, _, _, _ = time_ring(ctx, lambda first, n: ctx.check(lib.axq_bench_gemv_ring_streams(ctx.handle, arr, len(ws), first, x_dev, 1, y_dev, n, 3)),
+                                    len(ws), args.steps, args.warmup)
+    ms_read_streams, _, _, _ = time_ring(ctx, lambda first, n: ctx.check(lib.axq_bench_read_ring_ex(ctx.handle, arr, len(ws), first, sink, n, 1, 512, 16, 1, 0, 2)),
+                                         len(ws), args.steps, args.warmup)
     ctx.free(sink)
     read_gbps = lib.axq_packed_bytes(int(T.Q4_K), N_HEAD * K_HEAD) / (ms_read * 1e-3) / 1e9
-    log(f"read-only kernel over the same ring: {ms_read * 1e3:.2f} us/launch, {read_gbps:.0f} GB/s; "
-        f"the GEMV runs at {head['gbps'] / read_gbps:.2f} of it")
+    log(f"read-only kernel over the same ring: {ms_read * 1e3:.2f} us/launch ({ms_read_s * 1e3:.2f} as stream launches, {ms_read_g * 1e3:.2f} "
+        f"as a graph replay), {read_gbps:.0f} GB/s; the GEMV runs at {head['gbps'] / read_gbps:.2f} of it")
+    log(f"launches that may overlap: GEMV over 3 streams {ms_streams * 1e3:.2f} us/launch, read-only kernel over 2 streams "
+        f"{ms_read_streams * 1e3:.2f} us/launch")
     # cache-resident figure, labelled as such
     ms_hot = None if args.ring_only else time_gemv(ctx, ws[:1], x_dev, y_dev, 1, args.steps, args.warmup)[0]
+    if args.profile_graph:  # for kernel-trace profiles of the reported submission: replays of the recorded ring, nothing else after them
+        time_graph(ctx, ws, x_dev, y_dev, 1)
     free_case(ctx, ws, x_dev, y_dev)
 
     cpu = None
@@ -348,10 +393,24 @@ def main():
         cpu = cpu_baseline(packed, T.Q4_K, N_HEAD, K_HEAD, x)
         log(f"cpu baseline: {cpu['ms_per_step']:.1f} ms/step on {cpu['cores']} threads")
 
+    wq4k = lib.axq_packed_bytes(int(T.Q4_K), N_HEAD * K_HEAD)
     extra = {"read_ceiling_gbps": read_gbps, "read_ceiling_us": ms_read * 1e3,
+             "read_ceiling_us_stream_launches": ms_read_s * 1e3, "read_ceiling_us_graph_replay": ms_read_g * 1e3,
              "read_ceiling_note": "same run, same ring of weight copies, one 512-thread workgroup per compute unit reading each "
-                                  "copy's packed image with non-temporal 16-byte loads and keeping nothing",
+                                  "copy's packed image with non-temporal 16-byte loads and keeping nothing; the faster of stream "
+                                  "launches and a graph replay, as for the GEMV (profiles/read_only_kernel_sweep.txt: no grid, "
+                                  "workgroup size, depth or load type reads these 33 MB faster in launches that follow each other)",
              "frac_of_read_ceiling": head["gbps"] / read_gbps,
+             "headline_us_per_step_stream_launches": head["us_per_step_stream_launches"],
+             "headline_us_per_step_graph_replay": head["us_per_step_graph_replay"],
+             "overlapped_launches": {
+                 "note": "launches that do not wait for each other (ring spread over streams); beside the reported figure, which is "
+                         "for launches that follow each other on one stream",
+                 "gemv_3_streams_us_per_step": ms_streams * 1e3,
+                 "gemv_3_streams_gbps": head["algorithmic_bytes"] / (ms_streams * 1e-3) / 1e9,
+                 "gemv_3_streams_frac_of_hbm_peak": head["algorithmic_bytes"] / (ms_streams * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                 "read_only_2_streams_us_per_launch": ms_read_streams * 1e3,
+                 "read_only_2_streams_gbps": wq4k / (ms_read_streams * 1e-3) / 1e9},
              "headline_us_per_step_min_max_over_repeats": head["us_per_step_min_max"],
              "headline_cache_resident_us": ms_hot * 1e3 if ms_hot else None,
              "headline_cache_resident_gbps": head["algorithmic_bytes"] / (ms_hot * 1e-3) / 1e9 if ms_hot else None,
@@ -410,9 +469,11 @@ def main():
         "config": {"workload": "Q4_K GEMV 14336x4096, batch 1 (BASELINE config 3)", "quant_type": "Q4_K",
                    "n_rows": N_HEAD, "k": K_HEAD, "batch": 1, "ring_copies": head["ring_copies"],
                    "repeats": REPEATS, "launches_per_repeat": head["launches_per_repeat"],
-                   "internal_warmup": head["untimed_launches"],
-                   "timing": "median over `repeats` event-bracketed repeats of `launches_per_repeat` = max(200, steps / repeats) "
-                             "back-to-back launches each, after `internal_warmup` untimed launches",
+                   "internal_warmup": head["untimed_launches"], "submission": head["submission"],
+                   "timing": "median over `repeats` event-bracketed repeats of `launches_per_repeat` launches that follow each other "
+                             "on one stream, after `internal_warmup` untimed launches; measured twice, as plain stream launches "
+                             "(max(200, steps / repeats) per repeat) and as replays of one recorded hipGraph (a whole number of trips "
+                             "round the ring), and the faster way of handing the same launches over is reported (`submission`)",
                    "algorithmic_bytes_per_step": head["algorithmic_bytes"],
                    "inputs": "W~N(0,0.02) with 1% at +-0.5, x~N(0,1), generated and quantised on the device"},
         "roofline": {"bound": "hbm", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",

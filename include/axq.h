@@ -295,6 +295,17 @@ AXQ_API int axq_fill_normal_f32(axq_ctx *ctx, float *dst_dev, size_t n, float me
 AXQ_API int axq_bench_gemv_ring(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
                                 const float *x_dev, int batch, float *y_dev, int iters);
 
+/* The ring as a recorded graph: `iters` launches, launch i on weights[(first + i) % n_weights], captured once and replayed
+ * with one submission per axq_bench_graph_launch (`times` replays back to back).  Device pointers; the graph keeps
+ * them, so they must stay valid until axq_bench_graph_destroy. */
+typedef struct axq_bench_graph axq_bench_graph;
+AXQ_API int axq_bench_graph_create(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
+                                   const float *x_dev, int batch, float *y_dev, int iters, axq_bench_graph **out);
+AXQ_API int axq_bench_graph_create_read(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
+                                        uint32_t *sink_dev, int iters, axq_bench_graph **out); /* axq_bench_read_ring's launches */
+AXQ_API int axq_bench_graph_launch(axq_ctx *ctx, axq_bench_graph *g, int times);
+AXQ_API void axq_bench_graph_destroy(axq_ctx *ctx, axq_bench_graph *g);
+
 /* The same ring walked by a kernel that only reads each weight's device image (one 512-thread workgroup per
  * compute unit, non-temporal 16-byte loads): the rate the memory system gives a launch of that size, to set
  * beside the GEMV's.  sink_dev: four writable device bytes. */
