@@ -325,6 +325,85 @@ __global__ void quant_q4_k_kernel(const float *src, size_t numel, size_t nsb, ui
     }
 }
 
+// Q6_K (GGUF superblock of 16 sub-blocks of 16 elements, 210 bytes: ql[128], qh[64], int8 scales[16], f16 d).
+// One thread per sub-block, sixteen neighbouring lanes per superblock.  The quantiser rule is this build's own:
+// per sub-block a = max |x|, scale = a / 31; the superblock's d = max scale / 127 (stored as f16);
+// ls = round(127 / max_scale * scale) in 0..127; q = clamp(round(x / (d * ls)), -32, 31) with the f16-rounded d.
+// Element e = 128 n + 32 c + l keeps the low four bits of u = q + 32 in ql[64 n + 32 (c & 1) + l] (low nibble for
+// c < 2) and the upper two in qh[32 n + l] at bit 2 c.
+__global__ void quant_q6_k_kernel(const float *src, size_t numel, size_t nsb, uint8_t *out) {
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t sb = t >> 4;
+    const int s = (int)(t & 15);
+    const bool live = sb < nsb;
+    float x[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) x[i] = 0.0f;
+    if (live) {
+        const size_t start = sb * 256 + (size_t)s * 16;
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            if (start + i < numel) x[i] = src[start + i];
+    }
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) a = fmaxf(a, fabsf(x[i]));
+    const float scale = a / 31.0f;
+    float max_scale = scale;
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) max_scale = fmaxf(max_scale, __shfl_xor(max_scale, m));
+    const float inv = max_scale > 0.0f ? 127.0f / max_scale : 0.0f;
+    const int ls = round_clamp(inv * scale, 0.0f, 127.0f);
+    const uint16_t dh = f32_to_f16_bits(max_scale / 127.0f);
+    const float sd = f16_bits_to_f32(dh) * (float)ls;
+    // the sixteen codes u = q + 32, one per byte; low nibbles and upper bit pairs apart
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        lo[w] = hi[w] = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int q = sd == 0.0f ? 0 : round_clamp(x[4 * w + j] / sd, -32.0f, 31.0f);
+            const uint32_t u = (uint32_t)(q + 32);
+            lo[w] |= (u & 0x0Fu) << (8 * j);
+            hi[w] |= (u >> 4) << (8 * j);
+        }
+    }
+    // s = 8 n + 2 c + lh: the partner with c + 2 (lane s ^ 4) supplies the high nibbles of the same ql bytes; the
+    // lanes s + 2, s + 4, s + 6 supply the other bit pairs of the same qh bytes
+    const int c = (s >> 1) & 3, n = s >> 3, lh = s & 1;
+    uint32_t plo[4], h2[4], h4[4], h6[4];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        plo[w] = (uint32_t)__shfl_xor((int)lo[w], 4);
+        h2[w] = (uint32_t)__shfl_xor((int)hi[w], 2);
+        h4[w] = (uint32_t)__shfl_xor((int)hi[w], 4);
+        h6[w] = (uint32_t)__shfl_xor((int)hi[w], 6);
+    }
+    if (!live) return;
+    uint8_t *o = out + sb * 210;
+    if (c < 2) {
+        uint8_t *ql = o + 64 * n + 32 * c + 16 * lh;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t v = lo[w] | (plo[w] << 4);
+            store_u16(ql + 4 * w, (uint16_t)v);
+            store_u16(ql + 4 * w + 2, (uint16_t)(v >> 16));
+        }
+    }
+    if (c == 0) {
+        uint8_t *qh = o + 128 + 32 * n + 16 * lh;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t v = hi[w] | (h2[w] << 2) | (h4[w] << 4) | (h6[w] << 6);
+            store_u16(qh + 4 * w, (uint16_t)v);
+            store_u16(qh + 4 * w + 2, (uint16_t)(v >> 16));
+        }
+    }
+    o[192 + s] = (uint8_t)ls;
+    if (s == 0) store_u16(o + 208, dh);
+}
+
 // ---- F16: quantize.rs:212-218 --------------------------------------------
 // eight elements per thread where both sides are 16-byte aligned, one by one otherwise and for the last few
 __global__ void quant_f16_kernel(const float *src, size_t numel, uint16_t *out) {
@@ -465,6 +544,25 @@ __global__ void __launch_bounds__(128) dequant_kernel(int type, const uint8_t *p
             for (int j = 0; j < 4; j++) {
                 float a = sd * (float)((w >> (8 * j)) & 0x0F);
                 y[4 * i + j] = a - sm;
+            }
+        }
+        break;
+    }
+    case AXQ_Q6_K: { // elements 32 (t % 8) .. of superblock t / 8: two sub-blocks; y = (d * scale) * q
+        const size_t sb = t >> 3;
+        const int g = (int)(t & 7), n = g >> 2, c = g & 3;
+        const uint8_t *b = packed + sb * 210;
+        const float d = f16_bits_to_f32(load_u16(b + 208));
+        const float ds0 = d * (float)(int8_t)b[192 + 2 * g], ds1 = d * (float)(int8_t)b[192 + 2 * g + 1];
+        const uint8_t *ql = b + 64 * n + 32 * (c & 1), *qh = b + 128 + 32 * n;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const uint32_t wl = load_u16(ql + 2 * i), wh = load_u16(qh + 2 * i);
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int lo = (int)((wl >> (8 * j + 4 * (c >> 1))) & 0x0F), hi = (int)((wh >> (8 * j + 2 * c)) & 3);
+                const int q = (lo | (hi << 4)) - 32;
+                y[2 * i + j] = (i < 8 ? ds0 : ds1) * (float)q;
             }
         }
         break;
@@ -614,6 +712,27 @@ __global__ void __launch_bounds__(256) repack_lds_kernel(PlanarDesc d, uint8_t *
     }
 }
 
+// Q6_K: image [ql 128][qh 64][scales 16][d 2] <-> planes: codes = the rows' ql runs (128 bytes per superblock), qh = their
+// qh runs (64), meta = per row the superblocks' scales (16 bytes each) followed by their d values (2 bytes each).
+// One thread per 16-byte piece (13 per superblock, the last one scales and d); two bytes at a time on the image side.
+__global__ void __launch_bounds__(256) repack_q6k_kernel(PlanarDesc d, uint8_t *packed, bool to_planar, int64_t total) {
+    const int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= total * 13) return;
+    const int64_t t = v / 13;
+    const int piece = (int)(v - t * 13);
+    const int64_t row = t / d.blocks_per_row, sb = t - row * d.blocks_per_row;
+    uint8_t *img = packed + (size_t)t * 210;
+    uint8_t *pl, *im;
+    if (piece < 8) { pl = d.codes + (size_t)row * d.codes_pitch + (size_t)sb * 128 + 16 * piece; im = img + 16 * piece; }
+    else if (piece < 12) { pl = d.qh + (size_t)row * d.qh_pitch + (size_t)sb * 64 + 16 * (piece - 8); im = img + 128 + 16 * (piece - 8); }
+    else { pl = d.meta + (size_t)row * d.meta_pitch + (size_t)sb * 16; im = img + 192; }
+    if (to_planar) copy_u16s(pl, im, 16); else copy_u16s(im, pl, 16);
+    if (piece == 12) {
+        uint8_t *dp = d.meta + (size_t)row * d.meta_pitch + (size_t)d.blocks_per_row * 16 + (size_t)sb * 2;
+        if (to_planar) store_u16(dp, load_u16(img + 208)); else store_u16(img + 208, load_u16(dp));
+    }
+}
+
 inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
 
 } // namespace
@@ -629,6 +748,7 @@ int axq_dev_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, uin
     case AXQ_Q5_0: quant_q5_kernel<false><<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_Q5_1: quant_q5_kernel<true><<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_Q4_K: quant_q4_k_kernel<<<grid_for(nblk * 8, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_Q6_K: quant_q6_k_kernel<<<grid_for(nblk * 16, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_F16: quant_f16_kernel<<<grid_for((numel + 7) / 8, 256), 256, 0, ctx->stream>>>(src, numel, (uint16_t *)packed); break;
     case AXQ_F32:
         AXQ_HIP(ctx, hipMemcpyAsync(packed, src, numel * 4, hipMemcpyDeviceToDevice, ctx->stream), AXQ_ERR_COPY_FAILED);
@@ -642,7 +762,7 @@ int axq_dev_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, uin
 int axq_dev_dequantize(axq_ctx *ctx, int type, const uint8_t *packed, size_t numel, float *dst) {
     if (numel == 0) return AXQ_OK;
     switch (type) {
-    case AXQ_Q8_0: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q4_K: {
+    case AXQ_Q8_0: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q4_K: case AXQ_Q6_K: {
         size_t n32 = (numel + 31) / 32;
         dequant_kernel<<<grid_for(n32, 128), 128, 0, ctx->stream>>>(type, packed, numel, n32, dst);
         break;
@@ -674,6 +794,11 @@ int axq_dev_repack(axq_ctx *ctx, const axq_weight *w, uint8_t *packed, bool to_p
     d.type = w->type;
     size_t total = (size_t)(d.n_rows * d.blocks_per_row);
     if (total == 0) return AXQ_OK;
+    if (w->type == AXQ_Q6_K) {
+        repack_q6k_kernel<<<grid_for(total * 13, 256), 256, 0, ctx->stream>>>(d, packed, to_planar, (int64_t)total);
+        AXQ_LAUNCH_CHECK(ctx, "repack kernel");
+        return AXQ_OK;
+    }
     if ((reinterpret_cast<uintptr_t>(packed) & 15) == 0) { // the usual case: allocations are aligned far beyond that
         const unsigned grid = grid_for(total, 128);
         const int64_t n = (int64_t)total;

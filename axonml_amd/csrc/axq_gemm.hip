@@ -213,6 +213,37 @@ struct GQ80 {
     }
 };
 
+struct GQ6K { // GGUF Q6_K: a unit is one sub-block of 16 consecutive elements with its own int8 scale
+    static constexpr bool PRESCALED = true;
+    // d * scale * q reaches 127 * 32 times d: a smaller factor than WSCALE leaves weights up to 4000 finite in f16 and
+    // still keeps the low parts of weights above 8e-3 normal
+    static constexpr float WS = 16.0f;
+    struct Raw { uint4 ql, qh; int sc; uint32_t d; };
+    __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
+        // K step = 64 elements = sub-blocks 4 (kstep % 4) .. of superblock kstep / 4; s = 8 n + 2 c + lh
+        const int sb = kstep >> 2, s = (kstep & 3) * 4 + u4, n = s >> 3, c = (s >> 1) & 3, lh = s & 1;
+        r.ql = *reinterpret_cast<const uint4 *>(a.codes + row * a.codes_pitch + (size_t)sb * 128 + 64 * n + 32 * (c & 1) + 16 * lh);
+        r.qh = *reinterpret_cast<const uint4 *>(a.qh + row * a.qh_pitch + (size_t)sb * 64 + 32 * n + 16 * lh);
+        const uint8_t *m = a.meta + row * a.meta_pitch;
+        r.sc = (int)(int8_t)m[(size_t)sb * 16 + s];
+        r.d = *reinterpret_cast<const uint16_t *>(m + (size_t)(a.k >> 8) * 16 + (size_t)sb * 2);
+    }
+    __device__ static void cvt16(const Raw &r, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+        const int c = ((((kstep & 3) * 4 + u4) >> 1) & 3);
+        // (d * scale) * (u - 32) = u * ds - 32 ds: one rounding (fma) where the f32 reference has one as well
+        const float ds = WS * (h2f(r.d) * (float)r.sc), off = -32.0f * ds;
+        const uint32_t ql[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w}, qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t u = ((ql[j] >> (4 * (c >> 1))) & 0x0F0F0F0Fu) | (((qh[j] >> (2 * c)) & 0x03030303u) << 4);
+            w[4 * j + 0] = fmaf(ubyte<0>(u), ds, off); w[4 * j + 1] = fmaf(ubyte<1>(u), ds, off);
+            w[4 * j + 2] = fmaf(ubyte<2>(u), ds, off); w[4 * j + 3] = fmaf(ubyte<3>(u), ds, off);
+        }
+        k0 = u4 * 16;
+        k1 = k0 + 8;
+    }
+};
+
 struct GF16 {
     static constexpr bool PRESCALED = false;
     static constexpr float WS = 1.0f; // plain weights may be large: no headroom to give away
@@ -1542,6 +1573,7 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     if (p.q5) return launch_gemm_q5(ctx, a, p.splits, w->type);
     switch (w->type) {
     case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);
+    case AXQ_Q6_K: return launch_gemm<GQ6K>(ctx, a, p.splits);
     case AXQ_Q4_0: return launch_gemm<GQ4x<false>>(ctx, a, p.splits);
     case AXQ_Q4_1: return launch_gemm<GQ4x<true>>(ctx, a, p.splits);
     case AXQ_Q5_0: return launch_gemm<GQ5x<false>>(ctx, a, p.splits);

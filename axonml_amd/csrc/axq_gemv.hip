@@ -267,6 +267,43 @@ struct Q80 { // chunk = 16 int8 = half a block
     }
 };
 
+struct Q6K { // GGUF Q6_K; chunk = one sub-block of 16 elements: 16 bytes of low nibbles, 16 of bit pairs, an int8 scale
+    static constexpr int W = 16;
+    struct X { float xs[16]; };
+    struct Raw { uint4 ql, qh; int sc; uint32_t d; };
+    template <class F>
+    __device__ static void set_x(const GemvArgs &, F fetch, X &o) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float4 v = fetch(i);
+            o.xs[4 * i] = v.x; o.xs[4 * i + 1] = v.y; o.xs[4 * i + 2] = v.z; o.xs[4 * i + 3] = v.w;
+        }
+    }
+    __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
+        // sub-block s = 8 n + 2 c + lh of superblock sb: elements 128 n + 32 c + 16 lh ..
+        const int sb = chunk >> 4, s = chunk & 15, n = s >> 3, c = (s >> 1) & 3, lh = s & 1;
+        r.ql = *reinterpret_cast<const uint4 *>(a.codes + (size_t)row * a.codes_pitch + (size_t)sb * 128 + 64 * n + 32 * (c & 1) + 16 * lh);
+        r.qh = *reinterpret_cast<const uint4 *>(a.qh + (size_t)row * a.qh_pitch + (size_t)sb * 64 + 32 * n + 16 * lh);
+        const uint8_t *m = a.meta + (size_t)row * a.meta_pitch;
+        r.sc = (int)(int8_t)m[(size_t)sb * 16 + s];
+        r.d = *reinterpret_cast<const uint16_t *>(m + (size_t)(a.cpr >> 4) * 16 + (size_t)sb * 2);
+    }
+    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int chunk) {
+        const int c = (chunk >> 1) & 3;
+        const uint32_t ql[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w}, qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) { // codes centred before the multiply: no large sums cancel for an x with a mean
+            const uint32_t u = ((ql[w] >> (4 * (c >> 1))) & 0x0F0F0F0Fu) | (((qh[w] >> (2 * c)) & 0x03030303u) << 4);
+            a0 = fmaf(ubyte0(u) - 32.0f, x.xs[4 * w], a0);
+            a1 = fmaf(ubyte1(u) - 32.0f, x.xs[4 * w + 1], a1);
+            a0 = fmaf(ubyte2(u) - 32.0f, x.xs[4 * w + 2], a0);
+            a1 = fmaf(ubyte3(u) - 32.0f, x.xs[4 * w + 3], a1);
+        }
+        return (f16_bits_to_f32(r.d) * (float)r.sc) * (a0 + a1);
+    }
+};
+
 struct F16W { // chunk = 8 halfs
     static constexpr int W = 8;
     struct X { float xs[8]; };
@@ -601,6 +638,7 @@ int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, c
         if (rc == 1) continue;
         switch (w->type) {
         case AXQ_Q4_K: rc = launch<Q4K>(ctx, w, xb, bias, yb); break;
+        case AXQ_Q6_K: rc = launch<Q6K>(ctx, w, xb, bias, yb); break;
         case AXQ_Q4_0: rc = launch<Q4x<false>>(ctx, w, xb, bias, yb); break;
         case AXQ_Q4_1: rc = launch<Q4x<true>>(ctx, w, xb, bias, yb); break;
         case AXQ_Q5_0: rc = launch<Q5x<false>>(ctx, w, xb, bias, yb); break;

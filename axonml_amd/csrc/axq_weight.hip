@@ -62,10 +62,11 @@ int axq_weight_alloc(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, axq_weig
     case AXQ_Q5_0: w->codes_pitch = (size_t)k / 2; meta_per_block = 2; qh_per_block = 4; break;
     case AXQ_Q5_1: w->codes_pitch = (size_t)k / 2; meta_per_block = 4; qh_per_block = 4; break;
     case AXQ_Q4_K: w->codes_pitch = (size_t)k / 2; meta_per_block = 16; break;
+    case AXQ_Q6_K: w->codes_pitch = (size_t)k / 2; meta_per_block = 18; qh_per_block = 64; break; // scales, then the row's d values
     case AXQ_F16: w->codes_pitch = (size_t)k * 2; break;
     case AXQ_F32: w->codes_pitch = (size_t)k * 4; break;
     }
-    w->meta_pitch = nblk * meta_per_block;
+    w->meta_pitch = type == AXQ_Q6_K ? axq_align_up(nblk * meta_per_block, 16) : nblk * meta_per_block;
     w->qh_pitch = nblk * qh_per_block;
     size_t codes_bytes = axq_align_up(w->codes_pitch * (size_t)n_rows, 256);
     size_t meta_bytes = axq_align_up(w->meta_pitch * (size_t)n_rows, 256);

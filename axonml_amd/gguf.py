@@ -5,7 +5,8 @@ stops there; its `axonml quant convert` writes nothing a reader could load (quan
 implements the GGUF v2/v3 container as specified by ggml: little-endian header, typed metadata, tensor
 table, aligned data section.  Tensor payloads are ggml block images; `axq_gguf_convert_blocks` (device)
 turns Q4_0 / Q4_1 images into the reference's nibble order and back, every other supported type is
-byte-identical.  ggml types this library has no kernel for (Q2_K ... Q6_K, IQ*, ...) raise GGUFError.
+byte-identical (Q6_K among them: the reference has no such type, the block is ggml's).  ggml types this library
+has no kernel for (Q2_K, Q3_K, Q5_K, IQ*, ...) raise GGUFError.
 
 Tensor names and metadata keys of the loader follow llama.cpp's converter for the `llama` architecture,
 mapped onto the reference's LLaMA module names (crates/axonml-llm/src/llama.rs:782-822).
@@ -172,7 +173,7 @@ class GGUFReader:
         t = self.info(name)
         if t.quant_type is None:
             raise GGUFError(f"tensor {name}: ggml type {GGML_TYPE_NAMES.get(t.ggml_type, t.ggml_type)} is not supported "
-                            f"(supported: F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K)")
+                            f"(supported: F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q6_K)")
         return np.frombuffer(self._mm, dtype=np.uint8, count=t.nbytes, offset=self.data_start + t.offset)
 
     def close(self):
@@ -348,8 +349,20 @@ def load_llama(path, ctx=None, max_position_embeddings=None, permuted_qk=True):
 
         set_embedding(model, emb)
 
-        def linear(layer, which, name, heads=None):
-            qt = load_quantized_tensor(r, name, ctx)
+        def fused_as_f32(layer, group):
+            # q/k/v share one device weight and so do gate/up: one GEMV reads them all.  A file that mixes block
+            # types inside such a group (llama.cpp's Q4_K_M keeps some attn_v in Q6_K beside Q4_K q and k) has the
+            # group carried as f32 rows dequantised on the device: exact, at the price of the larger read.
+            names = [f"blk.{layer}.{_LINEAR_NAMES[w]}.weight" for w in group]
+            return len({r.info(n).ggml_type for n in names}) > 1
+
+        def linear(layer, which, name, heads=None, as_f32=False):
+            if as_f32:
+                from .quant import quantize_tensor
+
+                qt = quantize_tensor(load_f32(r, name, ctx), QuantType.F32, ctx)
+            else:
+                qt = load_quantized_tensor(r, name, ctx)
             if heads is not None and permuted_qk:
                 rows = qt.data.reshape(qt.shape[0], -1)
                 qt = QuantizedTensor(qt.shape, qt.quant_type, rows[rope_rows_to_half_split(qt.shape[0], heads)])
@@ -358,9 +371,10 @@ def load_llama(path, ctx=None, max_position_embeddings=None, permuted_qk=True):
         for layer in range(cfg["num_hidden_layers"]):
             model.set_norm(layer, 0, load_f32(r, f"blk.{layer}.attn_norm.weight", ctx))
             model.set_norm(layer, 1, load_f32(r, f"blk.{layer}.ffn_norm.weight", ctx))
+            mixed = {w: fused_as_f32(layer, g) for g in (("q", "k", "v"), ("gate", "up")) for w in g}
             for which, stem in _LINEAR_NAMES.items():
                 heads = {"q": cfg["num_attention_heads"], "k": cfg["num_key_value_heads"]}.get(which)
-                linear(layer, which, f"blk.{layer}.{stem}.weight", heads)
+                linear(layer, which, f"blk.{layer}.{stem}.weight", heads, mixed.get(which, False))
         model.set_norm(-1, 0, load_f32(r, "output_norm.weight", ctx))
         # tied embeddings: files without output.weight reuse the token embedding (llama.cpp does the same)
         linear(-1, "q", "output.weight" if "output.weight" in r.tensors else "token_embd.weight")

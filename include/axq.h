@@ -45,7 +45,9 @@ typedef struct axq_weight axq_weight;
 typedef struct axq_model axq_model;
 
 /* QuantType, crates/axonml-quant/src/types.rs:17-41, in the same order, with
- * Q4_K (256-element GGUF superblock) appended. */
+ * the 256-element GGUF superblock types appended: Q4_K (144 bytes) and Q6_K (210 bytes: 128 bytes of low nibbles,
+ * 64 of high bit pairs, sixteen int8 scales of 16 elements each, f16 d; w = d * scale * (q - 32)), the type llama.cpp
+ * keeps output.weight and part of the value and down projections in when it writes "Q4_0" and "Q4_K_M" files. */
 typedef enum {
     AXQ_Q8_0 = 0,
     AXQ_Q4_0 = 1,
@@ -55,7 +57,8 @@ typedef enum {
     AXQ_F16 = 5,
     AXQ_F32 = 6,
     AXQ_Q4_K = 7,
-    AXQ_TYPE_COUNT = 8
+    AXQ_Q6_K = 8,
+    AXQ_TYPE_COUNT = 9
 } axq_type;
 
 typedef enum {

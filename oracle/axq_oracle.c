@@ -37,6 +37,9 @@
  *     blocks derived from the reference source (zero block, ramp, half-way
  *     rounding cases, tail block, Q4_1 odd tail) and by the reference's own
  *     test inputs (types.rs:366-389, dequantize.rs:204-272).
+ *   Q6_K: as Q4_K below -- no reference code, no fixture; the layout and the dequantiser follow the published GGUF
+ *     block (pinned by hand-built superblocks, one-hot codes and an independent numpy statement of ggml's row
+ *     dequantiser), the QUANTISER rule is this build's own ("parity unpinned").
  *   Q5_0 / Q5_1 / Q4_K: the reference defines no codec for them (Q5_x silently
  *     aliases Q4_0, quantize.rs:47-50; Q4_K does not exist).  Byte layouts
  *     follow the public GGUF block spec and are pinned by hand-built blocks;
@@ -69,7 +72,8 @@ enum {
     AXO_Q5_1 = 4,
     AXO_F16 = 5,
     AXO_F32 = 6,
-    AXO_Q4_K = 7
+    AXO_Q4_K = 7,
+    AXO_Q6_K = 8
 };
 
 /* ------------------------------------------------------------------------- */
@@ -141,7 +145,7 @@ AXO_API float axo_f16_to_f32(uint16_t h) {
 AXO_API size_t axo_block_size(int type) {
     switch (type) {
     case AXO_Q8_0: case AXO_Q4_0: case AXO_Q4_1: case AXO_Q5_0: case AXO_Q5_1: return 32;
-    case AXO_Q4_K: return 256;
+    case AXO_Q4_K: case AXO_Q6_K: return 256;
     case AXO_F16: case AXO_F32: return 1;
     default: return 0;
     }
@@ -155,6 +159,7 @@ AXO_API size_t axo_bytes_per_block(int type) {
     case AXO_Q5_0: return 22;
     case AXO_Q5_1: return 24;
     case AXO_Q4_K: return 144;
+    case AXO_Q6_K: return 210;
     case AXO_F16: return 2;
     case AXO_F32: return 4;
     default: return 0;
@@ -355,6 +360,48 @@ static void quant_block_q4_k(const float *xin, size_t len, uint8_t *out) {
         for (int l = 0; l < 32; l++) qs[32 * p + l] = (uint8_t)(q[64 * p + l] | (q[64 * p + 32 + l] << 4));
 }
 
+/* Q6_K, GGUF layout [u8 ql[128]][u8 qh[64]][i8 scales[16]][f16 d] over 256 elements = 16 sub-blocks of 16, each
+ * with a signed 8-bit scale.  Element e = 128 n + 32 c + l (n = 0, 1; c = 0..3; l = 0..31) has the 6-bit code
+ * u = q + 32 with its low four bits in ql[64 n + 32 (c & 1) + l] (low nibble for c < 2, high for c >= 2) and its
+ * upper two bits in qh[32 n + l] at bit 2 c; its scale is scales[e / 16].  Dequant: w = (d * scale) * q.
+ *
+ * Quantiser rule (this build's; ggml's make_qx_quants search is not restated): per sub-block a_s = max |x|,
+ * scale_s = a_s / 31; max_scale = max scale_s; ls_s = round(127 / max_scale * scale_s) in 0..127 (0 if the
+ * maximum is 0); d = f16(max_scale / 127); with the f16-rounded d: sd = d * ls_s,
+ * q = clamp(round(x / sd), -32, 31)  (0 when sd == 0).  A short tail superblock is zero-padded. */
+static void quant_block_q6_k(const float *xin, size_t len, uint8_t *out) {
+    float x[256];
+    memset(x, 0, sizeof x);
+    memcpy(x, xin, len * sizeof(float));
+    float scales[16], max_scale = 0.0f;
+    for (int s = 0; s < 16; s++) {
+        float a = 0.0f;
+        for (int i = 0; i < 16; i++) a = rs_max(a, fabsf(x[16 * s + i]));
+        scales[s] = a / 31.0f;
+        max_scale = rs_max(max_scale, scales[s]);
+    }
+    float inv = max_scale > 0.0f ? 127.0f / max_scale : 0.0f;
+    uint16_t dh = axo_f32_to_f16(max_scale / 127.0f);
+    float d = axo_f16_to_f32(dh);
+    uint8_t *ql = out, *qh = out + 128;
+    int8_t *sc = (int8_t *)(out + 192);
+    memset(out, 0, 192);
+    for (int s = 0; s < 16; s++) {
+        int ls = rs_round_clamp(inv * scales[s], 0.0f, 127.0f);
+        sc[s] = (int8_t)ls;
+        float sd = d * (float)ls;
+        for (int i = 0; i < 16; i++) {
+            int e = 16 * s + i;
+            int q = sd == 0.0f ? 0 : rs_round_clamp(x[e] / sd, -32.0f, 31.0f);
+            unsigned u = (unsigned)(q + 32);
+            int n = e >> 7, c = (e >> 5) & 3, l = e & 31;
+            ql[64 * n + 32 * (c & 1) + l] |= (uint8_t)((u & 0x0F) << (4 * (c >> 1)));
+            qh[32 * n + l] |= (uint8_t)((u >> 4) << (2 * c));
+        }
+    }
+    put_u16(out + 208, dh);
+}
+
 /* quantize_tensor (quantize.rs:36-54): flat row-major f32 -> concatenated
  * `to_bytes` images in block order.  Unlike the reference, Q5_0/Q5_1 get
  * real codecs instead of aliasing Q4_0.  Returns 0, or -2 for an unknown type. */
@@ -383,6 +430,7 @@ AXO_API int axo_quantize(int type, const float *x, size_t numel, uint8_t *out) {
         case AXO_Q5_0: quant_block_q5_0(x + start, len, o); break;
         case AXO_Q5_1: quant_block_q5_1(x + start, len, o); break;
         case AXO_Q4_K: quant_block_q4_k(x + start, len, o); break;
+        case AXO_Q6_K: quant_block_q6_k(x + start, len, o); break;
         }
     }
     return 0;
@@ -468,6 +516,20 @@ static void dequant_block(int type, const uint8_t *b, float *y) {
                 float a = sd * (float)q;
                 y[32 * s + i] = a - sm;
             }
+        }
+        break;
+    }
+    case AXO_Q6_K: { /* ggml's dequantize_row_q6_K: y = d * scale * q, the product d * scale taken first */
+        const uint8_t *ql = b, *qh = b + 128;
+        const int8_t *sc = (const int8_t *)(b + 192);
+        float d = axo_f16_to_f32(get_u16(b + 208));
+        for (int e = 0; e < 256; e++) {
+            int n = e >> 7, c = (e >> 5) & 3, l = e & 31;
+            int lo = (ql[64 * n + 32 * (c & 1) + l] >> (4 * (c >> 1))) & 0x0F;
+            int hi = (qh[32 * n + l] >> (2 * c)) & 3;
+            int q = (lo | (hi << 4)) - 32;
+            float ds = d * (float)sc[e >> 4];
+            y[e] = ds * (float)q;
         }
         break;
     }

@@ -41,12 +41,13 @@ def load_oracle(c, w):
     m = o.DecodeModel(**c)
     m.set_embedding_f16(w["emb"])
     m.set_norm(-1, 0, w["final_norm"])
+    types = w.get("types", {})  # (layer, name) -> type of the linears that differ from w["qtype"]
     for l, L in enumerate(w["layers"]):
         m.set_norm(l, 0, L["norm0"])
         m.set_norm(l, 1, L["norm1"])
         for name in LIN_ID:
-            m.set_linear(l, LIN_ID[name], w["qtype"], L[name])
-    m.set_linear(-1, 0, w["qtype"], w["head"])
+            m.set_linear(l, LIN_ID[name], types.get((l, name), w["qtype"]), L[name])
+    m.set_linear(-1, 0, types.get((-1, "head"), w["qtype"]), w["head"])
     return m
 
 

@@ -79,7 +79,7 @@ def test_ggml_formula_against_numpy():
     assert np.array_equal(o.ggml_dequantize(o.Q4_1, g.reshape(-1)).reshape(40, 32), want)
 
 
-@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q5_0, o.Q5_1, o.Q4_K, o.F16, o.F32])
+@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K, o.F16, o.F32])
 def test_other_types_are_byte_identical(qtype):
     rng = np.random.default_rng(qtype)
     n = 512
@@ -158,10 +158,10 @@ def test_reader_errors(tmp_path):
         gguf.GGUFReader(_hand_made_file(tmp_path, truncate=8)[0])
     with pytest.raises(gguf.GGUFError, match="power of two"):
         gguf.GGUFReader(_hand_made_file(tmp_path, alignment=24)[0])
-    # a ggml type without a kernel here (Q6_K = 14) parses, and is refused when its data is asked for
-    with gguf.GGUFReader(_hand_made_file(tmp_path, tensor_type=14)[0]) as r:
+    # a ggml type without a kernel here (Q5_K = 13) parses, and is refused when its data is asked for
+    with gguf.GGUFReader(_hand_made_file(tmp_path, tensor_type=13)[0]) as r:
         assert r.info("blk.0.w").quant_type is None
-        with pytest.raises(gguf.GGUFError, match="Q6_K"):
+        with pytest.raises(gguf.GGUFError, match="Q5_K"):
             r.tensor_bytes("blk.0.w")
     assert issubclass(gguf.GGUFError, q.QuantError)
 
@@ -213,7 +213,7 @@ def test_write_then_read_round_trip_and_matmul_on_ggml_values(ctx, tmp_path):
     rng = np.random.default_rng(12)
     n, k = 48, 512
     tensors, packed = {}, {}
-    for qtype in (o.Q4_0, o.Q4_1, o.Q5_1, o.Q8_0, o.Q4_K):
+    for qtype in (o.Q4_0, o.Q4_1, o.Q5_1, o.Q8_0, o.Q4_K, o.Q6_K):
         packed[qtype] = o.quantize(qtype, (rng.standard_normal((n, k)) * 0.05).astype(np.float32))
         tensors[f"w.{o.TYPE_NAMES[qtype]}"] = q.QuantizedTensor([n, k], qtype, packed[qtype])
     tensors["norm"] = rng.standard_normal(k).astype(np.float32)
@@ -241,14 +241,39 @@ def test_write_then_read_round_trip_and_matmul_on_ggml_values(ctx, tmp_path):
         assert np.array_equal(gguf.load_f32(r, "w.Q4_0", ctx).reshape(-1), o.dequantize(o.Q4_0, packed[o.Q4_0], n * k))
 
 
+def _q4_k_m_like(c, w, seed):
+    """The weights of a Q4_K model with the linears llama.cpp's Q4_K_M recipe keeps at six bits requantised to Q6_K:
+    attn_v and ffn_down of every other layer, and the output matrix.  Returns name -> type for what changed."""
+    from tests.decode_common import LIN_SHAPES
+
+    rng = np.random.default_rng(seed)
+    types = {}
+    for i, L in enumerate(w["layers"]):
+        if i % 2 == 0:
+            for name in ("v", "down"):
+                n, k = LIN_SHAPES(c)[name]
+                L[name] = o.quantize(o.Q6_K, (rng.standard_normal((n, k)) * 0.06).astype(np.float32))
+                types[(i, name)] = o.Q6_K
+    w["head"] = o.quantize(o.Q6_K, (rng.standard_normal((c["vocab_size"], c["hidden_size"])) * 0.06).astype(np.float32))
+    types[(-1, "head")] = o.Q6_K
+    return types
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q6_K, "Q4_K_M"])
 def test_llama_loaded_from_gguf_decodes_like_the_oracle(ctx, tmp_path, qtype):
     from tests.decode_common import LIN_SHAPES, load_oracle, random_weights, tiny_config
     from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err
 
     c = tiny_config()
-    w = random_weights(c, 77, qtype=qtype)
+    mixed = {}
+    if qtype == "Q4_K_M":
+        qtype = o.Q4_K
+        w = random_weights(c, 77, qtype=qtype)
+        mixed = _q4_k_m_like(c, w, 78)
+    else:
+        w = random_weights(c, 77, qtype=qtype)
+    w["types"] = mixed
     cpu = load_oracle(c, w)
     # the file as llama.cpp's converter lays it out: q/k rows permuted per head, llama.* metadata, blk.N.* names
     md = {"general.architecture": "llama", "llama.block_count": c["num_layers"], "llama.embedding_length": c["hidden_size"],
@@ -270,8 +295,8 @@ def test_llama_loaded_from_gguf_decodes_like_the_oracle(ctx, tmp_path, qtype):
             data = L[name]
             if name in ("q", "k"):
                 data = converter_order(data, n, c["num_heads"] if name == "q" else c["num_kv_heads"])
-            tensors[f"blk.{i}.{stems[name]}.weight"] = q.QuantizedTensor([n, k], qtype, data)
-    tensors["output.weight"] = q.QuantizedTensor([c["vocab_size"], c["hidden_size"]], qtype, w["head"])
+            tensors[f"blk.{i}.{stems[name]}.weight"] = q.QuantizedTensor([n, k], mixed.get((i, name), qtype), data)
+    tensors["output.weight"] = q.QuantizedTensor([c["vocab_size"], c["hidden_size"]], mixed.get((-1, "head"), qtype), w["head"])
     path = str(tmp_path / "tiny-llama.gguf")
     gguf.write_gguf(path, md, tensors, ctx)
 

@@ -10,8 +10,9 @@ from tests.util import gen_weight
 
 pytestmark = pytest.mark.gpu
 
-ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.F16, o.F32]
-BLOCK = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K]
+ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K, o.F16, o.F32]
+BLOCK = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K]
+SUPER = (o.Q4_K, o.Q6_K)  # 256-element superblocks
 
 
 def _inputs(rng, n):
@@ -34,7 +35,7 @@ def test_quantize_bit_exact(ctx, qtype, n):
 
 @pytest.mark.parametrize("qtype", BLOCK)
 def test_quantize_special_blocks_bit_exact(ctx, qtype):
-    bs = 256 if qtype == o.Q4_K else 32
+    bs = 256 if qtype in SUPER else 32
     blocks = [
         np.zeros(bs), np.full(bs, 2.5), np.full(bs, -2.5), np.arange(bs) - bs / 2, np.arange(bs) / 10.0,
         np.where(np.arange(bs) % 2 == 0, 0.5, -0.5) * np.arange(bs),  # many exact half-way quotients
@@ -69,10 +70,11 @@ def test_dequantize_arbitrary_bytes_bit_exact(ctx, qtype):
     bb = o.lib().axo_bytes_per_block(qtype)
     nblk = 512
     raw = rng.integers(0, 256, size=(nblk, bb), dtype=np.uint8)
-    nscale = {o.Q8_0: 1, o.Q4_0: 1, o.Q5_0: 1, o.Q4_1: 2, o.Q5_1: 2, o.Q4_K: 2}[qtype]
+    nscale = {o.Q8_0: 1, o.Q4_0: 1, o.Q5_0: 1, o.Q4_1: 2, o.Q5_1: 2, o.Q4_K: 2, o.Q6_K: 1}[qtype]
     scales = (rng.standard_normal((nblk, nscale)) * 0.1).astype(np.float16)
-    raw[:, :2 * nscale] = scales.view(np.uint8)
-    n = nblk * (256 if qtype == o.Q4_K else 32)
+    at = 208 if qtype == o.Q6_K else 0  # Q6_K keeps its f16 d behind the codes and the int8 scales (all 256 values occur)
+    raw[:, at:at + 2 * nscale] = scales.view(np.uint8)
+    n = nblk * (256 if qtype in SUPER else 32)
     got = q.dequantize_tensor(q.QuantizedTensor([n], qtype, raw.reshape(-1)), ctx)
     want = o.dequantize(qtype, raw.reshape(-1), n)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
@@ -105,8 +107,8 @@ def test_dequantize_block_on_device(ctx):
 @pytest.mark.parametrize("shape", [(1, 256), (3, 512), (7, 2048), (5, 4096 + 256), (64, 11008)])
 def test_weight_upload_download_is_identity(ctx, qtype, shape):
     n, k = shape
-    if qtype == o.Q4_K and k % 256:
-        pytest.skip("k must be a multiple of 256 for Q4_K")
+    if qtype in SUPER and k % 256:
+        pytest.skip("k must be a multiple of 256 for the superblock types")
     w = gen_weight(np.random.default_rng(n * 1000 + k), n, k, outlier_p=0.01)
     packed = o.quantize(qtype, w)
     dw = q.DeviceWeight.upload(q.QuantizedTensor([n, k], qtype, packed), ctx)

@@ -60,7 +60,7 @@ def test_nan_keeps_being_nan():
 def test_registry_sizes():
     L = o.lib()
     expect = {o.Q8_0: (32, 34), o.Q4_0: (32, 18), o.Q4_1: (32, 20), o.Q5_0: (32, 22), o.Q5_1: (32, 24),
-              o.F16: (1, 2), o.F32: (1, 4), o.Q4_K: (256, 144)}
+              o.F16: (1, 2), o.F32: (1, 4), o.Q4_K: (256, 144), o.Q6_K: (256, 210)}
     for t, (bs, bb) in expect.items():
         assert L.axo_block_size(t) == bs and L.axo_bytes_per_block(t) == bb
     # quantize.rs:294-313: 8 elements -> 1 block, 64 -> 2 blocks
@@ -474,3 +474,154 @@ def test_empty_input():
     for t in range(8):
         assert o.quantize(t, np.zeros(0, np.float32)).size == 0
         assert o.dequantize(t, np.zeros(0, np.uint8), 0).size == 0
+
+
+# --------------------------------------------------------------------------- Q6_K (GGUF block; the reference has no such type)
+def _q6k_dequant_numpy(packed, numel):
+    """ggml's dequantize_row_q6_K, transcribed independently in numpy from its published loop: for each half n of
+    the superblock and l in 0..31, four values at 128 n + l + {0, 32, 64, 96} out of ql[64 n + l], ql[64 n + l + 32]
+    and qh[32 n + l], scales 8 n + l / 16 + {0, 2, 4, 6}."""
+    out = []
+    for b in packed.reshape(-1, 210):
+        ql, qh, sc = b[:128].astype(np.int32), b[128:192].astype(np.int32), b[192:208].view(np.int8).astype(np.float32)
+        d = b[208:210].view(np.float16).astype(np.float32)[0]
+        y = np.zeros(256, np.float32)
+        for n in range(2):
+            for l in range(32):
+                i = l // 16
+                q1 = ((ql[64 * n + l] & 0xF) | (((qh[32 * n + l] >> 0) & 3) << 4)) - 32
+                q2 = ((ql[64 * n + l + 32] & 0xF) | (((qh[32 * n + l] >> 2) & 3) << 4)) - 32
+                q3 = ((ql[64 * n + l] >> 4) | (((qh[32 * n + l] >> 4) & 3) << 4)) - 32
+                q4 = ((ql[64 * n + l + 32] >> 4) | (((qh[32 * n + l] >> 6) & 3) << 4)) - 32
+                y[128 * n + l + 0] = np.float32(d * sc[8 * n + i + 0]) * np.float32(q1)
+                y[128 * n + l + 32] = np.float32(d * sc[8 * n + i + 2]) * np.float32(q2)
+                y[128 * n + l + 64] = np.float32(d * sc[8 * n + i + 4]) * np.float32(q3)
+                y[128 * n + l + 96] = np.float32(d * sc[8 * n + i + 6]) * np.float32(q4)
+        out.append(y)
+    return np.concatenate(out)[:numel]
+
+
+def test_q6_k_zero_superblock_bytes():
+    # all codes q = 0 -> u = 32: low nibbles 0, every bit pair 0b10 -> qh bytes 0xAA; scales 0, d 0
+    p = o.quantize(o.Q6_K, np.zeros(256, np.float32))
+    assert p.tolist() == [0] * 128 + [0xAA] * 64 + [0] * 16 + [0, 0]
+    assert not o.dequantize(o.Q6_K, p, 256).any()
+
+
+def test_q6_k_layout_one_code_at_a_time():
+    """A superblock of all-zero codes (u = 32) in which one element holds another code: which byte and which bits
+    change, for elements of every (half, 32-group) and codes that exercise both the nibble and the bit pair."""
+    base = np.array([0] * 128 + [0xAA] * 64 + [1] * 16 + [0x00, 0x3C], np.uint8)  # scales 1, d = 1.0
+    assert not o.dequantize(o.Q6_K, base, 256).any()
+    for e, u in [(0, 0), (1, 63), (31, 17), (32, 5), (63, 48), (64, 0x2B), (95, 1), (96, 62), (127, 15), (128, 63), (160 + 7, 0),
+                 (192 + 16, 0x15), (224 + 31, 0x3A), (255, 0)]:
+        n, c, l = e >> 7, (e >> 5) & 3, e & 31
+        img = base.copy()
+        qi, hi = 64 * n + 32 * (c & 1) + l, 128 + 32 * n + l
+        img[qi] = (u & 15) << 4 if c >= 2 else (u & 15)
+        img[hi] = (0xAA & ~(3 << (2 * c))) | ((u >> 4) << (2 * c))
+        want = np.zeros(256, np.float32)
+        want[e] = u - 32
+        assert np.array_equal(o.dequantize(o.Q6_K, img, 256), want), (e, u)
+
+
+def test_q6_k_signed_scales_and_d():
+    # every int8 scale value, negative ones included, times d = 0.5; codes u = 33 (q = 1) everywhere
+    for first in range(-128, 128, 16):
+        sc = np.arange(first, first + 16, dtype=np.int8)
+        img = np.concatenate([np.full(128, 0x11, np.uint8), np.full(64, 0xAA, np.uint8), sc.view(np.uint8), np.array([0x00, 0x38], np.uint8)])
+        y = o.dequantize(o.Q6_K, img, 256)
+        assert np.array_equal(y, np.repeat(sc.astype(np.float32) * np.float32(0.5), 16))
+
+
+def test_q6_k_dequant_matches_ggml_loop_on_arbitrary_bytes():
+    rng = np.random.default_rng(61)
+    raw = rng.integers(0, 256, size=(64, 210), dtype=np.uint8)
+    raw[:, 208:210] = (rng.standard_normal((64, 1)) * 0.1).astype(np.float16).view(np.uint8)
+    assert np.array_equal(o.dequantize(o.Q6_K, raw.reshape(-1), 64 * 256), _q6k_dequant_numpy(raw.reshape(-1), 64 * 256))
+
+
+def test_q6_k_known_superblock_by_hand():
+    """Sub-block s holds multiples of its own step: max |x| = 31 * step_s with steps 2^-7 * ls_s for hand-picked ls
+    (the largest 127), so max_scale = 127 / 128, d = f16(2^-7) exactly, every x an exact grid point."""
+    ls = [127, 1, 2, 64, 100, 0, 33, 126, 5, 77, 127, 12, 90, 3, 50, 8]
+    q = [[((11 * i + 5 * s) % 63) - 31 for i in range(16)] for s in range(16)]  # codes -31..31
+    for s in range(16):
+        q[s][3] = 31 if s % 2 else -31  # the sub-block's maximum magnitude is code 31 exactly
+    x = np.zeros(256, np.float32)
+    for s in range(16):
+        for i in range(16):
+            x[16 * s + i] = ls[s] / 128 * q[s][i]
+    p = o.quantize(o.Q6_K, x)
+    assert p[208:210].tolist() == [0x00, 0x20]  # 2^-7
+    assert p[192:208].tolist() == ls
+    got_q = np.rint(o.dequantize(o.Q6_K, p, 256).astype(np.float64) * 128).reshape(16, 16)
+    for s in range(16):
+        if ls[s]:
+            assert (got_q[s] == np.array(q[s]) * ls[s]).all(), s
+    # codes read straight from the bytes, per the layout
+    for s in (0, 3, 9, 15):
+        for i in (0, 3, 15):
+            e = 16 * s + i
+            n, c, l = e >> 7, (e >> 5) & 3, e & 31
+            u = ((int(p[64 * n + 32 * (c & 1) + l]) >> (4 * (c >> 1))) & 15) | (((int(p[128 + 32 * n + l]) >> (2 * c)) & 3) << 4)
+            assert u - 32 == q[s][i], (s, i)
+    assert np.array_equal(o.dequantize(o.Q6_K, p, 256), x)
+
+
+def test_q6_k_half_way_values_round_away_and_clamp():
+    # sub-block 0: max |x| = 31 -> scale 1 = max_scale, d = f16(1 / 127), ls = 127, sd = d * 127 (in f32);
+    # x = (k + 0.5) sd -> k + 1, -(k + 0.5) sd -> -(k + 1): half-way quotients round away from zero
+    x = np.zeros(256, np.float32)
+    x[0] = 31.0
+    d = np.float32(np.float16(np.float32(1.0) / np.float32(127.0)))
+    sd = np.float32(d * np.float32(127.0))
+    vals = [0.5, 1.5, 2.5, -0.5, -1.5, 30.49, 7.0]
+    for i, v in enumerate(vals):
+        x[1 + i] = np.float32(v) * sd
+    # sub-block 1: scale 1.4 / 127 of the maximum -> ls = round(1.4) = 1, sd = d: its extremes lie 43 steps out and clamp
+    # to the ends of the code range, -32 and 31
+    x[16], x[17] = -31 * 1.4 / 127, 31 * 1.4 / 127
+    p = o.quantize(o.Q6_K, x)
+    assert p[208:210].view(np.float16)[0] == d
+    y = o.dequantize(o.Q6_K, p, 256)
+    got = np.rint(y[1:1 + len(vals)] / sd).astype(int).tolist()
+    assert got == [1, 2, 3, -1, -2, 30, 7]
+    assert p[192] == 127 and p[193] == 1 and not p[194:208].any()
+    code = lambda l: (int(p[l]) & 15) | ((int(p[128 + l]) & 3) << 4)  # elements 0..31: low nibble of ql[l], bits 0-1 of qh[l]
+    assert code(16) == 0 and code(17) == 63 and code(18) == 32
+    assert y[16] == -32 * d and y[17] == 31 * d
+
+
+def test_q6_k_roundtrip_error_is_what_the_rule_implies():
+    rng = np.random.default_rng(62)
+    n = 256 * 64
+    x = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    x[rng.random(n) < 0.01] = 0.5
+    packed = o.quantize(o.Q6_K, x)
+    y = o.dequantize(o.Q6_K, packed, n)
+    assert np.array_equal(y, _q6k_dequant_numpy(packed, n))
+    for b, p in enumerate(packed.reshape(-1, 210)):
+        d = float(p[208:210].view(np.float16)[0])
+        ls = p[192:208].view(np.int8).astype(np.float64)
+        xs = x[256 * b:256 * b + 256].astype(np.float64).reshape(16, 16)
+        ys = y[256 * b:256 * b + 256].astype(np.float64).reshape(16, 16)
+        scales = np.abs(xs).max(1) / 31
+        # f16 rounding of d; for weights of this size d is a subnormal f16 (spacing 2^-24), as it is in ggml's files
+        d_err = max(scales.max() / 127 * 2 ** -11, 2.0 ** -25)
+        assert abs(d - scales.max() / 127) <= d_err
+        assert ls.max() == 127 and ls.min() >= 0
+        for s in range(16):
+            sd = d * ls[s]
+            assert abs(sd - scales[s]) <= d * 0.5 + ls[s] * d_err + scales[s] * 2 ** -20, (b, s)
+            above = max(0.0, np.abs(xs[s]).max() - 31 * sd)  # how far the 7-bit rounding of the scale pushed the maximum out
+            assert np.abs(xs[s] - ys[s]).max() <= max(sd * 0.5, above) + 1e-6 * np.abs(xs[s]).max(), (b, s)
+
+
+def test_q6_k_tail_superblock_is_zero_padded():
+    x = (np.arange(300, dtype=np.float32) - 150) / 64
+    p = o.quantize(o.Q6_K, x)
+    assert p.size == 2 * 210
+    full = o.quantize(o.Q6_K, np.concatenate([x, np.zeros(212, np.float32)]))
+    assert np.array_equal(p, full)
+    assert o.dequantize(o.Q6_K, p, 300).shape == (300,)
