@@ -128,7 +128,7 @@ __global__ void __launch_bounds__(TPB) axq_read_kernel(const axq_u32x4 *__restri
 // The same bytes in the order the one-vector GEMV asks for them: a workgroup of eight waves owns `rows` consecutive rows of
 // the code plane (pitch bytes each, 2048 of them used), wave (g, s) walks the 4-row steps of half g and reads, per step,
 // two pieces of 256 bytes of each of the step's four rows (lane = (16-byte chunk, row)), NB steps in flight.
-template <int NB>
+template <int NB, int LIN = 0>
 __global__ void __launch_bounds__(512) axq_read_rows_kernel(const uint8_t *__restrict__ codes, size_t pitch, int n_rows, int rows_per_wg, uint32_t *sink) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = wave >> 2, s = wave & 3;
     const int blk = lane >> 2, j = lane & 3;
@@ -139,11 +139,24 @@ __global__ void __launch_bounds__(512) axq_read_rows_kernel(const uint8_t *__res
         axq_u32x4 v[NB][2];
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            int row = row0 + 4 * (st + b < steps ? st + b : 0);
+            const int sb = st + b < steps ? st + b : 0;
+            int row = row0 + 4 * sb;
             row = row < n_rows ? row : n_rows - 1;
             const uint8_t *p = codes + (size_t)row * pitch + s * 256 + blk * 16;
+            size_t second = 1024;
+            if (LIN == 1) { // the same bytes per wave and step (2 KB), each wave walking a contiguous run of its own
+                size_t off = (((size_t)blockIdx.x * 8 + wave) * steps + sb) * 2048;
+                const size_t total = (size_t)n_rows * pitch;
+                off = off + 2048 <= total ? off : 0;
+                p = codes + off + lane * 16;
+            } else if (LIN == 2) { // ... the workgroup's eight waves side by side, the workgroup walking one contiguous run
+                size_t off = (((size_t)blockIdx.x * steps + sb) * 8 + wave) * 2048;
+                const size_t total = (size_t)n_rows * pitch;
+                off = off + 2048 <= total ? off : 0;
+                p = codes + off + lane * 16;
+            }
             v[b][0] = __builtin_nontemporal_load(reinterpret_cast<const axq_u32x4 *>(p));
-            v[b][1] = __builtin_nontemporal_load(reinterpret_cast<const axq_u32x4 *>(p + 1024));
+            v[b][1] = __builtin_nontemporal_load(reinterpret_cast<const axq_u32x4 *>(p + second));
         }
 #pragma unroll
         for (int b = 0; b < NB; b++) acc ^= v[b][0].x ^ v[b][0].w ^ v[b][1].y ^ v[b][1].z;
@@ -517,7 +530,7 @@ int axq_bench_read_ring_ex(axq_ctx *ctx, const axq_weight *const *weights, int n
     if (!weights || n_weights <= 0 || first < 0 || !sink_dev)
         return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring: bad argument");
     if (wgs_per_cu < 1 || wgs_per_cu > 8 || (threads != 256 && threads != 512 && threads != 1024) || in_flight < 1 || in_flight > 32 ||
-        streams < 1 || streams > AXQ_AUX_STREAMS || pattern < 0 || pattern > 1)
+        streams < 1 || streams > AXQ_AUX_STREAMS || pattern < 0 || pattern > 3)
         return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring_ex: 1..8 workgroups per compute unit, 256/512/1024 threads, 1..32 "
                                                        "loads in flight, 1..%d streams, pattern 0 or 1", AXQ_AUX_STREAMS);
     AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
@@ -531,16 +544,19 @@ int axq_bench_read_ring_ex(axq_ctx *ctx, const axq_weight *const *weights, int n
         const axq_weight *w = weights[(first + i) % n_weights];
         if (!w) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring: NULL weight");
         hipStream_t st = streams > 1 ? ctx->aux_stream[i % streams] : ctx->stream;
-        if (pattern == 1) {
+        if (pattern >= 1) {
             // the code plane of a Q4_K weight with k = 4096, rows in the one-vector GEMV's order
             if (w->type != AXQ_Q4_K || w->k != 4096)
                 return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring_ex: the row pattern reads Q4_K weights with k = 4096");
             int rows_per_wg = (int)((w->n_rows + grid - 1) / grid);
             rows_per_wg = (rows_per_wg + 7) / 8 * 8;
             const unsigned g2 = (unsigned)((w->n_rows + rows_per_wg - 1) / rows_per_wg);
-            if (in_flight <= 4) axq_read_rows_kernel<2><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev);
-            else if (in_flight <= 8) axq_read_rows_kernel<4><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev);
-            else axq_read_rows_kernel<7><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev);
+#define AXQ_ROWS(L) \
+            if (in_flight <= 4) axq_read_rows_kernel<2, L><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev); \
+            else if (in_flight <= 8) axq_read_rows_kernel<4, L><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev); \
+            else axq_read_rows_kernel<7, L><<<g2, 512, 0, st>>>(w->codes, w->codes_pitch, (int)w->n_rows, rows_per_wg, sink_dev);
+            if (pattern == 1) { AXQ_ROWS(0) } else if (pattern == 2) { AXQ_ROWS(1) } else { AXQ_ROWS(2) }
+#undef AXQ_ROWS
         } else {
             const size_t n16 = w->alloc_bytes / 16;
             if (n16 == 0) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_read_ring: empty weight");

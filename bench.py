@@ -325,6 +325,65 @@ def codec_rates(ctx, n=N_HEAD, k=K_HEAD, iters=20):
     return out
 
 
+def read_sweep(ctx, steps, warmup):
+    """Prints a table: a kernel that only READS a ring copy of the headline weight (no arithmetic, one sink store per
+    workgroup), over workgroups per CU x threads x 16-byte loads in flight per thread x temporal / non-temporal loads,
+    launches following one another on one stream; the same kernel over several streams; a row-walking pattern; and the
+    GEMV itself on one and on several streams.  The best one-stream line is the ceiling the GEMV is held against."""
+    from axonml_amd import quant as q
+
+    lib, T = ctx.lib, q.QuantType
+    wbytes = lib.axq_packed_bytes(int(T.Q4_K), N_HEAD * K_HEAD)
+    ws = make_ring(ctx, T.Q4_K, N_HEAD, K_HEAD, int(RING_BYTES // wbytes) + 1, 0.01)
+    arr = (C.c_void_p * len(ws))(*[w.value for w in ws])
+    sink = ctx.malloc(256)
+    x_dev = ctx.to_device(np.random.default_rng(0).standard_normal((1, K_HEAD)).astype(np.float32))
+    y_dev = ctx.malloc(N_HEAD * 4)
+
+    def t_read(wg, th, u, nt, pattern, streams):
+        ms, _, _, _ = time_ring(ctx, lambda first, n: ctx.check(lib.axq_bench_read_ring_ex(ctx.handle, arr, len(ws), first, sink, n, wg, th, u,
+                                                                                              nt, pattern, streams)), len(ws), steps, warmup)
+        return ms * 1e3
+
+    def line(what, us, nbytes=wbytes):
+        print(f"{what:<72s} {us:7.2f} us  {nbytes / us / 1e3:7.1f} GB/s  {nbytes / us / 1e3 / HBM_PEAK_GBPS:5.3f} of peak", flush=True)
+
+    print(f"# Q4_K {N_HEAD} x {K_HEAD}: {wbytes} bytes per launch, ring of {len(ws)} copies, {steps} launches per figure (median of {REPEATS})")
+    line("GEMV, one stream", time_gemv(ctx, ws, x_dev, y_dev, 1, steps, warmup)[0] * 1e3)
+    for st in (2, 3, 4):
+        ms, _, _, _ = time_ring(ctx, lambda first, n: ctx.check(lib.axq_bench_gemv_ring_streams(ctx.handle, arr, len(ws), first, x_dev, 1, y_dev,
+                                                                                                 n, st)), len(ws), steps, warmup)
+        line(f"GEMV, launches dealt over {st} streams", ms * 1e3)
+    best = None
+    for wg in (1, 2, 4):
+        for th in (256, 512, 1024):
+            for u in (4, 8, 16, 32):
+                if th == 1024 and u == 32:
+                    continue
+                for nt in (1, 0):
+                    us = t_read(wg, th, u, nt, 0, 1)
+                    line(f"read: {wg} wg/CU x {th:4d} threads x {u:2d} loads in flight, {'non-temporal' if nt else 'temporal'}", us)
+                    if best is None or us < best[0]:
+                        best = (us, wg, th, u, nt)
+    # the code plane only (k / 2 bytes per row): in the order the one-vector GEMV asks for it (a wave's load takes 256 bytes
+    # of each of four rows), and the same count of bytes per wave and step from one contiguous run (what a tiled layout
+    # of the plane would give the GEMV), per wave or per workgroup
+    for pattern, what in ((1, "the GEMV's row order"), (2, "contiguous per wave"), (3, "contiguous per workgroup")):
+        for u in (4, 8, 14):
+            line(f"read, code plane, {what}, {u:2d} loads in flight per lane", t_read(1, 512, u, 1, pattern, 1), N_HEAD * K_HEAD // 2)
+    for st in (2, 4):
+        line(f"read: 1 wg/CU x  512 threads x 16 loads, launches dealt over {st} streams", t_read(1, 512, 16, 1, 0, st))
+        line(f"read: 2 wg/CU x  256 threads x 16 loads, launches dealt over {st} streams", t_read(2, 256, 16, 1, 0, st))
+    line("GEMV, one stream (again)", time_gemv(ctx, ws, x_dev, y_dev, 1, steps, warmup)[0] * 1e3)
+    print(f"# best read-only kernel on one stream: {best[1]} wg/CU x {best[2]} threads x {best[3]} loads in flight, "
+          f"{'non-temporal' if best[4] else 'temporal'}: {best[0]:.2f} us = {wbytes / best[0] / 1e3 / HBM_PEAK_GBPS:.3f} of peak")
+    for w in ws:
+        lib.axq_weight_free(ctx.handle, w)
+    ctx.free(sink)
+    ctx.free(x_dev)
+    ctx.free(y_dev)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -339,6 +398,9 @@ def main():
     ap.add_argument("--counter-probe", action="store_true",
                     help="for profiler counter runs: a few launches of a 256 MiB plain copy kernel, then the "
                          "headline GEMV ring; no oracle, no CPU leg, no JSON line")
+    ap.add_argument("--read-sweep", action="store_true",
+                    help="instead of the benchmark: time a read-only kernel over the headline weight in every launch shape, "
+                         "and print the table")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path is built or measured)")
@@ -353,6 +415,9 @@ def main():
 
     if args.counter_probe:
         counter_probe(ctx, args.steps)
+        return
+    if args.read_sweep:
+        read_sweep(ctx, args.steps, args.warmup)
         return
 
     # ---- headline: Q4_K GEMV 14336 x 4096, batch 1

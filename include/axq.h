@@ -319,7 +319,8 @@ AXQ_API int axq_bench_read_ring(axq_ctx *ctx, const axq_weight *const *weights, 
  * wgs_per_cu workgroups per compute unit (1..8) of `threads` (256, 512, 1024), each lane keeping `in_flight` 16-byte loads
  * in flight (4, 8, 16, 32; 16 at most with 1024 threads), non-temporal or plain loads; pattern 0 reads each weight's
  * device image as contiguous shares, pattern 1 reads the code plane of a Q4_K weight with k = 4096 row step by row step,
- * as the one-vector GEMV does (in_flight = 4, 8 or 14: two loads per step); streams > 1 spreads the launches over that
+ * as the one-vector GEMV does (in_flight = 4, 8 or 14: two loads per step), patterns 2 and 3 read as many bytes of that
+ * plane per wave and step from one contiguous run per wave / per workgroup; streams > 1 spreads the launches over that
  * many streams so that consecutive launches may overlap (the context's stream waits for all of them at the end).
  * axq_bench_read_ring is (1, 512, 16, 1, 0, 1). */
 AXQ_API int axq_bench_read_ring_ex(axq_ctx *ctx, const axq_weight *const *weights, int n_weights, int first,
