@@ -34,6 +34,9 @@ struct axq_model {
     float *norm_attn, *norm_ffn;    // [layers, hidden]
     float *norm_final;              // [hidden]
     std::vector<axq_weight *> w_qkv, w_o, w_gu, w_down;
+    // q, k or v of a layer whose block type differs from the fused weight's (GGUF files that keep attn_v at six bits
+    // beside four-bit attn_q and attn_k): a weight of its own, multiplied after the fused one into its rows of qkv
+    std::vector<axq_weight *> w_sep[3];
     axq_weight *w_head;
     std::vector<uint32_t> set_mask; // per layer: bit per axq_linear_id that has been set
     bool head_set;
@@ -796,6 +799,9 @@ void launch_attn_split(axq_model *m, int l, const float *qkv, int nseq, float *a
 // weight, silu(gate) * up over its row pairs (y then has half as many entries as W has rows).  The matrix-pipe
 // GEMV applies f while it stages x and g while it writes y; for a linear it does not cover (other weight types,
 // K not a multiple of 64 or beyond 16384) f and g run as kernels of their own around the f32 GEMV, through `tmp`.
+// First row of q (0), k (1) or v (2) in a row of qkv.
+inline int64_t qkv_part_offset(const axq_model *m, int part) { return part == 0 ? 0 : (part == 1 ? m->q_dim : m->q_dim + m->kv_dim); }
+
 int linear(axq_model *m, const axq_weight *w, const float *x, int xmode, const float *aux, int ymode, float *tmp,
            const float *bias, float *y) {
     axq_ctx *ctx = m->ctx;
@@ -835,6 +841,11 @@ int enqueue_step(axq_model *m, bool short_ctx) {
     for (int l = 0; l < c.num_hidden_layers; l++) {
         if ((rc = linear(m, m->w_qkv[l], m->h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, AXQ_Y_PLAIN, m->xn, nullptr, m->qkv)))
             return rc;
+        for (int part = 0; part < 3; part++)
+            if (const axq_weight *w = m->w_sep[part][l])
+                if ((rc = linear(m, w, m->h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, AXQ_Y_PLAIN, m->xn, nullptr,
+                                 m->qkv + qkv_part_offset(m, part))))
+                    return rc;
         if (short_ctx) {
             launch_attn_rows(m, l, m->qkv, 1, 0, m->pos, 0, prompt_attn_lds(m, m->fused_max), m->att, st);
         } else {
@@ -913,6 +924,12 @@ size_t prompt_attn_lds(const axq_model *m, int last) {
     return (size_t)((span + 255) / 256 * 256) * sizeof(float);
 }
 
+// dst[b, 0 .. n) = src[b, 0 .. n) for rows of different lengths (n a multiple of 4; both sides 16-byte aligned).
+__global__ void place_columns_kernel(const float *__restrict__ src, int n, float *__restrict__ dst, int dst_row) {
+    const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 4, b = blockIdx.y;
+    if (i < n) *reinterpret_cast<float4 *>(dst + (size_t)b * dst_row + i) = *reinterpret_cast<const float4 *>(src + (size_t)b * n + i);
+}
+
 enum RowsMode { ROWS_NONE = 0, ROWS_GEMV = 1, ROWS_GEMM = 2 };
 
 // Whether `nb` rows ending before position `last` can go through the layers together in that mode: the scores of the
@@ -922,16 +939,16 @@ bool rows_mode_covers(const axq_model *m, int mode, int last, int nb) {
     if (nb < 1 || prompt_attn_lds(m, last) > 128 * 1024) return false;
     if (mode == ROWS_GEMV) return nb <= PROMPT_BATCH;
     for (int l = 0; l < m->cfg.num_hidden_layers; l++)
-        for (const axq_weight *w : {m->w_qkv[l], m->w_o[l], m->w_gu[l], m->w_down[l]})
-            if (!axq_dev_gemm_f32_covers(w, nb)) return false;
+        for (const axq_weight *w : {m->w_qkv[l], m->w_o[l], m->w_gu[l], m->w_down[l], m->w_sep[0][l], m->w_sep[1][l], m->w_sep[2][l]})
+            if (w && !axq_dev_gemm_f32_covers(w, nb)) return false;
     return true;
 }
 
 bool all_layers_in_small_batch_reach(const axq_model *m, int nb) {
     if (nb < 2) return false;
     for (int l = 0; l < m->cfg.num_hidden_layers; l++)
-        for (const axq_weight *w : {m->w_qkv[l], m->w_o[l], m->w_gu[l], m->w_down[l]})
-            if (!axq_dev_gemv_batch_covers(w, nb < PROMPT_BATCH ? nb : PROMPT_BATCH)) return false;
+        for (const axq_weight *w : {m->w_qkv[l], m->w_o[l], m->w_gu[l], m->w_down[l], m->w_sep[0][l], m->w_sep[1][l], m->w_sep[2][l]})
+            if (w && !axq_dev_gemv_batch_covers(w, nb < PROMPT_BATCH ? nb : PROMPT_BATCH)) return false;
     return true;
 }
 
@@ -1060,6 +1077,13 @@ int enqueue_rows(axq_model *m, const Rows &r) {
     for (int l = 0; l < c.num_hidden_layers; l++) {
         const size_t off = (size_t)l * c.num_key_value_heads * c.max_position_embeddings * d + seq_off;
         if ((rc = lin(m->w_qkv[l], m->pb_h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, nullptr, m->pb_qkv, nullptr, nullptr))) return rc;
+        for (int part = 0; part < 3; part++)
+            if (const axq_weight *w = m->w_sep[part][l]) { // through the gate/up rows (free until the feed-forward) into its columns of qkv
+                if ((rc = lin(w, m->pb_h, AXQ_X_RMSNORM, m->norm_attn + (size_t)l * H, nullptr, m->pb_gu, nullptr, nullptr))) return rc;
+                const int rows = (int)w->n_rows;
+                place_columns_kernel<<<dim3((rows / 4 + 255) / 256, nb), 256, 0, st>>>(m->pb_gu, rows, m->pb_qkv + qkv_part_offset(m, part),
+                                                                                       m->qkv_rows);
+            }
         if (!r.per_seq)
             rope_append_kernel<<<dim3(c.num_key_value_heads, nb), d / 2, 0, st>>>(
                 m->pb_qkv, m->qkv_rows, m->q_dim, m->kv_dim, m->rope_cos, m->rope_sin, m->kcache + off, m->vcache + off, r.pos0, nullptr,
@@ -1262,6 +1286,7 @@ int axq_model_create(axq_ctx *ctx, const axq_model_config *cfg, axq_model **out)
     m->seq_pos.assign(1, 0);
     const int L = c.num_hidden_layers, H = c.hidden_size, I = c.intermediate_size;
     m->w_qkv.assign(L, nullptr); m->w_o.assign(L, nullptr); m->w_gu.assign(L, nullptr); m->w_down.assign(L, nullptr);
+    for (auto &v : m->w_sep) v.assign(L, nullptr);
     m->set_mask.assign(L, 0);
     m->prompt_cap = c.max_position_embeddings;
     m->out_cap = c.max_position_embeddings;
@@ -1342,6 +1367,8 @@ void axq_model_free(axq_model *m) {
     for (void *p : {(void *)m->bprompt, (void *)m->boffsets, (void *)m->bout})
         if (p) (void)hipFree(p);
     for (auto *w : m->w_qkv) axq_weight_free(ctx, w);
+    for (auto &v : m->w_sep)
+        for (auto *w : v) axq_weight_free(ctx, w);
     for (auto *w : m->w_o) axq_weight_free(ctx, w);
     for (auto *w : m->w_gu) axq_weight_free(ctx, w);
     for (auto *w : m->w_down) axq_weight_free(ctx, w);
@@ -1424,6 +1451,27 @@ int axq_model_set_linear(axq_model *m, int layer, int which, const axq_weight *w
     }
     int rc;
     if (!*slot && (rc = axq_weight_alloc(ctx, w->type, slot_rows, k, slot))) return rc;
+    const bool qkv_part = layer >= 0 && which <= AXQ_LIN_V;
+    if (qkv_part && (m->w_sep[which][layer] || (*slot)->type != w->type)) {
+        // the part's place in the fused weight is given up (a part of the fused weight's own type goes back into it)
+        AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+        axq_weight_free(ctx, m->w_sep[which][layer]);
+        m->w_sep[which][layer] = nullptr;
+        invalidate_graphs(m);
+    }
+    if (qkv_part && (*slot)->type != w->type) {
+        // q, k or v of another block type than the fused weight: kept apart (the fused weight's rows for it stay as they
+        // are and are multiplied for nothing; whoever sets q first gives the fused weight q's type)
+        if (rows % 4 != 0 || m->qkv_rows % 4 != 0)
+            return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: q, k and v of different block types need row counts that are multiples of 4");
+        axq_weight *sep = nullptr;
+        if ((rc = axq_weight_alloc(ctx, w->type, rows, k, &sep))) return rc;
+        if ((rc = copy_rows(ctx, sep, w, 0))) { axq_weight_free(ctx, sep); return rc; }
+        AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+        m->w_sep[which][layer] = sep;
+        m->set_mask[layer] |= 1u << which;
+        return AXQ_OK;
+    }
     if ((*slot)->type != w->type)
         return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: fused weight holds %s, got %s",
                         axq_type_name((*slot)->type), axq_type_name(w->type));

@@ -350,9 +350,10 @@ def load_llama(path, ctx=None, max_position_embeddings=None, permuted_qk=True):
         set_embedding(model, emb)
 
         def fused_as_f32(layer, group):
-            # q/k/v share one device weight and so do gate/up: one GEMV reads them all.  A file that mixes block
-            # types inside such a group (llama.cpp's Q4_K_M keeps some attn_v in Q6_K beside Q4_K q and k) has the
-            # group carried as f32 rows dequantised on the device: exact, at the price of the larger read.
+            # gate and up share one device weight, rows interleaved, so that one GEMV applies SwiGLU on the way out.
+            # A file that mixes block types inside that pair has it carried as f32 rows dequantised on the device:
+            # exact, at the price of the larger read.  (q, k and v may differ: the model keeps the odd one apart;
+            # llama.cpp's Q4_K_M has some attn_v in Q6_K beside Q4_K attn_q and attn_k.)
             names = [f"blk.{layer}.{_LINEAR_NAMES[w]}.weight" for w in group]
             return len({r.info(n).ggml_type for n in names}) > 1
 
@@ -371,7 +372,7 @@ def load_llama(path, ctx=None, max_position_embeddings=None, permuted_qk=True):
         for layer in range(cfg["num_hidden_layers"]):
             model.set_norm(layer, 0, load_f32(r, f"blk.{layer}.attn_norm.weight", ctx))
             model.set_norm(layer, 1, load_f32(r, f"blk.{layer}.ffn_norm.weight", ctx))
-            mixed = {w: fused_as_f32(layer, g) for g in (("q", "k", "v"), ("gate", "up")) for w in g}
+            mixed = {w: fused_as_f32(layer, g) for g in (("gate", "up"),) for w in g}
             for which, stem in _LINEAR_NAMES.items():
                 heads = {"q": cfg["num_attention_heads"], "k": cfg["num_key_value_heads"]}.get(which)
                 linear(layer, which, f"blk.{layer}.{stem}.weight", heads, mixed.get(which, False))

@@ -209,7 +209,9 @@ AXQ_API int axq_model_set_embedding_f16(axq_model *m, const uint16_t *table, int
 AXQ_API int axq_model_set_embedding_f32(axq_model *m, const float *table, int mem);
 /* layer -1 = final norm; which 0 = attention norm, 1 = ffn norm.  f32[hidden]. */
 AXQ_API int axq_model_set_norm(axq_model *m, int layer, int which, const float *w, int mem);
-/* layer -1 = lm_head.  The model copies the weight's blocks; the caller may free `w`. */
+/* layer -1 = lm_head.  The model copies the weight's blocks; the caller may free `w`.  q, k and v of a layer share one
+ * fused weight of the block type of whichever is set first; a q, k or v of another type is kept as a weight of its own
+ * (row counts must be multiples of 4 then).  gate and up share one weight and one type (AXQ_ERR_INVALID_QUANT_TYPE). */
 AXQ_API int axq_model_set_linear(axq_model *m, int layer, int which, const axq_weight *w);
 /* Fill every linear (Q4_K by default), the embedding and unit norms from a
  * seeded device generator: N(0, std) weights.  For benchmarks of random-init

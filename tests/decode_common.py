@@ -63,13 +63,30 @@ def load_gpu(ctx, c, w):
     m.set_embedding_f16(w["emb"])
     m.set_norm(-1, 0, w["final_norm"])
     shapes = LIN_SHAPES(c)
+    types = w.get("types", {})
     for l, L in enumerate(w["layers"]):
         m.set_norm(l, 0, L["norm0"])
         m.set_norm(l, 1, L["norm1"])
         for name, (n, k) in shapes.items():
-            m.set_linear(l, name, q.QuantizedTensor([n, k], w["qtype"], L[name]))
-    m.set_linear(-1, "q", q.QuantizedTensor([c["vocab_size"], c["hidden_size"]], w["qtype"], w["head"]))
+            m.set_linear(l, name, q.QuantizedTensor([n, k], types.get((l, name), w["qtype"]), L[name]))
+    m.set_linear(-1, "q", q.QuantizedTensor([c["vocab_size"], c["hidden_size"]], types.get((-1, "head"), w["qtype"]), w["head"]))
     return m
+
+
+def requantize(c, w, changes, seed):
+    """Replaces the linears named in `changes` ({(layer, name): type}; (-1, "head") is the lm_head) by fresh random
+    weights of that block type and records the types in w["types"] for the loaders above."""
+    rng = np.random.default_rng(seed)
+    shapes = dict(LIN_SHAPES(c), head=(c["vocab_size"], c["hidden_size"]))
+    for (l, name), t in changes.items():
+        n, k = shapes[name]
+        packed = o.quantize(t, (rng.standard_normal((n, k)) * 0.06).astype(np.float32))
+        if l < 0:
+            w["head"] = packed
+        else:
+            w["layers"][l][name] = packed
+    w.setdefault("types", {}).update(changes)
+    return w
 
 
 class NumpyDecoder:

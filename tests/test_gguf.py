@@ -241,16 +241,17 @@ def test_write_then_read_round_trip_and_matmul_on_ggml_values(ctx, tmp_path):
         assert np.array_equal(gguf.load_f32(r, "w.Q4_0", ctx).reshape(-1), o.dequantize(o.Q4_0, packed[o.Q4_0], n * k))
 
 
-def _q4_k_m_like(c, w, seed):
+def _q4_k_m_like(c, w, seed, ffn_too=False):
     """The weights of a Q4_K model with the linears llama.cpp's Q4_K_M recipe keeps at six bits requantised to Q6_K:
-    attn_v and ffn_down of every other layer, and the output matrix.  Returns name -> type for what changed."""
+    attn_v and ffn_down of every other layer, and the output matrix (ffn_too: ffn_up of those layers as well, which
+    no stock recipe does: a gate/up pair of two types).  Returns name -> type for what changed."""
     from tests.decode_common import LIN_SHAPES
 
     rng = np.random.default_rng(seed)
     types = {}
     for i, L in enumerate(w["layers"]):
         if i % 2 == 0:
-            for name in ("v", "down"):
+            for name in ("v", "down", "up") if ffn_too else ("v", "down"):
                 n, k = LIN_SHAPES(c)[name]
                 L[name] = o.quantize(o.Q6_K, (rng.standard_normal((n, k)) * 0.06).astype(np.float32))
                 types[(i, name)] = o.Q6_K
@@ -260,17 +261,18 @@ def _q4_k_m_like(c, w, seed):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q6_K, "Q4_K_M"])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q6_K, "Q4_K_M", "Q4_K_M+up"])
 def test_llama_loaded_from_gguf_decodes_like_the_oracle(ctx, tmp_path, qtype):
     from tests.decode_common import LIN_SHAPES, load_oracle, random_weights, tiny_config
     from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err
 
     c = tiny_config()
     mixed = {}
-    if qtype == "Q4_K_M":
+    if qtype in ("Q4_K_M", "Q4_K_M+up"):
+        ffn_too = qtype.endswith("+up")
         qtype = o.Q4_K
         w = random_weights(c, 77, qtype=qtype)
-        mixed = _q4_k_m_like(c, w, 78)
+        mixed = _q4_k_m_like(c, w, 78, ffn_too)
     else:
         w = random_weights(c, 77, qtype=qtype)
     w["types"] = mixed

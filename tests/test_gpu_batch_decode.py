@@ -58,6 +58,27 @@ def test_generate_batch_matches_the_oracle_sequence_by_sequence(ctx, n_seq, qtyp
     cpu.close()
 
 
+@pytest.mark.parametrize("n_seq", [3, 8, 12])
+def test_generate_batch_with_q_k_v_of_different_block_types(ctx, n_seq):
+    """A value projection at six bits and a key projection at eight beside four-bit queries (the mix of GGUF files):
+    the odd parts are multiplied apart in the batched step too (small-batch GEMV where it covers the type, row by row
+    where it does not, GEMM rows beyond eight sequences)."""
+    from tests.decode_common import requantize
+
+    c = tiny_config(max_seq_len=96)
+    w = requantize(c, random_weights(c, 260 + n_seq), {(0, "v"): o.Q6_K, (1, "k"): o.Q8_0, (1, "v"): o.Q6_K}, 261)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    gpu.set_batch(n_seq)
+    rng = np.random.default_rng(n_seq)
+    prompts = [rng.integers(0, c["vocab_size"], size=[1, 5, 40, 12][i % 4] + i) for i in range(n_seq)]
+    got, _, _ = gpu.generate_batch(prompts, 10)
+    for s, p in enumerate(prompts):
+        want, _ = _oracle_walk(cpu, p, 10)
+        assert got[s].tolist() == want, s
+    gpu.close()
+    cpu.close()
+
+
 def test_forward_batch_logits_at_different_positions(ctx):
     c = tiny_config(max_seq_len=64)
     w = random_weights(c, 300)

@@ -7,7 +7,7 @@ import pytest
 
 import oracle as o
 from axonml_amd import quant as q
-from tests.decode_common import load_gpu, load_oracle, random_weights, tiny_config
+from tests.decode_common import LIN_SHAPES, load_gpu, load_oracle, random_weights, requantize, tiny_config
 from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err
 
 pytestmark = pytest.mark.gpu
@@ -285,8 +285,8 @@ def test_error_paths(ctx):
     m = load_gpu(ctx, c, random_weights(c, 40))
     with pytest.raises(q.ShapeMismatch):  # wrong linear shape
         m.set_linear(0, "q", q.quantize_tensor(np.zeros((64, 256), np.float32), q.QuantType.Q4_K, ctx))
-    with pytest.raises(q.InvalidQuantType):  # fused q,k,v must share a type
-        m.set_linear(0, "k", q.quantize_tensor(np.zeros((128, 256), np.float32), q.QuantType.Q8_0, ctx))
+    with pytest.raises(q.InvalidQuantType):  # the fused gate/up weight holds one type (q, k, v may differ: kept apart)
+        m.set_linear(0, "gate", q.quantize_tensor(np.zeros((512, 256), np.float32), q.QuantType.Q8_0, ctx))
     with pytest.raises(q.QuantError):
         m.forward(10 ** 6)
     fresh = QuantizedLlama(ctx, vocab_size=64, hidden_size=256, intermediate_size=512, num_hidden_layers=1,
@@ -331,3 +331,51 @@ def test_the_two_prompt_attention_kernels_agree(ctx, monkeypatch, over, n_first,
     for a, b in zip(kv1, kv0):
         af, bf = a.view(np.float16).astype(np.float64), b.view(np.float16).astype(np.float64)
         assert np.abs(af - bf).max() <= 2.0 ** -9 * np.abs(af).max()  # isolated one-ulp f16 roundings at most
+
+
+@pytest.mark.parametrize("changes", [{(0, "v"): o.Q6_K}, {(0, "k"): o.Q8_0, (0, "v"): o.Q6_K, (1, "v"): o.Q5_1},
+                                     {(1, "q"): o.Q6_K, (0, "down"): o.Q6_K, (1, "o"): o.Q8_0, (-1, "head"): o.Q6_K}])
+def test_q_k_v_of_different_block_types(ctx, changes):
+    """GGUF files mix types inside a layer (llama.cpp's Q4_K_M keeps some attn_v at six bits): q, k or v of another type
+    than the fused weight is multiplied apart, into its rows of qkv.  One-token steps, the prompt path through the GEMM
+    and through the small-batch GEMV, and batched steps, all against the oracle with the same weights."""
+    c = tiny_config(max_seq_len=96)
+    w = requantize(c, random_weights(c, 70), changes, 71)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    prompt = np.random.default_rng(72).integers(0, c["vocab_size"], size=45)
+    for pos, t in enumerate(prompt):
+        c_next, c_logits = cpu.forward(int(t), pos)
+    g_next, g_logits = gpu.forward_tokens(prompt)  # 44 rows through the GEMM, the last as a one-token step
+    assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL and g_next == c_next
+    tok = c_next
+    for pos in range(45, 53):
+        c_next, c_logits = cpu.forward(tok, pos)
+        g_next, g_logits = gpu.forward(tok)
+        assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, pos
+        assert g_next == c_next, pos
+        tok = c_next
+    few = [int(t) for t in prompt[:6]]  # six more rows at once: the small-batch GEMV where it covers the types
+    for i, t in enumerate(few):
+        c_next, c_logits = cpu.forward(t, 53 + i)
+    g_next, g_logits = gpu.forward_tokens(few)
+    assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL and g_next == c_next
+    # going back to the fused weight's own type puts the part back into it
+    (l, name), _ = next(iter(changes.items()))
+    if l >= 0 and name in ("q", "k", "v"):
+        n, k = LIN_SHAPES(c)[name]
+        w2 = dict(w, types=dict(w["types"]))
+        w2["layers"] = [dict(L) for L in w["layers"]]
+        w2["layers"][l][name] = o.quantize(w["qtype"], (np.random.default_rng(73).standard_normal((n, k)) * 0.06).astype(np.float32))
+        del w2["types"][(l, name)]
+        gpu.set_linear(l, name, q.QuantizedTensor([n, k], w["qtype"], w2["layers"][l][name]))
+        gpu.reset()
+        cpu2 = load_oracle(c, w2)
+        tok = 7
+        for pos in range(6):
+            c_next, c_logits = cpu2.forward(tok, pos)
+            g_next, g_logits = gpu.forward(tok)
+            assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL and g_next == c_next
+            tok = c_next
+        cpu2.close()
+    gpu.close()
+    cpu.close()
