@@ -52,13 +52,13 @@ class CalibrationData:
 
     def symmetric_scale(self, quant_type):
         """max(|min|, |max|) / largest code (calibration.rs:93-102)."""
-        max_int = {QuantType.Q8_0: 127.0, QuantType.Q4_0: 7.0, QuantType.Q4_1: 7.0, QuantType.Q4_K: 7.0, QuantType.Q6_K: 31.0,
+        max_int = {QuantType.Q8_0: 127.0, QuantType.Q4_0: 7.0, QuantType.Q4_1: 7.0, QuantType.Q4_K: 7.0, QuantType.Q6_K: 31.0, QuantType.Q5_K: 15.0,
                    QuantType.Q5_0: 15.0, QuantType.Q5_1: 15.0, QuantType.F16: 1.0, QuantType.F32: 1.0}[QuantType(quant_type)]
         return float(_F(max(abs(self.min), abs(self.max))) / _F(max_int))
 
     def asymmetric_scale(self, quant_type):
         """(scale, zero_point) over the full unsigned code range (calibration.rs:105-117)."""
-        max_int = {QuantType.Q8_0: 255.0, QuantType.Q4_0: 15.0, QuantType.Q4_1: 15.0, QuantType.Q4_K: 15.0, QuantType.Q6_K: 63.0,
+        max_int = {QuantType.Q8_0: 255.0, QuantType.Q4_0: 15.0, QuantType.Q4_1: 15.0, QuantType.Q4_K: 15.0, QuantType.Q6_K: 63.0, QuantType.Q5_K: 31.0,
                    QuantType.Q5_0: 31.0, QuantType.Q5_1: 31.0, QuantType.F16: 1.0, QuantType.F32: 1.0}[QuantType(quant_type)]
         scale = (_F(self.max) - _F(self.min)) / _F(max_int)
         with np.errstate(divide="ignore", invalid="ignore"):

@@ -219,7 +219,12 @@ __global__ void __launch_bounds__(128) quant_q5_kernel(const float *src, size_t 
 // min = -mn; the superblock's d = max scale / 63, dmin = max min / 63 (stored
 // as f16); 6-bit ls = round(63/max_scale * scale), lm likewise; codes
 // q = clamp(round((x + dmin*lm) / (d*ls)), 0, 15) with the f16-rounded d, dmin.
-__global__ void quant_q4_k_kernel(const float *src, size_t numel, size_t nsb, uint8_t *out) {
+// BITS = 5 is Q5_K: the same rule with 31 steps; image [header 16][qh 32][qs 128], the low four bits of a code where
+// Q4_K has the code, the fifth bit of sub-block s, element l at bit s of qh[l].
+template <int BITS>
+__global__ void quant_qk_kernel(const float *src, size_t numel, size_t nsb, uint8_t *out) {
+    constexpr float TOP = BITS == 5 ? 31.0f : 15.0f;
+    constexpr int IMG = BITS == 5 ? 176 : 144, QS = BITS == 5 ? 48 : 16;
     size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     size_t sb = t >> 3;
     int s = (int)(t & 7);
@@ -254,7 +259,7 @@ __global__ void quant_q4_k_kernel(const float *src, size_t numel, size_t nsb, ui
         scale = 0.0f;
         smin = isfinite(mn) ? -mn : 0.0f;
     } else {
-        scale = (mx - mn) / 15.0f;
+        scale = (mx - mn) / TOP;
         smin = -mn;
     }
     float max_scale = scale, max_min = smin;
@@ -272,15 +277,16 @@ __global__ void quant_q4_k_kernel(const float *src, size_t numel, size_t nsb, ui
     float d = f16_bits_to_f32(dh), dmin = f16_bits_to_f32(dminh);
     float sd = d * (float)ls;
     float sm = dmin * (float)lm;
-    // codes as 8 dwords of one code per byte
-    uint32_t cb[8];
+    // codes as 8 dwords of one code per byte (their low four bits), the fifth bits as one bit per element
+    uint32_t cb[8], hb = 0;
 #pragma unroll
     for (int w = 0; w < 8; w++) {
         uint32_t v = 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            int q = sd == 0.0f ? 0 : round_clamp((x[4 * w + j] + sm) / sd, 0.0f, 15.0f);
-            v |= (uint32_t)q << (8 * j);
+            int q = sd == 0.0f ? 0 : round_clamp((x[4 * w + j] + sm) / sd, 0.0f, TOP);
+            v |= (uint32_t)(q & 15) << (8 * j);
+            hb |= (uint32_t)(q >> 4) << (4 * w + j);
         }
         cb[w] = v;
     }
@@ -290,14 +296,23 @@ __global__ void quant_q4_k_kernel(const float *src, size_t numel, size_t nsb, ui
     for (int w = 0; w < 8; w++) other[w] = (uint32_t)__shfl_xor((int)cb[w], 1);
     // header values of all 8 sub-blocks
     int base_lane = (int)(threadIdx.x & 63) & ~7;
-    uint32_t lsv[8], lmv[8];
+    uint32_t lsv[8], lmv[8], hbv[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         lsv[j] = (uint32_t)__shfl(ls, base_lane + j);
         lmv[j] = (uint32_t)__shfl(lm, base_lane + j);
+        if (BITS == 5) hbv[j] = (uint32_t)__shfl((int)hb, base_lane + j);
     }
     if (!live) return;
-    uint8_t *o = out + sb * 144;
+    uint8_t *o = out + sb * IMG;
+    if (BITS == 5) { // this lane's four bytes of qh: elements 4 s .. 4 s + 3, bit j from sub-block j
+        uint32_t v = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) v |= ((hbv[j] >> (4 * s + i)) & 1u) << (8 * i + j);
+        *reinterpret_cast<uint32_t *>(o + 16 + 4 * s) = v;
+    }
     if (s == 0) {
         uint32_t h[4];
         h[0] = (uint32_t)dh | ((uint32_t)dminh << 16);
@@ -319,7 +334,7 @@ __global__ void quant_q4_k_kernel(const float *src, size_t numel, size_t nsb, ui
         uint32_t pk[8];
 #pragma unroll
         for (int w = 0; w < 8; w++) pk[w] = cb[w] | (other[w] << 4);
-        uint4 *q = reinterpret_cast<uint4 *>(o + 16 + 32 * p);
+        uint4 *q = reinterpret_cast<uint4 *>(o + QS + 32 * p);
         q[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
         q[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
     }
@@ -518,10 +533,12 @@ __global__ void __launch_bounds__(128) dequant_kernel(int type, const uint8_t *p
         }
         break;
     }
-    case AXQ_Q4_K: {
+    case AXQ_Q4_K:
+    case AXQ_Q5_K: {
         size_t sb = t >> 3;
         int s = (int)(t & 7);
-        const uint8_t *b = packed + sb * 144;
+        const bool five = type == AXQ_Q5_K;
+        const uint8_t *b = packed + sb * (five ? 176 : 144);
         float d = f16_bits_to_f32(load_u16(b));
         float dmin = f16_bits_to_f32(load_u16(b + 2));
         const uint8_t *sc = b + 4;
@@ -535,14 +552,16 @@ __global__ void __launch_bounds__(128) dequant_kernel(int type, const uint8_t *p
         }
         float sd = d * (float)l;
         float sm = dmin * (float)m;
-        const uint32_t *qs = reinterpret_cast<const uint32_t *>(b + 16 + 32 * (s >> 1));
+        const uint32_t *qs = reinterpret_cast<const uint32_t *>(b + (five ? 48 : 16) + 32 * (s >> 1));
+        const uint32_t *qh = reinterpret_cast<const uint32_t *>(b + 16); // Q5_K: bit s of byte l = fifth bit of the sub-block's element l
         int shift = (s & 1) * 4;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            uint32_t w = qs[i] >> shift;
+            uint32_t w = (qs[i] >> shift) & 0x0F0F0F0Fu;
+            if (five) w |= ((qh[i] >> s) & 0x01010101u) << 4;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                float a = sd * (float)((w >> (8 * j)) & 0x0F);
+                float a = sd * (float)((w >> (8 * j)) & 0x1F);
                 y[4 * i + j] = a - sm;
             }
         }
@@ -733,6 +752,21 @@ __global__ void __launch_bounds__(256) repack_q6k_kernel(PlanarDesc d, uint8_t *
     }
 }
 
+// Q5_K: image [header 16][qh 32][qs 128] <-> planes: meta = the headers, qh = the fifth bits as they are, codes = the qs
+// runs laid out as Q4_K's (q4k_code_offset).  One thread per 16-byte piece, eleven per superblock.
+__global__ void __launch_bounds__(256) repack_q5k_kernel(PlanarDesc d, uint8_t *packed, bool to_planar, int64_t total) {
+    const int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= total * 11) return;
+    const int64_t t = v / 11;
+    const int piece = (int)(v - t * 11);
+    const int64_t row = t / d.blocks_per_row, sb = t - row * d.blocks_per_row;
+    uint8_t *im = packed + (size_t)t * 176 + 16 * piece, *pl;
+    if (piece == 0) pl = d.meta + (size_t)row * d.meta_pitch + (size_t)sb * 16;
+    else if (piece < 3) pl = d.qh + (size_t)row * d.qh_pitch + (size_t)sb * 32 + 16 * (piece - 1);
+    else pl = d.codes + (size_t)row * d.codes_pitch + q4k_code_offset(d.blocks_per_row, sb, 16 * (piece - 3));
+    if (to_planar) copy_u16s(pl, im, 16); else copy_u16s(im, pl, 16);
+}
+
 inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
 
 } // namespace
@@ -747,7 +781,8 @@ int axq_dev_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, uin
     case AXQ_Q4_1: quant_q4_1_kernel<<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_Q5_0: quant_q5_kernel<false><<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_Q5_1: quant_q5_kernel<true><<<grid_for(nblk, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
-    case AXQ_Q4_K: quant_q4_k_kernel<<<grid_for(nblk * 8, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_Q4_K: quant_qk_kernel<4><<<grid_for(nblk * 8, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
+    case AXQ_Q5_K: quant_qk_kernel<5><<<grid_for(nblk * 8, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_Q6_K: quant_q6_k_kernel<<<grid_for(nblk * 16, B), B, 0, ctx->stream>>>(src, numel, nblk, packed); break;
     case AXQ_F16: quant_f16_kernel<<<grid_for((numel + 7) / 8, 256), 256, 0, ctx->stream>>>(src, numel, (uint16_t *)packed); break;
     case AXQ_F32:
@@ -762,7 +797,7 @@ int axq_dev_quantize(axq_ctx *ctx, int type, const float *src, size_t numel, uin
 int axq_dev_dequantize(axq_ctx *ctx, int type, const uint8_t *packed, size_t numel, float *dst) {
     if (numel == 0) return AXQ_OK;
     switch (type) {
-    case AXQ_Q8_0: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q4_K: case AXQ_Q6_K: {
+    case AXQ_Q8_0: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q4_K: case AXQ_Q6_K: case AXQ_Q5_K: {
         size_t n32 = (numel + 31) / 32;
         dequant_kernel<<<grid_for(n32, 128), 128, 0, ctx->stream>>>(type, packed, numel, n32, dst);
         break;
@@ -794,6 +829,11 @@ int axq_dev_repack(axq_ctx *ctx, const axq_weight *w, uint8_t *packed, bool to_p
     d.type = w->type;
     size_t total = (size_t)(d.n_rows * d.blocks_per_row);
     if (total == 0) return AXQ_OK;
+    if (w->type == AXQ_Q5_K) {
+        repack_q5k_kernel<<<grid_for(total * 11, 256), 256, 0, ctx->stream>>>(d, packed, to_planar, (int64_t)total);
+        AXQ_LAUNCH_CHECK(ctx, "repack kernel");
+        return AXQ_OK;
+    }
     if (w->type == AXQ_Q6_K) {
         repack_q6k_kernel<<<grid_for(total * 13, 256), 256, 0, ctx->stream>>>(d, packed, to_planar, (int64_t)total);
         AXQ_LAUNCH_CHECK(ctx, "repack kernel");

@@ -24,7 +24,7 @@ extern "C" {
 size_t axq_type_block_size(int type) {
     switch (type) {
     case AXQ_Q8_0: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: return 32;
-    case AXQ_Q4_K: case AXQ_Q6_K: return 256;
+    case AXQ_Q4_K: case AXQ_Q6_K: case AXQ_Q5_K: return 256;
     case AXQ_F16: case AXQ_F32: return 1;
     default: return 0;
     }
@@ -39,6 +39,7 @@ size_t axq_type_bytes_per_block(int type) {
     case AXQ_Q5_1: return 4 + 20;
     case AXQ_Q4_K: return 4 + 12 + 128;
     case AXQ_Q6_K: return 128 + 64 + 16 + 2;
+    case AXQ_Q5_K: return 4 + 12 + 32 + 128;
     case AXQ_F16: return 2;
     case AXQ_F32: return 4;
     default: return 0;
@@ -49,7 +50,7 @@ size_t axq_type_bits_per_value(int type) {
     switch (type) {
     case AXQ_Q8_0: return 8;
     case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q4_K: return 4;
-    case AXQ_Q5_0: case AXQ_Q5_1: return 5;
+    case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q5_K: return 5;
     case AXQ_Q6_K: return 6;
     case AXQ_F16: return 16;
     case AXQ_F32: return 32;
@@ -59,7 +60,7 @@ size_t axq_type_bits_per_value(int type) {
 
 int axq_type_is_block_quantized(int type) {
     switch (type) {
-    case AXQ_Q8_0: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q4_K: case AXQ_Q6_K: return 1;
+    case AXQ_Q8_0: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q4_K: case AXQ_Q6_K: case AXQ_Q5_K: return 1;
     default: return 0;
     }
 }
@@ -75,6 +76,7 @@ const char *axq_type_name(int type) {
     case AXQ_F32: return "F32";
     case AXQ_Q4_K: return "Q4_K";
     case AXQ_Q6_K: return "Q6_K";
+    case AXQ_Q5_K: return "Q5_K";
     default: return NULL;
     }
 }
@@ -92,6 +94,7 @@ int axq_type_from_str(const char *s) {
         {"F32", AXQ_F32}, {"FLOAT32", AXQ_F32}, {"FLOAT", AXQ_F32},
         {"Q4_K", AXQ_Q4_K}, {"Q4K", AXQ_Q4_K},
         {"Q6_K", AXQ_Q6_K}, {"Q6K", AXQ_Q6_K},
+        {"Q5_K", AXQ_Q5_K}, {"Q5K", AXQ_Q5_K},
     };
     for (size_t i = 0; i < sizeof table / sizeof table[0]; i++)
         if (strcasecmp(s, table[i].name) == 0) return table[i].type;

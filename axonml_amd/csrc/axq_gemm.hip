@@ -213,6 +213,52 @@ struct GQ80 {
     }
 };
 
+struct GQ5K { // GGUF Q5_K on Q4_K's planes: the codes' low four bits as GQ4K reads them, the fifth bits from the qh plane
+    static constexpr bool PRESCALED = true;
+    static constexpr float WS = WSCALE;
+    struct Raw { uint2 q, b; uint4 h; };
+    __device__ static void load16(const GemmArgs &a, size_t row, int kstep, int u4, Raw &r) {
+        const int cpr = a.k >> 6;
+        const int pair = kstep;
+        const int slice = pair >> 6, pr = pair & 63;
+        int P = cpr - (slice << 6);
+        P = P < 64 ? P : 64;
+        const int half = u4 >> 1, part = u4 & 1;
+        r.q = *reinterpret_cast<const uint2 *>(a.codes + row * a.codes_pitch + (size_t)slice * 2048 + (size_t)half * 16 * P + (size_t)pr * 16 + part * 8);
+        r.h = *reinterpret_cast<const uint4 *>(a.meta + row * a.meta_pitch + (size_t)(pair >> 2) * 16);
+        // bytes l = 16 half + 8 part .. + 7 of the superblock's 32: bit 2 p (+ 1) = fifth bit of element l of the pair's low (high) sub-block
+        r.b = *reinterpret_cast<const uint2 *>(a.qh + row * a.qh_pitch + (size_t)(pair >> 2) * 32 + half * 16 + part * 8);
+    }
+    __device__ static void cvt16(const Raw &r, int kstep, int u4, float (&w)[16], int &k0, int &k1) {
+        const int pair = kstep, half = u4 >> 1, part = u4 & 1;
+        const int p = pair & 3, sh = (p & 1) * 16;
+        const uint32_t ya = r.h.y >> sh, za = r.h.z >> sh, wa = r.h.w >> sh;
+        uint32_t scp, mp;
+        if (p < 2) {
+            scp = ya & 0x3F3F;
+            mp = za & 0x3F3F;
+        } else {
+            scp = (wa & 0x0F0F) | ((ya >> 2) & 0x3030);
+            mp = ((wa >> 4) & 0x0F0F) | ((za >> 2) & 0x3030);
+        }
+        const float d = WSCALE * h2f(r.h.x & 0xFFFF), dmin = WSCALE * h2f(r.h.x >> 16);
+        const float sd0 = d * ubyte<0>(scp), sd1 = d * ubyte<1>(scp);
+        const float sm0 = dmin * ubyte<0>(mp), sm1 = dmin * ubyte<1>(mp);
+        const uint32_t q[2] = {r.q.x, r.q.y}, b[2] = {r.b.x, r.b.y};
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint32_t ul = (q[j] & 0x0F0F0F0Fu) | (((b[j] >> (2 * p)) & 0x01010101u) << 4);
+            const uint32_t uh = ((q[j] >> 4) & 0x0F0F0F0Fu) | (((b[j] >> (2 * p + 1)) & 0x01010101u) << 4);
+            w[4 * j + 0] = fmaf(sd0, ubyte<0>(ul), -sm0); w[4 * j + 1] = fmaf(sd0, ubyte<1>(ul), -sm0);
+            w[4 * j + 2] = fmaf(sd0, ubyte<2>(ul), -sm0); w[4 * j + 3] = fmaf(sd0, ubyte<3>(ul), -sm0);
+            w[8 + 4 * j + 0] = fmaf(sd1, ubyte<0>(uh), -sm1); w[8 + 4 * j + 1] = fmaf(sd1, ubyte<1>(uh), -sm1);
+            w[8 + 4 * j + 2] = fmaf(sd1, ubyte<2>(uh), -sm1); w[8 + 4 * j + 3] = fmaf(sd1, ubyte<3>(uh), -sm1);
+        }
+        k0 = half * 16 + part * 8;
+        k1 = 32 + k0;
+    }
+};
+
 struct GQ6K { // GGUF Q6_K: a unit is one sub-block of 16 consecutive elements with its own int8 scale
     static constexpr bool PRESCALED = true;
     // d * scale * q reaches 127 * 32 times d: a smaller factor than WSCALE leaves weights up to 4000 finite in f16 and
@@ -1574,6 +1620,7 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     switch (w->type) {
     case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);
     case AXQ_Q6_K: return launch_gemm<GQ6K>(ctx, a, p.splits);
+    case AXQ_Q5_K: return launch_gemm<GQ5K>(ctx, a, p.splits);
     case AXQ_Q4_0: return launch_gemm<GQ4x<false>>(ctx, a, p.splits);
     case AXQ_Q4_1: return launch_gemm<GQ4x<true>>(ctx, a, p.splits);
     case AXQ_Q5_0: return launch_gemm<GQ5x<false>>(ctx, a, p.splits);

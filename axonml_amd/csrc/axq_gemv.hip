@@ -267,6 +267,66 @@ struct Q80 { // chunk = 16 int8 = half a block
     }
 };
 
+struct Q5K { // GGUF Q5_K; chunk = one pair of sub-blocks (64 elements): Q4_K's codes and header, the fifth bits from the qh plane
+    static constexpr int W = 64;
+    struct X { float xs[64]; };
+    struct Raw { uint4 q0, q1, h, b0, b1; };
+    template <class F>
+    __device__ static void set_x(const GemvArgs &, F fetch, X &o) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float4 v = fetch(i);
+            o.xs[4 * i] = v.x; o.xs[4 * i + 1] = v.y; o.xs[4 * i + 2] = v.z; o.xs[4 * i + 3] = v.w;
+        }
+    }
+    __device__ static void load(const GemvArgs &a, int row, int chunk, Raw &r) {
+        int slice = chunk >> 6, lane_pair = chunk & 63;
+        int P = a.cpr - (slice << 6);
+        P = P < 64 ? P : 64;
+        const uint8_t *base = a.codes + (size_t)row * a.codes_pitch + (size_t)slice * 2048 + (size_t)lane_pair * 16;
+        r.q0 = *reinterpret_cast<const uint4 *>(base);
+        r.q1 = *reinterpret_cast<const uint4 *>(base + (size_t)P * 16);
+        r.h = *reinterpret_cast<const uint4 *>(a.meta + (size_t)row * a.meta_pitch + (size_t)(chunk >> 2) * 16);
+        const uint4 *qh = reinterpret_cast<const uint4 *>(a.qh + (size_t)row * a.qh_pitch + (size_t)(chunk >> 2) * 32);
+        r.b0 = qh[0]; // byte l: bit 2 p + h = fifth bit of element l of sub-block 2 p + h
+        r.b1 = qh[1];
+    }
+    __device__ static float dot(const GemvArgs &, const Raw &r, const X &x, int chunk) {
+        const int p = chunk & 3;
+        const int sh = (p & 1) * 16;
+        const uint32_t ya = r.h.y >> sh, za = r.h.z >> sh, wa = r.h.w >> sh;
+        uint32_t scp, mp;
+        if (p < 2) {
+            scp = ya & 0x3F3F;
+            mp = za & 0x3F3F;
+        } else {
+            scp = (wa & 0x0F0F) | ((ya >> 2) & 0x3030);
+            mp = ((wa >> 4) & 0x0F0F) | ((za >> 2) & 0x3030);
+        }
+        const float d = f16_bits_to_f32(r.h.x & 0xFFFF), dmin = f16_bits_to_f32(r.h.x >> 16);
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const uint32_t b[8] = {r.b0.x, r.b0.y, r.b0.z, r.b0.w, r.b1.x, r.b1.y, r.b1.z, r.b1.w};
+        float lo = 0.f, hi = 0.f, slo = 0.f, shi = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) { // bytes 4 w ..: elements 4 w .. of the low sub-block, 32 + 4 w .. of the high one
+            const uint32_t ul = (q[w] & 0x0F0F0F0Fu) | (((b[w] >> (2 * p)) & 0x01010101u) << 4);
+            const uint32_t uh = ((q[w] >> 4) & 0x0F0F0F0Fu) | (((b[w] >> (2 * p + 1)) & 0x01010101u) << 4);
+            // codes centred (u - 16) before the multiply: no large sums cancel for an x with a mean
+            lo = fmaf(ubyte0(ul) - 16.0f, x.xs[4 * w], lo);      hi = fmaf(ubyte0(uh) - 16.0f, x.xs[32 + 4 * w], hi);
+            lo = fmaf(ubyte1(ul) - 16.0f, x.xs[4 * w + 1], lo);  hi = fmaf(ubyte1(uh) - 16.0f, x.xs[32 + 4 * w + 1], hi);
+            lo = fmaf(ubyte2(ul) - 16.0f, x.xs[4 * w + 2], lo);  hi = fmaf(ubyte2(uh) - 16.0f, x.xs[32 + 4 * w + 2], hi);
+            lo = fmaf(ubyte3(ul) - 16.0f, x.xs[4 * w + 3], lo);  hi = fmaf(ubyte3(uh) - 16.0f, x.xs[32 + 4 * w + 3], hi);
+            slo += (x.xs[4 * w] + x.xs[4 * w + 1]) + (x.xs[4 * w + 2] + x.xs[4 * w + 3]);
+            shi += (x.xs[32 + 4 * w] + x.xs[32 + 4 * w + 1]) + (x.xs[32 + 4 * w + 2] + x.xs[32 + 4 * w + 3]);
+        }
+        const float s0 = d * ubyte0(scp), s1 = d * ubyte1(scp);
+        float y = fmaf(s0, lo, s1 * hi); // sum d * sc * (u - 16) * x
+        y = fmaf(fmaf(16.0f, s0, -(dmin * ubyte0(mp))), slo, y);
+        y = fmaf(fmaf(16.0f, s1, -(dmin * ubyte1(mp))), shi, y);
+        return y;
+    }
+};
+
 struct Q6K { // GGUF Q6_K; chunk = one sub-block of 16 elements: 16 bytes of low nibbles, 16 of bit pairs, an int8 scale
     static constexpr int W = 16;
     struct X { float xs[16]; };
@@ -639,6 +699,7 @@ int axq_dev_gemv(axq_ctx *ctx, const axq_weight *w, const float *x, int batch, c
         switch (w->type) {
         case AXQ_Q4_K: rc = launch<Q4K>(ctx, w, xb, bias, yb); break;
         case AXQ_Q6_K: rc = launch<Q6K>(ctx, w, xb, bias, yb); break;
+        case AXQ_Q5_K: rc = launch<Q5K>(ctx, w, xb, bias, yb); break;
         case AXQ_Q4_0: rc = launch<Q4x<false>>(ctx, w, xb, bias, yb); break;
         case AXQ_Q4_1: rc = launch<Q4x<true>>(ctx, w, xb, bias, yb); break;
         case AXQ_Q5_0: rc = launch<Q5x<false>>(ctx, w, xb, bias, yb); break;

@@ -109,6 +109,7 @@ int axq_type_from_ggml(int ggml_type) {
     case 7: return AXQ_Q5_1;
     case 8: return AXQ_Q8_0;
     case 12: return AXQ_Q4_K;
+    case 13: return AXQ_Q5_K;
     case 14: return AXQ_Q6_K;
     default: return -1;
     }
@@ -124,6 +125,7 @@ int axq_type_to_ggml(int type) {
     case AXQ_Q5_1: return 7;
     case AXQ_Q8_0: return 8;
     case AXQ_Q4_K: return 12;
+    case AXQ_Q5_K: return 13;
     case AXQ_Q6_K: return 14;
     default: return -1;
     }

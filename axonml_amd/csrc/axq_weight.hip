@@ -63,6 +63,7 @@ int axq_weight_alloc(axq_ctx *ctx, int type, int64_t n_rows, int64_t k, axq_weig
     case AXQ_Q5_1: w->codes_pitch = (size_t)k / 2; meta_per_block = 4; qh_per_block = 4; break;
     case AXQ_Q4_K: w->codes_pitch = (size_t)k / 2; meta_per_block = 16; break;
     case AXQ_Q6_K: w->codes_pitch = (size_t)k / 2; meta_per_block = 18; qh_per_block = 64; break; // scales, then the row's d values
+    case AXQ_Q5_K: w->codes_pitch = (size_t)k / 2; meta_per_block = 16; qh_per_block = 32; break; // Q4_K's planes and the fifth bits as they are
     case AXQ_F16: w->codes_pitch = (size_t)k * 2; break;
     case AXQ_F32: w->codes_pitch = (size_t)k * 4; break;
     }

@@ -5,8 +5,8 @@ stops there; its `axonml quant convert` writes nothing a reader could load (quan
 implements the GGUF v2/v3 container as specified by ggml: little-endian header, typed metadata, tensor
 table, aligned data section.  Tensor payloads are ggml block images; `axq_gguf_convert_blocks` (device)
 turns Q4_0 / Q4_1 images into the reference's nibble order and back, every other supported type is
-byte-identical (Q6_K among them: the reference has no such type, the block is ggml's).  ggml types this library
-has no kernel for (Q2_K, Q3_K, Q5_K, IQ*, ...) raise GGUFError.
+byte-identical (Q5_K and Q6_K among them: the reference has no such types, the blocks are ggml's).  ggml types this library
+has no kernel for (Q2_K, Q3_K, IQ*, ...) raise GGUFError.
 
 Tensor names and metadata keys of the loader follow llama.cpp's converter for the `llama` architecture,
 mapped onto the reference's LLaMA module names (crates/axonml-llm/src/llama.rs:782-822).
@@ -173,7 +173,7 @@ class GGUFReader:
         t = self.info(name)
         if t.quant_type is None:
             raise GGUFError(f"tensor {name}: ggml type {GGML_TYPE_NAMES.get(t.ggml_type, t.ggml_type)} is not supported "
-                            f"(supported: F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q6_K)")
+                            f"(supported: F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K)")
         return np.frombuffer(self._mm, dtype=np.uint8, count=t.nbytes, offset=self.data_start + t.offset)
 
     def close(self):

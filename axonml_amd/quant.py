@@ -11,7 +11,7 @@ Names, argument meaning and error behaviour follow the reference crate
 
 Every function computes on the GPU through ``libaxq.so``; tensors are numpy
 arrays on the host side of the boundary.  Differences from the reference, all
-additions: ``QuantType.Q4_K`` and ``QuantType.Q6_K`` (GGUF superblocks); Q5_0/Q5_1 have real codecs (the reference aliases
+additions: ``QuantType.Q4_K``, ``QuantType.Q5_K`` and ``QuantType.Q6_K`` (GGUF superblocks); Q5_0/Q5_1 have real codecs (the reference aliases
 them to Q4_0, quantize.rs:47-50); a ``QuantizedTensor`` holds its blocks as one
 flat byte buffer in ``to_bytes`` order instead of a Vec of enum values.
 """
@@ -93,6 +93,7 @@ class QuantType(enum.IntEnum):
     F32 = 6
     Q4_K = 7
     Q6_K = 8
+    Q5_K = 9
 
     def block_size(self):
         return _lib.load_library().axq_type_block_size(int(self))

@@ -47,7 +47,8 @@ typedef struct axq_model axq_model;
 /* QuantType, crates/axonml-quant/src/types.rs:17-41, in the same order, with
  * the 256-element GGUF superblock types appended: Q4_K (144 bytes) and Q6_K (210 bytes: 128 bytes of low nibbles,
  * 64 of high bit pairs, sixteen int8 scales of 16 elements each, f16 d; w = d * scale * (q - 32)), the type llama.cpp
- * keeps output.weight and part of the value and down projections in when it writes "Q4_0" and "Q4_K_M" files. */
+ * keeps output.weight and part of the value and down projections in when it writes "Q4_0" and "Q4_K_M" files; and
+ * Q5_K (176 bytes: Q4_K's header, 32 bytes of fifth bits, 128 of low nibbles; w = d * sc * q - dmin * m, q in 0..31). */
 typedef enum {
     AXQ_Q8_0 = 0,
     AXQ_Q4_0 = 1,
@@ -58,7 +59,8 @@ typedef enum {
     AXQ_F32 = 6,
     AXQ_Q4_K = 7,
     AXQ_Q6_K = 8,
-    AXQ_TYPE_COUNT = 9
+    AXQ_Q5_K = 9,
+    AXQ_TYPE_COUNT = 10
 } axq_type;
 
 typedef enum {

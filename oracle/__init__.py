@@ -12,8 +12,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
-Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, F16, F32, Q4_K, Q6_K = range(9)
-TYPE_NAMES = {Q8_0: "Q8_0", Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", F16: "F16", F32: "F32", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, F16, F32, Q4_K, Q6_K, Q5_K = range(10)
+TYPE_NAMES = {Q8_0: "Q8_0", Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", F16: "F16", F32: "F32", Q4_K: "Q4_K", Q6_K: "Q6_K", Q5_K: "Q5_K"}
 
 
 class ModelConfig(C.Structure):

@@ -43,7 +43,7 @@ int axo_gguf_convert(int type, const uint8_t *src, uint8_t *dst, size_t nblocks,
 int axo_ggml_dequantize(int type, const uint8_t *blocks, size_t nblocks, float *dst);
 int axo_get_next_token(float *logits, int n, const int32_t *generated, int n_generated, const axo_sampling_config *c, float u);
 
-enum { Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, F16, F32, Q4_K, Q6_K };
+enum { Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, F16, F32, Q4_K, Q6_K, Q5_K };
 
 static uint64_t rng_state = 0x9E3779B97F4A7C15ull;
 static float rnd(void) { /* uniform in (-1, 1) */
@@ -62,7 +62,7 @@ static void *exact(size_t bytes) {
 
 static void codecs(void) {
     static const size_t sizes[] = {1, 2, 31, 32, 33, 35, 40, 63, 255, 256, 257, 300, 1000, 4096};
-    for (int t = Q8_0; t <= Q6_K; t++) {
+    for (int t = Q8_0; t <= Q5_K; t++) {
         for (size_t si = 0; si < sizeof sizes / sizeof sizes[0]; si++) {
             const size_t n = sizes[si], nb = axo_packed_bytes(t, n);
             float *x = exact(n * sizeof(float)), *y = exact(n * sizeof(float));
@@ -78,7 +78,7 @@ static void codecs(void) {
 }
 
 static void matmul(void) {
-    for (int t = Q8_0; t <= Q6_K; t++) {
+    for (int t = Q8_0; t <= Q5_K; t++) {
         const size_t M = 3, N = 37, K = 512;
         float *w = exact(N * K * sizeof(float)), *x = exact(M * K * sizeof(float)), *b = exact(N * sizeof(float));
         float *y = exact(M * N * sizeof(float)), *scratch = exact(2 * N * K * sizeof(float)), *deq = exact(N * K * sizeof(float));
@@ -150,7 +150,7 @@ static void sampler(void) {
 }
 
 static void gguf(void) {
-    for (int t = Q8_0; t <= Q6_K; t++) {
+    for (int t = Q8_0; t <= Q5_K; t++) {
         if (t == F16 || t == F32) continue;
         const size_t nb = 9, bb = axo_bytes_per_block(t), total = nb * bb;
         uint8_t *a = exact(total), *b = exact(total), *c = exact(total);

@@ -37,6 +37,8 @@
  *     blocks derived from the reference source (zero block, ramp, half-way
  *     rounding cases, tail block, Q4_1 odd tail) and by the reference's own
  *     test inputs (types.rs:366-389, dequantize.rs:204-272).
+ *   Q5_K: Q4_K's rule with 31 steps and a fifth bit per code; layout and dequantiser from the published GGUF block
+ *     (hand-built superblocks, an independent numpy statement of ggml's row dequantiser); quantiser "parity unpinned".
  *   Q6_K: as Q4_K below -- no reference code, no fixture; the layout and the dequantiser follow the published GGUF
  *     block (pinned by hand-built superblocks, one-hot codes and an independent numpy statement of ggml's row
  *     dequantiser), the QUANTISER rule is this build's own ("parity unpinned").
@@ -73,7 +75,8 @@ enum {
     AXO_F16 = 5,
     AXO_F32 = 6,
     AXO_Q4_K = 7,
-    AXO_Q6_K = 8
+    AXO_Q6_K = 8,
+    AXO_Q5_K = 9
 };
 
 /* ------------------------------------------------------------------------- */
@@ -145,7 +148,7 @@ AXO_API float axo_f16_to_f32(uint16_t h) {
 AXO_API size_t axo_block_size(int type) {
     switch (type) {
     case AXO_Q8_0: case AXO_Q4_0: case AXO_Q4_1: case AXO_Q5_0: case AXO_Q5_1: return 32;
-    case AXO_Q4_K: case AXO_Q6_K: return 256;
+    case AXO_Q4_K: case AXO_Q6_K: case AXO_Q5_K: return 256;
     case AXO_F16: case AXO_F32: return 1;
     default: return 0;
     }
@@ -160,6 +163,7 @@ AXO_API size_t axo_bytes_per_block(int type) {
     case AXO_Q5_1: return 24;
     case AXO_Q4_K: return 144;
     case AXO_Q6_K: return 210;
+    case AXO_Q5_K: return 176;
     case AXO_F16: return 2;
     case AXO_F32: return 4;
     default: return 0;
@@ -304,7 +308,16 @@ static void quant_block_q5_1(const float *x, size_t len, uint8_t *out) {
  *   with the f16-rounded d,dmin:  sd = d*ls_s, sm = dmin*lm_s,
  *   q = clamp(round((x + sm)/sd), 0, 15)  (0 when sd == 0).
  * A short tail superblock is zero-padded before quantisation. */
-static void quant_block_q4_k(const float *xin, size_t len, uint8_t *out) {
+static void quant_block_qk(const float *xin, size_t len, uint8_t *out, int bits);
+static void quant_block_q4_k(const float *xin, size_t len, uint8_t *out) { quant_block_qk(xin, len, out, 4); }
+
+/* Q5_K, GGUF layout [f16 d][f16 dmin][u8 scales[12]][u8 qh[32]][u8 qs[128]] (176 bytes): header and qs as Q4_K's, with
+ * the low four bits of the 5-bit codes in qs; the fifth bit of element 64 p + 32 h + l (pair p, half h) is bit 2 p + h of
+ * qh[l].  Dequant: w = (d*sc_s)*q - (dmin*m_s), q in 0..31.  Quantiser rule: Q4_K's with 31 steps instead of 15. */
+static void quant_block_q5_k(const float *xin, size_t len, uint8_t *out) { quant_block_qk(xin, len, out, 5); }
+
+static void quant_block_qk(const float *xin, size_t len, uint8_t *out, int bits) {
+    const float top = bits == 5 ? 31.0f : 15.0f;
     float x[256];
     memset(x, 0, sizeof x);
     memcpy(x, xin, len * sizeof(float));
@@ -319,7 +332,7 @@ static void quant_block_q4_k(const float *xin, size_t len, uint8_t *out) {
             scales[s] = 0.0f;
             mins[s] = isfinite(mn) ? -mn : 0.0f;
         } else {
-            scales[s] = (mx - mn) / 15.0f;
+            scales[s] = (mx - mn) / top;
             mins[s] = -mn;
         }
         max_scale = rs_max(max_scale, scales[s]);
@@ -351,13 +364,21 @@ static void quant_block_q4_k(const float *xin, size_t len, uint8_t *out) {
             if (sd == 0.0f) {
                 q[32 * s + i] = 0;
             } else {
-                q[32 * s + i] = (uint8_t)rs_round_clamp((x[32 * s + i] + sm) / sd, 0.0f, 15.0f);
+                q[32 * s + i] = (uint8_t)rs_round_clamp((x[32 * s + i] + sm) / sd, 0.0f, top);
             }
         }
     }
     uint8_t *qs = out + 16;
+    if (bits == 5) {
+        uint8_t *qh = out + 16;
+        qs = out + 48;
+        memset(qh, 0, 32);
+        for (int p = 0; p < 4; p++)
+            for (int h = 0; h < 2; h++)
+                for (int l = 0; l < 32; l++) qh[l] |= (uint8_t)((q[64 * p + 32 * h + l] >> 4) << (2 * p + h));
+    }
     for (int p = 0; p < 4; p++)
-        for (int l = 0; l < 32; l++) qs[32 * p + l] = (uint8_t)(q[64 * p + l] | (q[64 * p + 32 + l] << 4));
+        for (int l = 0; l < 32; l++) qs[32 * p + l] = (uint8_t)((q[64 * p + l] & 0x0F) | ((q[64 * p + 32 + l] & 0x0F) << 4));
 }
 
 /* Q6_K, GGUF layout [u8 ql[128]][u8 qh[64]][i8 scales[16]][f16 d] over 256 elements = 16 sub-blocks of 16, each
@@ -430,6 +451,7 @@ AXO_API int axo_quantize(int type, const float *x, size_t numel, uint8_t *out) {
         case AXO_Q5_0: quant_block_q5_0(x + start, len, o); break;
         case AXO_Q5_1: quant_block_q5_1(x + start, len, o); break;
         case AXO_Q4_K: quant_block_q4_k(x + start, len, o); break;
+        case AXO_Q5_K: quant_block_q5_k(x + start, len, o); break;
         case AXO_Q6_K: quant_block_q6_k(x + start, len, o); break;
         }
     }
@@ -493,11 +515,13 @@ static void dequant_block(int type, const uint8_t *b, float *y) {
         }
         break;
     }
-    case AXO_Q4_K: {
+    case AXO_Q4_K:
+    case AXO_Q5_K: { /* ggml's dequantize_row_q4_K / _q5_K: y = (d * sc) * q - dmin * m */
         float d = axo_f16_to_f32(get_u16(b));
         float dmin = axo_f16_to_f32(get_u16(b + 2));
         const uint8_t *sc = b + 4;
-        const uint8_t *qs = b + 16;
+        const uint8_t *qh = b + 16; /* Q5_K only */
+        const uint8_t *qs = type == AXO_Q5_K ? b + 48 : b + 16;
         for (int s = 0; s < 8; s++) {
             uint8_t l, m;
             if (s < 4) {
@@ -513,6 +537,7 @@ static void dequant_block(int type, const uint8_t *b, float *y) {
             for (int i = 0; i < 32; i++) {
                 uint8_t byte = qs[32 * p + i];
                 int q = (s & 1) ? (byte >> 4) : (byte & 0x0F);
+                if (type == AXO_Q5_K) q |= ((qh[i] >> s) & 1) << 4;
                 float a = sd * (float)q;
                 y[32 * s + i] = a - sm;
             }

@@ -11,7 +11,7 @@
 //! Differences from the reference crate, all forced by the device library:
 //!  * a `QuantizedTensor` holds one flat byte buffer (the blocks' `to_bytes` images in block order) instead of a
 //!    `Vec<QuantizedBlock>`;
-//!  * `QuantType` has `Q4_K` and `Q6_K` (GGUF superblocks) behind `F32`, and `Q5_0` / `Q5_1` have codecs of their own
+//!  * `QuantType` has `Q4_K`, `Q6_K` and `Q5_K` (GGUF superblocks) behind `F32`, and `Q5_0` / `Q5_1` have codecs of their own
 //!    (`quantize.rs:47-50` sends them to Q4_0);
 //!  * every function takes the device context first.
 use axonml_quant_hip_sys as sys;
@@ -25,25 +25,25 @@ use std::os::raw::c_void;
 #[allow(non_camel_case_types)]
 #[derive(Clone, Copy, Debug, PartialEq, Eq, Hash)]
 #[repr(i32)]
-pub enum QuantType { Q8_0 = 0, Q4_0 = 1, Q4_1 = 2, Q5_0 = 3, Q5_1 = 4, F16 = 5, F32 = 6, Q4_K = 7, Q6_K = 8 }
+pub enum QuantType { Q8_0 = 0, Q4_0 = 1, Q4_1 = 2, Q5_0 = 3, Q5_1 = 4, F16 = 5, F32 = 6, Q4_K = 7, Q6_K = 8, Q5_K = 9 }
 
 impl QuantType {
     /// types.rs:45-52
     pub fn block_size(self) -> usize {
-        match self { QuantType::F16 | QuantType::F32 => 1, QuantType::Q4_K | QuantType::Q6_K => 256, _ => 32 }
+        match self { QuantType::F16 | QuantType::F32 => 1, QuantType::Q4_K | QuantType::Q6_K | QuantType::Q5_K => 256, _ => 32 }
     }
     /// types.rs:55-66
     pub fn bytes_per_block(self) -> usize {
         match self {
             QuantType::Q8_0 => 34, QuantType::Q4_0 => 18, QuantType::Q4_1 => 20, QuantType::Q5_0 => 22,
-            QuantType::Q5_1 => 24, QuantType::F16 => 2, QuantType::F32 => 4, QuantType::Q4_K => 144, QuantType::Q6_K => 210,
+            QuantType::Q5_1 => 24, QuantType::F16 => 2, QuantType::F32 => 4, QuantType::Q4_K => 144, QuantType::Q6_K => 210, QuantType::Q5_K => 176,
         }
     }
     /// types.rs:69-78
     pub fn bits_per_value(self) -> usize {
         match self {
             QuantType::Q8_0 => 8, QuantType::Q4_0 | QuantType::Q4_1 | QuantType::Q4_K => 4,
-            QuantType::Q5_0 | QuantType::Q5_1 => 5, QuantType::Q6_K => 6, QuantType::F16 => 16, QuantType::F32 => 32,
+            QuantType::Q5_0 | QuantType::Q5_1 | QuantType::Q5_K => 5, QuantType::Q6_K => 6, QuantType::F16 => 16, QuantType::F32 => 32,
         }
     }
     /// types.rs:81-83
@@ -62,6 +62,7 @@ impl QuantType {
             "F32" | "FLOAT32" | "FLOAT" => QuantType::F32,
             "Q4_K" | "Q4K" => QuantType::Q4_K,
             "Q6_K" | "Q6K" => QuantType::Q6_K,
+            "Q5_K" | "Q5K" => QuantType::Q5_K,
             _ => return None,
         })
     }

@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 import oracle as o  # noqa: E402
 
-TYPES = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.F16, o.F32, o.Q4_K, o.Q6_K]
+TYPES = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.F16, o.F32, o.Q4_K, o.Q6_K, o.Q5_K]
 
 
 def kat_inputs(block):
@@ -41,7 +41,7 @@ def main():
     out["x"] = x
     for t in TYPES:
         name = o.TYPE_NAMES[t]
-        block = 256 if t in (o.Q4_K, o.Q6_K) else 32
+        block = 256 if t in (o.Q4_K, o.Q6_K, o.Q5_K) else 32
         kin = kat_inputs(block)
         out[f"{name}.kat_in"] = kin
         out[f"{name}.kat_packed"] = np.stack([o.quantize(t, r) for r in kin])

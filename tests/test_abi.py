@@ -34,7 +34,7 @@ def test_type_registry_matches_reference(lib):
     # types.rs:45-78
     table = {0: ("Q8_0", 32, 34, 8), 1: ("Q4_0", 32, 18, 4), 2: ("Q4_1", 32, 20, 4), 3: ("Q5_0", 32, 22, 5),
              4: ("Q5_1", 32, 24, 5), 5: ("F16", 1, 2, 16), 6: ("F32", 1, 4, 32), 7: ("Q4_K", 256, 144, 4),
-             8: ("Q6_K", 256, 210, 6)}
+             8: ("Q6_K", 256, 210, 6), 9: ("Q5_K", 256, 176, 5)}
     for t, (name, bs, bb, bits) in table.items():
         assert lib.axq_type_name(t).decode() == name
         assert lib.axq_type_block_size(t) == bs
@@ -47,7 +47,7 @@ def test_type_registry_matches_reference(lib):
 def test_from_str_aliases(lib):
     # types.rs:94-105 and its test :356-363
     for s, t in [("Q8_0", 0), ("INT8", 0), ("q8", 0), ("Q4", 1), ("int4", 1), ("Q4_1", 2), ("Q5", 3), ("Q5_1", 4),
-                 ("F16", 5), ("half", 5), ("FLOAT16", 5), ("F32", 6), ("float", 6), ("Q4_K", 7), ("Q6_K", 8), ("q6k", 8)]:
+                 ("F16", 5), ("half", 5), ("FLOAT16", 5), ("F32", 6), ("float", 6), ("Q4_K", 7), ("Q6_K", 8), ("q6k", 8), ("Q5_K", 9), ("Q5K", 9)]:
         assert lib.axq_type_from_str(s.encode()) == t
     assert lib.axq_type_from_str(b"invalid") == -1
 

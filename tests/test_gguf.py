@@ -79,7 +79,7 @@ def test_ggml_formula_against_numpy():
     assert np.array_equal(o.ggml_dequantize(o.Q4_1, g.reshape(-1)).reshape(40, 32), want)
 
 
-@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K, o.F16, o.F32])
+@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q5_0, o.Q5_1, o.Q4_K, o.Q5_K, o.Q6_K, o.F16, o.F32])
 def test_other_types_are_byte_identical(qtype):
     rng = np.random.default_rng(qtype)
     n = 512
@@ -158,10 +158,10 @@ def test_reader_errors(tmp_path):
         gguf.GGUFReader(_hand_made_file(tmp_path, truncate=8)[0])
     with pytest.raises(gguf.GGUFError, match="power of two"):
         gguf.GGUFReader(_hand_made_file(tmp_path, alignment=24)[0])
-    # a ggml type without a kernel here (Q5_K = 13) parses, and is refused when its data is asked for
-    with gguf.GGUFReader(_hand_made_file(tmp_path, tensor_type=13)[0]) as r:
+    # a ggml type without a kernel here (Q3_K = 11) parses, and is refused when its data is asked for
+    with gguf.GGUFReader(_hand_made_file(tmp_path, tensor_type=11)[0]) as r:
         assert r.info("blk.0.w").quant_type is None
-        with pytest.raises(gguf.GGUFError, match="Q5_K"):
+        with pytest.raises(gguf.GGUFError, match="Q3_K"):
             r.tensor_bytes("blk.0.w")
     assert issubclass(gguf.GGUFError, q.QuantError)
 
@@ -213,7 +213,7 @@ def test_write_then_read_round_trip_and_matmul_on_ggml_values(ctx, tmp_path):
     rng = np.random.default_rng(12)
     n, k = 48, 512
     tensors, packed = {}, {}
-    for qtype in (o.Q4_0, o.Q4_1, o.Q5_1, o.Q8_0, o.Q4_K, o.Q6_K):
+    for qtype in (o.Q4_0, o.Q4_1, o.Q5_1, o.Q8_0, o.Q4_K, o.Q5_K, o.Q6_K):
         packed[qtype] = o.quantize(qtype, (rng.standard_normal((n, k)) * 0.05).astype(np.float32))
         tensors[f"w.{o.TYPE_NAMES[qtype]}"] = q.QuantizedTensor([n, k], qtype, packed[qtype])
     tensors["norm"] = rng.standard_normal(k).astype(np.float32)
@@ -261,7 +261,7 @@ def _q4_k_m_like(c, w, seed, ffn_too=False):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q6_K, "Q4_K_M", "Q4_K_M+up"])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q5_K, o.Q6_K, "Q4_K_M", "Q4_K_M+up"])
 def test_llama_loaded_from_gguf_decodes_like_the_oracle(ctx, tmp_path, qtype):
     from tests.decode_common import LIN_SHAPES, load_oracle, random_weights, tiny_config
     from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err

@@ -8,13 +8,13 @@ import pytest
 import oracle as o
 
 GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "blocks.npz"), allow_pickle=False)
-TYPES = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.F16, o.F32, o.Q4_K, o.Q6_K]
+TYPES = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.F16, o.F32, o.Q4_K, o.Q6_K, o.Q5_K]
 
 
 @pytest.mark.parametrize("t", TYPES)
 def test_oracle_reproduces_committed_vectors(t):
     name = o.TYPE_NAMES[t]
-    block = 256 if t in (o.Q4_K, o.Q6_K) else 32
+    block = 256 if t in (o.Q4_K, o.Q6_K, o.Q5_K) else 32
     for row, packed, deq in zip(GOLD[f"{name}.kat_in"], GOLD[f"{name}.kat_packed"], GOLD[f"{name}.kat_deq"]):
         assert np.array_equal(o.quantize(t, row), packed)
         assert np.array_equal(o.dequantize(t, packed, block), deq)

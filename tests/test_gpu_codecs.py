@@ -10,9 +10,9 @@ from tests.util import gen_weight
 
 pytestmark = pytest.mark.gpu
 
-ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K, o.F16, o.F32]
-BLOCK = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K]
-SUPER = (o.Q4_K, o.Q6_K)  # 256-element superblocks
+ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q5_K, o.Q6_K, o.F16, o.F32]
+BLOCK = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q5_K, o.Q6_K]
+SUPER = (o.Q4_K, o.Q5_K, o.Q6_K)  # 256-element superblocks
 
 
 def _inputs(rng, n):
@@ -70,7 +70,7 @@ def test_dequantize_arbitrary_bytes_bit_exact(ctx, qtype):
     bb = o.lib().axo_bytes_per_block(qtype)
     nblk = 512
     raw = rng.integers(0, 256, size=(nblk, bb), dtype=np.uint8)
-    nscale = {o.Q8_0: 1, o.Q4_0: 1, o.Q5_0: 1, o.Q4_1: 2, o.Q5_1: 2, o.Q4_K: 2, o.Q6_K: 1}[qtype]
+    nscale = {o.Q8_0: 1, o.Q4_0: 1, o.Q5_0: 1, o.Q4_1: 2, o.Q5_1: 2, o.Q4_K: 2, o.Q5_K: 2, o.Q6_K: 1}[qtype]
     scales = (rng.standard_normal((nblk, nscale)) * 0.1).astype(np.float16)
     at = 208 if qtype == o.Q6_K else 0  # Q6_K keeps its f16 d behind the codes and the int8 scales (all 256 values occur)
     raw[:, at:at + 2 * nscale] = scales.view(np.uint8)

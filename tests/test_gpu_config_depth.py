@@ -36,7 +36,7 @@ def device_normal(ctx, n, std, outlier_p, seed):
 
 
 @pytest.mark.parametrize("qtype,n,k,outliers", [(o.Q8_0, 4096, 4096, 0.0), (o.Q4_0, 11008, 4096, 0.0), (o.Q4_1, 11008, 4096, 0.0),
-                                                (o.Q4_K, 14336, 4096, 0.01), (o.Q5_1, 14336, 4096, 0.0), (o.Q6_K, 4096, 14336, 0.01)])
+                                                (o.Q4_K, 14336, 4096, 0.01), (o.Q5_1, 14336, 4096, 0.0), (o.Q6_K, 4096, 14336, 0.01), (o.Q5_K, 4096, 4096, 0.01)])
 def test_device_quantiser_is_bit_exact_at_the_configs_own_sizes(ctx, qtype, n, k, outliers):
     w = device_normal(ctx, n * k, 0.02, outliers, 900 + qtype)
     assert np.isfinite(w).all() and 0.015 < w.std() < (0.06 if outliers else 0.025)

@@ -13,7 +13,7 @@ from tests.util import DECODE_FLOOR, DECODE_RTOL, max_rel_err
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q4_0, o.Q8_0, o.Q5_1, o.Q6_K])
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q4_0, o.Q8_0, o.Q5_1, o.Q6_K, o.Q5_K])
 def test_step_by_step_logits_and_tokens(ctx, qtype):
     c = tiny_config()
     w = random_weights(c, 10 + qtype, qtype=qtype)

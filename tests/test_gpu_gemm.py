@@ -12,7 +12,7 @@ from tests.util import MATMUL_RTOL, STRICT_FLOOR, gen_weight, max_rel_err
 
 pytestmark = pytest.mark.gpu
 
-ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K, o.F16, o.F32]
+ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q5_K, o.Q6_K, o.F16, o.F32]
 
 
 def _check(ctx, qtype, m, n, k, seed, xscale=1.0):
@@ -42,7 +42,7 @@ def test_config_prefill_k4096(ctx, qtype, m):
     _check(ctx, qtype, m, 512, 4096, seed=m)
 
 
-@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K])
+@pytest.mark.parametrize("qtype", [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q5_K, o.Q6_K])
 @pytest.mark.parametrize("m,n,k", [(250, 300, 1024), (640, 136, 512), (1100, 520, 1024)])
 def test_many_rows(ctx, qtype, m, n, k):
     """Several row tiles per column tile, ragged in both directions."""

@@ -13,7 +13,7 @@ from tests.util import MATMUL_RTOL, STRICT_FLOOR, assert_close_ref_style, gen_we
 
 pytestmark = pytest.mark.gpu
 
-ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K, o.F16, o.F32]
+ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q5_K, o.Q6_K, o.F16, o.F32]
 
 
 def _check(ctx, qtype, n, k, batch, seed, outlier_p=0.0, bias=False):
@@ -38,7 +38,7 @@ def _check(ctx, qtype, n, k, batch, seed, outlier_p=0.0, bias=False):
 @pytest.mark.parametrize("n,k", [(1, 256), (5, 256), (64, 512), (33, 2048), (17, 4096), (130, 4096 + 512),
                                   (9, 11008), (12, 14336), (4, 32768 + 2048)])
 def test_gemv_small_shapes(ctx, qtype, n, k):
-    if qtype in (o.Q4_K, o.Q6_K) and k % 256:
+    if qtype in (o.Q4_K, o.Q5_K, o.Q6_K) and k % 256:
         pytest.skip("k must be a multiple of 256 for the superblock types")
     _check(ctx, qtype, n, k, 1, seed=n * 7 + k)
 
@@ -178,7 +178,7 @@ def test_small_batch_reads_weights_once(ctx, qtype, batch, n, k):
 
 
 # ---- many vectors: f32 rows through the matrix-pipe GEMM as two f16 rows each
-@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q6_K, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.F16, o.F32])
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.F16, o.F32])
 @pytest.mark.parametrize("batch,n,k", [(40, 96, 512), (64, 100, 1024), (130, 33, 4096), (9, 64, 2048), (300, 257, 768), (384, 132, 512),
                                        (777, 64, 1024)])
 def test_many_vectors_go_through_the_gemm_at_f32_accuracy(ctx, qtype, batch, n, k):

@@ -60,7 +60,7 @@ def test_nan_keeps_being_nan():
 def test_registry_sizes():
     L = o.lib()
     expect = {o.Q8_0: (32, 34), o.Q4_0: (32, 18), o.Q4_1: (32, 20), o.Q5_0: (32, 22), o.Q5_1: (32, 24),
-              o.F16: (1, 2), o.F32: (1, 4), o.Q4_K: (256, 144), o.Q6_K: (256, 210)}
+              o.F16: (1, 2), o.F32: (1, 4), o.Q4_K: (256, 144), o.Q6_K: (256, 210), o.Q5_K: (256, 176)}
     for t, (bs, bb) in expect.items():
         assert L.axo_block_size(t) == bs and L.axo_bytes_per_block(t) == bb
     # quantize.rs:294-313: 8 elements -> 1 block, 64 -> 2 blocks
@@ -625,3 +625,119 @@ def test_q6_k_tail_superblock_is_zero_padded():
     full = o.quantize(o.Q6_K, np.concatenate([x, np.zeros(212, np.float32)]))
     assert np.array_equal(p, full)
     assert o.dequantize(o.Q6_K, p, 300).shape == (300,)
+
+
+# --------------------------------------------------------------------------- Q5_K (GGUF block; the reference has no such type)
+def _q5k_dequant_numpy(packed, numel):
+    """ggml's dequantize_row_q5_K transcribed independently in numpy from its published loop: four chunks of 64, masks
+    u1 = 1 << 2j and u2 = 2 << 2j into qh[l], low and high nibbles of ql[32j + l]."""
+    out = []
+    for b in packed.reshape(-1, 176):
+        d, dmin = b[0:4].view(np.float16).astype(np.float32)
+        sc, qh, ql = b[4:16].astype(np.int32), b[16:48].astype(np.int32), b[48:176].astype(np.int32)
+        y = np.zeros(256, np.float32)
+        for j in range(4):
+            ls, lm = [], []
+            for s in (2 * j, 2 * j + 1):
+                if s < 4:
+                    ls.append(sc[s] & 63), lm.append(sc[s + 4] & 63)
+                else:
+                    ls.append((sc[s + 4] & 0xF) | ((sc[s - 4] >> 6) << 4)), lm.append((sc[s + 4] >> 4) | ((sc[s] >> 6) << 4))
+            d1, m1 = np.float32(d * np.float32(ls[0])), np.float32(dmin * np.float32(lm[0]))
+            d2, m2 = np.float32(d * np.float32(ls[1])), np.float32(dmin * np.float32(lm[1]))
+            u1, u2 = 1 << (2 * j), 2 << (2 * j)
+            for l in range(32):
+                y[64 * j + l] = d1 * np.float32((ql[32 * j + l] & 0xF) + (16 if qh[l] & u1 else 0)) - m1
+                y[64 * j + 32 + l] = d2 * np.float32((ql[32 * j + l] >> 4) + (16 if qh[l] & u2 else 0)) - m2
+        out.append(y)
+    return np.concatenate(out)[:numel]
+
+
+def test_q5_k_layout_one_code_at_a_time():
+    # d = 1, dmin = 0, all eight 6-bit scales 1 (bytes typed from get_scale_min_k4's packing: sc[0..3] = 1, sc[8..11] = 1)
+    base = np.zeros(176, np.uint8)
+    base[0:2] = [0x00, 0x3C]
+    base[4:8] = 1
+    base[12:16] = 1
+    assert not o.dequantize(o.Q5_K, base, 256).any()
+    for e, u in [(0, 31), (1, 16), (31, 15), (32, 1), (63, 30), (64, 17), (100, 31), (127, 8), (128, 24), (191, 31), (192, 16), (255, 31)]:
+        p, h, l = e >> 6, (e >> 5) & 1, e & 31
+        img = base.copy()
+        img[48 + 32 * p + l] = (u & 15) << (4 * h)
+        img[16 + l] = (u >> 4) << (2 * p + h)
+        want = np.zeros(256, np.float32)
+        want[e] = u
+        assert np.array_equal(o.dequantize(o.Q5_K, img, 256), want), (e, u)
+
+
+def test_q5_k_dequant_matches_ggml_loop_on_arbitrary_bytes():
+    rng = np.random.default_rng(51)
+    raw = rng.integers(0, 256, size=(64, 176), dtype=np.uint8)
+    raw[:, 0:4] = (rng.standard_normal((64, 2)) * 0.1).astype(np.float16).view(np.uint8)
+    assert np.array_equal(o.dequantize(o.Q5_K, raw.reshape(-1), 64 * 256), _q5k_dequant_numpy(raw.reshape(-1), 64 * 256))
+
+
+def test_q5_k_known_superblock_by_hand():
+    """Q4_K's hand-worked superblock with 31 steps: sub-block s spans [-lm_s / 32, ls_s / 64 * 31 - lm_s / 32] with
+    hand-picked 6-bit ls and lm (largest 63), so d = f16(63/64 / 63) = 2^-6, dmin = 2^-5, and every x is a grid point."""
+    ls = [63, 1, 2, 32, 33, 47, 16, 0]  # sub-block 7 is constant: scale 0, codes 0
+    lm = [63, 0, 5, 31, 32, 48, 17, 9]  # sub-block 1 has no negative value: min 0
+    q = [[(7 * i + 3 * s) % 32 for i in range(32)] for s in range(8)]  # every code 0..31 once per sub-block
+    q[7] = [0] * 32
+    x = np.zeros(256, np.float32)
+    for s in range(8):
+        for i in range(32):
+            x[32 * s + i] = ls[s] / 64 * q[s][i] - lm[s] / 32
+    scales = [191, 129, 66, 32, 191, 192, 69, 31, 1, 15, 16, 144]  # as in the Q4_K block: the same ls, lm
+    got = o.quantize(o.Q5_K, x)
+    assert got[:4].tolist() == [0x00, 0x24, 0x00, 0x28] and got[4:16].tolist() == scales
+    for s in range(8):
+        for i in range(32):
+            byte = int(got[48 + 32 * (s >> 1) + i])
+            u = ((byte >> 4) if s & 1 else (byte & 15)) | (((int(got[16 + i]) >> s) & 1) << 4)
+            assert u == q[s][i], (s, i)
+    assert np.array_equal(o.dequantize(o.Q5_K, got, 256), x)
+
+
+def test_q5_k_zero_and_tail_superblocks():
+    p = o.quantize(o.Q5_K, np.zeros(256, np.float32))
+    # as Q4_K's zero superblock: every field 0, dmin = -0.0 (the negated minimum of a block of zeros)
+    assert p.tolist() == [0, 0, 0, 0x80] + [0] * 172 and not o.dequantize(o.Q5_K, p, 256).any()
+    x = (np.arange(300, dtype=np.float32) - 150) / 64
+    p = o.quantize(o.Q5_K, x)
+    assert p.size == 2 * 176 and np.array_equal(p, o.quantize(o.Q5_K, np.concatenate([x, np.zeros(212, np.float32)])))
+    # half-way quotients round away from zero: one sub-block 0..31 (scale 1 -> d = f16(1/63), ls = 63, sd = 63 d)
+    x = np.zeros(256, np.float32)
+    sd = np.float32(np.float32(np.float16(np.float32(1.0) / np.float32(63.0))) * np.float32(63.0))
+    x[0] = 31.0
+    for i, v in enumerate([0.5, 1.5, 2.5, 29.5, 30.49]):
+        x[1 + i] = np.float32(v) * sd
+    y = o.dequantize(o.Q5_K, o.quantize(o.Q5_K, x), 256)
+    assert np.rint(y[1:6] / sd).astype(int).tolist() == [1, 2, 3, 30, 30]
+
+
+def test_q5_k_roundtrip_error_is_what_the_rule_implies():
+    rng = np.random.default_rng(53)
+    n = 256 * 64
+    x = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    x[rng.random(n) < 0.01] = 0.5
+    packed = o.quantize(o.Q5_K, x)
+    y = o.dequantize(o.Q5_K, packed, n)
+    assert np.array_equal(y, _q5k_dequant_numpy(packed, n))
+    for b, p in enumerate(packed.reshape(-1, 176)):
+        d, dmin, ls, lm = _q4k_fields(p[:16])
+        xs = x[256 * b:256 * b + 256].astype(np.float64).reshape(8, 32)
+        ys = y[256 * b:256 * b + 256].astype(np.float64).reshape(8, 32)
+        mins = np.maximum(0.0, -xs.min(1))
+        scales = (xs.max(1) + mins) / 31
+        # f16 rounding of d and dmin; with 31 steps d falls into f16's subnormal range (spacing 2^-24) for weights of this size
+        d_err, m_err = max(scales.max() / 63 * 2 ** -11, 2.0 ** -25), max(mins.max() / 63 * 2 ** -11, 2.0 ** -25)
+        assert abs(d - scales.max() / 63) <= d_err and abs(dmin - mins.max() / 63) <= m_err
+        for s in range(8):
+            sd, sm = d * ls[s], dmin * lm[s]
+            assert abs(sd - scales[s]) <= d * 0.5 + ls[s] * d_err + scales[s] * 2 ** -20, (b, s)
+            assert abs(sm - mins[s]) <= dmin * 0.5 + lm[s] * m_err + mins[s] * 2 ** -20, (b, s)
+            below = max(0.0, mins[s] - sm)
+            above = max(0.0, xs[s].max() + sm - 31 * sd)
+            bound = max(sd * 0.5, below, above) + 1e-6 * np.abs(xs[s]).max()
+            assert np.abs(xs[s] - ys[s]).max() <= bound, (b, s)

@@ -10,7 +10,7 @@ import pytest
 import oracle as o
 from tests.util import max_rel_err
 
-ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q6_K, o.F16, o.F32]
+ALL = [o.Q8_0, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q4_K, o.Q5_K, o.Q6_K, o.F16, o.F32]
 
 
 def test_reference_2x2_known_answer():
