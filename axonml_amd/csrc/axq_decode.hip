@@ -1049,6 +1049,8 @@ int enqueue_rows(axq_model *m, const Rows &r) {
                                             chain ? next : nullptr, chain ? next_aux : nullptr);
         }
         packed_for = nullptr;
+        if (r.mode == ROWS_GEMM && xmode == AXQ_X_SWIGLU && axq_dev_gemm_f32_takes_swiglu(w)) // the GEMM's row pass applies SwiGLU itself
+            return axq_dev_gemm_f32_ex(ctx, w, x, true, nb, nullptr, c.rms_norm_eps, nullptr, resid, y);
         if (xmode == AXQ_X_SWIGLU) {
             swiglu_kernel<<<dim3((I / 4 + 255) / 256, nb), 256, 0, st>>>(x, I, m->pb_act);
             x = m->pb_act;

@@ -1337,6 +1337,9 @@ int launch_gemm(axq_ctx *ctx, GemmArgs a, int splits) {
 // f32 rows, optionally RMS-normalised on the way ((x * inv_rms) * norm_w, RMSNorm::forward, llm/src/llama.rs:158-187),
 // -> two f16 rows each under one power-of-two scale: row 2t holds the leading 11 bits of every element, row 2t + 1
 // what those leave, so that their GEMM results add up to the f32 product (the GEMM's epilogue adds them: pair mode).
+// SWIGLU: x holds rows of 2 k gate/up values, four gate values followed by the four up values of the same indices (the row
+// order of the fused gate/up weight), and the row that is split is silu(gate) * up (k a multiple of 4, at most 16384).
+template <bool SWIGLU>
 __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, const float *norm_w, float eps, int m, int k,
                                                               _Float16 *xh, float *rowscale, XSums xs) {
     // the row stays in registers between the passes: 16 bytes per thread and step, up to 16 steps (k <= 16384);
@@ -1344,14 +1347,25 @@ __global__ void __launch_bounds__(256) gemm_prep_x_f32_kernel(const float *x, co
     constexpr int STEPS = 16;
     __shared__ float red[4];
     const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const float *xr = x + (size_t)row * k;
-    const bool in_regs = (k & 3) == 0 && k <= STEPS * 256 * 4;
+    const float *xr = x + (size_t)row * (SWIGLU ? 2 * k : k);
+    const bool in_regs = SWIGLU || ((k & 3) == 0 && k <= STEPS * 256 * 4);
     float4 v[STEPS];
     if (in_regs) {
 #pragma unroll
         for (int c = 0; c < STEPS; c++) {
             const int i4 = c * 256 + threadIdx.x;
-            v[c] = i4 * 4 < k ? reinterpret_cast<const float4 *>(xr)[i4] : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (SWIGLU) {
+                v[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (i4 * 4 < k) {
+                    const float4 g = reinterpret_cast<const float4 *>(xr)[2 * i4], u = reinterpret_cast<const float4 *>(xr)[2 * i4 + 1];
+                    v[c].x = (g.x * (1.0f / (1.0f + expf(-g.x)))) * u.x;
+                    v[c].y = (g.y * (1.0f / (1.0f + expf(-g.y)))) * u.y;
+                    v[c].z = (g.z * (1.0f / (1.0f + expf(-g.z)))) * u.z;
+                    v[c].w = (g.w * (1.0f / (1.0f + expf(-g.w)))) * u.w;
+                }
+            } else {
+                v[c] = i4 * 4 < k ? reinterpret_cast<const float4 *>(xr)[i4] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
         }
     }
     float inv = 1.0f;
@@ -1653,11 +1667,23 @@ bool axq_dev_gemm_f32_covers(const axq_weight *w, int m) {
 // when that is given.
 int axq_dev_gemm_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int m, const float *norm_w, float eps, const float *bias,
                      const float *resid, float *y) {
+    return axq_dev_gemm_f32_ex(ctx, w, x, false, m, norm_w, eps, bias, resid, y);
+}
+
+// The same with f = SwiGLU when `swiglu`: x holds m rows of 2 k interleaved gate/up values (see the pre-pass).
+bool axq_dev_gemm_f32_takes_swiglu(const axq_weight *w) { return w->k % 4 == 0 && w->k <= 16 * 256 * 4; }
+
+int axq_dev_gemm_f32_ex(axq_ctx *ctx, const axq_weight *w, const float *x, bool swiglu, int m, const float *norm_w, float eps,
+                        const float *bias, const float *resid, float *y) {
     GemmPlan p;
     int rc;
+    if (swiglu && (norm_w || !axq_dev_gemm_f32_takes_swiglu(w)))
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_dev_gemm_f32_ex: SwiGLU rows need k %% 4 == 0, k <= 16384 and no norm");
     if ((rc = plan_gemm(ctx, w, 2 * m, true, 0, &p))) return rc;
     uint8_t *base = reinterpret_cast<uint8_t *>(ctx->gemm_scratch);
-    gemm_prep_x_f32_kernel<<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, (int)w->k, reinterpret_cast<_Float16 *>(base),
-                                                       reinterpret_cast<float *>(base + p.xh_bytes), plan_sums(ctx, w, p));
+    _Float16 *xh = reinterpret_cast<_Float16 *>(base);
+    float *rowscale = reinterpret_cast<float *>(base + p.xh_bytes);
+    if (swiglu) gemm_prep_x_f32_kernel<true><<<m, 256, 0, ctx->stream>>>(x, nullptr, eps, m, (int)w->k, xh, rowscale, plan_sums(ctx, w, p));
+    else gemm_prep_x_f32_kernel<false><<<m, 256, 0, ctx->stream>>>(x, norm_w, eps, m, (int)w->k, xh, rowscale, plan_sums(ctx, w, p));
     return run_gemm(ctx, w, 2 * m, p, y, true, bias, resid);
 }

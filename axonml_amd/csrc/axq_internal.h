@@ -164,5 +164,8 @@ int axq_dev_attn_rows_mfma(axq_ctx *ctx, const float *qkv, int qkv_rows, const f
 int axq_dev_gemm_bf16(axq_ctx *ctx, const axq_weight *w, const uint16_t *x_dev, int m, float *y_dev);
 #define AXQ_GEMM_F32_MAX_ROWS 2048 // rows per call of the f32-activation GEMM (its scratch grows with them)
 bool axq_dev_gemm_f32_covers(const axq_weight *w, int m);
+bool axq_dev_gemm_f32_takes_swiglu(const axq_weight *w);
+int axq_dev_gemm_f32_ex(axq_ctx *ctx, const axq_weight *w, const float *x_dev, bool swiglu, int m, const float *norm_w, float eps,
+                        const float *bias, const float *resid, float *y_dev);
 int axq_dev_gemm_f32(axq_ctx *ctx, const axq_weight *w, const float *x_dev, int m, const float *norm_w, float eps,
                      const float *bias, const float *resid, float *y_dev);
