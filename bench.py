@@ -2,6 +2,7 @@
 """Headline benchmark of the block-quantized matmul path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
+    python bench.py --read-sweep      (a table instead: a read-only kernel over the same weight in every launch shape)
 
 A "step" is one Q4_K GEMV (decode-path quantized matmul), weight 14336 x 4096 drawn ~N(0, 0.02) with
 1 % of entries at +-0.5, activation f32[4096] ~N(0, 1), batch 1: the bandwidth headline case.  Launch i
@@ -9,7 +10,7 @@ reads copy i mod R of the weight from a ring of R copies (> 700 MB, beyond the 2
 so that every step streams its 33 MB from HBM; inputs are resident in HBM before the timed region.
 
 Prints ONE JSON line.  `value` is whole-job throughput in algorithmic GB/s (packed weight bytes + x + y
-per step, divided by the mean step time between two HIP events on the kernel's stream).  `roofline`
+per step, divided by the median step time of 25 event-bracketed repeats on the kernel's stream).  `roofline`
 prices the dominant kernel against the 8 TB/s HBM peak; `cpu_baseline` times the CPU oracle (a C
 restatement of the reference composition dequantize -> transpose -> one-thread sgemm) on this box's host
 cores on the same workload.  `extra` carries the other configurations (other block types, the 7B-shape
