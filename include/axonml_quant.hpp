@@ -33,7 +33,7 @@ constexpr size_t MAX_BLOCK_SIZE = 256;    // lib.rs:49
 
 // ---- QuantType (types.rs:17-41), discriminants equal to axq_type -----------------------------------
 enum class QuantType : int { Q8_0 = AXQ_Q8_0, Q4_0 = AXQ_Q4_0, Q4_1 = AXQ_Q4_1, Q5_0 = AXQ_Q5_0, Q5_1 = AXQ_Q5_1,
-                             F16 = AXQ_F16, F32 = AXQ_F32, Q4_K = AXQ_Q4_K };
+                             F16 = AXQ_F16, F32 = AXQ_F32, Q4_K = AXQ_Q4_K, Q6_K = AXQ_Q6_K, Q5_K = AXQ_Q5_K };
 inline size_t block_size(QuantType t) { return axq_type_block_size((int)t); }           // types.rs:45-54
 inline size_t bytes_per_block(QuantType t) { return axq_type_bytes_per_block((int)t); } // :57-67
 inline size_t bits_per_value(QuantType t) { return axq_type_bits_per_value((int)t); }   // :70-78

@@ -33,6 +33,8 @@ int main() {
     CHECK(block_size(QuantType::Q8_0) == 32 && bytes_per_block(QuantType::Q8_0) == 34);
     CHECK(bytes_per_block(QuantType::Q4_0) == 18 && bytes_per_block(QuantType::Q4_1) == 20);
     CHECK(block_size(QuantType::Q4_K) == 256 && bytes_per_block(QuantType::Q4_K) == 144);
+    CHECK(bytes_per_block(QuantType::Q6_K) == 210 && bytes_per_block(QuantType::Q5_K) == 176 && bits_per_value(QuantType::Q6_K) == 6);
+    CHECK(quant_type_from_str("q6_k") == QuantType::Q6_K && to_string(QuantType::Q5_K) == "Q5_K");
     CHECK(quant_type_from_str("int8") == QuantType::Q8_0 && quant_type_from_str("Q4_0") == QuantType::Q4_0);
     CHECK(throws(QuantError::Kind::InvalidQuantType, [] { quant_type_from_str("q3_k"); }));
     CHECK(to_string(QuantType::Q4_1) == "Q4_1");
