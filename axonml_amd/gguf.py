@@ -36,6 +36,9 @@ GGML_TYPE_NAMES = {0: "F32", 1: "F16", 2: "Q4_0", 3: "Q4_1", 6: "Q5_0", 7: "Q5_1
                    11: "Q3_K", 12: "Q4_K", 13: "Q5_K", 14: "Q6_K", 15: "Q8_K", 30: "BF16"}
 
 
+GGML_BF16 = 30
+
+
 class GGUFError(QuantError):
     pass
 
@@ -59,6 +62,8 @@ class GGUFTensorInfo:
             if inner % bs:
                 raise GGUFError(f"tensor {name}: innermost dimension {inner} is not a multiple of the {self.quant_type} block size {bs}")
             self.nbytes = self.numel // bs * self.quant_type.bytes_per_block()
+        elif self.ggml_type == GGML_BF16:  # no block type of its own here: widened to f32 (exactly) when it is read
+            self.nbytes = self.numel * 2
 
     def __repr__(self):
         return f"GGUFTensorInfo({self.name!r}, shape={self.shape}, ggml_type={GGML_TYPE_NAMES.get(self.ggml_type, self.ggml_type)})"
@@ -171,9 +176,9 @@ class GGUFReader:
     def tensor_bytes(self, name):
         """The tensor's ggml block images as a uint8 view of the mapped file."""
         t = self.info(name)
-        if t.quant_type is None:
+        if t.quant_type is None and t.ggml_type != GGML_BF16:
             raise GGUFError(f"tensor {name}: ggml type {GGML_TYPE_NAMES.get(t.ggml_type, t.ggml_type)} is not supported "
-                            f"(supported: F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K)")
+                            f"(supported: F32, F16, BF16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K)")
         return np.frombuffer(self._mm, dtype=np.uint8, count=t.nbytes, offset=self.data_start + t.offset)
 
     def close(self):
@@ -211,7 +216,14 @@ def load_quantized_tensor(reader, name, ctx=None):
     """GGUF tensor -> QuantizedTensor in the reference's block order (shape row-major)."""
     t = reader.info(name)
     raw = reader.tensor_bytes(name)
+    if t.ggml_type == GGML_BF16:  # as f32, which holds every bf16 value
+        return QuantizedTensor(list(t.shape), QuantType.F32, _bf16_to_f32(raw).view(np.uint8).reshape(-1))
     return QuantizedTensor(list(t.shape), t.quant_type, convert_blocks(t.quant_type, raw, False, ctx))
+
+
+def _bf16_to_f32(raw):
+    """bf16 bit patterns (little-endian bytes) -> float32: the pattern is the upper half of the f32 word."""
+    return (raw.view("<u2").astype(np.uint32) << 16).view(np.float32)
 
 
 def load_f32(reader, name, ctx=None):
@@ -224,6 +236,8 @@ def load_f32(reader, name, ctx=None):
         return raw.view("<f4").reshape(t.shape).copy()
     if t.quant_type == QuantType.F16:
         return raw.view("<f2").astype(np.float32).reshape(t.shape)
+    if t.ggml_type == GGML_BF16:
+        return _bf16_to_f32(raw).reshape(t.shape)
     return np.asarray(dequantize_tensor(load_quantized_tensor(reader, name, ctx), ctx)).reshape(t.shape)
 
 
@@ -259,7 +273,7 @@ def _enc_value(v):
 
 def write_gguf(path, metadata, tensors, ctx=None, alignment=DEFAULT_ALIGNMENT):
     """Writes a GGUF v3 file.  `tensors`: name -> QuantizedTensor (reference block order; converted to ggml
-    order on the device) or a float32 / float16 numpy array."""
+    order on the device), a float32 / float16 numpy array, or ("BF16", uint16 array of bf16 bit patterns)."""
     lib = _lib.load_library()
     metadata = dict(metadata)
     if alignment != DEFAULT_ALIGNMENT:
@@ -270,6 +284,9 @@ def write_gguf(path, metadata, tensors, ctx=None, alignment=DEFAULT_ALIGNMENT):
             ggml_type = lib.axq_type_to_ggml(int(t.quant_type))
             data = convert_blocks(t.quant_type, t.data, True, ctx)
             shape = t.shape
+        elif isinstance(t, tuple) and len(t) == 2 and t[0] == "BF16":
+            a = np.ascontiguousarray(t[1], dtype=np.uint16)
+            ggml_type, data, shape = GGML_BF16, a.view(np.uint8).reshape(-1), a.shape
         else:
             a = np.ascontiguousarray(t)
             if a.dtype not in (np.float32, np.float16):

@@ -122,6 +122,23 @@ def _hand_made_file(tmp_path, alignment=None, version=3, tensor_type=2, bad_offs
     return str(p), t0, t1
 
 
+def test_bf16_tensors_widen_exactly(tmp_path):
+    # ggml type 30: the bit pattern is the upper half of the f32 word (1.0 = 0x3F80, -2.5 = 0xC020, the largest finite
+    # value 0x7F7F, a subnormal 0x0001); such a tensor reads as f32, and as a linear it is carried as an F32 weight
+    bits = np.array([[0x3F80, 0xC020, 0x7F7F, 0x0001], [0x0000, 0x8000, 0x3DCD, 0x4049]], np.uint16)
+    path = str(tmp_path / "bf16.gguf")
+    gguf.write_gguf(path, {"general.architecture": "llama"}, {"w": ("BF16", bits)})
+    want = (bits.astype(np.uint32) << 16).view(np.float32)
+    assert want[0, 0] == 1.0 and want[0, 1] == -2.5
+    with gguf.GGUFReader(path) as r:
+        assert r.info("w").ggml_type == 30 and r.info("w").shape == (2, 4) and r.info("w").nbytes == 16
+        got = gguf.load_f32(r, "w")
+        assert got.dtype == np.float32 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        qt = gguf.load_quantized_tensor(r, "w")
+        assert qt.quant_type == q.QuantType.F32 and qt.shape == [2, 4]
+        assert np.array_equal(qt.data.view(np.float32).view(np.uint32), want.reshape(-1).view(np.uint32))
+
+
 @pytest.mark.parametrize("alignment", [None, 64])
 def test_reader_parses_a_hand_assembled_file(tmp_path, alignment):
     path, t0, t1 = _hand_made_file(tmp_path, alignment)
