@@ -399,6 +399,33 @@ def load_llama(path, ctx=None, max_position_embeddings=None, permuted_qk=True):
     return model
 
 
+def tokenizer_from_metadata(md):
+    """The file's vocabulary as the reference's tokenizer (`HFTokenizer`, tokenizer.rs:24-470): ids from
+    `tokenizer.ggml.tokens`, merges from `tokenizer.ggml.merges` ("left right" strings, in order), special tokens from the
+    `tokenizer.ggml.*_token_id` keys.  The algorithm is the reference's simple BPE, not llama.cpp's: a file whose
+    `tokenizer.ggml.model` is "llama" (SentencePiece scores, no merge list) encodes to single characters or bytes."""
+    from .tokenizer import HFTokenizer, SpecialTokens
+
+    tokens = md.get("tokenizer.ggml.tokens")
+    if not isinstance(tokens, (list, tuple)) or not all(isinstance(t, str) for t in tokens):
+        raise GGUFError("the file has no tokenizer.ggml.tokens string array")
+    vocab = {}
+    for i, t in enumerate(tokens):
+        vocab.setdefault(t, i)  # the first id of a repeated string, as a map built in order keeps it
+    merges = []
+    for m in md.get("tokenizer.ggml.merges", []) or []:
+        parts = m.split(" ")
+        if len(parts) == 2:
+            merges.append((parts[0], parts[1]))
+    special = SpecialTokens()
+    for kind, key in (("bos", "bos_token_id"), ("eos", "eos_token_id"), ("unk", "unknown_token_id"), ("pad", "padding_token_id")):
+        i = md.get(f"tokenizer.ggml.{key}")
+        if isinstance(i, int) and 0 <= i < len(tokens):
+            setattr(special, f"{kind}_token", tokens[i])
+            setattr(special, f"{kind}_token_id", i)
+    return HFTokenizer(vocab, {i: t for i, t in enumerate(tokens)}, merges, special, {})
+
+
 def bench(ctx, log=print, n_rows=11008, k=4096, copies=8, iters=20):
     """Device-side conversion rate of a Q4_0 tensor of the 7B FFN shape (ggml order -> reference order), on
     `copies` back-to-back images so that a launch moves far more than the last-level cache holds."""

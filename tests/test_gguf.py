@@ -122,6 +122,25 @@ def _hand_made_file(tmp_path, alignment=None, version=3, tensor_type=2, bad_offs
     return str(p), t0, t1
 
 
+def test_tokenizer_from_the_files_metadata(tmp_path):
+    # the reference's BPE over a GGUF vocabulary: "low" + "er" by the merge list, ids as the array orders them
+    tokens = ["<unk>", "<s>", "</s>", "l", "o", "w", "e", "r", " ", "lo", "low", "er", "lower"]
+    md = {"general.architecture": "llama", "tokenizer.ggml.model": "gpt2", "tokenizer.ggml.tokens": tokens,
+          "tokenizer.ggml.merges": ["l o", "lo w", "e r", "low er"], "tokenizer.ggml.bos_token_id": 1,
+          "tokenizer.ggml.eos_token_id": 2, "tokenizer.ggml.unknown_token_id": 0}
+    path = str(tmp_path / "tok.gguf")
+    gguf.write_gguf(path, md, {"norm": np.ones(4, np.float32)})
+    with gguf.GGUFReader(path) as r:
+        tok = gguf.tokenizer_from_metadata(r.metadata)
+    assert tok.vocab_size() == len(tokens) and tok.bos_token_id() == 1 and tok.eos_token_id() == 2
+    assert tok.encode("lower") == [1, 12] and tok.encode("low") == [1, 10]  # encode() puts the BOS token in front
+    assert tok.encode_with_options("lower", False, True) == [12, 2]
+    assert tok.decode([10, 11]) == "lower"
+    assert tok.encode_with_options("z", False, False) == [0]  # no such piece: the unknown token
+    with pytest.raises(gguf.GGUFError):
+        gguf.tokenizer_from_metadata({"general.architecture": "llama"})
+
+
 def test_bf16_tensors_widen_exactly(tmp_path):
     # ggml type 30: the bit pattern is the upper half of the f32 word (1.0 = 0x3F80, -2.5 = 0xC020, the largest finite
     # value 0x7F7F, a subnormal 0x0001); such a tensor reads as f32, and as a linear it is carried as an F32 weight
