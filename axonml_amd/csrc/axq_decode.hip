@@ -1469,7 +1469,10 @@ int axq_model_set_linear(axq_model *m, int layer, int which, const axq_weight *w
         axq_weight *sep = nullptr;
         if ((rc = axq_weight_alloc(ctx, w->type, rows, k, &sep))) return rc;
         if ((rc = copy_rows(ctx, sep, w, 0))) { axq_weight_free(ctx, sep); return rc; }
-        AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+        if (hipStreamSynchronize(ctx->stream) != hipSuccess) {
+            axq_weight_free(ctx, sep);
+            return axq_fail(ctx, AXQ_ERR_DRIVER, "axq_model_set_linear: the copy of the weight did not complete");
+        }
         m->w_sep[which][layer] = sep;
         m->set_mask[layer] |= 1u << which;
         return AXQ_OK;
