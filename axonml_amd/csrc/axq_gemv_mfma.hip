@@ -994,8 +994,14 @@ __global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__
         const int g_idx = ww / S, slice = ww - g_idx * S;
         const int blk = lane >> 2, j = lane & 3;
         const int c = (slice << 4) + blk; // this lane's 64-weight chunk of the row
-        const int my_steps = (steps - g_idx + G - 1) / G; // this group's share
-        float *red_lane = red + (4 * g_idx + j) * red_stride + slice * 4 + (lane >> 4);
+        // This group's steps: base, base + stride, ... (my_steps of them).  Dealt in turn, or, with two groups and a count n0
+        // in the flags, the first n0 steps to group 0 and the rest to group 1: the waves of group 1 issue their first
+        // requests behind group 0's and get every step later, so they are given fewer.
+        const int n0 = (flags >> 24) & 0xFF;
+        const bool uneven = n0 != 0 && G == 2;
+        const int base_step = uneven ? (g_idx ? n0 : 0) : g_idx, step_stride = uneven ? 1 : G;
+        const int my_steps = uneven ? (g_idx ? steps - n0 : n0) : (steps - g_idx + G - 1) / G;
+        float *red_lane = red + (4 * base_step + j) * red_stride + slice * 4 + (lane >> 4);
         uint4 *wmeta = lds_raw + n16 + 1 + 4 + (wg_rows * red_stride) / 4 + ww * 64 * NM;
         typename T::Raw buf[NB];
         uint4 hm[NM];
@@ -1003,8 +1009,8 @@ __global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__
         T::lane_offsets(k, c, lo);
         const int wg_row0 = blockIdx.x * wg_rows;
         const Bases bases = {codes + (size_t)wg_row0 * cp, meta + (size_t)wg_row0 * mp, qhp + (size_t)wg_row0 * qp};
-        const int rl0 = 4 * g_idx + j, rl_last = n_rows - 1 - wg_row0; // rows relative to the workgroup's first
-        const int gstride = 4 * G;                                            // rows from one of the group's steps to its next
+        const int rl0 = 4 * base_step + j, rl_last = n_rows - 1 - wg_row0; // rows relative to the workgroup's first
+        const int gstride = 4 * step_stride;                                  // rows from one of the group's steps to its next
         uint32_t moff[NM];
         int mrl0[NM], mst[NM];
         {
@@ -1014,7 +1020,7 @@ __global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__
                 const int flat = i * 64 + lane, off = slice * MSB + (flat % CPR) * 16;
                 const int r = flat / CPR < 4 * NB ? flat / CPR : 4 * NB - 1; // lanes beyond the round's rows repeat its last
                 moff[i] = (uint32_t)(off + 16 <= row_bytes ? off : row_bytes - 16);
-                mrl0[i] = 4 * g_idx + (r & 3); // row r of the round: row r % 4 of its step r / 4
+                mrl0[i] = 4 * base_step + (r & 3); // row r of the round: row r % 4 of its step r / 4
                 mst[i] = r >> 2;
             }
         }
@@ -1069,7 +1075,9 @@ __global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__
 #pragma unroll
             for (int b = 0; b < NB; b++) {
                 fold(b, step + b);
-                request(step + NB + b, b); // steps past the end re-read the first (cache hits): every wave's count of loads stays the same
+                // steps past the end re-read the first (cache hits): every wave's count of loads stays the same (leaving
+                // them out, with the last two rounds written out per count of steps, measured the same)
+                request(step + NB + b, b);
             }
         }
 #pragma unroll
@@ -1209,13 +1217,23 @@ int launch_sw(axq_ctx *ctx, const DpArgs &a) {
     if (a.ymode == AXQ_Y_SWIGLU && (steps & 1)) steps++; // a workgroup must hold whole gate/up groups of 8 rows
     if (steps < G) G = steps;
     const unsigned grid = (unsigned)((rowsteps + steps - 1) / steps);
-    const int per_group = (steps + G - 1) / G;
+    // Two groups: each takes a run of consecutive steps, group 0 three of every five.  Its waves issue their first requests
+    // ahead of group 1's and get every step sooner; measured against steps dealt in turn, launches of one kernel in a row:
+    // 8.2 -> 7.6 us at 14336 x 4096 (14 steps), 12.7 -> 12.2 us at 28672 x 4096, 14.1 -> 13.4 us at 32000 x 4096.  Not
+    // at six steps: 6144 x 4096 gains alone (5.6 -> 5.05 us) and loses inside the decode step (4 + 2 steps leave a ring of two).
+    static const int split0 = getenv("AXQ_GEMV_SPLIT0") ? atoi(getenv("AXQ_GEMV_SPLIT0")) : 60; // development knob, percent; 0 = dealt in turn
+    int n0 = 0;
+    if (G == 2 && steps >= 7 && steps < 256 && split0 > 0) {
+        n0 = (steps * split0 + 50) / 100;
+        n0 = n0 < 2 ? 2 : (n0 > steps - 2 ? steps - 2 : n0);
+    }
+    const int per_group = n0 ? (steps - n0 < n0 ? steps - n0 : n0) : (steps + G - 1) / G;
     const int nb = per_group < 4 ? per_group : 4; // ring depth: deeper rings measured slower (a wave that stands at its requests folds nothing)
     const int cpr = T::META_SLICE_BYTES / 16, nm = (4 * nb * cpr + 63) / 64;
     size_t lds = axq_split_bytes(a.k) + 16 + 64 + (size_t)steps * 4 * 4 * S * sizeof(float) + (size_t)(S * G) * nm * 1024;
     if (lds > 160 * 1024) return 0;
     const unsigned block = (unsigned)(64 * (S * G + NS));
-    const int flags = a.mode | (a.ymode << 8) | (G << 16);
+    const int flags = a.mode | (a.ymode << 8) | (G << 16) | (n0 << 24);
     auto go = [&](auto kern, std::atomic<uint64_t> &mask) -> int {
 #ifdef AXQ_STAMPS
         lds = 160 * 1024; // the stamps live in the last 4 KB
