@@ -84,7 +84,7 @@ __device__ inline float recombine(int4v d, float sg) {
 // MFMA A operands, and scale / plain sum of its two 32-element groups.
 struct XOp {
     int a[16];
-    float sg[2], xs[2];
+    float sg[4], xs[2]; // sg[2], sg[3]: types whose lane covers four runs of 16 (RUNS16)
     int4v init[2]; // -(code centre) * (limb sums of the group): the accumulators start here, so that the
                    // MFMAs sum (n - centre) * limb exactly and no large terms cancel in f32 afterwards
 };
@@ -93,7 +93,7 @@ struct XOp {
 // (uniform 64-bit plane base of the workgroup's first row) + (32-bit offset): one integer add per load.
 struct Bases { const uint8_t *codes, *meta, *qh; };  // planes at the workgroup's first row
 struct RowOff { uint32_t c, m, h; };                 // (row - first row) * pitch, per plane
-struct LaneOff { uint32_t c[2], m[2], h[2]; };       // the lane's byte offsets inside a row, per plane
+struct LaneOff { uint32_t c[2], m[2], h[2], d[2]; }; // the lane's byte offsets inside a row, per plane (d: a second kind of record in the meta plane)
 // Weights are read once per call: non-temporal loads keep them from displacing x and the other kernels' operands in
 // the caches, and stream measurably faster (a pure read of 33 MB: 6.2 against 6.75 us per launch).
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -112,6 +112,7 @@ __device__ inline uint32_t ld2(const uint8_t *base, uint32_t off) { return __bui
 // ---------------------------------------------------------------------------
 struct DQ4K {
     struct Raw { uint4 q0, q1, h; };
+    static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 8; // w = d*sc*(q - 8) + (8*d*sc - dmin*m)
     static constexpr int BIG_NB = 4; // row steps a lane can hold within 128 registers
@@ -184,12 +185,99 @@ struct DQ4K {
     }
 };
 
+// Q5_K (GGUF): Q4_K's code plane and headers; the fifth bits lie in a plane of their own, 32 bytes per superblock, byte l
+// bit s = fifth bit of element l of sub-block s.  A lane (pair p of its superblock) takes bits 2p and 2p + 1 of all 32
+// bytes.  Four lanes share those bytes, so they are not loaded per lane and step (a load of 1 KB of lane addresses for
+// 256 bytes) but fetched once per round with the headers, as part of the record that goes through LDS.
+struct DQ5K {
+    struct Raw { uint4 q0, q1, b0, b1, h; };
+    static constexpr bool RUNS16 = false, OWN_META_PIECES = true;
+    static constexpr bool PERM_A = false;
+    static constexpr int CENTRE = 16; // w = d*sc*(q - 16) + (16*d*sc - dmin*m)
+    static constexpr int BIG_NB = 4;
+    static constexpr bool ROUND_META = true;
+    static constexpr int META_SLICE_BYTES = 192; // per row and slice in LDS: four superblock headers, then their 4 x 32 bytes of fifth bits
+    __host__ __device__ static int meta_row_bytes(int k) { return (k >> 8) * 16; }
+    __device__ static int meta_piece(int k, int slice, int piece, bool &from_qh) {
+        const int nsb = k >> 8;
+        from_qh = piece >= 4;
+        if (!from_qh) {
+            const int off = slice * 64 + piece * 16;
+            return off + 16 <= nsb * 16 ? off : nsb * 16 - 16;
+        }
+        const int off = slice * 128 + (piece - 4) * 16;
+        return off + 16 <= nsb * 32 ? off : nsb * 32 - 16;
+    }
+    // with per-round records the fifth bits come with the headers, through LDS
+    __device__ static void load_codes(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+        r.q0 = ld16(b.codes, ro.c + o.c[0]);
+        r.q1 = ld16(b.codes, ro.c + o.c[1]);
+    }
+    __device__ static void set_meta(Raw &r, const uint8_t *row, int blk, int) {
+        r.h = *reinterpret_cast<const uint4 *>(row + (blk >> 2) * 16);
+        r.b0 = *reinterpret_cast<const uint4 *>(row + 64 + (blk >> 2) * 32);
+        r.b1 = *reinterpret_cast<const uint4 *>(row + 64 + (blk >> 2) * 32 + 16);
+    }
+    __device__ static int group_k(int c, int g) { return c * 64 + g * 32; }
+    __device__ static void lane_offsets(int k, int c, LaneOff &o) {
+        DQ4K::lane_offsets(k, c, o);
+        const int cpr = k >> 6;
+        c = c < cpr ? c : cpr - 1;
+        o.h[0] = (uint32_t)(c >> 2) * 32;
+    }
+    __device__ static void load(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+        load_codes(b, ro, o, r);
+        r.b0 = ld16(b.qh, ro.h + o.h[0]); // the four lanes of a superblock read the same 32 bytes
+        r.b1 = ld16(b.qh, ro.h + o.h[0] + 16);
+        r.h = ld16(b.meta, ro.m + o.m[0]);
+    }
+    __device__ static float dot(const Raw &r, const XOp &x, int c) {
+        const uint32_t q0[4] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w};
+        const uint32_t q1[4] = {r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const uint32_t b0[4] = {r.b0.x, r.b0.y, r.b0.z, r.b0.w};
+        const uint32_t b1[4] = {r.b1.x, r.b1.y, r.b1.z, r.b1.w};
+        const int p = c & 3;
+        int4v lo = x.init[0], hi = x.init[1];
+        uint32_t ml[8], mh[8];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t f0 = b0[w] >> (2 * p), f1 = b1[w] >> (2 * p); // bit 0 of a byte: sub-block 2p, bit 1: 2p + 1
+            ml[w] = (q0[w] & 0x0F0F0F0Fu) | ((f0 & 0x01010101u) << 4);
+            mh[w] = ((q0[w] >> 4) & 0x0F0F0F0Fu) | ((f0 & 0x02020202u) << 3);
+            ml[4 + w] = (q1[w] & 0x0F0F0F0Fu) | ((f1 & 0x01010101u) << 4);
+            mh[4 + w] = ((q1[w] >> 4) & 0x0F0F0F0Fu) | ((f1 & 0x02020202u) << 3);
+        }
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            lo = mfma(x.a[w], ml[w], lo);
+            hi = mfma(x.a[8 + w], mh[w], hi);
+        }
+        int sh = (p & 1) * 16;
+        uint32_t ya = r.h.y >> sh, za = r.h.z >> sh, wa = r.h.w >> sh;
+        uint32_t scp, mp;
+        if (p < 2) {
+            scp = ya & 0x3F3F;
+            mp = za & 0x3F3F;
+        } else {
+            scp = (wa & 0x0F0F) | ((ya >> 2) & 0x3030);
+            mp = ((wa >> 4) & 0x0F0F) | ((za >> 2) & 0x3030);
+        }
+        const float d = f16lo(r.h.x), dmin = f16hi(r.h.x);
+        const float s0 = d * ub0(scp), s1 = d * ub1(scp);
+        float y = fmaf(s0, recombine(lo, x.sg[0]), s1 * recombine(hi, x.sg[1]));
+        y = fmaf(fmaf(16.0f, s0, -(dmin * ub0(mp))), x.xs[0], y);
+        y = fmaf(fmaf(16.0f, s1, -(dmin * ub1(mp))), x.xs[1], y);
+        return y;
+    }
+};
+
 // Q4_0 / Q4_1 (reference nibble order, types.rs:179-198: byte i = elements 2i, 2i+1).  The lane's
 // two groups are the 32-element blocks c*2 and c*2+1... taken 16 blocks apart so that one load
 // instruction reads 256 contiguous bytes per row.
 template <bool WITH_MIN>
 struct DQ4x {
     struct Raw { uint4 q[2]; uint32_t m[2]; };
+    static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = true; // dword w of a block: low nibbles = elements 8w+{0,2,4,6}, high = 8w+{1,3,5,7}
     static constexpr int CENTRE = 8;
     static constexpr int BIG_NB = 4;
@@ -250,6 +338,7 @@ struct DQ4x {
 template <bool WITH_MIN>
 struct DQ5x {
     struct Raw { uint4 q[2]; uint32_t qh[2]; uint32_t m[2]; };
+    static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 16;
     static constexpr int BIG_NB = 4;
@@ -317,6 +406,7 @@ struct DQ5x {
 // Q8_0: four 16-byte vectors of int8 codes per lane per pass = two blocks; the codes are the B operand as they are.
 struct DQ80 {
     struct Raw { uint4 q[4]; uint32_t m[2]; };
+    static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 0;
     static constexpr int BIG_NB = 3;
@@ -373,6 +463,130 @@ struct DQ80 {
     }
 };
 
+// Q6_K (GGUF, planes in ggml's order: ql 128 bytes, qh 64 bytes per superblock; meta row = int8 scales 16 bytes per
+// superblock, then the f16 d of every superblock).  A 16-byte piece of ql holds two runs of 16 weights 64 apart (low and
+// high nibbles) with one scale each; their bit pairs lie in one 16-byte piece of qh.  A lane takes piece `blk` and piece
+// `blk + 16` of its wave's 1024-wide K slice (32 pieces), so that either load instruction reads 256 contiguous bytes of
+// each row: four runs of 16, four accumulators, four scales.  The slice has 16 pieces of bit pairs, each wanted by two
+// lanes: lane blk loads piece blk (one instruction, 256 contiguous bytes per row, nothing twice) and the lanes of a row
+// hand each other the two pieces they need when the step is folded.  The codes go in as signed bytes q - 32.
+struct DQ6K {
+    struct Raw { uint4 l0, l1, hq; uint32_t sc; uint32_t d; };
+    static constexpr bool RUNS16 = true, OWN_META_PIECES = true;
+    static constexpr bool PERM_A = false;
+    static constexpr int CENTRE = 0;
+    static constexpr int BIG_NB = 4;
+    static constexpr bool ROUND_META = true;
+    static constexpr int META_SLICE_BYTES = 128; // per row and slice in LDS: 64 bytes of scales, the 16-byte piece with its four d (four times)
+    __host__ __device__ static int meta_row_bytes(int k) { return (k >> 8) * 16 + ((((k >> 8) * 2) + 15) & ~15); }
+    __device__ static int meta_piece(int k, int slice, int piece, bool &from_qh) {
+        const int nsb = k >> 8;
+        from_qh = false;
+        if (piece < 4) {
+            const int off = slice * 64 + piece * 16;
+            return off + 16 <= nsb * 16 ? off : nsb * 16 - 16;
+        }
+        return nsb * 16 + ((slice * 8) & ~15);
+    }
+    // piece P (0..31) of a slice: superblock P / 8 of the slice, half n = (P / 4) % 2, h = P % 4; its runs are sub-blocks
+    // 8n + h (low nibbles, elements 128n + 16h ..) and 8n + 4 + h (high nibbles, 64 elements on)
+    __device__ static int run_k(int c, int r) {
+        const int P = (c & 15) + (r >> 1) * 16;
+        return (c >> 4) * 1024 + (P >> 3) * 256 + ((P >> 2) & 1) * 128 + (P & 3) * 16 + (r & 1) * 64;
+    }
+    __device__ static int group_k(int c, int g) { return run_k(c, 2 * g); } // not used by RUNS16 types
+    __device__ static void lane_offsets(int k, int c, LaneOff &o) {
+        const int ql_bytes = k >> 1, qh_bytes = k >> 2;
+        const int blk = c & 15, slice = c >> 4;
+        const int l0 = slice * 512 + blk * 16, l1 = l0 + 256, h0 = slice * 256 + blk * 16;
+        o.c[0] = (uint32_t)(l0 + 16 <= ql_bytes ? l0 : ql_bytes - 16); // pieces past the row's end meet x = 0
+        o.c[1] = (uint32_t)(l1 + 16 <= ql_bytes ? l1 : ql_bytes - 16);
+        o.h[0] = (uint32_t)(h0 + 16 <= qh_bytes ? h0 : qh_bytes - 16);
+        // without per-round records: the first scale byte and the d of either piece
+        const int nsb = k >> 8, in_sb = ((blk >> 2) & 1) * 8 + (blk & 3);
+        int sb0 = slice * 4 + (blk >> 3), sb1 = sb0 + 2;
+        sb0 = sb0 < nsb ? sb0 : nsb - 1;
+        sb1 = sb1 < nsb ? sb1 : nsb - 1;
+        o.m[0] = (uint32_t)(sb0 * 16 + in_sb);
+        o.m[1] = (uint32_t)(sb1 * 16 + in_sb);
+        o.d[0] = (uint32_t)(nsb * 16 + sb0 * 2);
+        o.d[1] = (uint32_t)(nsb * 16 + sb1 * 2);
+    }
+    __device__ static void load_codes(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+        r.l0 = ld16(b.codes, ro.c + o.c[0]);
+        r.l1 = ld16(b.codes, ro.c + o.c[1]);
+        r.hq = ld16(b.qh, ro.h + o.h[0]);
+    }
+    // row: this row's 128 bytes of the wave's patch (scales of the slice's four superblocks, then the piece with the d's)
+    __device__ static void set_meta(Raw &r, const uint8_t *row, int, int c) {
+        const int blk = c & 15, slice = c >> 4;
+        const int sbl = blk >> 3, n8 = ((blk >> 2) & 1) * 8, h = blk & 3;
+        const uint8_t *s0 = row + sbl * 16 + n8 + h, *s1 = s0 + 32;
+        r.sc = (uint32_t)s0[0] | ((uint32_t)s0[4] << 8) | ((uint32_t)s1[0] << 16) | ((uint32_t)s1[4] << 24);
+        const uint16_t *d = reinterpret_cast<const uint16_t *>(row + 64 + (slice & 1) * 8) + sbl;
+        r.d = (uint32_t)d[0] | ((uint32_t)d[2] << 16);
+    }
+    __device__ static void load(const Bases &b, const RowOff &ro, const LaneOff &o, Raw &r) {
+        load_codes(b, ro, o, r);
+        const uint8_t *m = b.meta + ro.m;
+        r.sc = (uint32_t)m[o.m[0]] | ((uint32_t)m[o.m[0] + 4] << 8) | ((uint32_t)m[o.m[1]] << 16) | ((uint32_t)m[o.m[1] + 4] << 24);
+        r.d = (uint32_t)*reinterpret_cast<const uint16_t *>(m + o.d[0]) | ((uint32_t)*reinterpret_cast<const uint16_t *>(m + o.d[1]) << 16);
+    }
+    __device__ static float dot(const Raw &r, const XOp &x, int c) {
+        const uint32_t ql[2][4] = {{r.l0.x, r.l0.y, r.l0.z, r.l0.w}, {r.l1.x, r.l1.y, r.l1.z, r.l1.w}};
+        // the bit pairs of piece P lie in piece (P / 8) * 4 + ((P / 4) % 2) * 2 + P % 2 of the slice's sixteen, those of piece
+        // P + 16 eight pieces on: held by the lanes of this row (lane % 4) whose blk is that number
+        const int lane = (int)(threadIdx.x & 63), blk = c & 15;
+        const int src0 = ((((blk >> 3) * 4 + ((blk >> 2) & 1) * 2 + (blk & 1)) << 2) | (lane & 3)) << 2, src1 = src0 + (8 << 4); // byte addresses of lanes
+        const int hq[4] = {(int)r.hq.x, (int)r.hq.y, (int)r.hq.z, (int)r.hq.w};
+        uint32_t qh[2][4];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            qh[0][w] = (uint32_t)__builtin_amdgcn_ds_bpermute(src0, hq[w]);
+            qh[1][w] = (uint32_t)__builtin_amdgcn_ds_bpermute(src1, hq[w]);
+        }
+        const int sh = ((c >> 1) & 1) * 2; // bit pair h / 2 for the low-nibble run, two pairs on for the high-nibble run
+        int4v acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            uint32_t bl[4], bh[4]; // the piece's eight B operands first, then its products
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const uint32_t f = qh[t][w] >> sh;
+                const uint32_t ul = (ql[t][w] & 0x0F0F0F0Fu) | ((f & 0x03030303u) << 4);
+                const uint32_t uh = ((ql[t][w] >> 4) & 0x0F0F0F0Fu) | (f & 0x30303030u);
+                bl[w] = (ul + 0x60606060u) ^ 0x80808080u; // q - 32 as a signed byte, no carry between bytes
+                bh[w] = (uh + 0x60606060u) ^ 0x80808080u;
+            }
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                acc[2 * t] = mfma(x.a[8 * t + w], bl[w], acc[2 * t]);
+                acc[2 * t + 1] = mfma(x.a[8 * t + 4 + w], bh[w], acc[2 * t + 1]);
+            }
+        }
+        const float d0 = f16lo(r.d), d1 = f16hi(r.d);
+        float y0 = (float)(int8_t)(r.sc & 0xFF) * recombine(acc[0], x.sg[0]);
+        y0 = fmaf((float)(int8_t)((r.sc >> 8) & 0xFF), recombine(acc[1], x.sg[1]), y0);
+        float y1 = (float)(int8_t)((r.sc >> 16) & 0xFF) * recombine(acc[2], x.sg[2]);
+        y1 = fmaf((float)(int8_t)(r.sc >> 24), recombine(acc[3], x.sg[3]), y1);
+        return fmaf(d0, y0, d1 * y1);
+    }
+};
+
+// The 16-byte piece `piece` of the record that a round fetches per row and K slice: its byte offset in the row of the meta
+// plane, or (from_qh) of the qh plane, for types that keep their high bits in the record as well.  Pieces past the end
+// of a row that does not fill its last slice are moved back inside it (they serve lanes whose x is zero).
+template <class T>
+__device__ inline int record_piece(int k, int slice, int piece, bool &from_qh) {
+    from_qh = false;
+    if constexpr (T::OWN_META_PIECES) {
+        return T::meta_piece(k, slice, piece, from_qh);
+    } else {
+        const int off = slice * T::META_SLICE_BYTES + piece * 16, row_bytes = T::meta_row_bytes(k);
+        return off + 16 <= row_bytes ? off : row_bytes - 16;
+    }
+}
+
 // Gather bytes {0,2} of lo and {0,2} of hi (sel = 0) or {1,3} of each (sel = 1)
 __device__ inline int pick_alt(uint32_t lo, uint32_t hi, int sel) {
     return (int)__builtin_amdgcn_perm(hi, lo, sel ? 0x07050301u : 0x06040200u);
@@ -380,6 +594,22 @@ __device__ inline int pick_alt(uint32_t lo, uint32_t hi, int sel) {
 
 template <class T>
 __device__ inline void fetch_xop(const uint8_t *planes, const uint4 *grp, int kpad, int k, int limb, int c, XOp &o) {
+    if constexpr (T::RUNS16) { // four runs of 16: one 16-byte piece of the limb plane and the scale of its 32-element group each
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int kb = T::run_k(c, r);
+            uint4 u = {0, 0, 0, 0};
+            o.sg[r] = 0.f;
+            if (kb < k) {
+                u = *reinterpret_cast<const uint4 *>(planes + (size_t)limb * kpad + kb);
+                o.sg[r] = __builtin_bit_cast(float, grp[kb >> 5].x);
+            }
+            o.a[4 * r] = (int)u.x; o.a[4 * r + 1] = (int)u.y; o.a[4 * r + 2] = (int)u.z; o.a[4 * r + 3] = (int)u.w;
+        }
+        o.xs[0] = o.xs[1] = 0.f;
+        o.init[0] = o.init[1] = int4v{0, 0, 0, 0};
+        return;
+    }
 #pragma unroll
     for (int g = 0; g < 2; g++) {
         int kb = T::group_k(c, g);
@@ -519,14 +749,17 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(DP
     const int rl0 = g_idx * rows_per_group + j, rl_last = last - wg_row0; // rows relative to the workgroup's first
     // scale loads of a round (RND): 64 * NM lanes = (row of the round's 16, 16-byte chunk of the slice's MSB bytes); chunks past
     // the row's end (a last slice that is not whole) are moved back inside it: they serve lanes whose x is zero
-    uint32_t moff[NM];
+    uint32_t moff[NM], mpitch[NM];
+    const uint8_t *mbase[NM];
     int mrl0[NM];
     {
-        const int row_bytes = T::meta_row_bytes(a.k);
 #pragma unroll
         for (int i = 0; i < NM; i++) {
-            const int flat = i * 64 + lane, off = slice * MSB + (flat % CPR) * 16;
-            moff[i] = (uint32_t)(off + 16 <= row_bytes ? off : row_bytes - 16);
+            const int flat = i * 64 + lane;
+            bool from_qh;
+            moff[i] = (uint32_t)record_piece<T>(a.k, slice, flat % CPR, from_qh);
+            mbase[i] = from_qh ? bases.qh : bases.meta;
+            mpitch[i] = from_qh ? qp : mp;
             mrl0[i] = g_idx * rows_per_group + flat / CPR;
         }
     }
@@ -541,7 +774,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(DP
                 for (int i = 0; i < NM; i++) {
                     int rlm = mrl0[i] + 4 * s;
                     rlm = rlm < rl_last ? rlm : rl_last;
-                    hm[i] = ld16(bases.meta, (uint32_t)rlm * mp + moff[i]);
+                    hm[i] = ld16(mbase[i], (uint32_t)rlm * mpitch[i] + moff[i]);
                 }
             }
             T::load_codes(bases, ro, lo, buf[b]);
@@ -727,14 +960,17 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     const int rl0 = g_idx * rows_per_group + j, rl_last = last - wg_row0; // rows relative to the workgroup's first
     // header loads of a round: 64 * NM lanes = (row of the round's 16, 16-byte chunk of the slice's MSB bytes); chunks past the
     // row's end (a last slice that is not whole) are moved back inside it: they serve lanes whose x is zero
-    uint32_t moff[NM];
+    uint32_t moff[NM], mpitch[NM];
+    const uint8_t *mbase[NM];
     int mrl0[NM];
     {
-        const int row_bytes = T::meta_row_bytes(a.k);
 #pragma unroll
         for (int i = 0; i < NM; i++) {
-            const int flat = i * 64 + lane, off = slice * MSB + (flat % CPR) * 16;
-            moff[i] = (uint32_t)(off + 16 <= row_bytes ? off : row_bytes - 16);
+            const int flat = i * 64 + lane;
+            bool from_qh;
+            moff[i] = (uint32_t)record_piece<T>(a.k, slice, flat % CPR, from_qh);
+            mbase[i] = from_qh ? bases.qh : bases.meta;
+            mpitch[i] = from_qh ? qp : mp;
             mrl0[i] = g_idx * rows_per_group + flat / CPR;
         }
     }
@@ -749,7 +985,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
                 for (int i = 0; i < NM; i++) {
                     int rlm = mrl0[i] + 4 * s;
                     rlm = rlm < rl_last ? rlm : rl_last;
-                    hm[i] = ld16(bases.meta, (uint32_t)rlm * mp + moff[i]);
+                    hm[i] = ld16(mbase[i], (uint32_t)rlm * mpitch[i] + moff[i]);
                 }
             }
             T::load_codes(bases, ro, lo, buf[b]);
@@ -1011,15 +1247,18 @@ __global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__
         const Bases bases = {codes + (size_t)wg_row0 * cp, meta + (size_t)wg_row0 * mp, qhp + (size_t)wg_row0 * qp};
         const int rl0 = 4 * base_step + j, rl_last = n_rows - 1 - wg_row0; // rows relative to the workgroup's first
         const int gstride = 4 * step_stride;                                  // rows from one of the group's steps to its next
-        uint32_t moff[NM];
+        uint32_t moff[NM], mpitch[NM];
+        const uint8_t *mbase[NM];
         int mrl0[NM], mst[NM];
         {
-            const int row_bytes = T::meta_row_bytes(k);
 #pragma unroll
             for (int i = 0; i < NM; i++) {
-                const int flat = i * 64 + lane, off = slice * MSB + (flat % CPR) * 16;
+                const int flat = i * 64 + lane;
                 const int r = flat / CPR < 4 * NB ? flat / CPR : 4 * NB - 1; // lanes beyond the round's rows repeat its last
-                moff[i] = (uint32_t)(off + 16 <= row_bytes ? off : row_bytes - 16);
+                bool from_qh;
+                moff[i] = (uint32_t)record_piece<T>(k, slice, flat % CPR, from_qh);
+                mbase[i] = from_qh ? bases.qh : bases.meta;
+                mpitch[i] = from_qh ? qp : mp;
                 mrl0[i] = 4 * base_step + (r & 3); // row r of the round: row r % 4 of its step r / 4
                 mst[i] = r >> 2;
             }
@@ -1036,7 +1275,7 @@ __global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__
                     sm = sm < my_steps ? sm : 0;
                     int rlm = mrl0[i] + gstride * sm;
                     rlm = rlm < rl_last ? rlm : rl_last;
-                    hm[i] = ld16(bases.meta, (uint32_t)rlm * mp + moff[i]);
+                    hm[i] = ld16(mbase[i], (uint32_t)rlm * mpitch[i] + moff[i]);
                 }
             }
             T::load_codes(bases, ro, lo, buf[b]);
@@ -1325,6 +1564,8 @@ int axq_dev_gemv_dp_ex(axq_ctx *ctx, const axq_weight *w, const float *x, const 
         return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "the SwiGLU epilogue needs whole groups of 8 rows and no bias");
     switch (w->type) {
     case AXQ_Q4_K: ok = launch_dp<DQ4K>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
+    case AXQ_Q5_K: ok = launch_dp<DQ5K>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
+    case AXQ_Q6_K: ok = launch_dp<DQ6K>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
     case AXQ_Q4_0: ok = launch_dp<DQ4x<false>>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
     case AXQ_Q4_1: ok = launch_dp<DQ4x<true>>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
     case AXQ_Q5_0: ok = launch_dp<DQ5x<false>>(ctx, w, x, xq, mode, aux, eps, ymode, bias, y); break;
@@ -1344,7 +1585,7 @@ int axq_dev_gemv_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uin
 // Whether axq_dev_gemv_dp_ex covers a weight of this type and width.
 bool axq_dev_gemv_dp_covers(const axq_weight *w) {
     switch (w->type) {
-    case AXQ_Q4_K: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q8_0:
+    case AXQ_Q4_K: case AXQ_Q5_K: case AXQ_Q6_K: case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q8_0:
         return w->k % 64 == 0 && w->k <= 16384;
     default: return false;
     }

@@ -76,6 +76,16 @@ def test_config_q4_k_headline(ctx, n, k):
     (o.Q5_0, 5000, 1536),
     (o.Q5_1, 5000, 1088),   # 136 bytes of scale records per row: the kernel without rounds
     (o.Q8_0, 5000, 2560),
+    (o.Q5_K, 7001, 2304),   # the fifth bits come with the headers once per round; last slice a quarter full
+    (o.Q5_K, 9000, 1280),
+    (o.Q5_K, 3000, 6144),
+    (o.Q5_K, 2000, 9216 + 256),  # beyond eight slices: per-wave staging, 37 superblocks
+    (o.Q6_K, 7001, 2304),   # bit pairs handed from lane to lane; pieces past the end of a last slice that is not whole
+    (o.Q6_K, 9000, 1280),
+    (o.Q6_K, 40000, 1024),
+    (o.Q6_K, 3000, 6144),
+    (o.Q6_K, 5000, 768),    # three superblocks: the second piece of most lanes lies past the row's end
+    (o.Q6_K, 2000, 9216 + 256),
 ])
 def test_gemv_scale_records_per_round(ctx, qtype, n, k):
     """Shapes that take the one-vector kernels through several rounds of row steps, partial K slices and ragged row counts."""
@@ -114,7 +124,7 @@ def test_linearity_and_determinism_at_full_size(ctx):
     dw.free()
 
 
-@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0])
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0])
 @pytest.mark.parametrize("k", [512, 4096, 32768 + 256])
 def test_activations_with_a_mean_do_not_cancel(ctx, qtype, k):
     # post-softmax / post-SiLU activations are not zero-mean: offsets of the unsigned codes must be
