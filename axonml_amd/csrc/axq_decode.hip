@@ -1452,6 +1452,15 @@ int axq_model_set_linear(axq_model *m, int layer, int which, const axq_weight *w
         row_off = which == AXQ_LIN_GATE ? 0 : m->cfg.intermediate_size;
     }
     int rc;
+    // a linear that has its slot to itself (o, down, lm_head) may come back in another block type: the slot is made anew
+    if (*slot && (*slot)->type != w->type && slot_rows == rows) {
+        AXQ_HIP(ctx, hipStreamSynchronize(ctx->stream), AXQ_ERR_DRIVER);
+        axq_weight *fresh = nullptr;
+        if ((rc = axq_weight_alloc(ctx, w->type, slot_rows, k, &fresh))) return rc;
+        axq_weight_free(ctx, *slot);
+        *slot = fresh;
+        invalidate_graphs(m);
+    }
     if (!*slot && (rc = axq_weight_alloc(ctx, w->type, slot_rows, k, slot))) return rc;
     const bool qkv_part = layer >= 0 && which <= AXQ_LIN_V;
     if (qkv_part && (m->w_sep[which][layer] || (*slot)->type != w->type)) {

@@ -170,6 +170,41 @@ class QuantizedLlama:
             pass
 
 
+def _bench_q4_k_m_mix(ctx, m, cfg, prompt, new_tokens, weight_elems, mean_ctx, log):
+    """The same model with the block types of llama.cpp's Q4_K_M recipe: attn_v and ffn_down of half the layers
+    (use_more_bits: the first and last eighth and every third between) and the output matrix in Q6_K, the rest Q4_K.
+    A v of another type than q and k is multiplied apart, one more GEMV in those layers."""
+    from ._lib import MEM_DEVICE
+    lib, L = ctx.lib, cfg["num_hidden_layers"]
+    more = [l for l in range(L) if l < L // 8 or l >= 7 * L // 8 or (l - L // 8) % 3 == 2]
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    kv = cfg["num_key_value_heads"] * cfg["head_dim"]
+    f = ctx.malloc(max(V * H, H * I) * 4)
+    seed, q6_elems = 1000, 0
+    for l, name, n, k in [(l, nm, n, k) for l in more for nm, n, k in (("v", kv, H), ("down", H, I))] + [(-1, "q", V, H)]:
+        seed += 1
+        ctx.check(lib.axq_fill_normal_f32(ctx.handle, f, n * k, 0.0, 0.02, 0.0, 0.0, seed))
+        h = C.c_void_p()
+        ctx.check(lib.axq_weight_quantize(ctx.handle, int(QuantType.Q6_K), n, k, f, MEM_DEVICE, C.byref(h)))
+        dw = DeviceWeight(ctx, h, QuantType.Q6_K, n, k)
+        m.set_linear(l, name, dw)
+        dw.free()
+        q6_elems += n * k
+    ctx.free(f)
+    m.reset()
+    m.generate(prompt, 4)
+    m.reset()
+    _, pre_ms, dec_ms = m.generate(prompt, new_tokens)
+    steps = new_tokens - 1
+    tok_s = steps / (dec_ms * 1e-3)
+    nbytes = (weight_elems - q6_elems) * 0.5625 + q6_elems * 210 / 256 + 131072 * mean_ctx + 131072
+    log(f"  Q4_K_M mix ({len(more)} layers with attn_v and ffn_down in Q6_K, output in Q6_K): {tok_s:.1f} tok/s, "
+        f"{nbytes * tok_s / 1e9:.0f} GB/s")
+    return {"q4_k_m_mix_tokens_per_s": tok_s, "q4_k_m_mix_algorithmic_bytes_per_token": nbytes,
+            "q4_k_m_mix_gbps": nbytes * tok_s / 1e9, "q4_k_m_mix_prefill_tokens_per_s": len(prompt) / (pre_ms * 1e-3),
+            "q4_k_m_mix_q6_k_layers": len(more)}
+
+
 def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128, one_sequence_only=False):
     """Decode benchmark: Mistral-7B shape, random init, all linears Q4_K, f16 KV cache; greedy, sampled, and several
     sequences side by side (one_sequence_only: the greedy single-sequence run alone, for kernel profiles)."""
@@ -233,5 +268,7 @@ def bench_7b(ctx, log=print, prompt_len=512, new_tokens=128, one_sequence_only=F
     res["batch64_tokens_per_s"] = 64 * new_tokens / (dec_b * 1e-3)
     res["batch64_ms_per_step"] = dec_b / new_tokens
     log(f"  64 sequences: {res['batch64_tokens_per_s']:.0f} tok/s in all ({res['batch64_ms_per_step']:.3f} ms per step)")
+    m.set_batch(1)
+    res.update(_bench_q4_k_m_mix(ctx, m, cfg, prompt, new_tokens, weights, mean_ctx, log))  # last: it changes the weights
     m.close()
     return res

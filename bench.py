@@ -488,7 +488,9 @@ def main():
         cases = [(T.Q4_K, 4096, 14336, 1, 0.01), (T.Q8_0, 4096, 4096, 1, 0.0), (T.Q4_0, 11008, 4096, 1, 0.0),
                  (T.Q4_0, 4096, 11008, 1, 0.0), (T.Q4_1, 11008, 4096, 1, 0.0), (T.Q4_1, 4096, 11008, 1, 0.0),
                  (T.Q4_0, 11008, 4096, 8, 0.0), (T.Q4_1, 11008, 4096, 8, 0.0), (T.Q4_0, 4096, 11008, 8, 0.0),
-                 (T.Q4_1, 4096, 11008, 8, 0.0)]
+                 (T.Q4_1, 4096, 11008, 8, 0.0),
+                 # the types a Q4_K_M or Q5_K_M GGUF file holds beside Q4_K
+                 (T.Q6_K, 14336, 4096, 1, 0.0), (T.Q6_K, 4096, 14336, 1, 0.0), (T.Q5_K, 14336, 4096, 1, 0.0)]
         gem = []
         for qt, n, k, b, op in cases:
             r, ws2, _, xd, yd = gemv_case(ctx, qt, n, k, b, args.steps, 50, outlier_p=op)

@@ -213,7 +213,8 @@ AXQ_API int axq_model_set_embedding_f32(axq_model *m, const float *table, int me
 AXQ_API int axq_model_set_norm(axq_model *m, int layer, int which, const float *w, int mem);
 /* layer -1 = lm_head.  The model copies the weight's blocks; the caller may free `w`.  q, k and v of a layer share one
  * fused weight of the block type of whichever is set first; a q, k or v of another type is kept as a weight of its own
- * (row counts must be multiples of 4 then).  gate and up share one weight and one type (AXQ_ERR_INVALID_QUANT_TYPE). */
+ * (row counts must be multiples of 4 then).  gate and up share one weight and one type (AXQ_ERR_INVALID_QUANT_TYPE).
+ * o, down and the lm_head may be set again in another block type. */
 AXQ_API int axq_model_set_linear(axq_model *m, int layer, int which, const axq_weight *w);
 /* Fill every linear (Q4_K by default), the embedding and unit norms from a
  * seeded device generator: N(0, std) weights.  For benchmarks of random-init

@@ -333,6 +333,34 @@ def test_the_two_prompt_attention_kernels_agree(ctx, monkeypatch, over, n_first,
         assert np.abs(af - bf).max() <= 2.0 ** -9 * np.abs(af).max()  # isolated one-ulp f16 roundings at most
 
 
+def test_a_linear_set_again_in_another_block_type(ctx):
+    """o, down and the lm_head have their slots to themselves: setting one again in another type replaces it (and drops
+    the recorded step, which holds the old weight's address); the walk then follows the oracle with the new weights."""
+    c = tiny_config(max_seq_len=64)
+    w = random_weights(c, 81)
+    gpu = load_gpu(ctx, c, w)
+    tok = 5
+    for _ in range(6):
+        tok, _ = gpu.forward(tok)
+    w2 = requantize(c, w, {(0, "down"): o.Q6_K, (1, "o"): o.Q8_0, (-1, "head"): o.Q6_K}, 82)
+    L = w2["layers"]
+    shapes = {"down": (c["hidden_size"], c["intermediate_size"]), "o": (c["hidden_size"], c["num_heads"] * c["head_dim"])}
+    gpu.set_linear(0, "down", q.QuantizedTensor(list(shapes["down"]), o.Q6_K, L[0]["down"]))
+    gpu.set_linear(1, "o", q.QuantizedTensor(list(shapes["o"]), o.Q8_0, L[1]["o"]))
+    gpu.set_linear(-1, "q", q.QuantizedTensor([c["vocab_size"], c["hidden_size"]], o.Q6_K, w2["head"]))
+    gpu.reset()
+    cpu = load_oracle(c, w2)
+    tok = 5
+    for pos in range(30):
+        c_next, c_logits = cpu.forward(tok, pos)
+        g_next, g_logits = gpu.forward(tok)
+        assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, pos
+        assert g_next == c_next, pos
+        tok = c_next
+    gpu.close()
+    cpu.close()
+
+
 @pytest.mark.parametrize("changes", [{(0, "v"): o.Q6_K}, {(0, "k"): o.Q8_0, (0, "v"): o.Q6_K, (1, "v"): o.Q5_1},
                                      {(1, "q"): o.Q6_K, (0, "down"): o.Q6_K, (1, "o"): o.Q8_0, (-1, "head"): o.Q6_K}])
 def test_q_k_v_of_different_block_types(ctx, changes):
