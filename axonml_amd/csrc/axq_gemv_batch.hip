@@ -32,8 +32,8 @@ constexpr int WAVE_K = 32 * UNITS;
 constexpr int MAX_BATCH = 8;
 
 struct MbArgs {
-    const uint8_t *codes, *meta;
-    size_t codes_pitch, meta_pitch;
+    const uint8_t *codes, *meta, *qh;
+    size_t codes_pitch, meta_pitch, qh_pitch;
     const uint8_t *xa;  // the batch's limbs as MFMA A operands: [block][h][row 4 b + l] x 16 bytes (pack_x_kernel)
     const float *xsg;   // [block][h][4]: group scales of vectors h, h + 2, h + 4, h + 6; then the plain sums, same layout
     const float *bias;
@@ -64,6 +64,8 @@ __device__ inline float recombine4(int d0, int d1, int d2, int d3) {
 // ---------------------------------------------------------------------------
 template <bool WITH_MIN>
 struct MQ4x {
+    static constexpr int NP2 = 0; // no second plane
+    static constexpr bool RUNS16 = false;
     static constexpr bool EVEN_ODD = true;
     static constexpr bool OFFSET = true; // w = d * code + mo with mo = min (Q4_1) or -8 d (Q4_0): the codes stay unsigned
     static constexpr int NV = UNITS * (WITH_MIN ? 4 : 2) / 16 > 0 ? UNITS * (WITH_MIN ? 4 : 2) / 16 : 1; // 16-byte vectors of scales per chunk
@@ -102,6 +104,8 @@ struct MQ4x {
 };
 
 struct MQ80 {
+    static constexpr int NP2 = 0; // no second plane
+    static constexpr bool RUNS16 = false;
     static constexpr bool EVEN_ODD = false;
     static constexpr bool OFFSET = false;
     static constexpr int NV = UNITS / 8 > 0 ? UNITS / 8 : 1;
@@ -132,6 +136,8 @@ struct MQ80 {
 // Q4_K: a block is a sub-block; the lane's 16-byte piece of pair p (first half for h = 0, second for h = 1)
 // holds its codes of sub-block 2p in the low nibbles and of sub-block 2p + 1 in the high ones.
 struct MQ4K {
+    static constexpr int NP2 = 0; // no second plane
+    static constexpr bool RUNS16 = false;
     static constexpr bool EVEN_ODD = false;
     static constexpr bool OFFSET = true;
     struct Raw { u32x4 q[UNITS / 2]; u32x4 h[UNITS / 8]; };
@@ -177,6 +183,117 @@ struct MQ4K {
     }
 };
 
+// Q5_K: Q4_K's pieces and headers; the fifth bits from the qh plane (32 bytes per superblock, byte l bit s = element l of
+// sub-block s): its two 16-byte pieces go through a second patch, lane half h wants piece h.
+struct MQ5K {
+    static constexpr int NP2 = 2, NQ2 = 1;
+    static constexpr bool RUNS16 = false;
+    static constexpr bool EVEN_ODD = false;
+    static constexpr bool OFFSET = true;
+    struct Raw { u32x4 q[UNITS / 2]; u32x4 h[UNITS / 8]; u32x4 q2[1]; };
+    static constexpr int NP = 8, NQ = 4;
+    __device__ static size_t piece_off(const MbArgs &a, int blk0, int p) { return MQ4K::piece_off(a, blk0, p); }
+    __device__ static int want(int j, int h) { return 4 * h + j; }
+    __device__ static size_t piece2_off(const MbArgs &, int blk0, int p) { return (size_t)(blk0 >> 3) * 32 + (size_t)p * 16; }
+    __device__ static int want2(int, int h) { return h; }
+    __device__ static void load_meta(const MbArgs &a, size_t row, int blk0, int, Raw &r) {
+        r.h[0] = ldg16(a.meta + row * a.meta_pitch + (size_t)(blk0 >> 3) * 16);
+    }
+    __device__ static int4v operand(const Raw &r, int u, int) {
+        const int sh = 4 * (u & 1);
+        int4v b;
+#pragma unroll
+        for (int i = 0; i < 4; i++) b[i] = (int)(((r.q[u >> 1][i] >> sh) & 0x0F0F0F0Fu) | (((r.q2[0][i] >> u) & 0x01010101u) << 4));
+        return b;
+    }
+    __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
+        MQ4K::Raw t;
+        t.h[0] = r.h[0];
+        MQ4K::coef(t, u, d, mo); // the codes stay unsigned 0..31: w = (d sc) code - dmin m
+    }
+};
+
+// Q6_K (planes in ggml's order): a chunk is one superblock, its blocks u = 4 n + c the 32 elements 128 n + 32 c ..; the two
+// halves of a block are sub-blocks with a scale each, so a block is two products, each with the other half's codes
+// as zeros.  ql piece 4 n + 2 (c % 2) + h holds the lane's 16 codes of blocks (n, c) and (n, c + 2) in its low and
+// high nibbles, qh piece 2 n + h their bit pairs c; the codes go in as signed bytes q - 32.
+struct MQ6K {
+    static constexpr int NP2 = 4, NQ2 = 2;
+    static constexpr bool RUNS16 = true;
+    static constexpr bool EVEN_ODD = false;
+    [[maybe_unused]] static constexpr bool OFFSET = false;
+    struct Raw { u32x4 q[4]; u32x4 m[1]; float d; u32x4 q2[2]; };
+    static_assert(UNITS == 8, "one superblock per chunk");
+    static constexpr int NP = 8, NQ = 4;
+    __device__ static size_t piece_off(const MbArgs &, int blk0, int p) { return (size_t)(blk0 >> 3) * 128 + (size_t)p * 16; }
+    __device__ static int want(int j, int h) { return 2 * j + h; }
+    __device__ static size_t piece2_off(const MbArgs &, int blk0, int p) { return (size_t)(blk0 >> 3) * 64 + (size_t)p * 16; }
+    __device__ static int want2(int j, int h) { return 2 * j + h; }
+    __device__ static void load_meta(const MbArgs &a, size_t row, int blk0, int nblk, Raw &r) {
+        const uint8_t *m = a.meta + row * a.meta_pitch;
+        r.m[0] = ldg16(m + (size_t)(blk0 >> 3) * 16);
+        r.d = __half2float(__ushort_as_half(*reinterpret_cast<const unsigned short *>(m + (size_t)(nblk >> 3) * 16 + (size_t)(blk0 >> 3) * 2)));
+    }
+    __device__ static int4v operand(const Raw &r, int u, int) {
+        const int n = u >> 2, c = u & 3, sh = 4 * (c >> 1);
+        int4v b;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t v = ((r.q[2 * n + (c & 1)][i] >> sh) & 0x0F0F0F0Fu) | (((r.q2[n][i] >> (2 * c)) & 0x03030303u) << 4);
+            b[i] = (int)((v + 0x60606060u) ^ 0x80808080u); // q - 32 as a signed byte, no carry between bytes
+        }
+        return b;
+    }
+    // d * scale of half `hh` of block u (sub-block 2 u + hh)
+    __device__ static float coef16(const Raw &r, int u, int hh) {
+        const int sb = 2 * u + hh;
+        return r.d * (float)(int8_t)((r.m[0][sb >> 2] >> (8 * (sb & 3))) & 0xFF);
+    }
+    __device__ static void coef(const Raw &, int, float &d, float &mo) { d = 0.f; mo = 0.f; } // not used (RUNS16)
+};
+
+// Q5_0 / Q5_1 (GGUF): byte j of a block's 16 = elements j (low nibble) and j + 16 (high); the qh plane holds the fifth bits,
+// 4 bytes per block: the chunk's 32 bytes are two pieces, every lane wants both.
+template <bool WITH_MIN>
+struct MQ5x {
+    static constexpr int NP2 = 2, NQ2 = 2;
+    static constexpr bool RUNS16 = false;
+    static constexpr bool EVEN_ODD = false;
+    static constexpr bool OFFSET = true;
+    static constexpr int NV = MQ4x<WITH_MIN>::NV;
+    struct Raw { u32x4 q[UNITS]; u32x4 m[NV]; u32x4 q2[2]; };
+    static constexpr int NP = UNITS, NQ = UNITS;
+    __device__ static size_t piece_off(const MbArgs &, int blk0, int p) { return (size_t)(blk0 + p) * 16; }
+    __device__ static int want(int j, int) { return j; }
+    __device__ static size_t piece2_off(const MbArgs &, int blk0, int p) { return (size_t)blk0 * 4 + (size_t)p * 16; }
+    __device__ static int want2(int j, int) { return j; }
+    __device__ static void load_meta(const MbArgs &a, size_t row, int blk0, int nblk, Raw &r) {
+        typename MQ4x<WITH_MIN>::Raw t;
+        MQ4x<WITH_MIN>::load_meta(a, row, blk0, nblk, t);
+#pragma unroll
+        for (int i = 0; i < NV; i++) r.m[i] = t.m[i];
+    }
+    __device__ static int4v operand(const Raw &r, int u, int h) {
+        const uint32_t bits = r.q2[u >> 2][u & 3] >> (16 * h);
+        int4v b;
+#pragma unroll
+        for (int i = 0; i < 4; i++) // four bits to bit 4 of four bytes: t * 0x00204081 puts bit i at bit 8 i
+            b[i] = (int)(((r.q[u][i] >> (4 * h)) & 0x0F0F0F0Fu) | (((((bits >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4));
+        return b;
+    }
+    __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
+        if (WITH_MIN) {
+            const uint32_t v = r.m[u >> 2][u & 3];
+            d = f16lo(v);
+            mo = f16hi(v);
+        } else {
+            const uint32_t v = r.m[u >> 3][(u >> 1) & 3];
+            d = (u & 1) ? f16hi(v) : f16lo(v);
+            mo = -16.0f * d;
+        }
+    }
+};
+
 template <class T>
 __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
     extern __shared__ float lds_f[];
@@ -187,7 +304,8 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
     float *sgs = lds_f;                    // [block of the row][h][4]: group scales of vectors h, h+2, h+4, h+6
     float *xss = sgs + (size_t)nblk * 8;   // same layout: plain sums of x over the group (contiguous with sgs)
     float *red = xss + (size_t)nblk * 8;   // [wave][vector][row]
-    u32x4 *patch = reinterpret_cast<u32x4 *>(red + (size_t)S * MAX_BATCH * 32) + (size_t)wave * 32 * T::NP; // this wave's 32 x NP pieces
+    u32x4 *patch = reinterpret_cast<u32x4 *>(red + (size_t)S * MAX_BATCH * 32) + (size_t)wave * 32 * (T::NP + T::NP2); // this wave's 32 x NP pieces
+    u32x4 *patch2 = patch + 32 * T::NP;                                                                              // and 32 x NP2 of the qh plane
 
     // scales and sums of all vectors -> LDS (already in the order the lanes read them).  Requesting the waves' first
     // chunks before this barrier instead of after it was slower (2.70 against 2.54 ms per batched 7B step): nobody
@@ -224,6 +342,16 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
             const int gr = row0 + r < a.n_rows ? row0 + r : a.n_rows - 1;
             stage[i] = ldg16(a.codes + (size_t)gr * a.codes_pitch + T::piece_off(a, blk0, pc));
         }
+        constexpr int NP2 = T::NP2, NI2 = (32 * NP2 + 63) / 64;
+        u32x4 stage2[NI2 > 0 ? NI2 : 1];
+        if constexpr (NP2 > 0) {
+#pragma unroll
+            for (int i = 0; i < NI2; i++) {
+                const int idx = i * 64 + lane, r = idx / NP2, pc = idx % NP2;
+                const int gr = row0 + r < a.n_rows ? row0 + r : a.n_rows - 1;
+                stage2[i] = ldg16(a.qh + (size_t)gr * a.qh_pitch + T::piece2_off(a, blk0, pc));
+            }
+        }
         typename T::Raw raw;
         T::load_meta(a, (size_t)row, blk0, nblk, raw);
 #pragma unroll
@@ -231,16 +359,43 @@ __global__ void __launch_bounds__(512, 4) gemv_mb_kernel(MbArgs a) {
             const int idx = i * 64 + lane, r = idx / NP, pc = idx % NP;
             patch[r * NP + (pc ^ (r & (NP - 1)))] = stage[i]; // rotated per row: the reads below spread over the banks
         }
+        if constexpr (NP2 > 0) {
+#pragma unroll
+            for (int i = 0; i < NI2; i++) {
+                const int idx = i * 64 + lane, r = idx / NP2, pc = idx % NP2;
+                patch2[r * NP2 + (pc ^ (r & (NP2 - 1)))] = stage2[i];
+            }
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the wave's LDS writes have landed
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
         for (int j = 0; j < T::NQ; j++) raw.q[j] = patch[n * NP + (T::want(j, h) ^ (n & (NP - 1)))];
+        if constexpr (NP2 > 0) {
+#pragma unroll
+            for (int j = 0; j < T::NQ2; j++) raw.q2[j] = patch2[n * NP2 + (T::want2(j, h) ^ (n & (NP2 - 1)))];
+        }
         // 3. one MFMA per block; the lane scales and adds its four vectors
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
-            if (u < nu) {
+            if constexpr (T::RUNS16) {
+                if (u < nu) { // a scale per half block: two products, each with the other half's codes as zeros
+                    const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    const int4v codes = T::operand(raw, u, h), none = {0, 0, 0, 0};
+                    const int g = blk0 + u;
+                    const float4 sg4 = *reinterpret_cast<const float4 *>(sgs + (size_t)(g * 2 + h) * 4);
+                    const float sgv[4] = {sg4.x, sg4.y, sg4.z, sg4.w};
+#pragma unroll
+                    for (int hh = 0; hh < 2; hh++) {
+                        const int16v D = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[u], h == hh ? codes : none, zero, 0, 0, 0);
+                        const float d = T::coef16(raw, u, hh);
+#pragma unroll
+                        for (int bi = 0; bi < 4; bi++)
+                            acc[bi] = fmaf(d * sgv[bi], recombine4(D[4 * bi], D[4 * bi + 1], D[4 * bi + 2], D[4 * bi + 3]), acc[bi]);
+                    }
+                }
+            } else if (u < nu) {
                 const int16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 const int16v D = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[u], T::operand(raw, u, h), zero, 0, 0, 0);
                 float d, mo;
@@ -466,7 +621,7 @@ int launch_mb(axq_ctx *ctx, MbArgs a, uint8_t *sc, const float *x, int xmode, co
     if (splits < 2) a.ypart = nullptr;
     const unsigned smax = mb_max_waves();
     const unsigned S = (unsigned)a.chunks_per_split < smax ? (unsigned)a.chunks_per_split : smax;
-    const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float) + (size_t)S * 32 * T::NP * 16;
+    const size_t lds = ((size_t)(a.k / 32) * 16 + (size_t)S * MAX_BATCH * 32) * sizeof(float) + (size_t)S * 32 * (T::NP + T::NP2) * 16;
     if (lds > 64 * 1024) {
         const int st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_mb_kernel<T>), mb_lds_mask<T>(), 160 * 1024);
         if (st != AXQ_OK) return st; // the refusal is the call's error: nothing is launched into it
@@ -497,8 +652,8 @@ int gemv_batch_in(axq_ctx *ctx, uint8_t *sc, const axq_weight *w, const float *x
                   const float *bias, const float *resid, float *y, int next_even_odd, const float *next_aux) {
     const int k = (int)w->k;
     MbArgs a;
-    a.codes = w->codes; a.meta = w->meta;
-    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch;
+    a.codes = w->codes; a.meta = w->meta; a.qh = w->qh;
+    a.codes_pitch = w->codes_pitch; a.meta_pitch = w->meta_pitch; a.qh_pitch = w->qh_pitch;
     a.xa = sc; a.xsg = reinterpret_cast<float *>(sc + (size_t)32 * k);
     a.bias = bias; a.resid = resid; a.y = y;
     a.ypart = w->n_rows <= AXQ_BATCH_SPLIT_ROWS ? reinterpret_cast<float *>(sc + (size_t)34 * AXQ_BATCH_MAX_K) : nullptr;
@@ -509,6 +664,10 @@ int gemv_batch_in(axq_ctx *ctx, uint8_t *sc, const axq_weight *w, const float *x
     case AXQ_Q4_1: st = launch_mb<MQ4x<true>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
     case AXQ_Q8_0: st = launch_mb<MQ80>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
     case AXQ_Q4_K: st = launch_mb<MQ4K>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q5_K: st = launch_mb<MQ5K>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q6_K: st = launch_mb<MQ6K>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q5_0: st = launch_mb<MQ5x<false>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
+    case AXQ_Q5_1: st = launch_mb<MQ5x<true>>(ctx, a, sc, x, xmode, aux, eps, next_even_odd, next_aux); break;
     default: return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "Invalid quantization type: %d", w->type);
     }
     if (st != AXQ_OK) return st;
@@ -522,7 +681,10 @@ int gemv_batch_in(axq_ctx *ctx, uint8_t *sc, const axq_weight *w, const float *x
 bool axq_dev_gemv_batch_covers(const axq_weight *w, int batch) {
     if (batch < 2 || batch > MAX_BATCH) return false;
     if (w->k % 256 != 0 || w->k > AXQ_BATCH_MAX_K) return false; // 34 k bytes of scratch: the context's x buffer holds that much
-    return w->type == AXQ_Q4_0 || w->type == AXQ_Q4_1 || w->type == AXQ_Q8_0 || w->type == AXQ_Q4_K;
+    switch (w->type) {
+    case AXQ_Q4_0: case AXQ_Q4_1: case AXQ_Q5_0: case AXQ_Q5_1: case AXQ_Q8_0: case AXQ_Q4_K: case AXQ_Q5_K: case AXQ_Q6_K: return true;
+    default: return false;
+    }
 }
 
 // Where a caller that prepares the operands of the call with w itself (axq_store_packed, then xmode = AXQ_X_PACKED) has
@@ -608,7 +770,7 @@ int axq_gemv_f32_static(axq_ctx *ctx, const axq_weight *w, const float *x, int b
     if (w->k % 256 != 0)
         return axq_fail(ctx, AXQ_ERR_SHAPE_MISMATCH, "Shape mismatch: axq_gemv_f32_static takes k a multiple of 256, got %lld", (long long)w->k);
     if (!axq_dev_gemv_batch_covers(w, batch))
-        return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "axq_gemv_f32_static covers Q4_0, Q4_1, Q8_0 and Q4_K weights (got type %d)", w->type);
+        return axq_fail(ctx, AXQ_ERR_INVALID_QUANT_TYPE, "axq_gemv_f32_static covers the block types (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K), not type %d", w->type);
     uint8_t *ptr = (ctx->device >= 0 && ctx->device < MAX_DEVICES) ? g_scratch_ptr[ctx->device] : nullptr;
     if (!ptr) return axq_fail(ctx, AXQ_ERR_DRIVER, "the static GEMV scratch of device %d was not set up (devices 0..%d have one)", ctx->device, MAX_DEVICES - 1);
     AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);

@@ -177,7 +177,7 @@ AXQ_API int axq_gemv_f32(axq_ctx *ctx, const axq_weight *w, const float *x, int 
  * reference: it exists for code under HIP graph capture, tight serving loops and harnesses that forbid
  * hipMalloc.  It allocates nothing: the scratch of its kernels (the batch's matrix-pipe operands and the
  * partial sums of a split K, 1,605,632 bytes) is a device array inside the library, one copy per GPU, held
- * until the process ends.  Limits: Q4_0, Q4_1, Q8_0 or Q4_K weights, k a multiple of 256 up to 16384, any
+ * until the process ends.  Limits: weights of a block type (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K), k a multiple of 256 up to 16384, any
  * n_rows, batch 2..8; anything else is refused with AXQ_ERR_SHAPE_MISMATCH / AXQ_ERR_INVALID_QUANT_TYPE.
  * x, bias (may be NULL) and y are device pointers; the launches go to the context's stream and nothing is
  * synchronised.  Every call on a GPU shares that GPU's array (it needs no clearing: each call writes what it
@@ -232,7 +232,7 @@ AXQ_API int axq_model_forward(axq_model *m, int32_t token, float *logits, int32_
 /* forward_with_cache (llama.rs:731-762) for n >= 1 tokens at once (a prompt): appends n positions to the
  * cache; logits / next_token are those of the last position.  Tokens before the last go through the
  * layers together: from 32 on through the GEMM (f32 activations, K a multiple of 64), fewer up to eight
- * per pass over the weights when every linear of the layers is Q4_0, Q4_1, Q8_0 or Q4_K with K a
+ * per pass over the weights when every linear of the layers is of a block type (Q4_0 ... Q6_K) with K a
  * multiple of 256 up to 16384, else one by one; results agree with n calls of axq_model_forward to
  * rounding (sums are taken in another order). */
 AXQ_API int axq_model_forward_tokens(axq_model *m, const int32_t *tokens, int n, float *logits, int32_t *next_token);

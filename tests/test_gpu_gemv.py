@@ -164,7 +164,7 @@ def test_gemv_shape_errors(ctx):
 
 
 # ---- small batches: one pass over the weights for up to eight vectors (v_mfma_i32_32x32x32_i8 path)
-@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q8_0, o.Q4_K])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q4_K, o.Q5_K, o.Q6_K])
 @pytest.mark.parametrize("batch,n,k", [(2, 32, 512), (3, 100, 1024), (8, 96, 4096), (8, 33, 512), (11, 64, 2048), (16, 40, 4096),
                                        (2, 32, 256), (8, 33, 768), (8, 40, 11008), (5, 64, 14336), (8, 32, 16384)])
 def test_small_batch_reads_weights_once(ctx, qtype, batch, n, k):

@@ -106,7 +106,7 @@ def test_static_entry_point_refuses_what_it_cannot_hold(ctx):
     wide = q.DeviceWeight.quantize(gen_weight(rng, 2, 16384 + 256), q.QuantType.Q8_0, ctx)
     assert call(wide, 4) == -3
     assert b"static scratch" in lib.axq_last_error(ctx.handle)
-    other = q.DeviceWeight.quantize(gen_weight(rng, 8, 512), q.QuantType.Q5_1, ctx)
+    other = q.DeviceWeight.quantize(gen_weight(rng, 8, 512), q.QuantType.F16, ctx)  # not a block type
     assert call(other, 4) == -2                                                      # AXQ_ERR_INVALID_QUANT_TYPE
     ragged = q.DeviceWeight.quantize(gen_weight(rng, 8, 288), q.QuantType.Q8_0, ctx)
     assert call(ragged, 4) == -3                                                     # a shape limit: k % 256
