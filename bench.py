@@ -402,6 +402,9 @@ def main():
     ap.add_argument("--read-sweep", action="store_true",
                     help="instead of the benchmark: time a read-only kernel over the headline weight in every launch shape, "
                          "and print the table")
+    ap.add_argument("--gemv-table", action="store_true",
+                    help="instead of the benchmark, for kernel-trace profiles: the one-vector and batch-8 GEMVs of every block "
+                         "type at 14336x4096 and 4096x14336 as plain stream launches over their rings, one line each")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path is built or measured)")
@@ -419,6 +422,14 @@ def main():
         return
     if args.read_sweep:
         read_sweep(ctx, args.steps, args.warmup)
+        return
+    if args.gemv_table:
+        for qt in (T.Q4_K, T.Q5_K, T.Q6_K, T.Q4_0, T.Q4_1, T.Q5_0, T.Q5_1, T.Q8_0):
+            for n, k in ((N_HEAD, K_HEAD), (K_HEAD, N_HEAD)):
+                for b in (1, 8):
+                    r, ws, _, xd, yd = gemv_case(ctx, qt, n, k, b, args.steps, 50, graph=False)
+                    free_case(ctx, ws, xd, yd)
+                    print(f"{r['type']} [{n},{k}] b={b}: {r['us_per_step']:.2f} us, {r['gbps']:.0f} GB/s, ring of {r['ring_copies']}", flush=True)
         return
 
     # ---- headline: Q4_K GEMV 14336 x 4096, batch 1
