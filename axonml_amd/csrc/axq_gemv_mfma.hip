@@ -112,6 +112,7 @@ __device__ inline uint32_t ld2(const uint8_t *base, uint32_t off) { return __bui
 // ---------------------------------------------------------------------------
 struct DQ4K {
     struct Raw { uint4 q0, q1, h; };
+    static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 8; // w = d*sc*(q - 8) + (8*d*sc - dmin*m)
@@ -191,6 +192,7 @@ struct DQ4K {
 // 256 bytes) but fetched once per round with the headers, as part of the record that goes through LDS.
 struct DQ5K {
     struct Raw { uint4 q0, q1, b0, b1, h; };
+    static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = true;
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 16; // w = d*sc*(q - 16) + (16*d*sc - dmin*m)
@@ -277,6 +279,7 @@ struct DQ5K {
 template <bool WITH_MIN>
 struct DQ4x {
     struct Raw { uint4 q[2]; uint32_t m[2]; };
+    static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = true; // dword w of a block: low nibbles = elements 8w+{0,2,4,6}, high = 8w+{1,3,5,7}
     static constexpr int CENTRE = 8;
@@ -338,6 +341,7 @@ struct DQ4x {
 template <bool WITH_MIN>
 struct DQ5x {
     struct Raw { uint4 q[2]; uint32_t qh[2]; uint32_t m[2]; };
+    static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 16;
@@ -406,6 +410,9 @@ struct DQ5x {
 // Q8_0: four 16-byte vectors of int8 codes per lane per pass = two blocks; the codes are the B operand as they are.
 struct DQ80 {
     struct Raw { uint4 q[4]; uint32_t m[2]; };
+    // K beyond eight slices: the split-wave kernel with two slices per weight wave (4096 x 14336: 14.0 against 19.0 us on the
+    // kernel with per-wave staging, whose ring holds three of these steps; every other type is ahead there, 8.9 against 9.7 us for Q4_K)
+    static constexpr bool TWO_SLICE_WAVES = true;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 0;
@@ -472,6 +479,7 @@ struct DQ80 {
 // hand each other the two pieces they need when the step is folded.  The codes go in as signed bytes q - 32.
 struct DQ6K {
     struct Raw { uint4 l0, l1, hq; uint32_t sc; uint32_t d; };
+    static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = true, OWN_META_PIECES = true;
     static constexpr bool PERM_A = false;
     static constexpr int CENTRE = 0;
@@ -1142,7 +1150,7 @@ __device__ unsigned int axq_stamp_launch;
 // registers when the wave starts (the file is compiled with -amdgpu-kernarg-preload-count), so the pointers the first
 // loads need are there without a trip to memory.
 // ---------------------------------------------------------------------------
-template <class T, int NB, int NB0, int NS>
+template <class T, int NB, int NB0, int NS, int KS = 1>
 __global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__ x, const uint8_t *__restrict__ codes,
                                                                const uint8_t *__restrict__ meta, uint32_t cp, uint32_t mp, int n_rows, int k,
                                                                int steps, int flags, float eps, float *__restrict__ y,
@@ -1224,6 +1232,89 @@ __global__ void __launch_bounds__(1024) gemv_sw_kernel(const float *__restrict__
         STAMP(2);
         lds_only_barrier(); // x is staged
         STAMP(3);
+    } else if constexpr (KS == 2) {
+        // ---- weight waves that cover two K slices each (K beyond eight slices, one row group): wave ww has slices ww
+        // and ww + W, its steps go through them in turn -- ring slot b holds a step of slice b % 2, a round of four steps is
+        // two row steps -- and the x operands of a step are fetched from LDS when it is folded (two sets do not fit the
+        // registers beside the ring).
+        static_assert(NB == 4 && NB0 <= 4, "ring slot parity = slice");
+        const int ww = wave - NS, W = (S + 1) >> 1;
+        const int blk = lane >> 2, j = lane & 3;
+        const bool live1 = ww + W < S; // an odd count of slices: the last wave has one, its other steps meet x = 0
+        const int sl[2] = {ww, live1 ? ww + W : ww};
+        const int cq[2] = {(sl[0] << 4) + blk, ((ww + W) << 4) + blk};
+        const int my_t = 2 * steps; // the wave's steps: row step t / 2 of slice t % 2
+        float *red_q[2] = {red + j * red_stride + sl[0] * 4 + (lane >> 4), red + j * red_stride + sl[1] * 4 + (lane >> 4)};
+        uint4 *wmeta = lds_raw + n16 + 1 + 4 + (wg_rows * red_stride) / 4 + ww * 64 * NM;
+        typename T::Raw buf[NB];
+        uint4 hm[NM];
+        LaneOff lo[2];
+        T::lane_offsets(k, cq[0], lo[0]);
+        T::lane_offsets(k, cq[1], lo[1]);
+        const int wg_row0 = blockIdx.x * wg_rows;
+        const Bases bases = {codes + (size_t)wg_row0 * cp, meta + (size_t)wg_row0 * mp, qhp + (size_t)wg_row0 * qp};
+        const int rl_last = n_rows - 1 - wg_row0; // rows relative to the workgroup's first
+        // the round's records: record 4 b + j = row j of ring slot b's row step, the slot's slice
+        uint32_t moff[NM], mpitch[NM];
+        const uint8_t *mbase[NM];
+        int mrow[NM];
+        {
+#pragma unroll
+            for (int i = 0; i < NM; i++) {
+                const int flat = i * 64 + lane;
+                const int rec = flat / CPR < 4 * NB ? flat / CPR : 4 * NB - 1; // lanes beyond the round's records repeat its last
+                const int slot = rec >> 2;
+                bool from_qh;
+                moff[i] = (uint32_t)record_piece<T>(k, sl[slot & 1], flat % CPR, from_qh);
+                mbase[i] = from_qh ? bases.qh : bases.meta;
+                mpitch[i] = from_qh ? qp : mp;
+                mrow[i] = (slot >> 1) * 4 + (rec & 3);
+            }
+        }
+        auto request = [&](int t, int b) { // b = t % NB
+            const int tt = t < my_t ? t : b; // steps past the end re-read the first round's
+            int rl = 4 * (tt >> 1) + j;
+            rl = rl < rl_last ? rl : rl_last;
+            const RowOff ro = {(uint32_t)rl * cp, (uint32_t)rl * mp, (uint32_t)rl * qp};
+            if (b == 0) {
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    int rlm = 4 * (tt >> 1) + mrow[i]; // rows past the workgroup's steps are the next workgroup's: read, not used
+                    rlm = rlm < rl_last ? rlm : rl_last;
+                    hm[i] = ld16(mbase[i], (uint32_t)rlm * mpitch[i] + moff[i]);
+                }
+            }
+            T::load_codes(bases, ro, lo[b & 1], buf[b]);
+        };
+#pragma unroll
+        for (int b = 0; b < NB0; b++) request(b, b);
+        lds_only_barrier(); // x is staged
+#pragma unroll
+        for (int b = NB0; b < NB; b++) request(b, b);
+        const bool writer = (blk & 3) == 3;
+        auto fold = [&](int b, int t) {
+            if (b == 0) {
+#pragma unroll
+                for (int i = 0; i < NM; i++) wmeta[i * 64 + lane] = hm[i];
+            }
+            XOp xo;
+            fetch_xop<T>(wplanes, wgrp, kpad, k, j, cq[b & 1], xo);
+            T::set_meta(buf[b], reinterpret_cast<const uint8_t *>(wmeta) + (b * 4 + j) * MSB, blk, cq[b & 1]);
+            const float tot = sum_within_row(T::dot(buf[b], xo, cq[b & 1]));
+            if (writer && ((b & 1) == 0 || live1)) red_q[b & 1][(t >> 1) * 4 * red_stride] = tot;
+        };
+        const int rounds = (my_t + NB - 1) / NB;
+        int step = 0;
+        for (int round = 0; round < rounds - 1; round++, step += NB) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                fold(b, step + b);
+                request(step + NB + b, b);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+            if (step + b < my_t) fold(b, step + b);
     } else {
         // ---- weight waves
         const int ww = wave - NS;
@@ -1493,6 +1584,42 @@ int launch_sw(axq_ctx *ctx, const DpArgs &a) {
     }
 }
 
+// The same kernel for K beyond eight slices (up to sixteen): eight split waves, and weight waves of two slices each.  Taken
+// by the types that say so (TWO_SLICE_WAVES).
+template <class T>
+int launch_sw2(axq_ctx *ctx, const DpArgs &a) {
+    if constexpr (!T::TWO_SLICE_WAVES) {
+        return 0;
+    } else {
+    constexpr int NS = 8;
+    static std::atomic<uint64_t> lds_allowed{0};
+    static const bool off = getenv("AXQ_GEMV_SW2") && getenv("AXQ_GEMV_SW2")[0] == '0'; // development knob: such K on the kernel with per-wave staging
+    const int S = a.S;
+    if (off || S <= 8 || S > 16 || (a.k >> 3) > 4 * 64 * NS) return 0;
+    if (T::meta_row_bytes(a.k) % 16 != 0 || a.meta_pitch % 16 != 0 || T::meta_row_bytes(a.k) < 16) return 0;
+    const int rowsteps = (a.n_rows + 3) / 4;
+    const int cus = ctx->prop.multiProcessorCount * ctx->gemv_wgs_per_cu;
+    int steps = (rowsteps + cus - 1) / cus;
+    if (a.ymode == AXQ_Y_SWIGLU && (steps & 1)) steps++; // a workgroup must hold whole gate/up groups of 8 rows
+    if (steps < 2 || steps > 64) return 0;               // a ring of four steps = two row steps at least
+    const unsigned grid = (unsigned)((rowsteps + steps - 1) / steps);
+    const int W = (S + 1) / 2;
+    const int cpr = T::META_SLICE_BYTES / 16, nm = (4 * 4 * cpr + 63) / 64;
+    const size_t lds = axq_split_bytes(a.k) + 16 + 64 + (size_t)steps * 4 * 4 * S * sizeof(float) + (size_t)W * nm * 1024;
+    if (lds > 160 * 1024) return 0;
+    const unsigned block = (unsigned)(64 * (W + NS));
+    const int flags = a.mode | (a.ymode << 8) | (1 << 16);
+    auto kern = &gemv_sw_kernel<T, 4, 3, NS, 2>;
+    if (lds > 64 * 1024) {
+        const int st = axq_allow_lds(ctx, reinterpret_cast<const void *>(kern), lds_allowed, 160 * 1024);
+        if (st != AXQ_OK) return st;
+    }
+    kern<<<grid, block, lds, ctx->stream>>>(a.x, a.codes, a.meta, (uint32_t)a.codes_pitch, (uint32_t)a.meta_pitch, a.n_rows, a.k, steps, flags,
+                                            a.eps, a.y, a.bias, a.aux, a.qh, (uint32_t)a.qh_pitch);
+    return 1;
+    }
+}
+
 // 1 = launched, 0 = the shape is not this kernel's, < 0 = status
 template <class T>
 int launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *xq, int mode, const float *aux, float eps,
@@ -1528,7 +1655,9 @@ int launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *
     if (lds > 160 * 1024) return 0;
     static const bool sw_off = getenv("AXQ_GEMV_SW") && getenv("AXQ_GEMV_SW")[0] == '0'; // development knob: no split waves
     if (!xq && !sw_off) {
-        const int r = launch_sw<T>(ctx, a);
+        int r = launch_sw<T>(ctx, a);
+        if (r != 0) return r;
+        r = launch_sw2<T>(ctx, a);
         if (r != 0) return r;
     }
     if (!xq) {

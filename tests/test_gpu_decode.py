@@ -333,6 +333,24 @@ def test_the_two_prompt_attention_kernels_agree(ctx, monkeypatch, over, n_first,
         assert np.abs(af - bf).max() <= 2.0 ** -9 * np.abs(af).max()  # isolated one-ulp f16 roundings at most
 
 
+def test_wide_layers_in_q8_0(ctx):
+    """Hidden and feed-forward widths beyond 8192 in Q8_0: gate/up (fused RMSNorm and SwiGLU, K = 9216: nine K slices, an odd
+    count) and down (K = 8448: the ninth slice a quarter full) take the split-wave GEMV whose weight waves cover two
+    slices each.  One layer, a few positions, against the oracle."""
+    c = tiny_config(hidden_size=9216, intermediate_size=8448, num_layers=1, num_heads=8, num_kv_heads=2, head_dim=64, max_seq_len=16)
+    w = random_weights(c, 5, qtype=o.Q8_0, std=0.02)
+    cpu, gpu = load_oracle(c, w), load_gpu(ctx, c, w)
+    tok = 7
+    for pos in range(5):
+        c_next, c_logits = cpu.forward(tok, pos)
+        g_next, g_logits = gpu.forward(tok)
+        assert max_rel_err(g_logits, c_logits, DECODE_FLOOR) <= DECODE_RTOL, pos
+        assert g_next == c_next, pos
+        tok = c_next
+    gpu.close()
+    cpu.close()
+
+
 def test_a_linear_set_again_in_another_block_type(ctx):
     """o, down and the lm_head have their slots to themselves: setting one again in another type replaces it (and drops
     the recorded step, which holds the old weight's address); the walk then follows the oracle with the new weights."""
