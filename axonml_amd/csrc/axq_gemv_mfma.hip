@@ -112,6 +112,7 @@ __device__ inline uint32_t ld2(const uint8_t *base, uint32_t off) { return __bui
 // ---------------------------------------------------------------------------
 struct DQ4K {
     struct Raw { uint4 q0, q1, h; };
+    static constexpr bool X_REQUESTS_FIRST = true; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = false;
@@ -192,6 +193,7 @@ struct DQ4K {
 // 256 bytes) but fetched once per round with the headers, as part of the record that goes through LDS.
 struct DQ5K {
     struct Raw { uint4 q0, q1, b0, b1, h; };
+    static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = true;
     static constexpr bool PERM_A = false;
@@ -279,6 +281,7 @@ struct DQ5K {
 template <bool WITH_MIN>
 struct DQ4x {
     struct Raw { uint4 q[2]; uint32_t m[2]; };
+    static constexpr bool X_REQUESTS_FIRST = true; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = true; // dword w of a block: low nibbles = elements 8w+{0,2,4,6}, high = 8w+{1,3,5,7}
@@ -341,6 +344,7 @@ struct DQ4x {
 template <bool WITH_MIN>
 struct DQ5x {
     struct Raw { uint4 q[2]; uint32_t qh[2]; uint32_t m[2]; };
+    static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
     static constexpr bool PERM_A = false;
@@ -410,6 +414,7 @@ struct DQ5x {
 // Q8_0: four 16-byte vectors of int8 codes per lane per pass = two blocks; the codes are the B operand as they are.
 struct DQ80 {
     struct Raw { uint4 q[4]; uint32_t m[2]; };
+    static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     // K beyond eight slices: the split-wave kernel with two slices per weight wave (4096 x 14336: 14.0 against 19.0 us on the
     // kernel with per-wave staging, whose ring holds three of these steps; every other type is ahead there, 8.9 against 9.7 us for Q4_K)
     static constexpr bool TWO_SLICE_WAVES = true;
@@ -479,6 +484,7 @@ struct DQ80 {
 // hand each other the two pieces they need when the step is folded.  The codes go in as signed bytes q - 32.
 struct DQ6K {
     struct Raw { uint4 l0, l1, hq; uint32_t sc; uint32_t d; };
+    static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = true, OWN_META_PIECES = true;
     static constexpr bool PERM_A = false;
@@ -907,6 +913,24 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dp_kernel(DP
     }
 }
 
+#ifdef AXQ_STAMPS
+// Development builds only (-DAXQ_STAMPS): every wave keeps wall-clock stamps (100 MHz) of its progress in LDS (the last
+// 4 KB of the 160) and copies them out when it ends, into a buffer the host has set with axq_debug_set_stamps:
+// [launch % 4][workgroup][wave (16)][slot (16)].
+__device__ unsigned long long *axq_stamps;
+__device__ unsigned int axq_stamp_launch;
+#define STAMP_INIT() unsigned long long *st_lds_ = reinterpret_cast<unsigned long long *>(reinterpret_cast<uint8_t *>(lds_raw) + 156 * 1024) + wave * 16; \
+                     if (lane < 16) st_lds_[lane] = 0
+#define STAMP(slot) do { if (lane == 0) st_lds_[slot] = wall_clock64(); } while (0)
+#define STAMP_END() do { unsigned long long *g_ = axq_stamps; if (g_ && lane < 16) { \
+                         g_[((((size_t)(*(volatile unsigned int *)&axq_stamp_launch & 3) * gridDim.x + blockIdx.x) * 16 + wave) * 16) + lane] = st_lds_[lane]; } \
+                         __syncthreads(); if (g_ && blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&axq_stamp_launch, 1u); } while (0)
+#else
+#define STAMP_INIT() do {} while (0)
+#define STAMP(slot) do {} while (0)
+#define STAMP_END() do {} while (0)
+#endif
+
 // ---------------------------------------------------------------------------
 // The same kernel with x staged per wave.  Timestamps of the kernel above showed its critical path: x requested
 // 0.4 us after entry, split by all waves together, two workgroup barriers (every wave waits for the one that was held
@@ -931,6 +955,8 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     const int nwaves = a.G * a.S;
     const int k0 = slice * SLICE_K;
     const int klen = a.k - k0 < SLICE_K ? a.k - k0 : SLICE_K; // a multiple of 64
+    STAMP_INIT();
+    STAMP(0);
 
     // 1. x first: this wave's slice, two 8-element tasks per lane (and the norm weights of a fused RMSNorm)
     const bool live0 = lane * 8 < klen, live1 = (lane + 64) * 8 < klen; // whole quads of lanes
@@ -1001,10 +1027,14 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
             T::load(bases, ro, lo, buf[b]);
         }
     };
-    constexpr int NB0 = NB < 2 ? NB : 2; // steps requested before x is split: enough to start the stream, few enough that
-                                         // the wave is not held up issuing them when its x arrives
+    // One step requested before x is split (two: 9.3 against 9.1 us at Q4_K 4096 x 14336; the stamps showed the workgroup's
+    // last six waves standing 2.5-3.5 us at their first loads, behind the first eight waves' x and weight requests).  Types
+    // with two loads per step gain again when every wave's x requests are out before any weight request (8.6-8.7 us).
+    constexpr int NB0 = 1;
+    if constexpr (T::X_REQUESTS_FIRST) __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int b = 0; b < NB0; b++) request(b, b);
+    STAMP(1);
     // 3. x -> split form in the wave's own LDS region -> this lane's A operands
     {
         auto unpack = [](const uint4 &lo4, const uint4 &hi4, float (&v)[8]) {
@@ -1046,10 +1076,12 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
         axq_split8(xv[0], lane, live0, wplanes, wgrp, SLICE_K);
         axq_split8(xv[1], lane + 64, live1, wplanes, wgrp, SLICE_K);
     }
+    STAMP(2);
     XOp xo;
     fetch_xop<T>(wplanes, wgrp, SLICE_K, klen, j, blk, xo); // same wave: LDS serves its stores and loads in order
 #pragma unroll
     for (int b = NB0; b < NB; b++) request(b, b);
+    STAMP(4);
 
     // 4. fold the steps through the ring
     const bool writer = (blk & 3) == 3;
@@ -1064,6 +1096,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
         }
         float tot = sum_within_row(T::dot(buf[b], xo, c));
         if (writer) red_lane[step * red_step] = tot;
+        STAMP(5 + (step < 8 ? step : 8));
     };
     const int rounds = (a.steps + NB - 1) / NB;
     int step = 0;
@@ -1080,6 +1113,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
 
     // partial sums -> y, in a fixed order
     __syncthreads();
+    STAMP(14);
     const int nthreads = 64 * nwaves;
     const int wg_rows = a.G * rows_per_group;
     float inv = 1.0f;
@@ -1107,6 +1141,8 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
                 a.y[(blockIdx.x * wg_rows >> 1) + t] = (g * (1.0f / (1.0f + expf(-g)))) * u;
             }
         }
+        STAMP(15);
+        STAMP_END();
         return;
     }
     for (int t = tid; t < wg_rows; t += nthreads) {
@@ -1116,25 +1152,10 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
             a.y[row] = a.bias ? tot + a.bias[row] : tot;
         }
     }
+    STAMP(15);
+    STAMP_END();
 }
 
-#ifdef AXQ_STAMPS
-// Development builds only (-DAXQ_STAMPS): every wave keeps wall-clock stamps (100 MHz) of its progress in LDS (the last
-// 4 KB of the 160) and copies them out when it ends, into a buffer the host has set with axq_debug_set_stamps:
-// [launch % 4][workgroup][wave (16)][slot (16)].
-__device__ unsigned long long *axq_stamps;
-__device__ unsigned int axq_stamp_launch;
-#define STAMP_INIT() unsigned long long *st_lds_ = reinterpret_cast<unsigned long long *>(reinterpret_cast<uint8_t *>(lds_raw) + 156 * 1024) + wave * 16; \
-                     if (lane < 16) st_lds_[lane] = 0
-#define STAMP(slot) do { if (lane == 0) st_lds_[slot] = wall_clock64(); } while (0)
-#define STAMP_END() do { unsigned long long *g_ = axq_stamps; if (g_ && lane < 16) { \
-                         g_[((((size_t)(*(volatile unsigned int *)&axq_stamp_launch & 3) * gridDim.x + blockIdx.x) * 16 + wave) * 16) + lane] = st_lds_[lane]; } \
-                         __syncthreads(); if (g_ && blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&axq_stamp_launch, 1u); } while (0)
-#else
-#define STAMP_INIT() do {} while (0)
-#define STAMP(slot) do {} while (0)
-#define STAMP_END() do {} while (0)
-#endif
 
 // ---------------------------------------------------------------------------
 // The kernel with waves of two kinds.  Whoever splits x cannot request weights meanwhile, and whoever stands at a
@@ -1478,11 +1499,19 @@ int launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, siz
         // x arrives raw: every wave stages its own slice
         const size_t lds_w = (size_t)(block / 64) * (4 * 1024 + 32 * 16 + (T::ROUND_META ? 16 * T::META_SLICE_BYTES : 0)) + 64 +
                              (size_t)a.G * a.steps * 4 * a.S * 4 * sizeof(float);
+#ifdef AXQ_STAMPS
+        if (lds_w <= 160 * 1024 &&
+#else
         if (lds_w > 64 * 1024 && lds_w <= 160 * 1024 &&
+#endif
             (st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), lds_allowed_w, 160 * 1024)) != AXQ_OK)
             return st;
         if (lds_w <= 160 * 1024) {
+#ifdef AXQ_STAMPS
+            gemv_dpw_kernel<T, NB><<<grid, block, 160 * 1024, ctx->stream>>>(DP_LAUNCH_ARGS(a)); // the stamps live in the last 4 KB
+#else
             gemv_dpw_kernel<T, NB><<<grid, block, lds_w, ctx->stream>>>(DP_LAUNCH_ARGS(a));
+#endif
             return AXQ_OK;
         }
     }
