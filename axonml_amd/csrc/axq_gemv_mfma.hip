@@ -112,6 +112,7 @@ __device__ inline uint32_t ld2(const uint8_t *base, uint32_t off) { return __bui
 // ---------------------------------------------------------------------------
 struct DQ4K {
     struct Raw { uint4 q0, q1, h; };
+    static constexpr bool SPLIT_HELPERS = true; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = true; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
@@ -193,6 +194,7 @@ struct DQ4K {
 // 256 bytes) but fetched once per round with the headers, as part of the record that goes through LDS.
 struct DQ5K {
     struct Raw { uint4 q0, q1, b0, b1, h; };
+    static constexpr bool SPLIT_HELPERS = true; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = true;
@@ -281,6 +283,7 @@ struct DQ5K {
 template <bool WITH_MIN>
 struct DQ4x {
     struct Raw { uint4 q[2]; uint32_t m[2]; };
+    static constexpr bool SPLIT_HELPERS = true; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = true; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
@@ -344,6 +347,7 @@ struct DQ4x {
 template <bool WITH_MIN>
 struct DQ5x {
     struct Raw { uint4 q[2]; uint32_t qh[2]; uint32_t m[2]; };
+    static constexpr bool SPLIT_HELPERS = true; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
@@ -414,6 +418,7 @@ struct DQ5x {
 // Q8_0: four 16-byte vectors of int8 codes per lane per pass = two blocks; the codes are the B operand as they are.
 struct DQ80 {
     struct Raw { uint4 q[4]; uint32_t m[2]; };
+    static constexpr bool SPLIT_HELPERS = false; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     // K beyond eight slices: the split-wave kernel with two slices per weight wave (4096 x 14336: 14.0 against 19.0 us on the
     // kernel with per-wave staging, whose ring holds three of these steps; every other type is ahead there, 8.9 against 9.7 us for Q4_K)
@@ -484,6 +489,7 @@ struct DQ80 {
 // hand each other the two pieces they need when the step is folded.  The codes go in as signed bytes q - 32.
 struct DQ6K {
     struct Raw { uint4 l0, l1, hq; uint32_t sc; uint32_t d; };
+    static constexpr bool SPLIT_HELPERS = false; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = true, OWN_META_PIECES = true;
@@ -1043,8 +1049,8 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     // last six waves standing 2.5-3.5 us at their first loads, behind the first eight waves' x and weight requests).  Types
     // with two loads per step gain again when every wave's x requests are out before any weight request (8.6-8.7 us).
     constexpr int NB0 = 1;
-    if (helped && lane == 0) *ready = 0; // (helpers only exist with the barrier below)
-    if constexpr (T::X_REQUESTS_FIRST) lds_only_barrier();
+    if (helped && lane == 0) *ready = 0;
+    if (T::X_REQUESTS_FIRST || a.H > 0) lds_only_barrier(); // with helpers: the flags are zero before any of them is set
     if (!helper) {
 #pragma unroll
         for (int b = 0; b < NB0; b++) request(b, b);
@@ -1534,7 +1540,7 @@ int launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, siz
             // fourteen or ten weight waves (four on two of the SIMDs, three on the others): two helper waves split x for the last two
             static const bool no_helpers = getenv("AXQ_GEMV_HELPERS") && getenv("AXQ_GEMV_HELPERS")[0] == '0'; // development knob
             DpArgs ah = a;
-            if (T::X_REQUESTS_FIRST && !no_helpers && a.G == 1 && (a.S & 3) == 2 && a.S >= 6 && block + 128 <= 1024 && NB <= T::BIG_NB) ah.H = 2;
+            if (T::SPLIT_HELPERS && !no_helpers && a.G == 1 && (a.S & 3) == 2 && a.S >= 6 && block + 128 <= 1024 && NB <= T::BIG_NB) ah.H = 2;
             const unsigned block_w = block + 64 * (unsigned)ah.H;
 #ifdef AXQ_STAMPS
             gemv_dpw_kernel<T, NB><<<grid, block_w, 160 * 1024, ctx->stream>>>(DP_LAUNCH_ARGS(ah)); // the stamps live in the last 4 KB
