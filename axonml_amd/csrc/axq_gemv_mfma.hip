@@ -46,7 +46,7 @@ struct DpArgs {
     const uint8_t *xq; // x already split into limbs (see stage_x), or NULL: the kernel splits it itself
     float *y;
     int n_rows, k;
-    int S, G, H;   // K slices per pass, row groups per workgroup, helper waves (gemv_dpw_kernel: waves that only split x, for the last H weight waves)
+    int S, G, P;   // K slices per pass, row groups per workgroup, passes over K per lane
     int steps;     // 4-row steps per group
     int mode;      // what x is: AXQ_X_PLAIN, or a vector still to be normalised (see axq_internal.h)
     const float *aux; // AXQ_X_RMSNORM: the norm weights
@@ -55,14 +55,14 @@ struct DpArgs {
 };
 // The kernels take these fields as scalar arguments, the ones the first loads need in front: the first fourteen dwords
 // are preloaded into scalar registers when a wave starts (-amdgpu-kernarg-preload-count), a struct passed by value is not.
-// shape = S | G << 8 | steps << 16, flags = mode | ymode << 8 | H << 16.
+// shape = S | G << 8 | steps << 16, flags = mode | ymode << 8.
 #define DP_KERNEL_PARAMS const float *p_x, const uint8_t *p_codes, const uint8_t *p_meta, uint32_t p_cp, uint32_t p_mp, int p_n_rows, int p_k, \
                          int p_shape, int p_flags, float p_eps, float *p_y, const float *p_bias, const float *p_aux, const uint8_t *p_qh, uint32_t p_qp, \
                          const uint8_t *p_xq
-#define DP_KERNEL_ARGS DpArgs{p_codes, p_meta, p_qh, p_cp, p_mp, p_qp, p_x, p_bias, p_xq, p_y, p_n_rows, p_k, p_shape & 0xFF, (p_shape >> 8) & 0xFF, (p_flags >> 16) & 0xFF, \
+#define DP_KERNEL_ARGS DpArgs{p_codes, p_meta, p_qh, p_cp, p_mp, p_qp, p_x, p_bias, p_xq, p_y, p_n_rows, p_k, p_shape & 0xFF, (p_shape >> 8) & 0xFF, 1, \
                               p_shape >> 16, p_flags & 0xFF, p_aux, p_eps, (p_flags >> 8) & 0xFF}
 #define DP_LAUNCH_ARGS(a) (a).x, (a).codes, (a).meta, (uint32_t)(a).codes_pitch, (uint32_t)(a).meta_pitch, (a).n_rows, (a).k, \
-                          ((a).S | ((a).G << 8) | ((a).steps << 16)), ((a).mode | ((a).ymode << 8) | ((a).H << 16)), (a).eps, (a).y, (a).bias, (a).aux, (a).qh, \
+                          ((a).S | ((a).G << 8) | ((a).steps << 16)), ((a).mode | ((a).ymode << 8)), (a).eps, (a).y, (a).bias, (a).aux, (a).qh, \
                           (uint32_t)(a).qh_pitch, (a).xq
 
 __device__ inline float f16lo(uint32_t v) { return __half2float(__ushort_as_half((unsigned short)(v & 0xFFFF))); }
@@ -112,7 +112,6 @@ __device__ inline uint32_t ld2(const uint8_t *base, uint32_t off) { return __bui
 // ---------------------------------------------------------------------------
 struct DQ4K {
     struct Raw { uint4 q0, q1, h; };
-    static constexpr bool SPLIT_HELPERS = true; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = true; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
@@ -194,7 +193,6 @@ struct DQ4K {
 // 256 bytes) but fetched once per round with the headers, as part of the record that goes through LDS.
 struct DQ5K {
     struct Raw { uint4 q0, q1, b0, b1, h; };
-    static constexpr bool SPLIT_HELPERS = true; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = true;
@@ -283,7 +281,6 @@ struct DQ5K {
 template <bool WITH_MIN>
 struct DQ4x {
     struct Raw { uint4 q[2]; uint32_t m[2]; };
-    static constexpr bool SPLIT_HELPERS = true; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = true; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
@@ -347,7 +344,6 @@ struct DQ4x {
 template <bool WITH_MIN>
 struct DQ5x {
     struct Raw { uint4 q[2]; uint32_t qh[2]; uint32_t m[2]; };
-    static constexpr bool SPLIT_HELPERS = true; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = false, OWN_META_PIECES = false;
@@ -418,7 +414,6 @@ struct DQ5x {
 // Q8_0: four 16-byte vectors of int8 codes per lane per pass = two blocks; the codes are the B operand as they are.
 struct DQ80 {
     struct Raw { uint4 q[4]; uint32_t m[2]; };
-    static constexpr bool SPLIT_HELPERS = false; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     // K beyond eight slices: the split-wave kernel with two slices per weight wave (4096 x 14336: 14.0 against 19.0 us on the
     // kernel with per-wave staging, whose ring holds three of these steps; every other type is ahead there, 8.9 against 9.7 us for Q4_K)
@@ -489,7 +484,6 @@ struct DQ80 {
 // hand each other the two pieces they need when the step is folded.  The codes go in as signed bytes q - 32.
 struct DQ6K {
     struct Raw { uint4 l0, l1, hq; uint32_t sc; uint32_t d; };
-    static constexpr bool SPLIT_HELPERS = false; // gemv_dpw_kernel: helper waves pay (measured per type at 4096 x 14336)
     static constexpr bool X_REQUESTS_FIRST = false; // gemv_dpw_kernel: a barrier between the waves' x requests and their weight requests
     static constexpr bool TWO_SLICE_WAVES = false;
     static constexpr bool RUNS16 = true, OWN_META_PIECES = true;
@@ -955,18 +949,10 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     constexpr int SLICE_K = 1024, REGION16 = (4 * SLICE_K + (SLICE_K / 32) * 16) / 16; // a wave's split x, in 16-byte units
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = a.G * a.S;
-    // Helper waves (a.H of them behind the weight waves, one row group): fourteen waves sit four, four, three and three on
-    // the SIMDs, and a wave's share of the vector ALU work (splitting its 1024 elements of x about 600 instructions,
-    // four folds about 360) makes the SIMDs with four the critical path.  A helper lands on a SIMD with three, splits x
-    // for one of the last a.H weight waves into that wave's region and says so through a flag in LDS; that wave requests
-    // its weights, waits for the flag and folds.
-    const bool helper = wave >= nwaves;
-    const int mine = helper ? nwaves - a.H + (wave - nwaves) : wave; // the weight wave whose K slice this wave splits
-    const bool helped = !helper && wave >= nwaves - a.H;
-    const int g_idx = helper ? 0 : wave / a.S, slice = helper ? mine : wave - g_idx * a.S;
+    const int g_idx = wave / a.S, slice = wave - g_idx * a.S;
     const int blk = lane >> 2, j = lane & 3;
     const int c = (slice << 4) + blk; // this lane's 64-weight chunk of the row
+    const int nwaves = a.G * a.S;
     const int k0 = slice * SLICE_K;
     const int klen = a.k - k0 < SLICE_K ? a.k - k0 : SLICE_K; // a multiple of 64
     STAMP_INIT();
@@ -976,22 +962,18 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     const bool live0 = lane * 8 < klen, live1 = (lane + 64) * 8 < klen; // whole quads of lanes
     const float *xs = a.x + k0 + (live0 ? lane * 8 : (lane & 3) * 8);
     const float *xs1 = a.x + k0 + (live1 ? (lane + 64) * 8 : (lane & 3) * 8);
-    uint4 x0 = {0, 0, 0, 0}, x1 = x0, x2 = x0, x3 = x0;
+    const uint4 x0 = reinterpret_cast<const uint4 *>(xs)[0], x1 = reinterpret_cast<const uint4 *>(xs)[1];
+    const uint4 x2 = reinterpret_cast<const uint4 *>(xs1)[0], x3 = reinterpret_cast<const uint4 *>(xs1)[1];
     uint4 e0 = {0, 0, 0, 0}, e1 = e0, e2 = e0, e3 = e0;
-    if (!helped) {
-        x0 = reinterpret_cast<const uint4 *>(xs)[0]; x1 = reinterpret_cast<const uint4 *>(xs)[1];
-        x2 = reinterpret_cast<const uint4 *>(xs1)[0]; x3 = reinterpret_cast<const uint4 *>(xs1)[1];
-        if (a.mode == AXQ_X_RMSNORM) {
-            const float *es = a.aux + (xs - a.x), *es1 = a.aux + (xs1 - a.x);
-            e0 = reinterpret_cast<const uint4 *>(es)[0]; e1 = reinterpret_cast<const uint4 *>(es)[1];
-            e2 = reinterpret_cast<const uint4 *>(es1)[0]; e3 = reinterpret_cast<const uint4 *>(es1)[1];
-        }
+    if (a.mode == AXQ_X_RMSNORM) {
+        const float *es = a.aux + (xs - a.x), *es1 = a.aux + (xs1 - a.x);
+        e0 = reinterpret_cast<const uint4 *>(es)[0]; e1 = reinterpret_cast<const uint4 *>(es)[1];
+        e2 = reinterpret_cast<const uint4 *>(es1)[0]; e3 = reinterpret_cast<const uint4 *>(es1)[1];
     }
     // 2. the ring: rows past the group's end re-read its first step (cache hits, no HBM traffic)
-    uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw + mine * REGION16);
+    uint8_t *wplanes = reinterpret_cast<uint8_t *>(lds_raw + wave * REGION16);
     uint4 *wgrp = reinterpret_cast<uint4 *>(wplanes + 4 * SLICE_K);
     float *wsum = reinterpret_cast<float *>(lds_raw + nwaves * REGION16); // one float per wave (64 bytes kept)
-    volatile uint32_t *ready = reinterpret_cast<volatile uint32_t *>(wsum) + 16 - a.H + (mine - (nwaves - a.H)); // the spare ones: flags of the helped waves
     float *red = wsum + 16;
     const int rows_per_group = a.steps * 4;
     const int last = a.n_rows - 1;
@@ -1049,15 +1031,12 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
     // last six waves standing 2.5-3.5 us at their first loads, behind the first eight waves' x and weight requests).  Types
     // with two loads per step gain again when every wave's x requests are out before any weight request (8.6-8.7 us).
     constexpr int NB0 = 1;
-    if (helped && lane == 0) *ready = 0;
-    if (T::X_REQUESTS_FIRST || a.H > 0) lds_only_barrier(); // with helpers: the flags are zero before any of them is set
-    if (!helper) {
+    if constexpr (T::X_REQUESTS_FIRST) __builtin_amdgcn_s_barrier();
 #pragma unroll
-        for (int b = 0; b < NB0; b++) request(b, b);
-    }
+    for (int b = 0; b < NB0; b++) request(b, b);
     STAMP(1);
-    // 3. x -> split form in the wave's own LDS region (a helper: in its weight wave's) -> this lane's A operands
-    if (!helped) {
+    // 3. x -> split form in the wave's own LDS region -> this lane's A operands
+    {
         auto unpack = [](const uint4 &lo4, const uint4 &hi4, float (&v)[8]) {
             v[0] = __builtin_bit_cast(float, lo4.x); v[1] = __builtin_bit_cast(float, lo4.y);
             v[2] = __builtin_bit_cast(float, lo4.z); v[3] = __builtin_bit_cast(float, lo4.w);
@@ -1079,7 +1058,7 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
             }
 #pragma unroll
             for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
-            if (lane == 0) wsum[mine] = ss; // read after the final barrier (group 0's waves cover K once)
+            if (lane == 0) wsum[wave] = ss; // read after the final barrier (group 0's waves cover K once)
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 xv[0][i] *= ev[0][i];
@@ -1098,14 +1077,6 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
         axq_split8(xv[1], lane + 64, live1, wplanes, wgrp, SLICE_K);
     }
     STAMP(2);
-    if (helper) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // the split form has landed in LDS
-        if (lane == 0) *ready = 1;
-    } else {
-    if (helped) { // every helper gets here whatever the others do; the bound is for a wave that would otherwise wait for ever
-        for (int spins = 0; *ready == 0 && spins < (1 << 22); spins++) __builtin_amdgcn_s_sleep(2);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    }
     XOp xo;
     fetch_xop<T>(wplanes, wgrp, SLICE_K, klen, j, blk, xo); // same wave: LDS serves its stores and loads in order
 #pragma unroll
@@ -1139,12 +1110,11 @@ __global__ void __launch_bounds__(NB > T::BIG_NB ? 512 : 1024) gemv_dpw_kernel(D
 #pragma unroll
     for (int b = 0; b < NB; b++)
         if (step + b < a.steps) fold(b, step + b); // the last round may be short: its spare slots hold re-reads
-    }
 
     // partial sums -> y, in a fixed order
     __syncthreads();
     STAMP(14);
-    const int nthreads = (int)blockDim.x;
+    const int nthreads = 64 * nwaves;
     const int wg_rows = a.G * rows_per_group;
     float inv = 1.0f;
     if (a.mode == AXQ_X_RMSNORM) {
@@ -1537,15 +1507,10 @@ int launch_one(axq_ctx *ctx, const DpArgs &a, unsigned grid, unsigned block, siz
             (st = axq_allow_lds(ctx, reinterpret_cast<const void *>(&gemv_dpw_kernel<T, NB>), lds_allowed_w, 160 * 1024)) != AXQ_OK)
             return st;
         if (lds_w <= 160 * 1024) {
-            // fourteen or ten weight waves (four on two of the SIMDs, three on the others): two helper waves split x for the last two
-            static const bool no_helpers = getenv("AXQ_GEMV_HELPERS") && getenv("AXQ_GEMV_HELPERS")[0] == '0'; // development knob
-            DpArgs ah = a;
-            if (T::SPLIT_HELPERS && !no_helpers && a.G == 1 && (a.S & 3) == 2 && a.S >= 6 && block + 128 <= 1024 && NB <= T::BIG_NB) ah.H = 2;
-            const unsigned block_w = block + 64 * (unsigned)ah.H;
 #ifdef AXQ_STAMPS
-            gemv_dpw_kernel<T, NB><<<grid, block_w, 160 * 1024, ctx->stream>>>(DP_LAUNCH_ARGS(ah)); // the stamps live in the last 4 KB
+            gemv_dpw_kernel<T, NB><<<grid, block, 160 * 1024, ctx->stream>>>(DP_LAUNCH_ARGS(a)); // the stamps live in the last 4 KB
 #else
-            gemv_dpw_kernel<T, NB><<<grid, block_w, lds_w, ctx->stream>>>(DP_LAUNCH_ARGS(ah));
+            gemv_dpw_kernel<T, NB><<<grid, block, lds_w, ctx->stream>>>(DP_LAUNCH_ARGS(a));
 #endif
             return AXQ_OK;
         }
@@ -1698,7 +1663,7 @@ int launch_dp(axq_ctx *ctx, const axq_weight *w, const float *x, const uint8_t *
     a.k = (int)w->k;
     a.S = (a.k + 1023) / 1024;            // waves that span K once (<= 16)
     a.G = a.S <= 8 ? 8 / a.S : 1;         // row groups per workgroup
-    a.H = 0;
+    a.P = 1;
     const unsigned block = (unsigned)(64 * a.S * a.G);
     // 4-row steps per group: one workgroup per compute unit unless that makes a group's share of the
     // reduction buffer too large; the ring depth is what a lane can hold in registers
