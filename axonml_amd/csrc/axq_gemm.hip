@@ -28,6 +28,7 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4))); // a 16-byte register quad (arrays of HIP's uint4 struct end up in scratch)
 
 constexpr int BN = 128;  // output columns (weight rows) per workgroup
@@ -520,23 +521,29 @@ __global__ void __launch_bounds__(512) gemm_kernel(GemmArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// Q4_K: one MFMA per product.
+// Q4_K and Q5_K: one MFMA per product.
 //
 // A Q4_K weight is w = d * (sc * q) - dmin * m with a 4-bit code q, 6-bit sub-block scale sc and minimum m, and
-// f16 d, dmin per 256-element superblock (GGUF layout).  sc * q <= 945 is an integer of ten bits, so it is
-// EXACT in f16 -- and, as the bit pattern of an f16 subnormal, it needs no conversion at all: the integer n as
-// 16 bits is the f16 number n * 2^-24, which the matrix pipe multiplies exactly.  So the B operand of the main
-// loop is sc * q itself (two integer instructions per pair of weights), products x * (sc * q) are exact in the
-// f32 accumulator, and the superblock's d is applied to the accumulator, not to the weights:
-//   - the accumulator of an output column n holds the running sum in units of u_n, the d of the superblock
-//     being added; at a superblock boundary it is multiplied by u_n / d_next (one multiply per accumulator
-//     register per 256 k; a lane of the 32x32 MFMA output owns one column, so the factor is one number per
-//     lane).  A superblock with d = 0 contributes zeros and leaves the unit alone.
-//   - the minimum term, - sum_g dmin * m[n, g] * (sum of x over sub-block g), is a second, short GEMM over
-//     K / 32 "columns" that runs through the same pipeline after the main loop: c = dmin * m has 17 bits and
-//     goes in as two f16 (c S = ch + cl under a power-of-two S chosen per workgroup from the largest dmin it
-//     meets), the sub-block sums of x as two f16 (hi + lo, written by the x pre-pass), three products
-//     hi ch + hi cl + lo ch laid side by side along the extended K axis.
+// f16 d, dmin per 256-element superblock (GGUF layout); Q5_K is the same with a 5-bit code.  It goes through the matrix
+// pipe as w = d * sc * (q - C) + (C d sc - dmin m) with C = 8 (16) in the middle of the codes:
+//   - sc * (q - C) is an integer of magnitude <= 504 (1008), so it is EXACT in f16, and cheap to make: 0x6400 | n is the
+//     f16 number 1024 + n for n < 1024, so q * sc + 0x6400 (one multiply-add on a pair of codes) less 1024 + 8 sc is
+//     sc * (q - 8) (Q5_K: 1024 + q less 1040, times sc).  That is the B operand of the main loop; products x * sc * (q - C)
+//     are exact in the f32 accumulator, and the superblock's d is applied to the accumulator, not to the weights:
+//     the accumulator of an output column n holds the running sum in units of u_n, the d of the superblock being
+//     added; at a superblock boundary it is multiplied by u_n / d_next (one multiply per accumulator register per
+//     256 k; a lane of the 32x32 MFMA output owns one column, so the factor is one number per lane).  A superblock
+//     with d = 0 contributes zeros and leaves the unit alone.
+//   - the offset term, sum_g c[n, g] * (sum of x over sub-block g) with c = C d sc - dmin m, is a second, short GEMM
+//     over K / 32 "columns" that runs through the same pipeline after the main loop: c goes in as two f16 (c S = ch + cl
+//     under a power-of-two S chosen per column from the largest d and dmin it meets), the sub-block sums of x as two
+//     f16 (hi + lo, written by the x pre-pass), three products hi ch + hi cl + lo ch laid side by side along the
+//     extended K axis.
+//   Why centred: with the codes as they are (0 .. 15) and - dmin m as the second term, both sums are a sub-block's
+//   range times sum x, and for activation rows with a mean (all positive, say) each is a hundred times their difference:
+//   their f32 rounding then shows in the result (4e-5 of a row's largest output at K = 4096, past the 1e-3 bound for its
+//   small outputs).  Centred, the first sum is as well conditioned as the weights themselves and c is a sub-block's
+//   middle, small for weights around zero: 2e-6.
 // Against two MFMAs per product over all of K (the other block types below) this is 1 + 3/32.
 //
 // Tiling: a workgroup computes BM x 256 outputs with eight waves, each a block of 128 x 64 (BM = 256: 4 x 2 MFMA
@@ -572,7 +579,7 @@ __device__ inline void wait_vm_and_lds() {
     __builtin_amdgcn_s_waitcnt(((N >> 4) << 14) | (7 << 4) | (N & 15));
 }
 
-template <int BM, int NT>
+template <int BM, int NT, bool Q5 = false>
 __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
     constexpr int NW = NT / 64;          // waves: NW / 4 rows of four, each wave a block of WROWS x 64
     constexpr int WROWS = BM / (NW / 4); // 128 or 64
@@ -605,7 +612,9 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
     // What a thread holds of a group of four steps: main loop = one superblock: the 16 code bytes of its (row, half) for
     // each of the four pairs (64 consecutive bytes in memory) and the superblock's header; minimum term: the headers of
     // the four steps' superblocks (in q) -- five, or four, loads per task and group.
-    struct Raw { u32x4 q[BT][4]; u32x4 h[BT]; };
+    // Q5_K: also the 16 bytes of fifth bits that go with the thread's code bytes (one set per superblock: bit 2 p and
+    // 2 p + 1 of a byte belong to the two sub-blocks of pair p).
+    struct Raw { u32x4 q[BT][4]; u32x4 h[BT]; u32x4 b[BT]; };
     const uint8_t *xbase = reinterpret_cast<const uint8_t *>(a.xh + (size_t)m0 * a.k + (size_t)kbeg * BK);
     const uint8_t *x3base = reinterpret_cast<const uint8_t *>(a.xs3 + (size_t)m0 * a.xs3_pitch + (size_t)(kbeg >> 2) * 32);
     // a lane's part of a wave's x load: row lane / 8 of the eight, and the chunk that belongs at slot lane % 8 of that row:
@@ -614,7 +623,8 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
     const uint32_t xoff = (xrow_l * (uint32_t)a.k + xchunk_l * 8) * 2, x3off = (xrow_l * (uint32_t)a.xs3_pitch + xchunk_l * 8) * 2;
     const size_t x8rows = (size_t)8 * a.k * 2, x38rows = (size_t)8 * a.xs3_pitch * 2;
     const uint8_t *cbase = a.codes + (size_t)n0 * a.codes_pitch, *mbase = a.meta + (size_t)n0 * a.meta_pitch;
-    uint32_t coff[BT], moff[BT];
+    const uint8_t *qbase = Q5 ? a.qh + (size_t)n0 * a.qh_pitch : nullptr;
+    uint32_t coff[BT], moff[BT], qoff[BT];
     const int cpr = a.k >> 6; // pairs of sub-blocks (K steps) per row
     const int bh = tid & 1;   // which 16 bytes of a pair's 32 (NT is even: the same for every task of the thread)
     int b_wr[BT];             // where the thread's operands go in a weight stage (halfs): row, and the chunk exchange
@@ -624,6 +634,7 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
         const int crow = n0 + row < a.n ? row : a.n - 1 - n0;
         coff[u] = (uint32_t)crow * (uint32_t)a.codes_pitch;
         moff[u] = (uint32_t)crow * (uint32_t)a.meta_pitch;
+        qoff[u] = Q5 ? (uint32_t)crow * (uint32_t)a.qh_pitch + (uint32_t)(bh * 16) : 0u;
         b_wr[u] = row * 64 + ((((row >> 1) & 7) ^ (bh * 2)) * 8);
     }
     // x tile of main step `step` (or, MIN, of step s2 of the minimum term, clamped to the last) -> x stage `stage`
@@ -652,6 +663,7 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 #pragma unroll
             for (int j = 0; j < 4; j++) r.q[u][j] = *reinterpret_cast<const u32x4 *>(cb + j * 16 + (coff[u] + hoff));
             r.h[u] = *reinterpret_cast<const u32x4 *>(mb + moff[u]);
+            if constexpr (Q5) r.b[u] = *reinterpret_cast<const u32x4 *>(qbase + (size_t)(pair >> 2) * 32 + qoff[u]);
         }
     };
     // The minimum term: steps 4 grp .. 4 grp + 3 (clamped to the last step); a step = 64 columns = two superblocks of
@@ -667,13 +679,14 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
             for (int u = 0; u < BT; u++) r.q[u][j] = *reinterpret_cast<const u32x4 *>(mbase + (size_t)sb * 16 + moff[u]);
         }
     };
-    // While the minimum term is added the accumulators of a column hold the result times S, a power of two chosen from the
-    // largest |dmin| (f16 bits) the column's weight row has in this part of K: dmin < 2^(e + 1) -> the operands are
-    // c * 2^(8 - e) < 2^15; they meet sub-block sums stored times 1 / 64, so S = 2^(2 - e).  No dmin, or inf / nan:
-    // operands c, S = 1 / 64.  The feeder of a row and the lanes that own its column both work it out from the row's headers.
+    // While the offset term is added the accumulators of a column hold the result times S, a power of two chosen from the
+    // largest |d| or |dmin| (f16 bits) the column's weight row has in this part of K: both < 2^(e + 1) -> |c| < 63 * 17 *
+    // 2^(e + 1) < 2^(e + 12), the operands are c * 2^(3 - e) < 2^15; they meet sub-block sums stored times 1 / 64, so
+    // S = 2^(-3 - e).  All zero, or inf / nan: e = 8.  The feeder of a row and the lanes that own its column both work it
+    // out from the row's headers.
     auto s_of = [](uint32_t mx) {
         const int e = (mx == 0 || mx >= 0x7C00u) ? 8 : (mx >= 0x400u ? (int)(mx >> 10) - 15 : -15);
-        return __builtin_bit_cast(float, (uint32_t)(127 + 2 - e) << 23);
+        return __builtin_bit_cast(float, (uint32_t)(127 - 3 - e) << 23);
     };
     uint32_t dmax_r[BT];
 #pragma unroll
@@ -690,17 +703,42 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
             q4k_scale_min(r.h[u], p, scp, mp);
             const uint32_t dd = r.h[u][0];
             scp = (dd & 0x7FFFu) == 0 ? 0u : scp; // d = 0: the superblock adds nothing and leaves the unit alone
-            const uint32_t dm = (dd >> 16) & 0x7FFFu;
+            const uint32_t dm = (dd >> 16) & 0x7FFFu, da = dd & 0x7FFFu;
             dmax_r[u] = dm > dmax_r[u] ? dm : dmax_r[u];
+            dmax_r[u] = da > dmax_r[u] ? da : dmax_r[u];
             const uint32_t s0 = scp & 0xFF, s1 = scp >> 8;
             uint32_t lo[4], hi[4];
+            auto bits = [](half2v v) { return __builtin_bit_cast(uint32_t, v); };
+            auto halfs = [](uint32_t v) { return __builtin_bit_cast(half2v, v); };
+            auto pk2 = [](float v) { return __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(v, v)); }; // v twice; exact for these
+            constexpr uint32_t K1024 = 0x64006400u; // 0x6400 | n is the f16 number 1024 + n for n < 1024
+            if constexpr (Q5) {
+                // (q - 16) * sc: 1024 + q less 1040, times sc, every step exact in f16 (|.| <= 16 * 63)
+                const half2v m0 = pk2((float)s0), m1 = pk2((float)s1);
+                const half2v off = {(_Float16)-1040.0f, (_Float16)-1040.0f};
 #pragma unroll
-            for (int d = 0; d < 2; d++) {
-                const uint32_t w = r.q[u][j][2 * c1 + d];
-                lo[2 * d] = (w & 0x000F000Fu) * s0;
-                lo[2 * d + 1] = ((w >> 8) & 0x000F000Fu) * s0;
-                hi[2 * d] = ((w >> 4) & 0x000F000Fu) * s1;
-                hi[2 * d + 1] = ((w >> 12) & 0x000F000Fu) * s1;
+                for (int d = 0; d < 2; d++) {
+                    const uint32_t w = r.q[u][j][2 * c1 + d], f = r.b[u][2 * c1 + d];
+                    const uint32_t fl = p < 2 ? f << (4 - 2 * p) : (p == 2 ? f : f >> 2); // bit 2 p of every byte at bit 4
+                    const uint32_t fh = p < 2 ? f << (3 - 2 * p) : f >> (2 * p - 3);      // bit 2 p + 1
+                    const uint32_t ql = (w & 0x0F0F0F0Fu) | (fl & 0x10101010u), qh = ((w >> 4) & 0x0F0F0F0Fu) | (fh & 0x10101010u);
+                    lo[2 * d] = bits((halfs((ql & 0x001F001Fu) | K1024) + off) * m0);
+                    lo[2 * d + 1] = bits((halfs(((ql >> 8) & 0x001F001Fu) | K1024) + off) * m0);
+                    hi[2 * d] = bits((halfs((qh & 0x001F001Fu) | K1024) + off) * m1);
+                    hi[2 * d + 1] = bits((halfs(((qh >> 8) & 0x001F001Fu) | K1024) + off) * m1);
+                }
+            } else {
+                // (q - 8) * sc: q * sc <= 945 as an integer, 1024 + that as f16, less 1024 + 8 sc (exact: below 2048)
+                const float f0 = -1024.0f - (float)(8 * s0), f1 = -1024.0f - (float)(8 * s1);
+                const half2v o0 = pk2(f0), o1 = pk2(f1);
+#pragma unroll
+                for (int d = 0; d < 2; d++) {
+                    const uint32_t w = r.q[u][j][2 * c1 + d];
+                    lo[2 * d] = bits(halfs((w & 0x000F000Fu) * s0 + K1024) + o0);
+                    lo[2 * d + 1] = bits(halfs(((w >> 8) & 0x000F000Fu) * s0 + K1024) + o0);
+                    hi[2 * d] = bits(halfs(((w >> 4) & 0x000F000Fu) * s1 + K1024) + o1);
+                    hi[2 * d + 1] = bits(halfs(((w >> 12) & 0x000F000Fu) * s1 + K1024) + o1);
+                }
             }
             const int at = b_wr[u] ^ (c1 * 8);
             *reinterpret_cast<u32x4 *>(bs + at) = u32x4{lo[0], lo[1], lo[2], lo[3]};
@@ -716,13 +754,15 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 #pragma unroll
         for (int u = 0; u < BT; u++) {
             const u32x4 h = r.q[u][j];
-            const float dmin = live ? (-64.0f * S_r[u]) * h2f(h[0] >> 16) : 0.f;
+            const float s64 = live ? 64.0f * S_r[u] : 0.f;
+            const float dmin = h2f(h[0] >> 16), dc = (Q5 ? 16.0f : 8.0f) * h2f(h[0] & 0xFFFFu);
             uint32_t o[4];
 #pragma unroll
             for (int p = 0; p < 4; p++) {
                 uint32_t scp, mp;
                 q4k_scale_min(h, p, scp, mp);
-                const float c0 = dmin * ubyte<0>(mp), c1 = dmin * ubyte<1>(mp); // exact: 11 x 6 bits
+                // what the centred codes leave: (8 or 16) d sc - dmin m per sub-block, both products exact (11 x 6 bits)
+                const float c0 = s64 * (dc * ubyte<0>(scp) - dmin * ubyte<0>(mp)), c1 = s64 * (dc * ubyte<1>(scp) - dmin * ubyte<1>(mp));
                 const float h0 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, c0) & 0xFFFFE000u);
                 const float h1 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, c1) & 0xFFFFE000u);
                 const float v0 = t == 1 ? c0 - h0 : h0, v1 = t == 1 ? c1 - h1 : h1; // t: 0 ch, 1 cl, 2 ch, 3 nothing
@@ -765,8 +805,9 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const float dn = h2f(dnext[j] & 0xFFFFu);
-            const uint32_t dm = (dnext[j] >> 16) & 0x7FFFu;
+            const uint32_t dm = (dnext[j] >> 16) & 0x7FFFu, da = dnext[j] & 0x7FFFu;
             dmax_c[j] = dm > dmax_c[j] ? dm : dmax_c[j];
+            dmax_c[j] = da > dmax_c[j] ? da : dmax_c[j];
             const bool some = dn != 0.f;
             const float q = unit[j] / (some ? dn : 1.0f);
             r[j] = some ? q : 1.0f;
@@ -811,7 +852,7 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
     // this one does not touch); grp: index of the group among those of its kind.
     auto group = [&](auto kg, auto kn, int grp) {
         constexpr bool KG = decltype(kg)::value, KN = decltype(kn)::value;
-        constexpr int F = KN ? 4 * BT : 5 * BT; // loads of the weight request
+        constexpr int F = KN ? 4 * BT : (Q5 ? 6 : 5) * BT; // loads of the weight request
         if (!KG) new_unit(sb0 + grp);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -873,7 +914,7 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         S_c[j] = s_of(dmax_c[j]);
-        const float f = unit[j] * 16777216.0f * S_c[j];
+        const float f = unit[j] * S_c[j];
 #pragma unroll
         for (int i = 0; i < MI; i++)
 #pragma unroll
@@ -930,8 +971,9 @@ __global__ void __launch_bounds__(NT) gemm_q4k_kernel(GemmArgs a) {
 // themselves (with q as it is, two sums three times the size of the result would cancel in f32).  The second,
 // sum_b (m + c d)[n, b] * (sum of x over block b), goes through the matrix pipe too, two MFMAs per tile and
 // superblock of 256 k: A = the eight block sums of the row as f16 pairs (hi for k 0..7, lo for k 8..15, written by the
-// x pre-pass for the Q4_K kernel's minimum term, times 1 / 64), B = the eight m of the column, twice, and then the
-// eight c d, both times 256; the main term's scales are d * 256 / 64 to match.
+// x pre-pass for the Q4_K kernel's offset term, times 1 / 64), B = the column's eight offsets m + c d as f16 pairs
+// (the leading halves twice, then the remainders against the sums' leading halves); the sum is added times 256 and
+// the main term's scales are d * 256 / 64 to match.
 //
 // The pipeline is the Q4_K kernel's: BM x 128 outputs per workgroup of eight waves (BM = 256: 64 x 64 each; 128: 32 x 64),
 // x tiles straight from memory into three LDS stages, two weight stages, one barrier per K step that waits for LDS only,
@@ -943,7 +985,6 @@ constexpr float XSUM_SCALE = 1.0f / 64.0f; // the x pre-pass stores the block su
 
 template <int BITS, bool WITH_MIN, int BM>
 __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
-    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
     constexpr int NW = 8, AROWS = BM / NW, XL = AROWS / 8; // BM = 256 or 128 rows of x per workgroup
     constexpr int MI = BM / 128;                           // MFMA tiles of a wave along M: the waves lie 4 x 2, (32 MI) x 64 each
     constexpr int ASTAGE = BM * 64, BSTAGE = PBN * 64, BOFF = 3 * ASTAGE; // halfs
@@ -1100,26 +1141,32 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
         }
     };
     auto multiply_min = [&](int sb) {
-        // The operands are the stored f16 numbers themselves, m and d: any f16 a block can hold goes through exactly (m times
-        // a power of two, or 16 d, would overflow f16 for minimums from 256 and scales from 16 on).  The powers of two --
-        // WSCALE for both, the code centre for the d sum -- are applied in f32 when the sums are added.
-        half8 bm[2], bd[2];
+        // B = the blocks' offsets m + CENTER d (the weight of the middle code), each worked out in f32 (exact to its last
+        // bit) and cut into two f16, vh + vl: the first product takes [vh | vh] against the sums' [hi | lo], the second
+        // [vl | 0].  Kept apart (m against the sums, then CENTER d against the sums, added afterwards) the two halves of the
+        // offset are each as large as a block's range times sum x and cancel in f32: 1.1e-3 at the strict floor of the
+        // parity test for rows with a mean; together they are the block's middle, small for weights around zero.  An
+        // offset beyond f16's range (weights past 65504) saturates.
+        half8 bh[2], bl[2];
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            uint32_t om[4], od[4];
+            uint32_t oh[4], ol[4];
 #pragma unroll
-            for (int q = 0; q < 4; q++) { // blocks 2 q, 2 q + 1: the (d, m) records' upper halves are the minimums
+            for (int q = 0; q < 4; q++) { // blocks 2 q, 2 q + 1: (d, m) records
                 // (read as a plain vector: a read through HIP's uint2 made the compiler wait for every load in flight)
                 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
                 const u32x2 r2 = *reinterpret_cast<const u32x2 *>(rlane + (sb & 1) * RECB + j * 32 * 16 * RV + q * 8);
-                const uint32_t r0 = r2[0], r1 = r2[1];
-                om[q] = (r0 >> 16) | (r1 & 0xFFFF0000u);
-                od[q] = (r0 & 0xFFFFu) | (r1 << 16);
+                const float v0 = fmaf((float)CENTER, h2f(r2[0] & 0xFFFFu), h2f(r2[0] >> 16));
+                const float v1 = fmaf((float)CENTER, h2f(r2[1] & 0xFFFFu), h2f(r2[1] >> 16));
+                const auto vh = __builtin_amdgcn_cvt_pkrtz(v0, v1);
+                oh[q] = __builtin_bit_cast(uint32_t, vh);
+                const uint32_t low = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(v0 - (float)vh[0], v1 - (float)vh[1]));
+                ol[q] = hh ? 0u : low; // the sums' low halves meet vh only
             }
-            bm[j] = __builtin_bit_cast(half8, u32x4{om[0], om[1], om[2], om[3]});
-            bd[j] = __builtin_bit_cast(half8, u32x4{od[0], od[1], od[2], od[3]});
+            bh[j] = __builtin_bit_cast(half8, u32x4{oh[0], oh[1], oh[2], oh[3]});
+            bl[j] = __builtin_bit_cast(half8, u32x4{ol[0], ol[1], ol[2], ol[3]});
         }
-        // the block sums are stored times XSUM_SCALE: with the factors below the accumulators receive the term times
+        // the block sums are stored times XSUM_SCALE: with the factor below the accumulators receive the term times
         // WSCALE * XSUM_SCALE, which is what the main term scales its sums to (scale_of)
         // (added by the vector ALU like the main term: accumulators that the matrix pipe also wrote would be kept twice)
         const float16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -1127,10 +1174,10 @@ __global__ void __launch_bounds__(512) gemm_blk32_kernel(GemmArgs a) {
         for (int i = 0; i < MI; i++) {
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const float16v Sm = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bm[j], zero, 0, 0, 0);
-                const float16v Sd = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bd[j], zero, 0, 0, 0);
+                float16v S = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bh[j], zero, 0, 0, 0);
+                S = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, mx[i]), bl[j], S, 0, 0, 0);
 #pragma unroll
-                for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(Sd[r], CENTER * WSCALE, fmaf(Sm[r], WSCALE, acc[i][j][r]));
+                for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(S[r], WSCALE, acc[i][j][r]);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -1495,7 +1542,8 @@ struct GemmPlan {
 // that fit its registers (f32 rows).
 bool q4k_route(const axq_weight *w, bool in_regs_only) {
     static const bool off = getenv("AXQ_GEMM_Q4K") && getenv("AXQ_GEMM_Q4K")[0] == '0'; // development knob
-    return !off && w->type == AXQ_Q4_K && w->k % 256 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
+    const bool type_ok = w->type == AXQ_Q4_K || (w->type == AXQ_Q5_K && w->qh_pitch % 16 == 0);
+    return !off && type_ok && w->k % 256 == 0 && (!in_regs_only || w->k <= 16 * 256 * 4);
 }
 
 // Whether gemm_blk32_kernel takes this call.
@@ -1552,19 +1600,23 @@ XSums plan_sums(axq_ctx *ctx, const axq_weight *w, const GemmPlan &p) {
     return xs;
 }
 
-int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits) {
+template <bool Q5>
+int launch_q4k_tiles(axq_ctx *ctx, const GemmArgs &a, dim3 grid, size_t lds) {
     static std::atomic<uint64_t> lds_allowed[2]; // per kernel: a bit per device
+    int rc;
+    if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<256, 512, Q5>), lds_allowed[1], (3 * 256 * 64 + 2 * QBN * 64) * 2))) return rc;
+    if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<128, 512, Q5>), lds_allowed[0], (3 * 128 * 64 + 2 * QBN * 64) * 2))) return rc;
+    if (a.wm == 2) gemm_q4k_kernel<256, 512, Q5><<<grid, 512, lds, ctx->stream>>>(a);
+    else gemm_q4k_kernel<128, 512, Q5><<<grid, 512, lds, ctx->stream>>>(a);
+    return AXQ_OK;
+}
+
+int launch_gemm_q4k(axq_ctx *ctx, GemmArgs a, int splits, bool q5k) {
     const int bm = 128 * a.wm;
     const unsigned tiles = (unsigned)(((a.n + QBN - 1) / QBN) * ((a.m + bm - 1) / bm));
     const dim3 grid(tiles, (unsigned)splits);
     const size_t lds = (size_t)(3 * bm * 64 + 2 * QBN * 64) * sizeof(_Float16); // three x stages, two weight stages
-    {
-        int rc;
-        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<256, 512>), lds_allowed[1], (3 * 256 * 64 + 2 * QBN * 64) * 2))) return rc;
-        if ((rc = axq_allow_lds(ctx, reinterpret_cast<const void *>(gemm_q4k_kernel<128, 512>), lds_allowed[0], (3 * 128 * 64 + 2 * QBN * 64) * 2))) return rc;
-    }
-    if (a.wm == 2) gemm_q4k_kernel<256, 512><<<grid, 512, lds, ctx->stream>>>(a);
-    else gemm_q4k_kernel<128, 512><<<grid, 512, lds, ctx->stream>>>(a);
+    if (int rc = q5k ? launch_q4k_tiles<true>(ctx, a, grid, lds) : launch_q4k_tiles<false>(ctx, a, grid, lds)) return rc;
     AXQ_LAUNCH_CHECK(ctx, "gemm_q4k_kernel");
     if (splits > 1) {
         const int rows = a.pair ? a.m / 2 : a.m;
@@ -1629,7 +1681,7 @@ int run_gemm(axq_ctx *ctx, const axq_weight *w, int m, const GemmPlan &p, float 
     a.pair = pair ? 1 : 0; a.bias = bias; a.resid = resid; a.wm = p.wm;
     const XSums xs = plan_sums(ctx, w, p);
     a.xs3 = xs.xs3; a.xs3_pitch = xs.pitch;
-    if (p.q4k) return launch_gemm_q4k(ctx, a, p.splits);
+    if (p.q4k) return launch_gemm_q4k(ctx, a, p.splits, w->type == AXQ_Q5_K);
     if (p.q5) return launch_gemm_q5(ctx, a, p.splits, w->type);
     switch (w->type) {
     case AXQ_Q4_K: return launch_gemm<GQ4K>(ctx, a, p.splits);

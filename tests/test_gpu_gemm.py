@@ -36,7 +36,7 @@ def test_gemm_small_shapes(ctx, qtype, m, n, k):
     _check(ctx, qtype, m, n, k, seed=m + n + k + qtype)
 
 
-@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_1])
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q5_1])
 @pytest.mark.parametrize("m", [128, 512])
 def test_config_prefill_k4096(ctx, qtype, m):
     _check(ctx, qtype, m, 512, 4096, seed=m)
@@ -65,7 +65,17 @@ def test_ragged_tiles_of_the_block_of_32_kernel(ctx, qtype, m, n, k):
     _check(ctx, qtype, m, n, k, seed=m * 3 + n + k + qtype)
 
 
-@pytest.mark.parametrize("qtype", [o.Q4_1, o.Q5_1, o.Q4_0, o.Q5_0, o.Q8_0, o.Q4_K, o.Q6_K])
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K])
+@pytest.mark.parametrize("m,n,k", [(1, 1, 256), (127, 31, 768), (129, 129, 256), (257, 255, 512), (300, 130, 2304), (513, 4, 1280),
+                                   (260, 520, 4352)])
+def test_ragged_tiles_of_the_superblock_kernel(ctx, qtype, m, n, k):
+    """Row and column counts on both sides of its tile edges (128 and 256 rows, 256 columns, 64 per wave), one superblock,
+    odd counts of them (the minimum term takes them in pairs) and a K that is split over workgroups unevenly; Q5_K's fifth
+    bits ride along with the codes."""
+    _check(ctx, qtype, m, n, k, seed=m * 3 + n + k + qtype)
+
+
+@pytest.mark.parametrize("qtype", [o.Q4_1, o.Q5_1, o.Q4_0, o.Q5_0, o.Q8_0, o.Q4_K, o.Q5_K, o.Q6_K])
 @pytest.mark.parametrize("m", [48, 300])
 def test_large_weights_block_minimums_beyond_256_and_scales_beyond_32(ctx, qtype, m):
     """Weights around 300 with a spread of 100: block minimums of magnitude 256 and more, block scales of 16 to 40.  The
@@ -86,9 +96,33 @@ def test_large_weights_block_minimums_beyond_256_and_scales_beyond_32(ctx, qtype
     assert max_rel_err(got, o.matmul_f64(deq.reshape(n, k), x), STRICT_FLOOR) <= MATMUL_RTOL
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K])
 @pytest.mark.parametrize("xscale", [1e-30, 1e30])
-def test_many_rows_of_extreme_magnitude(ctx, xscale):
-    _check(ctx, o.Q4_K, 1030, 128, 512, seed=11, xscale=xscale)
+def test_many_rows_of_extreme_magnitude(ctx, qtype, xscale):
+    _check(ctx, qtype, 1030, 128, 512, seed=11, xscale=xscale)
+
+
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q4_1, o.Q5_1, o.Q6_K])
+@pytest.mark.parametrize("m,n,k", [(130, 33, 4096), (300, 520, 2048)])
+def test_activation_rows_with_a_mean(ctx, qtype, m, n, k):
+    """Rows that are all positive or sit on an offset: the sums over the codes and over the block minimums are then each
+    far larger than the result, and a kernel that adds them separately has to keep their rounding below the bound for
+    the row's small outputs too (codes centred before they are summed).  Both entry points, row by row."""
+    rng = np.random.default_rng(m + n + k + qtype)
+    wq = o.quantize(qtype, gen_weight(rng, n, k))
+    deq = o.dequantize(qtype, wq, n * k).reshape(n, k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[1] = 0.3 + 0.05 * x[1]
+    x[5] = np.abs(x[5])
+    x[6] = 5.0 + x[6]
+    x[7] = -2.0 + 0.5 * x[7]
+    dw = q.DeviceWeight.upload(q.QuantizedTensor([n, k], qtype, wq), ctx)
+    xb = q.f32_to_bf16_bits(x)
+    for got, xin in ((q.quantized_matmul_bf16(xb, dw, ctx), q.bf16_bits_to_f32(xb)), (q.quantized_matmul(x, dw, None, ctx), x)):
+        exact = o.matmul_f64(deq, xin)
+        for r in range(m):
+            assert max_rel_err(got[r], exact[r], STRICT_FLOOR) <= MATMUL_RTOL, (r, o.TYPE_NAMES[qtype])
+    dw.free()
 
 
 @pytest.mark.parametrize("xscale", [1e-4, 1.0, 3e4])
