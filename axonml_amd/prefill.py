@@ -12,7 +12,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16, published
 BLK32_TYPES = (QuantType.Q4_0, QuantType.Q4_1, QuantType.Q5_0, QuantType.Q5_1, QuantType.Q8_0)
 
 
-def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(QuantType.Q4_K, QuantType.Q5_1), iters=20,
+def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(QuantType.Q4_K, QuantType.Q5_K, QuantType.Q5_1), iters=20,
           f32_rows=True):
     """Times axq_gemm_bf16 (and, with f32_rows, the same product from f32 rows through axq_gemv_f32) per shape and type."""
     lib = ctx.lib
@@ -38,7 +38,7 @@ def bench(ctx, log=print, ms=(128, 512, 2048), ns=(4096, 14336), k=4096, types=(
                 t = ctx.timer_stop() / iters
                 flops = 2.0 * m * n * k
                 r = {"type": str(qt), "m": m, "n": n, "k": k, "ms": t, "tflops": flops / (t * 1e-3) / 1e12,
-                     "route": "hand-written MFMA GEMM, scaled codes as f16, one product per weight" if qt == QuantType.Q4_K
+                     "route": "hand-written MFMA GEMM, centred scaled codes as f16, one product per weight" if qt in (QuantType.Q4_K, QuantType.Q5_K)
                      else "hand-written MFMA GEMM, centred codes as f16, one product per weight, block scales by the vector ALU"
                      if k % 256 == 0 and qt in BLK32_TYPES
                      else "hand-written MFMA GEMM, weights dequantised to two f16 terms, two products per weight"}
