@@ -2,7 +2,8 @@
 //
 // The weights are read once for the whole batch.  The dot products run on v_mfma_i32_32x32x32_i8 with
 //   A (32 x 32): row 4 b + l = limb l of activation vector b (the split form of axq_split.h), 32 k of one block,
-//   B (32 x 32): column n = one of 32 weight rows, the block's 32 codes as bytes (4-bit codes as they are, 0..15),
+//   B (32 x 32): column n = one of 32 weight rows, the block's 32 codes as signed bytes, centred (a 4-bit code q goes in
+//                as 16 (q - 8): its nibble moved to the top of the byte with the top bit flipped; a 5-bit one as 8 (q - 16)),
 // so one instruction multiplies a 32-element block of 32 weight rows with all vectors and limbs.  Lane
 // (n, h) = (lane % 32, lane / 32) supplies 16 of the block's codes of row n and receives D[4 b + l][n] for
 // b = h, h + 2, h + 4, h + 6: all four limbs of four vectors, which it recombines and scales by itself.
@@ -59,15 +60,18 @@ __device__ inline float recombine4(int d0, int d1, int d2, int d3) {
 // h = lane / 32 says which 16 of a block's 32 codes the lane supplies.
 //   EVEN_ODD : h = 0 supplies the even elements, h = 1 the odd ones (reference nibble order); otherwise
 //              h = 0 supplies elements 0..15, h = 1 elements 16..31
-//   coef()   : w = d * code + mo (the 4-bit codes unsigned: the integer sums are exact, and the two f32 terms
-//              that then cancel for an activation with a mean are each rounded once)
+//   coef()   : w = d * operand + mo with the operand the centred code times 16 (or 8), so d is the block's scale over
+//              16 (8) and mo the weight of the middle code (nothing for Q4_0, Q5_0).  Centred because the integer sums
+//              are exact but their f32 images are not: with codes 0..15 the sum over the codes and the offset term
+//              are each a block's range times sum x, and for an activation with a mean their roundings, 2^-24 of that,
+//              showed in the small outputs (4-8e-4 at the strict floor of the parity test; centred 1e-4)
 // ---------------------------------------------------------------------------
 template <bool WITH_MIN>
 struct MQ4x {
     static constexpr int NP2 = 0; // no second plane
     static constexpr bool RUNS16 = false;
     static constexpr bool EVEN_ODD = true;
-    static constexpr bool OFFSET = true; // w = d * code + mo with mo = min (Q4_1) or -8 d (Q4_0): the codes stay unsigned
+    static constexpr bool OFFSET = WITH_MIN; // w = d (q - 8) + mo with mo = min + 8 d (Q4_1) or nothing (Q4_0)
     static constexpr int NV = UNITS * (WITH_MIN ? 4 : 2) / 16 > 0 ? UNITS * (WITH_MIN ? 4 : 2) / 16 : 1; // 16-byte vectors of scales per chunk
     struct Raw { u32x4 q[UNITS]; u32x4 m[NV]; };
     // the chunk's codes of one row: NP 16-byte pieces, piece p = block blk0 + p; a lane wants piece u for block u
@@ -84,21 +88,22 @@ struct MQ4x {
         }
     }
     __device__ static int4v operand(const Raw &r, int u, int h) {
-        const int sh = 4 * h;
+        const int sh = 4 - 4 * h;
         int4v b;
 #pragma unroll
-        for (int i = 0; i < 4; i++) b[i] = (int)((r.q[u][i] >> sh) & 0x0F0F0F0Fu);
+        for (int i = 0; i < 4; i++) b[i] = (int)(((r.q[u][i] << sh) & 0xF0F0F0F0u) ^ 0x80808080u); // 16 (q - 8)
         return b;
     }
     __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
         if (WITH_MIN) {
             const uint32_t v = r.m[u >> 2][u & 3];
-            d = f16lo(v);
-            mo = f16hi(v);
+            const float dd = f16lo(v);
+            d = dd * 0.0625f;
+            mo = fmaf(8.0f, dd, f16hi(v));
         } else {
             const uint32_t v = r.m[u >> 3][(u >> 1) & 3];
-            d = (u & 1) ? f16hi(v) : f16lo(v);
-            mo = -8.0f * d;
+            d = ((u & 1) ? f16hi(v) : f16lo(v)) * 0.0625f;
+            mo = 0.f;
         }
     }
 };
@@ -157,16 +162,26 @@ struct MQ4K {
         r.h[0] = ldg16(a.meta + row * a.meta_pitch + (size_t)(blk0 >> 3) * 16);
     }
     __device__ static int4v operand(const Raw &r, int u, int) {
-        const int sh = 4 * (u & 1);
         int4v b;
 #pragma unroll
-        for (int i = 0; i < 4; i++) b[i] = (int)((r.q[u >> 1][i] >> sh) & 0x0F0F0F0Fu);
+        for (int i = 0; i < 4; i++) { // 16 (q - 8)
+            const uint32_t w = r.q[u >> 1][i];
+            b[i] = (int)((((u & 1) ? w : w << 4) & 0xF0F0F0F0u) ^ 0x80808080u);
+        }
         return b;
     }
     __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
-        // 6-bit scale and min of sub-block j = u % 8 of superblock u / 8 (ggml get_scale_min_k4 order)
-        const u32x4 h = r.h[u >> 3];
-        const int j = u & 7;
+        float dsc, dm;
+        scale_min(r.h[u >> 3], u & 7, dsc, dm);
+        coef_of(dsc, dm, 8.0f, d, mo);
+    }
+    // operand = (16 or 8) (q - C): the scale over that factor, and the weight of the middle code (both products exact)
+    __device__ static void coef_of(float dsc, float dm, float C, float &d, float &mo) {
+        d = dsc * (C == 8.0f ? 0.0625f : 0.125f);
+        mo = C * dsc - dm;
+    }
+    // the 6-bit scale and minimum of sub-block j of the superblock with header h (ggml get_scale_min_k4 order), times d and dmin
+    __device__ static void scale_min(const u32x4 &h, int j, float &dsc, float &dm) {
         const uint32_t sc_lo = (j & 4) ? h[3] : h[1], mn_lo = (j & 4) ? h[3] : h[2];
         const int sh = 8 * (j & 3);
         uint32_t sc, mn;
@@ -177,9 +192,8 @@ struct MQ4K {
             sc = ((sc_lo >> sh) & 0xF) | (((h[1] >> sh) >> 6 & 3) << 4);
             mn = ((mn_lo >> sh) >> 4 & 0xF) | (((h[2] >> sh) >> 6 & 3) << 4);
         }
-        const float dd = f16lo(h[0]), dmin = f16hi(h[0]);
-        d = dd * (float)sc;
-        mo = -(dmin * (float)mn);
+        dsc = f16lo(h[0]) * (float)sc;
+        dm = f16hi(h[0]) * (float)mn;
     }
 };
 
@@ -200,16 +214,19 @@ struct MQ5K {
         r.h[0] = ldg16(a.meta + row * a.meta_pitch + (size_t)(blk0 >> 3) * 16);
     }
     __device__ static int4v operand(const Raw &r, int u, int) {
-        const int sh = 4 * (u & 1);
         int4v b;
 #pragma unroll
-        for (int i = 0; i < 4; i++) b[i] = (int)(((r.q[u >> 1][i] >> sh) & 0x0F0F0F0Fu) | (((r.q2[0][i] >> u) & 0x01010101u) << 4));
+        for (int i = 0; i < 4; i++) { // 8 (q - 16): the nibble at bits 3..6, the fifth bit, flipped, at bit 7
+            const uint32_t w = r.q[u >> 1][i];
+            const uint32_t nib = ((u & 1) ? w >> 1 : w << 3) & 0x78787878u, fifth = (r.q2[0][i] << (7 - u)) & 0x80808080u;
+            b[i] = (int)(nib ^ fifth ^ 0x80808080u);
+        }
         return b;
     }
     __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
-        MQ4K::Raw t;
-        t.h[0] = r.h[0];
-        MQ4K::coef(t, u, d, mo); // the codes stay unsigned 0..31: w = (d sc) code - dmin m
+        float dsc, dm;
+        MQ4K::scale_min(r.h[u >> 3], u & 7, dsc, dm);
+        MQ4K::coef_of(dsc, dm, 16.0f, d, mo);
     }
 };
 
@@ -259,7 +276,7 @@ struct MQ5x {
     static constexpr int NP2 = 2, NQ2 = 2;
     static constexpr bool RUNS16 = false;
     static constexpr bool EVEN_ODD = false;
-    static constexpr bool OFFSET = true;
+    static constexpr bool OFFSET = WITH_MIN;
     static constexpr int NV = MQ4x<WITH_MIN>::NV;
     struct Raw { u32x4 q[UNITS]; u32x4 m[NV]; u32x4 q2[2]; };
     static constexpr int NP = UNITS, NQ = UNITS;
@@ -274,22 +291,23 @@ struct MQ5x {
         for (int i = 0; i < NV; i++) r.m[i] = t.m[i];
     }
     __device__ static int4v operand(const Raw &r, int u, int h) {
-        const uint32_t bits = r.q2[u >> 2][u & 3] >> (16 * h);
+        const uint32_t bits = ~(r.q2[u >> 2][u & 3] >> (16 * h)); // flipped: 8 (q - 16) has the fifth bit's complement on top
         int4v b;
 #pragma unroll
-        for (int i = 0; i < 4; i++) // four bits to bit 4 of four bytes: t * 0x00204081 puts bit i at bit 8 i
-            b[i] = (int)(((r.q[u][i] >> (4 * h)) & 0x0F0F0F0Fu) | (((((bits >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4));
+        for (int i = 0; i < 4; i++) // four bits to bit 7 of four bytes: t * 0x00204081 puts bit i at bit 8 i
+            b[i] = (int)((((r.q[u][i] >> (4 * h)) & 0x0F0F0F0Fu) << 3) | (((((bits >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 7));
         return b;
     }
     __device__ static void coef(const Raw &r, int u, float &d, float &mo) {
         if (WITH_MIN) {
             const uint32_t v = r.m[u >> 2][u & 3];
-            d = f16lo(v);
-            mo = f16hi(v);
+            const float dd = f16lo(v);
+            d = dd * 0.125f;
+            mo = fmaf(16.0f, dd, f16hi(v));
         } else {
             const uint32_t v = r.m[u >> 3][(u >> 1) & 3];
-            d = (u & 1) ? f16hi(v) : f16lo(v);
-            mo = -16.0f * d;
+            d = ((u & 1) ? f16hi(v) : f16lo(v)) * 0.125f;
+            mo = 0.f;
         }
     }
 };

@@ -144,6 +144,27 @@ def test_activations_with_a_mean_do_not_cancel(ctx, qtype, k):
     dw.free()
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K, o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0])
+@pytest.mark.parametrize("batch,n,k", [(8, 520, 4096), (3, 264, 14336)])
+def test_small_batch_activations_with_a_mean_do_not_cancel(ctx, qtype, batch, n, k):
+    """The same for the small-batch kernel: rows on an offset of 20 standard deviations, all positive, or negative.  Its
+    codes go into the matrix pipe centred; as unsigned codes with the offset in a separate sum over x these rows came out
+    at 4-8e-4 at the strict floor."""
+    rng = np.random.default_rng(batch + n + k + qtype)
+    wq = o.quantize(qtype, gen_weight(rng, n, k))
+    wd = o.dequantize(qtype, wq, n * k).reshape(n, k)
+    dw = q.DeviceWeight.upload(q.QuantizedTensor([n, k], qtype, wq), ctx)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    x[0] = 1.0 + 0.05 * x[0]
+    x[1] = 10.0 + x[1]
+    x[2] = -3.0 + 0.1 * x[2]
+    got = q.quantized_matmul(x, dw, None, ctx)
+    exact = o.matmul_f64(wd, x)
+    for r in range(batch):
+        assert max_rel_err(got[r], exact[r], STRICT_FLOOR) <= 3e-4, r
+    dw.free()
+
+
 def test_quantized_linear_keeps_leading_dims(ctx):
     rng = np.random.default_rng(4)
     w = gen_weight(rng, 48, 512)
