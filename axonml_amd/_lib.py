@@ -122,6 +122,7 @@ SIGNATURES = {
     "axq_bench_graph_launch": (_i, [_vp, _vp, _i]),
     "axq_bench_graph_destroy": (None, [_vp, _vp]),
     "axq_bench_copy": (_i, [_vp, _vp, _vp, _sz, _i]),
+    "axq_bench_grid_barrier": (_i, [_vp, _i, _i, _i, C.POINTER(C.c_float)]),
     "axq_sample_token": (_i, [_vp, _vp, _i, _vp, _i, C.POINTER(SamplingConfig), C.c_float, C.POINTER(C.c_int32), _vp, _i]),
     "axq_model_set_sampling": (_i, [_vp, C.POINTER(SamplingConfig), C.c_uint64]),
     "axq_type_from_ggml": (_i, [_i]),

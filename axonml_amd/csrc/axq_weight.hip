@@ -6,6 +6,9 @@
 #include <stdlib.h>
 #include <new>
 
+#include <algorithm>
+#include <vector>
+
 #include "axq_internal.h"
 
 namespace {
@@ -101,6 +104,51 @@ __global__ void axq_copy16_kernel(uint4 *__restrict__ dst, const uint4 *__restri
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
         dst[i] = src[i];
 }
+
+// A barrier over every workgroup of one launch, through device-scope atomics, timed: what a kernel that stays resident
+// across the steps of a decode layer would pay where separate kernels pay a launch boundary.  Each of `rounds` rounds:
+// every thread publishes `publish_bytes` / threads of data with device-scope stores and waits for their acknowledgement,
+// the workgroup counts itself in and polls (bounded: a round nobody completes sets `fail` and the kernel ends all the
+// same).  levels = 1: one counter; 2: 16 groups of workgroups count in separately, the last of a group counts the group
+// in, the last group writes a release word that everybody polls.
+constexpr int BARRIER_WORDS = 18 * 32;
+__global__ void __launch_bounds__(256) grid_barrier_kernel(int *words, int *fail, float *data, long long *stamps, int rounds, int levels,
+                                                          int floats_per_thread) {
+    const int tid = threadIdx.x, wg = blockIdx.x, nwg = gridDim.x;
+    for (int r = 0; r < rounds; r++) {
+        const long long t0 = wall_clock64();
+        for (int i = 0; i < floats_per_thread; i++)
+            __hip_atomic_store(data + ((size_t)wg * floats_per_thread + i) * 256 + tid, (float)(r + wg), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const long long t1 = wall_clock64();
+        if (tid == 0) {
+            // a round's words lie 128 bytes apart (polls and counts on one line queue behind each other): the one counter or
+            // the groups' counter, the release word, sixteen group counters
+            int *base = words + (size_t)r * BARRIER_WORDS;
+            int spins = 0, v = 0;
+            if (levels == 1) {
+                __hip_atomic_fetch_add(base, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                while ((v = __hip_atomic_load(base, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) < nwg && ++spins < (1 << 18)) __builtin_amdgcn_s_sleep(2);
+                if (v < nwg) atomicExch(fail, 1);
+            } else {
+                const int g = wg & 15, in_group = (nwg - g + 15) / 16;
+                if (__hip_atomic_fetch_add(base + (2 + g) * 32, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_group - 1)
+                    if (__hip_atomic_fetch_add(base, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (nwg < 16 ? nwg : 16) - 1)
+                        __hip_atomic_store(base + 32, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                while ((v = __hip_atomic_load(base + 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) == 0 && ++spins < (1 << 18)) __builtin_amdgcn_s_sleep(2);
+                if (v == 0) atomicExch(fail, 1);
+            }
+        }
+        __syncthreads();
+        const long long t2 = wall_clock64();
+        if (tid == 0) {
+            long long *st = stamps + ((size_t)r * nwg + wg) * 3;
+            st[0] = t0; st[1] = t1; st[2] = t2;
+        }
+    }
+}
+
 
 // Reads `n16*16` bytes and keeps nothing: what the memory system gives a launch that only streams a weight.  Each
 // workgroup takes one contiguous share and keeps U 16-byte loads per lane in flight (non-temporal when NT); a lane whose
@@ -567,6 +615,60 @@ int axq_bench_read_ring_ex(axq_ctx *ctx, const axq_weight *const *weights, int n
         AXQ_LAUNCH_CHECK(ctx, "axq_bench_read_ring");
     }
     if (streams > 1 && (rc = axq_aux_join(ctx, streams))) return rc;
+    return AXQ_OK;
+}
+
+int axq_bench_grid_barrier(axq_ctx *ctx, int levels, int publish_bytes, int rounds, float *out_us) {
+    if (!ctx || !out_us) return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_grid_barrier: NULL argument");
+    if (levels < 1 || levels > 2 || rounds < 2 || rounds > 4096 || publish_bytes < 0 || publish_bytes % 1024 || publish_bytes > (1 << 20))
+        return axq_fail(ctx, AXQ_ERR_INVALID_ARGUMENT, "axq_bench_grid_barrier: levels 1 or 2, 2..4096 rounds, publish_bytes a multiple of 1024 up to 1 MiB");
+    AXQ_HIP(ctx, hipSetDevice(ctx->device), AXQ_ERR_DRIVER);
+    const int nwg = ctx->prop.multiProcessorCount; // one workgroup per compute unit: all of them resident together
+    const int fpt = publish_bytes / 1024;
+    int *words = nullptr, *fail = nullptr;
+    float *data = nullptr;
+    long long *stamps = nullptr;
+    const size_t wbytes = (size_t)rounds * BARRIER_WORDS * sizeof(int), sbytes = (size_t)rounds * nwg * 3 * sizeof(long long);
+    int rc = AXQ_OK, failed = 0;
+    std::vector<long long> h((size_t)rounds * nwg * 3);
+    if (hipMalloc(&words, wbytes) != hipSuccess || hipMalloc(&fail, sizeof(int)) != hipSuccess ||
+        hipMalloc(&data, (size_t)nwg * (fpt ? fpt : 1) * 1024) != hipSuccess || hipMalloc(&stamps, sbytes) != hipSuccess) {
+        rc = axq_fail(ctx, AXQ_ERR_ALLOCATION_FAILED, "axq_bench_grid_barrier: device allocation failed");
+    } else {
+        for (int rep = 0; rep < 2 && rc == AXQ_OK; rep++) { // the second run is the one read
+            if (hipMemsetAsync(words, 0, wbytes, ctx->stream) != hipSuccess || hipMemsetAsync(fail, 0, sizeof(int), ctx->stream) != hipSuccess) {
+                rc = axq_fail(ctx, AXQ_ERR_DRIVER, "axq_bench_grid_barrier: memset failed");
+                break;
+            }
+            grid_barrier_kernel<<<nwg, 256, 0, ctx->stream>>>(words, fail, data, stamps, rounds, levels, fpt);
+            if (hipGetLastError() != hipSuccess || hipStreamSynchronize(ctx->stream) != hipSuccess)
+                rc = axq_fail(ctx, AXQ_ERR_DRIVER, "axq_bench_grid_barrier: launch failed");
+        }
+        if (rc == AXQ_OK && (hipMemcpy(&failed, fail, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess ||
+                             hipMemcpy(h.data(), stamps, sbytes, hipMemcpyDeviceToHost) != hipSuccess))
+            rc = axq_fail(ctx, AXQ_ERR_DRIVER, "axq_bench_grid_barrier: copy failed");
+        if (rc == AXQ_OK && failed) rc = axq_fail(ctx, AXQ_ERR_DRIVER, "axq_bench_grid_barrier: a round was not completed within its bounded wait");
+    }
+    (void)hipFree(words); (void)hipFree(fail); (void)hipFree(data); (void)hipFree(stamps);
+    if (rc != AXQ_OK) return rc;
+    // per round (the first quarter left out): from the last workgroup's arrival to the release as each workgroup sees it;
+    // wall_clock64 counts 100 MHz
+    std::vector<double> med, worst, pub;
+    for (int r = rounds / 4; r < rounds; r++) {
+        long long last = 0;
+        double p = 0;
+        for (int w = 0; w < nwg; w++) {
+            const long long *st = &h[((size_t)r * nwg + w) * 3];
+            last = st[1] > last ? st[1] : last;
+            p += (double)(st[1] - st[0]) * 0.01 / nwg;
+        }
+        std::vector<double> d(nwg);
+        for (int w = 0; w < nwg; w++) d[w] = (double)(h[((size_t)r * nwg + w) * 3 + 2] - last) * 0.01;
+        std::sort(d.begin(), d.end());
+        med.push_back(d[nwg / 2]); worst.push_back(d[nwg - 1]); pub.push_back(p);
+    }
+    auto median = [](std::vector<double> &v) { std::sort(v.begin(), v.end()); return (float)v[v.size() / 2]; };
+    out_us[0] = median(med); out_us[1] = median(worst); out_us[2] = median(pub);
     return AXQ_OK;
 }
 

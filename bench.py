@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
     python bench.py --read-sweep      (a table instead: a read-only kernel over the same weight in every launch shape)
+    python bench.py --grid-barrier    (a table instead: a barrier over all workgroups of a launch through device-scope atomics)
 
 A "step" is one Q4_K GEMV (decode-path quantized matmul), weight 14336 x 4096 drawn ~N(0, 0.02) with
 1 % of entries at +-0.5, activation f32[4096] ~N(0, 1), batch 1: the bandwidth headline case.  Launch i
@@ -405,6 +406,9 @@ def main():
     ap.add_argument("--gemv-table", action="store_true",
                     help="instead of the benchmark, for kernel-trace profiles: the one-vector and batch-8 GEMVs of every block "
                          "type at 14336x4096 and 4096x14336 as plain stream launches over their rings, one line each")
+    ap.add_argument("--grid-barrier", action="store_true",
+                    help="instead of the benchmark: time a barrier over all workgroups of one resident launch through device-scope "
+                         "atomics (what a kernel that spans dependent steps would pay per step), and print the table")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path is built or measured)")
@@ -422,6 +426,15 @@ def main():
         return
     if args.read_sweep:
         read_sweep(ctx, args.steps, args.warmup)
+        return
+    if args.grid_barrier:
+        out = (C.c_float * 3)()
+        print(f"{info.compute_units} workgroups of 256 threads, one per compute unit; 256 rounds per line, medians over the last 192; us")
+        print("counters  published bytes per workgroup   last arrival -> release seen by the median workgroup   by the slowest   publishing")
+        for levels in (1, 2):
+            for pub in (0, 1024, 4096, 16384):
+                ctx.check(lib.axq_bench_grid_barrier(ctx.handle, levels, pub, 256, out))
+                print(f"{'one' if levels == 1 else '16 + 1':8s}  {pub:8d}   {out[0]:6.2f}   {out[1]:6.2f}   {out[2]:6.2f}", flush=True)
         return
     if args.gemv_table:
         for qt in (T.Q4_K, T.Q5_K, T.Q6_K, T.Q4_0, T.Q4_1, T.Q5_0, T.Q5_1, T.Q8_0):

@@ -342,6 +342,15 @@ AXQ_API int axq_bench_gemv_ring_streams(axq_ctx *ctx, const axq_weight *const *w
  * size multiples of 16).  A kernel of known traffic against which profiler memory counters are scaled. */
 AXQ_API int axq_bench_copy(axq_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes, int iters);
 
+/* Measures a barrier over all workgroups of one resident launch (one workgroup per compute unit) through device-scope
+ * atomics: what a kernel that stays on the chip across dependent steps would pay where separate kernels pay a launch
+ * boundary.  levels = 1: one counter; 2: sixteen group counters, then a release word.  Before counting in, every
+ * workgroup publishes publish_bytes (a multiple of 1024, may be 0) with device-scope stores.  Waits are bounded: a round
+ * that does not complete returns AXQ_ERR_DRIVER.  out_us[0]: from the last workgroup's arrival to the release as the
+ * median workgroup sees it, [1]: as the slowest sees it, [2]: the publishing, all medians over the rounds.  Synchronous.
+ * No counterpart in the reference. */
+AXQ_API int axq_bench_grid_barrier(axq_ctx *ctx, int levels, int publish_bytes, int rounds, float *out_us);
+
 #ifdef __cplusplus
 }
 #endif
