@@ -7,7 +7,7 @@ one-token attention at head size 128 with four query heads per KV head, and the 
 layers instead of 32 keep the CPU decode oracle at seconds; every kernel instantiation is the 32-layer
 model's.
 
-Config 5 (prefill GEMM): all six (M, N) shapes at K = 4096 for Q4_K and Q5_1.  The GPU computes the whole
+Config 5 (prefill GEMM): all six (M, N) shapes at K = 4096 for Q4_K, Q5_K and Q5_1.  The GPU computes the whole
 [M, N] product; the oracle gets a random subset of the weight rows (output columns) and the matching
 columns are compared, which keeps the single-thread reference sgemm at a second per case.
 """
@@ -108,7 +108,7 @@ def prefill_weights():
     return get
 
 
-@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_1])
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q5_1])
 @pytest.mark.parametrize("n", [4096, 14336])
 @pytest.mark.parametrize("m", [128, 512, 2048])
 def test_config5_prefill_gemm_full_shapes(ctx, prefill_weights, qtype, m, n):
@@ -148,3 +148,14 @@ def test_quantize_model_keeps_names_and_order_and_stops_at_the_first_error(ctx):
         q.quantize_model(bad, q.QuantType.Q8_0, ctx)
     with pytest.raises(q.InvalidQuantType):
         q.quantize_model(tensors, 99, ctx)
+
+
+def test_the_grid_barrier_probe_completes(ctx):
+    """bench.py --grid-barrier's entry point: every round completes within its bounded wait, with one counter and with two
+    levels, and reports times of a plausible size (microseconds, not milliseconds)."""
+    import ctypes as C
+    out = (C.c_float * 3)()
+    for levels, publish in ((1, 0), (2, 1024)):
+        ctx.check(ctx.lib.axq_bench_grid_barrier(ctx.handle, levels, publish, 16, out))
+        assert 0.0 < out[0] <= out[1] < 1000.0 and 0.0 <= out[2] < 1000.0
+    assert ctx.lib.axq_bench_grid_barrier(ctx.handle, 3, 0, 16, out) != 0  # no such form
